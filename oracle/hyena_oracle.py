@@ -1,0 +1,546 @@
+"""CPU oracle for the Hyena operator hot path.  TEST INFRASTRUCTURE ONLY.
+
+This file restates, in plain PyTorch on the CPU, the arithmetic of the
+reference's Hyena operator path (vortex/model/engine.py and its callers),
+including every dtype rounding point.  It is the checker for the HIP kernels:
+only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may
+import it.  Nothing in the product package may call into this file.
+
+Each function cites the reference file:line it follows (paths relative to the
+reference checkout).  The reference is Python/torch, so the restatement is
+Python/torch too; torch's own conv1d / fft are the library routines the
+reference itself calls.
+
+How each function is pinned (see tests/test_oracle_*.py):
+  se_fir / parallel_fir(K<128) : brute-force O(L*K) float64 loops, impulse
+                                 response, and the two-pass Toeplitz identity
+                                 held by the reference's test_two_pass_ref.py
+  mr_fir / parallel_fir(K>=128): ref_fftconv of the reference's
+                                 test/test_forward.py:13-23 restated, direct
+                                 float64 convolution, equality with se_fir on
+                                 the flipped filter, impulse response
+  modal_filter                 : closed forms h[0]=sum(r), geometric series sum
+  parallel_iir / modal state   : FFT path == explicit recurrence (the identity
+                                 asserted by the reference's
+                                 test/test_prefill.py:85-229)
+  toeplitz / correction        : known-answer arange filter of
+                                 vortex/ops/hyena_se/tests/test_toeplitz.py
+  step_fir / step_iir          : no reference test touches these ("parity
+                                 unpinned" by the reference's own tests); they
+                                 are pinned here by prefill-vs-decode
+                                 consistency and the closed-form recurrence,
+                                 plus the committed golden vectors in
+                                 tests/golden/ when present.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+
+import torch
+import torch.nn.functional as F
+
+
+# --------------------------------------------------------------------------
+# layout glue  (vortex/model/utils.py:26-85)
+# --------------------------------------------------------------------------
+
+def interleave(z):
+    """De-interleave stride-3 channels into [x1 | x2 | v] blocks.
+
+    vortex/model/utils.py:26-38: channels 0::3, 1::3, 2::3 are concatenated
+    along the channel axis (axis 1 for [B, 3D, L], last axis for [B, 3D]).
+    """
+    if z.dim() == 3:
+        return torch.cat([z[:, 0::3], z[:, 1::3], z[:, 2::3]], dim=1)
+    return torch.cat([z[..., 0::3], z[..., 1::3], z[..., 2::3]], dim=-1)
+
+
+def column_split(x, num_heads, head_size):
+    """Head-blocked split of 3D channels into (x2, x1, v).
+
+    vortex/model/utils.py:41-85: channels are viewed as
+    [num_heads, 3*head_size]; the first/second/third head_size of each head go
+    to x2/x1/v.  Works for [B, 3D] and [B, 3D, L].
+    """
+    if x.dim() == 2:
+        xr = x.reshape(x.shape[0], num_heads, 3 * head_size)
+        parts = [xr[..., i * head_size:(i + 1) * head_size].reshape(x.shape[0], -1) for i in range(3)]
+    else:
+        xr = x.reshape(x.shape[0], num_heads, 3 * head_size, x.shape[2])
+        parts = [
+            xr[:, :, i * head_size:(i + 1) * head_size].reshape(x.shape[0], -1, x.shape[-1]) for i in range(3)
+        ]
+    return parts[0], parts[1], parts[2]
+
+
+def split_gates(u, dims, column_split_hyena=False, flip_x1x2=False):
+    """(x2, x1, v) from the [B, 3D, L] (or [B, 3D]) projection.
+
+    vortex/model/engine.py:150-158 and :283-310.
+    """
+    hidden, n_heads, head_dim = dims[0], dims[1], dims[2]
+    if column_split_hyena:
+        x2, x1, v = column_split(u, n_heads, head_dim)
+    else:
+        x2, x1, v = u.split([hidden, hidden, hidden], dim=1)
+    if flip_x1x2:
+        x1, x2 = x2, x1
+    return x2, x1, v
+
+
+# --------------------------------------------------------------------------
+# prefill FIR  (vortex/model/engine.py:131-260)
+# --------------------------------------------------------------------------
+
+def short_fir_fp32(u, weight, fir_length):
+    """fp32 depthwise cross-correlation with left zero padding.
+
+    vortex/model/engine.py:197-204: conv1d on fp32 copies, padding K-1,
+    groups = channel count, truncated to the first L outputs.  weight is
+    [D, 1, K]; weight[..., K-1] multiplies the current sample.
+    """
+    L = u.shape[-1]
+    return F.conv1d(
+        u.to(torch.float32), weight.to(torch.float32), bias=None, stride=1,
+        padding=fir_length - 1, groups=u.shape[1],
+    )[..., :L]
+
+
+def fft_causal_conv_fp32(u, k):
+    """Causal convolution y[t] = sum_j k[j] u[t-j] through a length-2L FFT.
+
+    vortex/model/engine.py:50-73 (non-bidirectional branch).  u: [B, D, L]
+    fp32, k: [D, 1, Lk] or [D, Lk] fp32.
+    """
+    L = u.shape[-1]
+    n = 2 * L
+    k_f = torch.fft.rfft(k, n=n) / n
+    k_f = k_f.squeeze()
+    if u.dim() > k_f.dim():
+        k_f = k_f.unsqueeze(0)
+    u_f = torch.fft.rfft(u.to(k.dtype), n=n)
+    return torch.fft.irfft(u_f * k_f, n=n, norm="forward")[..., :L]
+
+
+def fftconv_with_bias(u, k, D):
+    """engine.py:38-83: fft conv, then `+ u * D[:, None]` in fp32, cast to u.dtype."""
+    y = fft_causal_conv_fp32(u, k)
+    out = y + u * D.unsqueeze(-1)
+    return out.to(u.dtype)
+
+
+def parallel_fir(
+    u, weight, bias, L=None, dims=None, groups=None, gated_bias=False,
+    column_split_hyena=False, dim_last=True, fir_length=3, gate=False,
+    want_state=False, padding_mask=None, flip_x1x2=False,
+):
+    """Restatement of HyenaInferenceEngine.parallel_fir (engine.py:131-260).
+
+    Returns (z, fir_state) with z in [B, D, L] layout.  `want_state` stands
+    for `inference_params is not None` (engine.py:255-258).
+    """
+    x2 = None
+    if gate:
+        x2, x1, v = split_gates(u, dims, column_split_hyena, flip_x1x2)
+        u = x1 * v                                   # engine.py:159, input dtype
+    if fir_length >= 128:
+        # engine.py:174-187.  The fp32 upcast, FFT conv, fp32 bias add, then
+        # two casts back to the input dtype.
+        z = fftconv_with_bias(u.to(torch.float32), weight[:, :, : u.shape[-1]].to(torch.float32), bias)
+        z = z.to(u.dtype)
+    else:
+        if dim_last:
+            u = u.permute(0, 2, 1)
+        z = short_fir_fp32(u, weight, fir_length).to(u.dtype)     # engine.py:197-208
+        if bias is not None:                                       # engine.py:219-223
+            z = z + bias[None, :, None] * u if gated_bias else z + bias[None, :, None]
+    if isinstance(padding_mask, torch.Tensor):                     # engine.py:226-227
+        z = z * padding_mask[:, None]
+    if gate:
+        z = x2 * z                                                 # engine.py:232
+    state = u[..., -fir_length + 1:] if want_state else None      # engine.py:255-258
+    return z, state
+
+
+def se_fir(x2, x1, v, h_groups, fir_length=None):
+    """Hyena-SE gated short FIR on explicit gates.
+
+    Same arithmetic as parallel_fir(gate=True, K<128) after the split:
+    u = bf16(x1*v); z = bf16(corr_K(u)); out = bf16(x2*z).  h_groups is
+    [G, 1, K]; it is expanded with repeat_interleave(D/G) as in
+    vortex/model/model.py:261-262.
+    """
+    D = x1.shape[1]
+    K = h_groups.shape[-1] if fir_length is None else fir_length
+    w = h_groups.repeat_interleave(D // h_groups.shape[0], 0)
+    u = x1 * v
+    z = short_fir_fp32(u, w, K).to(u.dtype)
+    return x2 * z, u[..., -K + 1:]
+
+
+def mr_fir(x2, x1, v, h_groups, D_bias):
+    """Hyena-MR gated medium FIR (true convolution through FFT) on explicit gates.
+
+    parallel_fir(gate=True, K>=128): u = bf16(x1*v); y = fftconv(u, h);
+    z = bf16(y + u*D) ; out = bf16(x2*z).  (engine.py:174-187, :38-83, :232)
+    """
+    Dch = x1.shape[1]
+    w = h_groups.repeat_interleave(Dch // h_groups.shape[0], 0)
+    u = x1 * v
+    z = fftconv_with_bias(u.to(torch.float32), w[:, :, : u.shape[-1]].to(torch.float32), D_bias.to(torch.float32))
+    z = z.to(u.dtype)
+    K = h_groups.shape[-1]
+    return x2 * z, u[..., -K + 1:]
+
+
+# --------------------------------------------------------------------------
+# modal filter and Hyena-LI prefill  (model.py:377-398, engine.py:262-404)
+# --------------------------------------------------------------------------
+
+def modal_filter(log_poles, residues, L, dtype=None):
+    """h[g, t] = Re sum_s residues[g, s] * exp(log_poles[g, s, 0] * t), t < L.
+
+    vortex/model/model.py:390-398 (real parameters).  Complex parameters use
+    the same expression and the real part is taken, matching
+    `(residues * poles**t).real.sum(1)` of model.py:847.  Returns [1, G, L].
+    `dtype=torch.float64/complex128` evaluates the same formula in double.
+    """
+    t = torch.arange(L)[None, None]
+    if dtype is not None:
+        cdt = dtype
+        if log_poles.is_complex():
+            cdt = torch.complex128 if dtype == torch.float64 else torch.complex64
+        log_poles, residues = log_poles.to(cdt), residues.to(cdt)
+    h = (residues[..., None] * (log_poles * t).exp()).sum(1)[None]
+    return h.real if h.is_complex() else h
+
+
+def long_conv_fp32(x1v, h):
+    """engine.py:331-337: fp32 FFT long convolution, returns (y_fp32, X_s)."""
+    L = x1v.shape[-1]
+    n = 2 * L
+    H = torch.fft.rfft(h.to(torch.float32), n=n) / n
+    X_s = torch.fft.fft(x1v.to(torch.float32), n=n)
+    X = X_s[..., : H.shape[-1]]
+    y = torch.fft.irfft(X * H, n=n, norm="forward")[..., :L]
+    return y, X_s
+
+
+def modal_state_fft(X_s, log_poles, L, hidden, groups, keep_complex=False):
+    """engine.py:525-559: modal state after L tokens through the FFT of p^t.
+
+    state[b, d, s] = sum_j p^(L-1-j) x1v[b, d, j].  The reference casts the
+    complex result to float32, i.e. drops the imaginary part (engine.py:559);
+    keep_complex=True returns the complex state (needed for complex poles).
+    """
+    n = 2 * L
+    t = torch.arange(L)[None, None]
+    lp = log_poles.to(torch.complex64 if log_poles.is_complex() else torch.float32)
+    state_s = (lp * t).exp()                                     # [G, S, L]
+    state_S = torch.fft.fft(state_s, n=n)[None]                  # [1, G, S, 2L]
+    if groups > 1:
+        state_S = state_S.repeat_interleave(hidden // groups, 1)
+    state = torch.fft.ifft(X_s[..., None, :] * state_S, n=n)[..., L - 1]
+    if keep_complex:
+        return state
+    return state.real.to(torch.float32)
+
+
+def modal_state_closed_form(x1v, log_poles, dtype=torch.float64):
+    """Textbook form of the same state: sum_j p^(L-1-j) u[j], in double."""
+    L = x1v.shape[-1]
+    cdt = torch.complex128 if log_poles.is_complex() else dtype
+    lp = log_poles.to(cdt)[..., 0]                               # [G, S]
+    G = lp.shape[0]
+    Dch = x1v.shape[1]
+    lp = lp.repeat_interleave(Dch // G, 0)                       # [D, S]
+    e = torch.arange(L - 1, -1, -1, dtype=torch.float64)
+    w = (lp[..., None] * e).exp()                                # [D, S, L]
+    return torch.einsum("dsl,bdl->bds", w, x1v.to(cdt))
+
+
+def parallel_iir(
+    z_pre, h, D, L, poles, residues, dims, column_split_hyena=False,
+    flip_x1x2=False, want_state=False, keep_complex_state=False, return_fp32_conv=False,
+):
+    """Restatement of HyenaInferenceEngine.parallel_iir, default FFT branch.
+
+    engine.py:283-353 and :379-404.  Returns (y [B, L, D], state or None[,
+    y_conv_fp32]).  Cast order: y = bf16(conv); out = (y + x1v*D)*x2 in the
+    tensors' own dtypes.
+    """
+    hidden, _, _, state_size, groups = dims
+    x2, x1, v = split_gates(z_pre, dims, column_split_hyena, flip_x1x2)
+    x1v = x1 * v
+    y32, X_s = long_conv_fp32(x1v, h)
+    y = y32.to(x1v.dtype)
+    y = (y + x1v * D.unsqueeze(-1)) * x2
+    state = None
+    if want_state:
+        state = modal_state_fft(X_s, poles, L, hidden, groups, keep_complex=keep_complex_state)
+    out = (y.permute(0, 2, 1), state)
+    if return_fp32_conv:
+        out = out + (y32,)
+    return out
+
+
+def li_prefill(x2, x1, v, log_poles, residues, D_bias, want_state=True):
+    """Hyena-LI on explicit gates with grouped (possibly complex) poles.
+
+    Filter per group from modal_filter, expanded over the group's channels;
+    conv as engine.py:331-337; gating as engine.py:352-353.  Returns
+    (out [B, D, L], y_conv_fp32 [B, D, L], state [B, D, S] complex or real).
+    """
+    B, Dch, L = x1.shape
+    G = log_poles.shape[0]
+    h = modal_filter(log_poles, residues, L)[0]                  # [G, L]
+    h = h.repeat_interleave(Dch // G, 0)[None]                   # [1, D, L]
+    x1v = x1 * v
+    y32, X_s = long_conv_fp32(x1v, h)
+    y = y32.to(x1v.dtype)
+    out = (y + x1v * D_bias.unsqueeze(-1)) * x2
+    state = None
+    if want_state:
+        state = modal_state_closed_form(x1v, log_poles)
+        state = state.to(torch.complex64) if state.is_complex() else state.to(torch.float32)
+    return out, y32, state
+
+
+def prefill_direct_recurrence(x1v, log_poles, residues):
+    """Explicit modal recurrence  s_t = p s_{t-1} + u_t,  y_t = Re sum r s_t.
+
+    Same arithmetic as engine.py:473-504 (which carries separate re/im lanes),
+    written with complex tensors in double for use as the independent check
+    of the FFT path.  Returns (y [B, D, L] float64, final state [B, D, S]).
+    """
+    B, Dch, L = x1v.shape
+    G = log_poles.shape[0]
+    cplx = log_poles.is_complex() or residues.is_complex()
+    dt = torch.complex128 if cplx else torch.float64
+    p = log_poles.to(dt)[..., 0].exp().repeat_interleave(Dch // G, 0)[None]   # [1, D, S]
+    r = residues.to(dt).repeat_interleave(Dch // G, 0)[None]
+    s = torch.zeros(B, Dch, p.shape[-1], dtype=dt)
+    y = torch.zeros(B, Dch, L, dtype=torch.float64)
+    xu = x1v.to(dt)
+    for i in range(L):
+        s = p * s + xu[:, :, i, None]
+        acc = (r * s).sum(-1)
+        y[:, :, i] = acc.real if cplx else acc
+    return y, s
+
+
+# --------------------------------------------------------------------------
+# decode steps  (engine.py:406-467)
+# --------------------------------------------------------------------------
+
+def step_fir(u, fir_state, weight, bias=None, gated_bias=False, flip_filter=False):
+    """Restatement of HyenaInferenceEngine.step_fir (engine.py:406-449).
+
+    u: [B, D]; fir_state: [B, D, cache] oldest-first; weight: [D, 1, K].
+    Returns (y in u.dtype, new state in float32).
+    """
+    w = weight.squeeze()
+    cache = fir_state.shape[-1]
+    K = w.shape[-1]
+    if flip_filter:
+        w = w.flip(-1)[..., -cache - 1:].unsqueeze(0)
+    else:
+        w = w[..., : cache + 1].unsqueeze(0)
+    in_dtype = u.dtype
+    w = w.to(torch.float32)
+    uf = u.to(torch.float32)
+    st = fir_state.to(torch.float32)
+    y = w[..., -1] * uf + torch.sum(st * w[..., :-1], dim=-1)
+    if bias is not None:
+        b = bias.to(torch.float32)
+        y = y + b * uf if gated_bias else y + b
+    if cache < K - 1:
+        st = torch.cat([st, uf[..., None]], dim=-1)
+    else:
+        st = torch.roll(st, -1, dims=2)
+        st[..., -1] = uf
+    return y.to(in_dtype), st
+
+
+def step_iir(x2, x1, v, D, residues, log_poles, iir_state):
+    """Restatement of HyenaInferenceEngine.step_iir (engine.py:451-467).
+
+    x2, x1, v: [B, D]; log_poles [G, S, 1], residues [G, S] with G == D or 1
+    (broadcast); iir_state [B, D, S].  Complex parameters give a complex y;
+    callers take its real part.
+    """
+    x1v = x1 * v
+    p = torch.exp(log_poles)[..., 0][None]
+    r = residues[None]
+    iir_state = p * iir_state + x1v[..., None]
+    res = torch.sum(r * iir_state, dim=-1)
+    y = x2 * (res + D * x1v)
+    return y, iir_state
+
+
+# --------------------------------------------------------------------------
+# two-pass chunked Toeplitz form  (vortex/ops/hyena_se/utils.py, ref_fwd.py)
+# --------------------------------------------------------------------------
+
+def toeplitz(hf, size):
+    """T[g, i, j] = hf[g, i-j] for 0 <= i-j < K, else 0  (hyena_se/utils.py:5-25)."""
+    g, K = hf.shape
+    i = torch.arange(size)[:, None]
+    j = torch.arange(size)[None, :]
+    lag = i - j
+    ok = (lag >= 0) & (lag < K)
+    T = torch.zeros(g, size, size, dtype=hf.dtype)
+    T[:, ok] = hf[:, lag[ok]]
+    return T
+
+
+def correction_toeplitz(hf, size):
+    """T^[g, i, j] = hf[g, i+size-j] for j >= i and i+size-j < K  (utils.py:38-51)."""
+    g, K = hf.shape
+    i = torch.arange(size)[:, None]
+    j = torch.arange(size)[None, :]
+    lag = i + size - j
+    ok = (j >= i) & (lag < K)
+    T = torch.zeros(g, size, size, dtype=hf.dtype)
+    T[:, ok] = hf[:, lag[ok]]
+    return T
+
+
+def gcg_fwd_ref(x, B, C, h):
+    """Gate-conv-gate reference in the (b, l, g, dg) layout, input dtype throughout.
+
+    vortex/ops/hyena_se/ref_fwd.py:80-127: Bx = B*x; depthwise conv1d with
+    h.repeat_interleave(dg), padding K-1, first L outputs; C * y.
+    """
+    bs, l, g, dg = x.shape
+    K = h.shape[-1]
+    Bx = (B * x).permute(0, 2, 3, 1).reshape(bs, g * dg, l)
+    w = h.repeat_interleave(dg, dim=0)
+    y = F.conv1d(Bx, w, groups=g * dg, stride=1, padding=K - 1)[..., :l]
+    y = y.reshape(bs, g, dg, l).permute(0, 3, 1, 2)
+    return C * y
+
+
+def gcg_two_pass_chunked(x, B, C, h, chunk):
+    """Two-pass chunked Toeplitz algorithm (ref_fwd.py:216-266).
+
+    Per chunk c: y_c = T @ Bx_c + T^ @ Bx_{c-1} with T, T^ built from the
+    flipped filter; out = C * y.
+    """
+    b, l, g, dg = x.shape
+    n = l // chunk
+    hf = h.flip(-1)[:, 0]
+    Bx = (B * x).reshape(b, n, chunk, g, dg).permute(0, 1, 3, 2, 4)   # b n g chunk dg
+    T = toeplitz(hf, chunk).to(x.dtype)
+    Th = correction_toeplitz(hf, chunk).to(x.dtype)
+    y = torch.matmul(T, Bx)
+    prev = torch.roll(Bx, 1, dims=1)
+    prev[:, 0] = 0
+    y = y + torch.matmul(Th, prev)
+    y = y.permute(0, 1, 3, 2, 4).reshape(b, l, g, dg)
+    return C * y
+
+
+def causal_conv1d_ref(x, weight, bias=None, apply_gated_bias=False):
+    """vortex/ops/hyena_se/interface.py:207-244 with activation=None.
+
+    x [B, D, L], weight [D, K]; computed in weight.dtype, cast back to x.dtype.
+    """
+    dt = x.dtype
+    x = x.to(weight.dtype)
+    L = x.shape[-1]
+    Dch, K = weight.shape
+    gb = None
+    if apply_gated_bias:
+        gb, bias = bias, None
+    out = F.conv1d(x, weight.unsqueeze(1), bias, padding=K - 1, groups=Dch)[..., :L]
+    if apply_gated_bias:
+        out = out + x * gb
+    return out.to(dt)
+
+
+# --------------------------------------------------------------------------
+# engine-shaped wrapper so that parity tests read like calls into the reference
+# --------------------------------------------------------------------------
+
+@dataclass
+class OracleCache:
+    """Counterpart of vortex/model/cache.py:31-61 (dicts keyed by layer index)."""
+    fir_state_dict: dict = field(default_factory=dict)
+    fir_inner_state_dict: dict = field(default_factory=dict)
+    state_dict: dict = field(default_factory=dict)
+    seqlen_offset: int = 0
+
+
+class OracleEngine:
+    """Duck-type of HyenaInferenceEngine backed by the functions above."""
+
+    def __init__(self, layer_idx=None, hyena_flip_x1x2=False):
+        self.layer_idx = layer_idx
+        self.hyena_flip_x1x2 = hyena_flip_x1x2
+
+    def parallel_fir(self, fir_fn, u, weight, bias, L, dims, groups=None, gated_bias=False,
+                     column_split_hyena=False, dim_last=True, fir_length=3, gate=False,
+                     inference_params=None, prefill_mode=None, padding_mask=None):
+        return parallel_fir(u, weight, bias, L, dims, groups, gated_bias, column_split_hyena,
+                            dim_last, fir_length, gate, inference_params is not None,
+                            padding_mask, self.hyena_flip_x1x2)
+
+    def parallel_iir(self, z_pre, h, D, L, poles, residues, t, dims, layer_idx,
+                     inference_params=None, prefill_style="fft", fftconv_fn=None,
+                     padding_mask=None, use_flashfft=False, column_split_hyena=False,
+                     long_fir_threshold=None):
+        y, state = parallel_iir(z_pre, h, D, L, poles, residues, dims, column_split_hyena,
+                                self.hyena_flip_x1x2, inference_params is not None,
+                                keep_complex_state=poles.is_complex())
+        if inference_params is not None:
+            inference_params.state_dict[layer_idx] = state
+        return y
+
+    def step_fir(self, u, fir_state, weight, bias=None, gated_bias=False, flip_filter=False):
+        return step_fir(u, fir_state, weight, bias, gated_bias, flip_filter)
+
+    def step_iir(self, x2, x1, v, D, residues, poles, iir_state, iir_groups=1):
+        if iir_groups > 1:
+            raise NotImplementedError
+        return step_iir(x2, x1, v, D, residues, poles, iir_state)
+
+
+# --------------------------------------------------------------------------
+# synthetic inputs of the benchmark configurations (seeded on the CPU)
+# --------------------------------------------------------------------------
+
+def make_gates(B, D, L, seed=0, dtype=torch.bfloat16):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return tuple(torch.randn(B, D, L, generator=g).to(dtype) for _ in range(3))   # x2, x1, v
+
+
+def make_se_filter(G, K=7, seed=100):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return torch.randn(G, 1, K, generator=g) / math.sqrt(K)
+
+
+def make_mr_filter(G, K=128, seed=200):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    w = torch.randn(G, 1, K, generator=g) / math.sqrt(K)
+    a = 0.01 + 0.09 * torch.rand(G, 1, 1, generator=g)
+    return w * torch.exp(-a * torch.arange(K)[None, None])
+
+
+def make_modal_complex(G, S=16, seed=300, pmin=0.9, pmax=0.9999):
+    """Complex poles |p|~U(pmin,pmax), arg~U(0,pi); residues ~CN(0,1). log_poles [G,S,1] complex64."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    mag = pmin + (pmax - pmin) * torch.rand(G, S, generator=g, dtype=torch.float64)
+    ang = math.pi * torch.rand(G, S, generator=g, dtype=torch.float64)
+    log_poles = torch.complex(mag.log(), ang).to(torch.complex64)[..., None]
+    res = torch.complex(torch.randn(G, S, generator=g), torch.randn(G, S, generator=g)) / math.sqrt(2.0)
+    return log_poles, res.to(torch.complex64)
+
+
+def make_modal_real(G, S=16, seed=400, pmin=0.9, pmax=0.9999):
+    """Real poles in vortex's own parametrisation: log_poles [G,S,1] fp32 (<0), residues [G,S] fp32."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    mag = pmin + (pmax - pmin) * torch.rand(G, S, generator=g, dtype=torch.float64)
+    return mag.log().to(torch.float32)[..., None], torch.randn(G, S, generator=g)

@@ -1,0 +1,314 @@
+"""Pins the CPU oracle against what fixes it independently of its own formulas:
+brute-force float64 loops, impulse responses, closed forms, the reference's
+own known-answer tests, and cross-identities between its code paths."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import hyena_oracle as O
+
+
+def brute_corr(u, w):
+    """z[d,t] = sum_k w[d,k] u[d,t-(K-1)+k], float64 python loops."""
+    D, L = u.shape
+    K = w.shape[1]
+    z = np.zeros((D, L))
+    for d in range(D):
+        for t in range(L):
+            acc = 0.0
+            for k in range(K):
+                j = t - (K - 1) + k
+                if j >= 0:
+                    acc += w[d, k] * u[d, j]
+            z[d, t] = acc
+    return z
+
+
+def brute_conv(u, h):
+    """y[d,t] = sum_k h[d,k] u[d,t-k]"""
+    D, L = u.shape
+    K = h.shape[1]
+    y = np.zeros((D, L))
+    for d in range(D):
+        for t in range(L):
+            acc = 0.0
+            for k in range(min(K, t + 1)):
+                acc += h[d, k] * u[d, t - k]
+            y[d, t] = acc
+    return y
+
+
+def test_orientation_known_answer():
+    # cell 26 of the reference's test_log_analysis.ipynb: conv1d([0,1,2],[2,1,0]) = 1
+    # (cross-correlation: no flip of the kernel)
+    x = torch.tensor([[[0.0, 1.0, 2.0]]])
+    w = torch.tensor([[[2.0, 1.0, 0.0]]])
+    assert torch.nn.functional.conv1d(x, w).item() == 1.0
+    # and the short FIR of the oracle puts w[K-1] on the current sample
+    z = O.short_fir_fp32(torch.tensor([[[1.0, 0.0, 0.0, 0.0]]]), torch.tensor([[[5.0, 6.0, 7.0]]]), 3)
+    assert z.flatten().tolist() == [7.0, 6.0, 5.0, 0.0]
+
+
+@pytest.mark.parametrize("K", [3, 7, 16])
+def test_short_fir_vs_bruteforce(K):
+    g = torch.Generator().manual_seed(K)
+    D, L = 6, 37
+    u = torch.randn(1, D, L, generator=g)
+    w = torch.randn(D, 1, K, generator=g)
+    z = O.short_fir_fp32(u, w, K)[0].double().numpy()
+    ref = brute_corr(u[0].double().numpy(), w[:, 0].double().numpy())
+    np.testing.assert_allclose(z, ref, atol=1e-5)
+
+
+def test_se_rounding_points():
+    # u is rounded to bf16 before the FIR, z is rounded to bf16 before the gate
+    x2, x1, v = O.make_gates(2, 32, 64, seed=1)
+    h = O.make_se_filter(2, 7)
+    out, st = O.se_fir(x2, x1, v, h)
+    u = (x1.float() * v.float()).bfloat16()
+    w = h.repeat_interleave(16, 0)[:, 0].double().numpy()
+    z = np.stack([brute_corr(u[b].double().numpy(), w) for b in range(2)])
+    zb = torch.from_numpy(z).float().bfloat16()
+    exp = (x2.float() * zb.float()).bfloat16()
+    # F.conv1d sums in another order than the loop: allow 1 bf16 ulp on z
+    assert (out.float() - exp.float()).abs().max() <= 2 ** -7 * exp.float().abs().max()
+    assert torch.equal(st, u[..., -6:])
+    assert out.dtype == torch.bfloat16
+
+
+def test_parallel_fir_matches_se_fir_and_splits():
+    B, D, L, G = 2, 32, 48, 2
+    g = torch.Generator().manual_seed(3)
+    u = torch.randn(B, 3 * D, L, generator=g).bfloat16()
+    h = O.make_se_filter(G, 7).repeat_interleave(D // G, 0)
+    dims = (D, 4, D // 4, 16, G)
+    z, st = O.parallel_fir(u, h, None, L, dims, groups=G, dim_last=False, fir_length=7, gate=True, want_state=True)
+    x2, x1, v = u.split(D, 1)
+    out, st2 = O.se_fir(x2, x1, v, O.make_se_filter(G, 7))
+    assert torch.equal(z, out) and torch.equal(st, st2)
+    # column split: head h holds [x2 | x1 | v] of head_dim each
+    zc, _ = O.parallel_fir(u, h, None, L, dims, groups=G, dim_last=False, fir_length=7, gate=True,
+                           column_split_hyena=True)
+    ur = u.reshape(B, 4, 3, D // 4, L)
+    outc, _ = O.se_fir(ur[:, :, 0].reshape(B, D, L), ur[:, :, 1].reshape(B, D, L), ur[:, :, 2].reshape(B, D, L),
+                       O.make_se_filter(G, 7))
+    assert torch.equal(zc, outc)
+
+
+def test_interleave_index_map():
+    z = torch.arange(12.0).reshape(1, 12, 1)
+    assert O.interleave(z).flatten().tolist() == [0, 3, 6, 9, 1, 4, 7, 10, 2, 5, 8, 11]
+    assert O.interleave(z[..., 0]).flatten().tolist() == [0, 3, 6, 9, 1, 4, 7, 10, 2, 5, 8, 11]
+
+
+def test_featurizer_fir_dim_last_and_bias():
+    B, L, D3, K = 2, 20, 12, 3
+    g = torch.Generator().manual_seed(5)
+    u = torch.randn(B, L, D3, generator=g).bfloat16()
+    w = torch.randn(D3, 1, K, generator=g)
+    bias = torch.randn(D3, generator=g)
+    z, st = O.parallel_fir(u, w, bias, L, None, fir_length=K, dim_last=True, gate=False, want_state=True)
+    ut = u.permute(0, 2, 1)
+    ref = np.stack([brute_corr(ut[b].double().numpy(), w[:, 0].double().numpy()) for b in range(B)])
+    refb = torch.from_numpy(ref).float().bfloat16()
+    exp = refb + bias[None, :, None]          # bf16 + fp32 -> fp32 (torch promotion)
+    assert z.dtype == exp.dtype
+    assert (z - exp).abs().max() <= 2 ** -7 * exp.abs().max()
+    assert torch.equal(st, ut[..., -2:])
+
+
+def ref_fftconv(x, h):
+    # formula held by the reference's test/test_forward.py:13-23
+    n = 2 * x.shape[-1]
+    y = torch.fft.irfft(torch.fft.rfft(x.float(), n=n) * torch.fft.rfft(h.float(), n=n) / n, n=n, norm="forward")
+    return y[..., : x.shape[-1]]
+
+
+def test_fft_conv_vs_bruteforce_and_ref_fftconv():
+    g = torch.Generator().manual_seed(7)
+    D, L, K = 4, 50, 20
+    u = torch.randn(1, D, L, generator=g)
+    h = torch.randn(D, 1, K, generator=g)
+    y = O.fft_causal_conv_fp32(u, h)
+    ref = brute_conv(u[0].double().numpy(), h[:, 0].double().numpy())
+    np.testing.assert_allclose(y[0].double().numpy(), ref, atol=2e-5)
+    np.testing.assert_allclose(y.numpy(), ref_fftconv(u, h[:, 0][None]).numpy(), atol=1e-5)
+    # impulse response: y = h
+    e = torch.zeros(1, D, L)
+    e[..., 0] = 1
+    np.testing.assert_allclose(O.fft_causal_conv_fp32(e, h)[0, :, :K].numpy(), h[:, 0].numpy(), atol=1e-6)
+
+
+def test_mr_is_true_convolution_with_fp32_bias():
+    B, D, L, G, K = 1, 32, 256, 2, 128
+    x2, x1, v = O.make_gates(B, D, L, seed=11)
+    h = O.make_mr_filter(G, K)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(12))
+    out, st = O.mr_fir(x2, x1, v, h, Db)
+    u = (x1.float() * v.float()).bfloat16()
+    w = h.repeat_interleave(D // G, 0)[:, 0].double().numpy()
+    y = brute_conv(u[0].double().numpy(), w) + u[0].double().numpy() * Db.double().numpy()[:, None]
+    zb = torch.from_numpy(y).float().bfloat16()
+    exp = (x2[0].float() * zb.float()).bfloat16()
+    assert (out[0].float() - exp.float()).abs().max() <= 2 ** -7 * exp.float().abs().max()
+    assert torch.equal(st, u[..., -127:])
+    # same thing as the short-FIR form on the flipped filter (orientation cross-check)
+    z_corr = O.short_fir_fp32(u, h.flip(-1).repeat_interleave(D // G, 0), K)
+    z_conv = O.fft_causal_conv_fp32(u.float(), h.repeat_interleave(D // G, 0))
+    np.testing.assert_allclose(z_corr.numpy(), z_conv.numpy(), atol=2e-4)
+
+
+def test_parallel_fir_k128_branch_equals_mr_fir():
+    B, D, L, G, K = 2, 32, 160, 2, 128
+    g = torch.Generator().manual_seed(13)
+    u = torch.randn(B, 3 * D, L, generator=g).bfloat16()
+    h = O.make_mr_filter(G, K)
+    Db = torch.randn(D, generator=g).bfloat16()
+    dims = (D, 4, D // 4, 16, G)
+    z, st = O.parallel_fir(u, h.repeat_interleave(D // G, 0), Db, L, dims, groups=G, gated_bias=True,
+                           dim_last=False, fir_length=K, gate=True, want_state=True)
+    x2, x1, v = u.split(D, 1)
+    out, st2 = O.mr_fir(x2, x1, v, h, Db)
+    assert torch.equal(z, out) and torch.equal(st, st2)
+
+
+def test_toeplitz_known_answer_arange():
+    # vortex/ops/hyena_se/tests/test_toeplitz.py:33-66: h = arange, T built from the flipped filter
+    for g, K, C in [(1, 4, 16), (2, 4, 32), (2, 128, 128)]:
+        h = torch.arange(g * K).reshape(g, 1, K)
+        hf = h[:, 0].flip(-1)
+        T = O.toeplitz(hf, C)
+        Th = O.correction_toeplitz(hf, C)
+        for gi in range(g):
+            for i in range(C):
+                for j in range(C):
+                    lag = i - j
+                    exp = int(h[gi, 0, K - 1 - lag]) if 0 <= lag < K else 0
+                    assert int(T[gi, i, j]) == exp
+                    lag2 = i + C - j
+                    exp2 = int(h[gi, 0, K - 1 - lag2]) if (j >= i and lag2 < K) else 0
+                    assert int(Th[gi, i, j]) == exp2
+            if g * K * C > 4096:
+                break
+
+
+@pytest.mark.parametrize("g,K", [(1, 4), (2, 128), (4, 128)])
+def test_two_pass_equals_conv1d(g, K):
+    # the identity asserted by the reference's test_two_pass_ref.py::test_ref_chunked_fwd (atol 1e-4)
+    gen = torch.Generator().manual_seed(17)
+    bs, L, dg = 2, 512, 16
+    x, B, C = (torch.randn(bs, L, g, dg, generator=gen) for _ in range(3))
+    h = torch.randn(g, 1, K, generator=gen)
+    y1 = O.gcg_fwd_ref(x, B, C, h)
+    y2 = O.gcg_two_pass_chunked(x, B, C, h, L // 2)
+    assert torch.allclose(y1, y2, atol=1e-4)
+    y3 = O.gcg_two_pass_chunked(x, B, C, h, 128)
+    assert torch.allclose(y1, y3, atol=1e-4)
+
+
+def test_modal_filter_closed_forms():
+    lp, r = O.make_modal_complex(3, 16, seed=5, pmax=0.99)
+    L = 4096
+    h = O.modal_filter(lp, r, L)[0]
+    assert torch.allclose(h[:, 0], r.sum(1).real, atol=1e-5)
+    p = lp[..., 0].to(torch.complex128).exp()
+    geo = (r.to(torch.complex128) * (1 - p ** L) / (1 - p)).sum(1).real
+    assert torch.allclose(h.double().sum(1), geo, atol=1e-3)
+    lpr, rr = O.make_modal_real(3, 16, seed=6, pmax=0.99)
+    hr = O.modal_filter(lpr, rr, L)[0]
+    pr = lpr[..., 0].double().exp()
+    assert torch.allclose(hr[:, 0], rr.sum(1), atol=1e-5)
+    assert torch.allclose(hr.double().sum(1), (rr.double() * (1 - pr ** L) / (1 - pr)).sum(1), atol=1e-3)
+    # t=1 term pins the sign/index of the exponent
+    assert torch.allclose(hr[:, 1].double(), (rr.double() * pr).sum(1), atol=1e-5)
+
+
+@pytest.mark.parametrize("cplx", [False, True])
+def test_li_fft_equals_recurrence(cplx):
+    # FFT long conv + FFT state == explicit modal recurrence (reference test/test_prefill.py:85-229)
+    B, D, L, G = 2, 8, 192, 4
+    x2, x1, v = O.make_gates(B, D, L, seed=21)
+    lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(G, 16, seed=22, pmax=0.99)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(23)).bfloat16()
+    out, y32, state = O.li_prefill(x2, x1, v, lp, r, Db)
+    x1v = x1 * v
+    y_rec, s_rec = O.prefill_direct_recurrence(x1v, lp, r)
+    assert (y32.double() - y_rec).abs().max() <= 1e-4 * y_rec.abs().max()
+    assert (state.to(s_rec.dtype) - s_rec).abs().max() <= 1e-5 * s_rec.abs().max()
+    # the reference's own FFT state path agrees with the closed form (imag dropped for real poles)
+    h = O.modal_filter(lp, r, L)[0].repeat_interleave(D // G, 0)[None]
+    _, X_s = O.long_conv_fp32(x1v, h)
+    st_fft = O.modal_state_fft(X_s, lp, L, D, G, keep_complex=cplx)
+    assert (st_fft.to(s_rec.dtype) - s_rec).abs().max() <= 1e-3 * s_rec.abs().max()
+    # gate/cast order
+    yb = y32.bfloat16()
+    exp = (yb + x1v * Db[:, None]) * x2
+    assert torch.equal(out, exp)
+
+
+def test_parallel_iir_matches_li_prefill_when_G_equals_D():
+    B, D, L = 1, 8, 64
+    g = torch.Generator().manual_seed(31)
+    z_pre = torch.randn(B, 3 * D, L, generator=g).bfloat16()
+    lp, r = O.make_modal_real(D, 16, seed=32, pmax=0.99)
+    Db = torch.randn(D, generator=g).bfloat16()
+    dims = (D, 2, D // 2, 16, D)
+    h = O.modal_filter(lp, r, L)
+    y, st = O.parallel_iir(z_pre, h, Db, L, lp, r, dims, want_state=True)
+    x2, x1, v = z_pre.split(D, 1)
+    out, _, st2 = O.li_prefill(x2, x1, v, lp, r, Db)
+    assert torch.equal(y, out.permute(0, 2, 1))
+    assert torch.allclose(st, st2, atol=1e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("K,flip,gated", [(7, False, False), (128, True, True), (3, False, False)])
+def test_step_fir_consistent_with_prefill(K, flip, gated):
+    # feeding tokens one at a time from the prefill tail reproduces prefill outputs
+    B, D, L, n_dec = 2, 16, 160, 5
+    g = torch.Generator().manual_seed(41 + K)
+    u_all = torch.randn(B, D, L + n_dec, generator=g).bfloat16()
+    w = torch.randn(D, 1, K, generator=g) / math.sqrt(K)
+    bias = torch.randn(D, generator=g) if gated else None
+    if K >= 128:
+        full = O.fftconv_with_bias(u_all.float(), w.float(), bias.float()).to(u_all.dtype)
+    else:
+        full = O.short_fir_fp32(u_all, w, K).to(u_all.dtype)
+    state = u_all[..., L - (K - 1): L]
+    for i in range(n_dec):
+        y, state = O.step_fir(u_all[..., L + i], state, w, bias=bias, gated_bias=gated, flip_filter=flip)
+        assert y.dtype == torch.bfloat16 and state.dtype == torch.float32
+        assert (y.float() - full[..., L + i].float()).abs().max() <= 2 ** -7 * full.float().abs().max()
+        assert torch.equal(state, u_all[..., L + i + 1 - (K - 1): L + i + 1].float())
+
+
+def test_step_fir_partial_cache_growth():
+    # cache shorter than K-1: state is appended, taps are the first cache+1 (non-flip)
+    B, D, K = 1, 4, 7
+    g = torch.Generator().manual_seed(51)
+    w = torch.randn(D, 1, K, generator=g)
+    st = torch.randn(B, D, 2, generator=g).bfloat16()
+    u = torch.randn(B, D, generator=g).bfloat16()
+    y, st2 = O.step_fir(u, st, w)
+    exp = w[:, 0, 2] * u.float() + st[..., 0].float() * w[:, 0, 0] + st[..., 1].float() * w[:, 0, 1]
+    assert torch.allclose(y.float(), exp.bfloat16().float())
+    assert st2.shape[-1] == 3 and torch.equal(st2[..., -1], u.float())
+
+
+@pytest.mark.parametrize("cplx", [False, True])
+def test_step_iir_consistent_with_prefill(cplx):
+    B, D, L, n_dec = 2, 8, 96, 4
+    x2, x1, v = O.make_gates(B, D, L + n_dec, seed=61)
+    lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(D, 16, seed=62, pmax=0.99)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(63)).bfloat16()
+    _, _, state = O.li_prefill(x2[..., :L], x1[..., :L], v[..., :L], lp, r, Db)
+    out_full, y32_full, _ = O.li_prefill(x2, x1, v, lp, r, Db)
+    for i in range(n_dec):
+        y, state = O.step_iir(x2[..., L + i], x1[..., L + i], v[..., L + i], Db, r, lp, state)
+        yr = y.real if y.is_complex() else y
+        x1v = (x1[..., L + i] * v[..., L + i])
+        exp = x2[..., L + i].float() * (y32_full[..., L + i] + Db.float() * x1v.float())
+        assert (yr.float() - exp).abs().max() <= 2e-2 * exp.abs().max()
+    s_ref = O.modal_state_closed_form(x1 * v, lp)
+    assert (state.to(s_ref.dtype) - s_ref).abs().max() <= 1e-4 * s_ref.abs().max()
