@@ -1,0 +1,115 @@
+/* C ABI of libhyena_mi355x.so: hand-written gfx950 kernels for the Hyena
+ * operator hot path (Hyena-SE / MR / LI prefill and the cached decode step).
+ *
+ * Conventions (they mirror the reference's own native launcher,
+ * vortex/ops/conv/csrc/step_fir.cu:94-109, and its pybind glue,
+ * vortex/ops/conv/csrc/causal_conv1d.cpp:139-225):
+ *   - plain pointers, 64-bit sizes, a hipStream_t passed as void*;
+ *   - inputs are borrowed, outputs and state are caller-allocated device memory;
+ *   - a NULL optional pointer means "absent";
+ *   - every call only enqueues work on `stream` (no sync, no allocation, no host threads);
+ *   - return 0 on success, a negative HYENA_E* for a rejected argument,
+ *     a positive hipError_t if the launch failed; hyena_last_error_string()
+ *     describes the last failure on the calling thread.
+ * All activation tensors are bfloat16.  Filters, biases, poles are float32.
+ */
+#ifndef HYENA_MI355X_H
+#define HYENA_MI355X_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HYENA_EINVAL  (-1)   /* bad shape / size / enum                         */
+#define HYENA_EALIGN  (-2)   /* pointer or stride not aligned as required       */
+#define HYENA_ENOSUP  (-3)   /* valid request this build has no kernel for      */
+
+/* One gate operand of the [B, 3D, L] projection, seen as D rows of L samples.
+ * Channel d of batch b starts at
+ *   ptr + b*batch_stride + ((d / ch_inner)*ch_outer + d % ch_inner)*row_stride
+ * (all in elements).  A plain `u.split(D, dim=1)` has ch_inner = D; the
+ * head-blocked column_split of vortex/model/utils.py:41-85 has
+ * ch_inner = head_dim, ch_outer = 3*head_dim.  Samples of a row are contiguous. */
+typedef struct hyena_rows {
+    const void* ptr;
+    int64_t batch_stride;
+    int64_t row_stride;
+    int64_t ch_inner;
+    int64_t ch_outer;
+} hyena_rows;
+
+enum hyena_bias_mode {
+    HYENA_BIAS_NONE = 0,
+    HYENA_BIAS_ADD = 1,         /* z = bf16(bf16(conv) + bias[d])      vortex/model/engine.py:222-223 */
+    HYENA_BIAS_GATED_FP32 = 2   /* z = bf16(conv + bias[d]*u) in fp32  vortex/model/engine.py:78      */
+};
+
+const char* hyena_version(void);
+const char* hyena_last_error_string(void);
+
+/* Hyena-SE: gated causal depthwise short FIR (2 <= K <= 8), direct form.
+ * Replaces HyenaInferenceEngine.parallel_fir, K < 128 branch
+ * (vortex/model/engine.py:131-260, body :188-232):
+ *   u = bf16(x1*v)            (u = x1 when v == NULL)
+ *   z[t] = bf16( sum_k taps[g][k] * u[t-(K-1)+k] )   fp32 accumulate, zero left pad,
+ *                                                    taps[g][K-1] on the current sample
+ *   z = bias rule (enum above), out = bf16(x2*z)     (out = z when x2 == NULL)
+ * taps: [G][K] float32, group g covers channels g*D/G .. (g+1)*D/G-1
+ * (repeat_interleave of vortex/model/model.py:261-262).  out: [B][D][L] bf16, contiguous. */
+int hyena_se_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v,
+                 const float* taps, const float* bias, int bias_mode,
+                 void* out, int64_t B, int64_t D, int64_t L, int64_t G, int K,
+                 void* stream);
+
+/* Hyena-MR: gated causal depthwise FIR with 2 <= K <= 128 as a chunked,
+ * block-Toeplitz contraction on bf16 MFMA with fp32 accumulation.
+ * Replaces parallel_fir, K >= 128 branch + fftconv_func
+ * (vortex/model/engine.py:174-187, :38-83); algorithm after the two-pass
+ * Toeplitz form of vortex/ops/hyena_se/ref_fwd.py:216-266:
+ *   u = bf16(x1*v);  y[t] = sum_k h[g][k] * u[t-k]   (true convolution, h[g][0] on the current sample)
+ *   z = bias rule;   out = bf16(x2*z)
+ * With taps_reversed != 0 the filter is read in the SE orientation instead
+ * (h[g][K-1] on the current sample).  Requires D/G to be a multiple of 16 and
+ * L, strides multiples of 8.  out: [B][D][L] bf16. */
+int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v,
+                 const float* h, int taps_reversed, const float* bias, int bias_mode,
+                 void* out, int64_t B, int64_t D, int64_t L, int64_t G, int K,
+                 void* stream);
+
+/* Decode FIR step on a ring-buffer cache.  Replaces HyenaInferenceEngine.step_fir
+ * (vortex/model/engine.py:406-449; native precedent vortex/ops/conv/csrc/step_fir.cu:13-109)
+ * fused with the caller's gates (vortex/model/model.py:352, :359):
+ *   u = bf16(x1*v)                       (u = x1 when v == NULL)
+ *   y = w[g][R]*u + sum_{i<R} w[g][i]*state_i      state_i = i-th oldest cached input
+ *   y = y + bias[d]*u (bias_mode GATED_FP32) | y + bias[d] (ADD) ; y = bf16(y)
+ *   out = bf16(y*x2)                     (out = y when x2 == NULL)
+ *   the oldest slot is overwritten with u.
+ * ring: [B][R][D] bf16, slot (pos+i) % R holds the i-th oldest input, so the
+ * caller passes pos and afterwards uses (pos+1) % R.  w: [G][R+1] float32, the
+ * taps already sliced/flipped as engine.py:421-425 does, oldest first.
+ * x1, x2, v, out: [B][D] bf16 with the given batch strides (elements). */
+int hyena_fir_step(const void* x1, const void* x2, const void* v, int64_t in_batch_stride,
+                   void* ring, int64_t R, int64_t pos,
+                   const float* w, const float* bias, int bias_mode,
+                   void* out, int64_t out_batch_stride,
+                   int64_t B, int64_t D, int64_t G, void* stream);
+
+/* Decode modal IIR step.  Replaces HyenaInferenceEngine.step_iir
+ * (vortex/model/engine.py:451-467):
+ *   x1v = bf16(x1*v); state = p*state + x1v; y = x2*(Re sum_s r_s*state_s + Dcoef*x1v)
+ * state: [B][D][S] float32 (is_complex == 0) or [B][D][S][2] (re, im) float32, updated in place.
+ * poles (already exponentiated) and residues: [G][S] or [G][S][2] float32.
+ * Dcoef: [D] float32; d_is_bf16 != 0 rounds Dcoef*x1v to bf16 as a bf16 parameter does.
+ * out: [B][D] bf16 (out_is_fp32 == 0) or float32. */
+int hyena_iir_step(const void* x1, const void* x2, const void* v, int64_t in_batch_stride,
+                   float* state, const float* poles, const float* residues, int is_complex,
+                   const float* Dcoef, int d_is_bf16,
+                   void* out, int out_is_fp32, int64_t out_batch_stride,
+                   int64_t B, int64_t D, int64_t G, int64_t S, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HYENA_MI355X_H */

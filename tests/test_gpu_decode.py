@@ -1,0 +1,99 @@
+"""GPU parity of the decode-step kernels against the CPU oracle and the committed
+reference vectors (tests/golden/decode_steps.npz), through the C ABI."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import vortex_amd as va
+from oracle import hyena_oracle as O
+
+pytestmark = pytest.mark.gpu
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "decode_steps.npz"))
+
+
+def eff_taps(weight, cache, flip):
+    """Slicing of vortex/model/engine.py:417-425, as [G, cache+1] oldest tap first."""
+    w = weight.reshape(weight.shape[0], -1)
+    return (w.flip(-1)[..., -cache - 1:] if flip else w[..., : cache + 1]).contiguous()
+
+
+@pytest.mark.parametrize("name", ["se", "mr", "feat", "partial", "partial_flip"])
+def test_fir_step_golden(name):
+    K, cache, flip, gated, _, _ = GOLD[f"fir_{name}_meta"].tolist()
+    u = torch.from_numpy(GOLD[f"fir_{name}_u"]).bfloat16()
+    st = torch.from_numpy(GOLD[f"fir_{name}_state"]).bfloat16()
+    w = torch.from_numpy(GOLD[f"fir_{name}_w"])
+    bias = torch.from_numpy(GOLD[f"fir_{name}_bias"]) if f"fir_{name}_bias" in GOLD else None
+    ring = va.FirRing.from_reference(st.cuda())
+    y = va.fir_step(u.cuda(), ring, eff_taps(w, cache, flip).cuda(), bias=None if bias is None else bias.cuda(),
+                    gated_bias=bool(gated))
+    ye = torch.from_numpy(GOLD[f"fir_{name}_y"])
+    assert (y.float().cpu() - ye).abs().max() <= 2e-2 * ye.abs().max()
+    # cache after the step: reference appends while the cache is short, ring keeps its depth
+    exp_state = torch.from_numpy(GOLD[f"fir_{name}_state_out"])[..., -cache:]
+    assert torch.equal(ring.reference_order().cpu(), exp_state)
+
+
+@pytest.mark.parametrize("B,D,G,K,flip,gated", [
+    (4, 512, 32, 7, False, False),       # SE: dg = 16
+    (3, 1024, 64, 128, True, True),      # MR
+    (2, 1536, 1536, 3, False, False),    # featurizer: per-channel taps over 3D channels
+    (2, 520, 65, 128, True, True),       # D not a multiple of the 512-channel block
+])
+def test_fir_step_sequence_vs_oracle(B, D, G, K, flip, gated):
+    g = torch.Generator().manual_seed(K + D)
+    R = K - 1
+    w = torch.randn(G, 1, K, generator=g) / K ** 0.5
+    wD = w.repeat_interleave(D // G, 0)
+    bias = torch.randn(D, generator=g) if gated else None
+    st = torch.randn(B, D, R, generator=g).bfloat16()
+    ring = va.FirRing.from_reference(st.cuda())
+    taps = eff_taps(w, R, flip).cuda()
+    ref_state = st
+    for step in range(R + 3):            # wraps the ring at least once
+        x1, x2, v = (torch.randn(B, D, generator=g).bfloat16() for _ in range(3))
+        y_ref, ref_state = O.step_fir(x1 * v, ref_state, wD, bias=bias, gated_bias=gated, flip_filter=flip)
+        y_ref = y_ref * x2
+        y = va.fir_step(x1.cuda(), ring, taps, x2=x2.cuda(), v=v.cuda(), bias=None if bias is None else bias.cuda(),
+                        gated_bias=gated)
+        err = (y.float().cpu() - y_ref.float()).abs().max() / y_ref.float().abs().max()
+        assert err <= 2e-2, (step, err)
+        if step in (0, R - 1, R + 2):
+            assert torch.equal(ring.reference_order().cpu(), ref_state)
+
+
+@pytest.mark.parametrize("name", ["real_bf16D", "real_f32D", "cplx_f32D"])
+def test_iir_step_golden(name):
+    x2, x1, v = (torch.from_numpy(GOLD[f"iir_{name}_{k}"]).bfloat16().cuda() for k in ("x2", "x1", "v"))
+    Dp = torch.from_numpy(GOLD[f"iir_{name}_D"])
+    if "bf16D" in name:
+        Dp = Dp.bfloat16()
+    lp, r, st = (torch.from_numpy(GOLD[f"iir_{name}_{k}"]) for k in ("lp", "r", "state"))
+    state = st.clone().cuda()
+    y = va.iir_step(x1, x2, v, state, torch.exp(lp[..., 0]).cuda(), r.cuda(), Dp.cuda(), out_dtype=torch.float32)
+    ye = torch.from_numpy(GOLD[f"iir_{name}_y"])
+    ye = ye.real if ye.is_complex() else ye
+    se = torch.from_numpy(GOLD[f"iir_{name}_state_out"])
+    assert (y.cpu() - ye).abs().max() <= 1e-5 * ye.abs().max()
+    assert (state.cpu() - se).abs().max() <= 1e-5 * se.abs().max()
+
+
+@pytest.mark.parametrize("cplx,G", [(False, 256), (True, 256), (True, 16), (False, 1)])
+def test_iir_step_sequence_vs_oracle(cplx, G):
+    B, D, S = 5, 256, 16
+    g = torch.Generator().manual_seed(3)
+    lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(G, S, seed=4)
+    Dp = torch.randn(D, generator=g).bfloat16()
+    lpD, rD = lp.repeat_interleave(D // G, 0), r.repeat_interleave(D // G, 0)
+    st_ref = torch.zeros(B, D, S, dtype=torch.complex64 if cplx else torch.float32)
+    state = st_ref.clone().cuda()
+    poles = torch.exp(lp[..., 0]).cuda()
+    for step in range(20):
+        x1, x2, v = (torch.randn(B, D, generator=g).bfloat16() for _ in range(3))
+        y_ref, st_ref = O.step_iir(x2, x1, v, Dp, rD, lpD, st_ref)
+        y_ref = (y_ref.real if cplx else y_ref).to(torch.bfloat16)
+        y = va.iir_step(x1.cuda(), x2.cuda(), v.cuda(), state, poles, r.cuda(), Dp.cuda())
+        assert (y.float().cpu() - y_ref.float()).abs().max() <= 2e-2 * y_ref.float().abs().max()
+    assert (state.cpu() - st_ref).abs().max() <= 1e-4 * st_ref.abs().max()

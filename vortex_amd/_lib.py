@@ -1,0 +1,66 @@
+"""ctypes binding of libhyena_mi355x.so (the C ABI declared in include/hyena_mi355x.h).
+
+There is no fallback: if the library is missing, every operator raises.
+"""
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int64, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhyena_mi355x.so")
+
+HYENA_BIAS_NONE, HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32 = 0, 1, 2
+
+EXPORTS = [
+    "hyena_version", "hyena_last_error_string", "hyena_se_fwd", "hyena_mr_fwd",
+    "hyena_fir_step", "hyena_iir_step",
+]
+
+
+class Rows(Structure):
+    _fields_ = [("ptr", c_void_p), ("batch_stride", c_int64), ("row_stride", c_int64),
+                ("ch_inner", c_int64), ("ch_outer", c_int64)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is not built; run `python -m vortex_amd.build` (hipcc, gfx950). "
+            "There is no CPU or PyTorch fallback for the Hyena kernels.")
+    L = ctypes.CDLL(LIB_PATH)
+    L.hyena_version.restype = c_char_p
+    L.hyena_last_error_string.restype = c_char_p
+    R = POINTER(Rows)
+    L.hyena_se_fwd.argtypes = [R, R, R, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                               c_int, c_void_p]
+    L.hyena_mr_fwd.argtypes = [R, R, R, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64,
+                               c_int64, c_int, c_void_p]
+    L.hyena_fir_step.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p,
+                                 c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p]
+    L.hyena_iir_step.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int,
+                                 c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                 c_void_p]
+    for name in EXPORTS:
+        fn = getattr(L, name)
+        if name not in ("hyena_version", "hyena_last_error_string"):
+            fn.restype = c_int
+    _lib = L
+    return L
+
+
+def check(rc, what):
+    """Turns a non-zero return code into the exception TORCH_CHECK would have raised."""
+    if rc == 0:
+        return
+    msg = lib().hyena_last_error_string().decode()
+    if rc == -3:
+        raise NotImplementedError(msg or what)
+    if rc < 0:
+        raise ValueError(msg or what)
+    raise RuntimeError(msg or f"{what}: hipError {rc}")

@@ -1,0 +1,59 @@
+// Shared device/host helpers for the gfx950 Hyena kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/hyena_mi355x.h"
+
+typedef unsigned short bf16_t;                                   // raw bfloat16 bits
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2;
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+
+// bf16 <-> fp32.  Widening is a shift; narrowing is round-to-nearest-even,
+// the rounding torch applies when it casts float32 to bfloat16.
+__device__ __forceinline__ float bf_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__device__ __forceinline__ float bf_to_f(bf16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+
+__device__ __forceinline__ uint32_t f_to_bf_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;    // NaN stays NaN
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float round_bf(float f) { return __uint_as_float(f_to_bf_bits(f) << 16); }
+__device__ __forceinline__ uint32_t pack_bf2(float lo, float hi) {
+    return f_to_bf_bits(lo) | (f_to_bf_bits(hi) << 16);
+}
+
+struct RowMap {            // device copy of hyena_rows
+    const bf16_t* ptr;
+    int64_t batch_stride, row_stride, ch_inner, ch_outer;
+    __device__ __forceinline__ const bf16_t* row(int64_t b, int64_t d) const {
+        int64_t r = (d / ch_inner) * ch_outer + (d % ch_inner);
+        return ptr + b * batch_stride + r * row_stride;
+    }
+};
+
+static inline RowMap make_rowmap(const hyena_rows* r) {
+    RowMap m;
+    if (r) { m.ptr = (const bf16_t*)r->ptr; m.batch_stride = r->batch_stride; m.row_stride = r->row_stride;
+             m.ch_inner = r->ch_inner; m.ch_outer = r->ch_outer; }
+    else   { m.ptr = nullptr; m.batch_stride = m.row_stride = 0; m.ch_inner = m.ch_outer = 1; }
+    return m;
+}
+
+// error reporting shared by all entry points (api.hip owns the buffer)
+int hyena_fail(int code, const char* fmt, ...);
+int hyena_check_launch(const char* what);
+
+static inline bool rows_aligned8(const hyena_rows* r) {
+    return r == nullptr || ((((uintptr_t)r->ptr) & 15) == 0 && r->batch_stride % 8 == 0 && r->row_stride % 8 == 0);
+}
+static inline bool rows_valid(const hyena_rows* r, int64_t D) {
+    return r->ptr != nullptr && r->ch_inner > 0 && r->ch_outer >= 0 && D % r->ch_inner == 0 || (r->ch_inner >= D);
+}

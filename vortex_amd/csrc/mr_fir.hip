@@ -1,0 +1,263 @@
+// Hyena-MR: gated causal depthwise FIR, K <= 128, as a block-Toeplitz
+// contraction on bf16 MFMA (v_mfma_f32_32x32x16_bf16) with fp32 accumulation.
+//
+// For 32 output samples starting at T and filter lags 0..127 the inputs are the
+// ten 16-sample blocks that start at T-128+16m, m = 0..9, and the 32x16
+// Toeplitz block that weights block m, A_m[i][j] = h[i - j + 128 - 16m], does
+// not depend on T.  A wavefront therefore keeps all ten A_m of its filter group
+// in registers for the whole kernel and streams u = bf16(x1*v) through the B
+// operand.  The MFMA N dimension (32 columns) is 16 channels of the group x 2
+// time offsets.  This is the two-pass chunked Toeplitz form of
+// vortex/ops/hyena_se/ref_fwd.py:216-266 with the all-zero blocks of T and T^
+// dropped and the two passes merged into one accumulator.
+//
+// Data path per 512-sample step of a block (4 wavefronts, 16 channels):
+//   global (coalesced 16 B/lane) -> u = bf16(x1*v) -> LDS row-major [16][128+512]
+//   -> B fragments (ds_read_b128) -> MFMA -> z = bf16(acc + D*u) -> LDS
+//   -> coalesced read, * x2, 16 B/lane store.
+// The 128-sample tail of a step stays in LDS as the next step's halo, so each
+// input is read from HBM once per segment.
+#include "common.h"
+
+namespace {
+
+constexpr int TL = 512;        // samples per step
+constexpr int HALO = 128;      // samples kept from the previous step
+constexpr int URS = 648;       // u_lds row stride (elements): 1296 B = 16 * 81
+constexpr int ZRS = 520;       // z_lds row stride (elements): 1040 B = 16 * 65
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) {
+    union { u32x4 u; bf16x8 b; } c;
+    c.u = x;
+    return c.b;
+}
+
+template <bool PRE>
+__device__ __forceinline__ u32x4 gate_mul(u32x4 a, u32x4 b) {
+    if (!PRE) return a;
+    u32x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = pack_bf2(bf_lo(a[j]) * bf_lo(b[j]), bf_hi(a[j]) * bf_hi(b[j]));
+    return r;
+}
+
+template <bool PRE, bool POST, int BIAS>
+__global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, RowMap v, const float* __restrict__ h,
+                                                        int K, int reversed, const float* __restrict__ bias,
+                                                        bf16_t* __restrict__ out, int64_t D, int64_t L, int dg,
+                                                        int64_t seg_len, int nseg) {
+    __shared__ __attribute__((aligned(16))) bf16_t u_lds[16 * URS];
+    __shared__ __attribute__((aligned(16))) bf16_t z_lds[16 * ZRS];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t nslab = D / 16;
+    const int64_t bid = blockIdx.x;
+    const int seg = (int)(bid % nseg);
+    const int64_t slab = (bid / nseg) % nslab;
+    const int64_t b = bid / ((int64_t)nseg * nslab);
+    const int64_t d0 = slab * 16;
+    const int g = (int)(d0 / dg);
+
+    // ---- Toeplitz fragments of this group's filter (A operand, 32 x 16 each)
+    const int n = lane & 31, hh = lane >> 5;
+    // accumulator register r of lane (n, hh) is MFMA row 8*(r/4) + 4*hh + r%4; feeding the
+    // A rows in the order below makes that lane own the 16 consecutive samples 16*hh + r.
+    const int i_time = 16 * ((n >> 2) & 1) + 4 * (n >> 3) + (n & 3);
+    bf16x8 A[10];
+    const int m_min = (114 - K) > 0 ? (114 - K + 15) / 16 : 0;     // blocks below m_min are all zero
+#pragma unroll
+    for (int m = 0; m < 10; ++m) {
+        u32x4 pk;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float t[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int lag = i_time - (8 * hh + 2 * j + e) + 128 - 16 * m;
+                float val = 0.f;
+                if (lag >= 0 && lag < K) val = h[g * K + (reversed ? K - 1 - lag : lag)];
+                t[e] = val;
+            }
+            pk[j] = pack_bf2(t[0], t[1]);
+        }
+        A[m] = as_bf16x8(pk);
+    }
+
+    // ---- coalesced layout: this thread moves 16 B of rows 4*r4 + w, r4 = 0..3
+    const bf16_t *p1[4], *pv[4], *p2[4];
+    bf16_t* po[4];
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+        const int64_t d = d0 + 4 * r4 + w;
+        p1[r4] = x1.row(b, d) + lane * 8;
+        pv[r4] = PRE ? v.row(b, d) + lane * 8 : nullptr;
+        p2[r4] = POST ? x2.row(b, d) + lane * 8 : nullptr;
+        po[r4] = out + (b * D + d) * L + lane * 8;
+    }
+    const int64_t t_begin = (int64_t)seg * seg_len;
+    const int64_t t_end = (t_begin + seg_len < L) ? t_begin + seg_len : L;
+    if (t_begin >= t_end) return;
+
+    // ---- halo of the segment: the 128 samples before t_begin (zeros at the sequence start)
+    {
+        const int ch = tid >> 4, tt = (tid & 15) * 8;
+        u32x4 hu = {0, 0, 0, 0};
+        if (t_begin > 0) {
+            const u32x4 a = *(const u32x4*)(x1.row(b, d0 + ch) + t_begin - HALO + tt);
+            u32x4 c = {0, 0, 0, 0};
+            if (PRE) c = *(const u32x4*)(v.row(b, d0 + ch) + t_begin - HALO + tt);
+            hu = gate_mul<PRE>(a, c);
+        }
+        *(u32x4*)(u_lds + ch * URS + tt) = hu;
+    }
+
+    u32x4 c1[4], cv[4];
+    const u32x4 zero4 = {0, 0, 0, 0};
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+        const bool ok = t_begin + lane * 8 < L;
+        c1[r4] = ok ? *(const u32x4*)(p1[r4] + t_begin) : zero4;
+        cv[r4] = (PRE && ok) ? *(const u32x4*)(pv[r4] + t_begin) : zero4;
+    }
+
+    float bz = 0.f;
+    if (BIAS != HYENA_BIAS_NONE) bz = bias[d0 + (n & 15)];
+
+    for (int64_t ts = t_begin; ts < t_end; ts += TL) {
+        // u of this step -> LDS
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4)
+            *(u32x4*)(u_lds + (4 * r4 + w) * URS + HALO + lane * 8) = gate_mul<PRE>(c1[r4], cv[r4]);
+        __syncthreads();
+
+        // prefetch: next step's x1, v; this step's x2
+        u32x4 c2[4];
+        {
+            const int64_t tn = ts + TL;
+            const bool okn = (tn < t_end) && (tn + lane * 8 < L);
+            const bool okc = ts + lane * 8 < L;
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                c1[r4] = okn ? *(const u32x4*)(p1[r4] + tn) : zero4;
+                cv[r4] = (PRE && okn) ? *(const u32x4*)(pv[r4] + tn) : zero4;
+                c2[r4] = (POST && okc) ? *(const u32x4*)(p2[r4] + ts) : zero4;
+            }
+        }
+        // tail of this step = halo of the next one (read now, written after the MFMA phase)
+        const u32x4 tail = *(const u32x4*)(u_lds + (tid >> 4) * URS + TL + (tid & 15) * 8);
+
+        // ---- MFMA phase: wavefront w owns output blocks 2w, 2w+1 (+8 for the upper 16 columns)
+        const int c = n & 15, s = n >> 4;
+        f32x16 acc0, acc1;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
+        const bf16_t* ub = u_lds + c * URS + 64 * w + 256 * s + 8 * hh;
+#pragma unroll
+        for (int mm = 0; mm < 12; ++mm) {
+            const bf16x8 bf = *(const bf16x8*)(ub + 16 * mm);
+            if (mm <= 9 && mm >= m_min) acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm <= 9 ? mm : 0], bf, acc0, 0, 0, 0);
+            if (mm >= 2 && mm - 2 >= m_min) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm >= 2 ? mm - 2 : 0], bf, acc1, 0, 0, 0);
+        }
+        // ---- z = bf16(acc [+ D*u]) -> LDS, 16 consecutive samples per lane and tile
+#pragma unroll
+        for (int tau = 0; tau < 2; ++tau) {
+            const int tcol = 64 * w + 32 * tau + 256 * s + 16 * hh;
+            const f32x16 acc = tau ? acc1 : acc0;
+            u32x4 ua = {0, 0, 0, 0}, ub2 = {0, 0, 0, 0};
+            if (BIAS == HYENA_BIAS_GATED_FP32) {
+                ua = *(const u32x4*)(u_lds + c * URS + HALO + tcol);
+                ub2 = *(const u32x4*)(u_lds + c * URS + HALO + tcol + 8);
+            }
+            u32x4 z0, z1;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float a0 = acc[2 * j], a1 = acc[2 * j + 1];
+                if (BIAS == HYENA_BIAS_GATED_FP32) {
+                    const uint32_t uw = j < 4 ? ua[j] : ub2[j - 4];
+                    a0 = fmaf(bz, bf_lo(uw), a0);
+                    a1 = fmaf(bz, bf_hi(uw), a1);
+                }
+                if (BIAS == HYENA_BIAS_ADD) {
+                    a0 = round_bf(a0) + bz;
+                    a1 = round_bf(a1) + bz;
+                }
+                const uint32_t p = pack_bf2(a0, a1);
+                if (j < 4) z0[j] = p; else z1[j - 4] = p;
+            }
+            *(u32x4*)(z_lds + c * ZRS + tcol) = z0;
+            *(u32x4*)(z_lds + c * ZRS + tcol + 8) = z1;
+        }
+        __syncthreads();
+
+        *(u32x4*)(u_lds + (tid >> 4) * URS + (tid & 15) * 8) = tail;
+        // ---- gate with x2 and store, coalesced
+        if (ts + lane * 8 < t_end) {
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const u32x4 zz = *(const u32x4*)(z_lds + (4 * r4 + w) * ZRS + lane * 8);
+                u32x4 o = zz;
+                if (POST) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(c2[r4][j]), bf_hi(zz[j]) * bf_hi(c2[r4][j]));
+                }
+                *(u32x4*)(po[r4] + ts) = o;
+            }
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const float* h,
+                            int taps_reversed, const float* bias, int bias_mode, void* out, int64_t B, int64_t D,
+                            int64_t L, int64_t G, int K, void* stream) {
+    if (!x1 || !x1->ptr || !h || !out) return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: x1, h and out are required");
+    if (B < 0 || D <= 0 || L < 0 || G <= 0 || D % G != 0)
+        return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: bad sizes B=%lld D=%lld L=%lld G=%lld", (long long)B,
+                          (long long)D, (long long)L, (long long)G);
+    if (K < 1 || K > 128) return hyena_fail(HYENA_ENOSUP, "hyena_mr_fwd: K=%d outside 1..128", K);
+    if ((D / G) % 16 != 0)
+        return hyena_fail(HYENA_ENOSUP, "hyena_mr_fwd: D/G=%lld must be a multiple of 16", (long long)(D / G));
+    if (bias_mode < 0 || bias_mode > 2 || (bias_mode != HYENA_BIAS_NONE && !bias))
+        return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: bias_mode %d needs a bias pointer", bias_mode);
+    if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15))
+        return hyena_fail(HYENA_EALIGN, "hyena_mr_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
+    if (B == 0 || L == 0) return 0;
+    const bool pre = v && v->ptr, post = x2 && x2->ptr;
+
+    // segments along L: enough blocks to fill 256 CUs a few times over, segments >= 2048 samples
+    const int64_t rows = B * (D / 16);
+    int64_t nseg = (3072 + rows - 1) / rows;
+    const int64_t max_seg = (L + 2047) / 2048;
+    if (nseg > max_seg) nseg = max_seg;
+    if (nseg < 1) nseg = 1;
+    if (const char* e = getenv("HYENA_MR_NSEG")) { int64_t x = atoll(e); if (x >= 1) nseg = x; }
+    int64_t seg_len = (L + nseg - 1) / nseg;
+    seg_len = (seg_len + TL - 1) / TL * TL;
+    nseg = (L + seg_len - 1) / seg_len;
+    const int64_t nblk = rows * nseg;
+    if (nblk > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: problem too large for one launch");
+
+    RowMap m1 = make_rowmap(x1), m2 = make_rowmap(post ? x2 : nullptr), mv = make_rowmap(pre ? v : nullptr);
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((unsigned)nblk);
+    const int dg = (int)(D / G);
+    bool ok = false;
+#define MR_CASE(P, Q, M)                                                                                      \
+    if (pre == P && post == Q && bias_mode == M) {                                                            \
+        hipLaunchKernelGGL((mr_fir_kernel<P, Q, M>), grid, dim3(256), 0, s, m1, m2, mv, h, K, taps_reversed,  \
+                           bias, (bf16_t*)out, D, L, dg, seg_len, (int)nseg);                                 \
+        ok = true;                                                                                            \
+    }
+    MR_CASE(true, true, HYENA_BIAS_GATED_FP32)
+    MR_CASE(true, true, HYENA_BIAS_NONE)
+    MR_CASE(true, true, HYENA_BIAS_ADD)
+    MR_CASE(false, false, HYENA_BIAS_NONE)
+    MR_CASE(false, false, HYENA_BIAS_ADD)
+    MR_CASE(false, false, HYENA_BIAS_GATED_FP32)
+#undef MR_CASE
+    if (!ok) return hyena_fail(HYENA_ENOSUP, "hyena_mr_fwd: this gate/bias combination has no kernel");
+    return hyena_check_launch("hyena_mr_fwd");
+}

@@ -1,0 +1,193 @@
+// Hyena-SE: gated causal depthwise short FIR, direct form, HBM-bound.
+//
+// One lane owns 8 consecutive samples of one (batch, channel) row: three 16-byte
+// loads (x1, v, x2), one 16-byte store.  The K-1 samples a lane needs from
+// before its octet come from the neighbouring lane through a wavefront shuffle;
+// only lane 0 of a wavefront (or the first octet of a row) touches memory again
+// for them.  Accumulation is fp32; the two roundings to bf16 are where
+// vortex/model/engine.py:159 and :208 put them.
+#include "common.h"
+
+namespace {
+
+template <int K, bool PRE, bool POST, int BIAS, bool ROWU>
+__global__ __launch_bounds__(256) void se_fir_kernel(RowMap x1, RowMap x2, RowMap v,
+                                                     const float* __restrict__ taps,
+                                                     const float* __restrict__ bias,
+                                                     bf16_t* __restrict__ out,
+                                                     int64_t D, int64_t L, int dg,
+                                                     int64_t octs_per_row, int64_t total_octs) {
+    constexpr int H = K - 1;                 // halo samples
+    constexpr int HD = (H + 1) / 2;          // halo dwords taken from the previous lane
+    int64_t row, oct;
+    if (ROWU) {                              // a block never straddles rows: row is wave-uniform
+        const int64_t blocks_per_row = octs_per_row / 256;
+        row = blockIdx.x / blocks_per_row;
+        oct = (blockIdx.x - row * blocks_per_row) * 256 + threadIdx.x;
+    } else {
+        const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        row = idx / octs_per_row;
+        oct = idx - row * octs_per_row;
+    }
+    const bool active = ROWU ? true : (row * octs_per_row + oct < total_octs);
+    if (!active) { row = 0; oct = 0; }
+    const int64_t b = row / D, d = row - b * D;
+    const int64_t t0 = oct * 8;
+    const int g = (int)(d / dg);
+
+    float w[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) w[k] = taps[g * K + k];
+
+    const bf16_t* p1 = x1.row(b, d) + t0;
+    const u32x4 a1 = *(const u32x4*)p1;
+    u32x4 av = {0, 0, 0, 0}, a2 = {0, 0, 0, 0};
+    if (PRE) av = *(const u32x4*)(v.row(b, d) + t0);
+    if (POST) a2 = *(const u32x4*)(x2.row(b, d) + t0);
+
+    // u = bf16(x1*v), kept both as floats and as packed bf16 pairs
+    float u[8];
+    uint32_t pk[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (PRE) {
+            const uint32_t lo = f_to_bf_bits(bf_lo(a1[j]) * bf_lo(av[j]));
+            const uint32_t hi = f_to_bf_bits(bf_hi(a1[j]) * bf_hi(av[j]));
+            pk[j] = lo | (hi << 16);
+        } else {
+            pk[j] = a1[j];
+        }
+        u[2 * j] = bf_lo(pk[j]);
+        u[2 * j + 1] = bf_hi(pk[j]);
+    }
+
+    // halo: last HD dwords of the previous lane's octet
+    uint32_t hp[HD];
+#pragma unroll
+    for (int j = 0; j < HD; ++j) hp[j] = __shfl_up(pk[4 - HD + j], 1, 64);
+    const int lane = threadIdx.x & 63;
+    if (lane == 0 || oct == 0) {
+        if (oct == 0) {
+#pragma unroll
+            for (int j = 0; j < HD; ++j) hp[j] = 0;          // zero left padding
+        } else {
+            const u32x4 h1 = *(const u32x4*)(p1 - 8);
+            u32x4 hv = {0, 0, 0, 0};
+            if (PRE) hv = *(const u32x4*)(v.row(b, d) + t0 - 8);
+#pragma unroll
+            for (int j = 0; j < HD; ++j) {
+                const int q = 4 - HD + j;
+                if (PRE) {
+                    const uint32_t lo = f_to_bf_bits(bf_lo(h1[q]) * bf_lo(hv[q]));
+                    const uint32_t hi = f_to_bf_bits(bf_hi(h1[q]) * bf_hi(hv[q]));
+                    hp[j] = lo | (hi << 16);
+                } else {
+                    hp[j] = h1[q];
+                }
+            }
+        }
+    }
+
+    // ext = [K-1 halo samples | 8 own samples]
+    float ext[H + 8];
+#pragma unroll
+    for (int i = 0; i < H; ++i) {
+        const int e = 2 * HD - H + i;                      // element inside hp[] (skip one if H is odd)
+        ext[i] = (e & 1) ? bf_hi(hp[e >> 1]) : bf_lo(hp[e >> 1]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ext[H + i] = u[i];
+
+    float bz = 0.f;
+    if (BIAS != HYENA_BIAS_NONE) bz = bias[d];
+
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float z[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int i = 2 * j + e;
+            float acc = 0.f;
+#pragma unroll
+            for (int k = 0; k < K; ++k) acc = fmaf(w[k], ext[i + k], acc);
+            if (BIAS == HYENA_BIAS_GATED_FP32) acc = fmaf(bz, u[i], acc);
+            acc = round_bf(acc);
+            if (BIAS == HYENA_BIAS_ADD) acc = round_bf(acc + bz);
+            if (POST) acc = acc * (e ? bf_hi(a2[j]) : bf_lo(a2[j]));
+            z[e] = acc;
+        }
+        o[j] = pack_bf2(z[0], z[1]);
+    }
+    if (active) {
+        u32x4 ov = {o[0], o[1], o[2], o[3]};
+        *(u32x4*)(out + row * L + t0) = ov;
+    }
+}
+
+template <int K, bool PRE, bool POST, int BIAS>
+void launch_k(bool rowu, dim3 grid, hipStream_t s, RowMap x1, RowMap x2, RowMap v, const float* taps,
+              const float* bias, bf16_t* out, int64_t D, int64_t L, int dg, int64_t opr, int64_t tot) {
+    if (rowu)
+        hipLaunchKernelGGL((se_fir_kernel<K, PRE, POST, BIAS, true>), grid, dim3(256), 0, s, x1, x2, v, taps, bias,
+                           out, D, L, dg, opr, tot);
+    else
+        hipLaunchKernelGGL((se_fir_kernel<K, PRE, POST, BIAS, false>), grid, dim3(256), 0, s, x1, x2, v, taps, bias,
+                           out, D, L, dg, opr, tot);
+}
+
+template <int K>
+bool launch_gates(bool pre, bool post, int bias_mode, bool rowu, dim3 grid, hipStream_t s, RowMap x1, RowMap x2,
+                  RowMap v, const float* taps, const float* bias, bf16_t* out, int64_t D, int64_t L, int dg,
+                  int64_t opr, int64_t tot) {
+#define SE_CASE(P, Q, M)                                                                                    \
+    if (pre == P && post == Q && bias_mode == M) {                                                          \
+        launch_k<K, P, Q, M>(rowu, grid, s, x1, x2, v, taps, bias, out, D, L, dg, opr, tot);                \
+        return true;                                                                                        \
+    }
+    SE_CASE(true, true, HYENA_BIAS_NONE)
+    SE_CASE(false, false, HYENA_BIAS_NONE)
+    SE_CASE(false, false, HYENA_BIAS_ADD)
+    SE_CASE(true, true, HYENA_BIAS_ADD)
+    SE_CASE(true, true, HYENA_BIAS_GATED_FP32)
+    SE_CASE(true, false, HYENA_BIAS_NONE)
+    SE_CASE(false, true, HYENA_BIAS_NONE)
+    SE_CASE(false, false, HYENA_BIAS_GATED_FP32)
+#undef SE_CASE
+    return false;
+}
+
+}  // namespace
+
+extern "C" int hyena_se_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const float* taps,
+                            const float* bias, int bias_mode, void* out, int64_t B, int64_t D, int64_t L, int64_t G,
+                            int K, void* stream) {
+    if (!x1 || !x1->ptr || !taps || !out) return hyena_fail(HYENA_EINVAL, "hyena_se_fwd: x1, taps and out are required");
+    if (B < 0 || D <= 0 || L < 0 || G <= 0 || D % G != 0)
+        return hyena_fail(HYENA_EINVAL, "hyena_se_fwd: bad sizes B=%lld D=%lld L=%lld G=%lld", (long long)B,
+                          (long long)D, (long long)L, (long long)G);
+    if (K < 2 || K > 8) return hyena_fail(HYENA_ENOSUP, "hyena_se_fwd: K=%d outside 2..8 (use hyena_mr_fwd)", K);
+    if (bias_mode < 0 || bias_mode > 2 || (bias_mode != HYENA_BIAS_NONE && !bias))
+        return hyena_fail(HYENA_EINVAL, "hyena_se_fwd: bias_mode %d needs a bias pointer", bias_mode);
+    if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15))
+        return hyena_fail(HYENA_EALIGN, "hyena_se_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
+    const bool pre = v && v->ptr, post = x2 && x2->ptr;
+    if (B == 0 || L == 0) return 0;
+    const int64_t opr = L / 8, tot = B * D * opr;
+    const bool rowu = (opr % 256 == 0);
+    const int64_t nblk = (tot + 255) / 256;
+    if (nblk > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "hyena_se_fwd: problem too large for one launch");
+    dim3 grid((unsigned)nblk);
+    hipStream_t s = (hipStream_t)stream;
+    RowMap m1 = make_rowmap(x1), m2 = make_rowmap(post ? x2 : nullptr), mv = make_rowmap(pre ? v : nullptr);
+    const int dg = (int)(D / G);
+    bf16_t* o = (bf16_t*)out;
+    bool ok = false;
+    switch (K) {
+#define SE_K(KK) case KK: ok = launch_gates<KK>(pre, post, bias_mode, rowu, grid, s, m1, m2, mv, taps, bias, o, D, L, dg, opr, tot); break;
+        SE_K(2) SE_K(3) SE_K(4) SE_K(5) SE_K(6) SE_K(7) SE_K(8)
+#undef SE_K
+    }
+    if (!ok) return hyena_fail(HYENA_ENOSUP, "hyena_se_fwd: this gate/bias combination has no kernel");
+    return hyena_check_launch("hyena_se_fwd");
+}

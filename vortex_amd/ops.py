@@ -1,0 +1,215 @@
+"""Tensor-level wrappers over the C ABI: shape/dtype checks, row descriptors, stream.
+
+Every function enqueues on torch's current stream and returns torch tensors that
+it allocated; nothing here computes on the CPU or through PyTorch operators.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE, Rows
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("vortex_amd operators run on the GPU only (got a CPU tensor); there is no CPU fallback")
+
+
+def rows_of(t):
+    """Row descriptor of a [B, D, L] bf16 tensor whose samples are contiguous."""
+    if t is None:
+        return None
+    if t.dtype != torch.bfloat16:
+        raise TypeError(f"expected bfloat16 gates, got {t.dtype}")
+    if t.dim() != 3 or (t.shape[2] > 1 and t.stride(2) != 1):
+        raise ValueError("expected a [B, D, L] tensor with contiguous samples")
+    B, D, L = t.shape
+    return Rows(t.data_ptr(), t.stride(0), t.stride(1), D, D)
+
+
+def rows_of_projection(u, hidden, which, head_dim=None):
+    """Row descriptor of gate `which` (0, 1, 2) inside a [B, 3*hidden, L] projection.
+
+    head_dim=None is the plain split of vortex/model/engine.py:156; otherwise the
+    head-blocked column split of vortex/model/utils.py:41-85.
+    """
+    if u.dtype != torch.bfloat16 or u.dim() != 3 or u.stride(2) != 1:
+        raise ValueError("expected a [B, 3D, L] bfloat16 tensor with contiguous samples")
+    es = u.element_size()
+    if head_dim is None:
+        return Rows(u.data_ptr() + which * hidden * u.stride(1) * es, u.stride(0), u.stride(1), hidden, hidden)
+    return Rows(u.data_ptr() + which * head_dim * u.stride(1) * es, u.stride(0), u.stride(1), head_dim, 3 * head_dim)
+
+
+def _ref(r):
+    return ctypes.byref(r) if r is not None else None
+
+
+def _f32(t, shape=None):
+    if t is None:
+        return None
+    t = t.detach()
+    if t.dtype != torch.float32 or not t.is_contiguous():
+        t = t.to(torch.float32).contiguous()
+    return t
+
+
+def _bias_mode(bias, gated, fp32_gated):
+    if bias is None:
+        return HYENA_BIAS_NONE
+    if gated:
+        if not fp32_gated:
+            raise NotImplementedError("gated bias after the bf16 rounding (short-FIR branch) has no kernel")
+        return HYENA_BIAS_GATED_FP32
+    return HYENA_BIAS_ADD
+
+
+def fir_fwd_rows(x1r, x2r, vr, taps, B, D, L, K, *, device, bias=None, bias_mode=HYENA_BIAS_NONE,
+                 taps_reversed=False, force_mfma=False):
+    """Shared launcher of the prefill FIR kernels on row descriptors.
+
+    taps [G, K] float32.  taps_reversed=False means the convolution orientation
+    (taps[:, 0] on the current sample); True means the short-filter orientation of
+    vortex (taps[:, K-1] on the current sample).
+    """
+    taps = _f32(taps)
+    G = taps.shape[0]
+    out = torch.empty((B, D, L), dtype=torch.bfloat16, device=device)
+    L_ = _lib.lib()
+    if K <= 8 and not force_mfma:
+        if not taps_reversed:
+            taps = taps.flip(-1).contiguous()
+        rc = L_.hyena_se_fwd(_ref(x1r), _ref(x2r), _ref(vr), _ptr(taps), _ptr(bias), bias_mode, _ptr(out),
+                             B, D, L, G, K, _stream())
+        _lib.check(rc, "hyena_se_fwd")
+    else:
+        rc = L_.hyena_mr_fwd(_ref(x1r), _ref(x2r), _ref(vr), _ptr(taps), int(taps_reversed), _ptr(bias), bias_mode,
+                             _ptr(out), B, D, L, G, K, _stream())
+        _lib.check(rc, "hyena_mr_fwd")
+    return out
+
+
+def hyena_se_fwd(x1, x2, v, h, bias=None, *, force_mfma=False):
+    """Hyena-SE prefill: out = bf16(x2 * bf16(corr_K(bf16(x1*v)))) on [B, D, L] bf16 gates.
+
+    h: [G, 1, K] or [G, K] float32 in vortex's short-filter orientation (h[..., K-1]
+    multiplies the current sample; vortex/model/engine.py:197-204).  Returns [B, D, L] bf16.
+    """
+    _need_cuda(x1, x2, v, h)
+    B, D, L = x1.shape
+    taps = _f32(h).reshape(h.shape[0], -1)
+    K = taps.shape[1]
+    b = _f32(bias)
+    return fir_fwd_rows(rows_of(x1), rows_of(x2), rows_of(v), taps, B, D, L, K, device=x1.device, bias=b,
+                        bias_mode=_bias_mode(b, False, False), taps_reversed=True, force_mfma=force_mfma)
+
+
+def hyena_mr_fwd(x1, x2, v, h, D_bias=None):
+    """Hyena-MR prefill: out = bf16(x2 * bf16(conv(h, u) + D*u)), u = bf16(x1*v).
+
+    h: [G, 1, K] or [G, K] float32, true-convolution orientation (h[..., 0] on the
+    current sample; vortex/model/engine.py:174-187).  D_bias: [D] or None.
+    """
+    _need_cuda(x1, x2, v, h)
+    B, D, L = x1.shape
+    taps = _f32(h).reshape(h.shape[0], -1)
+    K = taps.shape[1]
+    b = _f32(D_bias)
+    return fir_fwd_rows(rows_of(x1), rows_of(x2), rows_of(v), taps, B, D, L, K, device=x1.device, bias=b,
+                        bias_mode=_bias_mode(b, True, True), taps_reversed=False, force_mfma=True)
+
+
+class FirRing:
+    """Ring-buffer FIR cache [B, R, D] bf16 plus the index of its oldest slot.
+
+    Holds the same samples as the reference's [B, D, R] oldest-first fir_state
+    (vortex/model/engine.py:414, :443-447); reference_order() returns that view.
+    """
+
+    def __init__(self, buf, pos=0):
+        self.buf, self.pos = buf, pos
+
+    @classmethod
+    def from_reference(cls, fir_state):
+        """fir_state: [B, D, R] oldest-first (any float dtype holding bf16-exact values)."""
+        return cls(fir_state.to(torch.bfloat16).permute(0, 2, 1).contiguous(), 0)
+
+    @property
+    def shape(self):   # what engine.step_fir reads as cache size: shape[-1]
+        B, R, D = self.buf.shape
+        return torch.Size((B, D, R))
+
+    def reference_order(self, dtype=torch.float32):
+        R = self.buf.shape[1]
+        idx = (torch.arange(R, device=self.buf.device) + self.pos) % R
+        return self.buf.index_select(1, idx).permute(0, 2, 1).to(dtype)
+
+
+def fir_step(x1, ring, w, *, x2=None, v=None, bias=None, gated_bias=False):
+    """One decode step of a FIR over its ring cache, fused with the gates.
+
+    x1 (and x2, v): [B, D] bf16.  w: [G, R+1] float32, oldest tap first, the last
+    column on the new sample.  Updates `ring` in place and returns y [B, D] bf16.
+    """
+    _need_cuda(x1, ring.buf, w)
+    B, D = x1.shape
+    R = ring.buf.shape[1]
+    w = _f32(w)
+    G = w.shape[0]
+    if w.shape[1] != R + 1:
+        raise ValueError(f"taps have {w.shape[1]} columns, cache depth {R} needs {R + 1}")
+    for t in (x1, x2, v):
+        if t is not None and (t.dtype != torch.bfloat16 or t.stride(1) != 1 or t.stride(0) != x1.stride(0)):
+            raise ValueError("gates must be bf16 [B, D] with unit channel stride and equal batch strides")
+    out = torch.empty((B, D), dtype=torch.bfloat16, device=x1.device)
+    b = _f32(bias)
+    mode = HYENA_BIAS_NONE if b is None else (HYENA_BIAS_GATED_FP32 if gated_bias else HYENA_BIAS_ADD)
+    rc = _lib.lib().hyena_fir_step(_ptr(x1), _ptr(x2), _ptr(v), x1.stride(0), _ptr(ring.buf), R, ring.pos,
+                                   _ptr(w), _ptr(b), mode, _ptr(out), out.stride(0), B, D, G, _stream())
+    _lib.check(rc, "hyena_fir_step")
+    ring.pos = (ring.pos + 1) % R
+    return out
+
+
+def iir_step(x1, x2, v, state, poles, residues, Dcoef, *, out_dtype=torch.bfloat16):
+    """One decode step of the modal IIR, fused with the gates; `state` is updated in place.
+
+    state: [B, D, S] float32 or complex64.  poles (exponentiated) and residues:
+    [G, S] of the same kind.  Dcoef: [D] bf16 or float32 (its dtype selects the
+    rounding of Dcoef*x1v, as torch promotion does in vortex/model/engine.py:465).
+    """
+    _need_cuda(x1, x2, v, state, poles, residues, Dcoef)
+    B, D = x1.shape
+    cplx = state.is_complex()
+    if not state.is_contiguous():
+        raise ValueError("state must be contiguous")
+    S = state.shape[-1]
+
+    def flat(t):
+        t = t.detach()
+        if cplx:
+            t = torch.view_as_real(t.to(torch.complex64).contiguous())
+        return _f32(t)
+
+    p, r = flat(poles), flat(residues)
+    G = poles.shape[0]
+    st = torch.view_as_real(state) if cplx else state
+    if st.dtype != torch.float32:
+        raise TypeError("state must be float32 or complex64")
+    out = torch.empty((B, D), dtype=out_dtype, device=x1.device)
+    dco = _f32(Dcoef)
+    rc = _lib.lib().hyena_iir_step(_ptr(x1), _ptr(x2), _ptr(v), x1.stride(0), _ptr(st), _ptr(p), _ptr(r), int(cplx),
+                                   _ptr(dco), int(Dcoef.dtype == torch.bfloat16), _ptr(out),
+                                   int(out_dtype == torch.float32), out.stride(0), B, D, G, S, _stream())
+    _lib.check(rc, "hyena_iir_step")
+    return out
