@@ -78,6 +78,34 @@ int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v
                  void* out, int64_t B, int64_t D, int64_t L, int64_t G, int K,
                  void* stream);
 
+/* Hyena-LI: long gated convolution with an implicit modal filter, one pass over L
+ * as a chunked modal scan on bf16 MFMA (split-precision, fp32 accumulate and state).
+ * Replaces HyenaInferenceEngine.parallel_iir (vortex/model/engine.py:262-404),
+ * the filter materialisation HyenaCascade.compute_filter (vortex/model/model.py:390-398)
+ * and the state prefill prefill_via_modal_fft (vortex/model/engine.py:525-559):
+ *   h[g][t] = Re sum_s r[g][s] * exp(t * log_p[g][s])          (never materialised)
+ *   x1v = bf16(x1*v);  y = conv(h, x1v) in fp32;  out = bf16((bf16(y) + Dcoef*x1v) * x2)
+ *   state_out[b][d][s] = sum_j p^(L-1-j) x1v[b][d][j]          (complex, (re, im) pairs)
+ *
+ * hyena_li_plan turns the modal parameters into the per-group coefficient tables the
+ * kernel streams from (filter head, state-in and state-out matrices, p^128), evaluated
+ * in double on the device.  log_poles and residues are [G][S][2] float32 (re, im) pairs;
+ * real poles have im = 0.  The caller owns the workspace: hyena_li_plan_bytes(G, S)
+ * bytes of device memory, reusable until the parameters change.  S must be 16.
+ *
+ * hyena_li_fwd: D/G must be a multiple of 16, L and strides multiples of 8.
+ * y_conv_fp32 (optional, [B][D][L]) receives the fp32 convolution before any rounding;
+ * state_out (optional, [B][D][S][2] float32) the modal state after the last sample.
+ * d_is_bf16 != 0 rounds Dcoef*x1v and the sum to bf16 as bf16 tensors do in
+ * vortex/model/engine.py:352-353. */
+int64_t hyena_li_plan_bytes(int64_t G, int64_t S);
+int hyena_li_plan(const float* log_poles, const float* residues, int64_t G, int64_t S,
+                  void* workspace, void* stream);
+int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v,
+                 const void* workspace, const float* Dcoef, int d_is_bf16,
+                 void* out, float* y_conv_fp32, float* state_out,
+                 int64_t B, int64_t D, int64_t L, int64_t G, int64_t S, void* stream);
+
 /* Decode FIR step on a ring-buffer cache.  Replaces HyenaInferenceEngine.step_fir
  * (vortex/model/engine.py:406-449; native precedent vortex/ops/conv/csrc/step_fir.cu:13-109)
  * fused with the caller's gates (vortex/model/model.py:352, :359):

@@ -13,7 +13,7 @@ HYENA_BIAS_NONE, HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32 = 0, 1, 2
 
 EXPORTS = [
     "hyena_version", "hyena_last_error_string", "hyena_se_fwd", "hyena_mr_fwd",
-    "hyena_fir_step", "hyena_iir_step",
+    "hyena_fir_step", "hyena_iir_step", "hyena_li_plan_bytes", "hyena_li_plan", "hyena_li_fwd",
 ]
 
 
@@ -46,10 +46,14 @@ def lib():
     L.hyena_iir_step.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int,
                                  c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int64,
                                  c_void_p]
+    L.hyena_li_plan_bytes.argtypes = [c_int64, c_int64]
+    L.hyena_li_plan.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]
+    L.hyena_li_fwd.argtypes = [R, R, R, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                               c_int64, c_int64, c_int64, c_void_p]
     for name in EXPORTS:
         fn = getattr(L, name)
         if name not in ("hyena_version", "hyena_last_error_string"):
-            fn.restype = c_int
+            fn.restype = c_int64 if name == "hyena_li_plan_bytes" else c_int
     _lib = L
     return L
 

@@ -129,6 +129,60 @@ def hyena_mr_fwd(x1, x2, v, h, D_bias=None):
                         bias_mode=_bias_mode(b, True, True), taps_reversed=False, force_mfma=True)
 
 
+class ModalPlan:
+    """Device-side coefficient tables of one modal filter bank (see hyena_li_plan)."""
+
+    def __init__(self, log_poles, residues):
+        _need_cuda(log_poles, residues)
+        lp = log_poles.detach().reshape(log_poles.shape[0], -1)
+        rs = residues.detach().reshape(residues.shape[0], -1)
+        self.G, self.S = lp.shape
+        self.is_complex = lp.is_complex() or rs.is_complex()
+
+        def pairs(t):
+            t = t.to(torch.complex64) if not t.is_complex() else t.to(torch.complex64)
+            return torch.view_as_real(t.contiguous()).contiguous()
+
+        self._lp, self._rs = pairs(lp), pairs(rs)
+        nbytes = _lib.lib().hyena_li_plan_bytes(self.G, self.S)
+        if nbytes <= 0:
+            raise NotImplementedError(f"modal state size {self.S} is not supported (16 only)")
+        self.workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=lp.device)
+        rc = _lib.lib().hyena_li_plan(_ptr(self._lp), _ptr(self._rs), self.G, self.S, _ptr(self.workspace), _stream())
+        _lib.check(rc, "hyena_li_plan")
+
+
+def li_fwd_rows(x1r, x2r, vr, plan, Dcoef, B, D, L, *, device, want_state=False, want_fp32=False):
+    out = torch.empty((B, D, L), dtype=torch.bfloat16, device=device)
+    y32 = torch.empty((B, D, L), dtype=torch.float32, device=device) if want_fp32 else None
+    state = torch.empty((B, D, plan.S, 2), dtype=torch.float32, device=device) if want_state else None
+    dco = _f32(Dcoef)
+    d_is_bf16 = int(Dcoef is None or Dcoef.dtype == torch.bfloat16)
+    rc = _lib.lib().hyena_li_fwd(_ref(x1r), _ref(x2r), _ref(vr), _ptr(plan.workspace), _ptr(dco), d_is_bf16,
+                                 _ptr(out), _ptr(y32), _ptr(state), B, D, L, plan.G, plan.S, _stream())
+    _lib.check(rc, "hyena_li_fwd")
+    if state is not None:
+        state = torch.view_as_complex(state) if plan.is_complex else state[..., 0].contiguous()
+    return out, y32, state
+
+
+def hyena_li_fwd(x1, x2, v, log_poles, residues, D_bias=None, *, plan=None, want_state=False, want_fp32=False):
+    """Hyena-LI prefill on [B, D, L] bf16 gates with grouped modal parameters.
+
+    log_poles [G, S, 1] (or [G, S]) and residues [G, S], float32 or complex64
+    (vortex/model/model.py:202-209, :390-398).  Returns (out [B, D, L] bf16,
+    y_conv fp32 or None, state [B, D, S] or None); the state is complex64 for complex
+    poles and float32 for real ones (the real part, as vortex/model/engine.py:559 keeps).
+    Pass a ModalPlan to reuse the coefficient tables between calls.
+    """
+    _need_cuda(x1, x2, v, log_poles, residues)
+    B, D, L = x1.shape
+    if plan is None:
+        plan = ModalPlan(log_poles, residues)
+    return li_fwd_rows(rows_of(x1), rows_of(x2), rows_of(v), plan, D_bias, B, D, L, device=x1.device,
+                       want_state=want_state, want_fp32=want_fp32)
+
+
 class FirRing:
     """Ring-buffer FIR cache [B, R, D] bf16 plus the index of its oldest slot.
 
