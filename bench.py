@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Benchmark of the Hyena operator hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mr|se|li|decode] [--no-extras]
+
+A "step" is one pass of the operator over one batch of synthetic input that is
+already resident in HBM.  The headline workload is the Hyena-MR prefill
+configuration (B=2, L=32768, D=4096, 256 filter groups, K=128); the other
+configurations (Hyena-SE, Hyena-LI prefill, the cached decode step) are
+measured the same way and reported under "extra" unless --no-extras is given.
+Prints ONE JSON line.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0     # MI355X published HBM3E bandwidth
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="mr", choices=["mr", "se", "li", "decode"])
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    return ap.parse_args()
+
+
+def gates(B, D, L, seed, device):
+    g = torch.Generator(device=device).manual_seed(seed)
+    return tuple(torch.randn(B, D, L, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+                 for _ in range(3))
+
+
+def time_steps(fn, steps, warmup):
+    """(wall seconds for `steps` calls, average kernel-side ms per call from HIP events on the launch stream)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(steps):
+        fn()
+    ev1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return t1 - t0, ev0.elapsed_time(ev1) / steps
+
+
+def build_workload(name, device):
+    """Returns (callable, description dict) for one configuration."""
+    import vortex_amd as va
+    from oracle import hyena_oracle as O          # input generators only (filters, poles)
+    from vortex_amd import ops
+
+    if name == "se":
+        B, D, L, G, K = 1, 4096, 8192, 256, 7
+        x2, x1, v = gates(B, D, L, 1, device)
+        h = O.make_se_filter(G, K).reshape(G, K).to(device)
+        r1, r2, rv = ops.rows_of(x1), ops.rows_of(x2), ops.rows_of(v)
+        out = torch.empty(B, D, L, dtype=torch.bfloat16, device=device)
+        fn = lambda: ops.fir_fwd_rows(r1, r2, rv, h, B, D, L, K, device=device, taps_reversed=True, out=out)
+        return fn, dict(workload=f"hyena_se_prefill B={B} L={L} D={D} groups={G} K={K}", tokens=B * L,
+                        bytes=8 * B * D * L, kernel="se_fir_kernel", keep=(x1, x2, v, h, out))
+    if name == "mr":
+        B, D, L, G, K = 2, 4096, 32768, 256, 128
+        x2, x1, v = gates(B, D, L, 2, device)
+        h = O.make_mr_filter(G, K).reshape(G, K).to(device)
+        Db = torch.randn(D, generator=torch.Generator().manual_seed(3)).to(device)
+        r1, r2, rv = ops.rows_of(x1), ops.rows_of(x2), ops.rows_of(v)
+        out = torch.empty(B, D, L, dtype=torch.bfloat16, device=device)
+        fn = lambda: ops.fir_fwd_rows(r1, r2, rv, h, B, D, L, K, device=device, bias=Db,
+                                      bias_mode=ops.HYENA_BIAS_GATED_FP32, force_mfma=True, out=out)
+        return fn, dict(workload=f"hyena_mr_prefill B={B} L={L} D={D} groups={G} K={K}", tokens=B * L,
+                        bytes=8 * B * D * L, kernel="mr_fir_kernel", keep=(x1, x2, v, h, Db, out))
+    if name == "li":
+        B, D, L, G, S = 1, 4096, 262144, 256, 16
+        x2, x1, v = gates(B, D, L, 4, device)
+        lp, r = O.make_modal_complex(G, S)
+        Db = torch.randn(D, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).to(device)
+        plan = va.ModalPlan(lp.to(device), r.to(device))
+        r1, r2, rv = ops.rows_of(x1), ops.rows_of(x2), ops.rows_of(v)
+        out = torch.empty(B, D, L, dtype=torch.bfloat16, device=device)
+        fn = lambda: ops.li_fwd_rows(r1, r2, rv, plan, Db, B, D, L, device=device, out=out)
+        return fn, dict(workload=f"hyena_li_prefill B={B} L={L} D={D} groups={G} poles={S} complex", tokens=B * L,
+                        bytes=8 * B * D * L, kernel="li_kernel", keep=(x1, x2, v, plan, Db, out))
+    raise ValueError(name)
+
+
+def decode_layer_set(D, device, steps, warmup):
+    """One [SE, MR, LI] layer set of cached decode at batch 64: three fused launches per token."""
+    import vortex_amd as va
+    from oracle import hyena_oracle as O
+    B, S = 64, 16
+    g = torch.Generator(device=device).manual_seed(6)
+    rnd = lambda *s: torch.randn(*s, generator=g, device=device, dtype=torch.float32)
+    x = [tuple(rnd(B, D).to(torch.bfloat16) for _ in range(3)) for _ in range(3)]
+    G = D // 16
+    ring_se = va.FirRing(rnd(B, 6, D).to(torch.bfloat16))
+    ring_mr = va.FirRing(rnd(B, 127, D).to(torch.bfloat16))
+    w_se, w_mr = rnd(G, 7) * 7 ** -0.5, rnd(G, 128) * 128 ** -0.5
+    Dmr = rnd(D)
+    lp, r = O.make_modal_complex(G, S)
+    poles, res = torch.exp(lp[..., 0]).to(device), r.to(device)
+    state = torch.zeros(B, D, S, dtype=torch.complex64, device=device)
+    Dli = rnd(D).to(torch.bfloat16)
+    step = va.DecodeLayerSet(ring_se, w_se, ring_mr, w_mr, Dmr, state, poles, res, Dli)
+
+    def fn():
+        step(x[0], x[1], x[2])
+
+    wall, ms = time_steps(fn, steps, warmup)
+    # algorithmic bytes: caches read once, one ring slot written per FIR, modal state read+written,
+    # 3 gate vectors in and 1 output vector out per operator
+    byts = B * D * 2 * (6 + 127) + 2 * B * D * 2 + 2 * state.numel() * 8 + 3 * 4 * B * D * 2
+    return dict(us_per_step=ms * 1e3, wall_us_per_step=wall / steps * 1e6, bytes=byts,
+                hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
+
+
+def cpu_baseline(name):
+    """The oracle (a PyTorch port of the reference path) timed on the host cores, on a channel slice."""
+    from oracle import hyena_oracle as O
+    threads = torch.get_num_threads()
+    if name == "mr":
+        B, D, L, G, K, Ds = 2, 4096, 32768, 256, 128, 256
+        x2, x1, v = O.make_gates(B, Ds, L, seed=2)
+        h = O.make_mr_filter(Ds // 16, K)
+        Db = torch.randn(Ds)
+        f = lambda: O.mr_fir(x2, x1, v, h, Db)
+    elif name == "se":
+        B, D, L, G, K, Ds = 1, 4096, 8192, 256, 7, 1024
+        x2, x1, v = O.make_gates(B, Ds, L, seed=1)
+        h = O.make_se_filter(Ds // 16, K)
+        f = lambda: O.se_fir(x2, x1, v, h)
+    elif name == "li":
+        B, D, L, G, K, Ds = 1, 4096, 262144, 256, 0, 32
+        x2, x1, v = O.make_gates(B, Ds, L, seed=4)
+        lp, r = O.make_modal_complex(Ds // 16, 16)
+        Db = torch.randn(Ds).bfloat16()
+        f = lambda: O.li_prefill(x2, x1, v, lp, r, Db, want_state=False)
+    else:
+        return None
+    f()
+    ts = []
+    t_all = time.perf_counter()
+    while len(ts) < 3 or (time.perf_counter() - t_all < 10 and len(ts) < 20):
+        t0 = time.perf_counter()
+        f()
+        ts.append(time.perf_counter() - t0)
+    t = sorted(ts)[len(ts) // 2]
+    return dict(value=B * L / (t * D / Ds), unit="tokens/s", cores=threads, kind="port",
+                sample=f"oracle (PyTorch fp32 conv1d/FFT restatement) on {Ds} of {D} channels at full B, L; "
+                       f"median of {len(ts)} runs, scaled linearly to {D} channels")
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; the Hyena operator path shards over channels "
+              "without communication, so --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    def run(name, steps, warmup):
+        fn, d = build_workload(name, device)
+        wall, ms = time_steps(fn, steps, warmup)
+        d.pop("keep")
+        d.update(wall_s=wall, kernel_ms=ms, tokens_per_s=d["tokens"] * steps / wall,
+                 hbm_gbs=d["bytes"] / (ms * 1e-3) / 1e9)
+        torch.cuda.empty_cache()
+        return d
+
+    main_name = args.workload if args.workload != "decode" else "mr"
+    m = run(main_name, args.steps, args.warmup)
+    result = {
+        "metric": "Hyena-SE/MR/LI prefill tokens/s/GPU at D=4096 + % roofline; decode step us",
+        "value": m["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": m["wall_s"] / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16 in/out, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": m["workload"]},
+        "roofline": {"bound": "hbm", "achieved": m["hbm_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": m["hbm_gbs"] / HBM_PEAK_GBS, "traffic": None, "kernel": m["kernel"],
+                     "algorithmic_bytes_per_launch": m["bytes"], "kernel_ms": m["kernel_ms"]},
+    }
+    if not args.no_extras:
+        extra = {}
+        for name in ("se", "mr", "li"):
+            if name == main_name:
+                continue
+            steps = max(3, min(args.steps, 20 if name == "li" else args.steps))
+            e = run(name, steps, min(args.warmup, 3))
+            extra[name] = {"workload": e["workload"], "tokens_per_s": e["tokens_per_s"],
+                           "kernel_us": e["kernel_ms"] * 1e3, "hbm_gbs": e["hbm_gbs"],
+                           "roofline_frac": e["hbm_gbs"] / HBM_PEAK_GBS}
+        for D in (4096, 8192):
+            extra[f"decode_D{D}"] = decode_layer_set(D, device, max(args.steps, 50), max(args.warmup, 5))
+        result["extra"] = extra
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(main_name)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

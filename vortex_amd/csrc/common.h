@@ -20,15 +20,18 @@ __device__ __forceinline__ float bf_lo(uint32_t w) { return __uint_as_float(w <<
 __device__ __forceinline__ float bf_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 __device__ __forceinline__ float bf_to_f(bf16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
 
-__device__ __forceinline__ uint32_t f_to_bf_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;    // NaN stays NaN
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-}
-__device__ __forceinline__ float round_bf(float f) { return __uint_as_float(f_to_bf_bits(f) << 16); }
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_t;
+
+// fp32 -> bf16 goes through the gfx950 conversion instruction (v_cvt_pk_bf16_f32, RNE).
 __device__ __forceinline__ uint32_t pack_bf2(float lo, float hi) {
-    return f_to_bf_bits(lo) | (f_to_bf_bits(hi) << 16);
+    const f32x2_t f = {lo, hi};
+    union { bf16x2_t h; uint32_t u; } c;
+    c.h = __builtin_convertvector(f, bf16x2_t);
+    return c.u;
 }
+__device__ __forceinline__ uint32_t f_to_bf_bits(float f) { return pack_bf2(f, 0.f) & 0xffffu; }
+__device__ __forceinline__ float round_bf(float f) { return __uint_as_float(pack_bf2(f, 0.f) << 16); }
 
 struct RowMap {            // device copy of hyena_rows
     const bf16_t* ptr;

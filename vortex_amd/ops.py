@@ -75,7 +75,7 @@ def _bias_mode(bias, gated, fp32_gated):
 
 
 def fir_fwd_rows(x1r, x2r, vr, taps, B, D, L, K, *, device, bias=None, bias_mode=HYENA_BIAS_NONE,
-                 taps_reversed=False, force_mfma=False):
+                 taps_reversed=False, force_mfma=False, out=None):
     """Shared launcher of the prefill FIR kernels on row descriptors.
 
     taps [G, K] float32.  taps_reversed=False means the convolution orientation
@@ -84,7 +84,8 @@ def fir_fwd_rows(x1r, x2r, vr, taps, B, D, L, K, *, device, bias=None, bias_mode
     """
     taps = _f32(taps)
     G = taps.shape[0]
-    out = torch.empty((B, D, L), dtype=torch.bfloat16, device=device)
+    if out is None:
+        out = torch.empty((B, D, L), dtype=torch.bfloat16, device=device)
     L_ = _lib.lib()
     if K <= 8 and not force_mfma:
         if not taps_reversed:
@@ -152,8 +153,9 @@ class ModalPlan:
         _lib.check(rc, "hyena_li_plan")
 
 
-def li_fwd_rows(x1r, x2r, vr, plan, Dcoef, B, D, L, *, device, want_state=False, want_fp32=False):
-    out = torch.empty((B, D, L), dtype=torch.bfloat16, device=device)
+def li_fwd_rows(x1r, x2r, vr, plan, Dcoef, B, D, L, *, device, want_state=False, want_fp32=False, out=None):
+    if out is None:
+        out = torch.empty((B, D, L), dtype=torch.bfloat16, device=device)
     y32 = torch.empty((B, D, L), dtype=torch.float32, device=device) if want_fp32 else None
     state = torch.empty((B, D, plan.S, 2), dtype=torch.float32, device=device) if want_state else None
     dco = _f32(Dcoef)
@@ -267,3 +269,74 @@ def iir_step(x1, x2, v, state, poles, residues, Dcoef, *, out_dtype=torch.bfloat
                                    int(out_dtype == torch.float32), out.stride(0), B, D, G, S, _stream())
     _lib.check(rc, "hyena_iir_step")
     return out
+
+
+class FirStepper:
+    """A decode FIR step with every argument except the gates bound once (low host overhead)."""
+
+    def __init__(self, ring, w, bias=None, gated_bias=False, gated=True):
+        _need_cuda(ring.buf, w)
+        self.ring, self.w, self.bias = ring, _f32(w), _f32(bias)
+        self.R, self.D = ring.buf.shape[1], ring.buf.shape[2]
+        self.G = self.w.shape[0]
+        if self.w.shape[1] != self.R + 1:
+            raise ValueError(f"taps have {self.w.shape[1]} columns, cache depth {self.R} needs {self.R + 1}")
+        self.mode = HYENA_BIAS_NONE if bias is None else (HYENA_BIAS_GATED_FP32 if gated_bias else HYENA_BIAS_ADD)
+        self.gated = gated
+        self._fn = _lib.lib().hyena_fir_step
+
+    def __call__(self, x1, x2, v, out):
+        B = x1.shape[0]
+        rc = self._fn(x1.data_ptr(), x2.data_ptr() if self.gated else None, v.data_ptr() if self.gated else None,
+                      x1.stride(0), self.ring.buf.data_ptr(), self.R, self.ring.pos, self.w.data_ptr(),
+                      self.bias.data_ptr() if self.bias is not None else None, self.mode, out.data_ptr(),
+                      out.stride(0), B, self.D, self.G, torch.cuda.current_stream().cuda_stream)
+        if rc:
+            _lib.check(rc, "hyena_fir_step")
+        self.ring.pos = (self.ring.pos + 1) % self.R
+        return out
+
+
+class IirStepper:
+    """A decode modal-IIR step with the state and modal parameters bound once."""
+
+    def __init__(self, state, poles, residues, Dcoef):
+        _need_cuda(state, poles, residues, Dcoef)
+        self.cplx = state.is_complex()
+        flat = (lambda t: _f32(torch.view_as_real(t.detach().to(torch.complex64).contiguous()))) if self.cplx \
+            else (lambda t: _f32(t.detach()))
+        self.state = state
+        self.st = torch.view_as_real(state) if self.cplx else state
+        self.p, self.r = flat(poles), flat(residues)
+        self.dco, self.d_is_bf16 = _f32(Dcoef), int(Dcoef.dtype == torch.bfloat16)
+        self.G, self.S = poles.shape[0], state.shape[-1]
+        self.D = state.shape[1]
+        self._fn = _lib.lib().hyena_iir_step
+
+    def __call__(self, x1, x2, v, out):
+        B = x1.shape[0]
+        rc = self._fn(x1.data_ptr(), x2.data_ptr(), v.data_ptr(), x1.stride(0), self.st.data_ptr(), self.p.data_ptr(),
+                      self.r.data_ptr(), int(self.cplx), self.dco.data_ptr(), self.d_is_bf16, out.data_ptr(),
+                      int(out.dtype == torch.float32), out.stride(0), B, self.D, self.G, self.S,
+                      torch.cuda.current_stream().cuda_stream)
+        if rc:
+            _lib.check(rc, "hyena_iir_step")
+        return out
+
+
+class DecodeLayerSet:
+    """Cached decode step of one [Hyena-SE, Hyena-MR, Hyena-LI] layer set: three fused launches."""
+
+    def __init__(self, ring_se, w_se, ring_mr, w_mr, D_mr, state_li, poles, residues, D_li):
+        self.se = FirStepper(ring_se, w_se)
+        self.mr = FirStepper(ring_mr, w_mr, bias=D_mr, gated_bias=True)
+        self.li = IirStepper(state_li, poles, residues, D_li)
+        B, D = state_li.shape[0], state_li.shape[1]
+        self.out = [torch.empty(B, D, dtype=torch.bfloat16, device=state_li.device) for _ in range(3)]
+
+    def __call__(self, g_se, g_mr, g_li):
+        """Each argument is (x2, x1, v), bf16 [B, D]; returns the three outputs."""
+        self.se(g_se[1], g_se[0], g_se[2], self.out[0])
+        self.mr(g_mr[1], g_mr[0], g_mr[2], self.out[1])
+        self.li(g_li[1], g_li[0], g_li[2], self.out[2])
+        return self.out
