@@ -63,6 +63,20 @@ int hyena_se_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v
                  void* out, int64_t B, int64_t D, int64_t L, int64_t G, int K,
                  void* stream);
 
+/* Featurizer short FIR (2 <= K <= 8) over the C = 3D channels of the input projection,
+ * fused with the [B][L][C] -> [B][C][L] layout change.  Replaces parallel_fir with
+ * gate=False, dim_last=True (vortex/model/engine.py:188-223; call site
+ * vortex/model/model.py:233-246; native precedent: the channel-last kernel
+ * vortex/ops/conv/csrc/causal_conv1d_fwd.cu:210):
+ *   z[b][c][t] = bf16( sum_k taps[g(c)][k] * u[b][t-(K-1)+k][c] )   (+ bias[c], rounded again)
+ * u: bf16, channels contiguous, sample t of batch b at u + b*u_batch_stride + t*u_time_stride.
+ * taps: [G][K] float32 (G = C for vortex's per-channel short filter).  out: [B][C][L] bf16.
+ * interleave3 != 0 also applies the channel de-interleave of vortex/model/utils.py:26-38
+ * (input channel 3j+i is written to output row i*C/3 + j). */
+int hyena_featurizer_fwd(const void* u, int64_t u_batch_stride, int64_t u_time_stride,
+                         const float* taps, const float* bias, int interleave3, void* out,
+                         int64_t B, int64_t L, int64_t C, int64_t G, int K, void* stream);
+
 /* Hyena-MR: gated causal depthwise FIR with 2 <= K <= 128 as a chunked,
  * block-Toeplitz contraction on bf16 MFMA with fp32 accumulation.
  * Replaces parallel_fir, K >= 128 branch + fftconv_func

@@ -207,7 +207,7 @@ def modal_filter(log_poles, residues, L, dtype=None):
     `(residues * poles**t).real.sum(1)` of model.py:847.  Returns [1, G, L].
     `dtype=torch.float64/complex128` evaluates the same formula in double.
     """
-    t = torch.arange(L)[None, None]
+    t = torch.arange(L, device=log_poles.device)[None, None]
     if dtype is not None:
         cdt = dtype
         if log_poles.is_complex():
@@ -544,3 +544,92 @@ def make_modal_real(G, S=16, seed=400, pmin=0.9, pmax=0.9999):
     g = torch.Generator(device="cpu").manual_seed(seed)
     mag = pmin + (pmax - pmin) * torch.rand(G, S, generator=g, dtype=torch.float64)
     return mag.log().to(torch.float32)[..., None], torch.randn(G, S, generator=g)
+
+
+# --------------------------------------------------------------------------
+# the operator module's call sequence  (vortex/model/model.py:214-398)
+# --------------------------------------------------------------------------
+
+class OracleCascade:
+    """Restatement of HyenaCascade.forward on top of any engine with the four
+    HyenaInferenceEngine methods (the oracle's or the product's), so that a parity
+    test drives both through the same call sequence.
+
+    params: dict with short_filter_weight [3D,1,Ks], short_filter_bias or None, and either
+    h [G,1,K] (+ D [hidden] when K >= 128) or log_poles [G,S,1], residues [G,S], D [hidden].
+    """
+
+    def __init__(self, engine, params, hidden, n_heads, groups, layer_idx=0, fir_inner_filter_length=None,
+                 column_split_hyena=False, interleave=False, state_size=16):
+        self.engine, self.p = engine, params
+        self.hidden, self.n_heads, self.groups = hidden, n_heads, groups
+        self.layer_idx, self.K = layer_idx, fir_inner_filter_length
+        self.column_split_hyena, self.interleave, self.state_size = column_split_hyena, interleave, state_size
+        self.Ks = params["short_filter_weight"].shape[-1]
+
+    def forward(self, u, inference_params=None):
+        # model.py:214-219
+        if inference_params is not None and self.layer_idx in inference_params.fir_state_dict.keys():
+            return self.sequential_forward(u, inference_params)
+        return self.parallel_forward(u, inference_params)
+
+    def parallel_forward(self, u, inference_params=None):
+        # model.py:221-316
+        p, L = self.p, u.shape[1]
+        dims = (self.hidden, self.n_heads, self.hidden // self.n_heads, self.state_size, self.groups)
+        z_pre, fir_state = self.engine.parallel_fir(
+            F.conv1d, u, p["short_filter_weight"], p.get("short_filter_bias"), L, dims=dims, gate=False,
+            column_split_hyena=self.column_split_hyena, fir_length=self.Ks, inference_params=inference_params,
+            padding_mask=None, dim_last=True)
+        if inference_params:
+            inference_params.fir_state_dict[self.layer_idx] = fir_state
+        if self.interleave:
+            z_pre = interleave(z_pre)
+        if self.K is None:
+            h = modal_filter(p["log_poles"].to(u.device), p["residues"].to(u.device), L)     # model.py:390-398
+            h = h.to(u.device)
+        else:
+            h = p["h"]
+        if self.groups > 1:
+            h = h.repeat_interleave(self.hidden // self.groups, 0)                          # model.py:261-262
+        if self.K is not None:
+            y, inner = self.engine.parallel_fir(
+                F.conv1d, z_pre, h, p.get("D"), L, dims=dims, gate=True, gated_bias=self.K >= 128, dim_last=False,
+                column_split_hyena=self.column_split_hyena, fir_length=self.K, inference_params=inference_params,
+                padding_mask=None, groups=self.groups)
+            y = y.permute(0, 2, 1)
+            if inference_params:
+                inference_params.fir_inner_state_dict[self.layer_idx] = inner
+        else:
+            y = self.engine.parallel_iir(
+                z_pre, h, p["D"], L, t=None, poles=p["log_poles"], residues=p["residues"], dims=dims,
+                inference_params=inference_params, layer_idx=self.layer_idx, prefill_style="fft",
+                use_flashfft=False, fftconv_fn=None, column_split_hyena=self.column_split_hyena,
+                long_fir_threshold=None, padding_mask=None)
+        return y, inference_params
+
+    def sequential_forward(self, u, inference_params):
+        # model.py:318-375
+        p = self.p
+        if u.dim() > 2:
+            u = u[:, -1]
+        z_pre, fir_state = self.engine.step_fir(u, inference_params.fir_state_dict[self.layer_idx],
+                                                weight=p["short_filter_weight"], bias=p.get("short_filter_bias"))
+        inference_params.fir_state_dict[self.layer_idx] = fir_state
+        if self.interleave:
+            z_pre = interleave(z_pre)
+        hd = self.hidden // self.n_heads
+        x2, x1, v = (column_split(z_pre, self.n_heads, hd) if self.column_split_hyena
+                     else z_pre.split([self.hidden] * 3, dim=1))
+        if self.K is not None:
+            h = p["h"].repeat_interleave(self.hidden // self.groups, 0) if self.groups > 1 else p["h"]
+            y, inner = self.engine.step_fir(x1 * v, inference_params.fir_inner_state_dict[self.layer_idx], weight=h,
+                                            bias=p.get("D"), flip_filter=self.K >= 128, gated_bias=self.K >= 128)
+            y = y * x2
+            inference_params.fir_inner_state_dict[self.layer_idx] = inner
+        else:
+            y, st = self.engine.step_iir(x2, x1, v, p["D"], p["residues"], p["log_poles"],
+                                         inference_params.state_dict[self.layer_idx], iir_groups=1)
+            inference_params.state_dict[self.layer_idx] = st
+        y = y.to(dtype=u.dtype)
+        return y[:, None], inference_params

@@ -1,0 +1,200 @@
+"""The Hyena operator module on the gfx950 kernels: counterpart of vortex's HyenaCascade.
+
+Reproduces the call sequence of vortex/model/model.py:125-398 (featurizer FIR ->
+interleave -> split -> inner operator; prefill when the layer has no cached state,
+one-token decode afterwards) but hands the kernels what they want directly: grouped
+filters without repeat_interleave, modal parameters without a materialised filter,
+ring-buffer FIR caches, and the modal state emitted by the prefill kernel itself.
+Cache containers mirror vortex/model/cache.py:31-61.
+"""
+from dataclasses import dataclass, field
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from ._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE
+
+
+@dataclass
+class HyenaCascadeIIRInferenceParams:
+    """vortex/model/cache.py:31-44."""
+    fir_filter_length: int = 3
+    state_dim: int = 16
+    seqlen_offset: int = 0
+    fir_state_dict: dict = field(default_factory=dict)
+    state_dict: dict = field(default_factory=dict)
+
+    def reset(self):
+        self.fir_filter_length, self.state_dim, self.seqlen_offset = 3, 16, 0
+
+
+@dataclass
+class HyenaCascadeFIRInferenceParams:
+    """vortex/model/cache.py:47-61."""
+    fir_filter_length: int = 3
+    fir_inner_filter_length: int = 4
+    seqlen_offset: int = 0
+    fir_inner_state_dict: dict = field(default_factory=dict)
+    fir_state_dict: dict = field(default_factory=dict)
+    state_dict: dict = field(default_factory=dict)
+
+    def reset(self):
+        self.fir_filter_length, self.fir_inner_filter_length, self.seqlen_offset = 3, 4, 0
+
+
+def _cfg(config, key, default=None):
+    v = config.get(key, default) if hasattr(config, "get") else getattr(config, key, default)
+    return default if v is None else v
+
+
+class HyenaCascade(nn.Module):
+    """Parameters and forward of one Hyena operator (SE / MR when fir_inner_filter_length is set, LI otherwise).
+
+    Parameter names and shapes follow vortex/model/model.py:152-210 so that vortex state
+    dicts load: short_filter_weight [3D, 1, Ks], short_filter_bias [3D] (optional),
+    h [G, 1, K] + D [hidden] (MR only) for FIR layers, log_poles [G, S, 1] + residues [G, S] + D
+    for modal layers.  log_poles / residues may be complex64.
+    """
+
+    def __init__(self, config, layer_idx, hyena_filter_groups=None, fir_inner_filter_length=None,
+                 complex_modal=False):
+        super().__init__()
+        self.config, self.layer_idx = config, layer_idx
+        self.hidden_size = config["hidden_size"] if isinstance(config, dict) else config.hidden_size
+        D = self.hidden_size
+        self.hyena_filter_groups = hyena_filter_groups or D
+        self.state_size = _cfg(config, "state_size", 16)
+        self.num_attention_heads = _cfg(config, "num_attention_heads", 1)
+        self.hidden_size_per_attention_head = D // self.num_attention_heads
+        self.column_split_hyena = _cfg(config, "column_split_hyena", True)
+        self.hyena_flip_x1x2 = _cfg(config, "hyena_flip_x1x2", False)
+        self.interleave = _cfg(config, "interleave", False)
+        self.short_filter_length = _cfg(config, "short_filter_length", 3)
+        self.fir_inner_filter_length = fir_inner_filter_length
+        self.short_filter_weight = nn.Parameter(torch.randn(3 * D, 1, self.short_filter_length))
+        self.short_filter_bias = nn.Parameter(torch.randn(3 * D)) if _cfg(config, "short_filter_bias", False) else None
+        G = self.hyena_filter_groups
+        if fir_inner_filter_length:
+            self.h = nn.Parameter(torch.randn(G, 1, fir_inner_filter_length))
+            self.D = nn.Parameter(torch.zeros(D)) if fir_inner_filter_length >= 128 else None
+        else:
+            dt = torch.complex64 if complex_modal else torch.float32
+            self.log_poles = nn.Parameter(torch.randn(G, self.state_size, 1, dtype=dt))
+            self.residues = nn.Parameter(torch.randn(G, self.state_size, dtype=dt))
+            self.D = nn.Parameter(torch.zeros(D))
+            self.h = None
+        self._plan = None
+        self._decode = None
+
+    # ------------------------------------------------------------------
+    def forward(self, u, inference_params=None, padding_mask=None, *args, **kwargs):
+        if inference_params is not None and self.layer_idx in inference_params.fir_state_dict.keys():
+            return self.sequential_forward(u, inference_params)
+        return self.parallel_forward(u, inference_params, padding_mask)
+
+    def _rows(self, z_pre):
+        D = self.hidden_size
+        hd = self.hidden_size_per_attention_head if self.column_split_hyena else None
+        r2, r1, rv = (ops.rows_of_projection(z_pre, D, i, hd) for i in range(3))
+        if self.hyena_flip_x1x2:
+            r1, r2 = r2, r1
+        return r1, r2, rv
+
+    def _split(self, z):
+        """(x2, x1, v) views of a [B, 3D] or [B, 3D, R] tensor, as vortex/model/model.py:336-343."""
+        D, hd = self.hidden_size, self.hidden_size_per_attention_head
+        if self.column_split_hyena:
+            zr = z.reshape(z.shape[0], -1, 3, hd, *z.shape[2:])
+            x2, x1, v = (zr[:, :, i].reshape(z.shape[0], D, *z.shape[2:]) for i in range(3))
+        else:
+            x2, x1, v = z.split([D, D, D], dim=1)
+        if self.hyena_flip_x1x2:
+            x1, x2 = x2, x1
+        return x2, x1, v
+
+    def modal_plan(self):
+        key = (self.log_poles._version, self.residues._version, self.log_poles.data_ptr())
+        if self._plan is None or self._plan[0] != key:
+            self._plan = (key, ops.ModalPlan(self.log_poles, self.residues))
+        return self._plan[1]
+
+    def parallel_forward(self, u, inference_params=None, padding_mask=None):
+        """Prefill: u [B, L, 3D] bf16 -> y [B, L, D] bf16 (vortex/model/model.py:221-316)."""
+        if padding_mask is not None:
+            raise NotImplementedError("padding_mask is handled by the drop-in engine, not by this module")
+        B, L, C = u.shape
+        D, Ks = self.hidden_size, self.short_filter_length
+        w = self.short_filter_weight.detach().reshape(C, Ks)
+        z_pre = ops.featurizer_fwd(u, w, self.short_filter_bias, interleave=self.interleave)
+        r1, r2, rv = self._rows(z_pre)
+        K = self.fir_inner_filter_length
+        caching = inference_params is not None
+        if K:
+            taps = self.h.detach().reshape(self.h.shape[0], K)
+            if K >= 128:
+                y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, K, device=u.device, bias=ops._f32(self.D),
+                                     bias_mode=HYENA_BIAS_GATED_FP32, taps_reversed=False, force_mfma=True)
+            else:
+                y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, K, device=u.device, taps_reversed=True)
+        else:
+            y, _, state = ops.li_fwd_rows(r1, r2, rv, self.modal_plan(), self.D, B, D, L, device=u.device,
+                                          want_state=caching)
+            if caching:
+                inference_params.state_dict[self.layer_idx] = state
+        if caching:
+            if L < Ks - 1 or (K and L < K - 1):
+                raise NotImplementedError("prompts shorter than the filters are not supported by the cached path")
+            # the channel-last tail of u is already the ring layout [B, R, 3D]
+            inference_params.fir_state_dict[self.layer_idx] = ops.FirRing(u[:, L - (Ks - 1):].contiguous(), 0)
+            if K:
+                _, x1, v = self._split(z_pre[..., L - (K - 1):])
+                inference_params.fir_inner_state_dict[self.layer_idx] = ops.FirRing(
+                    (x1 * v).permute(0, 2, 1).contiguous(), 0)
+            self._decode = None
+        return y.permute(0, 2, 1), inference_params
+
+    # ------------------------------------------------------------------
+    def _decode_plan(self, inference_params):
+        """Binds the decode kernels to this layer's caches once per generation."""
+        i = self.layer_idx
+        ring = inference_params.fir_state_dict[i]
+        if self._decode is not None and self._decode["ring"] is ring:
+            return self._decode
+        C, Ks, D = 3 * self.hidden_size, self.short_filter_length, self.hidden_size
+        dev = ring.buf.device
+        d = {"ring": ring}
+        d["feat"] = ops.FirStepper(ring, self.short_filter_weight.detach().reshape(C, Ks), bias=self.short_filter_bias,
+                                   gated=False)
+        if self.interleave:
+            j = torch.arange(C, device=dev)
+            d["perm"] = (j % (C // 3)) * 3 + j // (C // 3)      # output row r = i*C/3 + j'  <-  channel 3j' + i
+        K = self.fir_inner_filter_length
+        if K:
+            taps = self.h.detach().reshape(self.h.shape[0], K)
+            taps = taps if K < 128 else taps.flip(-1)           # oldest tap first (engine.py:421-425)
+            d["inner"] = ops.FirStepper(inference_params.fir_inner_state_dict[i], taps.contiguous(),
+                                        bias=self.D if K >= 128 else None, gated_bias=K >= 128)
+        else:
+            st = inference_params.state_dict[i]
+            poles = torch.exp(self.log_poles.detach())[..., 0].contiguous()
+            d["inner"] = ops.IirStepper(st, poles, self.residues.detach(), self.D.detach())
+        self._decode = d
+        return d
+
+    def sequential_forward(self, u, inference_params):
+        """Decode: u [B, 3D] or [B, 1, 3D] bf16 -> y [B, 1, D] (vortex/model/model.py:318-375)."""
+        if u.dim() > 2:
+            u = u[:, -1]
+        d = self._decode_plan(inference_params)
+        B = u.shape[0]
+        z_pre = torch.empty(B, 3 * self.hidden_size, dtype=torch.bfloat16, device=u.device)
+        d["feat"](u, None, None, z_pre)
+        if self.interleave:
+            z_pre = z_pre[:, d["perm"]]
+        x2, x1, v = self._split(z_pre)
+        if self.column_split_hyena:
+            x2, x1, v = x2.contiguous(), x1.contiguous(), v.contiguous()
+        y = torch.empty(B, self.hidden_size, dtype=torch.bfloat16, device=u.device)
+        d["inner"](x1, x2, v, y)
+        return y[:, None], inference_params

@@ -1,0 +1,176 @@
+"""Drop-in replacement for vortex's HyenaInferenceEngine, backed by the gfx950 kernels.
+
+Same four methods, argument names and return conventions as
+vortex/model/engine.py:112-467, so that `block.filter.engine = HyenaInferenceEngine(...)`
+switches a vortex HyenaCascade to the HIP path with no other source change.
+Everything here runs on the GPU through the C ABI; there is no PyTorch fallback
+for the convolutions, and CPU tensors are rejected.
+"""
+import torch
+
+from . import ops
+from ._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE
+
+IIR_PREFILL_MODES = ["recurrence", "modal-fft", "hybrid-modal-recurrence", "modal-scan", "canonical-fft",
+                     "iir-fir-caching"]
+
+
+def _group_taps(weight, D, groups):
+    """[D, 1, K] (a [G, 1, K] filter bank expanded with repeat_interleave, vortex/model/model.py:261-262)
+    or [G, 1, K] -> ([G', K] float32, G')."""
+    w = weight.detach().reshape(weight.shape[0], -1)
+    rows = w.shape[0]
+    if groups is not None and rows == D and groups < D and D % groups == 0:
+        w = w[:: D // groups]
+    return w.to(torch.float32).contiguous()
+
+
+class HyenaInferenceEngine:
+    def __init__(self, fir_fn=None, iir_prefill_style="modal-fft", layer_idx=None,
+                 ground_truth_activations_path=None, print_activations=False, hyena_flip_x1x2=False) -> None:
+        self.fir_fn = fir_fn
+        assert iir_prefill_style in IIR_PREFILL_MODES, f"iir_prefill_style must be one of {IIR_PREFILL_MODES}"
+        self.iir_prefill_style = iir_prefill_style
+        self.layer_idx = layer_idx
+        self.low_mem_mode = False
+        self.ground_truth_activations_path = ground_truth_activations_path
+        self.print_activations = print_activations
+        self.hyena_flip_x1x2 = hyena_flip_x1x2
+        self._plans = {}
+        self._poles = {}
+
+    # ------------------------------------------------------------------ prefill FIR
+    def parallel_fir(self, fir_fn, u, weight, bias, L, dims, groups=None, gated_bias=False,
+                     column_split_hyena=False, dim_last=True, fir_length=3, gate=False,
+                     inference_params=None, prefill_mode=None, padding_mask=None):
+        """vortex/model/engine.py:131-260.  Returns (z [B, D, L], fir_state or None)."""
+        if fir_fn is not None and fir_fn is not torch.nn.functional.conv1d:
+            raise NotImplementedError("custom fir_fn callables (deprecated in vortex) are not supported")
+        if u.dtype != torch.bfloat16:
+            raise TypeError(f"the gfx950 Hyena kernels take bfloat16 activations, got {u.dtype}")
+        K = fir_length
+        if gate:
+            hidden, n_heads, head_dim = dims[0], dims[1], dims[2]
+            if dim_last:
+                raise NotImplementedError("gated FIR expects the [B, 3D, L] layout (dim_last=False)")
+            B, _, L = u.shape
+            hd = head_dim if column_split_hyena else None
+            r2, r1, rv = (ops.rows_of_projection(u, hidden, i, hd) for i in range(3))
+            if self.hyena_flip_x1x2:
+                r1, r2 = r2, r1
+            D = hidden
+            taps = _group_taps(weight, D, groups)
+            if K >= 128:
+                # true convolution with the fp32 `+ D*u` term (engine.py:174-187, :78)
+                mode = HYENA_BIAS_NONE if bias is None else HYENA_BIAS_GATED_FP32
+                z = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, taps.shape[1], device=u.device,
+                                     bias=ops._f32(bias), bias_mode=mode, taps_reversed=False, force_mfma=True)
+            else:
+                if bias is not None and gated_bias:
+                    raise NotImplementedError("gated bias on the short-FIR branch has no kernel")
+                mode = HYENA_BIAS_NONE if bias is None else HYENA_BIAS_ADD
+                z = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, taps.shape[1], device=u.device,
+                                     bias=ops._f32(bias), bias_mode=mode, taps_reversed=True)
+            state = None
+            if inference_params is not None:
+                x1, v = self._gate_tails(u, hidden, hd, K - 1)
+                state = x1 * v
+        else:
+            if bias is not None and bias.dtype != torch.bfloat16:
+                raise NotImplementedError("a float32 short-filter bias promotes the output to float32 in vortex; "
+                                          "only bfloat16 (or no) bias is supported")
+            if dim_last:
+                B, L, C = u.shape
+                taps = _group_taps(weight, C, groups)
+                z = ops.featurizer_fwd(u, taps, bias)                      # [B, C, L], fused transpose
+                ut = u.permute(0, 2, 1)
+            else:
+                B, C, L = u.shape
+                taps = _group_taps(weight, C, groups)
+                mode = HYENA_BIAS_NONE if bias is None else HYENA_BIAS_ADD
+                z = ops.fir_fwd_rows(ops.rows_of(u), None, None, taps, B, C, L, taps.shape[1], device=u.device,
+                                     bias=ops._f32(bias), bias_mode=mode, taps_reversed=True)
+                ut = u
+            state = ut[..., -K + 1:] if inference_params is not None else None
+        if isinstance(padding_mask, torch.Tensor):
+            z = z * padding_mask[:, None].to(z.dtype)      # 0/1 masks commute exactly with the gate
+        return z, state
+
+    def _gate_tails(self, u, hidden, head_dim, n):
+        t = u[..., -n:]
+        if head_dim is None:
+            x2, x1, v = t.split([hidden, hidden, hidden], dim=1)
+        else:
+            tr = t.reshape(t.shape[0], -1, 3, head_dim, t.shape[-1])
+            x2, x1, v = (tr[:, :, i].reshape(t.shape[0], hidden, t.shape[-1]) for i in range(3))
+        if self.hyena_flip_x1x2:
+            x1, x2 = x2, x1
+        return x1, v
+
+    # ------------------------------------------------------------------ prefill IIR
+    def _plan(self, poles, residues):
+        key = (poles.data_ptr(), poles._version, residues.data_ptr(), residues._version)
+        p = self._plans.get(key)
+        if p is None:
+            self._plans.clear()
+            p = self._plans[key] = ops.ModalPlan(poles, residues)
+        return p
+
+    def parallel_iir(self, z_pre, h, D, L, poles, residues, t, dims, layer_idx, inference_params=None,
+                     prefill_style="fft", fftconv_fn=None, padding_mask=None, use_flashfft=False,
+                     column_split_hyena=False, long_fir_threshold=None):
+        """vortex/model/engine.py:262-404.  `h` (the materialised filter) is not read: the kernel works
+        from `poles` (log-poles) and `residues` directly.  Returns y [B, L, D]; writes the modal state
+        into inference_params.state_dict[layer_idx]."""
+        if long_fir_threshold is not None:
+            raise NotImplementedError("long_fir_threshold (truncated bf16 FIR) is not supported")
+        if z_pre.dtype != torch.bfloat16:
+            raise TypeError(f"the gfx950 Hyena kernels take bfloat16 activations, got {z_pre.dtype}")
+        hidden, n_heads, head_dim = dims[0], dims[1], dims[2]
+        B, _, L = z_pre.shape
+        hd = head_dim if column_split_hyena else None
+        r2, r1, rv = (ops.rows_of_projection(z_pre, hidden, i, hd) for i in range(3))
+        if self.hyena_flip_x1x2:
+            r1, r2 = r2, r1
+        plan = self._plan(poles, residues)
+        want_state = inference_params is not None
+        out, _, state = ops.li_fwd_rows(r1, r2, rv, plan, D, B, hidden, L, device=z_pre.device,
+                                        want_state=want_state)
+        if want_state:
+            inference_params.state_dict[layer_idx] = state
+        return out.permute(0, 2, 1)
+
+    # ------------------------------------------------------------------ decode
+    def step_fir(self, u, fir_state, weight, bias=None, gated_bias=False, flip_filter=False):
+        """vortex/model/engine.py:406-449.  `fir_state` is the reference's [B, D, cache] tensor
+        (oldest first) on the first call and the FirRing this method returned afterwards."""
+        w = weight.detach().reshape(weight.shape[0], -1).to(torch.float32)
+        K = w.shape[-1]
+        if not isinstance(fir_state, ops.FirRing):
+            fir_state = ops.FirRing.from_reference(fir_state)
+        cache = fir_state.shape[-1]
+        taps = (w.flip(-1)[..., -cache - 1:] if flip_filter else w[..., : cache + 1]).contiguous()
+        if cache < K - 1:
+            # short prompt: vortex grows the cache by one sample per step (engine.py:443-444)
+            if cache == 0:
+                raise NotImplementedError("decode from an empty FIR cache is not supported")
+            ref = fir_state.reference_order(torch.bfloat16)
+            y = ops.fir_step(u, fir_state, taps, bias=bias, gated_bias=gated_bias)
+            return y, ops.FirRing.from_reference(torch.cat([ref, u[..., None].to(ref.dtype)], dim=-1))
+        y = ops.fir_step(u, fir_state, taps, bias=bias, gated_bias=gated_bias)
+        return y, fir_state
+
+    def step_iir(self, x2, x1, v, D, residues, poles, iir_state, iir_groups=1):
+        """vortex/model/engine.py:451-467.  The state is updated in place and returned; y is float32
+        as torch promotion makes it in the reference."""
+        if iir_groups > 1:
+            raise NotImplementedError
+        key = (poles.data_ptr(), poles._version)
+        p = self._poles.get(key)
+        if p is None:
+            self._poles.clear()
+            p = self._poles[key] = torch.exp(poles.detach())[..., 0].contiguous()
+        if not iir_state.is_contiguous():
+            iir_state = iir_state.contiguous()
+        y = ops.iir_step(x1, x2, v, iir_state, p, residues.detach(), D, out_dtype=torch.float32)
+        return y, iir_state

@@ -130,6 +130,27 @@ def hyena_mr_fwd(x1, x2, v, h, D_bias=None):
                         bias_mode=_bias_mode(b, True, True), taps_reversed=False, force_mfma=True)
 
 
+def featurizer_fwd(u, taps, bias=None, interleave=False):
+    """Featurizer short FIR on the channel-last projection: u [B, L, C] bf16 -> z [B, C, L] bf16.
+
+    taps: [G, K] float32 in vortex's short-filter orientation (taps[:, K-1] on the current
+    sample), G = C or a divisor of C.  bias: [C] or None (added after the bf16 rounding of the
+    convolution, vortex/model/engine.py:208-223).  interleave=True also applies
+    vortex/model/utils.py:26-38 (channels 0::3 | 1::3 | 2::3) while writing.
+    """
+    _need_cuda(u, taps)
+    if u.dtype != torch.bfloat16 or u.dim() != 3 or u.stride(2) != 1:
+        raise ValueError("expected a [B, L, C] bfloat16 tensor with contiguous channels")
+    B, L, C = u.shape
+    taps = _f32(taps)
+    out = torch.empty((B, C, L), dtype=torch.bfloat16, device=u.device)
+    b = _f32(bias)
+    rc = _lib.lib().hyena_featurizer_fwd(_ptr(u), u.stride(0), u.stride(1), _ptr(taps), _ptr(b), int(interleave), _ptr(out),
+                                         B, L, C, taps.shape[0], taps.shape[1], _stream())
+    _lib.check(rc, "hyena_featurizer_fwd")
+    return out
+
+
 class ModalPlan:
     """Device-side coefficient tables of one modal filter bank (see hyena_li_plan)."""
 
