@@ -33,6 +33,8 @@ def parse():
     ap.add_argument("--workload", default="mr", choices=["mr", "se", "li", "decode"])
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 1 GiB device copy (calibration of FETCH_SIZE / WRITE_SIZE counters)")
     return ap.parse_args()
 
 
@@ -185,6 +187,19 @@ def main():
                  hbm_gbs=d["bytes"] / (ms * 1e-3) / 1e9)
         torch.cuda.empty_cache()
         return d
+
+    if args.copy_probe:
+        a = torch.empty(1 << 29, dtype=torch.bfloat16, device=device).normal_()
+        b = torch.empty_like(a)
+        from vortex_amd import _lib
+        stream = torch.cuda.current_stream().cuda_stream
+        nbytes = a.numel() * 2
+        wall, ms = time_steps(lambda: _lib.check(_lib.lib().hyena_copy_probe(a.data_ptr(), b.data_ptr(), nbytes,
+                                                                             stream), "copy"), 5, 2)
+        print(f"copy probe (copy_probe_kernel, 16 B/lane): 1 GiB read + 1 GiB written per launch, "
+              f"{ms * 1e3:.1f} us, {2 * nbytes / (ms * 1e-3) / 1e9:.0f} GB/s", file=sys.stderr)
+        del a, b
+        torch.cuda.empty_cache()
 
     main_name = args.workload if args.workload != "decode" else "mr"
     m = run(main_name, args.steps, args.warmup)

@@ -49,6 +49,11 @@ enum hyena_bias_mode {
 const char* hyena_version(void);
 const char* hyena_last_error_string(void);
 
+/* Plain device-to-device copy of nbytes (multiple of 16) with the kernels' own access shape,
+ * 16 bytes per lane.  No counterpart in the reference: it is the calibration launch for
+ * hardware traffic counters and the bandwidth yardstick printed by bench.py. */
+int hyena_copy_probe(const void* src, void* dst, int64_t nbytes, void* stream);
+
 /* Hyena-SE: gated causal depthwise short FIR (2 <= K <= 8), direct form.
  * Replaces HyenaInferenceEngine.parallel_fir, K < 128 branch
  * (vortex/model/engine.py:131-260, body :188-232):

@@ -13,7 +13,7 @@ HYENA_BIAS_NONE, HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32 = 0, 1, 2
 
 EXPORTS = [
     "hyena_version", "hyena_last_error_string", "hyena_se_fwd", "hyena_mr_fwd",
-    "hyena_fir_step", "hyena_iir_step", "hyena_li_plan_bytes", "hyena_li_plan", "hyena_li_fwd", "hyena_featurizer_fwd",
+    "hyena_fir_step", "hyena_iir_step", "hyena_li_plan_bytes", "hyena_li_plan", "hyena_li_fwd", "hyena_featurizer_fwd", "hyena_copy_probe",
 ]
 
 
@@ -52,6 +52,7 @@ def lib():
                                c_int64, c_int64, c_int64, c_void_p]
     L.hyena_featurizer_fwd.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int64,
                                        c_int64, c_int64, c_int64, c_int, c_void_p]
+    L.hyena_copy_probe.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
     for name in EXPORTS:
         fn = getattr(L, name)
         if name not in ("hyena_version", "hyena_last_error_string"):
