@@ -33,19 +33,21 @@ __device__ __forceinline__ uint32_t pack_bf2(float lo, float hi) {
 __device__ __forceinline__ uint32_t f_to_bf_bits(float f) { return pack_bf2(f, 0.f) & 0xffffu; }
 __device__ __forceinline__ float round_bf(float f) { return __uint_as_float(pack_bf2(f, 0.f) << 16); }
 
-struct RowMap {            // device copy of hyena_rows
+struct RowMap {            // device copy of hyena_rows; channel arithmetic in 32 bits (64-bit division is emulated)
     const bf16_t* ptr;
-    int64_t batch_stride, row_stride, ch_inner, ch_outer;
+    int64_t batch_stride, row_stride;
+    uint32_t ch_inner, ch_outer;
     __device__ __forceinline__ const bf16_t* row(int64_t b, int64_t d) const {
-        int64_t r = (d / ch_inner) * ch_outer + (d % ch_inner);
-        return ptr + b * batch_stride + r * row_stride;
+        const uint32_t du = (uint32_t)d;
+        const uint32_t r = (du < ch_inner) ? du : (du / ch_inner) * ch_outer + (du % ch_inner);
+        return ptr + b * batch_stride + (int64_t)r * row_stride;
     }
 };
 
 static inline RowMap make_rowmap(const hyena_rows* r) {
     RowMap m;
     if (r) { m.ptr = (const bf16_t*)r->ptr; m.batch_stride = r->batch_stride; m.row_stride = r->row_stride;
-             m.ch_inner = r->ch_inner; m.ch_outer = r->ch_outer; }
+             m.ch_inner = (uint32_t)r->ch_inner; m.ch_outer = (uint32_t)r->ch_outer; }
     else   { m.ptr = nullptr; m.batch_stride = m.row_stride = 0; m.ch_inner = m.ch_outer = 1; }
     return m;
 }
@@ -57,6 +59,7 @@ int hyena_check_launch(const char* what);
 static inline bool rows_aligned8(const hyena_rows* r) {
     return r == nullptr || ((((uintptr_t)r->ptr) & 15) == 0 && r->batch_stride % 8 == 0 && r->row_stride % 8 == 0);
 }
-static inline bool rows_valid(const hyena_rows* r, int64_t D) {
-    return r->ptr != nullptr && r->ch_inner > 0 && r->ch_outer >= 0 && D % r->ch_inner == 0 || (r->ch_inner >= D);
+static inline bool rows_valid(const hyena_rows* r) {
+    return r == nullptr || (r->ptr != nullptr && r->ch_inner > 0 && r->ch_inner < (1LL << 31) && r->ch_outer >= 0 &&
+                            r->ch_outer < (1LL << 31));
 }

@@ -4,43 +4,63 @@
 //   chunk c (128 samples):  y_c = T * u_c  +  Pout * X_c ,   X_{c+1} = p^128 (.) X_c + Pin * u_c
 //
 //   T    [128 x 128]  lower-triangular Toeplitz of the filter head h[0..127]
-//   Pin  [2S  x 128]  rows (Re, Im) of p_s^(127-j): the chunk's contribution to the state
-//   Pout [128 x 2S ]  (Re, -Im) of r_s p_s^(i+1):  what the incoming state adds to sample i
+//   Pin  [2S  x 128]  (Re, Im) of p_s^(127-j): the chunk's contribution to the state
+//   Pout [128 x 2S ]  (Re, -Im) of r_s p_s^(i+1): what the incoming state adds to sample i
 //   X_c  [2S]         complex modal state after the samples before chunk c
 //
-// All three contractions run on bf16 MFMA with fp32 accumulation.  To keep the
-// fp32 long-convolution output within 1e-4 of an fp32 evaluation, every fp32
-// coefficient is split into two bf16 terms (hi + lo) and the state, which is not
-// bf16-exact, is split as well (hi*hi + hi*lo + lo*hi); the inputs u = bf16(x1*v)
-// are exact.  The state recurrence itself is carried in fp32 registers.  The final
-// X is the decode state of vortex/model/engine.py:525-559 for free.
+// All three contractions run on v_mfma_f32_16x16x32_bf16 with fp32 accumulation.  To keep the
+// fp32 long-convolution output within 1e-4 of an fp32 evaluation, every fp32 coefficient is
+// split into two bf16 terms (hi + lo) and the state, which is not bf16-exact, is split as well
+// (hi*hi + hi*lo + lo*hi); the inputs u = bf16(x1*v) are exact.  The recurrence itself is carried
+// in fp32 registers.  The final X is the decode state of vortex/model/engine.py:525-559 for free.
 //
-// One block (4 wavefronts) owns 16 channels of one filter group and walks the
-// whole sequence in 512-sample steps (4 chunks); global traffic is the same
-// coalesced 16 B/lane pattern as the Hyena-MR kernel: x1, v, x2 read once, out
-// written once.
+// Work decomposition: a WAVEFRONT owns 4 channels of one filter group and walks the whole
+// sequence alone, 512 samples (4 chunks) per step.  The 16 MFMA columns are 4 channels x 4
+// chunks, so one B fragment serves all four chunks of the step; the 64 lanes hold the 4 x 16
+// complex states of the scan, one each.  Nothing is shared between wavefronts: there is no
+// block barrier anywhere, only the in-order LDS pipe of the wavefront itself, and the four
+// wavefronts of a CU drift apart and cover each other's memory latency.  Global traffic is
+// coalesced 16 B per lane (1 KiB per row and instruction), prefetched PF steps ahead in registers.
 #include "common.h"
 
 namespace {
 
-constexpr int TL = 512;
+constexpr int TL = 512;        // samples per step
 constexpr int C = 128;         // chunk
-constexpr int URS = 520;       // u_lds / z_lds row stride (elements): 1040 B = 16 * 65
 constexpr int S = 16;          // modal state size (poles per group)
-constexpr int R2 = 2 * S;      // real rows of the state
+constexpr int R2 = 2 * S;      // real rows of the state, row 2*pole + (0: Re, 1: Im)
 
-// workspace layout per group (floats)
-constexpr int WS_HEAD = 0;                 // [128]
-constexpr int WS_PIN = WS_HEAD + C;        // [32][128]
-constexpr int WS_POUT = WS_PIN + R2 * C;   // [128][32]
-constexpr int WS_PC = WS_POUT + C * R2;    // [16][2]
-constexpr int WS_PINV = WS_PC + 2 * S;     // [16][2]  1/p
-constexpr int WS_GROUP = WS_PINV + 2 * S;  // 8384 floats
+// per-wavefront LDS slices (elements)
+constexpr int CHS = 160;                 // chunk stride inside a row: 128 samples + 64 B pad
+constexpr int URS = 4 * CHS + 8;         // row stride 648 elements = 1296 B (odd multiple of 16 B)
+constexpr int LRS = R2 + 4;              // row of chunk contributions: 32 floats + 16 B pad
+constexpr int XRS = R2 + 8;              // row of split states: 32 bf16 + 16 B pad
+constexpr int WAVE_LDS_BYTES = 2 * 4 * URS * 2 + 16 * LRS * 4 + 2 * 16 * XRS * 2;   // u, z, l, xh, xl
+
+// Workspace per group: 48 MFMA A-operand fragments, already split into bf16 hi / lo terms and laid
+// out per lane (64 lanes x 16 B each), then p^128 and p^-1.
+//   [ 0.. 7] Toeplitz hi, index 2*delta + ib    [ 8..15] Toeplitz lo      (delta = 0..3 superblocks back)
+//   [16..23] Pout hi, index 2*Sigma + ib        [24..31] Pout lo
+//   [32..39] Pin  hi, index 4*mu + kappa        [40..47] Pin  lo
+constexpr int FR_T = 0, FR_PO = 16, FR_PI = 32, N_FRAG = 48;
+constexpr int WS_FRAG_FLOATS = N_FRAG * 64 * 4;    // 12288 dwords
+constexpr int WS_PC = WS_FRAG_FLOATS;              // [16][2]  p^128
+constexpr int WS_PINV = WS_PC + 2 * S;             // [16][2]  1/p
+constexpr int WS_GROUP = WS_PINV + 2 * S;          // 12352 floats
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) {
     union { u32x4 u; bf16x8 b; } c;
     c.u = x;
     return c.b;
+}
+
+template <bool NT>
+__device__ __forceinline__ u32x4 ld16(const bf16_t* p) {
+    return NT ? __builtin_nontemporal_load((const u32x4*)p) : *(const u32x4*)p;
+}
+template <bool NT>
+__device__ __forceinline__ void st16(bf16_t* p, u32x4 v) {
+    if (NT) __builtin_nontemporal_store(v, (u32x4*)p); else *(u32x4*)p = v;
 }
 
 template <bool PRE>
@@ -52,26 +72,28 @@ __device__ __forceinline__ u32x4 gate_mul(u32x4 a, u32x4 b) {
     return r;
 }
 
-// hi/lo bf16 split of eight fp32 values produced by f(e), e = 0..7
-template <typename F>
-__device__ __forceinline__ void split8(F f, bf16x8& hi, bf16x8& lo) {
-    u32x4 ph, pl;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const float a = f(2 * j), b = f(2 * j + 1);
-        const float ah = round_bf(a), bh = round_bf(b);
-        ph[j] = (__float_as_uint(ah) >> 16) | (__float_as_uint(bh) & 0xffff0000u);
-        pl[j] = pack_bf2(a - ah, b - bh);
-    }
-    hi = as_bf16x8(ph);
-    lo = as_bf16x8(pl);
+// LDS traffic of one wavefront is in order in hardware; this only stops the compiler from moving
+// LDS accesses of different lanes across the hand-off points.
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Sample (inside a 32-sample superblock) that MFMA row m of half-block ib stands for.  Feeding the
+// A rows in this order makes lane quad q of the 16x16 accumulators own samples 8q..8q+7.
+__device__ __forceinline__ int li_sample(int ib, int m) { return 8 * (m >> 2) + 4 * ib + (m & 3); }
+
 // ------------------------------------------------------------------ plan kernel
-// One block per group; coefficients evaluated in double from the fp32 parameters.
+// One block per group; coefficients evaluated in double from the fp32 parameters, then cut into
+// the per-lane fragments the main kernel loads with one 16-byte read each.
+// 16x16x32 A operand: lane holds row m = lane & 15, k = 8*(lane >> 4) + e, e = 0..7.
 __global__ __launch_bounds__(256) void li_plan_kernel(const float* __restrict__ log_poles,   // [G][S][2]
                                                       const float* __restrict__ residues,    // [G][S][2]
                                                       float* __restrict__ ws) {
+    __shared__ float head[C];
+    __shared__ float pin[R2 * C];       // [row 2s+part][j]
+    __shared__ float pout[C * R2];      // [i][row 2s+part]
     const int g = blockIdx.x, tid = threadIdx.x;
     float* w = ws + (size_t)g * WS_GROUP;
     const float* lp = log_poles + (size_t)g * S * 2;
@@ -83,25 +105,25 @@ __global__ __launch_bounds__(256) void li_plan_kernel(const float* __restrict__ 
         re = m * cos(a);
         im = m * sin(a);
     };
-    if (tid < C) {                                  // filter head
+    if (tid < C) {                                  // filter head h[0..127]
         double acc = 0.0;
         for (int s = 0; s < S; ++s) {
             double re, im;
             ppow(s, tid, re, im);
             acc += (double)rs[2 * s] * re - (double)rs[2 * s + 1] * im;
         }
-        w[WS_HEAD + tid] = (float)acc;
+        head[tid] = (float)acc;
     }
     for (int e = tid; e < S * C; e += 256) {        // Pin and Pout
         const int s = e / C, j = e - s * C;
         double re, im;
         ppow(s, C - 1 - j, re, im);
-        w[WS_PIN + s * C + j] = (float)re;
-        w[WS_PIN + (S + s) * C + j] = (float)im;
+        pin[(2 * s) * C + j] = (float)re;
+        pin[(2 * s + 1) * C + j] = (float)im;
         ppow(s, j + 1, re, im);                     // here j plays the role of the output sample i
         const double rr = rs[2 * s], ri = rs[2 * s + 1];
-        w[WS_POUT + j * R2 + s] = (float)(rr * re - ri * im);          //  Re(r p^(i+1))
-        w[WS_POUT + j * R2 + S + s] = (float)(-(rr * im + ri * re));   // -Im(r p^(i+1))
+        pout[j * R2 + 2 * s] = (float)(rr * re - ri * im);            //  Re(r p^(i+1))
+        pout[j * R2 + 2 * s + 1] = (float)(-(rr * im + ri * re));     // -Im(r p^(i+1))
     }
     if (tid < S) {
         double re, im;
@@ -111,6 +133,40 @@ __global__ __launch_bounds__(256) void li_plan_kernel(const float* __restrict__ 
         ppow(tid, -1, re, im);
         w[WS_PINV + 2 * tid] = (float)re;
         w[WS_PINV + 2 * tid + 1] = (float)im;
+    }
+    __syncthreads();
+    u32x4* fr = (u32x4*)w;
+    for (int e = tid; e < 24 * 64; e += 256) {      // 24 (hi, lo) fragment pairs
+        const int f = e >> 6, lane = e & 63;
+        const int m = lane & 15, qa = lane >> 4;
+        float val[8];
+        if (f < 8) {                                // Toeplitz: rows of (superblock Sigma, half ib) x inputs of block J
+            const int delta = f >> 1, ib = f & 1;   // delta = Sigma - J
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int lag = 32 * delta + li_sample(ib, m) - (8 * qa + k);
+                val[k] = (lag >= 0 && lag < C) ? head[lag] : 0.f;
+            }
+        } else if (f < 16) {                        // Pout rows of (Sigma, ib), all 32 state rows in one k-step
+            const int Sg = (f - 8) >> 1, ib = (f - 8) & 1;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) val[k] = pout[(32 * Sg + li_sample(ib, m)) * R2 + 8 * qa + k];
+        } else {                                    // Pin state rows 16*mu + m, inputs 32*kappa + 8*qa + k
+            const int mu = (f - 16) >> 2, kp = (f - 16) & 3;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) val[k] = pin[(16 * mu + m) * C + 32 * kp + 8 * qa + k];
+        }
+        u32x4 ph, pl;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float a = val[2 * j], b = val[2 * j + 1];
+            const float ah = round_bf(a), bh = round_bf(b);
+            ph[j] = (__float_as_uint(ah) >> 16) | (__float_as_uint(bh) & 0xffff0000u);
+            pl[j] = pack_bf2(a - ah, b - bh);
+        }
+        const int base = f < 8 ? FR_T + f : (f < 16 ? FR_PO + (f - 8) : FR_PI + (f - 16));
+        fr[(base) * 64 + lane] = ph;
+        fr[(base + 8) * 64 + lane] = pl;
     }
 }
 
@@ -125,247 +181,231 @@ struct LiArgs {
     int64_t D, L;
     int dg;
     int d_is_bf16;
+    int64_t nquads;           // B * D / 4 wavefront-sized work items
 };
 
-template <int W, bool PRE, bool POST>
-__device__ __forceinline__ void li_body(const LiArgs& a, bf16_t* u_lds, bf16_t* z_lds, float* l_lds, bf16_t* xh_lds,
-                                        bf16_t* xl_lds) {
+#define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0)
+
+template <bool PRE, bool POST, bool NT, int PF>
+__global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds_all[4 * WAVE_LDS_BYTES];
     const int tid = threadIdx.x, lane = tid & 63;
-    const int64_t nslab = a.D / 16;
-    const int64_t slab = blockIdx.x % nslab, b = blockIdx.x / nslab;
-    const int64_t d0 = slab * 16;
-    const int g = (int)(d0 / a.dg);
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t quad = (int64_t)blockIdx.x * 4 + w;          // 4 channels of one batch element
+    if (quad >= a.nquads) return;                              // whole wavefront leaves; no barriers below
+    const uint32_t qpb = (uint32_t)(a.D / 4);
+    const int64_t b = (uint32_t)quad / qpb;
+    const int64_t d0 = (int64_t)((uint32_t)quad % qpb) * 4;
+    const int g = (int)((uint32_t)d0 / (uint32_t)a.dg);
     const float* ws = a.ws + (size_t)g * WS_GROUP;
     const int64_t L = a.L;
 
-    // ---- A fragments -----------------------------------------------------------------
-    const int n = lane & 31, hh = lane >> 5;
-    const int i_time = 16 * ((n >> 2) & 1) + 4 * (n >> 3) + (n & 3);   // sample owned through MFMA row n
-    bf16x8 Th[8], Tl[8];                 // Toeplitz blocks, delta = -1..6 at index delta+1
-#pragma unroll
-    for (int q = 0; q < 8; ++q) {
-        split8([&](int e) {
-            const int lag = 16 * (q - 1) + i_time - (8 * hh + e);
-            return (lag >= 0 && lag < C) ? ws[WS_HEAD + lag] : 0.f;
-        }, Th[q], Tl[q]);
-    }
-    constexpr int I0 = W, I1 = 3 - W;    // 32-row output blocks of this wavefront (column group 0 / 1)
-    bf16x8 Poh[2][2], Pol[2][2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int k = 0; k < 2; ++k)
-            split8([&](int e) { return ws[WS_POUT + (32 * (t ? I1 : I0) + i_time) * R2 + 16 * k + 8 * hh + e]; },
-                   Poh[t][k], Pol[t][k]);
-    const int m16 = lane & 15, q4 = lane >> 4;
-    bf16x8 Pih[2][4], Pil[2][4];
-#pragma unroll
-    for (int mu = 0; mu < 2; ++mu)
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-            split8([&](int e) { return ws[WS_PIN + (16 * mu + m16) * C + 32 * k + 8 * q4 + e]; }, Pih[mu][k],
-                   Pil[mu][k]);
+    unsigned char* lds = lds_all + w * WAVE_LDS_BYTES;
+    bf16_t* u_w = (bf16_t*)lds;                                // [4][URS]
+    bf16_t* z_w = u_w + 4 * URS;                               // [4][URS]
+    float* l_w = (float*)(z_w + 4 * URS);                      // [4 chunks][4 ch][LRS]
+    bf16_t* xh_w = (bf16_t*)(l_w + 16 * LRS);                  // [4][4][XRS]
+    bf16_t* xl_w = xh_w + 16 * XRS;
 
-    // ---- state owned by this thread: channel sc, pole ss
-    const int sc = tid >> 4, ss = tid & 15;
+    // ---- A fragments: one 16-byte load each, pinned in registers for the whole kernel
+    const u32x4* fr = (const u32x4*)ws + lane;
+    bf16x8 Th[8], Tl[8], Poh[8], Pol[8], Pih[8], Pil[8];
+    {
+        u32x4 t;
+#define LI_FRAG(dst, idx) t = fr[(idx) * 64]; asm volatile("" : "+v"(t)); dst = as_bf16x8(t);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            LI_FRAG(Th[q], FR_T + q) LI_FRAG(Tl[q], FR_T + 8 + q)
+            LI_FRAG(Poh[q], FR_PO + q) LI_FRAG(Pol[q], FR_PO + 8 + q)
+            LI_FRAG(Pih[q], FR_PI + q) LI_FRAG(Pil[q], FR_PI + 8 + q)
+        }
+#undef LI_FRAG
+    }
+
+    // MFMA-side lane geometry: column n = channel c + 4 * chunk s, k / row quad q
+    const int n = lane & 15, q = lane >> 4;
+    const int c = n & 3, s = n >> 2;
+    // scan-side lane geometry: one complex state per lane
+    const int sc = lane >> 4, sp = lane & 15;
     float Xr = 0.f, Xi = 0.f;
-    const float pcr = ws[WS_PC + 2 * ss], pci = ws[WS_PC + 2 * ss + 1];
-
-    // ---- coalesced layout: 16 B of rows 4*r4 + W
-    const bf16_t *p1[4], *pv[4], *p2[4];
-    bf16_t* po[4];
-#pragma unroll
-    for (int r4 = 0; r4 < 4; ++r4) {
-        const int64_t d = d0 + 4 * r4 + W;
-        p1[r4] = a.x1.row(b, d) + lane * 8;
-        pv[r4] = PRE ? a.v.row(b, d) + lane * 8 : nullptr;
-        p2[r4] = POST ? a.x2.row(b, d) + lane * 8 : nullptr;
-        po[r4] = a.out + (b * a.D + d) * L + lane * 8;
-    }
-    const u32x4 zero4 = {0, 0, 0, 0};
-    u32x4 c1[4], cv[4];
-#pragma unroll
-    for (int r4 = 0; r4 < 4; ++r4) {
-        const bool ok = lane * 8 < L;
-        c1[r4] = ok ? *(const u32x4*)(p1[r4]) : zero4;
-        cv[r4] = (PRE && ok) ? *(const u32x4*)(pv[r4]) : zero4;
-    }
-    const int c = n & 15, s = n >> 4;
+    const float pcr = ws[WS_PC + 2 * sp], pci = ws[WS_PC + 2 * sp + 1];
     float dco = 0.f;
     if (a.Dcoef) dco = a.Dcoef[d0 + c];
 
-    for (int64_t ts = 0; ts < L; ts += TL) {
+    // ---- coalesced layout: lane moves samples 8*lane..8*lane+7 of each of the 4 rows
+    const int lofs = lane * 8 + 32 * (lane >> 4);              // position inside a padded LDS row
+    const bf16_t *p1[4], *pv[4], *p2[4];
+    bf16_t* po[4];
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4)
-            *(u32x4*)(u_lds + (4 * r4 + W) * URS + lane * 8) = gate_mul<PRE>(c1[r4], cv[r4]);
-        __syncthreads();                                                      // (1) u ready
-
-        u32x4 c2[4];
-        {
-            const int64_t tn = ts + TL;
-            const bool okn = tn + lane * 8 < L, okc = ts + lane * 8 < L;
+    for (int r = 0; r < 4; ++r) {
+        p1[r] = a.x1.row(b, d0 + r) + lane * 8;
+        pv[r] = PRE ? a.v.row(b, d0 + r) + lane * 8 : nullptr;
+        p2[r] = POST ? a.x2.row(b, d0 + r) + lane * 8 : nullptr;
+        po[r] = a.out + (b * a.D + d0 + r) * L + lane * 8;
+    }
+    const u32x4 zero4 = {0, 0, 0, 0};
+    u32x4 c1[PF][4], cv[PF][4], c2[PF][4];
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                c1[r4] = okn ? *(const u32x4*)(p1[r4] + tn) : zero4;
-                cv[r4] = (PRE && okn) ? *(const u32x4*)(pv[r4] + tn) : zero4;
-                c2[r4] = (POST && okc) ? *(const u32x4*)(p2[r4] + ts) : zero4;
-            }
+    for (int p = 0; p < PF; ++p)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int64_t t = (int64_t)p * TL;
+            const bool ok = t + lane * 8 < L;
+            c1[p][r] = ok ? ld16<NT>(p1[r] + t) : zero4;
+            cv[p][r] = (PRE && ok) ? ld16<NT>(pv[r] + t) : zero4;
+            c2[p][r] = (POST && ok) ? ld16<NT>(p2[r] + t) : zero4;
         }
 
-        // ---- state-in of chunk W: Pin[32 x 128] * u_chunk[128 x 16], 16x16x32 MFMA
-        {
+    for (int64_t ts0 = 0; ts0 < L; ts0 += PF * TL) {
+#pragma unroll
+        for (int p = 0; p < PF; ++p) {
+            const int64_t ts = ts0 + (int64_t)p * TL;
+            if (ts >= L) break;
+            const int64_t tn = ts + (int64_t)PF * TL;          // step that reuses this register stage
+            const bool okn = tn + lane * 8 < L;
+
+            // u = bf16(x1*v) of this step -> LDS; refill the stage with step ts + PF*TL
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                *(u32x4*)(u_w + r * URS + lofs) = gate_mul<PRE>(c1[p][r], cv[p][r]);
+                c1[p][r] = okn ? ld16<NT>(p1[r] + tn) : zero4;
+                cv[p][r] = (PRE && okn) ? ld16<NT>(pv[r] + tn) : zero4;
+            }
+            wave_sync();
+
+            // B fragments: column (c, s) x inputs 32*J + 8*q.. of its chunk; shared by every MFMA below
+            bf16x8 bu[4];
+#pragma unroll
+            for (int J = 0; J < 4; ++J) bu[J] = *(const bf16x8*)(u_w + c * URS + s * CHS + 32 * J + 8 * q);
+
+            // ---- state-in: L[32 x 16 cols] = Pin[32 x 128] * u
             f32x4 l0 = {0, 0, 0, 0}, l1 = {0, 0, 0, 0};
-            const bf16_t* ub = u_lds + m16 * URS + C * W + 8 * q4;
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                const bf16x8 bf = *(const bf16x8*)(ub + 32 * k);
-                l0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Pih[0][k], bf, l0, 0, 0, 0);
-                l0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Pil[0][k], bf, l0, 0, 0, 0);
-                l1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Pih[1][k], bf, l1, 0, 0, 0);
-                l1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Pil[1][k], bf, l1, 0, 0, 0);
+                l0 = MFMA16(Pih[k], bu[k], l0);
+                l1 = MFMA16(Pih[4 + k], bu[k], l1);
+                l0 = MFMA16(Pil[k], bu[k], l0);
+                l1 = MFMA16(Pil[4 + k], bu[k], l1);
             }
-            // lane (column m16, quad q4) holds state rows 4*q4..+3 of each half
-            float* lp = l_lds + (W * 16 + m16) * R2 + 4 * q4;
-            *(f32x4*)lp = l0;
-            *(f32x4*)(lp + 16) = l1;
-        }
+            {   // lane (column n, quad q) holds state rows 4q..4q+3 of each half
+                float* lp = l_w + n * LRS + 4 * q;             // row index s*4 + c == n'  (n = c + 4s)
+                *(f32x4*)lp = l0;
+                *(f32x4*)(lp + 16) = l1;
+            }
 
-        // ---- Toeplitz: tile 0 = (column group 0, rows I0), tile 1 = (column group 1, rows I1)
-        f32x16 acc0, acc1;
+            // ---- Toeplitz: superblock Sigma (32 samples) x half ib, inputs J <= Sigma
+            f32x4 acc[4][2];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
-        {
-            const bf16_t* ub0 = u_lds + c * URS + C * s + 8 * hh;            // chunks 0,1
-            const bf16_t* ub1 = ub0 + 2 * C;                                  // chunks 2,3
+            for (int Sg = 0; Sg < 4; ++Sg)
 #pragma unroll
-            for (int J = 0; J <= 2 * I0 + 1; ++J) {
-                const bf16x8 bf = *(const bf16x8*)(ub0 + 16 * J);
-                acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Th[2 * I0 - J + 1], bf, acc0, 0, 0, 0);
-                acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Tl[2 * I0 - J + 1], bf, acc0, 0, 0, 0);
-            }
+                for (int ib = 0; ib < 2; ++ib) {
+                    f32x4 t = {0, 0, 0, 0};
 #pragma unroll
-            for (int J = 0; J <= 2 * I1 + 1; ++J) {
-                const bf16x8 bf = *(const bf16x8*)(ub1 + 16 * J);
-                acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Th[2 * I1 - J + 1], bf, acc1, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Tl[2 * I1 - J + 1], bf, acc1, 0, 0, 0);
-            }
-        }
-        __syncthreads();                                                      // (2) chunk contributions ready
+                    for (int J = 0; J <= Sg; ++J) {
+                        t = MFMA16(Th[2 * (Sg - J) + ib], bu[J], t);
+                        t = MFMA16(Tl[2 * (Sg - J) + ib], bu[J], t);
+                    }
+                    acc[Sg][ib] = t;
+                }
+            wave_sync();
 
-        // ---- state scan over the 4 chunks of this step (thread = one channel x one pole)
-        {
+            // ---- scan over the 4 chunks: lane = (channel sc, pole sp)
+            {
+                float lr[4], li[4];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const float xrh = round_bf(Xr), xih = round_bf(Xi);
-                const int o = (k * 16 + sc) * R2;
-                xh_lds[o + ss] = (bf16_t)(__float_as_uint(xrh) >> 16);
-                xh_lds[o + S + ss] = (bf16_t)(__float_as_uint(xih) >> 16);
-                xl_lds[o + ss] = (bf16_t)f_to_bf_bits(Xr - xrh);
-                xl_lds[o + S + ss] = (bf16_t)f_to_bf_bits(Xi - xih);
-                const float lr = l_lds[o + ss], li = l_lds[o + S + ss];
-                const float nr = fmaf(pcr, Xr, fmaf(-pci, Xi, lr));
-                const float ni = fmaf(pcr, Xi, fmaf(pci, Xr, li));
-                Xr = nr;
-                Xi = ni;
+                for (int k = 0; k < 4; ++k) {
+                    const float2 t = *(const float2*)(l_w + (k * 4 + sc) * LRS + 2 * sp);
+                    lr[k] = t.x;
+                    li[k] = t.y;
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float xrh = round_bf(Xr), xih = round_bf(Xi);
+                    const int o = (k * 4 + sc) * XRS + 2 * sp;
+                    *(uint32_t*)(xh_w + o) = (__float_as_uint(xrh) >> 16) | (__float_as_uint(xih) & 0xffff0000u);
+                    *(uint32_t*)(xl_w + o) = pack_bf2(Xr - xrh, Xi - xih);
+                    const float nr = fmaf(pcr, Xr, fmaf(-pci, Xi, lr[k]));
+                    const float ni = fmaf(pcr, Xi, fmaf(pci, Xr, li[k]));
+                    Xr = nr;
+                    Xi = ni;
+                }
             }
-        }
-        __syncthreads();                                                      // (3) chunk states ready
+            wave_sync();
 
-        // ---- state-out: Pout[rows x 32] * X[32 x columns], three bf16 products
-        {
-            const bf16_t* xb0h = xh_lds + ((0 + s) * 16 + c) * R2 + 8 * hh;
-            const bf16_t* xb0l = xl_lds + ((0 + s) * 16 + c) * R2 + 8 * hh;
-            const bf16_t* xb1h = xh_lds + ((2 + s) * 16 + c) * R2 + 8 * hh;
-            const bf16_t* xb1l = xl_lds + ((2 + s) * 16 + c) * R2 + 8 * hh;
+            // ---- state-out: acc += Pout[rows x 32] * X[32 x cols], three bf16 products
+            {
+                const bf16x8 xh = *(const bf16x8*)(xh_w + n * XRS + 8 * q);     // row s*4 + c == n
+                const bf16x8 xl = *(const bf16x8*)(xl_w + n * XRS + 8 * q);
 #pragma unroll
-            for (int k = 0; k < 2; ++k) {
-                const bf16x8 h0 = *(const bf16x8*)(xb0h + 16 * k), l0 = *(const bf16x8*)(xb0l + 16 * k);
-                acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Poh[0][k], h0, acc0, 0, 0, 0);
-                acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Poh[0][k], l0, acc0, 0, 0, 0);
-                acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Pol[0][k], h0, acc0, 0, 0, 0);
-                const bf16x8 h1 = *(const bf16x8*)(xb1h + 16 * k), l1 = *(const bf16x8*)(xb1l + 16 * k);
-                acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Poh[1][k], h1, acc1, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Poh[1][k], l1, acc1, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Pol[1][k], h1, acc1, 0, 0, 0);
-            }
-        }
-
-        // ---- epilogue: y = bf16(conv); z = bf16(y + bf16(D*u)) -> LDS (engine.py:352-353)
+                for (int Sg = 0; Sg < 4; ++Sg)
 #pragma unroll
-        for (int tau = 0; tau < 2; ++tau) {
-            const int tcol = C * (2 * tau + s) + 32 * (tau ? I1 : I0) + 16 * hh;
-            const f32x16 acc = tau ? acc1 : acc0;
-            if (a.y32) {
-                const int64_t t0 = ts + tcol;
-                float* yp = a.y32 + (b * a.D + d0 + c) * L + t0;
-#pragma unroll
-                for (int r = 0; r < 16; r += 4)
-                    if (t0 + r < L) {
-                        const f32x4 q = {acc[r], acc[r + 1], acc[r + 2], acc[r + 3]};
-                        *(f32x4*)(yp + r) = q;
+                    for (int ib = 0; ib < 2; ++ib) {
+                        f32x4 t = acc[Sg][ib];
+                        t = MFMA16(Poh[2 * Sg + ib], xh, t);
+                        t = MFMA16(Poh[2 * Sg + ib], xl, t);
+                        t = MFMA16(Pol[2 * Sg + ib], xh, t);
+                        acc[Sg][ib] = t;
                     }
             }
-            const u32x4 ua = *(const u32x4*)(u_lds + c * URS + tcol);
-            const u32x4 ub2 = *(const u32x4*)(u_lds + c * URS + tcol + 8);
-            u32x4 z0, z1;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint32_t uw = j < 4 ? ua[j] : ub2[j - 4];
-                float y0 = round_bf(acc[2 * j]), y1 = round_bf(acc[2 * j + 1]);
-                float t0 = dco * bf_lo(uw), t1 = dco * bf_hi(uw);
-                if (a.d_is_bf16) { t0 = round_bf(t0); t1 = round_bf(t1); }
-                const uint32_t p = pack_bf2(y0 + t0, y1 + t1);
-                if (j < 4) z0[j] = p; else z1[j - 4] = p;
-            }
-            *(u32x4*)(z_lds + c * URS + tcol) = z0;
-            *(u32x4*)(z_lds + c * URS + tcol + 8) = z1;
-        }
-        __syncthreads();                                                      // (4) z ready, u and X consumed
 
-        if (ts + lane * 8 < L) {
+            // ---- epilogue: y = bf16(conv); z = bf16(y + bf16(D*u)) -> LDS  (engine.py:352-353)
+            // lane (column (c, s), quad q) owns samples 32*Sigma + 8q .. +7 of chunk s
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const u32x4 zz = *(const u32x4*)(z_lds + (4 * r4 + W) * URS + lane * 8);
+            for (int Sg = 0; Sg < 4; ++Sg) {
+                const int tl = 32 * Sg + 8 * q;                 // inside the chunk
+                if (a.y32) {
+                    const int64_t t0 = ts + C * s + tl;
+                    if (t0 < L) {
+                        float* yp = a.y32 + (b * a.D + d0 + c) * L + t0;
+                        *(f32x4*)yp = acc[Sg][0];
+                        *(f32x4*)(yp + 4) = acc[Sg][1];
+                    }
+                }
+                const u32x4 uu = *(const u32x4*)(u_w + c * URS + s * CHS + tl);
+                u32x4 z;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const f32x4 av = acc[Sg][j >> 1];
+                    const float y0 = round_bf(av[2 * (j & 1)]), y1 = round_bf(av[2 * (j & 1) + 1]);
+                    float t0 = dco * bf_lo(uu[j]), t1 = dco * bf_hi(uu[j]);
+                    if (a.d_is_bf16) { t0 = round_bf(t0); t1 = round_bf(t1); }
+                    z[j] = pack_bf2(y0 + t0, y1 + t1);
+                }
+                *(u32x4*)(z_w + c * URS + s * CHS + tl) = z;
+            }
+            wave_sync();
+
+            // ---- gate with x2 and store, coalesced; refill x2 of the stage
+            const bool okc = ts + lane * 8 < L;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const u32x4 zz = *(const u32x4*)(z_w + r * URS + lofs);
                 u32x4 o = zz;
                 if (POST) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(c2[r4][j]), bf_hi(zz[j]) * bf_hi(c2[r4][j]));
+                        o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(c2[p][r][j]), bf_hi(zz[j]) * bf_hi(c2[p][r][j]));
                 }
-                *(u32x4*)(po[r4] + ts) = o;
+                if (okc) st16<NT>(po[r] + ts, o);
+                c2[p][r] = (POST && okn) ? ld16<NT>(p2[r] + tn) : zero4;
             }
+            wave_sync();      // z and u of this step are consumed before the next step overwrites them
         }
     }
 
     if (a.state_out) {
         // the scan ran over ceil(L/512)*512 samples with zero inputs past L: undo the padding, X *= p^-pad
         int pad = (int)(((L + TL - 1) / TL) * TL - L);
-        float qr = ws[WS_PINV + 2 * ss], qi = ws[WS_PINV + 2 * ss + 1];
-        float fr = 1.f, fi = 0.f;
+        float qr = ws[WS_PINV + 2 * sp], qi = ws[WS_PINV + 2 * sp + 1];
+        float fr_ = 1.f, fi = 0.f;
         while (pad) {
-            if (pad & 1) { const float t = fr * qr - fi * qi; fi = fr * qi + fi * qr; fr = t; }
+            if (pad & 1) { const float t = fr_ * qr - fi * qi; fi = fr_ * qi + fi * qr; fr_ = t; }
             const float t = qr * qr - qi * qi; qi = 2.f * qr * qi; qr = t;
             pad >>= 1;
         }
-        float* sp = a.state_out + ((b * a.D + d0 + sc) * S + ss) * 2;
-        sp[0] = Xr * fr - Xi * fi;
-        sp[1] = Xr * fi + Xi * fr;
-    }
-}
-
-template <bool PRE, bool POST>
-__global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
-    __shared__ __attribute__((aligned(16))) bf16_t u_lds[16 * URS];
-    __shared__ __attribute__((aligned(16))) bf16_t z_lds[16 * URS];
-    __shared__ __attribute__((aligned(16))) float l_lds[4 * 16 * R2];
-    __shared__ __attribute__((aligned(16))) bf16_t xh_lds[4 * 16 * R2];
-    __shared__ __attribute__((aligned(16))) bf16_t xl_lds[4 * 16 * R2];
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    switch (w) {
-        case 0: li_body<0, PRE, POST>(a, u_lds, z_lds, l_lds, xh_lds, xl_lds); break;
-        case 1: li_body<1, PRE, POST>(a, u_lds, z_lds, l_lds, xh_lds, xl_lds); break;
-        case 2: li_body<2, PRE, POST>(a, u_lds, z_lds, l_lds, xh_lds, xl_lds); break;
-        default: li_body<3, PRE, POST>(a, u_lds, z_lds, l_lds, xh_lds, xl_lds); break;
+        float* sp_ = a.state_out + ((b * a.D + d0 + sc) * S + sp) * 2;
+        sp_[0] = Xr * fr_ - Xi * fi;
+        sp_[1] = Xr * fi + Xi * fr_;
     }
 }
 
@@ -381,6 +421,7 @@ extern "C" int hyena_li_plan(const float* log_poles, const float* residues, int6
     if (!log_poles || !residues || !workspace) return hyena_fail(HYENA_EINVAL, "hyena_li_plan: null pointer");
     if (G <= 0 || G > 0x7fffffff) return hyena_fail(HYENA_EINVAL, "hyena_li_plan: bad G=%lld", (long long)G);
     if (S_ != S) return hyena_fail(HYENA_ENOSUP, "hyena_li_plan: state size %lld (only 16)", (long long)S_);
+    if (((uintptr_t)workspace) & 15) return hyena_fail(HYENA_EALIGN, "hyena_li_plan: workspace must be 16-byte aligned");
     hipLaunchKernelGGL(li_plan_kernel, dim3((unsigned)G), dim3(256), 0, (hipStream_t)stream, log_poles, residues,
                        (float*)workspace);
     return hyena_check_launch("hyena_li_plan");
@@ -395,15 +436,16 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
         return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: bad sizes B=%lld D=%lld L=%lld G=%lld", (long long)B,
                           (long long)D, (long long)L, (long long)G);
     if (S_ != S) return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: state size %lld (only 16)", (long long)S_);
-    if ((D / G) % 16 != 0)
-        return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: D/G=%lld must be a multiple of 16", (long long)(D / G));
+    if ((D / G) % 4 != 0)
+        return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: D/G=%lld must be a multiple of 4", (long long)(D / G));
     if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15) ||
-        (((uintptr_t)y_conv_fp32) & 15))
+        (((uintptr_t)y_conv_fp32) & 15) || (((uintptr_t)workspace) & 15))
         return hyena_fail(HYENA_EALIGN, "hyena_li_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
     if (B == 0 || L == 0) return 0;
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
-    const int64_t nblk = B * (D / 16);
-    if (nblk > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: problem too large for one launch");
+    const int64_t nquads = B * (D / 4);
+    const int64_t nblk = (nquads + 3) / 4;
+    if (nquads > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: problem too large for one launch");
     LiArgs a;
     a.x1 = make_rowmap(x1);
     a.x2 = make_rowmap(post ? x2 : nullptr);
@@ -417,10 +459,24 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     a.L = L;
     a.dg = (int)(D / G);
     a.d_is_bf16 = d_is_bf16;
+    a.nquads = nquads;
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)nblk);
-    if (pre && post) hipLaunchKernelGGL((li_kernel<true, true>), grid, dim3(256), 0, s, a);
-    else if (!pre && !post) hipLaunchKernelGGL((li_kernel<false, false>), grid, dim3(256), 0, s, a);
-    else return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: pass both v and x2 or neither");
+    bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
+    if (const char* e = getenv("HYENA_LI_NT")) nt = atoi(e) != 0;
+    int pf = 3;
+    if (const char* e = getenv("HYENA_LI_PF")) pf = atoi(e);
+#define LI_LAUNCH(P, Q, N, F) hipLaunchKernelGGL((li_kernel<P, Q, N, F>), grid, dim3(256), 0, s, a)
+#define LI_PF(P, Q, N) \
+    if (pf <= 1) LI_LAUNCH(P, Q, N, 1); else if (pf == 2) LI_LAUNCH(P, Q, N, 2); else LI_LAUNCH(P, Q, N, 3)
+    if (pre && post) {
+        if (nt) { LI_PF(true, true, true); } else { LI_PF(true, true, false); }
+    } else if (!pre && !post) {
+        if (nt) { LI_PF(false, false, true); } else { LI_PF(false, false, false); }
+    } else {
+        return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: pass both v and x2 or neither");
+    }
+#undef LI_PF
+#undef LI_LAUNCH
     return hyena_check_launch("hyena_li_fwd");
 }

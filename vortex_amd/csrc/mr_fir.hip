@@ -32,6 +32,16 @@ __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) {
     return c.b;
 }
 
+// streaming accesses: every activation is touched once, so keep it out of the caches' way
+template <bool NT>
+__device__ __forceinline__ u32x4 ld16(const bf16_t* p) {
+    return NT ? __builtin_nontemporal_load((const u32x4*)p) : *(const u32x4*)p;
+}
+template <bool NT>
+__device__ __forceinline__ void st16(bf16_t* p, u32x4 v) {
+    if (NT) __builtin_nontemporal_store(v, (u32x4*)p); else *(u32x4*)p = v;
+}
+
 template <bool PRE>
 __device__ __forceinline__ u32x4 gate_mul(u32x4 a, u32x4 b) {
     if (!PRE) return a;
@@ -41,7 +51,7 @@ __device__ __forceinline__ u32x4 gate_mul(u32x4 a, u32x4 b) {
     return r;
 }
 
-template <bool PRE, bool POST, int BIAS>
+template <bool PRE, bool POST, int BIAS, bool NT, bool FULL>
 __global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, RowMap v, const float* __restrict__ h,
                                                         int K, int reversed, const float* __restrict__ bias,
                                                         bf16_t* __restrict__ out, int64_t D, int64_t L, int dg,
@@ -51,13 +61,13 @@ __global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int64_t nslab = D / 16;
-    const int64_t bid = blockIdx.x;
-    const int seg = (int)(bid % nseg);
-    const int64_t slab = (bid / nseg) % nslab;
-    const int64_t b = bid / ((int64_t)nseg * nslab);
-    const int64_t d0 = slab * 16;
-    const int g = (int)(d0 / dg);
+    const uint32_t nslab = (uint32_t)(D / 16);
+    const uint32_t bid = blockIdx.x;
+    const int seg = (int)(bid % (uint32_t)nseg);
+    const uint32_t slab = (bid / (uint32_t)nseg) % nslab;
+    const int64_t b = bid / ((uint32_t)nseg * nslab);
+    const int64_t d0 = (int64_t)slab * 16;
+    const int g = (int)((uint32_t)d0 / (uint32_t)dg);
 
     // ---- Toeplitz fragments of this group's filter (A operand, 32 x 16 each)
     const int n = lane & 31, hh = lane >> 5;
@@ -65,7 +75,8 @@ __global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
     // A rows in the order below makes that lane own the 16 consecutive samples 16*hh + r.
     const int i_time = 16 * ((n >> 2) & 1) + 4 * (n >> 3) + (n & 3);
     bf16x8 A[10];
-    const int m_min = (114 - K) > 0 ? (114 - K + 15) / 16 : 0;     // blocks below m_min are all zero
+    // blocks below m_min are all zero; FULL (K > 98) means every block is live and the MFMA chain is branch-free
+    const int m_min = FULL ? 0 : ((114 - K) > 0 ? (114 - K + 15) / 16 : 0);
 #pragma unroll
     for (int m = 0; m < 10; ++m) {
         u32x4 pk;
@@ -112,13 +123,14 @@ __global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
         *(u32x4*)(u_lds + ch * URS + tt) = hu;
     }
 
-    u32x4 c1[4], cv[4];
+    u32x4 c1[4], cv[4], c2n[4];      // x1, v, x2 of the step about to be processed
     const u32x4 zero4 = {0, 0, 0, 0};
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
         const bool ok = t_begin + lane * 8 < L;
-        c1[r4] = ok ? *(const u32x4*)(p1[r4] + t_begin) : zero4;
-        cv[r4] = (PRE && ok) ? *(const u32x4*)(pv[r4] + t_begin) : zero4;
+        c1[r4] = ok ? ld16<NT>(p1[r4] + t_begin) : zero4;
+        cv[r4] = (PRE && ok) ? ld16<NT>(pv[r4] + t_begin) : zero4;
+        c2n[r4] = (POST && ok) ? ld16<NT>(p2[r4] + t_begin) : zero4;
     }
 
     float bz = 0.f;
@@ -131,17 +143,17 @@ __global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
             *(u32x4*)(u_lds + (4 * r4 + w) * URS + HALO + lane * 8) = gate_mul<PRE>(c1[r4], cv[r4]);
         __syncthreads();
 
-        // prefetch: next step's x1, v; this step's x2
+        // prefetch the next step's x1, v, x2 (x2 of this step moves to c2)
         u32x4 c2[4];
         {
             const int64_t tn = ts + TL;
             const bool okn = (tn < t_end) && (tn + lane * 8 < L);
-            const bool okc = ts + lane * 8 < L;
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
-                c1[r4] = okn ? *(const u32x4*)(p1[r4] + tn) : zero4;
-                cv[r4] = (PRE && okn) ? *(const u32x4*)(pv[r4] + tn) : zero4;
-                c2[r4] = (POST && okc) ? *(const u32x4*)(p2[r4] + ts) : zero4;
+                c2[r4] = c2n[r4];
+                c1[r4] = okn ? ld16<NT>(p1[r4] + tn) : zero4;
+                cv[r4] = (PRE && okn) ? ld16<NT>(pv[r4] + tn) : zero4;
+                c2n[r4] = (POST && okn) ? ld16<NT>(p2[r4] + tn) : zero4;
             }
         }
         // tail of this step = halo of the next one (read now, written after the MFMA phase)
@@ -202,7 +214,7 @@ __global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
                     for (int j = 0; j < 4; ++j)
                         o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(c2[r4][j]), bf_hi(zz[j]) * bf_hi(c2[r4][j]));
                 }
-                *(u32x4*)(po[r4] + ts) = o;
+                st16<NT>(po[r4] + ts, o);
             }
         }
     }
@@ -227,9 +239,9 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     if (B == 0 || L == 0) return 0;
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
 
-    // segments along L: enough blocks to fill 256 CUs a few times over, segments >= 2048 samples
+    // segments along L: >= 4096 blocks (256 CUs x 3 resident blocks, several rounds), segments >= 2048 samples
     const int64_t rows = B * (D / 16);
-    int64_t nseg = (3072 + rows - 1) / rows;
+    int64_t nseg = (4096 + rows - 1) / rows;
     const int64_t max_seg = (L + 2047) / 2048;
     if (nseg > max_seg) nseg = max_seg;
     if (nseg < 1) nseg = 1;
@@ -245,10 +257,19 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     dim3 grid((unsigned)nblk);
     const int dg = (int)(D / G);
     bool ok = false;
+    // activations larger than the last-level cache stream through it: use non-temporal accesses then
+    bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
+    if (const char* e = getenv("HYENA_MR_NT")) nt = atoi(e) != 0;
+    const bool full = K > 98;
+#define MR_LAUNCH(P, Q, M, N, F)                                                                              \
+    hipLaunchKernelGGL((mr_fir_kernel<P, Q, M, N, F>), grid, dim3(256), 0, s, m1, m2, mv, h, K, taps_reversed, \
+                       bias, (bf16_t*)out, D, L, dg, seg_len, (int)nseg)
 #define MR_CASE(P, Q, M)                                                                                      \
     if (pre == P && post == Q && bias_mode == M) {                                                            \
-        hipLaunchKernelGGL((mr_fir_kernel<P, Q, M>), grid, dim3(256), 0, s, m1, m2, mv, h, K, taps_reversed,  \
-                           bias, (bf16_t*)out, D, L, dg, seg_len, (int)nseg);                                 \
+        if (nt && full) MR_LAUNCH(P, Q, M, true, true);                                                       \
+        else if (nt) MR_LAUNCH(P, Q, M, true, false);                                                         \
+        else if (full) MR_LAUNCH(P, Q, M, false, true);                                                       \
+        else MR_LAUNCH(P, Q, M, false, false);                                                                \
         ok = true;                                                                                            \
     }
     MR_CASE(true, true, HYENA_BIAS_GATED_FP32)
@@ -258,6 +279,7 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     MR_CASE(false, false, HYENA_BIAS_ADD)
     MR_CASE(false, false, HYENA_BIAS_GATED_FP32)
 #undef MR_CASE
+#undef MR_LAUNCH
     if (!ok) return hyena_fail(HYENA_ENOSUP, "hyena_mr_fwd: this gate/bias combination has no kernel");
     return hyena_check_launch("hyena_mr_fwd");
 }

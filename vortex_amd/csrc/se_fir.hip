@@ -10,7 +10,12 @@
 
 namespace {
 
-template <int K, bool PRE, bool POST, int BIAS, bool ROWU>
+template <bool NT>
+__device__ __forceinline__ u32x4 ld16(const bf16_t* p) {
+    return NT ? __builtin_nontemporal_load((const u32x4*)p) : *(const u32x4*)p;
+}
+
+template <int K, bool PRE, bool POST, int BIAS, bool ROWU, bool NT>
 __global__ __launch_bounds__(256) void se_fir_kernel(RowMap x1, RowMap x2, RowMap v,
                                                      const float* __restrict__ taps,
                                                      const float* __restrict__ bias,
@@ -19,31 +24,32 @@ __global__ __launch_bounds__(256) void se_fir_kernel(RowMap x1, RowMap x2, RowMa
                                                      int64_t octs_per_row, int64_t total_octs) {
     constexpr int H = K - 1;                 // halo samples
     constexpr int HD = (H + 1) / 2;          // halo dwords taken from the previous lane
-    int64_t row, oct;
+    // all index arithmetic in 32 bits: the host checks that B*D and L/8 fit
+    uint32_t row, oct;
     if (ROWU) {                              // a block never straddles rows: row is wave-uniform
-        const int64_t blocks_per_row = octs_per_row / 256;
+        const uint32_t blocks_per_row = (uint32_t)octs_per_row / 256u;
         row = blockIdx.x / blocks_per_row;
-        oct = (blockIdx.x - row * blocks_per_row) * 256 + threadIdx.x;
+        oct = (blockIdx.x - row * blocks_per_row) * 256u + threadIdx.x;
     } else {
-        const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-        row = idx / octs_per_row;
-        oct = idx - row * octs_per_row;
+        const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+        row = (uint32_t)(idx / (uint32_t)octs_per_row);
+        oct = (uint32_t)(idx - (uint64_t)row * (uint32_t)octs_per_row);
     }
-    const bool active = ROWU ? true : (row * octs_per_row + oct < total_octs);
+    const bool active = ROWU ? true : ((uint64_t)row * (uint64_t)octs_per_row + oct < (uint64_t)total_octs);
     if (!active) { row = 0; oct = 0; }
-    const int64_t b = row / D, d = row - b * D;
-    const int64_t t0 = oct * 8;
-    const int g = (int)(d / dg);
+    const uint32_t b = row / (uint32_t)D, d = row - b * (uint32_t)D;
+    const int64_t t0 = (int64_t)oct * 8;
+    const int g = (int)(d / (uint32_t)dg);
 
     float w[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) w[k] = taps[g * K + k];
 
     const bf16_t* p1 = x1.row(b, d) + t0;
-    const u32x4 a1 = *(const u32x4*)p1;
+    const u32x4 a1 = ld16<NT>(p1);
     u32x4 av = {0, 0, 0, 0}, a2 = {0, 0, 0, 0};
-    if (PRE) av = *(const u32x4*)(v.row(b, d) + t0);
-    if (POST) a2 = *(const u32x4*)(x2.row(b, d) + t0);
+    if (PRE) av = ld16<NT>(v.row(b, d) + t0);
+    if (POST) a2 = ld16<NT>(x2.row(b, d) + t0);
 
     // u = bf16(x1*v), kept both as floats and as packed bf16 pairs
     float u[8];
@@ -121,28 +127,30 @@ __global__ __launch_bounds__(256) void se_fir_kernel(RowMap x1, RowMap x2, RowMa
     }
     if (active) {
         u32x4 ov = {o[0], o[1], o[2], o[3]};
-        *(u32x4*)(out + row * L + t0) = ov;
+        if (NT) __builtin_nontemporal_store(ov, (u32x4*)(out + (int64_t)row * L + t0));
+        else *(u32x4*)(out + (int64_t)row * L + t0) = ov;
     }
 }
 
 template <int K, bool PRE, bool POST, int BIAS>
-void launch_k(bool rowu, dim3 grid, hipStream_t s, RowMap x1, RowMap x2, RowMap v, const float* taps,
+void launch_k(bool rowu, bool nt, dim3 grid, hipStream_t s, RowMap x1, RowMap x2, RowMap v, const float* taps,
               const float* bias, bf16_t* out, int64_t D, int64_t L, int dg, int64_t opr, int64_t tot) {
-    if (rowu)
-        hipLaunchKernelGGL((se_fir_kernel<K, PRE, POST, BIAS, true>), grid, dim3(256), 0, s, x1, x2, v, taps, bias,
-                           out, D, L, dg, opr, tot);
-    else
-        hipLaunchKernelGGL((se_fir_kernel<K, PRE, POST, BIAS, false>), grid, dim3(256), 0, s, x1, x2, v, taps, bias,
-                           out, D, L, dg, opr, tot);
+#define SE_GO(R, N) hipLaunchKernelGGL((se_fir_kernel<K, PRE, POST, BIAS, R, N>), grid, dim3(256), 0, s, x1, x2, v, \
+                                      taps, bias, out, D, L, dg, opr, tot)
+    if (rowu && nt) SE_GO(true, true);
+    else if (rowu) SE_GO(true, false);
+    else if (nt) SE_GO(false, true);
+    else SE_GO(false, false);
+#undef SE_GO
 }
 
 template <int K>
-bool launch_gates(bool pre, bool post, int bias_mode, bool rowu, dim3 grid, hipStream_t s, RowMap x1, RowMap x2,
+bool launch_gates(bool pre, bool post, int bias_mode, bool rowu, bool nt, dim3 grid, hipStream_t s, RowMap x1, RowMap x2,
                   RowMap v, const float* taps, const float* bias, bf16_t* out, int64_t D, int64_t L, int dg,
                   int64_t opr, int64_t tot) {
 #define SE_CASE(P, Q, M)                                                                                    \
     if (pre == P && post == Q && bias_mode == M) {                                                          \
-        launch_k<K, P, Q, M>(rowu, grid, s, x1, x2, v, taps, bias, out, D, L, dg, opr, tot);                \
+        launch_k<K, P, Q, M>(rowu, nt, grid, s, x1, x2, v, taps, bias, out, D, L, dg, opr, tot);                \
         return true;                                                                                        \
     }
     SE_CASE(true, true, HYENA_BIAS_NONE)
@@ -172,9 +180,14 @@ extern "C" int hyena_se_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15))
         return hyena_fail(HYENA_EALIGN, "hyena_se_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
+    if (!rows_valid(x1) || !rows_valid(x2) || !rows_valid(v) || B * D >= (1LL << 31) || L / 8 >= (1LL << 31))
+        return hyena_fail(HYENA_EINVAL, "hyena_se_fwd: B*D, L/8 and the channel map must fit 31 bits");
     if (B == 0 || L == 0) return 0;
     const int64_t opr = L / 8, tot = B * D * opr;
     const bool rowu = (opr % 256 == 0);
+    // activations larger than the last-level cache stream through it: non-temporal accesses then
+    bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
+    if (const char* e = getenv("HYENA_SE_NT")) nt = atoi(e) != 0;
     const int64_t nblk = (tot + 255) / 256;
     if (nblk > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "hyena_se_fwd: problem too large for one launch");
     dim3 grid((unsigned)nblk);
@@ -184,7 +197,7 @@ extern "C" int hyena_se_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     bf16_t* o = (bf16_t*)out;
     bool ok = false;
     switch (K) {
-#define SE_K(KK) case KK: ok = launch_gates<KK>(pre, post, bias_mode, rowu, grid, s, m1, m2, mv, taps, bias, o, D, L, dg, opr, tot); break;
+#define SE_K(KK) case KK: ok = launch_gates<KK>(pre, post, bias_mode, rowu, nt, grid, s, m1, m2, mv, taps, bias, o, D, L, dg, opr, tot); break;
         SE_K(2) SE_K(3) SE_K(4) SE_K(5) SE_K(6) SE_K(7) SE_K(8)
 #undef SE_K
     }
