@@ -7,12 +7,13 @@
 namespace {
 
 // ---------------------------------------------------------------- FIR step
-// Block = 4 wavefronts over the same 512 channels; wavefront sg handles cache
-// slots sg, sg+4, ... so every load instruction reads 1 KiB of one slot row.
+// Block = NSG wavefronts over the same 512 channels; wavefront sg handles cache
+// slots sg, sg+NSG, ... so every load instruction reads 1 KiB of one slot row.
+// NSG = 8 for deep caches (enough loads in flight to cover HBM latency), 2 for shallow ones.
 // Ring layout [B][R][D]: channels contiguous, so the slot written back is one
 // coalesced row per batch element.
-template <bool PRE, bool POST, int BIAS, bool GROUPED>
-__global__ __launch_bounds__(256) void fir_step_kernel(const bf16_t* __restrict__ x1, const bf16_t* __restrict__ x2,
+template <bool PRE, bool POST, int BIAS, bool GROUPED, int NSG>
+__global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __restrict__ x1, const bf16_t* __restrict__ x2,
                                                        const bf16_t* __restrict__ v, int64_t in_bs,
                                                        bf16_t* __restrict__ ring, int R, int pos,
                                                        const float* __restrict__ w, const float* __restrict__ bias,
@@ -25,67 +26,75 @@ __global__ __launch_bounds__(256) void fir_step_kernel(const bf16_t* __restrict_
     const bool live = d0 < D;
     const int W = R + 1;
 
-    // taps of the groups this block touches, transposed to [i][group] (GROUPED only)
     const int ng = GROUPED ? (512 / dg) : 0;
-    float* wl = smem;                       // [W][ng]
-    float* red = smem + (GROUPED ? W * ng : 0);   // [4][64][8]
-    if (GROUPED) {
-        const int64_t g0 = dblk / dg;
-        const int64_t gmax = (D + dg - 1) / dg;
-        for (int e = tid; e < W * ng; e += 256) {
-            const int gl = e / W, i = e - gl * W;
-            wl[i * ng + gl] = (g0 + gl < gmax) ? w[(g0 + gl) * W + i] : 0.f;
-        }
-        __syncthreads();
-    }
+    float* wl = smem;                       // [W][ng]  taps of the block's groups, transposed
+    float* red = smem + (GROUPED ? W * ng : 0);   // [NSG-1][64][8]
     const int gl = GROUPED ? (oc * 8) / dg : 0;
+    constexpr int UF = 8;                   // cache slots in flight per lane
+    const bf16_t* rb = ring + (b * R) * D + d0;
+    const u32x4 zero4 = {0, 0, 0, 0};
 
+    auto load_batch = [&](int i, u32x4* q) {
+#pragma unroll
+        for (int k = 0; k < UF; ++k) {
+            const int ii = i + NSG * k;
+            int s = pos + ii;
+            if (s >= R) s -= R;
+            q[k] = (live && ii < R) ? *(const u32x4*)(rb + (int64_t)s * D) : zero4;
+        }
+    };
     float acc[8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) acc[c] = 0.f;
-
-    const bf16_t* rb = ring + (b * R) * D + d0;
-    if (live) {
-        int i = sg;
-        for (; i + 12 < R; i += 16) {                       // four slots in flight per lane
-            u32x4 q[4];
+    auto fma_batch = [&](int i, const u32x4* q) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                int s = pos + i + 4 * k;
-                if (s >= R) s -= R;
-                q[k] = *(const u32x4*)(rb + (int64_t)s * D);
-            }
+        for (int k = 0; k < UF; ++k) {
+            int ii = i + NSG * k;
+            if (ii >= R) ii = R - 1;        // the slot was loaded as zeros; any finite tap will do
+            if (GROUPED) {
+                const float t = wl[ii * ng + gl];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int ii = i + 4 * k;
-                if (GROUPED) {
-                    const float t = wl[ii * ng + gl];
+                for (int j = 0; j < 4; ++j) {
+                    acc[2 * j] = fmaf(t, bf_lo(q[k][j]), acc[2 * j]);
+                    acc[2 * j + 1] = fmaf(t, bf_hi(q[k][j]), acc[2 * j + 1]);
+                }
+            } else if (live) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        acc[2 * j] = fmaf(t, bf_lo(q[k][j]), acc[2 * j]);
-                        acc[2 * j + 1] = fmaf(t, bf_hi(q[k][j]), acc[2 * j + 1]);
-                    }
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        acc[2 * j] = fmaf(w[(d0 + 2 * j) * W + ii], bf_lo(q[k][j]), acc[2 * j]);
-                        acc[2 * j + 1] = fmaf(w[(d0 + 2 * j + 1) * W + ii], bf_hi(q[k][j]), acc[2 * j + 1]);
-                    }
+                for (int j = 0; j < 4; ++j) {
+                    acc[2 * j] = fmaf(w[(d0 + 2 * j) * W + ii], bf_lo(q[k][j]), acc[2 * j]);
+                    acc[2 * j + 1] = fmaf(w[(d0 + 2 * j + 1) * W + ii], bf_hi(q[k][j]), acc[2 * j + 1]);
                 }
             }
         }
-        for (; i < R; i += 4) {
-            int s = pos + i;
-            if (s >= R) s -= R;
-            const u32x4 q = *(const u32x4*)(rb + (int64_t)s * D);
+    };
+
+    // the first batch of cache reads goes out before the tap table is staged, so HBM is busy from the start
+    u32x4 q0[UF];
+    load_batch(sg, q0);
+    if (GROUPED) {
+        const int64_t g0 = dblk / dg;
+        const int64_t gmax = (D + dg - 1) / dg;
+        if ((W & 3) == 0) {
+            for (int e = tid; e < (W / 4) * ng; e += 64 * NSG) {
+                const int gl2 = e / (W / 4), i4 = (e - gl2 * (W / 4)) * 4;
+                f32x4 t = {0.f, 0.f, 0.f, 0.f};
+                if (g0 + gl2 < gmax) t = *(const f32x4*)(w + (g0 + gl2) * W + i4);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float t0 = GROUPED ? wl[i * ng + gl] : w[(d0 + 2 * j) * W + i];
-                const float t1 = GROUPED ? t0 : w[(d0 + 2 * j + 1) * W + i];
-                acc[2 * j] = fmaf(t0, bf_lo(q[j]), acc[2 * j]);
-                acc[2 * j + 1] = fmaf(t1, bf_hi(q[j]), acc[2 * j + 1]);
+                for (int k = 0; k < 4; ++k) wl[(i4 + k) * ng + gl2] = t[k];
+            }
+        } else {
+            for (int e = tid; e < W * ng; e += 64 * NSG) {
+                const int gl2 = e / W, i = e - gl2 * W;
+                wl[i * ng + gl2] = (g0 + gl2 < gmax) ? w[(g0 + gl2) * W + i] : 0.f;
             }
         }
+        __syncthreads();
+    }
+    fma_batch(sg, q0);
+    for (int i = sg + UF * NSG; i < R; i += UF * NSG) {
+        u32x4 q[UF];
+        load_batch(i, q);
+        fma_batch(i, q);
     }
     if (sg > 0) {
 #pragma unroll
@@ -94,7 +103,7 @@ __global__ __launch_bounds__(256) void fir_step_kernel(const bf16_t* __restrict_
     __syncthreads();          // also orders every read of slot `pos` before its overwrite below
     if (sg != 0 || !live) return;
 #pragma unroll
-    for (int k = 0; k < 3; ++k)
+    for (int k = 0; k < NSG - 1; ++k)
 #pragma unroll
         for (int c = 0; c < 8; ++c) acc[c] += red[(k * 64 + oc) * 8 + c];
 
@@ -203,19 +212,21 @@ extern "C" int hyena_fir_step(const void* x1, const void* x2, const void* v, int
         return hyena_fail(HYENA_ENOSUP, "hyena_fir_step: D/G=%d needs per-channel taps (pass G=D)", dg);
     const bool pre = v != nullptr, post = x2 != nullptr;
     dim3 grid((unsigned)((D + 511) / 512), (unsigned)B);
-    size_t sh = 3 * 64 * 8 * sizeof(float) + (grouped ? (size_t)(R + 1) * (512 / dg) * sizeof(float) : 0);
+    const int nsg = R >= 32 ? 8 : 2;
+    size_t sh = (size_t)(nsg - 1) * 64 * 8 * sizeof(float) + (grouped ? (size_t)(R + 1) * (512 / dg) * sizeof(float) : 0);
     if (sh > 160 * 1024) return hyena_fail(HYENA_ENOSUP, "hyena_fir_step: R too large for the LDS tap table");
     hipStream_t s = (hipStream_t)stream;
     const bf16_t *p1 = (const bf16_t*)x1, *p2 = (const bf16_t*)x2, *pv = (const bf16_t*)v;
     bool ok = false;
+#define FS_GO(P, Q, M, GR, N)                                                                                 \
+    hipLaunchKernelGGL((fir_step_kernel<P, Q, M, GR, N>), grid, dim3(64 * N), sh, s, p1, p2, pv, in_bs,       \
+                       (bf16_t*)ring, (int)R, (int)pos, w, bias, (bf16_t*)out, out_bs, D, dg)
 #define FS_CASE(P, Q, M)                                                                                      \
     if (pre == P && post == Q && bias_mode == M) {                                                            \
-        if (grouped)                                                                                          \
-            hipLaunchKernelGGL((fir_step_kernel<P, Q, M, true>), grid, dim3(256), sh, s, p1, p2, pv, in_bs,   \
-                               (bf16_t*)ring, (int)R, (int)pos, w, bias, (bf16_t*)out, out_bs, D, dg);        \
-        else                                                                                                  \
-            hipLaunchKernelGGL((fir_step_kernel<P, Q, M, false>), grid, dim3(256), sh, s, p1, p2, pv, in_bs,  \
-                               (bf16_t*)ring, (int)R, (int)pos, w, bias, (bf16_t*)out, out_bs, D, dg);        \
+        if (grouped && nsg == 8) FS_GO(P, Q, M, true, 8);                                                     \
+        else if (grouped) FS_GO(P, Q, M, true, 2);                                                            \
+        else if (nsg == 8) FS_GO(P, Q, M, false, 8);                                                          \
+        else FS_GO(P, Q, M, false, 2);                                                                        \
         ok = true;                                                                                            \
     }
     FS_CASE(true, true, HYENA_BIAS_NONE)
@@ -225,6 +236,7 @@ extern "C" int hyena_fir_step(const void* x1, const void* x2, const void* v, int
     FS_CASE(false, false, HYENA_BIAS_GATED_FP32)
     FS_CASE(true, true, HYENA_BIAS_ADD)
 #undef FS_CASE
+#undef FS_GO
     if (!ok) return hyena_fail(HYENA_ENOSUP, "hyena_fir_step: this gate/bias combination has no kernel");
     return hyena_check_launch("hyena_fir_step");
 }
