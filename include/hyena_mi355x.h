@@ -115,8 +115,9 @@ int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v
  * hyena_li_fwd: D/G must be a multiple of 16, L and strides multiples of 8.
  * y_conv_fp32 (optional, [B][D][L]) receives the fp32 convolution before any rounding;
  * state_out (optional, [B][D][S][2] float32) the modal state after the last sample.
- * d_is_bf16 != 0 rounds Dcoef*x1v and the sum to bf16 as bf16 tensors do in
- * vortex/model/engine.py:352-353. */
+ * d_is_bf16 selects the rounding of z = y + Dcoef*x1v: 1 = bf16(bf16(y) + bf16(Dcoef*x1v)), what
+ * bf16 tensors give in vortex/model/engine.py:352-353; 0 = bf16(bf16(y) + Dcoef*x1v), a float32
+ * Dcoef; 2 = bf16(y + Dcoef*x1v), a single rounding (cheaper, within one bf16 ulp of mode 1). */
 int64_t hyena_li_plan_bytes(int64_t G, int64_t S);
 int hyena_li_plan(const float* log_poles, const float* residues, int64_t G, int64_t S,
                   void* workspace, void* stream);

@@ -21,6 +21,8 @@
 // block barrier anywhere, only the in-order LDS pipe of the wavefront itself, and the four
 // wavefronts of a CU drift apart and cover each other's memory latency.  Global traffic is
 // coalesced 16 B per lane (1 KiB per row and instruction), prefetched PF steps ahead in registers.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -186,7 +188,7 @@ struct LiArgs {
 
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0)
 
-template <bool PRE, bool POST, bool NT, int PF>
+template <bool PRE, bool POST, bool NT, int PF, int DMODE, bool Y32>
 __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     __shared__ __attribute__((aligned(16))) unsigned char lds_all[4 * WAVE_LDS_BYTES];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -256,140 +258,185 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
             c2[p][r] = (POST && ok) ? ld16<NT>(p2[r] + t) : zero4;
         }
 
-    for (int64_t ts0 = 0; ts0 < L; ts0 += PF * TL) {
-#pragma unroll
-        for (int p = 0; p < PF; ++p) {
-            const int64_t ts = ts0 + (int64_t)p * TL;
-            if (ts >= L) break;
-            const int64_t tn = ts + (int64_t)PF * TL;          // step that reuses this register stage
-            const bool okn = tn + lane * 8 < L;
+    // One 512-sample step.  GUARD = true predicates every access on the sequence bounds.  The
+    // unguarded form exists, but straight-line code lets the compiler hoist so many loads that it
+    // spills registers, so every step runs guarded.
+    auto step = [&](auto guard_tag, const int p, const int64_t ts) {
+        constexpr bool GUARD = decltype(guard_tag)::value;
+        const int pp = (p + PF - 1) % PF;                      // register stage of the previous step
+        const int64_t tn = ts + (int64_t)PF * TL;              // step that reuses this register stage
+        const bool okn = !GUARD || (tn + lane * 8 < L);
 
-            // u = bf16(x1*v) of this step -> LDS; refill the stage with step ts + PF*TL
+        // u = bf16(x1*v) of this step -> LDS; refill the stage with step ts + PF*TL
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            *(u32x4*)(u_w + r * URS + lofs) = gate_mul<PRE>(c1[p][r], cv[p][r]);
+            c1[p][r] = okn ? ld16<NT>(p1[r] + tn) : zero4;
+            cv[p][r] = (PRE && okn) ? ld16<NT>(pv[r] + tn) : zero4;
+        }
+        wave_sync();
+
+        // B fragments: column (c, s) x inputs 32*J + 8*q.. of its chunk; shared by every MFMA below
+        bf16x8 bu[4];
+#pragma unroll
+        for (int J = 0; J < 4; ++J) bu[J] = *(const bf16x8*)(u_w + c * URS + s * CHS + 32 * J + 8 * q);
+        // z of the previous step, coalesced layout
+        u32x4 zz[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) zz[r] = *(const u32x4*)(z_w + r * URS + lofs);
+
+        // ---- state-in: L[32 x 16 cols] = Pin[32 x 128] * u
+        f32x4 l0 = {0, 0, 0, 0}, l1 = {0, 0, 0, 0};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            l0 = MFMA16(Pih[k], bu[k], l0);
+            l1 = MFMA16(Pih[4 + k], bu[k], l1);
+            l0 = MFMA16(Pil[k], bu[k], l0);
+            l1 = MFMA16(Pil[4 + k], bu[k], l1);
+        }
+        {   // lane (column n, quad q) holds state rows 4q..4q+3 of each half
+            float* lp = l_w + n * LRS + 4 * q;                 // row index s*4 + c == n  (n = c + 4s)
+            *(f32x4*)lp = l0;
+            *(f32x4*)(lp + 16) = l1;
+        }
+
+        // ---- Toeplitz: superblock Sigma (32 samples) x half ib, inputs J <= Sigma
+        f32x4 acc[4][2];
+#pragma unroll
+        for (int Sg = 0; Sg < 4; ++Sg)
+#pragma unroll
+            for (int ib = 0; ib < 2; ++ib) {
+                f32x4 t = {0, 0, 0, 0};
+#pragma unroll
+                for (int J = 0; J <= Sg; ++J) {
+                    t = MFMA16(Th[2 * (Sg - J) + ib], bu[J], t);
+                    t = MFMA16(Tl[2 * (Sg - J) + ib], bu[J], t);
+                }
+                acc[Sg][ib] = t;
+            }
+
+        // ---- deferred output of the previous step: gate with x2, store, refill its x2 stage
+        {
+            const int64_t ts_out = ts - TL, t_refill = ts - TL + (int64_t)PF * TL;
+            const bool okc = !GUARD || (ts_out >= 0 && ts_out + lane * 8 < L);
+            const bool okr = !GUARD || (ts_out >= 0 && t_refill + lane * 8 < L);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                *(u32x4*)(u_w + r * URS + lofs) = gate_mul<PRE>(c1[p][r], cv[p][r]);
-                c1[p][r] = okn ? ld16<NT>(p1[r] + tn) : zero4;
-                cv[p][r] = (PRE && okn) ? ld16<NT>(pv[r] + tn) : zero4;
-            }
-            wave_sync();
-
-            // B fragments: column (c, s) x inputs 32*J + 8*q.. of its chunk; shared by every MFMA below
-            bf16x8 bu[4];
+                u32x4 o = zz[r];
+                if (POST) {
 #pragma unroll
-            for (int J = 0; J < 4; ++J) bu[J] = *(const bf16x8*)(u_w + c * URS + s * CHS + 32 * J + 8 * q);
+                    for (int j = 0; j < 4; ++j)
+                        o[j] = pack_bf2(bf_lo(zz[r][j]) * bf_lo(c2[pp][r][j]), bf_hi(zz[r][j]) * bf_hi(c2[pp][r][j]));
+                }
+                if (okc) st16<NT>(po[r] + ts_out, o);
+                if (!GUARD || ts_out >= 0) c2[pp][r] = (POST && okr) ? ld16<NT>(p2[r] + t_refill) : zero4;
+            }
+        }
+        wave_sync();
 
-            // ---- state-in: L[32 x 16 cols] = Pin[32 x 128] * u
-            f32x4 l0 = {0, 0, 0, 0}, l1 = {0, 0, 0, 0};
+        // ---- scan over the 4 chunks: lane = (channel sc, pole sp)
+        {
+            float lr[4], li[4];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                l0 = MFMA16(Pih[k], bu[k], l0);
-                l1 = MFMA16(Pih[4 + k], bu[k], l1);
-                l0 = MFMA16(Pil[k], bu[k], l0);
-                l1 = MFMA16(Pil[4 + k], bu[k], l1);
+                const float2 t = *(const float2*)(l_w + (k * 4 + sc) * LRS + 2 * sp);
+                lr[k] = t.x;
+                li[k] = t.y;
             }
-            {   // lane (column n, quad q) holds state rows 4q..4q+3 of each half
-                float* lp = l_w + n * LRS + 4 * q;             // row index s*4 + c == n'  (n = c + 4s)
-                *(f32x4*)lp = l0;
-                *(f32x4*)(lp + 16) = l1;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t xh = pack_bf2(Xr, Xi);
+                const int o = (k * 4 + sc) * XRS + 2 * sp;
+                *(uint32_t*)(xh_w + o) = xh;
+                *(uint32_t*)(xl_w + o) = pack_bf2(Xr - bf_lo(xh), Xi - bf_hi(xh));
+                const float nr = fmaf(pcr, Xr, fmaf(-pci, Xi, lr[k]));
+                const float ni = fmaf(pcr, Xi, fmaf(pci, Xr, li[k]));
+                Xr = nr;
+                Xi = ni;
             }
+        }
+        wave_sync();
 
-            // ---- Toeplitz: superblock Sigma (32 samples) x half ib, inputs J <= Sigma
-            f32x4 acc[4][2];
+        // ---- state-out: acc += Pout[rows x 32] * X[32 x cols], three bf16 products
+        {
+            const bf16x8 xh = *(const bf16x8*)(xh_w + n * XRS + 8 * q);     // row s*4 + c == n
+            const bf16x8 xl = *(const bf16x8*)(xl_w + n * XRS + 8 * q);
 #pragma unroll
             for (int Sg = 0; Sg < 4; ++Sg)
 #pragma unroll
                 for (int ib = 0; ib < 2; ++ib) {
-                    f32x4 t = {0, 0, 0, 0};
-#pragma unroll
-                    for (int J = 0; J <= Sg; ++J) {
-                        t = MFMA16(Th[2 * (Sg - J) + ib], bu[J], t);
-                        t = MFMA16(Tl[2 * (Sg - J) + ib], bu[J], t);
-                    }
+                    f32x4 t = acc[Sg][ib];
+                    t = MFMA16(Poh[2 * Sg + ib], xh, t);
+                    t = MFMA16(Poh[2 * Sg + ib], xl, t);
+                    t = MFMA16(Pol[2 * Sg + ib], xh, t);
                     acc[Sg][ib] = t;
                 }
-            wave_sync();
+        }
 
-            // ---- scan over the 4 chunks: lane = (channel sc, pole sp)
-            {
-                float lr[4], li[4];
+        // ---- epilogue -> LDS.  lane (column (c, s), quad q) owns samples 32*Sigma + 8q .. +7 of chunk s
+        //   DMODE 1: y = bf16(conv); z = bf16(y + bf16(D*u))   (bf16 tensors, vortex/model/engine.py:352-353)
+        //   DMODE 0: y = bf16(conv); z = bf16(y + D*u)          (float32 D)
+        //   DMODE 2: z = bf16(conv + D*u)                       (one rounding)
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const float2 t = *(const float2*)(l_w + (k * 4 + sc) * LRS + 2 * sp);
-                    lr[k] = t.x;
-                    li[k] = t.y;
-                }
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const float xrh = round_bf(Xr), xih = round_bf(Xi);
-                    const int o = (k * 4 + sc) * XRS + 2 * sp;
-                    *(uint32_t*)(xh_w + o) = (__float_as_uint(xrh) >> 16) | (__float_as_uint(xih) & 0xffff0000u);
-                    *(uint32_t*)(xl_w + o) = pack_bf2(Xr - xrh, Xi - xih);
-                    const float nr = fmaf(pcr, Xr, fmaf(-pci, Xi, lr[k]));
-                    const float ni = fmaf(pcr, Xi, fmaf(pci, Xr, li[k]));
-                    Xr = nr;
-                    Xi = ni;
+        for (int Sg = 0; Sg < 4; ++Sg) {
+            const int tl = 32 * Sg + 8 * q;                     // inside the chunk
+            if (Y32) {
+                const int64_t t0 = ts + C * s + tl;
+                if (t0 < L) {
+                    float* yp = a.y32 + (b * a.D + d0 + c) * L + t0;
+                    *(f32x4*)yp = acc[Sg][0];
+                    *(f32x4*)(yp + 4) = acc[Sg][1];
                 }
             }
-            wave_sync();
-
-            // ---- state-out: acc += Pout[rows x 32] * X[32 x cols], three bf16 products
-            {
-                const bf16x8 xh = *(const bf16x8*)(xh_w + n * XRS + 8 * q);     // row s*4 + c == n
-                const bf16x8 xl = *(const bf16x8*)(xl_w + n * XRS + 8 * q);
+            const u32x4 uu = *(const u32x4*)(u_w + c * URS + s * CHS + tl);
+            u32x4 z;
 #pragma unroll
-                for (int Sg = 0; Sg < 4; ++Sg)
-#pragma unroll
-                    for (int ib = 0; ib < 2; ++ib) {
-                        f32x4 t = acc[Sg][ib];
-                        t = MFMA16(Poh[2 * Sg + ib], xh, t);
-                        t = MFMA16(Poh[2 * Sg + ib], xl, t);
-                        t = MFMA16(Pol[2 * Sg + ib], xh, t);
-                        acc[Sg][ib] = t;
-                    }
-            }
-
-            // ---- epilogue: y = bf16(conv); z = bf16(y + bf16(D*u)) -> LDS  (engine.py:352-353)
-            // lane (column (c, s), quad q) owns samples 32*Sigma + 8q .. +7 of chunk s
-#pragma unroll
-            for (int Sg = 0; Sg < 4; ++Sg) {
-                const int tl = 32 * Sg + 8 * q;                 // inside the chunk
-                if (a.y32) {
-                    const int64_t t0 = ts + C * s + tl;
-                    if (t0 < L) {
-                        float* yp = a.y32 + (b * a.D + d0 + c) * L + t0;
-                        *(f32x4*)yp = acc[Sg][0];
-                        *(f32x4*)(yp + 4) = acc[Sg][1];
+            for (int j = 0; j < 4; ++j) {
+                const f32x4 av = acc[Sg][j >> 1];
+                const float a0 = av[2 * (j & 1)], a1 = av[2 * (j & 1) + 1];
+                const float u0 = bf_lo(uu[j]), u1 = bf_hi(uu[j]);
+                if (DMODE == 2) {
+                    z[j] = pack_bf2(fmaf(dco, u0, a0), fmaf(dco, u1, a1));
+                } else {
+                    const uint32_t yp = pack_bf2(a0, a1);
+                    if (DMODE == 1) {
+                        const uint32_t tp = pack_bf2(dco * u0, dco * u1);
+                        z[j] = pack_bf2(bf_lo(yp) + bf_lo(tp), bf_hi(yp) + bf_hi(tp));
+                    } else {
+                        z[j] = pack_bf2(fmaf(dco, u0, bf_lo(yp)), fmaf(dco, u1, bf_hi(yp)));
                     }
                 }
-                const u32x4 uu = *(const u32x4*)(u_w + c * URS + s * CHS + tl);
-                u32x4 z;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const f32x4 av = acc[Sg][j >> 1];
-                    const float y0 = round_bf(av[2 * (j & 1)]), y1 = round_bf(av[2 * (j & 1) + 1]);
-                    float t0 = dco * bf_lo(uu[j]), t1 = dco * bf_hi(uu[j]);
-                    if (a.d_is_bf16) { t0 = round_bf(t0); t1 = round_bf(t1); }
-                    z[j] = pack_bf2(y0 + t0, y1 + t1);
-                }
-                *(u32x4*)(z_w + c * URS + s * CHS + tl) = z;
             }
-            wave_sync();
+            *(u32x4*)(z_w + c * URS + s * CHS + tl) = z;
+        }
+        // the wave_sync after the next step's u write orders these z writes before their coalesced reads
+    };
 
-            // ---- gate with x2 and store, coalesced; refill x2 of the stage
-            const bool okc = ts + lane * 8 < L;
+    const std::integral_constant<bool, true> guarded;
+    for (int64_t ts = 0; ts < L; ts += (int64_t)PF * TL) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const u32x4 zz = *(const u32x4*)(z_w + r * URS + lofs);
-                u32x4 o = zz;
-                if (POST) {
+        for (int p = 0; p < PF; ++p)
+            if (ts + (int64_t)p * TL < L) step(guarded, p, ts + (int64_t)p * TL);
+    }
+    {   // output of the last step
+        const int64_t ts_last = ((L + TL - 1) / TL - 1) * TL;
+        wave_sync();
+        const bool okc = ts_last + lane * 8 < L;
+        const int pl = (int)((ts_last / TL) % PF);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(c2[p][r][j]), bf_hi(zz[j]) * bf_hi(c2[p][r][j]));
-                }
-                if (okc) st16<NT>(po[r] + ts, o);
-                c2[p][r] = (POST && okn) ? ld16<NT>(p2[r] + tn) : zero4;
+        for (int r = 0; r < 4; ++r) {
+            const u32x4 zz = *(const u32x4*)(z_w + r * URS + lofs);
+            u32x4 x2v = c2[0][r];
+#pragma unroll
+            for (int p = 1; p < PF; ++p)
+                if (p == pl) x2v = c2[p][r];
+            u32x4 o = zz;
+            if (POST) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(x2v[j]), bf_hi(zz[j]) * bf_hi(x2v[j]));
             }
-            wave_sync();      // z and u of this step are consumed before the next step overwrites them
+            if (okc) st16<NT>(po[r] + ts_last, o);
         }
     }
 
@@ -441,6 +488,7 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15) ||
         (((uintptr_t)y_conv_fp32) & 15) || (((uintptr_t)workspace) & 15))
         return hyena_fail(HYENA_EALIGN, "hyena_li_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
+    if (d_is_bf16 < 0 || d_is_bf16 > 2) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: d_is_bf16 must be 0, 1 or 2");
     if (B == 0 || L == 0) return 0;
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
     const int64_t nquads = B * (D / 4);
@@ -464,19 +512,19 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     dim3 grid((unsigned)nblk);
     bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
     if (const char* e = getenv("HYENA_LI_NT")) nt = atoi(e) != 0;
-    int pf = 3;
-    if (const char* e = getenv("HYENA_LI_PF")) pf = atoi(e);
-#define LI_LAUNCH(P, Q, N, F) hipLaunchKernelGGL((li_kernel<P, Q, N, F>), grid, dim3(256), 0, s, a)
-#define LI_PF(P, Q, N) \
-    if (pf <= 1) LI_LAUNCH(P, Q, N, 1); else if (pf == 2) LI_LAUNCH(P, Q, N, 2); else LI_LAUNCH(P, Q, N, 3)
-    if (pre && post) {
-        if (nt) { LI_PF(true, true, true); } else { LI_PF(true, true, false); }
-    } else if (!pre && !post) {
-        if (nt) { LI_PF(false, false, true); } else { LI_PF(false, false, false); }
-    } else {
-        return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: pass both v and x2 or neither");
-    }
-#undef LI_PF
+    // DMODE and Y32 are compile-time so that the hot loop carries no uniform branches.  The fp32
+    // side output is a verification path: it always uses cached accesses.
+    const int dmode = d_is_bf16;
+    const bool y32 = y_conv_fp32 != nullptr;
+    if (y32) nt = false;
+#define LI_LAUNCH(P, Q, N, M, Y) hipLaunchKernelGGL((li_kernel<P, Q, N, 3, M, Y>), grid, dim3(256), 0, s, a)
+#define LI_M(P, Q, N, Y) do { if (dmode == 1) LI_LAUNCH(P, Q, N, 1, Y); else if (dmode == 2) LI_LAUNCH(P, Q, N, 2, Y); else LI_LAUNCH(P, Q, N, 0, Y); } while (0)
+#define LI_N(P, Q) do { if (y32) LI_M(P, Q, false, true); else if (nt) LI_M(P, Q, true, false); else LI_M(P, Q, false, false); } while (0)
+    if (pre && post) LI_N(true, true);
+    else if (!pre && !post) LI_N(false, false);
+    else return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: pass both v and x2 or neither");
+#undef LI_N
+#undef LI_M
 #undef LI_LAUNCH
     return hyena_check_launch("hyena_li_fwd");
 }

@@ -174,13 +174,14 @@ class ModalPlan:
         _lib.check(rc, "hyena_li_plan")
 
 
-def li_fwd_rows(x1r, x2r, vr, plan, Dcoef, B, D, L, *, device, want_state=False, want_fp32=False, out=None):
+def li_fwd_rows(x1r, x2r, vr, plan, Dcoef, B, D, L, *, device, want_state=False, want_fp32=False, out=None,
+                single_rounding=False):
     if out is None:
         out = torch.empty((B, D, L), dtype=torch.bfloat16, device=device)
     y32 = torch.empty((B, D, L), dtype=torch.float32, device=device) if want_fp32 else None
     state = torch.empty((B, D, plan.S, 2), dtype=torch.float32, device=device) if want_state else None
     dco = _f32(Dcoef)
-    d_is_bf16 = int(Dcoef is None or Dcoef.dtype == torch.bfloat16)
+    d_is_bf16 = 2 if single_rounding else int(Dcoef is None or Dcoef.dtype == torch.bfloat16)
     rc = _lib.lib().hyena_li_fwd(_ref(x1r), _ref(x2r), _ref(vr), _ptr(plan.workspace), _ptr(dco), d_is_bf16,
                                  _ptr(out), _ptr(y32), _ptr(state), B, D, L, plan.G, plan.S, _stream())
     _lib.check(rc, "hyena_li_fwd")
@@ -189,21 +190,24 @@ def li_fwd_rows(x1r, x2r, vr, plan, Dcoef, B, D, L, *, device, want_state=False,
     return out, y32, state
 
 
-def hyena_li_fwd(x1, x2, v, log_poles, residues, D_bias=None, *, plan=None, want_state=False, want_fp32=False):
+def hyena_li_fwd(x1, x2, v, log_poles, residues, D_bias=None, *, plan=None, want_state=False, want_fp32=False,
+                 single_rounding=False):
     """Hyena-LI prefill on [B, D, L] bf16 gates with grouped modal parameters.
 
     log_poles [G, S, 1] (or [G, S]) and residues [G, S], float32 or complex64
     (vortex/model/model.py:202-209, :390-398).  Returns (out [B, D, L] bf16,
     y_conv fp32 or None, state [B, D, S] or None); the state is complex64 for complex
     poles and float32 for real ones (the real part, as vortex/model/engine.py:559 keeps).
-    Pass a ModalPlan to reuse the coefficient tables between calls.
+    Pass a ModalPlan to reuse the coefficient tables between calls.  single_rounding=True computes
+    z = bf16(conv + D*x1v) with one rounding instead of the three of the reference's bf16 tensor
+    arithmetic (fewer vector instructions; within one bf16 ulp of the default).
     """
     _need_cuda(x1, x2, v, log_poles, residues)
     B, D, L = x1.shape
     if plan is None:
         plan = ModalPlan(log_poles, residues)
     return li_fwd_rows(rows_of(x1), rows_of(x2), rows_of(v), plan, D_bias, B, D, L, device=x1.device,
-                       want_state=want_state, want_fp32=want_fp32)
+                       want_state=want_state, want_fp32=want_fp32, single_rounding=single_rounding)
 
 
 class FirRing:
