@@ -631,5 +631,7 @@ class OracleCascade:
             y, st = self.engine.step_iir(x2, x1, v, p["D"], p["residues"], p["log_poles"],
                                          inference_params.state_dict[self.layer_idx], iir_groups=1)
             inference_params.state_dict[self.layer_idx] = st
+            if y.is_complex():          # complex poles (not in vortex, where parameters are real): keep Re
+                y = y.real
         y = y.to(dtype=u.dtype)
         return y[:, None], inference_params

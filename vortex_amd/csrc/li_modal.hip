@@ -14,10 +14,12 @@
 // (hi*hi + hi*lo + lo*hi); the inputs u = bf16(x1*v) are exact.  The recurrence itself is carried
 // in fp32 registers.  The final X is the decode state of vortex/model/engine.py:525-559 for free.
 //
-// Work decomposition: a WAVEFRONT owns 4 channels of one filter group and walks the whole
-// sequence alone, 512 samples (4 chunks) per step.  The 16 MFMA columns are 4 channels x 4
-// chunks, so one B fragment serves all four chunks of the step; the 64 lanes hold the 4 x 16
-// complex states of the scan, one each.  Nothing is shared between wavefronts: there is no
+// Work decomposition: a WAVEFRONT owns CPW channels of one filter group and walks the whole
+// sequence alone.  With CPW = 4 a step is 512 samples (4 chunks) and the 16 MFMA columns are
+// 4 channels x 4 chunks; the 64 lanes hold the 4 x 16 complex states of the scan, one each.
+// With CPW = 1 (filter groups narrower than 4 channels, e.g. one filter per channel) a step is
+// 2048 samples of one channel and the 16 columns are its 16 chunks.  Either way one B fragment
+// serves every column of the step.  Nothing is shared between wavefronts: there is no
 // block barrier anywhere, only the in-order LDS pipe of the wavefront itself, and the four
 // wavefronts of a CU drift apart and cover each other's memory latency.  Global traffic is
 // coalesced 16 B per lane (1 KiB per row and instruction), prefetched PF steps ahead in registers.
@@ -188,16 +190,18 @@ struct LiArgs {
 
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0)
 
-template <bool PRE, bool POST, bool NT, int PF, int DMODE, bool Y32>
+template <bool PRE, bool POST, bool NT, int PF, int DMODE, bool Y32, int CPW>
 __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
+    static_assert(CPW == 4 || CPW == 1, "4 channels x 512 samples or 1 channel x 2048 samples per step");
+    constexpr int TLW = TL * (4 / CPW);                        // samples of one channel per step
     __shared__ __attribute__((aligned(16))) unsigned char lds_all[4 * WAVE_LDS_BYTES];
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int64_t quad = (int64_t)blockIdx.x * 4 + w;          // 4 channels of one batch element
+    const int64_t quad = (int64_t)blockIdx.x * 4 + w;          // CPW channels of one batch element
     if (quad >= a.nquads) return;                              // whole wavefront leaves; no barriers below
-    const uint32_t qpb = (uint32_t)(a.D / 4);
+    const uint32_t qpb = (uint32_t)(a.D / CPW);
     const int64_t b = (uint32_t)quad / qpb;
-    const int64_t d0 = (int64_t)((uint32_t)quad % qpb) * 4;
+    const int64_t d0 = (int64_t)((uint32_t)quad % qpb) * CPW;
     const int g = (int)((uint32_t)d0 / (uint32_t)a.dg);
     const float* ws = a.ws + (size_t)g * WS_GROUP;
     const int64_t L = a.L;
@@ -228,22 +232,26 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     const int n = lane & 15, q = lane >> 4;
     const int c = n & 3, s = n >> 2;
     // scan-side lane geometry: one complex state per lane
-    const int sc = lane >> 4, sp = lane & 15;
+    const int sc = CPW == 4 ? (lane >> 4) : 0, sp = lane & 15;
     float Xr = 0.f, Xi = 0.f;
+    float Xfr = 0.f, Xfi = 0.f;                                // state after the chunk that holds sample L-1
     const float pcr = ws[WS_PC + 2 * sp], pci = ws[WS_PC + 2 * sp + 1];
     float dco = 0.f;
-    if (a.Dcoef) dco = a.Dcoef[d0 + c];
+    if (a.Dcoef) dco = a.Dcoef[d0 + (CPW == 4 ? c : 0)];
 
     // ---- coalesced layout: lane moves samples 8*lane..8*lane+7 of each of the 4 rows
     const int lofs = lane * 8 + 32 * (lane >> 4);              // position inside a padded LDS row
     const bf16_t *p1[4], *pv[4], *p2[4];
     bf16_t* po[4];
+    // LDS row r is channel d0 + r (CPW = 4) or the r-th 512-sample piece of channel d0 (CPW = 1)
+    auto roff = [](int r) -> int64_t { return CPW == 4 ? 0 : (int64_t)TL * r; };
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-        p1[r] = a.x1.row(b, d0 + r) + lane * 8;
-        pv[r] = PRE ? a.v.row(b, d0 + r) + lane * 8 : nullptr;
-        p2[r] = POST ? a.x2.row(b, d0 + r) + lane * 8 : nullptr;
-        po[r] = a.out + (b * a.D + d0 + r) * L + lane * 8;
+        const int64_t d = d0 + (CPW == 4 ? r : 0);
+        p1[r] = a.x1.row(b, d) + roff(r) + lane * 8;
+        pv[r] = PRE ? a.v.row(b, d) + roff(r) + lane * 8 : nullptr;
+        p2[r] = POST ? a.x2.row(b, d) + roff(r) + lane * 8 : nullptr;
+        po[r] = a.out + (b * a.D + d) * L + roff(r) + lane * 8;
     }
     const u32x4 zero4 = {0, 0, 0, 0};
     u32x4 c1[PF][4], cv[PF][4], c2[PF][4];
@@ -251,8 +259,8 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     for (int p = 0; p < PF; ++p)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int64_t t = (int64_t)p * TL;
-            const bool ok = t + lane * 8 < L;
+            const int64_t t = (int64_t)p * TLW;
+            const bool ok = t + roff(r) + lane * 8 < L;
             c1[p][r] = ok ? ld16<NT>(p1[r] + t) : zero4;
             cv[p][r] = (PRE && ok) ? ld16<NT>(pv[r] + t) : zero4;
             c2[p][r] = (POST && ok) ? ld16<NT>(p2[r] + t) : zero4;
@@ -264,12 +272,12 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     auto step = [&](auto guard_tag, const int p, const int64_t ts) {
         constexpr bool GUARD = decltype(guard_tag)::value;
         const int pp = (p + PF - 1) % PF;                      // register stage of the previous step
-        const int64_t tn = ts + (int64_t)PF * TL;              // step that reuses this register stage
-        const bool okn = !GUARD || (tn + lane * 8 < L);
+        const int64_t tn = ts + (int64_t)PF * TLW;             // step that reuses this register stage
 
-        // u = bf16(x1*v) of this step -> LDS; refill the stage with step ts + PF*TL
+        // u = bf16(x1*v) of this step -> LDS; refill the stage with step ts + PF*TLW
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
+            const bool okn = !GUARD || (tn + roff(r) + lane * 8 < L);
             *(u32x4*)(u_w + r * URS + lofs) = gate_mul<PRE>(c1[p][r], cv[p][r]);
             c1[p][r] = okn ? ld16<NT>(p1[r] + tn) : zero4;
             cv[p][r] = (PRE && okn) ? ld16<NT>(pv[r] + tn) : zero4;
@@ -317,11 +325,11 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
 
         // ---- deferred output of the previous step: gate with x2, store, refill its x2 stage
         {
-            const int64_t ts_out = ts - TL, t_refill = ts - TL + (int64_t)PF * TL;
-            const bool okc = !GUARD || (ts_out >= 0 && ts_out + lane * 8 < L);
-            const bool okr = !GUARD || (ts_out >= 0 && t_refill + lane * 8 < L);
+            const int64_t ts_out = ts - TLW, t_refill = ts - TLW + (int64_t)PF * TLW;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
+                const bool okc = !GUARD || (ts_out >= 0 && ts_out + roff(r) + lane * 8 < L);
+                const bool okr = !GUARD || (ts_out >= 0 && t_refill + roff(r) + lane * 8 < L);
                 u32x4 o = zz[r];
                 if (POST) {
 #pragma unroll
@@ -334,25 +342,34 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
         }
         wave_sync();
 
-        // ---- scan over the 4 chunks: lane = (channel sc, pole sp)
+        // ---- scan over the chunks of the step in time order: lane = (channel sc, pole sp).
+        // Column n = c + 4s sits in row n of l_w / x*_w; in time order chunk k is (c, s) = (sc, k) for
+        // CPW = 4 and (k / 4, k % 4) for CPW = 1, where all 64 lanes repeat the work of lanes 0..15.
         {
-            float lr[4], li[4];
+            constexpr int NK = 16 / CPW;
+            float lr[NK], li[NK];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const float2 t = *(const float2*)(l_w + (k * 4 + sc) * LRS + 2 * sp);
+            for (int k = 0; k < NK; ++k) {
+                const int row = CPW == 4 ? (k * 4 + sc) : ((k & 3) * 4 + (k >> 2));
+                const float2 t = *(const float2*)(l_w + row * LRS + 2 * sp);
                 lr[k] = t.x;
                 li[k] = t.y;
             }
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
+            for (int k = 0; k < NK; ++k) {
+                const int row = CPW == 4 ? (k * 4 + sc) : ((k & 3) * 4 + (k >> 2));
                 const uint32_t xh = pack_bf2(Xr, Xi);
-                const int o = (k * 4 + sc) * XRS + 2 * sp;
+                const int o = row * XRS + 2 * sp;
                 *(uint32_t*)(xh_w + o) = xh;
                 *(uint32_t*)(xl_w + o) = pack_bf2(Xr - bf_lo(xh), Xi - bf_hi(xh));
                 const float nr = fmaf(pcr, Xr, fmaf(-pci, Xi, lr[k]));
                 const float ni = fmaf(pcr, Xi, fmaf(pci, Xr, li[k]));
                 Xr = nr;
                 Xi = ni;
+                if (GUARD) {                                   // chunk k of the step covers ts + 128k .. + 127
+                    const int64_t te = ts + (int64_t)C * (k + 1);
+                    if (te >= L && te - C < L) { Xfr = Xr; Xfi = Xi; }
+                }
             }
         }
         wave_sync();
@@ -381,9 +398,9 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
         for (int Sg = 0; Sg < 4; ++Sg) {
             const int tl = 32 * Sg + 8 * q;                     // inside the chunk
             if (Y32) {
-                const int64_t t0 = ts + C * s + tl;
+                const int64_t t0 = ts + roff(c) + C * s + tl;
                 if (t0 < L) {
-                    float* yp = a.y32 + (b * a.D + d0 + c) * L + t0;
+                    float* yp = a.y32 + (b * a.D + d0 + (CPW == 4 ? c : 0)) * L + t0;
                     *(f32x4*)yp = acc[Sg][0];
                     *(f32x4*)(yp + 4) = acc[Sg][1];
                 }
@@ -413,18 +430,18 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     };
 
     const std::integral_constant<bool, true> guarded;
-    for (int64_t ts = 0; ts < L; ts += (int64_t)PF * TL) {
+    for (int64_t ts = 0; ts < L; ts += (int64_t)PF * TLW) {
 #pragma unroll
         for (int p = 0; p < PF; ++p)
-            if (ts + (int64_t)p * TL < L) step(guarded, p, ts + (int64_t)p * TL);
+            if (ts + (int64_t)p * TLW < L) step(guarded, p, ts + (int64_t)p * TLW);
     }
     {   // output of the last step
-        const int64_t ts_last = ((L + TL - 1) / TL - 1) * TL;
+        const int64_t ts_last = ((L + TLW - 1) / TLW - 1) * TLW;
         wave_sync();
-        const bool okc = ts_last + lane * 8 < L;
-        const int pl = (int)((ts_last / TL) % PF);
+        const int pl = (int)((ts_last / TLW) % PF);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
+            const bool okc = ts_last + roff(r) + lane * 8 < L;
             const u32x4 zz = *(const u32x4*)(z_w + r * URS + lofs);
             u32x4 x2v = c2[0][r];
 #pragma unroll
@@ -441,8 +458,8 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     }
 
     if (a.state_out) {
-        // the scan ran over ceil(L/512)*512 samples with zero inputs past L: undo the padding, X *= p^-pad
-        int pad = (int)(((L + TL - 1) / TL) * TL - L);
+        // the captured chunk ends (-L) % 128 samples past L with zero inputs: undo that, X *= p^-pad
+        int pad = (int)((C - L % C) % C);
         float qr = ws[WS_PINV + 2 * sp], qi = ws[WS_PINV + 2 * sp + 1];
         float fr_ = 1.f, fi = 0.f;
         while (pad) {
@@ -450,9 +467,13 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
             const float t = qr * qr - qi * qi; qi = 2.f * qr * qi; qr = t;
             pad >>= 1;
         }
-        float* sp_ = a.state_out + ((b * a.D + d0 + sc) * S + sp) * 2;
-        sp_[0] = Xr * fr_ - Xi * fi;
-        sp_[1] = Xr * fi + Xi * fr_;
+        Xr = Xfr;
+        Xi = Xfi;
+        if (CPW == 4 || lane < 16) {
+            float* sp_ = a.state_out + ((b * a.D + d0 + sc) * S + sp) * 2;
+            sp_[0] = Xr * fr_ - Xi * fi;
+            sp_[1] = Xr * fi + Xi * fr_;
+        }
     }
 }
 
@@ -483,15 +504,14 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
         return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: bad sizes B=%lld D=%lld L=%lld G=%lld", (long long)B,
                           (long long)D, (long long)L, (long long)G);
     if (S_ != S) return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: state size %lld (only 16)", (long long)S_);
-    if ((D / G) % 4 != 0)
-        return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: D/G=%lld must be a multiple of 4", (long long)(D / G));
     if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15) ||
         (((uintptr_t)y_conv_fp32) & 15) || (((uintptr_t)workspace) & 15))
         return hyena_fail(HYENA_EALIGN, "hyena_li_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
     if (d_is_bf16 < 0 || d_is_bf16 > 2) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: d_is_bf16 must be 0, 1 or 2");
     if (B == 0 || L == 0) return 0;
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
-    const int64_t nquads = B * (D / 4);
+    const int cpw = ((D / G) % 4 == 0) ? 4 : 1;              // channels per wavefront (they share one filter)
+    const int64_t nquads = B * (D / cpw);
     const int64_t nblk = (nquads + 3) / 4;
     if (nquads > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: problem too large for one launch");
     LiArgs a;
@@ -517,7 +537,11 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     const int dmode = d_is_bf16;
     const bool y32 = y_conv_fp32 != nullptr;
     if (y32) nt = false;
-#define LI_LAUNCH(P, Q, N, M, Y) hipLaunchKernelGGL((li_kernel<P, Q, N, 3, M, Y>), grid, dim3(256), 0, s, a)
+#define LI_LAUNCH(P, Q, N, M, Y)                                                                           \
+    do {                                                                                                   \
+        if (cpw == 4) hipLaunchKernelGGL((li_kernel<P, Q, N, 3, M, Y, 4>), grid, dim3(256), 0, s, a);      \
+        else hipLaunchKernelGGL((li_kernel<P, Q, N, 3, M, Y, 1>), grid, dim3(256), 0, s, a);               \
+    } while (0)
 #define LI_M(P, Q, N, Y) do { if (dmode == 1) LI_LAUNCH(P, Q, N, 1, Y); else if (dmode == 2) LI_LAUNCH(P, Q, N, 2, Y); else LI_LAUNCH(P, Q, N, 0, Y); } while (0)
 #define LI_N(P, Q) do { if (y32) LI_M(P, Q, false, true); else if (nt) LI_M(P, Q, true, false); else LI_M(P, Q, false, false); } while (0)
     if (pre && post) LI_N(true, true);
