@@ -33,6 +33,7 @@ def parse():
     ap.add_argument("--workload", default="mr", choices=["mr", "se", "li", "decode"])
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-model", action="store_true", help="skip the end-to-end model prefill legs")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 1 GiB device copy (calibration of FETCH_SIZE / WRITE_SIZE counters)")
     return ap.parse_args()
@@ -131,6 +132,24 @@ def decode_layer_set(D, device, steps, warmup):
                 hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
 
 
+def model_prefill(device, L, iters=2):
+    """Evo 2 7B-shaped random-init StripedHyena 2 prefill (32 blocks [SE, MR, LI, attention], hidden 4096,
+    MLP 11008, vocab 512): Hyena operators on the HIP kernels, projections / MLP / attention through torch."""
+    from vortex_amd.model import StripedHyena2
+    m = StripedHyena2(device=device).to_inference(device)
+    ids = torch.randint(0, 512, (1, L), device=device, generator=torch.Generator(device=device).manual_seed(8))
+    m(ids)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        m(ids)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / iters
+    del m
+    torch.cuda.empty_cache()
+    return {"workload": f"striped_hyena2_7b_shaped_prefill B=1 L={L}", "tokens_per_s": L / dt, "ms": dt * 1e3}
+
+
 def cpu_baseline(name):
     """The oracle (a PyTorch port of the reference path) timed on the host cores, on a channel slice."""
     from oracle import hyena_oracle as O
@@ -225,6 +244,9 @@ def main():
                            "roofline_frac": e["hbm_gbs"] / HBM_PEAK_GBS}
         for D in (4096, 8192):
             extra[f"decode_D{D}"] = decode_layer_set(D, device, max(args.steps, 50), max(args.warmup, 5))
+        if not args.no_model:
+            for L in (8192, 131072):
+                extra[f"model_L{L}"] = model_prefill(device, L)
         result["extra"] = extra
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(main_name)

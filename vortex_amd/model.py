@@ -1,0 +1,167 @@
+"""Minimal StripedHyena 2 stack around the gfx950 Hyena operators (random-init, inference only).
+
+Only the Hyena operators (featurizer FIR, Hyena-SE / MR / LI, decode steps) are this package's
+kernels; projections, MLP and attention are plain torch matmul / SDPA, as the Evo 2 7B-shaped
+end-to-end configuration prescribes.  Formulas follow the reference:
+  RMSNorm            vortex/model/layers.py:178-196   y = scale * x / (||x||_2 * D^-1/2 + eps)
+  gated MLP          vortex/model/layers.py:199-246   l3(act(l1 z) * l2 z), act = GELU on layer 0,
+                                                      identity afterwards (evo2_style_activations)
+  Hyena block        vortex/model/model.py:523-575    u + W_o * cascade(W_p * norm(u)), then + MLP
+  attention block    vortex/model/model.py:48-122     u + MHA(norm(u)) with rotary embedding, then + MLP
+  tied unembedding   vortex/model/layers.py:309-311   logits = x @ E^T
+"""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .cascade import HyenaCascade, HyenaCascadeFIRInferenceParams, HyenaCascadeIIRInferenceParams
+
+EVO2_7B = dict(
+    vocab_size=512, hidden_size=4096, num_layers=32, num_attention_heads=32, inner_mlp_size=11008,
+    short_filter_length=3, short_filter_bias=False, state_size=16, eps=1e-6,
+    hcs_filter_length=7, hcm_filter_length=128, hcs_filter_groups=256, hcm_filter_groups=256,
+    hcl_filter_groups=4096, pattern=("hcs", "hcm", "hcl", "attn"), column_split_hyena=False, interleave=True,
+    rotary_emb_base=10000, evo2_style_activations=True,
+)
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, hidden, eps):
+        super().__init__()
+        self.eps, self.hidden = eps, hidden
+        self.scale = nn.Parameter(torch.ones(hidden))
+
+    def forward(self, x):
+        y = x / (x.norm(2, dim=-1, keepdim=True) * self.hidden ** -0.5 + self.eps)
+        return self.scale * y
+
+
+class GatedMLP(nn.Module):
+    def __init__(self, hidden, inner, identity_act, chunk=16384):
+        super().__init__()
+        self.l1 = nn.Linear(hidden, inner, bias=False)
+        self.l2 = nn.Linear(hidden, inner, bias=False)
+        self.l3 = nn.Linear(inner, hidden, bias=False)
+        self.identity_act, self.chunk = identity_act, chunk
+
+    def _f(self, z):
+        a = self.l1(z)
+        if not self.identity_act:
+            a = F.gelu(a)
+        return self.l3(a * self.l2(z))
+
+    def forward(self, z):
+        if z.shape[1] <= self.chunk:
+            return self._f(z)
+        return torch.cat([self._f(z[:, i:i + self.chunk]) for i in range(0, z.shape[1], self.chunk)], dim=1)
+
+
+def _rotary(x, base, offset=0):
+    """x [B, L, H, hd]; non-interleaved rotary embedding over the whole head dimension."""
+    B, L, H, hd = x.shape
+    inv = 1.0 / (base ** (torch.arange(0, hd, 2, device=x.device, dtype=torch.float32) / hd))
+    t = torch.arange(offset, offset + L, device=x.device, dtype=torch.float32)
+    f = torch.outer(t, inv)
+    cos, sin = f.cos()[None, :, None].to(x.dtype), f.sin()[None, :, None].to(x.dtype)
+    x1, x2 = x[..., : hd // 2], x[..., hd // 2:]
+    return torch.cat([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1)
+
+
+class AttentionBlock(nn.Module):
+    def __init__(self, cfg, layer_idx):
+        super().__init__()
+        D, H = cfg["hidden_size"], cfg["num_attention_heads"]
+        self.H, self.base = H, cfg["rotary_emb_base"]
+        self.pre_norm, self.post_norm = RMSNorm(D, cfg["eps"]), RMSNorm(D, cfg["eps"])
+        self.Wqkv = nn.Linear(D, 3 * D, bias=False)
+        self.out_proj = nn.Linear(D, D, bias=True)
+        self.mlp = GatedMLP(D, cfg["inner_mlp_size"], cfg["evo2_style_activations"] and layer_idx > 0)
+
+    def forward(self, u, inference_params=None):
+        B, L, D = u.shape
+        qkv = self.Wqkv(self.pre_norm(u)).view(B, L, 3, self.H, D // self.H)
+        q, k, v = _rotary(qkv[:, :, 0], self.base), _rotary(qkv[:, :, 1], self.base), qkv[:, :, 2]
+        o = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True)
+        u = self.out_proj(o.transpose(1, 2).reshape(B, L, D)) + u
+        return self.mlp(self.post_norm(u)) + u, None
+
+
+class HyenaBlock(nn.Module):
+    def __init__(self, cfg, layer_idx, kind):
+        super().__init__()
+        D = cfg["hidden_size"]
+        self.pre_norm, self.post_norm = RMSNorm(D, cfg["eps"]), RMSNorm(D, cfg["eps"])
+        self.projections = nn.Linear(D, 3 * D, bias=False)
+        groups = cfg[f"{kind}_filter_groups"]
+        K = {"hcs": cfg["hcs_filter_length"], "hcm": cfg["hcm_filter_length"], "hcl": None}[kind]
+        self.filter = HyenaCascade(cfg, layer_idx, hyena_filter_groups=groups, fir_inner_filter_length=K)
+        self.out_filter_dense = nn.Linear(D, D, bias=True)
+        self.mlp = GatedMLP(D, cfg["inner_mlp_size"], cfg["evo2_style_activations"] and layer_idx > 0)
+
+    def forward(self, u, inference_params=None):
+        z = self.projections(self.pre_norm(u))
+        z, _ = self.filter(z, inference_params=inference_params)
+        z_in = self.out_filter_dense(z) + u
+        return self.mlp(self.post_norm(z_in)) + z_in, None
+
+
+class StripedHyena2(nn.Module):
+    """Embedding -> [SE, MR, LI, attention] x N/4 -> RMSNorm -> tied unembedding."""
+
+    def __init__(self, cfg=None, seed=0, device=None):
+        super().__init__()
+        cfg = dict(EVO2_7B if cfg is None else cfg)
+        self.cfg = cfg
+        D = cfg["hidden_size"]
+        with torch.device(device if device is not None else "cpu"):
+            self.embedding = nn.Embedding(cfg["vocab_size"], D)
+            pat = cfg["pattern"]
+            self.kinds = [pat[i % len(pat)] for i in range(cfg["num_layers"])]
+            self.blocks = nn.ModuleList(
+                AttentionBlock(cfg, i) if k == "attn" else HyenaBlock(cfg, i, k) for i, k in enumerate(self.kinds))
+            self.norm = RMSNorm(D, cfg["eps"])
+        self.reset_parameters(seed)
+
+    @torch.no_grad()
+    def reset_parameters(self, seed=0):
+        dev = self.embedding.weight.device
+        g = torch.Generator(device=dev).manual_seed(seed)
+        for name, p in self.named_parameters():
+            if name.endswith("scale"):
+                p.fill_(1.0)
+            elif name.endswith("log_poles"):        # real, stable poles (vortex parametrisation)
+                p.copy_(-(0.01 + 0.5 * torch.rand(p.shape, generator=g, device=dev)))
+            elif name.endswith(".h"):
+                p.copy_(torch.randn(p.shape, generator=g, device=dev) / math.sqrt(p.shape[-1]))
+            elif name.endswith("short_filter_weight"):
+                p.copy_(torch.randn(p.shape, generator=g, device=dev) / math.sqrt(p.shape[-1]))
+            elif name.endswith("residues"):
+                p.copy_(torch.randn(p.shape, generator=g, device=dev) / 4.0)
+            elif name.endswith(".D") or name.endswith("bias"):
+                p.zero_()
+            else:
+                p.copy_(0.02 * torch.randn(p.shape, generator=g, device=dev))
+
+    def to_inference(self, device):
+        """bf16 everywhere except the modal parameters (vortex/model/model.py:1014-1030)."""
+        self.to(device)
+        for name, p in self.named_parameters():
+            if not (name.endswith("log_poles") or name.endswith("residues")):
+                p.data = p.data.to(torch.bfloat16)
+        return self.eval()
+
+    def initialize_inference_params(self):
+        """vortex/model/model.py:796-830: one cache object per operator family."""
+        return {"hcl": HyenaCascadeIIRInferenceParams(), "hcm": HyenaCascadeFIRInferenceParams(),
+                "hcs": HyenaCascadeFIRInferenceParams()}
+
+    @torch.no_grad()
+    def forward(self, input_ids, inference_params_dict=None):
+        x = self.embedding(input_ids)
+        for kind, block in zip(self.kinds, self.blocks):
+            ip = None if inference_params_dict is None or kind == "attn" else inference_params_dict[kind]
+            x, _ = block(x, inference_params=ip)
+        x = self.norm(x)
+        return x @ self.embedding.weight.T
