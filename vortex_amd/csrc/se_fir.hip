@@ -46,51 +46,41 @@ __global__ __launch_bounds__(256) void se_fir_kernel(RowMap x1, RowMap x2, RowMa
     for (int k = 0; k < K; ++k) w[k] = taps[g * K + k];
 
     const bf16_t* p1 = x1.row(b, d) + t0;
+    const bf16_t* pvv = PRE ? v.row(b, d) + t0 : nullptr;
     const u32x4 a1 = ld16<NT>(p1);
     u32x4 av = {0, 0, 0, 0}, a2 = {0, 0, 0, 0};
-    if (PRE) av = ld16<NT>(v.row(b, d) + t0);
+    if (PRE) av = ld16<NT>(pvv);
     if (POST) a2 = ld16<NT>(x2.row(b, d) + t0);
+    // lane 0 of a wavefront cannot get its halo from a neighbour: it reloads the previous octet, and
+    // the reload is issued here, together with the main loads, so that its latency is not exposed
+    const int lane = threadIdx.x & 63;
+    const bool reload = (lane == 0) && (oct != 0);
+    u32x4 h1 = {0, 0, 0, 0}, hv = {0, 0, 0, 0};
+    if (reload) {
+        h1 = *(const u32x4*)(p1 - 8);
+        if (PRE) hv = *(const u32x4*)(pvv - 8);
+    }
 
     // u = bf16(x1*v), kept both as floats and as packed bf16 pairs
     float u[8];
     uint32_t pk[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        if (PRE) {
-            const uint32_t lo = f_to_bf_bits(bf_lo(a1[j]) * bf_lo(av[j]));
-            const uint32_t hi = f_to_bf_bits(bf_hi(a1[j]) * bf_hi(av[j]));
-            pk[j] = lo | (hi << 16);
-        } else {
-            pk[j] = a1[j];
-        }
+        if (PRE) pk[j] = pack_bf2(bf_lo(a1[j]) * bf_lo(av[j]), bf_hi(a1[j]) * bf_hi(av[j]));
+        else pk[j] = a1[j];
         u[2 * j] = bf_lo(pk[j]);
         u[2 * j + 1] = bf_hi(pk[j]);
     }
 
-    // halo: last HD dwords of the previous lane's octet
+    // halo: last HD dwords of the previous lane's octet (zeros at the start of a row)
     uint32_t hp[HD];
 #pragma unroll
-    for (int j = 0; j < HD; ++j) hp[j] = __shfl_up(pk[4 - HD + j], 1, 64);
-    const int lane = threadIdx.x & 63;
-    if (lane == 0 || oct == 0) {
-        if (oct == 0) {
-#pragma unroll
-            for (int j = 0; j < HD; ++j) hp[j] = 0;          // zero left padding
-        } else {
-            const u32x4 h1 = *(const u32x4*)(p1 - 8);
-            u32x4 hv = {0, 0, 0, 0};
-            if (PRE) hv = *(const u32x4*)(v.row(b, d) + t0 - 8);
-#pragma unroll
-            for (int j = 0; j < HD; ++j) {
-                const int q = 4 - HD + j;
-                if (PRE) {
-                    const uint32_t lo = f_to_bf_bits(bf_lo(h1[q]) * bf_lo(hv[q]));
-                    const uint32_t hi = f_to_bf_bits(bf_hi(h1[q]) * bf_hi(hv[q]));
-                    hp[j] = lo | (hi << 16);
-                } else {
-                    hp[j] = h1[q];
-                }
-            }
+    for (int j = 0; j < HD; ++j) {
+        const int q = 4 - HD + j;
+        hp[j] = __shfl_up(pk[q], 1, 64);
+        if (lane == 0 || oct == 0) {
+            hp[j] = 0;
+            if (reload) hp[j] = PRE ? pack_bf2(bf_lo(h1[q]) * bf_lo(hv[q]), bf_hi(h1[q]) * bf_hi(hv[q])) : h1[q];
         }
     }
 
