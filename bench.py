@@ -24,6 +24,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0     # MI355X published HBM3E bandwidth
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
+# counter reads for the plain copy launch of known size (profiles/bench_default_hbm_traffic.txt).
+MEASURED_TRAFFIC = {"mr": 2178.42e6, "se": 271.75e6, "li": 8603.44e6}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -229,7 +233,8 @@ def main():
         "vs_baseline": None, "dtype": "bf16 in/out, fp32 accumulate", "data": "synthetic",
         "config": {"workload": m["workload"]},
         "roofline": {"bound": "hbm", "achieved": m["hbm_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": m["hbm_gbs"] / HBM_PEAK_GBS, "traffic": None, "kernel": m["kernel"],
+                     "frac": m["hbm_gbs"] / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(main_name),
+                     "kernel": m["kernel"],
                      "algorithmic_bytes_per_launch": m["bytes"], "kernel_ms": m["kernel_ms"]},
     }
     if not args.no_extras:
