@@ -152,3 +152,35 @@ def test_mr_full_size_rows():
     z = (O.fft_causal_conv_fp32(u.float(), w) + u.float() * Db[rows][:, None]).to(torch.bfloat16)
     ref = x2[:, rows] * z
     assert rel_err(out[:, rows], ref) <= TOL
+
+
+def test_se_nontemporal_variant_matches(monkeypatch):
+    # large activations take the non-temporal (streaming) code path; force it on a small case
+    B, D, L, G, K = 2, 64, 2048, 4, 7
+    x2, x1, v = O.make_gates(B, D, L, seed=13)
+    h = O.make_se_filter(G, K)
+    a = va.hyena_se_fwd(x1.cuda(), x2.cuda(), v.cuda(), h.cuda())
+    monkeypatch.setenv("HYENA_SE_NT", "1")
+    b = va.hyena_se_fwd(x1.cuda(), x2.cuda(), v.cuda(), h.cuda())
+    assert torch.equal(a, b)
+    monkeypatch.setenv("HYENA_MR_NT", "1")
+    hm = O.make_mr_filter(G, 128)
+    c = va.hyena_mr_fwd(x1.cuda(), x2.cuda(), v.cuda(), hm.cuda())
+    monkeypatch.setenv("HYENA_MR_NT", "0")
+    d = va.hyena_mr_fwd(x1.cuda(), x2.cuda(), v.cuda(), hm.cuda())
+    assert torch.equal(c, d)
+
+
+def test_argument_errors():
+    x = torch.zeros(1, 32, 64, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):                       # L not a multiple of 8
+        va.hyena_se_fwd(x[..., :60].contiguous(), x[..., :60].contiguous(), x[..., :60].contiguous(),
+                        torch.zeros(2, 1, 7, device="cuda"))
+    with pytest.raises(NotImplementedError):              # 8 channels per group: no MFMA tiling
+        va.hyena_mr_fwd(x, x, x, torch.zeros(4, 1, 128, device="cuda"))
+    with pytest.raises(NotImplementedError):              # K > 128
+        va.hyena_mr_fwd(x, x, x, torch.zeros(2, 1, 200, device="cuda"))
+    with pytest.raises(TypeError):
+        va.hyena_se_fwd(x.float(), x, x, torch.zeros(2, 1, 7, device="cuda"))
+    out = va.hyena_se_fwd(x[:0], x[:0], x[:0], torch.zeros(2, 1, 7, device="cuda"))     # empty batch
+    assert out.shape == (0, 32, 64)

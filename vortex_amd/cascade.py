@@ -86,6 +86,7 @@ class HyenaCascade(nn.Module):
             self.h = None
         self._plan = None
         self._decode = None
+        self._f32_cache = {}
 
     # ------------------------------------------------------------------
     def forward(self, u, inference_params=None, padding_mask=None, *args, **kwargs):
@@ -113,6 +114,19 @@ class HyenaCascade(nn.Module):
             x1, x2 = x2, x1
         return x2, x1, v
 
+    def _f32_param(self, name, shape=None):
+        """float32 contiguous copy of a (possibly bf16) parameter, rebuilt only when the parameter changes."""
+        p = getattr(self, name)
+        if p is None:
+            return None
+        key = (p.data_ptr(), p._version, p.dtype)
+        hit = self._f32_cache.get(name)
+        if hit is None or hit[0] != key:
+            t = p.detach().to(torch.float32)
+            hit = (key, (t.reshape(shape) if shape is not None else t).contiguous())
+            self._f32_cache[name] = hit
+        return hit[1]
+
     def modal_plan(self):
         key = (self.log_poles._version, self.residues._version, self.log_poles.data_ptr())
         if self._plan is None or self._plan[0] != key:
@@ -125,15 +139,15 @@ class HyenaCascade(nn.Module):
             raise NotImplementedError("padding_mask is handled by the drop-in engine, not by this module")
         B, L, C = u.shape
         D, Ks = self.hidden_size, self.short_filter_length
-        w = self.short_filter_weight.detach().reshape(C, Ks)
-        z_pre = ops.featurizer_fwd(u, w, self.short_filter_bias, interleave=self.interleave)
+        w = self._f32_param("short_filter_weight", (C, Ks))
+        z_pre = ops.featurizer_fwd(u, w, self._f32_param("short_filter_bias"), interleave=self.interleave)
         r1, r2, rv = self._rows(z_pre)
         K = self.fir_inner_filter_length
         caching = inference_params is not None
         if K:
-            taps = self.h.detach().reshape(self.h.shape[0], K)
+            taps = self._f32_param("h", (self.h.shape[0], K))
             if K >= 128:
-                y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, K, device=u.device, bias=ops._f32(self.D),
+                y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, K, device=u.device, bias=self._f32_param("D"),
                                      bias_mode=HYENA_BIAS_GATED_FP32, taps_reversed=False, force_mfma=True)
             else:
                 y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, K, device=u.device, taps_reversed=True)

@@ -86,6 +86,8 @@ def fir_fwd_rows(x1r, x2r, vr, taps, B, D, L, K, *, device, bias=None, bias_mode
     G = taps.shape[0]
     if out is None:
         out = torch.empty((B, D, L), dtype=torch.bfloat16, device=device)
+    if out.numel() == 0:
+        return out
     L_ = _lib.lib()
     if K <= 8 and not force_mfma:
         if not taps_reversed:
@@ -144,6 +146,8 @@ def featurizer_fwd(u, taps, bias=None, interleave=False):
     B, L, C = u.shape
     taps = _f32(taps)
     out = torch.empty((B, C, L), dtype=torch.bfloat16, device=u.device)
+    if out.numel() == 0:
+        return out
     b = _f32(bias)
     rc = _lib.lib().hyena_featurizer_fwd(_ptr(u), u.stride(0), u.stride(1), _ptr(taps), _ptr(b), int(interleave), _ptr(out),
                                          B, L, C, taps.shape[0], taps.shape[1], _stream())
@@ -179,7 +183,11 @@ def li_fwd_rows(x1r, x2r, vr, plan, Dcoef, B, D, L, *, device, want_state=False,
     if out is None:
         out = torch.empty((B, D, L), dtype=torch.bfloat16, device=device)
     y32 = torch.empty((B, D, L), dtype=torch.float32, device=device) if want_fp32 else None
-    state = torch.empty((B, D, plan.S, 2), dtype=torch.float32, device=device) if want_state else None
+    state = torch.zeros((B, D, plan.S, 2), dtype=torch.float32, device=device) if want_state else None
+    if out.numel() == 0:
+        if state is not None:
+            state = torch.view_as_complex(state) if plan.is_complex else state[..., 0].contiguous()
+        return out, y32, state
     dco = _f32(Dcoef)
     d_is_bf16 = 2 if single_rounding else int(Dcoef is None or Dcoef.dtype == torch.bfloat16)
     rc = _lib.lib().hyena_li_fwd(_ref(x1r), _ref(x2r), _ref(vr), _ptr(plan.workspace), _ptr(dco), d_is_bf16,
