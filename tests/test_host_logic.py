@@ -1,0 +1,92 @@
+"""Host-side logic that needs no GPU: row descriptors against the reference's split / column_split
+index maps, the ring-cache ordering, tap slicing, and the interleave permutation of the decode path."""
+import ctypes
+
+import pytest
+import torch
+
+from oracle import hyena_oracle as O
+from vortex_amd import ops
+from vortex_amd.engine import _group_taps
+
+
+def gather_rows(u, r, D):
+    """Reads channel d of batch b the way the kernels do: through the descriptor arithmetic."""
+    B, C, L = u.shape
+    flat = u.reshape(-1)
+    base = (r.ptr - u.data_ptr()) // u.element_size()
+    out = torch.empty(B, D, L, dtype=u.dtype)
+    for b in range(B):
+        for d in range(D):
+            row = (d // r.ch_inner) * r.ch_outer + d % r.ch_inner
+            s = base + b * r.batch_stride + row * r.row_stride
+            out[b, d] = flat[s:s + L]
+    return out
+
+
+@pytest.mark.parametrize("cs", [False, True])
+def test_row_descriptors_match_reference_split(cs):
+    B, D, L, H = 2, 24, 8, 4
+    u = torch.arange(B * 3 * D * L, dtype=torch.float32).reshape(B, 3 * D, L).bfloat16()
+    hd = D // H
+    ref = O.column_split(u, H, hd) if cs else u.split(D, dim=1)
+    for i in range(3):
+        r = ops.rows_of_projection(u, D, i, hd if cs else None)
+        assert torch.equal(gather_rows(u, r, D), ref[i])
+
+
+def test_rows_of_strided_view():
+    u = torch.arange(2 * 12 * 16, dtype=torch.float32).reshape(2, 12, 16).bfloat16()
+    x = u[:, 4:8]
+    r = ops.rows_of(x)
+    assert torch.equal(gather_rows(u, r, 4), x)
+    with pytest.raises(ValueError):
+        ops.rows_of(u.permute(0, 2, 1))           # samples not contiguous
+    with pytest.raises(TypeError):
+        ops.rows_of(u.float())
+
+
+def test_fir_ring_reference_order_and_rotation():
+    B, D, R = 2, 3, 5
+    st = torch.arange(B * D * R, dtype=torch.float32).reshape(B, D, R)
+    ring = ops.FirRing.from_reference(st)
+    assert ring.shape == torch.Size((B, D, R))
+    assert torch.equal(ring.reference_order(), st)
+    # emulate two steps: the oldest slot is overwritten, then the oldest moves on
+    for step in range(2):
+        new = torch.full((B, D), 100.0 + step)
+        ring.buf[:, ring.pos] = new.bfloat16()
+        ring.pos = (ring.pos + 1) % R
+        st = torch.cat([st[..., 1:], new[..., None]], dim=-1)
+        assert torch.equal(ring.reference_order(), st)
+
+
+def test_group_taps_undoes_repeat_interleave():
+    G, D, K = 4, 32, 7
+    h = torch.randn(G, 1, K)
+    assert torch.equal(_group_taps(h.repeat_interleave(D // G, 0), D, G), h[:, 0])
+    assert torch.equal(_group_taps(h, D, G), h[:, 0])
+    w = torch.randn(D, 1, 3)
+    assert torch.equal(_group_taps(w, D, None), w[:, 0])
+
+
+def test_decode_interleave_permutation_matches_reference():
+    C = 24
+    z = torch.arange(2 * C, dtype=torch.float32).reshape(2, C)
+    j = torch.arange(C)
+    perm = (j % (C // 3)) * 3 + j // (C // 3)      # the index map vortex_amd.cascade builds for decode
+    assert torch.equal(z[:, perm], O.interleave(z))
+
+
+def test_return_codes_map_to_exceptions():
+    from vortex_amd import _lib
+    assert _lib.check(0, "x") is None
+    for rc, exc in ((-1, ValueError), (-2, ValueError), (-3, NotImplementedError), (700, RuntimeError)):
+        with pytest.raises(exc):
+            _lib.check(rc, "some call")
+
+
+def test_rows_struct_layout_matches_header():
+    # hyena_rows: one pointer and four int64, no padding
+    assert ctypes.sizeof(ops.Rows) == 40
+    assert [f[0] for f in ops.Rows._fields_] == ["ptr", "batch_stride", "row_stride", "ch_inner", "ch_outer"]

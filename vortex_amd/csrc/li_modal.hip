@@ -510,7 +510,8 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     if (d_is_bf16 < 0 || d_is_bf16 > 2) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: d_is_bf16 must be 0, 1 or 2");
     if (B == 0 || L == 0) return 0;
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
-    const int cpw = ((D / G) % 4 == 0) ? 4 : 1;              // channels per wavefront (they share one filter)
+    int cpw = ((D / G) % 4 == 0) ? 4 : 1;                    // channels per wavefront (they share one filter)
+    if (const char* e = getenv("HYENA_LI_CPW")) { if (atoi(e) == 1) cpw = 1; }
     const int64_t nquads = B * (D / cpw);
     const int64_t nblk = (nquads + 3) / 4;
     if (nquads > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: problem too large for one launch");
