@@ -20,16 +20,18 @@ __global__ __launch_bounds__(256) void se_fir_kernel(RowMap x1, RowMap x2, RowMa
                                                      const float* __restrict__ taps,
                                                      const float* __restrict__ bias,
                                                      bf16_t* __restrict__ out,
-                                                     int64_t D, int64_t L, int dg,
+                                                     int64_t D, int64_t L, int dg, int dg_shift,
                                                      int64_t octs_per_row, int64_t total_octs) {
     constexpr int H = K - 1;                 // halo samples
     constexpr int HD = (H + 1) / 2;          // halo dwords taken from the previous lane
     // all index arithmetic in 32 bits: the host checks that B*D and L/8 fit
     uint32_t row, oct;
-    if (ROWU) {                              // a block never straddles rows: row is wave-uniform
-        const uint32_t blocks_per_row = (uint32_t)octs_per_row / 256u;
-        row = blockIdx.x / blocks_per_row;
-        oct = (blockIdx.x - row * blocks_per_row) * 256u + threadIdx.x;
+    uint32_t b, d;
+    if (ROWU) {                              // a block never straddles rows: grid = (blocks per row, D, B)
+        d = blockIdx.y;
+        b = blockIdx.z;
+        row = b * (uint32_t)D + d;
+        oct = blockIdx.x * 256u + threadIdx.x;
     } else {
         const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
         row = (uint32_t)(idx / (uint32_t)octs_per_row);
@@ -37,9 +39,10 @@ __global__ __launch_bounds__(256) void se_fir_kernel(RowMap x1, RowMap x2, RowMa
     }
     const bool active = ROWU ? true : ((uint64_t)row * (uint64_t)octs_per_row + oct < (uint64_t)total_octs);
     if (!active) { row = 0; oct = 0; }
-    const uint32_t b = row / (uint32_t)D, d = row - b * (uint32_t)D;
+    if (!ROWU) { b = row / (uint32_t)D; d = row - b * (uint32_t)D; }
     const int64_t t0 = (int64_t)oct * 8;
-    const int g = (int)(d / (uint32_t)dg);
+    // dg_shift >= 0: D/G is a power of two and the group index is a shift
+    const int g = dg_shift >= 0 ? (int)(d >> dg_shift) : (int)(d / (uint32_t)dg);
 
     float w[K];
 #pragma unroll
@@ -108,12 +111,11 @@ __global__ __launch_bounds__(256) void se_fir_kernel(RowMap x1, RowMap x2, RowMa
 #pragma unroll
             for (int k = 0; k < K; ++k) acc = fmaf(w[k], ext[i + k], acc);
             if (BIAS == HYENA_BIAS_GATED_FP32) acc = fmaf(bz, u[i], acc);
-            acc = round_bf(acc);
-            if (BIAS == HYENA_BIAS_ADD) acc = round_bf(acc + bz);
-            if (POST) acc = acc * (e ? bf_hi(a2[j]) : bf_lo(a2[j]));
             z[e] = acc;
         }
-        o[j] = pack_bf2(z[0], z[1]);
+        uint32_t zp = pack_bf2(z[0], z[1]);                      // z = bf16(conv), one conversion per pair
+        if (BIAS == HYENA_BIAS_ADD) zp = pack_bf2(bf_lo(zp) + bz, bf_hi(zp) + bz);
+        o[j] = POST ? pack_bf2(bf_lo(zp) * bf_lo(a2[j]), bf_hi(zp) * bf_hi(a2[j])) : zp;
     }
     if (active) {
         u32x4 ov = {o[0], o[1], o[2], o[3]};
@@ -125,8 +127,10 @@ __global__ __launch_bounds__(256) void se_fir_kernel(RowMap x1, RowMap x2, RowMa
 template <int K, bool PRE, bool POST, int BIAS>
 void launch_k(bool rowu, bool nt, dim3 grid, hipStream_t s, RowMap x1, RowMap x2, RowMap v, const float* taps,
               const float* bias, bf16_t* out, int64_t D, int64_t L, int dg, int64_t opr, int64_t tot) {
+    int dg_shift = -1;
+    if ((dg & (dg - 1)) == 0) { dg_shift = 0; while ((1 << dg_shift) < dg) ++dg_shift; }
 #define SE_GO(R, N) hipLaunchKernelGGL((se_fir_kernel<K, PRE, POST, BIAS, R, N>), grid, dim3(256), 0, s, x1, x2, v, \
-                                      taps, bias, out, D, L, dg, opr, tot)
+                                      taps, bias, out, D, L, dg, dg_shift, opr, tot)
     if (rowu && nt) SE_GO(true, true);
     else if (rowu) SE_GO(true, false);
     else if (nt) SE_GO(false, true);
@@ -174,13 +178,14 @@ extern "C" int hyena_se_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
         return hyena_fail(HYENA_EINVAL, "hyena_se_fwd: B*D, L/8 and the channel map must fit 31 bits");
     if (B == 0 || L == 0) return 0;
     const int64_t opr = L / 8, tot = B * D * opr;
-    const bool rowu = (opr % 256 == 0);
+    const bool rowu = (opr % 256 == 0) && D <= 65535 && B <= 65535;
     // activations larger than the last-level cache stream through it: non-temporal accesses then
     bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
     if (const char* e = getenv("HYENA_SE_NT")) nt = atoi(e) != 0;
     const int64_t nblk = (tot + 255) / 256;
     if (nblk > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "hyena_se_fwd: problem too large for one launch");
     dim3 grid((unsigned)nblk);
+    if (rowu) grid = dim3((unsigned)(opr / 256), (unsigned)D, (unsigned)B);
     hipStream_t s = (hipStream_t)stream;
     RowMap m1 = make_rowmap(x1), m2 = make_rowmap(post ? x2 : nullptr), mv = make_rowmap(pre ? v : nullptr);
     const int dg = (int)(D / G);
