@@ -136,6 +136,40 @@ def decode_layer_set(D, device, steps, warmup):
                 hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
 
 
+def decode_layers_from_projection(D, device, steps, warmup):
+    """The same layer set stepped from each layer's projection output u [B, 3D] (Evo 2 layout: interleaved
+    gates, K=3 featurizer): featurizer step, split, gates and inner step in one launch per layer."""
+    import vortex_amd as va
+    from vortex_amd import ops
+    from oracle import hyena_oracle as O
+    B, S, C = 64, 16, 3 * D
+    g = torch.Generator(device=device).manual_seed(7)
+    rnd = lambda *s: torch.randn(*s, generator=g, device=device, dtype=torch.float32)
+    G = D // 16
+    cmap = ops.gate_channel_map(D, interleave=True)
+    lp, r = O.make_modal_complex(G, S)
+    state = torch.zeros(B, D, S, dtype=torch.complex64, device=device)
+    inner = [ops.FirStepper(va.FirRing(rnd(B, 6, D).to(torch.bfloat16)), rnd(G, 7) * 7 ** -0.5),
+             ops.FirStepper(va.FirRing(rnd(B, 127, D).to(torch.bfloat16)), rnd(G, 128) * 128 ** -0.5, bias=rnd(D),
+                            gated_bias=True),
+             ops.IirStepper(state, torch.exp(lp[..., 0]).to(device), r.to(device), rnd(D).to(torch.bfloat16))]
+    layers = [ops.LayerStepper(va.FirRing(rnd(B, 2, C).to(torch.bfloat16)), rnd(C, 3) * 3 ** -0.5, None, cmap, n)
+              for n in inner]
+    u = [rnd(B, C).to(torch.bfloat16) for _ in range(3)]
+    out = [torch.empty(B, D, dtype=torch.bfloat16, device=device) for _ in range(3)]
+
+    def fn():
+        for l, x, o in zip(layers, u, out):
+            l(x, o)
+
+    wall, ms = time_steps(fn, steps, warmup)
+    # inner caches / state as in decode_layer_set; per layer the projection row, two featurizer slots read and
+    # one written (3D channels each) and one output row
+    byts = B * D * 2 * (6 + 127) + 2 * B * D * 2 + 2 * state.numel() * 8 + 3 * (4 * B * C * 2 + B * D * 2)
+    return dict(us_per_step=ms * 1e3, wall_us_per_step=wall / steps * 1e6, bytes=byts,
+                hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
+
+
 def model_prefill(device, L, iters=2):
     """Evo 2 7B-shaped random-init StripedHyena 2 prefill (32 blocks [SE, MR, LI, attention], hidden 4096,
     MLP 11008, vocab 512): Hyena operators on the HIP kernels, projections / MLP / attention through torch."""
@@ -249,6 +283,8 @@ def main():
                            "roofline_frac": e["hbm_gbs"] / HBM_PEAK_GBS}
         for D in (4096, 8192):
             extra[f"decode_D{D}"] = decode_layer_set(D, device, max(args.steps, 50), max(args.warmup, 5))
+        extra["decode_from_projection_D4096"] = decode_layers_from_projection(4096, device, max(args.steps, 50),
+                                                                              max(args.warmup, 5))
         if not args.no_model:
             for L in (8192, 131072):
                 extra[f"model_L{L}"] = model_prefill(device, L)

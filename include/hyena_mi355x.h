@@ -157,6 +157,44 @@ int hyena_iir_step(const void* x1, const void* x2, const void* v, int64_t in_bat
                    void* out, int out_is_fp32, int64_t out_batch_stride,
                    int64_t B, int64_t D, int64_t G, int64_t S, void* stream);
 
+/* The featurizer's own decode step (vortex/model/model.py:325-330: step_fir on the 3D-channel
+ * projection with the short filter, then interleave / split, model.py:332-343), described so that a
+ * layer step can evaluate it on the fly and the gates x2, x1, v never pass through device memory:
+ *   z[c] = bf16( sum_{i<Rf} w[i][c]*slot_i[c] + w[Rf][c]*u[c] (+ bias[c]) ),  slot (pos) <- u
+ * Gate i (0: x2, 1: x1, 2: v) of operator channel d is z at channel
+ *   (d / ch_inner)*ch_outer + i*gate_stride + (d % ch_inner)*ch_stride
+ * plain split: ch_inner = D, gate_stride = D, ch_stride = 1; head-blocked column_split
+ * (vortex/model/utils.py:41-85): ch_inner = gate_stride = head_dim, ch_outer = 3*head_dim, ch_stride = 1;
+ * interleave (utils.py:26-38) followed by the plain split: ch_inner = D, gate_stride = 1, ch_stride = 3.
+ * flip_x1x2 != 0 swaps gates 0 and 1 (vortex/model/engine.py:160-161). */
+typedef struct hyena_proj_step {
+    const void* u;            /* [B][3D] bf16: this token's projection, channels contiguous        */
+    int64_t u_batch_stride;   /* elements                                                          */
+    void* ring;               /* [B][Rf][3D] bf16 featurizer cache; slot (pos+i) % Rf = i-th oldest */
+    int64_t Rf, pos;          /* the caller advances pos to (pos+1) % Rf after the call            */
+    const float* w;           /* [Rf+1][3D] float32, tap-major, oldest tap first                   */
+    const float* bias;        /* [3D] float32 or NULL                                              */
+    int64_t ch_inner, ch_outer, gate_stride, ch_stride;
+    int flip_x1x2;
+} hyena_proj_step;
+
+/* hyena_fir_step / hyena_iir_step with the featurizer step of the same layer fused in: one launch per
+ * Hyena layer and token.  Same arithmetic as the featurizer's hyena_fir_step (bias rule ADD) followed by
+ * the gated step; the featurizer cache slot and the inner cache / state are both updated.
+ * hyena_fir_layer_step needs one of the three channel maps listed above, 16-byte aligned pointers and
+ * head_dim % 8 == 0; it takes bias_mode NONE or GATED_FP32.  hyena_iir_layer_step takes any map; not
+ * available for 8 real states. */
+int hyena_fir_layer_step(const hyena_proj_step* proj,
+                         void* ring, int64_t R, int64_t pos,
+                         const float* w, const float* bias, int bias_mode,
+                         void* out, int64_t out_batch_stride,
+                         int64_t B, int64_t D, int64_t G, void* stream);
+int hyena_iir_layer_step(const hyena_proj_step* proj,
+                         float* state, const float* poles, const float* residues, int is_complex,
+                         const float* Dcoef, int d_is_bf16,
+                         void* out, int out_is_fp32, int64_t out_batch_stride,
+                         int64_t B, int64_t D, int64_t G, int64_t S, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -124,9 +124,11 @@ def test_engine_dropin_modal_layer_per_channel_filters(cs, il):
         assert rel_err(y_hip, y_ref) <= 2e-2, i
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("kind,cs,il", [("se", False, True), ("mr", False, True), ("mr", True, False),
-                                         ("li_cplx", False, True), ("li_real", True, False)])
-def test_operator_module_prefill_then_decode(kind, cs, il):
+                                         ("li_cplx", False, True), ("li_real", True, False), ("se", False, False),
+                                         ("li_real", False, False), ("mr", True, True)])
+def test_operator_module_prefill_then_decode(kind, cs, il, fused):
     # vortex_amd.cascade.HyenaCascade (fused fast path) against the oracle call sequence
     B, L, D, H, n_dec = 2, 512, 64, 4, 4
     K = {"se": 7, "mr": 128}.get(kind)
@@ -145,6 +147,7 @@ def test_operator_module_prefill_then_decode(kind, cs, il):
         if mod.D is not None:
             mod.D.data = p["D"].clone()
     mod = mod.to(DEV)
+    mod.fuse_decode = fused
     if K is None:     # oracle needs per-channel modal parameters
         pr = dict(p, log_poles=p["log_poles"].repeat_interleave(D // G, 0),
                   residues=p["residues"].repeat_interleave(D // G, 0))
@@ -164,6 +167,8 @@ def test_operator_module_prefill_then_decode(kind, cs, il):
         y_ref, _ = ref.forward(tok, ip_ref)
         y_hip, _ = mod(tok.to(DEV), ip_hip)
         assert rel_err(y_hip, y_ref) <= 2e-2, i
+    if fused:   # one launch per step wherever a closed channel map exists (not interleave + column split)
+        assert (mod._decode["layer"] is not None) == (not (cs and il))
 
 
 def test_hyena_ops_interface_layouts():

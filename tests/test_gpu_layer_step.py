@@ -1,0 +1,126 @@
+"""GPU parity of the one-launch decode layer steps (featurizer step + split + gated FIR / IIR step)
+against the oracle's step_fir / step_iir chain, through the C ABI."""
+import pytest
+import torch
+
+import vortex_amd as va
+from vortex_amd import ops
+from oracle import hyena_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def rel_err(a, b):
+    a, b = a.float().cpu(), b.float().cpu()
+    return ((a - b).abs().max() / b.abs().max().clamp_min(1e-30)).item()
+
+
+def oracle_gates(z, D, H, cs, il, flip):
+    """Interleave / split of vortex/model/model.py:332-343 on a [B, 3D] featurizer output."""
+    if il:
+        z = O.interleave(z)
+    if cs:
+        x2, x1, v = O.column_split(z, H, D // H)
+    else:
+        x2, x1, v = z.split([D, D, D], dim=1)
+    return (x1, x2, v) if flip else (x2, x1, v)
+
+
+@pytest.mark.parametrize("B,D,H,G,K,Ks,cs,il,flip,sbias", [
+    (3, 512, 8, 32, 7, 3, False, True, False, False),      # Evo 2 layout: interleave, grouped SE taps
+    (2, 1024, 16, 64, 128, 3, False, True, False, True),   # MR, gated fp32 bias, featurizer bias
+    (2, 256, 4, 256, 7, 4, True, False, False, False),     # head-blocked column split, per-channel taps
+    (2, 520, 5, 65, 128, 3, False, False, True, False),    # plain split, x1/x2 flipped, D % 512 != 0
+    (1, 64, 4, 4, 7, 2, True, False, True, True),
+])
+def test_fir_layer_step_sequence_vs_oracle(B, D, H, G, K, Ks, cs, il, flip, sbias):
+    g = torch.Generator().manual_seed(K * 100 + D + Ks)
+    C, R, Rf = 3 * D, K - 1, Ks - 1
+    mr = K >= 128
+    wf = torch.randn(C, 1, Ks, generator=g) / Ks ** 0.5
+    bf = torch.randn(C, generator=g) if sbias else None
+    w = torch.randn(G, 1, K, generator=g) / K ** 0.5
+    wD = w.repeat_interleave(D // G, 0)
+    bias = torch.randn(D, generator=g) if mr else None
+    fst = torch.randn(B, C, Rf, generator=g).bfloat16()
+    st = torch.randn(B, D, R, generator=g).bfloat16()
+    fring, ring = va.FirRing.from_reference(fst.to(DEV)), va.FirRing.from_reference(st.to(DEV))
+    taps = (w.reshape(G, K).flip(-1) if mr else w.reshape(G, K)).contiguous().to(DEV)
+    inner = ops.FirStepper(ring, taps, bias=None if bias is None else bias.to(DEV), gated_bias=mr)
+    cmap = ops.gate_channel_map(D, interleave=il, head_dim=D // H if cs else None)
+    step = ops.LayerStepper(fring, wf.reshape(C, Ks).to(DEV), None if bf is None else bf.to(DEV), cmap, inner,
+                            flip_x1x2=flip)
+    ref_f, ref_s = fst, st
+    for i in range(max(R, Rf) + 3):
+        u = torch.randn(B, C, generator=g).bfloat16()
+        z, ref_f = O.step_fir(u, ref_f, wf, bias=bf)
+        x2, x1, v = oracle_gates(z, D, H, cs, il, flip)
+        y_ref, ref_s = O.step_fir(x1 * v, ref_s, wD, bias=bias, gated_bias=mr, flip_filter=mr)
+        y_ref = y_ref * x2
+        y = torch.empty(B, D, dtype=torch.bfloat16, device=DEV)
+        step(u.to(DEV), y)
+        assert rel_err(y, y_ref) <= 2e-2, i
+        if i in (0, Rf, R - 1, R + 2):
+            assert torch.equal(fring.reference_order().cpu(), ref_f.float())          # copies of u: exact
+            assert rel_err(ring.reference_order(), ref_s) <= 1e-2
+
+
+@pytest.mark.parametrize("B,D,H,G,S,cplx,cs,il,flip,d_bf16", [
+    (3, 512, 8, 512, 16, False, False, True, False, True),    # Evo 2 layout: real poles, one filter per channel
+    (2, 256, 4, 16, 16, True, False, True, False, False),     # complex poles, grouped
+    (2, 96, 4, 96, 16, True, True, False, True, False),       # column split (head_dim 24), flipped
+    (2, 200, 5, 200, 32, False, False, False, False, True),   # plain split, 32 states
+    (1, 64, 4, 64, 8, True, True, True, False, False),        # interleave + column split has no fused map
+])
+def test_iir_layer_step_sequence_vs_oracle(B, D, H, G, S, cplx, cs, il, flip, d_bf16):
+    g = torch.Generator().manual_seed(D + S)
+    C, Ks = 3 * D, 3
+    wf = torch.randn(C, 1, Ks, generator=g) / Ks ** 0.5
+    if cplx:
+        lp, r = O.make_modal_complex(G, S, seed=D)
+    else:
+        lp, r = O.make_modal_real(G, S, seed=D)
+    Dc = torch.randn(D, generator=g)
+    Dc = Dc.bfloat16() if d_bf16 else Dc
+    fst = torch.randn(B, C, Ks - 1, generator=g).bfloat16()
+    st0 = torch.randn(B, D, S, generator=g)
+    if cplx:
+        st0 = torch.complex(st0, torch.randn(B, D, S, generator=g))
+    cmap = ops.gate_channel_map(D, interleave=il, head_dim=D // H if cs else None)
+    if cmap is None:
+        return
+    state = st0.clone().to(DEV)
+    fring = va.FirRing.from_reference(fst.to(DEV))
+    poles = torch.exp(lp)[..., 0].contiguous()
+    inner = ops.IirStepper(state, poles.to(DEV), r.to(DEV), Dc.to(DEV))
+    step = ops.LayerStepper(fring, wf.reshape(C, Ks).to(DEV), None, cmap, inner, flip_x1x2=flip)
+    dg = D // G
+    lpD, rD = lp.repeat_interleave(dg, 0), r.repeat_interleave(dg, 0)
+    ref_f, ref_s = fst, st0
+    for i in range(5):
+        u = torch.randn(B, C, generator=g).bfloat16()
+        z, ref_f = O.step_fir(u, ref_f, wf)
+        x2, x1, v = oracle_gates(z, D, H, cs, il, flip)
+        y_ref, ref_s = O.step_iir(x2, x1, v, Dc, rD, lpD, ref_s)
+        y_ref = y_ref.real if y_ref.is_complex() else y_ref
+        y = torch.empty(B, D, dtype=torch.bfloat16, device=DEV)
+        step(u.to(DEV), y)
+        assert rel_err(y, y_ref) <= 2e-2, i
+        assert torch.equal(fring.reference_order().cpu(), ref_f.float())
+        sr = torch.view_as_real(ref_s) if cplx else ref_s
+        sh = torch.view_as_real(state) if cplx else state
+        assert rel_err(sh, sr) <= 1e-2, i
+
+
+def test_layer_step_rejects_bad_maps():
+    D = 64
+    fring = va.FirRing(torch.zeros(1, 2, 3 * D, dtype=torch.bfloat16, device=DEV))
+    ring = va.FirRing(torch.zeros(1, 6, D, dtype=torch.bfloat16, device=DEV))
+    inner = ops.FirStepper(ring, torch.zeros(D, 7, device=DEV))
+    wf = torch.zeros(3 * D, 3, device=DEV)
+    u, y = torch.zeros(1, 3 * D, dtype=torch.bfloat16, device=DEV), torch.empty(1, D, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):          # map runs past the 3D channels
+        ops.LayerStepper(fring, wf, None, (D, 0, D + 8, 1), inner)(u, y)
+    with pytest.raises(NotImplementedError):  # head_dim not a multiple of 8 has no vector kernel
+        ops.LayerStepper(fring, wf, None, (4, 12, 4, 1), inner)(u, y)

@@ -14,12 +14,20 @@ HYENA_BIAS_NONE, HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32 = 0, 1, 2
 EXPORTS = [
     "hyena_version", "hyena_last_error_string", "hyena_se_fwd", "hyena_mr_fwd",
     "hyena_fir_step", "hyena_iir_step", "hyena_li_plan_bytes", "hyena_li_plan", "hyena_li_fwd", "hyena_featurizer_fwd", "hyena_copy_probe",
+    "hyena_fir_layer_step", "hyena_iir_layer_step",
 ]
 
 
 class Rows(Structure):
     _fields_ = [("ptr", c_void_p), ("batch_stride", c_int64), ("row_stride", c_int64),
                 ("ch_inner", c_int64), ("ch_outer", c_int64)]
+
+
+class ProjStep(Structure):
+    """hyena_proj_step: the featurizer decode step a layer step evaluates on the fly."""
+    _fields_ = [("u", c_void_p), ("u_batch_stride", c_int64), ("ring", c_void_p), ("Rf", c_int64), ("pos", c_int64),
+                ("w", c_void_p), ("bias", c_void_p), ("ch_inner", c_int64), ("ch_outer", c_int64),
+                ("gate_stride", c_int64), ("ch_stride", c_int64), ("flip_x1x2", c_int)]
 
 
 _lib = None
@@ -53,6 +61,11 @@ def lib():
     L.hyena_featurizer_fwd.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int64,
                                        c_int64, c_int64, c_int64, c_int, c_void_p]
     L.hyena_copy_probe.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
+    P = POINTER(ProjStep)
+    L.hyena_fir_layer_step.argtypes = [P, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int64,
+                                       c_int64, c_int64, c_int64, c_void_p]
+    L.hyena_iir_layer_step.argtypes = [P, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+                                       c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p]
     for name in EXPORTS:
         fn = getattr(L, name)
         if name not in ("hyena_version", "hyena_last_error_string"):

@@ -86,6 +86,7 @@ class HyenaCascade(nn.Module):
             self.h = None
         self._plan = None
         self._decode = None
+        self.fuse_decode = True        # one launch per decode step where the fused layer-step kernels apply
         self._f32_cache = {}
 
     # ------------------------------------------------------------------
@@ -193,8 +194,24 @@ class HyenaCascade(nn.Module):
             st = inference_params.state_dict[i]
             poles = torch.exp(self.log_poles.detach())[..., 0].contiguous()
             d["inner"] = ops.IirStepper(st, poles, self.residues.detach(), self.D.detach())
+        d["layer"] = self._fused_step(ring, d["inner"])
         self._decode = d
         return d
+
+    def _fused_step(self, ring, inner):
+        """The one-launch layer step, or None where the fused kernels do not apply (then three launches are used)."""
+        cmap = ops.gate_channel_map(self.hidden_size, interleave=self.interleave,
+                                    head_dim=self.hidden_size_per_attention_head if self.column_split_hyena else None)
+        Ks, hd = self.short_filter_length, self.hidden_size_per_attention_head
+        fir = isinstance(inner, ops.FirStepper)
+        if cmap is None or Ks < 2 or Ks > 8 or self.hidden_size % 8:
+            return None
+        if fir and (inner.mode == HYENA_BIAS_ADD or (self.column_split_hyena and hd % 8)):
+            return None
+        if not fir and inner.S == 8 and not inner.cplx:
+            return None
+        return ops.LayerStepper(ring, self.short_filter_weight.detach().reshape(3 * self.hidden_size, Ks),
+                                self.short_filter_bias, cmap, inner, flip_x1x2=self.hyena_flip_x1x2)
 
     def sequential_forward(self, u, inference_params):
         """Decode: u [B, 3D] or [B, 1, 3D] bf16 -> y [B, 1, D] (vortex/model/model.py:318-375)."""
@@ -202,6 +219,10 @@ class HyenaCascade(nn.Module):
             u = u[:, -1]
         d = self._decode_plan(inference_params)
         B = u.shape[0]
+        if self.fuse_decode and d["layer"] is not None and u.stride(1) == 1 and u.stride(0) % 8 == 0 and u.data_ptr() % 16 == 0:
+            y = torch.empty(B, self.hidden_size, dtype=torch.bfloat16, device=u.device)
+            d["layer"](u, y)
+            return y[:, None], inference_params
         z_pre = torch.empty(B, 3 * self.hidden_size, dtype=torch.bfloat16, device=u.device)
         d["feat"](u, None, None, z_pre)
         if self.interleave:

@@ -6,15 +6,89 @@
 
 namespace {
 
+// ---------------------------------------------------------------- fused featurizer step
+// Device copy of hyena_proj_step.  The featurizer (short FIR over the 3D projection
+// channels, vortex/model/model.py:325-330) is evaluated for exactly the channels a
+// lane needs, and the lane that evaluates a channel also writes the new sample into
+// that channel's ring slot, so no other lane ever reads a slot that is being replaced.
+struct ProjArgs {
+    const bf16_t* u;
+    int64_t u_bs;
+    bf16_t* ring;
+    int Rf, pos, C;
+    const float* w;        // [Rf+1][C], tap-major
+    const float* bias;     // [C] or null
+    uint32_t ch_inner, ch_outer, gate_stride, ch_stride;
+    int flip;
+    __device__ __forceinline__ uint32_t chan(uint32_t gate, uint32_t d) const {
+        return (d / ch_inner) * ch_outer + gate * gate_stride + (d % ch_inner) * ch_stride;
+    }
+};
+
+// z[j] = bf16( sum_i w[i][c0+j]*slot_i[c0+j] + w[Rf][c0+j]*u[c0+j] (+ bias) ) for 8 consecutive channels
+__device__ __forceinline__ void proj_step8(const ProjArgs& pj, int64_t b, uint32_t c0, float* z) {
+    const u32x4 un = *(const u32x4*)(pj.u + b * pj.u_bs + c0);
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    bf16_t* rb = pj.ring + (b * pj.Rf) * pj.C + c0;
+    for (int i = 0; i < pj.Rf; ++i) {
+        int s = pj.pos + i;
+        if (s >= pj.Rf) s -= pj.Rf;
+        const u32x4 q = *(const u32x4*)(rb + (int64_t)s * pj.C);
+        const f32x4 t0 = *(const f32x4*)(pj.w + (int64_t)i * pj.C + c0);
+        const f32x4 t1 = *(const f32x4*)(pj.w + (int64_t)i * pj.C + c0 + 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            acc[2 * j] = fmaf(j < 2 ? t0[2 * j] : t1[2 * j - 4], bf_lo(q[j]), acc[2 * j]);
+            acc[2 * j + 1] = fmaf(j < 2 ? t0[2 * j + 1] : t1[2 * j - 3], bf_hi(q[j]), acc[2 * j + 1]);
+        }
+    }
+    const f32x4 h0 = *(const f32x4*)(pj.w + (int64_t)pj.Rf * pj.C + c0);
+    const f32x4 h1 = *(const f32x4*)(pj.w + (int64_t)pj.Rf * pj.C + c0 + 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        acc[2 * j] = fmaf(j < 2 ? h0[2 * j] : h1[2 * j - 4], bf_lo(un[j]), acc[2 * j]);
+        acc[2 * j + 1] = fmaf(j < 2 ? h0[2 * j + 1] : h1[2 * j - 3], bf_hi(un[j]), acc[2 * j + 1]);
+    }
+    if (pj.bias) {
+        const f32x4 b0 = *(const f32x4*)(pj.bias + c0), b1 = *(const f32x4*)(pj.bias + c0 + 4);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] += j < 4 ? b0[j] : b1[j - 4];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) z[j] = round_bf(acc[j]);
+    *(u32x4*)(rb + (int64_t)pj.pos * pj.C) = un;        // the oldest slot takes the new sample
+}
+
+// the three gates of 8 consecutive operator channels d0..d0+7: g[0] = x2, g[1] = x1, g[2] = v (before any flip)
+template <int FEAT>
+__device__ __forceinline__ void proj_gates8(const ProjArgs& pj, int64_t b, uint32_t d0, float (*g)[8]) {
+    if (FEAT == 3) {            // interleaved: channels 3*d0 .. 3*d0+23, gate = channel % 3
+        float z[24];
+        proj_step8(pj, b, 3 * d0, z);
+        proj_step8(pj, b, 3 * d0 + 8, z + 8);
+        proj_step8(pj, b, 3 * d0 + 16, z + 16);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int i = 0; i < 3; ++i) g[i][j] = z[3 * j + i];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 3; ++i) proj_step8(pj, b, pj.chan(i, d0), g[i]);
+    }
+}
+
 // ---------------------------------------------------------------- FIR step
 // Block = NSG wavefronts over the same 512 channels; wavefront sg handles cache
 // slots sg, sg+NSG, ... so every load instruction reads 1 KiB of one slot row.
 // NSG = 8 for deep caches (enough loads in flight to cover HBM latency), 2 for shallow ones.
 // Ring layout [B][R][D]: channels contiguous, so the slot written back is one
 // coalesced row per batch element.
-template <bool PRE, bool POST, int BIAS, bool GROUPED, int NSG>
+// FEAT != 0: the gates come from the fused featurizer step (ProjArgs) instead of x1, x2, v.
+template <bool PRE, bool POST, int BIAS, bool GROUPED, int NSG, int FEAT>
 __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __restrict__ x1, const bf16_t* __restrict__ x2,
-                                                       const bf16_t* __restrict__ v, int64_t in_bs,
+                                                       const bf16_t* __restrict__ v, int64_t in_bs, ProjArgs pj,
                                                        bf16_t* __restrict__ ring, int R, int pos,
                                                        const float* __restrict__ w, const float* __restrict__ bias,
                                                        bf16_t* __restrict__ out, int64_t out_bs, int64_t D, int dg) {
@@ -71,6 +145,17 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
     // the first batch of cache reads goes out before the tap table is staged, so HBM is busy from the start
     u32x4 q0[UF];
     load_batch(sg, q0);
+    uint32_t f1[4], f2[4], fv[4];           // packed gates from the fused featurizer
+    if (FEAT != 0 && sg == 0 && live) {
+        float g[3][8];
+        proj_gates8<FEAT>(pj, b, (uint32_t)d0, g);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            f1[j] = pack_bf2(pj.flip ? g[0][2 * j] : g[1][2 * j], pj.flip ? g[0][2 * j + 1] : g[1][2 * j + 1]);
+            f2[j] = pack_bf2(pj.flip ? g[1][2 * j] : g[0][2 * j], pj.flip ? g[1][2 * j + 1] : g[0][2 * j + 1]);
+            fv[j] = pack_bf2(g[2][2 * j], g[2][2 * j + 1]);
+        }
+    }
     if (GROUPED) {
         const int64_t g0 = dblk / dg;
         const int64_t gmax = (D + dg - 1) / dg;
@@ -107,10 +192,15 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
 #pragma unroll
         for (int c = 0; c < 8; ++c) acc[c] += red[(k * 64 + oc) * 8 + c];
 
-    const u32x4 a1 = *(const u32x4*)(x1 + b * in_bs + d0);
-    u32x4 av = {0, 0, 0, 0}, a2 = {0, 0, 0, 0};
-    if (PRE) av = *(const u32x4*)(v + b * in_bs + d0);
-    if (POST) a2 = *(const u32x4*)(x2 + b * in_bs + d0);
+    u32x4 a1, av = {0, 0, 0, 0}, a2 = {0, 0, 0, 0};
+    if (FEAT != 0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { a1[j] = f1[j]; av[j] = fv[j]; a2[j] = f2[j]; }
+    } else {
+        a1 = *(const u32x4*)(x1 + b * in_bs + d0);
+        if (PRE) av = *(const u32x4*)(v + b * in_bs + d0);
+        if (POST) a2 = *(const u32x4*)(x2 + b * in_bs + d0);
+    }
     uint32_t up[4], o[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -141,9 +231,10 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
 // LPB lanes share one (batch, channel): each holds 16 bytes of its modal state
 // (4 real or 2 complex states), so state traffic is fully coalesced.  The
 // residue-weighted sum is reduced with xor shuffles inside the lane group.
-template <int S, bool CPLX>
+// FEAT: lanes 0..2 of a lane group evaluate the fused featurizer step for gates x2, x1, v of their channel.
+template <int S, bool CPLX, bool FEAT>
 __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict__ x1, const bf16_t* __restrict__ x2,
-                                                       const bf16_t* __restrict__ v, int64_t in_bs,
+                                                       const bf16_t* __restrict__ v, int64_t in_bs, ProjArgs pj,
                                                        float* __restrict__ state, const float* __restrict__ poles,
                                                        const float* __restrict__ residues,
                                                        const float* __restrict__ Dcoef, int d_is_bf16,
@@ -162,7 +253,34 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
     const f32x4 st = *(const f32x4*)sp;
     const f32x4 pp = *(const f32x4*)(poles + (g * S) * FPS + q * 4);
     const f32x4 rr = *(const f32x4*)(residues + (g * S) * FPS + q * 4);
-    const float a = bf_to_f(x1[b * in_bs + d]), c = bf_to_f(v[b * in_bs + d]);
+    float a, c, gate2 = 0.f;
+    if (FEAT) {
+        static_assert(!FEAT || LPB >= 4, "the fused featurizer needs three lanes per channel");
+        float z = 0.f;
+        if (q < 3) {
+            const uint32_t ch = pj.chan((uint32_t)q, (uint32_t)d);
+            bf16_t* rb = pj.ring + (b * pj.Rf) * pj.C + ch;
+            const bf16_t un = pj.u[b * pj.u_bs + ch];
+            float acc = 0.f;
+            for (int i = 0; i < pj.Rf; ++i) {
+                int s = pj.pos + i;
+                if (s >= pj.Rf) s -= pj.Rf;
+                acc = fmaf(pj.w[(int64_t)i * pj.C + ch], bf_to_f(rb[(int64_t)s * pj.C]), acc);
+            }
+            acc = fmaf(pj.w[(int64_t)pj.Rf * pj.C + ch], bf_to_f(un), acc);
+            if (pj.bias) acc += pj.bias[ch];
+            z = round_bf(acc);
+            if (live) rb[(int64_t)pj.pos * pj.C] = un;
+        }
+        const int base = (threadIdx.x & 63) & ~(LPB - 1);
+        const float g2 = __shfl(z, base, 64), g1 = __shfl(z, base + 1, 64);
+        c = __shfl(z, base + 2, 64);
+        a = pj.flip ? g2 : g1;
+        gate2 = pj.flip ? g1 : g2;
+    } else {
+        a = bf_to_f(x1[b * in_bs + d]);
+        c = bf_to_f(v[b * in_bs + d]);
+    }
     const float x1v = round_bf(a * c);
     f32x4 ns;
     float part;
@@ -184,7 +302,7 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
     if (live && q == 0) {
         float dx = Dcoef[d] * x1v;
         if (d_is_bf16) dx = round_bf(dx);
-        const float y = bf_to_f(x2[b * in_bs + d]) * (part + dx);
+        const float y = (FEAT ? gate2 : bf_to_f(x2[b * in_bs + d])) * (part + dx);
         if (out_is_fp32) ((float*)out)[b * out_bs + d] = y;
         else ((bf16_t*)out)[b * out_bs + d] = (bf16_t)f_to_bf_bits(y);
     }
@@ -192,68 +310,129 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
 
 }  // namespace
 
-extern "C" int hyena_fir_step(const void* x1, const void* x2, const void* v, int64_t in_bs, void* ring, int64_t R,
-                              int64_t pos, const float* w, const float* bias, int bias_mode, void* out,
-                              int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream) {
-    if (!x1 || !ring || !w || !out) return hyena_fail(HYENA_EINVAL, "hyena_fir_step: x1, ring, w, out are required");
+// Validates a fused-featurizer descriptor and converts it; returns 0 or an error code.
+static int make_proj(const hyena_proj_step* p, int64_t D, const char* who, ProjArgs* out) {
+    if (!p->u || !p->ring || !p->w) return hyena_fail(HYENA_EINVAL, "%s: proj u, ring, w are required", who);
+    if (p->Rf < 1 || p->Rf > 7 || p->pos < 0 || p->pos >= p->Rf)
+        return hyena_fail(HYENA_EINVAL, "%s: featurizer cache depth %lld / position %lld", who, (long long)p->Rf,
+                          (long long)p->pos);
+    const int64_t C = 3 * D;
+    if (p->ch_inner <= 0 || p->ch_outer < 0 || p->gate_stride <= 0 || p->ch_stride <= 0 || C >= (1LL << 31))
+        return hyena_fail(HYENA_EINVAL, "%s: bad featurizer channel map", who);
+    const int64_t last = ((D - 1) / p->ch_inner) * p->ch_outer + 2 * p->gate_stride + ((D - 1) % p->ch_inner) * p->ch_stride;
+    if (last >= C) return hyena_fail(HYENA_EINVAL, "%s: featurizer channel map reaches channel %lld of %lld", who,
+                                     (long long)last, (long long)C);
+    out->u = (const bf16_t*)p->u; out->u_bs = p->u_batch_stride; out->ring = (bf16_t*)p->ring;
+    out->Rf = (int)p->Rf; out->pos = (int)p->pos; out->C = (int)C; out->w = p->w; out->bias = p->bias;
+    out->ch_inner = (uint32_t)(p->ch_inner > D ? D : p->ch_inner); out->ch_outer = (uint32_t)p->ch_outer;
+    out->gate_stride = (uint32_t)p->gate_stride; out->ch_stride = (uint32_t)p->ch_stride; out->flip = p->flip_x1x2 != 0;
+    return 0;
+}
+
+// 0: not vectorisable, 1: unit channel stride, 3: interleaved gates
+static int proj_vector_mode(const hyena_proj_step* p, int64_t D) {
+    const bool al = !(((uintptr_t)p->u | (uintptr_t)p->ring | (uintptr_t)p->w | (uintptr_t)p->bias) & 15) &&
+                    p->u_batch_stride % 8 == 0 && D % 8 == 0;
+    if (!al) return 0;
+    if (p->ch_stride == 1 && p->ch_inner % 8 == 0 && p->ch_outer % 8 == 0 && p->gate_stride % 8 == 0) return 1;
+    if (p->ch_stride == 3 && p->gate_stride == 1 && p->ch_inner >= D) return 3;
+    return 0;
+}
+
+static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_t in_bs, const hyena_proj_step* proj,
+                           void* ring, int64_t R, int64_t pos, const float* w, const float* bias, int bias_mode,
+                           void* out, int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream, const char* who) {
+    if ((!proj && !x1) || !ring || !w || !out) return hyena_fail(HYENA_EINVAL, "%s: x1, ring, w, out are required", who);
     if (B < 0 || D <= 0 || G <= 0 || D % G != 0 || R < 1 || R > 4096 || pos < 0 || pos >= R)
-        return hyena_fail(HYENA_EINVAL, "hyena_fir_step: bad sizes B=%lld D=%lld G=%lld R=%lld pos=%lld", (long long)B,
+        return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld G=%lld R=%lld pos=%lld", who, (long long)B,
                           (long long)D, (long long)G, (long long)R, (long long)pos);
     if (bias_mode < 0 || bias_mode > 2 || (bias_mode != HYENA_BIAS_NONE && !bias))
-        return hyena_fail(HYENA_EINVAL, "hyena_fir_step: bias_mode %d needs a bias pointer", bias_mode);
+        return hyena_fail(HYENA_EINVAL, "%s: bias_mode %d needs a bias pointer", who, bias_mode);
     if (D % 8 != 0 || in_bs % 8 != 0 || out_bs % 8 != 0 || ((uintptr_t)x1 & 15) || ((uintptr_t)ring & 15) ||
         ((uintptr_t)out & 15) || (x2 && ((uintptr_t)x2 & 15)) || (v && ((uintptr_t)v & 15)))
-        return hyena_fail(HYENA_EALIGN, "hyena_fir_step: D and strides must be multiples of 8, pointers 16-byte aligned");
-    if (B > 65535) return hyena_fail(HYENA_EINVAL, "hyena_fir_step: B > 65535");
+        return hyena_fail(HYENA_EALIGN, "%s: D and strides must be multiples of 8, pointers 16-byte aligned", who);
+    if (B > 65535) return hyena_fail(HYENA_EINVAL, "%s: B > 65535", who);
+    ProjArgs pj = {};
+    int feat = 0;
+    if (proj) {
+        if (int rc = make_proj(proj, D, who, &pj)) return rc;
+        feat = proj_vector_mode(proj, D);
+        if (!feat) return hyena_fail(HYENA_ENOSUP, "%s: this featurizer channel map / alignment has no fused kernel", who);
+        if (bias_mode == HYENA_BIAS_ADD) return hyena_fail(HYENA_ENOSUP, "%s: fused featurizer with an additive bias", who);
+    }
     if (B == 0) return 0;
     const int dg = (int)(D / G);
     const bool grouped = (dg % 8 == 0) && (512 % dg == 0);
     if (!grouped && G != D)
-        return hyena_fail(HYENA_ENOSUP, "hyena_fir_step: D/G=%d needs per-channel taps (pass G=D)", dg);
-    const bool pre = v != nullptr, post = x2 != nullptr;
+        return hyena_fail(HYENA_ENOSUP, "%s: D/G=%d needs per-channel taps (pass G=D)", who, dg);
+    const bool pre = proj || v != nullptr, post = proj || x2 != nullptr;
     dim3 grid((unsigned)((D + 511) / 512), (unsigned)B);
     const int nsg = R >= 32 ? 8 : 2;
     size_t sh = (size_t)(nsg - 1) * 64 * 8 * sizeof(float) + (grouped ? (size_t)(R + 1) * (512 / dg) * sizeof(float) : 0);
-    if (sh > 160 * 1024) return hyena_fail(HYENA_ENOSUP, "hyena_fir_step: R too large for the LDS tap table");
+    if (sh > 160 * 1024) return hyena_fail(HYENA_ENOSUP, "%s: R too large for the LDS tap table", who);
     hipStream_t s = (hipStream_t)stream;
     const bf16_t *p1 = (const bf16_t*)x1, *p2 = (const bf16_t*)x2, *pv = (const bf16_t*)v;
     bool ok = false;
-#define FS_GO(P, Q, M, GR, N)                                                                                 \
-    hipLaunchKernelGGL((fir_step_kernel<P, Q, M, GR, N>), grid, dim3(64 * N), sh, s, p1, p2, pv, in_bs,       \
+#define FS_GO(P, Q, M, GR, N, F)                                                                              \
+    hipLaunchKernelGGL((fir_step_kernel<P, Q, M, GR, N, F>), grid, dim3(64 * N), sh, s, p1, p2, pv, in_bs, pj, \
                        (bf16_t*)ring, (int)R, (int)pos, w, bias, (bf16_t*)out, out_bs, D, dg)
-#define FS_CASE(P, Q, M)                                                                                      \
-    if (pre == P && post == Q && bias_mode == M) {                                                            \
-        if (grouped && nsg == 8) FS_GO(P, Q, M, true, 8);                                                     \
-        else if (grouped) FS_GO(P, Q, M, true, 2);                                                            \
-        else if (nsg == 8) FS_GO(P, Q, M, false, 8);                                                          \
-        else FS_GO(P, Q, M, false, 2);                                                                        \
+#define FS_CASE(P, Q, M, F)                                                                                   \
+    if (!ok && pre == P && post == Q && bias_mode == M && feat == F) {                                        \
+        if (grouped && nsg == 8) FS_GO(P, Q, M, true, 8, F);                                                  \
+        else if (grouped) FS_GO(P, Q, M, true, 2, F);                                                         \
+        else if (nsg == 8) FS_GO(P, Q, M, false, 8, F);                                                       \
+        else FS_GO(P, Q, M, false, 2, F);                                                                     \
         ok = true;                                                                                            \
     }
-    FS_CASE(true, true, HYENA_BIAS_NONE)
-    FS_CASE(true, true, HYENA_BIAS_GATED_FP32)
-    FS_CASE(false, false, HYENA_BIAS_NONE)
-    FS_CASE(false, false, HYENA_BIAS_ADD)
-    FS_CASE(false, false, HYENA_BIAS_GATED_FP32)
-    FS_CASE(true, true, HYENA_BIAS_ADD)
+    FS_CASE(true, true, HYENA_BIAS_NONE, 0)
+    FS_CASE(true, true, HYENA_BIAS_GATED_FP32, 0)
+    FS_CASE(false, false, HYENA_BIAS_NONE, 0)
+    FS_CASE(false, false, HYENA_BIAS_ADD, 0)
+    FS_CASE(false, false, HYENA_BIAS_GATED_FP32, 0)
+    FS_CASE(true, true, HYENA_BIAS_ADD, 0)
+    FS_CASE(true, true, HYENA_BIAS_NONE, 1)
+    FS_CASE(true, true, HYENA_BIAS_GATED_FP32, 1)
+    FS_CASE(true, true, HYENA_BIAS_NONE, 3)
+    FS_CASE(true, true, HYENA_BIAS_GATED_FP32, 3)
 #undef FS_CASE
 #undef FS_GO
-    if (!ok) return hyena_fail(HYENA_ENOSUP, "hyena_fir_step: this gate/bias combination has no kernel");
-    return hyena_check_launch("hyena_fir_step");
+    if (!ok) return hyena_fail(HYENA_ENOSUP, "%s: this gate/bias combination has no kernel", who);
+    return hyena_check_launch(who);
 }
 
-extern "C" int hyena_iir_step(const void* x1, const void* x2, const void* v, int64_t in_bs, float* state,
-                              const float* poles, const float* residues, int is_complex, const float* Dcoef,
-                              int d_is_bf16, void* out, int out_is_fp32, int64_t out_bs, int64_t B, int64_t D,
-                              int64_t G, int64_t S, void* stream) {
-    if (!x1 || !x2 || !v || !state || !poles || !residues || !Dcoef || !out)
-        return hyena_fail(HYENA_EINVAL, "hyena_iir_step: all pointers are required");
+extern "C" int hyena_fir_step(const void* x1, const void* x2, const void* v, int64_t in_bs, void* ring, int64_t R,
+                              int64_t pos, const float* w, const float* bias, int bias_mode, void* out,
+                              int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream) {
+    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, pos, w, bias, bias_mode, out, out_bs, B, D, G, stream,
+                           "hyena_fir_step");
+}
+
+extern "C" int hyena_fir_layer_step(const hyena_proj_step* proj, void* ring, int64_t R, int64_t pos, const float* w,
+                                    const float* bias, int bias_mode, void* out, int64_t out_bs, int64_t B,
+                                    int64_t D, int64_t G, void* stream) {
+    if (!proj) return hyena_fail(HYENA_EINVAL, "hyena_fir_layer_step: proj is required");
+    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, pos, w, bias, bias_mode, out, out_bs, B, D, G,
+                           stream, "hyena_fir_layer_step");
+}
+
+static int iir_step_launch(const void* x1, const void* x2, const void* v, int64_t in_bs, const hyena_proj_step* proj,
+                           float* state, const float* poles, const float* residues, int is_complex,
+                           const float* Dcoef, int d_is_bf16, void* out, int out_is_fp32, int64_t out_bs, int64_t B,
+                           int64_t D, int64_t G, int64_t S, void* stream, const char* who) {
+    if ((!proj && (!x1 || !x2 || !v)) || !state || !poles || !residues || !Dcoef || !out)
+        return hyena_fail(HYENA_EINVAL, "%s: all pointers are required", who);
     if (B < 0 || D <= 0 || G <= 0 || D % G != 0)
-        return hyena_fail(HYENA_EINVAL, "hyena_iir_step: bad sizes B=%lld D=%lld G=%lld", (long long)B, (long long)D,
+        return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld G=%lld", who, (long long)B, (long long)D,
                           (long long)G);
     if (S != 16 && S != 8 && S != 32)
-        return hyena_fail(HYENA_ENOSUP, "hyena_iir_step: state size %lld (8, 16 or 32 supported)", (long long)S);
+        return hyena_fail(HYENA_ENOSUP, "%s: state size %lld (8, 16 or 32 supported)", who, (long long)S);
     if (((uintptr_t)state & 15) || ((uintptr_t)poles & 15) || ((uintptr_t)residues & 15))
-        return hyena_fail(HYENA_EALIGN, "hyena_iir_step: state, poles, residues must be 16-byte aligned");
+        return hyena_fail(HYENA_EALIGN, "%s: state, poles, residues must be 16-byte aligned", who);
+    ProjArgs pj = {};
+    if (proj) {
+        if (int rc = make_proj(proj, D, who, &pj)) return rc;
+        if (!is_complex && S == 8) return hyena_fail(HYENA_ENOSUP, "%s: fused featurizer with 8 real states", who);
+    }
     if (B == 0) return 0;
     const int dg = (int)(D / G);
     const int lpb = is_complex ? (int)S / 2 : (int)S / 4;
@@ -261,12 +440,32 @@ extern "C" int hyena_iir_step(const void* x1, const void* x2, const void* v, int
     dim3 grid((unsigned)((nthr + 255) / 256));
     hipStream_t s = (hipStream_t)stream;
     const bf16_t *p1 = (const bf16_t*)x1, *p2 = (const bf16_t*)x2, *pv = (const bf16_t*)v;
-#define IIR_CASE(SS, C)                                                                                        \
-    if (S == SS && (is_complex != 0) == C)                                                                      \
-        hipLaunchKernelGGL((iir_step_kernel<SS, C>), grid, dim3(256), 0, s, p1, p2, pv, in_bs, state, poles,    \
-                           residues, Dcoef, d_is_bf16, out, out_is_fp32, out_bs, B, D, dg);
-    IIR_CASE(8, false) IIR_CASE(16, false) IIR_CASE(32, false)
-    IIR_CASE(8, true) IIR_CASE(16, true) IIR_CASE(32, true)
+    const bool feat = proj != nullptr;
+#define IIR_CASE(SS, C, F)                                                                                      \
+    if (S == SS && (is_complex != 0) == C && feat == F)                                                         \
+        hipLaunchKernelGGL((iir_step_kernel<SS, C, F>), grid, dim3(256), 0, s, p1, p2, pv, in_bs, pj, state,    \
+                           poles, residues, Dcoef, d_is_bf16, out, out_is_fp32, out_bs, B, D, dg);
+    IIR_CASE(8, false, false) IIR_CASE(16, false, false) IIR_CASE(32, false, false)
+    IIR_CASE(8, true, false) IIR_CASE(16, true, false) IIR_CASE(32, true, false)
+    IIR_CASE(16, false, true) IIR_CASE(32, false, true)
+    IIR_CASE(8, true, true) IIR_CASE(16, true, true) IIR_CASE(32, true, true)
 #undef IIR_CASE
-    return hyena_check_launch("hyena_iir_step");
+    return hyena_check_launch(who);
+}
+
+extern "C" int hyena_iir_step(const void* x1, const void* x2, const void* v, int64_t in_bs, float* state,
+                              const float* poles, const float* residues, int is_complex, const float* Dcoef,
+                              int d_is_bf16, void* out, int out_is_fp32, int64_t out_bs, int64_t B, int64_t D,
+                              int64_t G, int64_t S, void* stream) {
+    return iir_step_launch(x1, x2, v, in_bs, nullptr, state, poles, residues, is_complex, Dcoef, d_is_bf16, out,
+                           out_is_fp32, out_bs, B, D, G, S, stream, "hyena_iir_step");
+}
+
+extern "C" int hyena_iir_layer_step(const hyena_proj_step* proj, float* state, const float* poles,
+                                    const float* residues, int is_complex, const float* Dcoef, int d_is_bf16,
+                                    void* out, int out_is_fp32, int64_t out_bs, int64_t B, int64_t D, int64_t G,
+                                    int64_t S, void* stream) {
+    if (!proj) return hyena_fail(HYENA_EINVAL, "hyena_iir_layer_step: proj is required");
+    return iir_step_launch(nullptr, nullptr, nullptr, 0, proj, state, poles, residues, is_complex, Dcoef, d_is_bf16,
+                           out, out_is_fp32, out_bs, B, D, G, S, stream, "hyena_iir_layer_step");
 }

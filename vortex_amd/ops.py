@@ -8,7 +8,7 @@ import ctypes
 import torch
 
 from . import _lib
-from ._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE, Rows
+from ._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE, ProjStep, Rows
 
 
 def _stream():
@@ -354,6 +354,63 @@ class IirStepper:
                       torch.cuda.current_stream().cuda_stream)
         if rc:
             _lib.check(rc, "hyena_iir_step")
+        return out
+
+
+def gate_channel_map(hidden, *, interleave=False, head_dim=None):
+    """(ch_inner, ch_outer, gate_stride, ch_stride) of hyena_proj_step for a [.., 3*hidden] projection.
+
+    interleave: vortex/model/utils.py:26-38 then the plain split; head_dim: the head-blocked
+    column_split of utils.py:41-85.  The two together have no closed channel map (returns None).
+    """
+    if interleave and head_dim is not None:
+        return None
+    if interleave:
+        return hidden, 0, 1, 3
+    if head_dim is not None:
+        return head_dim, 3 * head_dim, head_dim, 1
+    return hidden, 0, hidden, 1
+
+
+class LayerStepper:
+    """One launch per Hyena layer and token: featurizer step, split, gates and the inner FIR / IIR step.
+
+    feat_ring: FirRing over the 3D projection channels; feat_w [3D, Rf+1] (oldest tap first), feat_bias [3D] or None.
+    inner: a FirStepper or IirStepper already bound to the layer's inner cache / modal state.
+    """
+
+    def __init__(self, feat_ring, feat_w, feat_bias, channel_map, inner, flip_x1x2=False):
+        _need_cuda(feat_ring.buf, feat_w)
+        self.ring, self.inner = feat_ring, inner
+        self.Rf, C = feat_ring.buf.shape[1], feat_ring.buf.shape[2]
+        self.w = _f32(feat_w).reshape(C, self.Rf + 1).t().contiguous()        # tap-major [Rf+1, C]
+        self.bias = _f32(feat_bias)
+        ci, co, gs, cs = channel_map
+        self.proj = ProjStep(None, 0, feat_ring.buf.data_ptr(), self.Rf, 0, self.w.data_ptr(),
+                             self.bias.data_ptr() if self.bias is not None else None, ci, co, gs, cs, int(flip_x1x2))
+        self._pref = ctypes.byref(self.proj)
+        self.is_fir = isinstance(inner, FirStepper)
+        self._fn = _lib.lib().hyena_fir_layer_step if self.is_fir else _lib.lib().hyena_iir_layer_step
+
+    def __call__(self, u, out):
+        """u: [B, 3D] bf16 with contiguous channels; out: [B, D] bf16 (float32 allowed for the IIR step)."""
+        B = u.shape[0]
+        p, n = self.proj, self.inner
+        p.u, p.u_batch_stride, p.pos = u.data_ptr(), u.stride(0), self.ring.pos
+        stream = torch.cuda.current_stream().cuda_stream
+        if self.is_fir:
+            rc = self._fn(self._pref, n.ring.buf.data_ptr(), n.R, n.ring.pos, n.w.data_ptr(),
+                          n.bias.data_ptr() if n.bias is not None else None, n.mode, out.data_ptr(), out.stride(0),
+                          B, n.D, n.G, stream)
+        else:
+            rc = self._fn(self._pref, n.st.data_ptr(), n.p.data_ptr(), n.r.data_ptr(), int(n.cplx), n.dco.data_ptr(),
+                          n.d_is_bf16, out.data_ptr(), int(out.dtype == torch.float32), out.stride(0), B, n.D, n.G,
+                          n.S, stream)
+        if rc:
+            _lib.check(rc, "hyena_fir_layer_step" if self.is_fir else "hyena_iir_layer_step")
+        self.ring.pos = (self.ring.pos + 1) % self.Rf
+        if self.is_fir:
+            n.ring.pos = (n.ring.pos + 1) % n.R
         return out
 
 
