@@ -195,6 +195,52 @@ int hyena_iir_layer_step(const hyena_proj_step* proj,
                          void* out, int out_is_fp32, int64_t out_batch_stride,
                          int64_t B, int64_t D, int64_t G, int64_t S, void* stream);
 
+/* Channel-last operand [B][L][D]: element (b, t, d) at ptr + b*batch_stride + t*time_stride + d (elements).
+ * This is the (batch, seqlen, groups, group_dim) layout of vortex/ops/hyena_se/fwd.py:17-43 with D = groups*group_dim. */
+typedef struct hyena_cl {
+    const void* ptr;
+    int64_t batch_stride;
+    int64_t time_stride;
+} hyena_cl;
+
+/* Gated causal FIR (1 <= K <= 128) on channel-last tensors, block-Toeplitz MFMA contraction.
+ * Replaces two_pass_fwd_grouped (vortex/ops/hyena_se/fwd.py:17-290; kernels fwd_kernels.py:631-794) and the
+ * layout handling of inner_hyena_se_ref (vortex/ops/hyena_se/interface.py:272-397):
+ *   bx = bf16(x1*v);  y2[t] = bias rule( sum_k h[g][k]*bx[t-k] );  out = bf16(x2*y2)
+ * (x1 = B, v = x, x2 = C in the reference's naming; v == x2 == NULL gives the ungated FIR.)
+ * h: [G][K] float32, h[g][0] on the current sample unless taps_reversed.  D/G % 16 == 0, D % 8 == 0.
+ * out: [B][L][D] bf16 contiguous.  Optional outputs, the intermediates fwd.py:23-25 can return:
+ *   y2_out [B][L][D]: the convolution before the x2 gate;
+ *   bx_out [B][L-bx_from][D]: rows t >= bx_from of bx (bx_from = 0: all of it; bx_from = L-(K-1): the FIR
+ *   cache a decode step continues from, vortex/model/engine.py:255-258). */
+int hyena_fir_cl_fwd(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v,
+                     const float* h, int taps_reversed, const float* bias, int bias_mode,
+                     void* out, void* y2_out, void* bx_out, int64_t bx_from,
+                     int64_t B, int64_t L, int64_t D, int64_t G, int K, void* stream);
+
+/* The featurizer of a Hyena layer at prefill (vortex/model/model.py:233-252: short FIR over the 3D channels
+ * of the dense projection, then interleave / split), described so that hyena_fir_layer_fwd can evaluate it on
+ * the fly:  z[t][c] = bf16( sum_k w[k][c]*u[t-(Ks-1)+k][c] )  (then + bias[c], rounded again).
+ * Gate i (0: x2, 1: x1, 2: v) of operator channel d is z at channel
+ *   (d / ch_inner)*ch_outer + i*gate_stride + (d % ch_inner)*ch_stride      (maps as in hyena_proj_step). */
+typedef struct hyena_proj_fwd {
+    const void* u;              /* [B][L][3D] bf16, channels contiguous */
+    int64_t u_batch_stride, u_time_stride;
+    const float* w;             /* [Ks][3D] float32, tap-major, w[Ks-1] on the current sample */
+    const float* bias;          /* [3D] float32 or NULL */
+    int Ks;                     /* 3 or 4 */
+    int flip_x1x2;
+    int64_t ch_inner, ch_outer, gate_stride, ch_stride;
+} hyena_proj_fwd;
+
+/* A whole Hyena-SE / Hyena-MR layer at prefill in one launch: featurizer FIR, split, x1*v gate, inner FIR,
+ * bias rule (NONE or GATED_FP32), x2 gate; u [B][L][3D] in, out [B][L][D], nothing in between touches device
+ * memory.  Replaces the two parallel_fir calls of vortex/model/model.py:233-291.  bx_out / bx_from as above. */
+int hyena_fir_layer_fwd(const hyena_proj_fwd* proj,
+                        const float* h, int taps_reversed, const float* bias, int bias_mode,
+                        void* out, void* bx_out, int64_t bx_from,
+                        int64_t B, int64_t L, int64_t D, int64_t G, int K, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,153 @@
+"""GPU parity of the channel-last FIR kernel (hyena_fir_cl_fwd) and the one-launch prefill layer
+(hyena_fir_layer_fwd) against the CPU oracle, through the C ABI."""
+import os
+
+import pytest
+import torch
+
+from vortex_amd import ops
+from vortex_amd._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE
+from oracle import hyena_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def rel_err(a, b):
+    a, b = a.double().cpu(), b.double().cpu()
+    return ((a - b).abs().max() / b.abs().max().clamp_min(1e-30)).item()
+
+
+def cl(t):
+    """[B, D, L] -> channel-last [B, L, D] contiguous on the GPU."""
+    return t.permute(0, 2, 1).contiguous().to(DEV)
+
+
+@pytest.fixture
+def segments(request):
+    """Forces a number of segments along L so that short sequences exercise the halo rebuild."""
+    old = os.environ.get("HYENA_CL_NSEG")
+    os.environ["HYENA_CL_NSEG"] = str(request.param)
+    yield request.param
+    if old is None:
+        del os.environ["HYENA_CL_NSEG"]
+    else:
+        os.environ["HYENA_CL_NSEG"] = old
+
+
+@pytest.mark.parametrize("segments", [1, 3], indirect=True)
+@pytest.mark.parametrize("B,D,G,L,K", [
+    (2, 64, 4, 512, 7), (1, 80, 5, 1000, 7), (2, 128, 8, 131, 4), (1, 64, 2, 8, 7), (1, 192, 12, 777, 2),
+])
+def test_cl_short_filter_vs_oracle(B, D, G, L, K, segments):
+    x2, x1, v = O.make_gates(B, D, L, seed=L + K)
+    h = O.make_se_filter(G, K, seed=K)
+    ref = O.se_fir(x2, x1, v, h)
+    ref = ref[0] if isinstance(ref, tuple) else ref
+    y = ops.fir_cl_fwd(cl(x1), cl(x2), cl(v), h.reshape(G, K).to(DEV), taps_reversed=True)
+    assert y.shape == (B, L, D)
+    assert rel_err(y.permute(0, 2, 1), ref) <= 2e-2
+
+
+@pytest.mark.parametrize("segments", [1, 2], indirect=True)
+@pytest.mark.parametrize("B,D,G,L,K", [(2, 64, 4, 640, 128), (1, 96, 6, 1333, 128), (1, 64, 1, 300, 100),
+                                       (1, 32, 2, 64, 128)])
+def test_cl_medium_filter_gated_bias_vs_oracle(B, D, G, L, K, segments):
+    x2, x1, v = O.make_gates(B, D, L, seed=L)
+    h = O.make_mr_filter(G, K, seed=K)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(5))
+    ref, _ = O.mr_fir(x2, x1, v, h, Db)
+    y = ops.fir_cl_fwd(cl(x1), cl(x2), cl(v), h.reshape(G, K).to(DEV), bias=Db.to(DEV),
+                       bias_mode=HYENA_BIAS_GATED_FP32)
+    assert rel_err(y.permute(0, 2, 1), ref) <= 2e-2
+
+
+def test_cl_strided_views_and_intermediates():
+    # gates as slices of one [B, L, 3D] projection (time stride 3D); y2 and bx as two_pass_fwd_grouped returns them
+    B, D, G, L, K = 2, 128, 8, 515, 33
+    g = torch.Generator().manual_seed(9)
+    u = torch.randn(B, L, 3 * D, generator=g).bfloat16()
+    h = torch.randn(G, 1, K, generator=g) / K ** 0.5
+    ud = u.to(DEV)
+    x2, x1, v = (ud[..., i * D:(i + 1) * D] for i in range(3))
+    out, y2, bx = ops.fir_cl_fwd(x1, x2, v, h.reshape(G, K).to(DEV), want_y2=True, want_bx=True, bx_from=L - (K - 1))
+    x2c, x1c, vc = (u[..., i * D:(i + 1) * D].permute(0, 2, 1) for i in range(3))
+    bx_ref = x1c * vc
+    w = h.repeat_interleave(D // G, 0)
+    z_ref = O.short_fir_fp32(bx_ref, w.flip(-1), K).bfloat16()          # convolution = correlation with flipped taps
+    assert rel_err(y2.permute(0, 2, 1), z_ref) <= 2e-2
+    assert rel_err(out.permute(0, 2, 1), x2c * z_ref) <= 2e-2
+    assert torch.equal(bx.cpu(), bx_ref[..., L - (K - 1):].permute(0, 2, 1))
+
+
+@pytest.mark.parametrize("bias_mode", [HYENA_BIAS_NONE, HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32])
+def test_cl_ungated_fir_bias_rules(bias_mode):
+    B, D, G, L, K = 1, 64, 64 // 16, 400, 5
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(B, D, L, generator=g).bfloat16()
+    h = torch.randn(G, 1, K, generator=g) / K ** 0.5
+    bias = torch.randn(D, generator=g)
+    w = h.repeat_interleave(D // G, 0)
+    conv = O.short_fir_fp32(x, w, K)
+    if bias_mode == HYENA_BIAS_NONE:
+        ref = conv.bfloat16()
+    elif bias_mode == HYENA_BIAS_ADD:
+        ref = (conv.bfloat16() + bias.bfloat16()[None, :, None])
+    else:
+        ref = (conv + bias[None, :, None] * x.float()).bfloat16()
+    y = ops.fir_cl_fwd(cl(x), None, None, h.reshape(G, K).to(DEV), bias=bias.to(DEV) if bias_mode else None,
+                       bias_mode=bias_mode, taps_reversed=True)
+    assert rel_err(y.permute(0, 2, 1), ref) <= 2e-2
+
+
+def oracle_layer(u, wf, bf, h, Dcoef, D, H, cs, il, flip):
+    """Featurizer -> interleave -> split -> inner FIR of vortex/model/model.py:221-291 on u [B, L, 3D]."""
+    Ks, K = wf.shape[-1], h.shape[-1]
+    z, _ = O.parallel_fir(u, wf, bf, fir_length=Ks, dim_last=True, gate=False)
+    if il:
+        z = O.interleave(z)
+    x2, x1, v = O.split_gates(z, (D, H, D // H, 16, h.shape[0]), cs, flip)
+    if K >= 128:
+        y, tail = O.mr_fir(x2, x1, v, h, Dcoef)
+    else:
+        y = O.se_fir(x2, x1, v, h)
+        y = y[0] if isinstance(y, tuple) else y
+        tail = (x1 * v)[..., -(K - 1):]
+    return y, tail
+
+
+@pytest.mark.parametrize("segments", [1, 2], indirect=True)
+@pytest.mark.parametrize("B,L,D,H,G,K,Ks,cs,il,flip,sbias", [
+    (2, 512, 64, 4, 4, 7, 3, False, True, False, False),       # Evo 2 layout, Hyena-SE
+    (1, 700, 128, 4, 8, 128, 3, False, True, False, False),    # Evo 2 layout, Hyena-MR
+    (1, 384, 64, 4, 4, 7, 3, True, False, False, True),        # head-blocked split (head_dim 16), featurizer bias
+    (2, 300, 96, 2, 6, 128, 3, False, False, True, False),     # plain split, flipped gates, D % 64 != 0
+    (1, 520, 64, 2, 4, 7, 4, False, True, False, True),        # 4-tap featurizer
+    (1, 260, 64, 2, 4, 128, 4, True, False, True, False),
+])
+def test_layer_fwd_vs_oracle(B, L, D, H, G, K, Ks, cs, il, flip, sbias, segments):
+    g = torch.Generator().manual_seed(L + K + Ks)
+    C = 3 * D
+    u = torch.randn(B, L, C, generator=g).bfloat16()
+    wf = torch.randn(C, 1, Ks, generator=g) / Ks ** 0.5
+    bf = torch.randn(C, generator=g).bfloat16() if sbias else None
+    mr = K >= 128
+    h = O.make_mr_filter(G, K, seed=3) if mr else O.make_se_filter(G, K, seed=3)
+    Dcoef = torch.randn(D, generator=g) if mr else None
+    ref, tail = oracle_layer(u, wf, bf, h, Dcoef, D, H, cs, il, flip)
+    cmap = ops.gate_channel_map(D, interleave=il, head_dim=D // H if cs else None)
+    y, bx = ops.fir_layer_fwd(u.to(DEV), wf.reshape(C, Ks).t().contiguous().to(DEV), None if bf is None else bf.to(DEV),
+                              cmap, h.reshape(G, K).to(DEV), bias=None if Dcoef is None else Dcoef.to(DEV),
+                              bias_mode=HYENA_BIAS_GATED_FP32 if mr else HYENA_BIAS_NONE, taps_reversed=not mr,
+                              flip_x1x2=flip, bx_from=L - (K - 1))
+    assert y.shape == (B, L, D)
+    assert rel_err(y.permute(0, 2, 1), ref) <= 2e-2
+    assert rel_err(bx.permute(0, 2, 1), tail) <= 1e-2
+
+
+def test_cl_rejects_unsupported():
+    x = torch.zeros(1, 16, 24, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(NotImplementedError):       # 24 channels in 3 groups: group size 8 is not a multiple of 16
+        ops.fir_cl_fwd(x, x, x, torch.zeros(3, 4, device=DEV))
+    with pytest.raises(NotImplementedError):
+        ops.fir_cl_fwd(torch.zeros(1, 16, 32, dtype=torch.bfloat16, device=DEV), None, None, torch.zeros(2, 200, device=DEV))

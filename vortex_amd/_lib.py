@@ -14,7 +14,7 @@ HYENA_BIAS_NONE, HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32 = 0, 1, 2
 EXPORTS = [
     "hyena_version", "hyena_last_error_string", "hyena_se_fwd", "hyena_mr_fwd",
     "hyena_fir_step", "hyena_iir_step", "hyena_li_plan_bytes", "hyena_li_plan", "hyena_li_fwd", "hyena_featurizer_fwd", "hyena_copy_probe",
-    "hyena_fir_layer_step", "hyena_iir_layer_step",
+    "hyena_fir_layer_step", "hyena_iir_layer_step", "hyena_fir_cl_fwd", "hyena_fir_layer_fwd",
 ]
 
 
@@ -28,6 +28,18 @@ class ProjStep(Structure):
     _fields_ = [("u", c_void_p), ("u_batch_stride", c_int64), ("ring", c_void_p), ("Rf", c_int64), ("pos", c_int64),
                 ("w", c_void_p), ("bias", c_void_p), ("ch_inner", c_int64), ("ch_outer", c_int64),
                 ("gate_stride", c_int64), ("ch_stride", c_int64), ("flip_x1x2", c_int)]
+
+
+class Cl(Structure):
+    """hyena_cl: a channel-last [B, L, D] operand."""
+    _fields_ = [("ptr", c_void_p), ("batch_stride", c_int64), ("time_stride", c_int64)]
+
+
+class ProjFwd(Structure):
+    """hyena_proj_fwd: the featurizer a fused prefill layer evaluates on the fly."""
+    _fields_ = [("u", c_void_p), ("u_batch_stride", c_int64), ("u_time_stride", c_int64), ("w", c_void_p),
+                ("bias", c_void_p), ("Ks", c_int), ("flip_x1x2", c_int), ("ch_inner", c_int64), ("ch_outer", c_int64),
+                ("gate_stride", c_int64), ("ch_stride", c_int64)]
 
 
 _lib = None
@@ -66,6 +78,11 @@ def lib():
                                        c_int64, c_int64, c_int64, c_void_p]
     L.hyena_iir_layer_step.argtypes = [P, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                                        c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p]
+    C = POINTER(Cl)
+    L.hyena_fir_cl_fwd.argtypes = [C, C, C, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64,
+                                   c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]
+    L.hyena_fir_layer_fwd.argtypes = [POINTER(ProjFwd), c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int64,
+                                      c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]
     for name in EXPORTS:
         fn = getattr(L, name)
         if name not in ("hyena_version", "hyena_last_error_string"):

@@ -10,7 +10,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libhyena_mi355x.so")
-SOURCES = ["api.hip", "se_fir.hip", "mr_fir.hip", "li_modal.hip", "decode.hip", "featurizer.hip"]
+SOURCES = ["api.hip", "se_fir.hip", "mr_fir.hip", "li_modal.hip", "decode.hip", "featurizer.hip", "fir_cl.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

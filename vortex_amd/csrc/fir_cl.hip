@@ -1,0 +1,491 @@
+// Channel-last gated FIR (2 <= K <= 128): the Hyena-SE / Hyena-MR operator on
+// [B][L][D] tensors, the (batch, seqlen, groups, group_dim) layout of
+// vortex/ops/hyena_se/fwd.py:17-43, and, with the featurizer fused in, a whole
+// Hyena-SE / MR layer from the dense projection u [B][L][3D] to y [B][L][D]
+// (vortex/model/model.py:221-291) with no intermediate in device memory.
+//
+// Same block-Toeplitz MFMA contraction as mr_fir.hip (ten 32x16 Toeplitz blocks
+// per filter group held in registers, u = bf16(x1*v) streamed through the B
+// operand), but the block is 64 channels x 128 samples per step so that every
+// global access is a full 128-byte line of one time row:
+//   global rows (16 B/lane = 8 channels, 4 rows per lane) [-> featurizer FIR in registers]
+//   -> u = bf16(x1*v) -> 4x8 register transpose -> LDS [64 ch][256-sample ring]
+//   -> B fragments (ds_read_b128) -> MFMA -> z = bf16(acc [+ D*u]) -> LDS [64][128]
+//   -> 8x4 register transpose -> * x2 -> global rows.
+// Wavefront w of a block contracts channels 16w..16w+15 (one filter group per wavefront).
+// The LDS input tile is a two-chunk ring: the chunk written in one step is the
+// 128-sample halo of the next, so nothing is copied between steps.
+#include "common.h"
+
+namespace {
+
+constexpr int TL = 128;        // samples per step (= halo length)
+constexpr int CB = 64;         // channels per block
+constexpr int URS = 264;       // u_lds row stride (elements): 528 B = 16 * 33
+constexpr int ZRS = 136;       // z_lds row stride (elements): 272 B = 16 * 17
+
+struct ClMap {                 // channel-last operand: (b, t, d) at ptr + b*bs + t*ts + d
+    const bf16_t* ptr;
+    int64_t bs, ts;
+};
+
+struct ProjFwd {               // device copy of hyena_proj_fwd
+    const bf16_t* u;
+    int64_t bs, ts;
+    const float* w;            // [KS][3D], tap-major, oldest tap first
+    const float* bias;         // [3D] or null
+    uint32_t ch_inner, ch_outer, gate_stride;
+    int flip;
+    __device__ __forceinline__ uint32_t chan(uint32_t gate, uint32_t d) const {
+        return (d / ch_inner) * ch_outer + gate * gate_stride + (d % ch_inner);
+    }
+};
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) {
+    union { u32x4 u; bf16x8 b; } c;
+    c.u = x;
+    return c.b;
+}
+
+// 16-bit halves of two dwords: (lo(a), lo(b)) or (hi(a), hi(b)) packed as (first, second)
+__device__ __forceinline__ uint32_t pair_lo(uint32_t first, uint32_t second) {
+    return __builtin_amdgcn_perm(second, first, 0x05040100u);
+}
+__device__ __forceinline__ uint32_t pair_hi(uint32_t first, uint32_t second) {
+    return __builtin_amdgcn_perm(second, first, 0x07060302u);
+}
+
+// element e (0..7) of a packed row of 8 bf16, as float
+__device__ __forceinline__ float el(const u32x4& r, int e) { return (e & 1) ? bf_hi(r[e >> 1]) : bf_lo(r[e >> 1]); }
+
+// FEAT: 0 = gates given as three channel-last tensors; 1 = gates from the fused featurizer, unit channel
+// stride (plain or head-blocked split); 3 = fused featurizer with interleaved gates (channel 3d+i).
+// KS = featurizer taps (FEAT != 0).  AUX = also store y2 (z before the x2 gate) and / or bx = bf16(x1*v).
+template <bool PRE, bool POST, int BIAS, int FEAT, int KS, bool AUX>
+__global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMap v, ProjFwd pj,
+                                                        const float* __restrict__ h, int K, int reversed,
+                                                        const float* __restrict__ bias, bf16_t* __restrict__ out,
+                                                        bf16_t* __restrict__ y2_out, bf16_t* __restrict__ bx_out,
+                                                        int64_t bx_from, int64_t L, int64_t D, int dg,
+                                                        int64_t seg_len, int nseg, int ndb) {
+    constexpr int RF = FEAT ? KS - 1 : 0;          // extra rows a lane reads before its own four
+    constexpr int NR = 4 + RF;                     // rows per lane and load piece
+    constexpr int NP = (FEAT || (PRE && POST)) ? 3 : (PRE ? 2 : 1);   // load pieces per row
+    __shared__ __attribute__((aligned(16))) bf16_t u_lds[CB * URS];
+    __shared__ __attribute__((aligned(16))) bf16_t z_lds[CB * ZRS];
+    __shared__ __attribute__((aligned(16))) float w_lds[FEAT ? (KS + 1) * 3 * CB : 4];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t bid = blockIdx.x;
+    const int seg = (int)(bid % (uint32_t)nseg);
+    const uint32_t db = (bid / (uint32_t)nseg) % (uint32_t)ndb;
+    const int64_t b = bid / ((uint32_t)nseg * (uint32_t)ndb);
+    const uint32_t d0 = db * CB;
+
+    // ---- Toeplitz fragments of this wavefront's filter group (see mr_fir.hip for the index algebra)
+    const int n = lane & 31, hh = lane >> 5;
+    const bool slab_live = d0 + 16 * w < (uint32_t)D;
+    const int g = slab_live ? (int)((d0 + 16 * w) / (uint32_t)dg) : 0;
+    const int i_time = 16 * ((n >> 2) & 1) + 4 * (n >> 3) + (n & 3);
+    bf16x8 A[10];
+    const int m_min = (114 - K) > 0 ? (114 - K + 15) / 16 : 0;      // blocks below m_min are all zero
+#pragma unroll
+    for (int m = 0; m < 10; ++m) {
+        u32x4 pk;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float t[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int lag = i_time - (8 * hh + 2 * j + e) + 128 - 16 * m;
+                float val = 0.f;
+                if (lag >= 0 && lag < K) val = h[g * K + (reversed ? K - 1 - lag : lag)];
+                t[e] = val;
+            }
+            pk[j] = pack_bf2(t[0], t[1]);
+        }
+        A[m] = as_bf16x8(pk);
+    }
+
+    // ---- this lane's I/O block: rows 4*rb .. 4*rb+3 of the step, channels d0 + 8*cb .. +7
+    const int cb = tid & 7, rb = tid >> 3;
+    const uint32_t dch = d0 + 8 * cb;
+    const bool ch_ok = dch < (uint32_t)D;
+    const bf16_t* pp[NP];
+    int64_t pts;
+    if (FEAT == 3) {
+#pragma unroll
+        for (int i = 0; i < NP; ++i) pp[i] = pj.u + b * pj.bs + 3 * (int64_t)dch + 8 * i;
+        pts = pj.ts;
+    } else if (FEAT == 1) {
+#pragma unroll
+        for (int i = 0; i < NP; ++i) pp[i] = pj.u + b * pj.bs + pj.chan(i, ch_ok ? dch : 0);
+        pts = pj.ts;
+    } else {
+        pp[0] = x1.ptr + b * x1.bs + dch;
+        if (NP >= 2) pp[1] = v.ptr + b * v.bs + dch;
+        if (NP >= 3) pp[2] = x2.ptr + b * x2.bs + dch;
+        pts = 0;
+    }
+    const int64_t pstr[3] = {FEAT ? pts : x1.ts, FEAT ? pts : v.ts, FEAT ? pts : x2.ts};
+
+    // featurizer taps / bias of this block's channels, in the lane-piece order the loads use
+    if (FEAT) {
+        for (int e = tid; e < (KS + 1) * 3 * CB; e += 256) {
+            const int k = e / (3 * CB), r = e - k * 3 * CB, i = r / CB, dl = r - i * CB;   // piece i, local channel dl
+            const uint32_t dd = d0 + dl;
+            float val = 0.f;
+            if (dd < (uint32_t)D) {
+                const uint32_t ch = FEAT == 3 ? 3 * (d0 + (dl & ~7)) + 8 * i + (dl & 7) : pj.chan(i, dd);
+                if (k < KS) val = pj.w[(int64_t)k * 3 * D + ch];
+                else if (pj.bias) val = pj.bias[ch];
+            }
+            w_lds[e] = val;
+        }
+    }
+
+    const int64_t t_begin = (int64_t)seg * seg_len;
+    const int64_t t_end = (t_begin + seg_len < L) ? t_begin + seg_len : L;
+    if (t_begin >= t_end) return;
+    const int64_t ts0 = t_begin > 0 ? t_begin - TL : 0;      // one extra step rebuilds the halo of a later segment
+
+    // zero halo at the sequence start
+    if (t_begin == 0) {
+        const u32x4 zero4 = {0, 0, 0, 0};
+        for (int e = tid; e < CB * (TL / 8); e += 256)
+            *(u32x4*)(u_lds + (e >> 4) * URS + TL + (e & 15) * 8) = zero4;
+    }
+    __syncthreads();           // featurizer table and zeroed halo visible to every wavefront
+
+    u32x4 raw[NP][NR];
+    const u32x4 zero4 = {0, 0, 0, 0};
+    auto load_step = [&](int64_t ts) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int64_t t = ts + 4 * rb + r - RF;
+            const bool ok = ch_ok && t >= 0 && t < t_end;
+#pragma unroll
+            for (int i = 0; i < NP; ++i) raw[i][r] = ok ? *(const u32x4*)(pp[i] + t * pstr[i]) : zero4;
+        }
+    };
+    load_step(ts0);
+
+    float bz = 0.f;
+    if (BIAS != HYENA_BIAS_NONE && slab_live) bz = bias[d0 + 16 * w + (n & 15)];
+
+    int cur = 0;                       // ring chunk the current step writes; the other one is its halo
+    for (int64_t ts = ts0; ts < t_end; ts += TL) {
+        const bool compute = ts >= t_begin;
+        // ---- (a) gates of this lane's 4 x 8 block
+        u32x4 bx[4], g2[4];
+        if (FEAT) {
+            u32x4 zq[3][4];
+            int woff = 8 * cb;
+            asm volatile("" : "+v"(woff));      // re-read the tap table every step instead of pinning 96 registers
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                float tw[KS][8], bb[8];
+#pragma unroll
+                for (int k = 0; k <= KS; ++k) {
+                    const f32x4 t0 = *(const f32x4*)(w_lds + (k * 3 + i) * CB + woff);
+                    const f32x4 t1 = *(const f32x4*)(w_lds + (k * 3 + i) * CB + woff + 4);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (k < KS) { tw[k][j] = t0[j]; tw[k][4 + j] = t1[j]; }
+                        else { bb[j] = t0[j]; bb[4 + j] = t1[j]; }
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float acc[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+#pragma unroll
+                    for (int k = 0; k < KS; ++k) {
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) acc[j] = fmaf(tw[k][j], el(raw[i][q + k], j), acc[j]);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) zq[i][q][j] = pack_bf2(acc[2 * j], acc[2 * j + 1]);
+                }
+                if (pj.bias) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            zq[i][q][j] = pack_bf2(bf_lo(zq[i][q][j]) + bb[2 * j], bf_hi(zq[i][q][j]) + bb[2 * j + 1]);
+                }
+                __builtin_amdgcn_sched_barrier(0);      // one piece at a time: its rows are dead before the next starts
+            }
+            // rows past the end of the sequence hold bias-only values; they are never stored and never feed a
+            // valid output (causality), so they need no masking.  Rows before t = 0 do not exist (ts0 >= 0).
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float a1[2], a2[2], av[2];
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        const int jd = 2 * j + e;
+                        if (FEAT == 3) {        // channel 3*jd + gate of the lane's 24
+                            const int e0 = 3 * jd, e1 = 3 * jd + 1, e2 = 3 * jd + 2;
+                            a2[e] = el(zq[e0 >> 3][q], e0 & 7);
+                            a1[e] = el(zq[e1 >> 3][q], e1 & 7);
+                            av[e] = el(zq[e2 >> 3][q], e2 & 7);
+                        } else {
+                            a2[e] = el(zq[0][q], jd);
+                            a1[e] = el(zq[1][q], jd);
+                            av[e] = el(zq[2][q], jd);
+                        }
+                        if (pj.flip) { const float t = a1[e]; a1[e] = a2[e]; a2[e] = t; }
+                    }
+                    bx[q][j] = pack_bf2(a1[0] * av[0], a1[1] * av[1]);
+                    g2[q][j] = pack_bf2(a2[0], a2[1]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (PRE) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        bx[q][j] = pack_bf2(bf_lo(raw[0][q][j]) * bf_lo(raw[1][q][j]),
+                                            bf_hi(raw[0][q][j]) * bf_hi(raw[1][q][j]));
+                } else {
+                    bx[q] = raw[0][q];
+                }
+                if (POST) g2[q] = raw[NP - 1][q];
+            }
+        }
+        // ---- (b) next step's rows are requested now and arrive during the MFMA phase
+        // With the featurizer fused in, a lane holds 18 row pieces; keeping them in flight across the MFMA phase
+        // does not fit the register budget of two blocks per CU, so they are requested after it instead.
+        __builtin_amdgcn_sched_barrier(0);
+        if (!FEAT && ts + TL < t_end) load_step(ts + TL);
+
+        // ---- (c) 4 x 8 transpose into the ring chunk `cur`
+        {
+            bf16_t* ub = u_lds + (8 * cb) * URS + cur * TL + 4 * rb;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                u32x2 t2;
+                if (c & 1) { t2[0] = pair_hi(bx[0][c >> 1], bx[1][c >> 1]); t2[1] = pair_hi(bx[2][c >> 1], bx[3][c >> 1]); }
+                else       { t2[0] = pair_lo(bx[0][c >> 1], bx[1][c >> 1]); t2[1] = pair_lo(bx[2][c >> 1], bx[3][c >> 1]); }
+                *(u32x2*)(ub + c * URS) = t2;
+            }
+        }
+        if (AUX && bx_out && compute && ch_ok) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int64_t t = ts + 4 * rb + q;
+                if (t < t_end && t >= bx_from) *(u32x4*)(bx_out + (b * (L - bx_from) + (t - bx_from)) * D + dch) = bx[q];
+            }
+        }
+        __syncthreads();
+
+        if (compute && slab_live) {
+            // ---- MFMA phase: this wavefront's 16 channels x 128 samples
+            const int c = n & 15, s = n >> 4;
+            f32x16 acc0, acc1;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
+            const bf16_t* urow = u_lds + (16 * w + c) * URS;
+            const int c0 = 64 * s + 8 * hh + (cur ^ 1) * TL;     // ring position of the halo chunk's first sample
+#pragma unroll
+            for (int mm = 0; mm < 12; ++mm) {
+                const bf16x8 bf = *(const bf16x8*)(urow + ((c0 + 16 * mm) & (2 * TL - 1)));
+                if (mm <= 9 && mm >= m_min) acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm <= 9 ? mm : 0], bf, acc0, 0, 0, 0);
+                if (mm >= 2 && mm - 2 >= m_min) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm >= 2 ? mm - 2 : 0], bf, acc1, 0, 0, 0);
+                if ((mm & 3) == 3) __builtin_amdgcn_sched_barrier(0);    // at most four B fragments in registers at a time
+            }
+#pragma unroll
+            for (int tau = 0; tau < 2; ++tau) {
+                const int tcol = 32 * tau + 64 * s + 16 * hh;
+                const f32x16 acc = tau ? acc1 : acc0;
+                u32x4 ua = {0, 0, 0, 0}, ub2 = {0, 0, 0, 0};
+                if (BIAS == HYENA_BIAS_GATED_FP32) {
+                    ua = *(const u32x4*)(urow + cur * TL + tcol);
+                    ub2 = *(const u32x4*)(urow + cur * TL + tcol + 8);
+                }
+                u32x4 z0, z1;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    float a0 = acc[2 * j], a1 = acc[2 * j + 1];
+                    if (BIAS == HYENA_BIAS_GATED_FP32) {
+                        const uint32_t uw = j < 4 ? ua[j] : ub2[j - 4];
+                        a0 = fmaf(bz, bf_lo(uw), a0);
+                        a1 = fmaf(bz, bf_hi(uw), a1);
+                    }
+                    if (BIAS == HYENA_BIAS_ADD) {
+                        a0 = round_bf(a0) + bz;
+                        a1 = round_bf(a1) + bz;
+                    }
+                    const uint32_t p = pack_bf2(a0, a1);
+                    if (j < 4) z0[j] = p; else z1[j - 4] = p;
+                }
+                *(u32x4*)(z_lds + (16 * w + c) * ZRS + tcol) = z0;
+                *(u32x4*)(z_lds + (16 * w + c) * ZRS + tcol + 8) = z1;
+            }
+        }
+        __syncthreads();
+        if (FEAT) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (ts + TL < t_end) load_step(ts + TL);
+        }
+
+        // ---- 8 x 4 transpose back, gate with x2, store rows
+        if (compute && ch_ok) {
+            u32x2 zc[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) zc[c] = *(const u32x2*)(z_lds + (8 * cb + c) * ZRS + 4 * rb);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int64_t t = ts + 4 * rb + q;
+                u32x4 zz;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    zz[j] = (q & 1) ? pair_hi(zc[2 * j][q >> 1], zc[2 * j + 1][q >> 1])
+                                    : pair_lo(zc[2 * j][q >> 1], zc[2 * j + 1][q >> 1]);
+                if (t < t_end) {
+                    if (AUX && y2_out) *(u32x4*)(y2_out + (b * L + t) * D + dch) = zz;
+                    u32x4 o = zz;
+                    if (POST) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(g2[q][j]), bf_hi(zz[j]) * bf_hi(g2[q][j]));
+                    }
+                    *(u32x4*)(out + (b * L + t) * D + dch) = o;
+                }
+            }
+        }
+        cur ^= 1;
+    }
+}
+
+struct LaunchArgs {
+    ClMap x1, x2, v;
+    ProjFwd pj;
+    int feat, ks;
+    bool pre, post;
+};
+
+static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed, const float* bias, int bias_mode,
+                         void* out, void* y2_out, void* bx_out, int64_t bx_from, int64_t B, int64_t L, int64_t D,
+                         int64_t G, int K, void* stream, const char* who) {
+    if (!h || !out) return hyena_fail(HYENA_EINVAL, "%s: h and out are required", who);
+    if (B < 0 || D <= 0 || L < 0 || G <= 0 || D % G != 0 || D >= (1LL << 30))
+        return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld L=%lld G=%lld", who, (long long)B, (long long)D,
+                          (long long)L, (long long)G);
+    if (K < 1 || K > 128) return hyena_fail(HYENA_ENOSUP, "%s: K=%d outside 1..128", who, K);
+    if ((D / G) % 16 != 0)
+        return hyena_fail(HYENA_ENOSUP, "%s: D/G=%lld must be a multiple of 16", who, (long long)(D / G));
+    if (bias_mode < 0 || bias_mode > 2 || (bias_mode != HYENA_BIAS_NONE && !bias))
+        return hyena_fail(HYENA_EINVAL, "%s: bias_mode %d needs a bias pointer", who, bias_mode);
+    if (bx_out && (bx_from < 0 || bx_from > L)) return hyena_fail(HYENA_EINVAL, "%s: bx_from outside 0..L", who);
+    if ((((uintptr_t)out | (uintptr_t)y2_out | (uintptr_t)bx_out) & 15))
+        return hyena_fail(HYENA_EALIGN, "%s: outputs must be 16-byte aligned", who);
+    if (B == 0 || L == 0) return 0;
+
+    // segments along L: enough blocks for several rounds over 256 CUs, segments of at least 1024 samples
+    const int64_t ndb = (D + CB - 1) / CB;
+    const int64_t rows = B * ndb;
+    int64_t nseg = (2048 + rows - 1) / rows;
+    const int64_t max_seg = (L + 1023) / 1024;
+    if (nseg > max_seg) nseg = max_seg;
+    if (nseg < 1) nseg = 1;
+    if (const char* e = getenv("HYENA_CL_NSEG")) { int64_t x = atoll(e); if (x >= 1) nseg = x; }
+    int64_t seg_len = (L + nseg - 1) / nseg;
+    seg_len = (seg_len + TL - 1) / TL * TL;
+    nseg = (L + seg_len - 1) / seg_len;
+    const int64_t nblk = rows * nseg;
+    if (nblk > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: problem too large for one launch", who);
+
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((unsigned)nblk);
+    const int dg = (int)(D / G);
+    const bool aux = y2_out || bx_out;
+    bool ok = false;
+#define CL_GO(P, Q, M, F, KSV, AX)                                                                                \
+    hipLaunchKernelGGL((fir_cl_kernel<P, Q, M, F, KSV, AX>), grid, dim3(256), 0, s, a.x1, a.x2, a.v, a.pj, h, K,   \
+                       taps_reversed, bias, (bf16_t*)out, (bf16_t*)y2_out, (bf16_t*)bx_out, bx_from, L, D, dg,      \
+                       seg_len, (int)nseg, (int)ndb)
+#define CL_CASE(P, Q, M, F, KSV)                                                                                  \
+    if (!ok && a.pre == P && a.post == Q && bias_mode == M && a.feat == F && (F == 0 || a.ks == KSV)) {           \
+        if (aux) CL_GO(P, Q, M, F, KSV, true); else CL_GO(P, Q, M, F, KSV, false);                                \
+        ok = true;                                                                                                \
+    }
+    CL_CASE(true, true, HYENA_BIAS_NONE, 0, 3)
+    CL_CASE(true, true, HYENA_BIAS_GATED_FP32, 0, 3)
+    CL_CASE(true, true, HYENA_BIAS_ADD, 0, 3)
+    CL_CASE(false, false, HYENA_BIAS_NONE, 0, 3)
+    CL_CASE(false, false, HYENA_BIAS_ADD, 0, 3)
+    CL_CASE(false, false, HYENA_BIAS_GATED_FP32, 0, 3)
+    CL_CASE(true, true, HYENA_BIAS_NONE, 1, 3)
+    CL_CASE(true, true, HYENA_BIAS_GATED_FP32, 1, 3)
+    CL_CASE(true, true, HYENA_BIAS_NONE, 3, 3)
+    CL_CASE(true, true, HYENA_BIAS_GATED_FP32, 3, 3)
+    CL_CASE(true, true, HYENA_BIAS_NONE, 1, 4)
+    CL_CASE(true, true, HYENA_BIAS_GATED_FP32, 1, 4)
+    CL_CASE(true, true, HYENA_BIAS_NONE, 3, 4)
+    CL_CASE(true, true, HYENA_BIAS_GATED_FP32, 3, 4)
+#undef CL_CASE
+#undef CL_GO
+    if (!ok) return hyena_fail(HYENA_ENOSUP, "%s: this gate / bias / featurizer-length combination has no kernel", who);
+    return hyena_check_launch(who);
+}
+
+static bool cl_ok(const hyena_cl* c) {
+    return c && c->ptr && !((uintptr_t)c->ptr & 15) && c->batch_stride % 8 == 0 && c->time_stride % 8 == 0;
+}
+
+}  // namespace
+
+extern "C" int hyena_fir_cl_fwd(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, const float* h,
+                                int taps_reversed, const float* bias, int bias_mode, void* out, void* y2_out,
+                                void* bx_out, int64_t bx_from, int64_t B, int64_t L, int64_t D, int64_t G, int K,
+                                void* stream) {
+    const char* who = "hyena_fir_cl_fwd";
+    if (!x1 || !x1->ptr) return hyena_fail(HYENA_EINVAL, "%s: x1 is required", who);
+    const bool pre = v && v->ptr, post = x2 && x2->ptr;
+    if (pre != post) return hyena_fail(HYENA_ENOSUP, "%s: pass both gates v and x2, or neither", who);
+    if (!cl_ok(x1) || (pre && (!cl_ok(v) || !cl_ok(x2))) || D % 8 != 0)
+        return hyena_fail(HYENA_EALIGN, "%s: D and strides must be multiples of 8, pointers 16-byte aligned", who);
+    LaunchArgs a = {};
+    a.x1 = {(const bf16_t*)x1->ptr, x1->batch_stride, x1->time_stride};
+    if (pre) {
+        a.v = {(const bf16_t*)v->ptr, v->batch_stride, v->time_stride};
+        a.x2 = {(const bf16_t*)x2->ptr, x2->batch_stride, x2->time_stride};
+    }
+    a.feat = 0; a.ks = 3; a.pre = pre; a.post = post;
+    return fir_cl_launch(a, h, taps_reversed, bias, bias_mode, out, y2_out, bx_out, bx_from, B, L, D, G, K, stream, who);
+}
+
+extern "C" int hyena_fir_layer_fwd(const hyena_proj_fwd* proj, const float* h, int taps_reversed, const float* bias,
+                                   int bias_mode, void* out, void* bx_out, int64_t bx_from, int64_t B, int64_t L,
+                                   int64_t D, int64_t G, int K, void* stream) {
+    const char* who = "hyena_fir_layer_fwd";
+    if (!proj || !proj->u || !proj->w) return hyena_fail(HYENA_EINVAL, "%s: proj, proj->u, proj->w are required", who);
+    if (proj->Ks != 3 && proj->Ks != 4)
+        return hyena_fail(HYENA_ENOSUP, "%s: featurizer length %d (3 or 4 supported)", who, proj->Ks);
+    if (D <= 0 || D % 8 != 0 || ((uintptr_t)proj->u & 15) || proj->u_batch_stride % 8 != 0 ||
+        proj->u_time_stride % 8 != 0)
+        return hyena_fail(HYENA_EALIGN, "%s: D and strides must be multiples of 8, u 16-byte aligned", who);
+    if (proj->ch_inner <= 0 || proj->ch_outer < 0 || proj->gate_stride <= 0)
+        return hyena_fail(HYENA_EINVAL, "%s: bad featurizer channel map", who);
+    LaunchArgs a = {};
+    a.pj.u = (const bf16_t*)proj->u; a.pj.bs = proj->u_batch_stride; a.pj.ts = proj->u_time_stride;
+    a.pj.w = proj->w; a.pj.bias = proj->bias;
+    a.pj.ch_inner = (uint32_t)(proj->ch_inner > D ? D : proj->ch_inner); a.pj.ch_outer = (uint32_t)proj->ch_outer;
+    a.pj.gate_stride = (uint32_t)proj->gate_stride; a.pj.flip = proj->flip_x1x2 != 0;
+    if (proj->ch_stride == 3 && proj->gate_stride == 1 && proj->ch_inner >= D) a.feat = 3;
+    else if (proj->ch_stride == 1 && proj->ch_inner % 8 == 0 && proj->ch_outer % 8 == 0 && proj->gate_stride % 8 == 0) {
+        a.feat = 1;
+        const int64_t last = ((D - 1) / proj->ch_inner) * proj->ch_outer + 2 * proj->gate_stride + (D - 1) % proj->ch_inner;
+        if (last >= 3 * D) return hyena_fail(HYENA_EINVAL, "%s: featurizer channel map reaches channel %lld of %lld", who,
+                                             (long long)last, (long long)(3 * D));
+    } else return hyena_fail(HYENA_ENOSUP, "%s: this featurizer channel map has no fused kernel", who);
+    a.ks = proj->Ks; a.pre = true; a.post = true;
+    if (bias_mode == HYENA_BIAS_ADD) return hyena_fail(HYENA_ENOSUP, "%s: additive inner bias", who);
+    return fir_cl_launch(a, h, taps_reversed, bias, bias_mode, out, nullptr, bx_out, bx_from, B, L, D, G, K, stream, who);
+}

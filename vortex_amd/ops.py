@@ -8,7 +8,7 @@ import ctypes
 import torch
 
 from . import _lib
-from ._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE, ProjStep, Rows
+from ._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE, Cl, ProjFwd, ProjStep, Rows
 
 
 def _stream():
@@ -100,6 +100,67 @@ def fir_fwd_rows(x1r, x2r, vr, taps, B, D, L, K, *, device, bias=None, bias_mode
                              _ptr(out), B, D, L, G, K, _stream())
         _lib.check(rc, "hyena_mr_fwd")
     return out
+
+
+def _cl_of(t):
+    """hyena_cl of a [B, L, D] bf16 tensor with contiguous channels (any batch / time stride)."""
+    if t is None:
+        return None
+    if t.dtype != torch.bfloat16 or t.dim() != 3 or (t.shape[2] > 1 and t.stride(2) != 1):
+        raise ValueError("expected a [B, L, D] bfloat16 tensor with contiguous channels")
+    return Cl(t.data_ptr(), t.stride(0), t.stride(1))
+
+
+def fir_cl_fwd(x1, x2, v, taps, *, bias=None, bias_mode=HYENA_BIAS_NONE, taps_reversed=False, want_y2=False,
+               want_bx=False, bx_from=0):
+    """Gated FIR on channel-last [B, L, D] tensors: out = x2 * conv(taps, x1*v), MFMA kernel, 1 <= K <= 128.
+
+    taps [G, K] float32, convolution orientation unless taps_reversed.  Returns out, or (out, y2, bx) when an
+    intermediate is requested (y2: the convolution before the x2 gate; bx: rows bx_from.. of bf16(x1*v)).
+    """
+    _need_cuda(x1, x2, v, taps)
+    taps = _f32(taps)
+    G, K = taps.shape
+    B, L, D = x1.shape
+    out = torch.empty((B, L, D), dtype=torch.bfloat16, device=x1.device)
+    y2 = torch.empty_like(out) if want_y2 else None
+    bx = torch.empty((B, L - bx_from, D), dtype=torch.bfloat16, device=x1.device) if want_bx else None
+    if out.numel():
+        c1, c2, cv = _cl_of(x1), _cl_of(x2), _cl_of(v)
+        rc = _lib.lib().hyena_fir_cl_fwd(_ref(c1), _ref(c2), _ref(cv), _ptr(taps), int(taps_reversed), _ptr(_f32(bias)),
+                                         bias_mode, _ptr(out), _ptr(y2), _ptr(bx), bx_from, B, L, D, G, K, _stream())
+        _lib.check(rc, "hyena_fir_cl_fwd")
+    return (out, y2, bx) if (want_y2 or want_bx) else out
+
+
+def fir_layer_fwd(u, feat_w, feat_bias, channel_map, taps, *, bias=None, bias_mode=HYENA_BIAS_NONE,
+                  taps_reversed=False, flip_x1x2=False, bx_from=None):
+    """A whole Hyena-SE / MR layer at prefill in one launch: u [B, L, 3D] bf16 -> out [B, L, D] bf16.
+
+    feat_w [Ks, 3D] float32 (tap-major, last row on the current sample), feat_bias [3D] or None, channel_map from
+    gate_channel_map().  bx_from: also return rows bx_from.. of bf16(x1*v) (the inner FIR cache of a decode step).
+    """
+    _need_cuda(u, feat_w, taps)
+    if u.dtype != torch.bfloat16 or u.dim() != 3 or u.stride(2) != 1:
+        raise ValueError("expected a [B, L, 3D] bfloat16 projection with contiguous channels")
+    taps = _f32(taps)
+    G, K = taps.shape
+    B, L, C = u.shape
+    D = C // 3
+    feat_w, feat_bias = _f32(feat_w), _f32(feat_bias)
+    if feat_w.shape[1] != C:
+        raise ValueError("feat_w must be [Ks, 3D] (tap-major)")
+    ci, co, gs, cs = channel_map
+    out = torch.empty((B, L, D), dtype=torch.bfloat16, device=u.device)
+    bx = torch.empty((B, L - bx_from, D), dtype=torch.bfloat16, device=u.device) if bx_from is not None else None
+    if out.numel():
+        pj = ProjFwd(u.data_ptr(), u.stride(0), u.stride(1), feat_w.data_ptr(),
+                     feat_bias.data_ptr() if feat_bias is not None else None, feat_w.shape[0], int(flip_x1x2),
+                     ci, co, gs, cs)
+        rc = _lib.lib().hyena_fir_layer_fwd(ctypes.byref(pj), _ptr(taps), int(taps_reversed), _ptr(_f32(bias)),
+                                            bias_mode, _ptr(out), _ptr(bx), bx_from or 0, B, L, D, G, K, _stream())
+        _lib.check(rc, "hyena_fir_layer_fwd")
+    return out if bx_from is None else (out, bx)
 
 
 def hyena_se_fwd(x1, x2, v, h, bias=None, *, force_mfma=False):
