@@ -147,7 +147,7 @@ def test_operator_module_prefill_then_decode(kind, cs, il, fused):
         if mod.D is not None:
             mod.D.data = p["D"].clone()
     mod = mod.to(DEV)
-    mod.fuse_decode = fused
+    mod.fuse_decode = mod.fuse_prefill = fused
     if K is None:     # oracle needs per-channel modal parameters
         pr = dict(p, log_poles=p["log_poles"].repeat_interleave(D // G, 0),
                   residues=p["residues"].repeat_interleave(D // G, 0))

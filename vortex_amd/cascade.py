@@ -87,6 +87,7 @@ class HyenaCascade(nn.Module):
         self._plan = None
         self._decode = None
         self.fuse_decode = True        # one launch per decode step where the fused layer-step kernels apply
+        self.fuse_prefill = True       # one launch per SE / MR prefill where the fused layer kernel applies
         self._f32_cache = {}
 
     # ------------------------------------------------------------------
@@ -140,11 +141,13 @@ class HyenaCascade(nn.Module):
             raise NotImplementedError("padding_mask is handled by the drop-in engine, not by this module")
         B, L, C = u.shape
         D, Ks = self.hidden_size, self.short_filter_length
+        caching = inference_params is not None
+        if self.fuse_prefill and self._can_fuse_prefill(u, L, caching):
+            return self._fused_prefill(u, inference_params), inference_params
         w = self._f32_param("short_filter_weight", (C, Ks))
         z_pre = ops.featurizer_fwd(u, w, self._f32_param("short_filter_bias"), interleave=self.interleave)
         r1, r2, rv = self._rows(z_pre)
         K = self.fir_inner_filter_length
-        caching = inference_params is not None
         if K:
             taps = self._f32_param("h", (self.h.shape[0], K))
             if K >= 128:
@@ -168,6 +171,46 @@ class HyenaCascade(nn.Module):
                     (x1 * v).permute(0, 2, 1).contiguous(), 0)
             self._decode = None
         return y.permute(0, 2, 1), inference_params
+
+    def _channel_map(self):
+        return ops.gate_channel_map(self.hidden_size, interleave=self.interleave,
+                                    head_dim=self.hidden_size_per_attention_head if self.column_split_hyena else None)
+
+    def _can_fuse_prefill(self, u, L, caching):
+        """Whether hyena_fir_layer_fwd covers this layer: an SE / MR layer with a 3- or 4-tap featurizer, a closed
+        channel map, 16-channel filter groups and an aligned projection."""
+        K, D, hd = self.fir_inner_filter_length, self.hidden_size, self.hidden_size_per_attention_head
+        if not K or K > 128 or self.short_filter_length not in (3, 4) or self._channel_map() is None:
+            return False
+        if (D // self.hyena_filter_groups) % 16 or D % 8 or (self.column_split_hyena and hd % 8):
+            return False
+        if caching and (L < K - 1 or L < self.short_filter_length - 1):
+            return False
+        return u.stride(2) == 1 and u.stride(1) % 8 == 0 and u.stride(0) % 8 == 0 and u.data_ptr() % 16 == 0
+
+    def _fused_prefill(self, u, inference_params):
+        """u [B, L, 3D] -> y [B, L, D] in one launch; with a cache object also the two FIR caches."""
+        B, L, C = u.shape
+        K, Ks = self.fir_inner_filter_length, self.short_filter_length
+        key = ("short_filter_weight_t", self.short_filter_weight.data_ptr(), self.short_filter_weight._version)
+        hit = self._f32_cache.get("wf_t")
+        if hit is None or hit[0] != key:
+            hit = (key, self._f32_param("short_filter_weight", (C, Ks)).t().contiguous())
+            self._f32_cache["wf_t"] = hit
+        mr = K >= 128
+        taps = self._f32_param("h", (self.h.shape[0], K))
+        caching = inference_params is not None
+        res = ops.fir_layer_fwd(u, hit[1], self._f32_param("short_filter_bias"), self._channel_map(), taps,
+                                bias=self._f32_param("D") if mr else None,
+                                bias_mode=HYENA_BIAS_GATED_FP32 if mr else HYENA_BIAS_NONE, taps_reversed=not mr,
+                                flip_x1x2=self.hyena_flip_x1x2, bx_from=L - (K - 1) if caching else None)
+        if not caching:
+            return res
+        y, bx = res
+        inference_params.fir_state_dict[self.layer_idx] = ops.FirRing(u[:, L - (Ks - 1):].contiguous(), 0)
+        inference_params.fir_inner_state_dict[self.layer_idx] = ops.FirRing(bx, 0)
+        self._decode = None
+        return y
 
     # ------------------------------------------------------------------
     def _decode_plan(self, inference_params):
@@ -200,8 +243,7 @@ class HyenaCascade(nn.Module):
 
     def _fused_step(self, ring, inner):
         """The one-launch layer step, or None where the fused kernels do not apply (then three launches are used)."""
-        cmap = ops.gate_channel_map(self.hidden_size, interleave=self.interleave,
-                                    head_dim=self.hidden_size_per_attention_head if self.column_split_hyena else None)
+        cmap = self._channel_map()
         Ks, hd = self.short_filter_length, self.hidden_size_per_attention_head
         fir = isinstance(inner, ops.FirStepper)
         if cmap is None or Ks < 2 or Ks > 8 or self.hidden_size % 8:

@@ -67,7 +67,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                                                         const float* __restrict__ bias, bf16_t* __restrict__ out,
                                                         bf16_t* __restrict__ y2_out, bf16_t* __restrict__ bx_out,
                                                         int64_t bx_from, int64_t L, int64_t D, int dg,
-                                                        int64_t seg_len, int nseg, int ndb) {
+                                                        int64_t seg_len, int nseg, int ndb, int flags) {
     constexpr int RF = FEAT ? KS - 1 : 0;          // extra rows a lane reads before its own four
     constexpr int NR = 4 + RF;                     // rows per lane and load piece
     constexpr int NP = (FEAT || (PRE && POST)) ? 3 : (PRE ? 2 : 1);   // load pieces per row
@@ -78,8 +78,10 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t bid = blockIdx.x;
-    const int seg = (int)(bid % (uint32_t)nseg);
-    const uint32_t db = (bid / (uint32_t)nseg) % (uint32_t)ndb;
+    // channel blocks fastest: the blocks resident at one time read neighbouring 128-byte pieces of the same rows
+    int seg; uint32_t db;
+    if (flags & 1) { seg = (int)(bid % (uint32_t)nseg); db = (bid / (uint32_t)nseg) % (uint32_t)ndb; }
+    else { db = bid % (uint32_t)ndb; seg = (int)((bid / (uint32_t)ndb) % (uint32_t)nseg); }
     const int64_t b = bid / ((uint32_t)nseg * (uint32_t)ndb);
     const uint32_t d0 = db * CB;
 
@@ -99,9 +101,9 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
                 const int lag = i_time - (8 * hh + 2 * j + e) + 128 - 16 * m;
-                float val = 0.f;
-                if (lag >= 0 && lag < K) val = h[g * K + (reversed ? K - 1 - lag : lag)];
-                t[e] = val;
+                const int li = lag < 0 ? 0 : (lag >= K ? K - 1 : lag);       // unconditional load, then select
+                const float hv = h[g * K + (reversed ? K - 1 - li : li)];
+                t[e] = (lag >= 0 && lag < K) ? hv : 0.f;
             }
             pk[j] = pack_bf2(t[0], t[1]);
         }
@@ -405,11 +407,13 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     dim3 grid((unsigned)nblk);
     const int dg = (int)(D / G);
     const bool aux = y2_out || bx_out;
+    int flags = 0;
+    if (const char* e = getenv("HYENA_CL_FLAGS")) flags = atoi(e);      // 1: segments fastest in the block order
     bool ok = false;
 #define CL_GO(P, Q, M, F, KSV, AX)                                                                                \
     hipLaunchKernelGGL((fir_cl_kernel<P, Q, M, F, KSV, AX>), grid, dim3(256), 0, s, a.x1, a.x2, a.v, a.pj, h, K,   \
                        taps_reversed, bias, (bf16_t*)out, (bf16_t*)y2_out, (bf16_t*)bx_out, bx_from, L, D, dg,      \
-                       seg_len, (int)nseg, (int)ndb)
+                       seg_len, (int)nseg, (int)ndb, flags)
 #define CL_CASE(P, Q, M, F, KSV)                                                                                  \
     if (!ok && a.pre == P && a.post == Q && bias_mode == M && a.feat == F && (F == 0 || a.ks == KSV)) {           \
         if (aux) CL_GO(P, Q, M, F, KSV, true); else CL_GO(P, Q, M, F, KSV, false);                                \
