@@ -103,6 +103,29 @@ def build_workload(name, device):
         fn = lambda: ops.li_fwd_rows(r1, r2, rv, plan, Db, B, D, L, device=device, out=out)
         return fn, dict(workload=f"hyena_li_prefill B={B} L={L} D={D} groups={G} poles={S} complex", tokens=B * L,
                         bytes=8 * B * D * L, kernel="li_kernel", keep=(x1, x2, v, plan, Db, out))
+    if name in ("mr_cl", "mr_layer", "se_layer"):
+        # channel-last variants: gates as three [B, L, D] tensors, or the whole layer from the projection
+        # u [B, L, 3D] (Evo 2 layout: interleaved gates, 3-tap featurizer); 8 bytes per output element either way
+        mr = name != "se_layer"
+        B, D, L, G, K = (2, 4096, 32768, 256, 128) if mr else (1, 4096, 8192, 256, 7)
+        g = torch.Generator(device=device).manual_seed(9)
+        rnd = lambda *s: torch.randn(*s, generator=g, device=device, dtype=torch.float32)
+        h = (O.make_mr_filter(G, K) if mr else O.make_se_filter(G, K)).reshape(G, K).to(device)
+        Db = rnd(D) if mr else None
+        mode = ops.HYENA_BIAS_GATED_FP32 if mr else ops.HYENA_BIAS_NONE
+        out = torch.empty(B, L, D, dtype=torch.bfloat16, device=device)
+        if name == "mr_cl":
+            x = [rnd(B, L, D).to(torch.bfloat16) for _ in range(3)]
+            fn = lambda: ops.fir_cl_fwd(x[1], x[0], x[2], h, bias=Db, bias_mode=mode, out=out)
+            what, keep = "hyena_mr_prefill channel-last gates", (x, h, Db, out)
+        else:
+            u = rnd(B, L, 3 * D).to(torch.bfloat16)
+            wf = rnd(3, 3 * D) * 3 ** -0.5
+            cmap = ops.gate_channel_map(D, interleave=True)
+            fn = lambda: ops.fir_layer_fwd(u, wf, None, cmap, h, bias=Db, bias_mode=mode, taps_reversed=not mr, out=out)
+            what, keep = ("hyena_mr" if mr else "hyena_se") + "_layer featurizer+operator from the projection", (u, wf, h, Db, out)
+        return fn, dict(workload=f"{what} B={B} L={L} D={D} groups={G} K={K}", tokens=B * L, bytes=8 * B * D * L,
+                        kernel="fir_cl_kernel", keep=keep)
     raise ValueError(name)
 
 
@@ -278,6 +301,11 @@ def main():
                 continue
             steps = max(3, min(args.steps, 20 if name == "li" else args.steps))
             e = run(name, steps, min(args.warmup, 3))
+            extra[name] = {"workload": e["workload"], "tokens_per_s": e["tokens_per_s"],
+                           "kernel_us": e["kernel_ms"] * 1e3, "hbm_gbs": e["hbm_gbs"],
+                           "roofline_frac": e["hbm_gbs"] / HBM_PEAK_GBS}
+        for name in ("mr_cl", "mr_layer", "se_layer"):
+            e = run(name, max(3, min(args.steps, 20)), min(args.warmup, 3))
             extra[name] = {"workload": e["workload"], "tokens_per_s": e["tokens_per_s"],
                            "kernel_us": e["kernel_ms"] * 1e3, "hbm_gbs": e["hbm_gbs"],
                            "roofline_frac": e["hbm_gbs"] / HBM_PEAK_GBS}

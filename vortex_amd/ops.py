@@ -112,7 +112,7 @@ def _cl_of(t):
 
 
 def fir_cl_fwd(x1, x2, v, taps, *, bias=None, bias_mode=HYENA_BIAS_NONE, taps_reversed=False, want_y2=False,
-               want_bx=False, bx_from=0):
+               want_bx=False, bx_from=0, out=None):
     """Gated FIR on channel-last [B, L, D] tensors: out = x2 * conv(taps, x1*v), MFMA kernel, 1 <= K <= 128.
 
     taps [G, K] float32, convolution orientation unless taps_reversed.  Returns out, or (out, y2, bx) when an
@@ -122,7 +122,8 @@ def fir_cl_fwd(x1, x2, v, taps, *, bias=None, bias_mode=HYENA_BIAS_NONE, taps_re
     taps = _f32(taps)
     G, K = taps.shape
     B, L, D = x1.shape
-    out = torch.empty((B, L, D), dtype=torch.bfloat16, device=x1.device)
+    if out is None:
+        out = torch.empty((B, L, D), dtype=torch.bfloat16, device=x1.device)
     y2 = torch.empty_like(out) if want_y2 else None
     bx = torch.empty((B, L - bx_from, D), dtype=torch.bfloat16, device=x1.device) if want_bx else None
     if out.numel():
@@ -134,7 +135,7 @@ def fir_cl_fwd(x1, x2, v, taps, *, bias=None, bias_mode=HYENA_BIAS_NONE, taps_re
 
 
 def fir_layer_fwd(u, feat_w, feat_bias, channel_map, taps, *, bias=None, bias_mode=HYENA_BIAS_NONE,
-                  taps_reversed=False, flip_x1x2=False, bx_from=None):
+                  taps_reversed=False, flip_x1x2=False, bx_from=None, out=None):
     """A whole Hyena-SE / MR layer at prefill in one launch: u [B, L, 3D] bf16 -> out [B, L, D] bf16.
 
     feat_w [Ks, 3D] float32 (tap-major, last row on the current sample), feat_bias [3D] or None, channel_map from
@@ -151,7 +152,8 @@ def fir_layer_fwd(u, feat_w, feat_bias, channel_map, taps, *, bias=None, bias_mo
     if feat_w.shape[1] != C:
         raise ValueError("feat_w must be [Ks, 3D] (tap-major)")
     ci, co, gs, cs = channel_map
-    out = torch.empty((B, L, D), dtype=torch.bfloat16, device=u.device)
+    if out is None:
+        out = torch.empty((B, L, D), dtype=torch.bfloat16, device=u.device)
     bx = torch.empty((B, L - bx_from, D), dtype=torch.bfloat16, device=u.device) if bx_from is not None else None
     if out.numel():
         pj = ProjFwd(u.data_ptr(), u.stride(0), u.stride(1), feat_w.data_ptr(),
