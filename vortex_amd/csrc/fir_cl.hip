@@ -101,9 +101,9 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
                 const int lag = i_time - (8 * hh + 2 * j + e) + 128 - 16 * m;
-                const int li = lag < 0 ? 0 : (lag >= K ? K - 1 : lag);       // unconditional load, then select
-                const float hv = h[g * K + (reversed ? K - 1 - li : li)];
-                t[e] = (lag >= 0 && lag < K) ? hv : 0.f;
+                float val = 0.f;
+                if (lag >= 0 && lag < K) val = h[g * K + (reversed ? K - 1 - lag : lag)];
+                t[e] = val;
             }
             pk[j] = pack_bf2(t[0], t[1]);
         }
