@@ -389,13 +389,22 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
         return hyena_fail(HYENA_EALIGN, "%s: outputs must be 16-byte aligned", who);
     if (B == 0 || L == 0) return 0;
 
-    // segments along L: enough blocks for several rounds over 256 CUs, segments of at least 1024 samples
+    // Segments along L.  512 blocks are resident at a time (2 per CU); pick the segment count whose block
+    // count fills whole rounds of 512 best, charging each segment its extra 128-sample halo step.
     const int64_t ndb = (D + CB - 1) / CB;
     const int64_t rows = B * ndb;
-    int64_t nseg = (2048 + rows - 1) / rows;
-    const int64_t max_seg = (L + 1023) / 1024;
-    if (nseg > max_seg) nseg = max_seg;
-    if (nseg < 1) nseg = 1;
+    int64_t nseg = 1;
+    {
+        const int64_t max_seg = (L + 1023) / 1024 < 64 ? (L + 1023) / 1024 : 64;
+        double best = -1.0;
+        for (int64_t c = 1; c <= (max_seg < 1 ? 1 : max_seg); ++c) {
+            const int64_t sl = ((L + c - 1) / c + TL - 1) / TL * TL;
+            const int64_t nb = rows * ((L + sl - 1) / sl);
+            const double fill = (double)nb / (double)((nb + 511) / 512 * 512);
+            const double score = fill * (double)sl / (double)(sl + TL);
+            if (score > best + 1e-9) { best = score; nseg = c; }
+        }
+    }
     if (const char* e = getenv("HYENA_CL_NSEG")) { int64_t x = atoll(e); if (x >= 1) nseg = x; }
     int64_t seg_len = (L + nseg - 1) / nseg;
     seg_len = (seg_len + TL - 1) / TL * TL;
