@@ -70,15 +70,42 @@ def _gcg(x, k, q, h, bias, apply_gated_bias):
                             force_mfma=(K > 8 or mode == HYENA_BIAS_GATED_FP32))
 
 
+def _cl_ok(x, h):
+    """Whether the channel-last MFMA kernel covers (b, l, g, dg) inputs with this filter."""
+    return x.dim() == 4 and x.shape[3] % 16 == 0 and h.shape[-1] <= 128
+
+
+def _gcg_cl(x, k, q, h, bias, apply_gated_bias, want_y2=False, want_bx=False):
+    """q * conv(k*x) on (b, l, g, dg) bf16 tensors without leaving the channel-last layout."""
+    b, l, g, dg = x.shape
+    taps = ops._f32(h).reshape(h.shape[0], -1)
+    mode = HYENA_BIAS_NONE if bias is None else (HYENA_BIAS_GATED_FP32 if apply_gated_bias else HYENA_BIAS_ADD)
+    flat = lambda t: t.reshape(b, l, g * dg)
+    return ops.fir_cl_fwd(flat(k), flat(q), flat(x), taps, bias=ops._f32(bias), bias_mode=mode, taps_reversed=True,
+                          want_y2=want_y2, want_bx=want_bx)
+
+
 def inner_hyena_se(x, k, q, h, bias=None, input_layout="bdl", output_layout="bdl", inner_layout="bdl",
                    apply_gated_bias=False, schedule="default", autotune=False, fwd_kernel_cfg=None,
                    bwd_kernel_cfg=None, use_fast_causal_conv1d=False, kernel_path=None):
     """y = q * causal_depthwise_conv(h, k * x)  (vortex/ops/hyena_se/interface.py:342-397).
 
     h: [G, 1, K]; group g filters channels g*dg .. (g+1)*dg-1.  Layouts: "bdl" [B, D, L],
-    "blgdg" [B, L, G, dg], "bgdgl" [B, G, dg, L] in; "bdl", "bld", "blgdg" out.
+    "blgdg" [B, L, G, dg], "bgdgl" [B, G, dg, L] in; "bdl", "bld", "blgdg" out.  (b, l, g, dg) inputs
+    with dg a multiple of 16 stay channel-last through the kernel; other cases go through [B, D, L].
     """
     G = h.shape[0]
+    if input_layout == "blgdg" and _cl_ok(x, h):
+        assert k.shape == q.shape == x.shape, "feature groups must have the same shape"
+        b, l, g, dg = x.shape
+        y = _gcg_cl(x, k, q, h, bias, apply_gated_bias)
+        if output_layout == "bld":
+            return y
+        if output_layout == "blgdg":
+            return y.reshape(b, l, g, dg)
+        if output_layout == "bdl":
+            return y.transpose(1, 2)
+        raise NotImplementedError("output_layout must be bld, bdl or blgdg")
     xb, kb, qb = (_to_bdl(t, input_layout) for t in (x, k, q))
     assert kb.shape == qb.shape == xb.shape, "feature groups must have the same shape"
     y = _gcg(xb, kb, qb, h, bias, apply_gated_bias)
@@ -114,15 +141,59 @@ def two_pass_chunked_gate_conv_gate(x, B, C, h, return_toeplitz=True, schedule="
     return inner_hyena_se(x, B, C, h, input_layout="blgdg", output_layout="blgdg")
 
 
-def two_pass_fwd_grouped(x, B, C, h, *args, **kwargs):
-    """(y, T, T_hat, y2, bx_lag) of vortex/ops/hyena_se/fwd.py:17-43, :290 with the
-    intermediates, which exist only for the backward pass, returned as None."""
-    return two_pass_chunked_gate_conv_gate(x, B, C, h), None, None, None, None
+def _toeplitz_pair(h, chunk, dtype):
+    """T[g, i, j] = hf[g, i-j] (0 <= i-j < K) and T_hat[g, i, j] = hf[g, i+chunk-j] (i+chunk-j < K) with
+    hf = h.flip(-1): the within-chunk and previous-chunk Toeplitz factors of
+    vortex/ops/hyena_se/utils.py:5-25, :38-51."""
+    g, K = h.shape[0], h.shape[-1]
+    hf = h.reshape(g, K).flip(-1)
+    idx = torch.arange(chunk, device=h.device)
+    lag = idx[:, None] - idx[None, :]
+    def gather(l):
+        ok = (l >= 0) & (l < K)
+        return torch.where(ok[None], hf[:, l.clamp(0, K - 1)], torch.zeros((), device=h.device, dtype=hf.dtype)).to(dtype)
+    return gather(lag), gather(lag + chunk)
+
+
+def two_pass_fwd_grouped(x, B, C, h, y=None, return_y2=False, return_toeplitz=False, return_bx_lag=False,
+                         verbose=False, schedule="default", autotune=False, version="refactor", CHUNK_SIZE=None,
+                         *args, **kwargs):
+    """(y, T, T_hat, y2, bx_lag) of vortex/ops/hyena_se/fwd.py:17-43, :290 on (b, l, g, dg) tensors.
+
+    y2 is the convolution before the C gate; bx_lag holds B*x for every chunk but the last (zeros there), as
+    fwd_kernels.py:400-409 stores it; T, T_hat are the chunk Toeplitz factors (CHUNK_SIZE required, as in
+    fwd.py:199-203).  The kernel itself is not chunk-parametrised; CHUNK_SIZE only shapes these by-products.
+    """
+    T = T_hat = y2 = bx_lag = None
+    b, l, g, dg = x.shape
+    if _cl_ok(x, h):
+        res = _gcg_cl(x, B, C, h, None, False, want_y2=return_y2, want_bx=return_bx_lag)
+        out, y2f, bxf = res if (return_y2 or return_bx_lag) else (res, None, None)
+        out = out.reshape(b, l, g, dg)
+        if return_y2:
+            y2 = y2f.reshape(b, l, g, dg)
+        if return_bx_lag:
+            assert CHUNK_SIZE is not None, "CHUNK_SIZE must be specified for return_bx_lag"
+            bxf[:, max(l - CHUNK_SIZE, 0):] = 0
+            bx_lag = bxf.reshape(b, l, g, dg)
+    else:
+        if return_y2 or return_bx_lag:
+            raise NotImplementedError("intermediates need group_dim % 16 == 0 and K <= 128")
+        out = two_pass_chunked_gate_conv_gate(x, B, C, h)
+    if return_toeplitz:
+        assert CHUNK_SIZE is not None, "CHUNK_SIZE must be specified for return_toeplitz"
+        T, T_hat = _toeplitz_pair(h, CHUNK_SIZE, x.dtype)
+    if y is not None:
+        y.copy_(out)
+        out = y
+    return out, T, T_hat, y2, bx_lag
 
 
 def hyena_se(x, B, C, h, bias=None, apply_gated_bias=False, schedule="default", autotune=False, fwd_kernel_cfg=None,
              bwd_kernel_cfg=None):
     """vortex/ops/hyena_se/interface.py:247-269 (whose own body passes mismatched arguments);
     computes C * conv(h, B * x) + bias rule on (b, l, g, dg) tensors."""
+    if _cl_ok(x, h):
+        return _gcg_cl(x, B, C, h, bias, apply_gated_bias).reshape(x.shape)
     xb, kb, qb = (_to_bdl(t, "blgdg") for t in (x, B, C))
     return _from_bdl(_gcg(xb, kb, qb, h, bias, apply_gated_bias), "blgdg", h.shape[0])

@@ -202,3 +202,24 @@ def test_featurizer_full_width():
     ref = O.interleave(ref)
     assert rel_err(z, ref) <= 2e-2
     assert (z.cpu() == ref).float().mean() > 0.98
+
+
+def test_two_pass_fwd_grouped_intermediates():
+    # (y, T, T_hat, y2, bx_lag) of vortex/ops/hyena_se/fwd.py:290 on (b, l, g, dg) tensors, channel-last kernel
+    from hyena_ops import interface as I
+    B, L, G, dg, K, CH = 2, 512, 3, 32, 33, 128
+    gen = torch.Generator().manual_seed(6)
+    x, Bm, Cm = (torch.randn(B, L, G, dg, generator=gen).bfloat16() for _ in range(3))
+    h = torch.randn(G, 1, K, generator=gen) / K ** 0.5
+    y, T, T_hat, y2, bx_lag = I.two_pass_fwd_grouped(x.to(DEV), Bm.to(DEV), Cm.to(DEV), h.to(DEV), return_y2=True,
+                                                     return_toeplitz=True, return_bx_lag=True, CHUNK_SIZE=CH)
+    ref = O.gcg_fwd_ref(x.float(), Bm.float(), Cm.float(), h)
+    assert y.shape == ref.shape and rel_err(y, ref) <= 2e-2
+    assert rel_err(y, O.gcg_two_pass_chunked(x.float(), Bm.float(), Cm.float(), h, CH)) <= 2e-2
+    y2_ref = O.gcg_fwd_ref(x.float(), Bm.float(), torch.ones_like(Cm).float(), h)
+    assert rel_err(y2, y2_ref) <= 2e-2
+    bx = Bm * x
+    assert torch.equal(bx_lag[:, :L - CH].cpu(), bx[:, :L - CH]) and not bx_lag[:, L - CH:].any()
+    hf = h.flip(-1)[:, 0]
+    assert torch.equal(T.cpu(), O.toeplitz(hf, CH).bfloat16())
+    assert torch.equal(T_hat.cpu(), O.correction_toeplitz(hf, CH).bfloat16())
