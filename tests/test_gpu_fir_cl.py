@@ -151,3 +151,55 @@ def test_cl_rejects_unsupported():
         ops.fir_cl_fwd(x, x, x, torch.zeros(3, 4, device=DEV))
     with pytest.raises(NotImplementedError):
         ops.fir_cl_fwd(torch.zeros(1, 16, 32, dtype=torch.bfloat16, device=DEV), None, None, torch.zeros(2, 200, device=DEV))
+
+
+def test_cl_impulse_response_across_steps_and_segments():
+    # bf16-exact taps, unit gates: the output is the filter itself wherever an impulse sits, bit for bit
+    B, D, L, G, K = 1, 64, 4096, 4, 128
+    h = O.make_mr_filter(G, K).bfloat16().float()
+    x1 = torch.zeros(B, L, D, dtype=torch.bfloat16)
+    pos = [0, 127, 300, 1023, 2047, 2050, L - 5]          # step boundaries (128) and segment boundaries (1024)
+    for p in pos:
+        x1[:, p] = 1
+    one = torch.ones(B, L, D, dtype=torch.bfloat16)
+    os.environ["HYENA_CL_NSEG"] = "4"
+    try:
+        out = ops.fir_cl_fwd(x1.to(DEV), one.to(DEV), one.to(DEV), h.reshape(G, K).to(DEV)).cpu().float()
+    finally:
+        del os.environ["HYENA_CL_NSEG"]
+    hw = h.repeat_interleave(D // G, 0)[:, 0]            # [D, K]
+    exp = torch.zeros(B, L, D)
+    for p in pos:
+        n = min(K, L - p)
+        exp[0, p:p + n] += hw[:, :n].t()
+    assert torch.equal(out, exp.bfloat16().float())
+
+
+def test_layer_full_size_config2():
+    # Hyena-MR layer at config 2's shape (B=2, L=32768, D=4096, 256 groups, K=128) from an interleaved projection:
+    # the one-launch kernel against the featurizer + sequence-major MR kernels, and sampled channels against the oracle
+    B, L, D, G, K, Ks = 2, 32768, 4096, 256, 128, 3
+    C = 3 * D
+    g = torch.Generator(device=DEV).manual_seed(12)
+    u = torch.randn(B, L, C, generator=g, device=DEV, dtype=torch.float32).bfloat16()
+    wf = (torch.randn(C, Ks, generator=g, device=DEV) / Ks ** 0.5)
+    h = O.make_mr_filter(G, K)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(13))
+    cmap = ops.gate_channel_map(D, interleave=True)
+    y, bx = ops.fir_layer_fwd(u, wf.t().contiguous(), None, cmap, h.reshape(G, K).to(DEV), bias=Db.to(DEV),
+                              bias_mode=HYENA_BIAS_GATED_FP32, bx_from=L - (K - 1))
+    z = ops.featurizer_fwd(u, wf, None, interleave=True)
+    r2, r1, rv = (ops.rows_of_projection(z, D, i) for i in range(3))
+    y2 = ops.fir_fwd_rows(r1, r2, rv, h.reshape(G, K).to(DEV), B, D, L, K, device=u.device, bias=Db.to(DEV),
+                          bias_mode=HYENA_BIAS_GATED_FP32, force_mfma=True)
+    assert rel_err(y, y2.permute(0, 2, 1)) <= 2e-2
+    x1v_tail = (z[:, D:2 * D, L - (K - 1):] * z[:, 2 * D:, L - (K - 1):]).permute(0, 2, 1)
+    assert rel_err(bx, x1v_tail) <= 1e-2
+    del z, y2
+    ds = torch.arange(5, D, 409)                                   # sampled operator channels
+    ch = (3 * ds[:, None] + torch.arange(3)[None]).reshape(-1)      # their interleaved projection channels
+    us = u[:, :, ch.to(DEV)].cpu()
+    n = len(ds)
+    ref, _ = oracle_layer(us, wf.cpu()[ch][:, None, :], None, h.repeat_interleave(D // G, 0)[ds], Db[ds], n, 1, False,
+                          True, False)
+    assert rel_err(y[:, :, ds.to(DEV)].permute(0, 2, 1), ref) <= 2e-2

@@ -90,3 +90,30 @@ def test_rows_struct_layout_matches_header():
     # hyena_rows: one pointer and four int64, no padding
     assert ctypes.sizeof(ops.Rows) == 40
     assert [f[0] for f in ops.Rows._fields_] == ["ptr", "batch_stride", "row_stride", "ch_inner", "ch_outer"]
+
+
+@pytest.mark.parametrize("cs,il", [(False, False), (True, False), (False, True)])
+def test_gate_channel_map_matches_reference_split(cs, il):
+    # the closed channel maps the fused layer kernels use == interleave / split / column_split of the reference
+    D, H = 48, 4
+    z = torch.arange(3 * D, dtype=torch.float32)[None]            # value = projection channel index
+    ref = O.interleave(z) if il else z
+    x2, x1, v = O.split_gates(ref, (D, H, D // H), cs, False)
+    ci, co, gs, cst = ops.gate_channel_map(D, interleave=il, head_dim=D // H if cs else None)
+    d = torch.arange(D)
+    for gate, want in enumerate((x2, x1, v)):
+        ch = (d // ci) * co + gate * gs + (d % ci) * cst
+        assert torch.equal(ch.float(), want[0])
+    assert ops.gate_channel_map(D, interleave=True, head_dim=D // H) is None
+
+
+def test_proj_structs_match_header():
+    from vortex_amd import _lib
+    # hyena_proj_step: 7 pointer/int64 fields, 4 int64 map fields, one int (padded to 8)
+    assert ctypes.sizeof(_lib.ProjStep) == 12 * 8
+    assert _lib.ProjStep.flip_x1x2.offset == 11 * 8
+    # hyena_proj_fwd: 5 pointer/int64 fields, two ints, 4 int64 map fields
+    assert ctypes.sizeof(_lib.ProjFwd) == 10 * 8
+    assert _lib.ProjFwd.Ks.offset == 5 * 8 and _lib.ProjFwd.flip_x1x2.offset == 5 * 8 + 4
+    assert _lib.ProjFwd.ch_inner.offset == 6 * 8
+    assert ctypes.sizeof(_lib.Cl) == 3 * 8
