@@ -61,13 +61,16 @@ __device__ __forceinline__ float el(const u32x4& r, int e) { return (e & 1) ? bf
 // FEAT: 0 = gates given as three channel-last tensors; 1 = gates from the fused featurizer, unit channel
 // stride (plain or head-blocked split); 3 = fused featurizer with interleaved gates (channel 3d+i).
 // KS = featurizer taps (FEAT != 0).  AUX = also store y2 (z before the x2 gate) and / or bx = bf16(x1*v).
-template <bool PRE, bool POST, int BIAS, int FEAT, int KS, bool AUX>
+// MLO = first Toeplitz block that can be non-zero: 0 for any K <= 128, 7 for K <= 17 (lags 0..16 touch only
+// blocks 7..9), which leaves three A fragments in registers and five B reads / six MFMAs per step.
+template <bool PRE, bool POST, int BIAS, int FEAT, int KS, bool AUX, int MLO>
 __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMap v, ProjFwd pj,
                                                         const float* __restrict__ h, int K, int reversed,
                                                         const float* __restrict__ bias, bf16_t* __restrict__ out,
                                                         bf16_t* __restrict__ y2_out, bf16_t* __restrict__ bx_out,
                                                         int64_t bx_from, int64_t L, int64_t D, int dg,
-                                                        int64_t seg_len, int nseg, int ndb, int flags) {
+                                                        int64_t seg_len, int nseg, int ndb) {
+    constexpr bool EARLY = !FEAT;                  // next step's rows requested before (true) or after the MFMA phase
     constexpr int RF = FEAT ? KS - 1 : 0;          // extra rows a lane reads before its own four
     constexpr int NR = 4 + RF;                     // rows per lane and load piece
     constexpr int NP = (FEAT || (PRE && POST)) ? 3 : (PRE ? 2 : 1);   // load pieces per row
@@ -79,9 +82,8 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t bid = blockIdx.x;
     // channel blocks fastest: the blocks resident at one time read neighbouring 128-byte pieces of the same rows
-    int seg; uint32_t db;
-    if (flags & 1) { seg = (int)(bid % (uint32_t)nseg); db = (bid / (uint32_t)nseg) % (uint32_t)ndb; }
-    else { db = bid % (uint32_t)ndb; seg = (int)((bid / (uint32_t)ndb) % (uint32_t)nseg); }
+    const uint32_t db = bid % (uint32_t)ndb;
+    const int seg = (int)((bid / (uint32_t)ndb) % (uint32_t)nseg);
     const int64_t b = bid / ((uint32_t)nseg * (uint32_t)ndb);
     const uint32_t d0 = db * CB;
 
@@ -90,10 +92,9 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     const bool slab_live = d0 + 16 * w < (uint32_t)D;
     const int g = slab_live ? (int)((d0 + 16 * w) / (uint32_t)dg) : 0;
     const int i_time = 16 * ((n >> 2) & 1) + 4 * (n >> 3) + (n & 3);
-    bf16x8 A[10];
-    const int m_min = (114 - K) > 0 ? (114 - K + 15) / 16 : 0;      // blocks below m_min are all zero
+    bf16x8 A[10 - MLO];
 #pragma unroll
-    for (int m = 0; m < 10; ++m) {
+    for (int m = MLO; m < 10; ++m) {
         u32x4 pk;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             }
             pk[j] = pack_bf2(t[0], t[1]);
         }
-        A[m] = as_bf16x8(pk);
+        A[m - MLO] = as_bf16x8(pk);
     }
 
     // ---- this lane's I/O block: rows 4*rb .. 4*rb+3 of the step, channels d0 + 8*cb .. +7
@@ -261,10 +262,11 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             }
         }
         // ---- (b) next step's rows are requested now and arrive during the MFMA phase
-        // With the featurizer fused in, a lane holds 18 row pieces; keeping them in flight across the MFMA phase
-        // does not fit the register budget of two blocks per CU, so they are requested after it instead.
+        // With the featurizer fused in, a lane holds 18 row pieces; next to all ten A fragments, keeping them in
+        // flight across the MFMA phase does not fit the register budget of two blocks per CU, so they are
+        // requested after it instead (measured: no slower than the early request where both fit).
         __builtin_amdgcn_sched_barrier(0);
-        if (!FEAT && ts + TL < t_end) load_step(ts + TL);
+        if (EARLY && ts + TL < t_end) load_step(ts + TL);
 
         // ---- (c) 4 x 8 transpose into the ring chunk `cur`
         {
@@ -295,10 +297,10 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             const bf16_t* urow = u_lds + (16 * w + c) * URS;
             const int c0 = 64 * s + 8 * hh + (cur ^ 1) * TL;     // ring position of the halo chunk's first sample
 #pragma unroll
-            for (int mm = 0; mm < 12; ++mm) {
+            for (int mm = MLO; mm < 12; ++mm) {
                 const bf16x8 bf = *(const bf16x8*)(urow + ((c0 + 16 * mm) & (2 * TL - 1)));
-                if (mm <= 9 && mm >= m_min) acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm <= 9 ? mm : 0], bf, acc0, 0, 0, 0);
-                if (mm >= 2 && mm - 2 >= m_min) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm >= 2 ? mm - 2 : 0], bf, acc1, 0, 0, 0);
+                if (mm <= 9) acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm <= 9 ? mm - MLO : 0], bf, acc0, 0, 0, 0);
+                if (mm - 2 >= MLO) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm - 2 >= MLO ? mm - 2 - MLO : 0], bf, acc1, 0, 0, 0);
                 if ((mm & 3) == 3) __builtin_amdgcn_sched_barrier(0);    // at most four B fragments in registers at a time
             }
 #pragma unroll
@@ -331,7 +333,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             }
         }
         __syncthreads();
-        if (FEAT) {
+        if (!EARLY) {
             __builtin_amdgcn_sched_barrier(0);
             if (ts + TL < t_end) load_step(ts + TL);
         }
@@ -416,16 +418,17 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     dim3 grid((unsigned)nblk);
     const int dg = (int)(D / G);
     const bool aux = y2_out || bx_out;
-    int flags = 0;
-    if (const char* e = getenv("HYENA_CL_FLAGS")) flags = atoi(e);      // 1: segments fastest in the block order
+    const bool shortk = K <= 17;
     bool ok = false;
-#define CL_GO(P, Q, M, F, KSV, AX)                                                                                \
-    hipLaunchKernelGGL((fir_cl_kernel<P, Q, M, F, KSV, AX>), grid, dim3(256), 0, s, a.x1, a.x2, a.v, a.pj, h, K,   \
-                       taps_reversed, bias, (bf16_t*)out, (bf16_t*)y2_out, (bf16_t*)bx_out, bx_from, L, D, dg,      \
-                       seg_len, (int)nseg, (int)ndb, flags)
+#define CL_GO(P, Q, M, F, KSV, AX, ML)                                                                            \
+    hipLaunchKernelGGL((fir_cl_kernel<P, Q, M, F, KSV, AX, ML>), grid, dim3(256), 0, s, a.x1, a.x2, a.v, a.pj, h, \
+                       K, taps_reversed, bias, (bf16_t*)out, (bf16_t*)y2_out, (bf16_t*)bx_out, bx_from, L, D, dg,   \
+                       seg_len, (int)nseg, (int)ndb)
 #define CL_CASE(P, Q, M, F, KSV)                                                                                  \
     if (!ok && a.pre == P && a.post == Q && bias_mode == M && a.feat == F && (F == 0 || a.ks == KSV)) {           \
-        if (aux) CL_GO(P, Q, M, F, KSV, true); else CL_GO(P, Q, M, F, KSV, false);                                \
+        if (aux) CL_GO(P, Q, M, F, KSV, true, 0);                                                                 \
+        else if (shortk && P && M == HYENA_BIAS_NONE) CL_GO(P, Q, M, F, KSV, false, (P && M == HYENA_BIAS_NONE) ? 7 : 0); \
+        else CL_GO(P, Q, M, F, KSV, false, 0);                                                                    \
         ok = true;                                                                                                \
     }
     CL_CASE(true, true, HYENA_BIAS_NONE, 0, 3)
