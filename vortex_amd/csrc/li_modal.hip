@@ -213,19 +213,22 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     bf16_t* xh_w = (bf16_t*)(l_w + 16 * LRS);                  // [4][4][XRS]
     bf16_t* xl_w = xh_w + 16 * XRS;
 
-    // ---- A fragments: one 16-byte load each, pinned in registers for the whole kernel
+    // ---- A fragments: one 16-byte load each, pinned in registers for the whole kernel.  All 48 loads are issued
+    // before the first is pinned, so they overlap instead of paying one memory round trip each.
     const u32x4* fr = (const u32x4*)ws + lane;
     bf16x8 Th[8], Tl[8], Poh[8], Pol[8], Pih[8], Pil[8];
     {
-        u32x4 t;
-#define LI_FRAG(dst, idx) t = fr[(idx) * 64]; asm volatile("" : "+v"(t)); dst = as_bf16x8(t);
+        u32x4 t[N_FRAG];
+#pragma unroll
+        for (int i = 0; i < N_FRAG; ++i) t[i] = fr[i * 64];
+#pragma unroll
+        for (int i = 0; i < N_FRAG; ++i) asm volatile("" : "+v"(t[i]));
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
-            LI_FRAG(Th[q], FR_T + q) LI_FRAG(Tl[q], FR_T + 8 + q)
-            LI_FRAG(Poh[q], FR_PO + q) LI_FRAG(Pol[q], FR_PO + 8 + q)
-            LI_FRAG(Pih[q], FR_PI + q) LI_FRAG(Pil[q], FR_PI + 8 + q)
+            Th[q] = as_bf16x8(t[FR_T + q]);   Tl[q] = as_bf16x8(t[FR_T + 8 + q]);
+            Poh[q] = as_bf16x8(t[FR_PO + q]); Pol[q] = as_bf16x8(t[FR_PO + 8 + q]);
+            Pih[q] = as_bf16x8(t[FR_PI + q]); Pil[q] = as_bf16x8(t[FR_PI + 8 + q]);
         }
-#undef LI_FRAG
     }
 
     // MFMA-side lane geometry: column n = channel c + 4 * chunk s, k / row quad q
