@@ -93,3 +93,63 @@ def test_featurizer_random(B, L, seed):
     if il:
         ref = O.interleave(ref)
     assert rel_err(z, ref) <= 2e-2, (B, L, C, K, il)
+
+
+def cl_cases(seed, n):
+    rng = random.Random(seed)
+    return [(rng.choice([1, 2, 3]), rng.randint(1, 3000), rng.randint(0, 10 ** 6)) for _ in range(n)]
+
+
+@pytest.mark.parametrize("B,L,seed", cl_cases(7, 14))
+def test_channel_last_fir_random(B, L, seed, monkeypatch):
+    # channel-last kernel: any L (rows are independent), channel counts that leave partial 64-channel blocks,
+    # every filter length class, forced segment counts
+    rng = random.Random(seed)
+    K = rng.choice([1, 2, 7, 16, 17, 18, 33, 64, 97, 98, 99, 127, 128])
+    G = rng.randint(1, 5)
+    D = G * 16 * rng.randint(1, 3)
+    monkeypatch.setenv("HYENA_CL_NSEG", str(rng.randint(1, 5)))
+    x2, x1, v = O.make_gates(B, D, L, seed=seed)
+    h = O.make_mr_filter(G, K, seed=seed + 1)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(seed))
+    gated = rng.random() < 0.5
+    u = x1 * v
+    w = h.repeat_interleave(D // G, 0)
+    conv = O.short_fir_fp32(u, w.flip(-1), K)                       # convolution = correlation with flipped taps
+    z = (conv + (u.float() * Db[None, :, None] if gated else 0)).bfloat16()
+    ref = x2 * z
+    cl = lambda t: t.permute(0, 2, 1).contiguous().cuda()
+    out = ops.fir_cl_fwd(cl(x1), cl(x2), cl(v), h.reshape(G, K).cuda(), bias=Db.cuda() if gated else None,
+                         bias_mode=ops.HYENA_BIAS_GATED_FP32 if gated else ops.HYENA_BIAS_NONE)
+    assert rel_err(out.permute(0, 2, 1), ref) <= 2e-2, (B, D, L, G, K, gated)
+
+
+@pytest.mark.parametrize("B,L,seed", cl_cases(8, 12))
+def test_fused_layer_random(B, L, seed, monkeypatch):
+    rng = random.Random(seed)
+    K = rng.choice([2, 4, 7, 17, 18, 64, 128])
+    Ks = rng.choice([3, 4])
+    G = rng.randint(1, 4)
+    H = rng.choice([1, 2])
+    D = G * 16 * H
+    cs, il = rng.choice([(False, False), (True, False), (False, True)])
+    flip, sbias = rng.random() < 0.5, rng.random() < 0.5
+    L = max(L, K)
+    monkeypatch.setenv("HYENA_CL_NSEG", str(rng.randint(1, 4)))
+    g = torch.Generator().manual_seed(seed)
+    C = 3 * D
+    u = torch.randn(B, L, C, generator=g).bfloat16()
+    wf = torch.randn(C, 1, Ks, generator=g) / Ks ** 0.5
+    bf = torch.randn(C, generator=g).bfloat16() if sbias else None
+    h = O.make_se_filter(G, K, seed=seed)
+    z, _ = O.parallel_fir(u, wf, bf, fir_length=Ks, dim_last=True, gate=False)
+    if il:
+        z = O.interleave(z)
+    x2, x1, v = O.split_gates(z, (D, H, D // H), cs, flip)
+    ref = O.se_fir(x2, x1, v, h)[0]
+    cmap = ops.gate_channel_map(D, interleave=il, head_dim=D // H if cs else None)
+    y, bx = ops.fir_layer_fwd(u.cuda(), wf.reshape(C, Ks).t().contiguous().cuda(), None if bf is None else bf.cuda(),
+                              cmap, h.reshape(G, K).cuda(), taps_reversed=True, flip_x1x2=flip, bx_from=L - (K - 1))
+    assert rel_err(y.permute(0, 2, 1), ref) <= 2e-2, (B, D, L, G, K, Ks, cs, il, flip, sbias)
+    if K > 1:
+        assert rel_err(bx.permute(0, 2, 1), (x1 * v)[..., L - (K - 1):]) <= 1e-2
