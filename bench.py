@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Hyena operator hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mr|se|li|decode] [--no-extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mr|se|li|decode|mr_cl|mr_layer|se_layer] [--no-extras]
 
 A "step" is one pass of the operator over one batch of synthetic input that is
 already resident in HBM.  The headline workload is the Hyena-MR prefill
@@ -34,7 +34,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="mr", choices=["mr", "se", "li", "decode"])
+    ap.add_argument("--workload", default="mr", choices=["mr", "se", "li", "decode", "mr_cl", "mr_layer", "se_layer"])
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-model", action="store_true", help="skip the end-to-end model prefill legs")
