@@ -44,3 +44,30 @@ def test_cpu_tensors_are_rejected():
     x = torch.zeros(1, 16, 8, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="GPU only"):
         va.hyena_se_fwd(x, x, x, torch.zeros(1, 1, 7))
+
+
+def test_new_entry_points_validate_before_touching_the_device():
+    # every call below is rejected by the argument checks; the dummy non-null pointers are never dereferenced
+    from vortex_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built in this tree")
+    L = _lib.lib()
+    P = 4096                      # aligned, non-null
+    cl = _lib.Cl(P, 64, 64)
+    ref = ctypes.byref
+    assert L.hyena_fir_cl_fwd(ref(cl), ref(cl), ref(cl), P, 0, None, 0, P, None, None, 0, 1, 8, 64, 4, 200, None) == -3
+    assert b"K=200" in L.hyena_last_error_string()
+    assert L.hyena_fir_cl_fwd(ref(cl), ref(cl), ref(cl), P, 0, None, 0, P, None, None, 0, 1, 8, 24, 3, 4, None) == -3
+    assert L.hyena_fir_cl_fwd(ref(cl), None, ref(cl), P, 0, None, 0, P, None, None, 0, 1, 8, 64, 4, 4, None) == -3
+    assert L.hyena_fir_cl_fwd(ref(_lib.Cl(P + 2, 64, 64)), None, None, P, 0, None, 0, P, None, None, 0, 1, 8, 64, 4,
+                              4, None) == -2
+    assert L.hyena_fir_cl_fwd(ref(cl), None, None, P, 0, None, 2, P, None, None, 0, 1, 8, 64, 4, 4, None) == -1
+    pj = _lib.ProjFwd(P, 192, 192, P, None, 5, 0, 64, 0, 64, 1)
+    assert L.hyena_fir_layer_fwd(ref(pj), P, 0, None, 0, P, None, 0, 1, 8, 64, 4, 7, None) == -3      # 5-tap featurizer
+    pj = _lib.ProjFwd(P, 192, 192, P, None, 3, 0, 64, 0, 80, 1)
+    assert L.hyena_fir_layer_fwd(ref(pj), P, 0, None, 0, P, None, 0, 1, 8, 64, 4, 7, None) == -1      # map past 3D
+    ps = _lib.ProjStep(P, 192, P, 0, 0, P, None, 64, 0, 64, 1, 0)
+    assert L.hyena_fir_layer_step(ref(ps), P, 6, 0, P, None, 0, P, 64, 1, 64, 4, None) == -1          # empty cache
+    ps = _lib.ProjStep(P, 192, P, 2, 0, P, None, 4, 12, 4, 1, 0)
+    assert L.hyena_fir_layer_step(ref(ps), P, 6, 0, P, None, 0, P, 64, 1, 64, 4, None) == -3          # head_dim 4
+    assert L.hyena_iir_layer_step(None, P, P, P, 0, P, 0, P, 0, 64, 1, 64, 64, 16, None) == -1
