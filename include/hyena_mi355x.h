@@ -106,11 +106,12 @@ int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v
  *   x1v = bf16(x1*v);  y = conv(h, x1v) in fp32;  out = bf16((bf16(y) + Dcoef*x1v) * x2)
  *   state_out[b][d][s] = sum_j p^(L-1-j) x1v[b][d][j]          (complex, (re, im) pairs)
  *
- * hyena_li_plan turns the modal parameters into the per-group coefficient tables the
- * kernel streams from (filter head, state-in and state-out matrices, p^128), evaluated
- * in double on the device.  log_poles and residues are [G][S][2] float32 (re, im) pairs;
- * real poles have im = 0.  The caller owns the workspace: hyena_li_plan_bytes(G, S)
- * bytes of device memory, reusable until the parameters change.  S must be 16.
+ * hyena_li_plan turns the modal parameters into a 6 KB per-group coefficient table, evaluated in double on
+ * the device: the filter head h[0..127], coarse and fine powers of every pole (p^(16a), p^b, r*p^b) and 1/p.
+ * Each wavefront of hyena_li_fwd expands its group's table once into the MFMA operand fragments it keeps in
+ * registers.  log_poles and residues are [G][S][2] float32 (re, im) pairs; real poles have im = 0.  The caller
+ * owns the workspace: hyena_li_plan_bytes(G, S) bytes of device memory, reusable until the parameters change.
+ * S must be 16.
  *
  * hyena_li_fwd: D/G must be a multiple of 16, L and strides multiples of 8.
  * y_conv_fp32 (optional, [B][D][L]) receives the fp32 convolution before any rounding;

@@ -41,16 +41,20 @@ constexpr int LRS = R2 + 4;              // row of chunk contributions: 32 float
 constexpr int XRS = R2 + 8;              // row of split states: 32 bf16 + 16 B pad
 constexpr int WAVE_LDS_BYTES = 2 * 4 * URS * 2 + 16 * LRS * 4 + 2 * 16 * XRS * 2;   // u, z, l, xh, xl
 
-// Workspace per group: 48 MFMA A-operand fragments, already split into bf16 hi / lo terms and laid
-// out per lane (64 lanes x 16 B each), then p^128 and p^-1.
+// The 48 MFMA A-operand fragments a wavefront keeps in registers (bf16 hi / lo terms, 16 B per lane each):
 //   [ 0.. 7] Toeplitz hi, index 2*delta + ib    [ 8..15] Toeplitz lo      (delta = 0..3 superblocks back)
 //   [16..23] Pout hi, index 2*Sigma + ib        [24..31] Pout lo
 //   [32..39] Pin  hi, index 4*mu + kappa        [40..47] Pin  lo
 constexpr int FR_T = 0, FR_PO = 16, FR_PI = 32, N_FRAG = 48;
-constexpr int WS_FRAG_FLOATS = N_FRAG * 64 * 4;    // 12288 dwords
-constexpr int WS_PC = WS_FRAG_FLOATS;              // [16][2]  p^128
-constexpr int WS_PINV = WS_PC + 2 * S;             // [16][2]  1/p
-constexpr int WS_GROUP = WS_PINV + 2 * S;          // 12352 floats
+// Workspace per group (floats), evaluated in double by the plan kernel.  Every power of a pole the fragments
+// need is one fp32 complex product of a coarse and a fine table entry, p^(16a+b) = P16[a] * P1[b]:
+constexpr int WS_HEAD = 0;                         // [128]        filter head h[0..127]
+constexpr int WS_P16 = WS_HEAD + C;                // [16][9][2]   p^(16a), a = 0..8  (a = 8: the chunk factor p^128)
+constexpr int WS_P1 = WS_P16 + S * 9 * 2;          // [16][16][2]  p^b
+constexpr int WS_R1 = WS_P1 + S * 16 * 2;          // [16][16][2]  r * p^b
+constexpr int WS_PINV = WS_R1 + S * 16 * 2;        // [16][2]      1/p
+constexpr int WS_GROUP = 1536;                     // 1472 used; 6 KB, a whole number of 16-byte lane loads
+static_assert(WS_PINV + 2 * S <= WS_GROUP, "workspace layout");
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) {
     union { u32x4 u; bf16x8 b; } c;
@@ -89,15 +93,10 @@ __device__ __forceinline__ void wave_sync() {
 __device__ __forceinline__ int li_sample(int ib, int m) { return 8 * (m >> 2) + 4 * ib + (m & 3); }
 
 // ------------------------------------------------------------------ plan kernel
-// One block per group; coefficients evaluated in double from the fp32 parameters, then cut into
-// the per-lane fragments the main kernel loads with one 16-byte read each.
-// 16x16x32 A operand: lane holds row m = lane & 15, k = 8*(lane >> 4) + e, e = 0..7.
+// One block per group; coefficients evaluated in double from the fp32 parameters.
 __global__ __launch_bounds__(256) void li_plan_kernel(const float* __restrict__ log_poles,   // [G][S][2]
                                                       const float* __restrict__ residues,    // [G][S][2]
                                                       float* __restrict__ ws) {
-    __shared__ float head[C];
-    __shared__ float pin[R2 * C];       // [row 2s+part][j]
-    __shared__ float pout[C * R2];      // [i][row 2s+part]
     const int g = blockIdx.x, tid = threadIdx.x;
     float* w = ws + (size_t)g * WS_GROUP;
     const float* lp = log_poles + (size_t)g * S * 2;
@@ -116,61 +115,42 @@ __global__ __launch_bounds__(256) void li_plan_kernel(const float* __restrict__ 
             ppow(s, tid, re, im);
             acc += (double)rs[2 * s] * re - (double)rs[2 * s + 1] * im;
         }
-        head[tid] = (float)acc;
+        w[WS_HEAD + tid] = (float)acc;
     }
-    for (int e = tid; e < S * C; e += 256) {        // Pin and Pout
-        const int s = e / C, j = e - s * C;
+    for (int e = tid; e < S * 9; e += 256) {        // coarse powers
+        const int s = e / 9, a = e - 9 * s;
         double re, im;
-        ppow(s, C - 1 - j, re, im);
-        pin[(2 * s) * C + j] = (float)re;
-        pin[(2 * s + 1) * C + j] = (float)im;
-        ppow(s, j + 1, re, im);                     // here j plays the role of the output sample i
+        ppow(s, 16 * a, re, im);
+        w[WS_P16 + 2 * e] = (float)re;
+        w[WS_P16 + 2 * e + 1] = (float)im;
+    }
+    {                                               // fine powers, plain and times the residue: 256 threads = 16 x 16
+        const int s = tid >> 4, b = tid & 15;
+        double re, im;
+        ppow(s, b, re, im);
+        w[WS_P1 + 2 * tid] = (float)re;
+        w[WS_P1 + 2 * tid + 1] = (float)im;
         const double rr = rs[2 * s], ri = rs[2 * s + 1];
-        pout[j * R2 + 2 * s] = (float)(rr * re - ri * im);            //  Re(r p^(i+1))
-        pout[j * R2 + 2 * s + 1] = (float)(-(rr * im + ri * re));     // -Im(r p^(i+1))
+        w[WS_R1 + 2 * tid] = (float)(rr * re - ri * im);
+        w[WS_R1 + 2 * tid + 1] = (float)(rr * im + ri * re);
     }
     if (tid < S) {
         double re, im;
-        ppow(tid, C, re, im);
-        w[WS_PC + 2 * tid] = (float)re;
-        w[WS_PC + 2 * tid + 1] = (float)im;
         ppow(tid, -1, re, im);
         w[WS_PINV + 2 * tid] = (float)re;
         w[WS_PINV + 2 * tid + 1] = (float)im;
     }
-    __syncthreads();
-    u32x4* fr = (u32x4*)w;
-    for (int e = tid; e < 24 * 64; e += 256) {      // 24 (hi, lo) fragment pairs
-        const int f = e >> 6, lane = e & 63;
-        const int m = lane & 15, qa = lane >> 4;
-        float val[8];
-        if (f < 8) {                                // Toeplitz: rows of (superblock Sigma, half ib) x inputs of block J
-            const int delta = f >> 1, ib = f & 1;   // delta = Sigma - J
+    for (int e = WS_PINV + 2 * S + tid; e < WS_GROUP; e += 256) w[e] = 0.f;
+}
+
+// (hi, lo) bf16 split of eight fp32 coefficients into two A-operand fragments
+__device__ __forceinline__ void li_split(const float* val, u32x4& ph, u32x4& pl) {
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const int lag = 32 * delta + li_sample(ib, m) - (8 * qa + k);
-                val[k] = (lag >= 0 && lag < C) ? head[lag] : 0.f;
-            }
-        } else if (f < 16) {                        // Pout rows of (Sigma, ib), all 32 state rows in one k-step
-            const int Sg = (f - 8) >> 1, ib = (f - 8) & 1;
-#pragma unroll
-            for (int k = 0; k < 8; ++k) val[k] = pout[(32 * Sg + li_sample(ib, m)) * R2 + 8 * qa + k];
-        } else {                                    // Pin state rows 16*mu + m, inputs 32*kappa + 8*qa + k
-            const int mu = (f - 16) >> 2, kp = (f - 16) & 3;
-#pragma unroll
-            for (int k = 0; k < 8; ++k) val[k] = pin[(16 * mu + m) * C + 32 * kp + 8 * qa + k];
-        }
-        u32x4 ph, pl;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const float a = val[2 * j], b = val[2 * j + 1];
-            const float ah = round_bf(a), bh = round_bf(b);
-            ph[j] = (__float_as_uint(ah) >> 16) | (__float_as_uint(bh) & 0xffff0000u);
-            pl[j] = pack_bf2(a - ah, b - bh);
-        }
-        const int base = f < 8 ? FR_T + f : (f < 16 ? FR_PO + (f - 8) : FR_PI + (f - 16));
-        fr[(base) * 64 + lane] = ph;
-        fr[(base + 8) * 64 + lane] = pl;
+    for (int j = 0; j < 4; ++j) {
+        const float a = val[2 * j], b = val[2 * j + 1];
+        const float ah = round_bf(a), bh = round_bf(b);
+        ph[j] = (__float_as_uint(ah) >> 16) | (__float_as_uint(bh) & 0xffff0000u);
+        pl[j] = pack_bf2(a - ah, b - bh);
     }
 }
 
@@ -213,22 +193,69 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     bf16_t* xh_w = (bf16_t*)(l_w + 16 * LRS);                  // [4][4][XRS]
     bf16_t* xl_w = xh_w + 16 * XRS;
 
-    // ---- A fragments: one 16-byte load each, pinned in registers for the whole kernel.  All 48 loads are issued
-    // before the first is pinned, so they overlap instead of paying one memory round trip each.
-    const u32x4* fr = (const u32x4*)ws + lane;
+    // ---- A fragments, built once per wavefront from the group's 6 KB coefficient table (staged in the
+    // wavefront's own LDS slice, which the main loop only uses afterwards) and pinned in registers.
+    // 16x16x32 A operand: lane holds row m = lane & 15, k = 8*(lane >> 4) + e, e = 0..7.
     bf16x8 Th[8], Tl[8], Poh[8], Pol[8], Pih[8], Pil[8];
     {
-        u32x4 t[N_FRAG];
+        float* tb = (float*)lds;
+        static_assert(WS_GROUP * 4 <= 2 * 4 * URS * 2, "coefficient table must fit the u / z rows");
 #pragma unroll
-        for (int i = 0; i < N_FRAG; ++i) t[i] = fr[i * 64];
+        for (int i = 0; i < WS_GROUP / 4 / 64; ++i)
+            ((f32x4*)tb)[i * 64 + lane] = ((const f32x4*)ws)[i * 64 + lane];
+        wave_sync();
+        const int m = lane & 15, qa = lane >> 4;
+        const float2* t16 = (const float2*)(tb + WS_P16);
+        const float2* t1 = (const float2*)(tb + WS_P1);
+        const float2* tr = (const float2*)(tb + WS_R1);
+        u32x4 th[N_FRAG];
+        float val[8];
 #pragma unroll
-        for (int i = 0; i < N_FRAG; ++i) asm volatile("" : "+v"(t[i]));
+        for (int f = 0; f < 8; ++f) {               // Toeplitz: rows of (superblock Sigma, half ib) x inputs of block J
+            const int delta = f >> 1, ib = f & 1;   // delta = Sigma - J
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int lag = 32 * delta + li_sample(ib, m) - (8 * qa + k);
+                const float hv = tb[WS_HEAD + (lag < 0 ? 0 : (lag >= C ? C - 1 : lag))];
+                val[k] = (lag >= 0 && lag < C) ? hv : 0.f;
+            }
+            li_split(val, th[FR_T + f], th[FR_T + 8 + f]);
+        }
+#pragma unroll
+        for (int f = 0; f < 8; ++f) {               // Pout: output sample i of (Sigma, ib) x state rows 8*qa + k
+            const int Sg = f >> 1, ib = f & 1;
+            const int e = 32 * Sg + li_sample(ib, m) + 1;          // Re / -Im of r * p^(i+1)
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const int s = 4 * qa + kk;
+                const float2 pa = t16[s * 9 + (e >> 4)], pb = tr[s * 16 + (e & 15)];
+                val[2 * kk] = pa.x * pb.x - pa.y * pb.y;
+                val[2 * kk + 1] = -(pa.x * pb.y + pa.y * pb.x);
+            }
+            li_split(val, th[FR_PO + f], th[FR_PO + 8 + f]);
+        }
+#pragma unroll
+        for (int f = 0; f < 8; ++f) {               // Pin: state row 16*mu + m x inputs 32*kappa + 8*qa + k
+            const int mu = f >> 2, kp = f & 3;
+            const int s = 8 * mu + (m >> 1);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int e = C - 1 - (32 * kp + 8 * qa + k);      // p^(127 - j)
+                const float2 pa = t16[s * 9 + (e >> 4)], pb = t1[s * 16 + (e & 15)];
+                const float re = pa.x * pb.x - pa.y * pb.y, im = pa.x * pb.y + pa.y * pb.x;
+                val[k] = (m & 1) ? im : re;
+            }
+            li_split(val, th[FR_PI + f], th[FR_PI + 8 + f]);
+        }
+#pragma unroll
+        for (int i = 0; i < N_FRAG; ++i) asm volatile("" : "+v"(th[i]));
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
-            Th[q] = as_bf16x8(t[FR_T + q]);   Tl[q] = as_bf16x8(t[FR_T + 8 + q]);
-            Poh[q] = as_bf16x8(t[FR_PO + q]); Pol[q] = as_bf16x8(t[FR_PO + 8 + q]);
-            Pih[q] = as_bf16x8(t[FR_PI + q]); Pil[q] = as_bf16x8(t[FR_PI + 8 + q]);
+            Th[q] = as_bf16x8(th[FR_T + q]);   Tl[q] = as_bf16x8(th[FR_T + 8 + q]);
+            Poh[q] = as_bf16x8(th[FR_PO + q]); Pol[q] = as_bf16x8(th[FR_PO + 8 + q]);
+            Pih[q] = as_bf16x8(th[FR_PI + q]); Pil[q] = as_bf16x8(th[FR_PI + 8 + q]);
         }
+        wave_sync();                                // the table's LDS rows are free for the main loop from here on
     }
 
     // MFMA-side lane geometry: column n = channel c + 4 * chunk s, k / row quad q
@@ -238,7 +265,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     const int sc = CPW == 4 ? (lane >> 4) : 0, sp = lane & 15;
     float Xr = 0.f, Xi = 0.f;
     float Xfr = 0.f, Xfi = 0.f;                                // state after the chunk that holds sample L-1
-    const float pcr = ws[WS_PC + 2 * sp], pci = ws[WS_PC + 2 * sp + 1];
+    const float pcr = ws[WS_P16 + 2 * (9 * sp + 8)], pci = ws[WS_P16 + 2 * (9 * sp + 8) + 1];   // p^128
     float dco = 0.f;
     if (a.Dcoef) dco = a.Dcoef[d0 + (CPW == 4 ? c : 0)];
 
