@@ -117,3 +117,30 @@ def test_proj_structs_match_header():
     assert _lib.ProjFwd.Ks.offset == 5 * 8 and _lib.ProjFwd.flip_x1x2.offset == 5 * 8 + 4
     assert _lib.ProjFwd.ch_inner.offset == 6 * 8
     assert ctypes.sizeof(_lib.Cl) == 3 * 8
+
+
+def test_from_vortex_shares_parameters_and_config():
+    # a stand-in with the attributes of vortex's HyenaCascade (vortex/model/model.py:125-210)
+    import types
+    from vortex_amd.cascade import HyenaCascade, use_hip_filters
+
+    class Cfg(dict):
+        __getattr__ = dict.__getitem__
+
+    cfg = Cfg(hidden_size=64, num_attention_heads=4, state_size=16, short_filter_length=3, short_filter_bias=False,
+              interleave=True, column_split_hyena=False, hyena_flip_x1x2=True)
+    ref = types.SimpleNamespace(config=cfg, layer_idx=3, hyena_filter_groups=4, fir_inner_filter_length=7,
+                                short_filter_weight=torch.nn.Parameter(torch.randn(192, 1, 3)), short_filter_bias=None,
+                                h=torch.nn.Parameter(torch.randn(4, 1, 7)), D=None)
+    m = HyenaCascade.from_vortex(ref)
+    assert m.h is ref.h and m.short_filter_weight is ref.short_filter_weight and m.D is None
+    assert (m.layer_idx, m.interleave, m.column_split_hyena, m.hyena_flip_x1x2) == (3, True, False, True)
+    modal = types.SimpleNamespace(config=cfg, layer_idx=5, hyena_filter_groups=64, fir_inner_filter_length=None,
+                                  short_filter_weight=torch.nn.Parameter(torch.randn(192, 1, 3)), short_filter_bias=None,
+                                  h=None, D=torch.nn.Parameter(torch.zeros(64)),
+                                  log_poles=torch.nn.Parameter(torch.randn(64, 16, 1)),
+                                  residues=torch.nn.Parameter(torch.randn(64, 16)))
+    blocks = [types.SimpleNamespace(filter=ref), types.SimpleNamespace(), types.SimpleNamespace(filter=modal)]
+    model = types.SimpleNamespace(blocks=blocks)
+    assert use_hip_filters(model) == 2 and use_hip_filters(model) == 0
+    assert isinstance(blocks[2].filter, HyenaCascade) and blocks[2].filter.log_poles is modal.log_poles

@@ -48,6 +48,19 @@ def _cfg(config, key, default=None):
     return default if v is None else v
 
 
+def use_hip_filters(model):
+    """Replaces the `filter` of every Hyena block of a vortex model (an object with `.blocks`, each Hyena block
+    holding its HyenaCascade as `.filter`, vortex/model/model.py:523-575) by its counterpart on the HIP kernels.
+    Returns the number of blocks switched."""
+    n = 0
+    for block in model.blocks:
+        f = getattr(block, "filter", None)
+        if f is not None and hasattr(f, "short_filter_weight") and not isinstance(f, HyenaCascade):
+            block.filter = HyenaCascade.from_vortex(f)
+            n += 1
+    return n
+
+
 class HyenaCascade(nn.Module):
     """Parameters and forward of one Hyena operator (SE / MR when fir_inner_filter_length is set, LI otherwise).
 
@@ -89,6 +102,20 @@ class HyenaCascade(nn.Module):
         self.fuse_decode = True        # one launch per decode step where the fused layer-step kernels apply
         self.fuse_prefill = True       # one launch per SE / MR prefill where the fused layer kernel applies
         self._f32_cache = {}
+
+    @classmethod
+    def from_vortex(cls, ref):
+        """A module on the HIP kernels with the configuration and the parameters (shared storage, not copied) of a
+        vortex HyenaCascade instance (vortex/model/model.py:125-210)."""
+        complex_modal = getattr(ref, "log_poles", None) is not None and ref.log_poles.is_complex()
+        new = cls(ref.config, ref.layer_idx, hyena_filter_groups=ref.hyena_filter_groups,
+                  fir_inner_filter_length=ref.fir_inner_filter_length, complex_modal=complex_modal)
+        for name in ("short_filter_weight", "short_filter_bias", "h", "D", "log_poles", "residues"):
+            p = getattr(ref, name, None)
+            if p is not None and not isinstance(p, nn.Parameter):
+                p = nn.Parameter(p, requires_grad=False)
+            setattr(new, name, p)
+        return new
 
     # ------------------------------------------------------------------
     def forward(self, u, inference_params=None, padding_mask=None, *args, **kwargs):
