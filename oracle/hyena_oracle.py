@@ -567,20 +567,20 @@ class OracleCascade:
         self.column_split_hyena, self.interleave, self.state_size = column_split_hyena, interleave, state_size
         self.Ks = params["short_filter_weight"].shape[-1]
 
-    def forward(self, u, inference_params=None):
+    def forward(self, u, inference_params=None, padding_mask=None):
         # model.py:214-219
         if inference_params is not None and self.layer_idx in inference_params.fir_state_dict.keys():
             return self.sequential_forward(u, inference_params)
-        return self.parallel_forward(u, inference_params)
+        return self.parallel_forward(u, inference_params, padding_mask)
 
-    def parallel_forward(self, u, inference_params=None):
+    def parallel_forward(self, u, inference_params=None, padding_mask=None):
         # model.py:221-316
         p, L = self.p, u.shape[1]
         dims = (self.hidden, self.n_heads, self.hidden // self.n_heads, self.state_size, self.groups)
         z_pre, fir_state = self.engine.parallel_fir(
             F.conv1d, u, p["short_filter_weight"], p.get("short_filter_bias"), L, dims=dims, gate=False,
             column_split_hyena=self.column_split_hyena, fir_length=self.Ks, inference_params=inference_params,
-            padding_mask=None, dim_last=True)
+            padding_mask=padding_mask, dim_last=True)
         if inference_params:
             inference_params.fir_state_dict[self.layer_idx] = fir_state
         if self.interleave:
@@ -596,7 +596,7 @@ class OracleCascade:
             y, inner = self.engine.parallel_fir(
                 F.conv1d, z_pre, h, p.get("D"), L, dims=dims, gate=True, gated_bias=self.K >= 128, dim_last=False,
                 column_split_hyena=self.column_split_hyena, fir_length=self.K, inference_params=inference_params,
-                padding_mask=None, groups=self.groups)
+                padding_mask=padding_mask, groups=self.groups)
             y = y.permute(0, 2, 1)
             if inference_params:
                 inference_params.fir_inner_state_dict[self.layer_idx] = inner
@@ -605,7 +605,7 @@ class OracleCascade:
                 z_pre, h, p["D"], L, t=None, poles=p["log_poles"], residues=p["residues"], dims=dims,
                 inference_params=inference_params, layer_idx=self.layer_idx, prefill_style="fft",
                 use_flashfft=False, fftconv_fn=None, column_split_hyena=self.column_split_hyena,
-                long_fir_threshold=None, padding_mask=None)
+                long_fir_threshold=None, padding_mask=padding_mask)
         return y, inference_params
 
     def sequential_forward(self, u, inference_params):

@@ -223,3 +223,36 @@ def test_two_pass_fwd_grouped_intermediates():
     hf = h.flip(-1)[:, 0]
     assert torch.equal(T.cpu(), O.toeplitz(hf, CH).bfloat16())
     assert torch.equal(T_hat.cpu(), O.correction_toeplitz(hf, CH).bfloat16())
+
+
+@pytest.mark.parametrize("kind", ["se", "mr", "li_real"])
+def test_operator_module_padding_mask(kind):
+    # left-padded batch: the 0/1 mask of vortex/model/engine.py:226-227 on both FIR outputs
+    B, L, D, H, G = 2, 384, 64, 4, 4
+    K = {"se": 7, "mr": 128}.get(kind)
+    p = make_params(kind, D, G, seed=21)
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=False, interleave=True, short_filter_length=3,
+               short_filter_bias=False, state_size=16)
+    mod = HyenaCascade(cfg, 0, hyena_filter_groups=G, fir_inner_filter_length=K)
+    with torch.no_grad():
+        mod.short_filter_weight.copy_(p["short_filter_weight"])
+        if K:
+            mod.h.copy_(p["h"])
+        else:
+            mod.log_poles.copy_(p["log_poles"])
+            mod.residues.copy_(p["residues"])
+        if mod.D is not None:
+            mod.D.data = p["D"].clone()
+    mod = mod.to(DEV)
+    if K is None:
+        pr = dict(p, log_poles=p["log_poles"].repeat_interleave(D // G, 0), residues=p["residues"].repeat_interleave(D // G, 0))
+        ref = O.OracleCascade(O.OracleEngine(), pr, D, H, D, interleave=True)
+    else:
+        ref = O.OracleCascade(O.OracleEngine(), p, D, H, G, fir_inner_filter_length=K, interleave=True)
+    u = torch.randn(B, L, 3 * D, generator=torch.Generator().manual_seed(4)).bfloat16()
+    mask = torch.ones(B, L)
+    mask[0, :37] = 0
+    mask[1, :5] = 0
+    y_ref, _ = ref.forward(u, None, padding_mask=mask)
+    y_hip, _ = mod(u.to(DEV), None, padding_mask=mask.to(DEV))
+    assert rel_err(y_hip, y_ref) <= 2e-2

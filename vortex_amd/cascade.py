@@ -164,15 +164,17 @@ class HyenaCascade(nn.Module):
 
     def parallel_forward(self, u, inference_params=None, padding_mask=None):
         """Prefill: u [B, L, 3D] bf16 -> y [B, L, D] bf16 (vortex/model/model.py:221-316)."""
-        if padding_mask is not None:
-            raise NotImplementedError("padding_mask is handled by the drop-in engine, not by this module")
+        masked = isinstance(padding_mask, torch.Tensor)
         B, L, C = u.shape
         D, Ks = self.hidden_size, self.short_filter_length
         caching = inference_params is not None
-        if self.fuse_prefill and self._can_fuse_prefill(u, L, caching):
+        if not masked and self.fuse_prefill and self._can_fuse_prefill(u, L, caching):
             return self._fused_prefill(u, inference_params), inference_params
         w = self._f32_param("short_filter_weight", (C, Ks))
         z_pre = ops.featurizer_fwd(u, w, self._f32_param("short_filter_bias"), interleave=self.interleave)
+        if masked:      # rare path (padded batches): the 0/1 mask of vortex/model/engine.py:226-227 through torch
+            mask = padding_mask[:, None].to(z_pre.dtype)
+            z_pre = z_pre * mask
         r1, r2, rv = self._rows(z_pre)
         K = self.fir_inner_filter_length
         if K:
@@ -182,6 +184,8 @@ class HyenaCascade(nn.Module):
                                      bias_mode=HYENA_BIAS_GATED_FP32, taps_reversed=False, force_mfma=True)
             else:
                 y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, K, device=u.device, taps_reversed=True)
+            if masked:
+                y = y * mask     # a 0/1 mask on the convolution commutes with the x2 gate
         else:
             y, _, state = ops.li_fwd_rows(r1, r2, rv, self.modal_plan(), self.D, B, D, L, device=u.device,
                                           want_state=caching)
