@@ -77,10 +77,14 @@ int hyena_se_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v
  * u: bf16, channels contiguous, sample t of batch b at u + b*u_batch_stride + t*u_time_stride.
  * taps: [G][K] float32 (G = C for vortex's per-channel short filter).  out: [B][C][L] bf16.
  * interleave3 != 0 also applies the channel de-interleave of vortex/model/utils.py:26-38
- * (input channel 3j+i is written to output row i*C/3 + j). */
+ * (input channel 3j+i is written to output row i*C/3 + j).
+ * front_pad (0..7) makes sequence lengths that are not a multiple of 8 usable by the sequence-major
+ * kernels: out is [B][C][L + front_pad] with front_pad leading zero columns (L + front_pad % 8 == 0).
+ * Zero samples ahead of a causal filter with zero history change nothing, so the operators run on
+ * L + front_pad samples and the caller drops the first front_pad outputs. */
 int hyena_featurizer_fwd(const void* u, int64_t u_batch_stride, int64_t u_time_stride,
                          const float* taps, const float* bias, int interleave3, void* out,
-                         int64_t B, int64_t L, int64_t C, int64_t G, int K, void* stream);
+                         int64_t B, int64_t L, int64_t C, int64_t G, int K, int front_pad, void* stream);
 
 /* Hyena-MR: gated causal depthwise FIR with 2 <= K <= 128 as a chunked,
  * block-Toeplitz contraction on bf16 MFMA with fp32 accumulation.

@@ -41,6 +41,8 @@ def to_dev(p):
 CASES = [
     # kind, B, L, D, heads, G(inner), column_split, interleave, short bias
     ("se", 2, 512, 64, 4, 4, False, True, False),
+    ("se", 1, 333, 64, 4, 4, False, True, True),          # lengths that are not multiples of 8
+    ("mr", 2, 509, 64, 4, 4, True, False, False),
     ("se", 1, 256, 64, 4, 4, True, False, True),
     ("mr", 2, 640, 64, 4, 4, False, True, False),
     ("mr", 1, 512, 32, 2, 2, True, False, False),
@@ -122,6 +124,46 @@ def test_engine_dropin_modal_layer_per_channel_filters(cs, il):
         y_ref, _ = ref.forward(tok, ip_ref)
         y_hip, _ = hip.forward(tok.to(DEV), ip_hip)
         assert rel_err(y_hip, y_ref) <= 2e-2, i
+
+
+@pytest.mark.parametrize("L", [517, 200])
+@pytest.mark.parametrize("kind", ["se", "mr", "li_real", "li_cplx"])
+def test_operator_module_any_prompt_length(kind, L):
+    # prompts whose length is not a multiple of 8, through prefill and two decode steps (fused and two-kernel paths)
+    B, D, H, G = 2, 64, 4, 4
+    K = {"se": 7, "mr": 128}.get(kind)
+    p = make_params(kind, D, G, seed=31)
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=False, interleave=True, short_filter_length=3,
+               short_filter_bias=False, state_size=16)
+    if K is None:
+        pr = dict(p, log_poles=p["log_poles"].repeat_interleave(D // G, 0), residues=p["residues"].repeat_interleave(D // G, 0))
+        ref = O.OracleCascade(O.OracleEngine(), pr, D, H, D, interleave=True)
+    else:
+        ref = O.OracleCascade(O.OracleEngine(), p, D, H, G, fir_inner_filter_length=K, interleave=True)
+    u_all = torch.randn(B, L + 2, 3 * D, generator=torch.Generator().manual_seed(L)).bfloat16()
+    for fused in (True, False):
+        mod = HyenaCascade(cfg, 0, hyena_filter_groups=G, fir_inner_filter_length=K, complex_modal=(kind == "li_cplx"))
+        with torch.no_grad():
+            mod.short_filter_weight.copy_(p["short_filter_weight"])
+            if K:
+                mod.h.copy_(p["h"])
+            else:
+                mod.log_poles.copy_(p["log_poles"])
+                mod.residues.copy_(p["residues"])
+            if mod.D is not None:
+                mod.D.data = p["D"].clone()
+        mod = mod.to(DEV)
+        mod.fuse_prefill = mod.fuse_decode = fused
+        ip_ref = O.OracleCache()
+        ip_hip = HyenaCascadeFIRInferenceParams() if K else HyenaCascadeIIRInferenceParams()
+        y_ref, _ = ref.forward(u_all[:, :L], ip_ref)
+        y_hip, _ = mod(u_all[:, :L].to(DEV), ip_hip)
+        assert y_hip.shape == (B, L, D) and rel_err(y_hip, y_ref) <= 2e-2
+        for i in range(2):
+            tok = u_all[:, L + i: L + i + 1]
+            y_ref, _ = ref.forward(tok, ip_ref)
+            y_hip, _ = mod(tok.to(DEV), ip_hip)
+            assert rel_err(y_hip, y_ref) <= 2e-2, (fused, i)
 
 
 @pytest.mark.parametrize("fused", [True, False])

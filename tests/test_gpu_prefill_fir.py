@@ -173,9 +173,10 @@ def test_se_nontemporal_variant_matches(monkeypatch):
 
 def test_argument_errors():
     x = torch.zeros(1, 32, 64, dtype=torch.bfloat16, device="cuda")
-    with pytest.raises(ValueError):                       # L not a multiple of 8
-        va.hyena_se_fwd(x[..., :60].contiguous(), x[..., :60].contiguous(), x[..., :60].contiguous(),
-                        torch.zeros(2, 1, 7, device="cuda"))
+    from vortex_amd import ops                            # the C ABI itself takes multiples of 8 samples only
+    r = ops.rows_of(x)
+    with pytest.raises(ValueError):
+        ops.fir_fwd_rows(r, r, r, torch.zeros(2, 7, device="cuda"), 1, 32, 60, 7, device=x.device)
     with pytest.raises(NotImplementedError):              # 8 channels per group: no MFMA tiling
         va.hyena_mr_fwd(x, x, x, torch.zeros(4, 1, 128, device="cuda"))
     with pytest.raises(NotImplementedError):              # K > 128

@@ -153,3 +153,38 @@ def test_fused_layer_random(B, L, seed, monkeypatch):
     assert rel_err(y.permute(0, 2, 1), ref) <= 2e-2, (B, D, L, G, K, Ks, cs, il, flip, sbias)
     if K > 1:
         assert rel_err(bx.permute(0, 2, 1), (x1 * v)[..., L - (K - 1):]) <= 1e-2
+
+
+@pytest.mark.parametrize("L", [1, 5, 63, 1001, 2049])
+def test_lengths_that_are_not_multiples_of_8(L):
+    # the tensor-level operators accept any length: they run behind -L % 8 zero samples (ops.front_pad8)
+    B, D, G = 2, 32, 2
+    x2, x1, v = O.make_gates(B, D, L, seed=L)
+    d = lambda t: t.cuda()
+    h = O.make_se_filter(G, 7, seed=L)
+    assert rel_err(va.hyena_se_fwd(d(x1), d(x2), d(v), d(h)), O.se_fir(x2, x1, v, h)[0]) <= 2e-2
+    hm = O.make_mr_filter(G, 128, seed=L)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(L))
+    assert rel_err(va.hyena_mr_fwd(d(x1), d(x2), d(v), d(hm), d(Db)), O.mr_fir(x2, x1, v, hm, Db)[0]) <= 2e-2
+    lp, r = O.make_modal_complex(G, 16, seed=L, pmax=0.999)
+    Dl = torch.randn(D, generator=torch.Generator().manual_seed(L + 1)).bfloat16()
+    ref, y32_ref, st_ref = O.li_prefill(x2, x1, v, lp, r, Dl)
+    out, y32, st = va.hyena_li_fwd(d(x1), d(x2), d(v), d(lp), d(r), d(Dl), want_state=True, want_fp32=True)
+    assert out.shape == (B, D, L) and y32.shape == (B, D, L)
+    assert rel_err(out, ref) <= 2e-2 and rel_err(y32, y32_ref) <= 1e-4
+    assert rel_err(torch.view_as_real(st), torch.view_as_real(st_ref)) <= 1e-4
+
+
+@pytest.mark.parametrize("L,bias", [(13, False), (250, True), (1021, False)])
+def test_featurizer_front_pad(L, bias):
+    B, C, K = 2, 96, 3
+    g = torch.Generator().manual_seed(L)
+    u = torch.randn(B, L, C, generator=g).bfloat16()
+    w = torch.randn(C, 1, K, generator=g) / K ** 0.5
+    b = torch.randn(C, generator=g).bfloat16() if bias else None
+    pad = (-L) % 8
+    z = ops.featurizer_fwd(u.cuda(), w.reshape(C, K).cuda(), None if b is None else b.cuda(), interleave=True,
+                           front_pad=pad)
+    ref, _ = O.parallel_fir(u, w, b, fir_length=K, dim_last=True, gate=False)
+    assert z.shape == (B, C, L + pad) and not z[..., :pad].any()
+    assert rel_err(z[..., pad:], O.interleave(ref)) <= 2e-2

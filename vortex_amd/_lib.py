@@ -71,7 +71,7 @@ def lib():
     L.hyena_li_fwd.argtypes = [R, R, R, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
                                c_int64, c_int64, c_int64, c_void_p]
     L.hyena_featurizer_fwd.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int64,
-                                       c_int64, c_int64, c_int64, c_int, c_void_p]
+                                       c_int64, c_int64, c_int64, c_int, c_int, c_void_p]
     L.hyena_copy_probe.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
     P = POINTER(ProjStep)
     L.hyena_fir_layer_step.argtypes = [P, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int64,

@@ -171,9 +171,13 @@ class HyenaCascade(nn.Module):
         if not masked and self.fuse_prefill and self._can_fuse_prefill(u, L, caching):
             return self._fused_prefill(u, inference_params), inference_params
         w = self._f32_param("short_filter_weight", (C, Ks))
-        z_pre = ops.featurizer_fwd(u, w, self._f32_param("short_filter_bias"), interleave=self.interleave)
+        # the sequence-major kernels take multiples of 8 samples: other lengths run behind -L % 8 zero samples
+        pad, L_true = (-L) % 8, L
+        L += pad
+        z_pre = ops.featurizer_fwd(u, w, self._f32_param("short_filter_bias"), interleave=self.interleave,
+                                   front_pad=pad)
         if masked:      # rare path (padded batches): the 0/1 mask of vortex/model/engine.py:226-227 through torch
-            mask = padding_mask[:, None].to(z_pre.dtype)
+            mask = torch.nn.functional.pad(padding_mask, (pad, 0))[:, None].to(z_pre.dtype)
             z_pre = z_pre * mask
         r1, r2, rv = self._rows(z_pre)
         K = self.fir_inner_filter_length
@@ -192,15 +196,17 @@ class HyenaCascade(nn.Module):
             if caching:
                 inference_params.state_dict[self.layer_idx] = state
         if caching:
-            if L < Ks - 1 or (K and L < K - 1):
+            if L_true < Ks - 1 or (K and L_true < K - 1):
                 raise NotImplementedError("prompts shorter than the filters are not supported by the cached path")
             # the channel-last tail of u is already the ring layout [B, R, 3D]
-            inference_params.fir_state_dict[self.layer_idx] = ops.FirRing(u[:, L - (Ks - 1):].contiguous(), 0)
+            inference_params.fir_state_dict[self.layer_idx] = ops.FirRing(u[:, L_true - (Ks - 1):].contiguous(), 0)
             if K:
                 _, x1, v = self._split(z_pre[..., L - (K - 1):])
                 inference_params.fir_inner_state_dict[self.layer_idx] = ops.FirRing(
                     (x1 * v).permute(0, 2, 1).contiguous(), 0)
             self._decode = None
+        if pad:
+            y = y[..., pad:]
         return y.permute(0, 2, 1), inference_params
 
     def _channel_map(self):

@@ -16,7 +16,8 @@ template <int K, bool BIAS>
 __global__ __launch_bounds__(256) void featurizer_kernel(const bf16_t* __restrict__ u, int64_t u_bs, int64_t u_ts,
                                                          const float* __restrict__ taps, int dg,
                                                          const float* __restrict__ bias, bf16_t* __restrict__ z,
-                                                         int64_t C, int64_t L, int interleave3) {
+                                                         int64_t C, int64_t L, int interleave3, int pad) {
+    // L counts output columns; column t holds input sample t - pad, the first `pad` columns are zeros
     constexpr int ROWS = TT + K - 1;
     constexpr int A_ELEMS = ROWS * TC, B_ELEMS = TC * TBP;
     __shared__ __attribute__((aligned(16))) bf16_t lds[A_ELEMS > B_ELEMS ? A_ELEMS : B_ELEMS];
@@ -27,9 +28,9 @@ __global__ __launch_bounds__(256) void featurizer_kernel(const bf16_t* __restric
     // phase 1: [time][channel] tile, rows t0-(K-1) .. t0+TT-1
     for (int e = tid; e < ROWS * (TC / 8); e += 256) {
         const int row = e / (TC / 8), lc = e - row * (TC / 8);
-        const int64_t t = t0 - (K - 1) + row, c = c0 + 8 * lc;
+        const int64_t t = t0 - (K - 1) + row - pad, c = c0 + 8 * lc;
         u32x4 q = {0, 0, 0, 0};
-        if (t >= 0 && t < L && c < C) q = *(const u32x4*)(ub + t * u_ts + c);
+        if (t >= 0 && t < L - pad && c < C) q = *(const u32x4*)(ub + t * u_ts + c);
         *(u32x4*)(lds + row * TC + 8 * lc) = q;
     }
     __syncthreads();
@@ -73,7 +74,11 @@ __global__ __launch_bounds__(256) void featurizer_kernel(const bf16_t* __restric
         }
         a0 = round_bf(a0);
         a1 = round_bf(a1);
-        if (BIAS) { a0 += b0; a1 += b1; }
+        if (BIAS) {
+            const bool live = t0 + tg * 32 + i >= pad;       // padding columns stay zero, bias or not
+            a0 = live ? a0 + b0 : 0.f;
+            a1 = live ? a1 + b1 : 0.f;
+        }
         if (i & 1) {
             o0[i >> 1] = pack_bf2(__uint_as_float(o0[i >> 1]), a0);
             o1[i >> 1] = pack_bf2(__uint_as_float(o1[i >> 1]), a1);
@@ -110,15 +115,17 @@ __global__ __launch_bounds__(256) void featurizer_kernel(const bf16_t* __restric
 
 extern "C" int hyena_featurizer_fwd(const void* u, int64_t u_batch_stride, int64_t u_time_stride, const float* taps,
                                     const float* bias, int interleave3, void* out, int64_t B, int64_t L, int64_t C,
-                                    int64_t G, int K, void* stream) {
+                                    int64_t G, int K, int front_pad, void* stream) {
     if (!u || !taps || !out) return hyena_fail(HYENA_EINVAL, "hyena_featurizer_fwd: u, taps and out are required");
     if (B < 0 || L < 0 || C <= 0 || G <= 0 || C % G != 0)
         return hyena_fail(HYENA_EINVAL, "hyena_featurizer_fwd: bad sizes B=%lld L=%lld C=%lld G=%lld", (long long)B,
                           (long long)L, (long long)C, (long long)G);
     if (K < 2 || K > 8) return hyena_fail(HYENA_ENOSUP, "hyena_featurizer_fwd: K=%d outside 2..8", K);
+    if (front_pad < 0 || front_pad > 7) return hyena_fail(HYENA_EINVAL, "hyena_featurizer_fwd: front_pad %d outside 0..7", front_pad);
+    if (L > 0) L += front_pad;            // from here on L counts output columns
     if (C % 8 != 0 || L % 8 != 0 || u_batch_stride % 8 != 0 || u_time_stride % 8 != 0 || ((uintptr_t)u & 15) ||
         ((uintptr_t)out & 15))
-        return hyena_fail(HYENA_EALIGN, "hyena_featurizer_fwd: C, L, strides must be multiples of 8, pointers 16-byte aligned");
+        return hyena_fail(HYENA_EALIGN, "hyena_featurizer_fwd: C, L + front_pad, strides must be multiples of 8, pointers 16-byte aligned");
     if (interleave3 && C % 3 != 0) return hyena_fail(HYENA_EINVAL, "hyena_featurizer_fwd: interleave needs C %% 3 == 0");
     if (B > 65535 || (L + TT - 1) / TT > 65535) return hyena_fail(HYENA_EINVAL, "hyena_featurizer_fwd: grid too large");
     if (B == 0 || L == 0) return 0;
@@ -129,10 +136,10 @@ extern "C" int hyena_featurizer_fwd(const void* u, int64_t u_batch_stride, int64
     case KK:                                                                                                        \
         if (bias)                                                                                                   \
             hipLaunchKernelGGL((featurizer_kernel<KK, true>), grid, dim3(256), 0, s, (const bf16_t*)u,              \
-                               u_batch_stride, u_time_stride, taps, dg, bias, (bf16_t*)out, C, L, interleave3);                  \
+                               u_batch_stride, u_time_stride, taps, dg, bias, (bf16_t*)out, C, L, interleave3, front_pad);                  \
         else                                                                                                        \
             hipLaunchKernelGGL((featurizer_kernel<KK, false>), grid, dim3(256), 0, s, (const bf16_t*)u,             \
-                               u_batch_stride, u_time_stride, taps, dg, bias, (bf16_t*)out, C, L, interleave3);                  \
+                               u_batch_stride, u_time_stride, taps, dg, bias, (bf16_t*)out, C, L, interleave3, front_pad);                  \
         break;
     switch (K) { FZ_CASE(2) FZ_CASE(3) FZ_CASE(4) FZ_CASE(5) FZ_CASE(6) FZ_CASE(7) FZ_CASE(8) }
 #undef FZ_CASE

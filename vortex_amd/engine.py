@@ -55,7 +55,9 @@ class HyenaInferenceEngine:
                 raise NotImplementedError("gated FIR expects the [B, 3D, L] layout (dim_last=False)")
             B, _, L = u.shape
             hd = head_dim if column_split_hyena else None
-            r2, r1, rv = (ops.rows_of_projection(u, hidden, i, hd) for i in range(3))
+            up, pad = ops.front_pad8(u)                 # a copy only for lengths / strides the kernels cannot take
+            L += pad
+            r2, r1, rv = (ops.rows_of_projection(up, hidden, i, hd) for i in range(3))
             if self.hyena_flip_x1x2:
                 r1, r2 = r2, r1
             D = hidden
@@ -71,6 +73,8 @@ class HyenaInferenceEngine:
                 mode = HYENA_BIAS_NONE if bias is None else HYENA_BIAS_ADD
                 z = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, taps.shape[1], device=u.device,
                                      bias=ops._f32(bias), bias_mode=mode, taps_reversed=True)
+            if pad:
+                z = z[..., pad:]
             state = None
             if inference_params is not None:
                 x1, v = self._gate_tails(u, hidden, hd, K - 1)
@@ -82,14 +86,20 @@ class HyenaInferenceEngine:
             if dim_last:
                 B, L, C = u.shape
                 taps = _group_taps(weight, C, groups)
-                z = ops.featurizer_fwd(u, taps, bias)                      # [B, C, L], fused transpose
+                pad = (-L) % 8
+                z = ops.featurizer_fwd(u, taps, bias, front_pad=pad)       # [B, C, L + pad], fused transpose
+                if pad:
+                    z = z[..., pad:]
                 ut = u.permute(0, 2, 1)
             else:
                 B, C, L = u.shape
                 taps = _group_taps(weight, C, groups)
                 mode = HYENA_BIAS_NONE if bias is None else HYENA_BIAS_ADD
-                z = ops.fir_fwd_rows(ops.rows_of(u), None, None, taps, B, C, L, taps.shape[1], device=u.device,
+                up, pad = ops.front_pad8(u)
+                z = ops.fir_fwd_rows(ops.rows_of(up), None, None, taps, B, C, L + pad, taps.shape[1], device=u.device,
                                      bias=ops._f32(bias), bias_mode=mode, taps_reversed=True)
+                if pad:
+                    z = z[..., pad:]
                 ut = u
             state = ut[..., -K + 1:] if inference_params is not None else None
         if isinstance(padding_mask, torch.Tensor):
@@ -129,15 +139,18 @@ class HyenaInferenceEngine:
         hidden, n_heads, head_dim = dims[0], dims[1], dims[2]
         B, _, L = z_pre.shape
         hd = head_dim if column_split_hyena else None
-        r2, r1, rv = (ops.rows_of_projection(z_pre, hidden, i, hd) for i in range(3))
+        zp, pad = ops.front_pad8(z_pre)
+        r2, r1, rv = (ops.rows_of_projection(zp, hidden, i, hd) for i in range(3))
         if self.hyena_flip_x1x2:
             r1, r2 = r2, r1
         plan = self._plan(poles, residues)
         want_state = inference_params is not None
-        out, _, state = ops.li_fwd_rows(r1, r2, rv, plan, D, B, hidden, L, device=z_pre.device,
+        out, _, state = ops.li_fwd_rows(r1, r2, rv, plan, D, B, hidden, L + pad, device=z_pre.device,
                                         want_state=want_state)
         if want_state:
             inference_params.state_dict[layer_idx] = state
+        if pad:
+            out = out[..., pad:]
         return out.permute(0, 2, 1)
 
     # ------------------------------------------------------------------ decode

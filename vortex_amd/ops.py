@@ -64,6 +64,26 @@ def _f32(t, shape=None):
     return t
 
 
+def front_pad8(t):
+    """Makes a [B, D, L] bf16 tensor usable by the sequence-major kernels: (tensor, pad).
+
+    The kernels move 8 samples (16 bytes) per lane, so rows must start 16-byte aligned and hold a multiple
+    of 8 samples.  A tensor that already does is returned as is (pad = 0); otherwise it is copied behind
+    pad = -L % 8 zero columns.  Zero samples ahead of a causal filter with zero history change neither the
+    later outputs nor the final modal state, so callers run on L + pad samples and drop the first pad outputs.
+    """
+    B, D, L = t.shape
+    pad = (-L) % 8
+    if pad == 0 and (L <= 1 or t.stride(2) == 1) and t.stride(1) % 8 == 0 and t.stride(0) % 8 == 0 \
+            and t.data_ptr() % 16 == 0:
+        return t, 0
+    buf = torch.empty((B, D, L + pad), dtype=t.dtype, device=t.device)
+    if pad:
+        buf[..., :pad] = 0
+    buf[..., pad:] = t
+    return buf, pad
+
+
 def _bias_mode(bias, gated, fp32_gated):
     if bias is None:
         return HYENA_BIAS_NONE
@@ -176,8 +196,10 @@ def hyena_se_fwd(x1, x2, v, h, bias=None, *, force_mfma=False):
     taps = _f32(h).reshape(h.shape[0], -1)
     K = taps.shape[1]
     b = _f32(bias)
-    return fir_fwd_rows(rows_of(x1), rows_of(x2), rows_of(v), taps, B, D, L, K, device=x1.device, bias=b,
-                        bias_mode=_bias_mode(b, False, False), taps_reversed=True, force_mfma=force_mfma)
+    (x1, pad), (x2, _), (v, _) = front_pad8(x1), front_pad8(x2), front_pad8(v)
+    out = fir_fwd_rows(rows_of(x1), rows_of(x2), rows_of(v), taps, B, D, L + pad, K, device=x1.device, bias=b,
+                       bias_mode=_bias_mode(b, False, False), taps_reversed=True, force_mfma=force_mfma)
+    return out[..., pad:] if pad else out
 
 
 def hyena_mr_fwd(x1, x2, v, h, D_bias=None):
@@ -191,29 +213,32 @@ def hyena_mr_fwd(x1, x2, v, h, D_bias=None):
     taps = _f32(h).reshape(h.shape[0], -1)
     K = taps.shape[1]
     b = _f32(D_bias)
-    return fir_fwd_rows(rows_of(x1), rows_of(x2), rows_of(v), taps, B, D, L, K, device=x1.device, bias=b,
-                        bias_mode=_bias_mode(b, True, True), taps_reversed=False, force_mfma=True)
+    (x1, pad), (x2, _), (v, _) = front_pad8(x1), front_pad8(x2), front_pad8(v)
+    out = fir_fwd_rows(rows_of(x1), rows_of(x2), rows_of(v), taps, B, D, L + pad, K, device=x1.device, bias=b,
+                       bias_mode=_bias_mode(b, True, True), taps_reversed=False, force_mfma=True)
+    return out[..., pad:] if pad else out
 
 
-def featurizer_fwd(u, taps, bias=None, interleave=False):
-    """Featurizer short FIR on the channel-last projection: u [B, L, C] bf16 -> z [B, C, L] bf16.
+def featurizer_fwd(u, taps, bias=None, interleave=False, front_pad=0):
+    """Featurizer short FIR on the channel-last projection: u [B, L, C] bf16 -> z [B, C, L + front_pad] bf16.
 
     taps: [G, K] float32 in vortex's short-filter orientation (taps[:, K-1] on the current
     sample), G = C or a divisor of C.  bias: [C] or None (added after the bf16 rounding of the
     convolution, vortex/model/engine.py:208-223).  interleave=True also applies
-    vortex/model/utils.py:26-38 (channels 0::3 | 1::3 | 2::3) while writing.
+    vortex/model/utils.py:26-38 (channels 0::3 | 1::3 | 2::3) while writing.  front_pad = -L % 8 leading zero
+    columns make a length that is not a multiple of 8 usable by the sequence-major kernels (see front_pad8).
     """
     _need_cuda(u, taps)
     if u.dtype != torch.bfloat16 or u.dim() != 3 or u.stride(2) != 1:
         raise ValueError("expected a [B, L, C] bfloat16 tensor with contiguous channels")
     B, L, C = u.shape
     taps = _f32(taps)
-    out = torch.empty((B, C, L), dtype=torch.bfloat16, device=u.device)
+    out = torch.empty((B, C, L + front_pad), dtype=torch.bfloat16, device=u.device)
     if out.numel() == 0:
         return out
     b = _f32(bias)
     rc = _lib.lib().hyena_featurizer_fwd(_ptr(u), u.stride(0), u.stride(1), _ptr(taps), _ptr(b), int(interleave), _ptr(out),
-                                         B, L, C, taps.shape[0], taps.shape[1], _stream())
+                                         B, L, C, taps.shape[0], taps.shape[1], front_pad, _stream())
     _lib.check(rc, "hyena_featurizer_fwd")
     return out
 
@@ -277,8 +302,12 @@ def hyena_li_fwd(x1, x2, v, log_poles, residues, D_bias=None, *, plan=None, want
     B, D, L = x1.shape
     if plan is None:
         plan = ModalPlan(log_poles, residues)
-    return li_fwd_rows(rows_of(x1), rows_of(x2), rows_of(v), plan, D_bias, B, D, L, device=x1.device,
-                       want_state=want_state, want_fp32=want_fp32, single_rounding=single_rounding)
+    (x1, pad), (x2, _), (v, _) = front_pad8(x1), front_pad8(x2), front_pad8(v)
+    out, y32, state = li_fwd_rows(rows_of(x1), rows_of(x2), rows_of(v), plan, D_bias, B, D, L + pad, device=x1.device,
+                                  want_state=want_state, want_fp32=want_fp32, single_rounding=single_rounding)
+    if pad:
+        out, y32 = out[..., pad:], (y32[..., pad:] if y32 is not None else None)
+    return out, y32, state
 
 
 class FirRing:
