@@ -126,10 +126,11 @@ def test_engine_dropin_modal_layer_per_channel_filters(cs, il):
         assert rel_err(y_hip, y_ref) <= 2e-2, i
 
 
-@pytest.mark.parametrize("L", [517, 200])
+@pytest.mark.parametrize("L", [517, 200, 40, 3, 1])
 @pytest.mark.parametrize("kind", ["se", "mr", "li_real", "li_cplx"])
 def test_operator_module_any_prompt_length(kind, L):
-    # prompts whose length is not a multiple of 8, through prefill and two decode steps (fused and two-kernel paths)
+    # prompts whose length is not a multiple of 8, or shorter than the filters (the reference then grows its caches
+    # step by step, engine.py:443-444), through prefill and decode steps (fused and two-kernel paths)
     B, D, H, G = 2, 64, 4, 4
     K = {"se": 7, "mr": 128}.get(kind)
     p = make_params(kind, D, G, seed=31)
@@ -140,7 +141,8 @@ def test_operator_module_any_prompt_length(kind, L):
         ref = O.OracleCascade(O.OracleEngine(), pr, D, H, D, interleave=True)
     else:
         ref = O.OracleCascade(O.OracleEngine(), p, D, H, G, fir_inner_filter_length=K, interleave=True)
-    u_all = torch.randn(B, L + 2, 3 * D, generator=torch.Generator().manual_seed(L)).bfloat16()
+    n_dec = 2 if L > 100 else 6
+    u_all = torch.randn(B, L + n_dec, 3 * D, generator=torch.Generator().manual_seed(L)).bfloat16()
     for fused in (True, False):
         mod = HyenaCascade(cfg, 0, hyena_filter_groups=G, fir_inner_filter_length=K, complex_modal=(kind == "li_cplx"))
         with torch.no_grad():
@@ -159,7 +161,7 @@ def test_operator_module_any_prompt_length(kind, L):
         y_ref, _ = ref.forward(u_all[:, :L], ip_ref)
         y_hip, _ = mod(u_all[:, :L].to(DEV), ip_hip)
         assert y_hip.shape == (B, L, D) and rel_err(y_hip, y_ref) <= 2e-2
-        for i in range(2):
+        for i in range(n_dec):
             tok = u_all[:, L + i: L + i + 1]
             y_ref, _ = ref.forward(tok, ip_ref)
             y_hip, _ = mod(tok.to(DEV), ip_hip)

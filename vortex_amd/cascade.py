@@ -43,6 +43,32 @@ class HyenaCascadeFIRInferenceParams:
         self.fir_filter_length, self.fir_inner_filter_length, self.seqlen_offset = 3, 4, 0
 
 
+def _ring(tail, depth, flipped=False):
+    """FirRing of `depth` slots from the channel-last tail [B, n <= depth, C] of a prompt.
+
+    A prompt shorter than the filter leaves the oldest slots zero and records how many are real (`valid`).
+    With the flipped (Hyena-MR) tap slicing of vortex/model/engine.py:421-422 the reference's growing cache is
+    exactly this zero history.  With the plain slicing (:424-425) it is not: the reference then puts tap
+    `cache` on the new sample; _grown_taps reproduces that while the cache fills up."""
+    n = tail.shape[1]
+    if n < depth:
+        tail = torch.cat([tail.new_zeros(tail.shape[0], depth - n, tail.shape[2]), tail], dim=1)
+    ring = ops.FirRing(tail.contiguous(), 0)
+    ring.valid = depth if flipped else n
+    return ring
+
+
+def _grown_taps(w, valid):
+    """Taps [G, R+1] (oldest first) the reference applies to a cache holding `valid` < R samples with the plain
+    slicing weight[..., :valid+1] (vortex/model/engine.py:424-425): tap i on the i-th oldest real sample, tap
+    `valid` on the new one.  Laid out for a full-depth ring whose R - valid oldest slots are zero."""
+    R = w.shape[1] - 1
+    t = torch.zeros_like(w)
+    t[:, R - valid:R] = w[:, :valid]
+    t[:, R] = w[:, valid]
+    return t
+
+
 def _cfg(config, key, default=None):
     v = config.get(key, default) if hasattr(config, "get") else getattr(config, key, default)
     return default if v is None else v
@@ -196,14 +222,12 @@ class HyenaCascade(nn.Module):
             if caching:
                 inference_params.state_dict[self.layer_idx] = state
         if caching:
-            if L_true < Ks - 1 or (K and L_true < K - 1):
-                raise NotImplementedError("prompts shorter than the filters are not supported by the cached path")
             # the channel-last tail of u is already the ring layout [B, R, 3D]
-            inference_params.fir_state_dict[self.layer_idx] = ops.FirRing(u[:, L_true - (Ks - 1):].contiguous(), 0)
+            inference_params.fir_state_dict[self.layer_idx] = _ring(u[:, max(L_true - (Ks - 1), 0):], Ks - 1)
             if K:
-                _, x1, v = self._split(z_pre[..., L - (K - 1):])
-                inference_params.fir_inner_state_dict[self.layer_idx] = ops.FirRing(
-                    (x1 * v).permute(0, 2, 1).contiguous(), 0)
+                _, x1, v = self._split(z_pre[..., max(L - (K - 1), pad):])
+                inference_params.fir_inner_state_dict[self.layer_idx] = _ring((x1 * v).permute(0, 2, 1), K - 1,
+                                                                              flipped=K >= 128)
             self._decode = None
         if pad:
             y = y[..., pad:]
@@ -220,8 +244,6 @@ class HyenaCascade(nn.Module):
         if not K or K > 128 or self.short_filter_length not in (3, 4) or self._channel_map() is None:
             return False
         if (D // self.hyena_filter_groups) % 16 or D % 8 or (self.column_split_hyena and hd % 8):
-            return False
-        if caching and (L < K - 1 or L < self.short_filter_length - 1):
             return False
         return u.stride(2) == 1 and u.stride(1) % 8 == 0 and u.stride(0) % 8 == 0 and u.data_ptr() % 16 == 0
 
@@ -240,12 +262,12 @@ class HyenaCascade(nn.Module):
         res = ops.fir_layer_fwd(u, hit[1], self._f32_param("short_filter_bias"), self._channel_map(), taps,
                                 bias=self._f32_param("D") if mr else None,
                                 bias_mode=HYENA_BIAS_GATED_FP32 if mr else HYENA_BIAS_NONE, taps_reversed=not mr,
-                                flip_x1x2=self.hyena_flip_x1x2, bx_from=L - (K - 1) if caching else None)
+                                flip_x1x2=self.hyena_flip_x1x2, bx_from=max(L - (K - 1), 0) if caching else None)
         if not caching:
             return res
         y, bx = res
-        inference_params.fir_state_dict[self.layer_idx] = ops.FirRing(u[:, L - (Ks - 1):].contiguous(), 0)
-        inference_params.fir_inner_state_dict[self.layer_idx] = ops.FirRing(bx, 0)
+        inference_params.fir_state_dict[self.layer_idx] = _ring(u[:, max(L - (Ks - 1), 0):], Ks - 1)
+        inference_params.fir_inner_state_dict[self.layer_idx] = _ring(bx, K - 1, flipped=mr)
         self._decode = None
         return y
 
@@ -292,12 +314,44 @@ class HyenaCascade(nn.Module):
         return ops.LayerStepper(ring, self.short_filter_weight.detach().reshape(3 * self.hidden_size, Ks),
                                 self.short_filter_bias, cmap, inner, flip_x1x2=self.hyena_flip_x1x2)
 
+    def _growing_step(self, u, d):
+        """Decode step while a cache still holds fewer samples than its filter needs (prompt shorter than the
+        filter): the reference's tap slicing for that case, with tap tables rebuilt per step."""
+        B, D = u.shape[0], self.hidden_size
+
+        def fir(stepper, x1, x2, v, out):
+            ring = stepper.ring
+            valid, R = getattr(ring, "valid", stepper.R), stepper.R
+            if valid < R:
+                full = stepper.w
+                stepper.w = _grown_taps(full, valid)
+                stepper(x1, x2, v, out)
+                stepper.w = full
+                ring.valid = valid + 1
+            else:
+                stepper(x1, x2, v, out)
+
+        z_pre = torch.empty(B, 3 * D, dtype=torch.bfloat16, device=u.device)
+        fir(d["feat"], u.contiguous(), None, None, z_pre)
+        if self.interleave:
+            z_pre = z_pre[:, d["perm"]]
+        x2, x1, v = (t.contiguous() for t in self._split(z_pre))
+        y = torch.empty(B, D, dtype=torch.bfloat16, device=u.device)
+        if self.fir_inner_filter_length:
+            fir(d["inner"], x1, x2, v, y)
+        else:
+            d["inner"](x1, x2, v, y)
+        return y[:, None]
+
     def sequential_forward(self, u, inference_params):
         """Decode: u [B, 3D] or [B, 1, 3D] bf16 -> y [B, 1, D] (vortex/model/model.py:318-375)."""
         if u.dim() > 2:
             u = u[:, -1]
         d = self._decode_plan(inference_params)
         B = u.shape[0]
+        rings = [d["ring"]] + ([d["inner"].ring] if self.fir_inner_filter_length else [])
+        if any(getattr(r, "valid", r.buf.shape[1]) < r.buf.shape[1] for r in rings):
+            return self._growing_step(u, d), inference_params
         if self.fuse_decode and d["layer"] is not None and u.stride(1) == 1 and u.stride(0) % 8 == 0 and u.data_ptr() % 16 == 0:
             y = torch.empty(B, self.hidden_size, dtype=torch.bfloat16, device=u.device)
             d["layer"](u, y)
