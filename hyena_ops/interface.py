@@ -65,9 +65,11 @@ def _gcg(x, k, q, h, bias, apply_gated_bias):
     taps = ops._f32(h).reshape(h.shape[0], -1)
     K = taps.shape[1]
     mode = HYENA_BIAS_NONE if bias is None else (HYENA_BIAS_GATED_FP32 if apply_gated_bias else HYENA_BIAS_ADD)
-    return ops.fir_fwd_rows(ops.rows_of(x), ops.rows_of(q), ops.rows_of(k), taps, B, D, L, K, device=x.device,
-                            bias=ops._f32(bias), bias_mode=mode, taps_reversed=True,
-                            force_mfma=(K > 8 or mode == HYENA_BIAS_GATED_FP32))
+    (x, pad), (k, _), (q, _) = ops.front_pad8(x), ops.front_pad8(k), ops.front_pad8(q)     # any length, any strides
+    y = ops.fir_fwd_rows(ops.rows_of(x), ops.rows_of(q), ops.rows_of(k), taps, B, D, L + pad, K, device=x.device,
+                         bias=ops._f32(bias), bias_mode=mode, taps_reversed=True,
+                         force_mfma=(K > 8 or mode == HYENA_BIAS_GATED_FP32))
+    return y[..., pad:] if pad else y
 
 
 def _cl_ok(x, h):
@@ -129,8 +131,11 @@ def causal_conv1d_ref(x, weight, bias=None, apply_gated_bias=False, return_final
     mode = HYENA_BIAS_NONE if bias is None else (HYENA_BIAS_GATED_FP32 if apply_gated_bias else HYENA_BIAS_ADD)
     if mode == HYENA_BIAS_GATED_FP32 or K > 8:
         raise NotImplementedError("ungated FIR with per-channel taps is limited to K <= 8 without gated bias")
-    out = ops.fir_fwd_rows(ops.rows_of(x), None, None, ops._f32(weight).reshape(D, K), B, D, L, K, device=x.device,
-                           bias=ops._f32(bias), bias_mode=mode, taps_reversed=True)
+    xp, pad = ops.front_pad8(x)
+    out = ops.fir_fwd_rows(ops.rows_of(xp), None, None, ops._f32(weight).reshape(D, K), B, D, L + pad, K,
+                           device=x.device, bias=ops._f32(bias), bias_mode=mode, taps_reversed=True)
+    if pad:
+        out = out[..., pad:]
     return out if not return_final_states else (out, final_states_out)
 
 

@@ -248,6 +248,21 @@ def test_featurizer_full_width():
     assert (z.cpu() == ref).float().mean() > 0.98
 
 
+def test_hyena_ops_any_length():
+    from hyena_ops import interface as I
+    B, L, G, dg, K = 2, 203, 2, 16, 5
+    gen = torch.Generator().manual_seed(8)
+    x, k, q = (torch.randn(B, G * dg, L, generator=gen).bfloat16() for _ in range(3))
+    h = O.make_se_filter(G, K)
+    ref = O.se_fir(q, k, x, h)[0]
+    assert rel_err(I.inner_hyena_se(x.to(DEV), k.to(DEV), q.to(DEV), h.to(DEV)), ref) <= 2e-2
+    w = h.repeat_interleave(dg, 0)[:, 0]
+    assert rel_err(I.causal_conv1d_ref(x.to(DEV), w.to(DEV)), O.short_fir_fp32(x, w[:, None], K).bfloat16()) <= 2e-2
+    xl, kl, ql = (t.permute(0, 2, 1).reshape(B, L, G, dg).contiguous() for t in (x, k, q))
+    y = I.two_pass_chunked_gate_conv_gate(xl.to(DEV), kl.to(DEV), ql.to(DEV), h.to(DEV))
+    assert rel_err(y.reshape(B, L, G * dg).permute(0, 2, 1), ref) <= 2e-2
+
+
 def test_two_pass_fwd_grouped_intermediates():
     # (y, T, T_hat, y2, bx_lag) of vortex/ops/hyena_se/fwd.py:290 on (b, l, g, dg) tensors, channel-last kernel
     from hyena_ops import interface as I
