@@ -160,8 +160,8 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
         const int64_t g0 = dblk / dg;
         const int64_t gmax = (D + dg - 1) / dg;
         if ((W & 3) == 0) {
-            for (int e = tid; e < (W / 4) * ng; e += 64 * NSG) {
-                const int gl2 = e / (W / 4), i4 = (e - gl2 * (W / 4)) * 4;
+            for (int e = tid; e < (W / 4) * ng; e += 64 * NSG) {      // groups fastest: conflict-free LDS stores
+                const int i4 = (e / ng) * 4, gl2 = e - (e / ng) * ng;
                 f32x4 t = {0.f, 0.f, 0.f, 0.f};
                 if (g0 + gl2 < gmax) t = *(const f32x4*)(w + (g0 + gl2) * W + i4);
 #pragma unroll
@@ -169,7 +169,7 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
             }
         } else {
             for (int e = tid; e < W * ng; e += 64 * NSG) {
-                const int gl2 = e / W, i = e - gl2 * W;
+                const int i = e / ng, gl2 = e - i * ng;
                 wl[i * ng + gl2] = (g0 + gl2 < gmax) ? w[(g0 + gl2) * W + i] : 0.f;
             }
         }
