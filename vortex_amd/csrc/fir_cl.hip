@@ -113,6 +113,10 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
 
     // ---- this lane's I/O block: rows 4*rb .. 4*rb+3 of the step, channels d0 + 8*cb .. +7
     const int cb = tid & 7, rb = tid >> 3;
+    // Inside a 128-sample chunk the samples of channel slab j (16 channels) sit at position t ^ 32*j.  Both LDS
+    // row strides are 32 banks modulo 64 per 8 channels, so without this the 8-byte transposed accesses of the
+    // lanes cb = 0, 2, 4, 6 (and 1, 3, 5, 7) would fall on the same banks; a slab's own MFMA reads are unaffected.
+    const int swz_io = 32 * (cb >> 1), swz_mm = 32 * w;
     const uint32_t dch = d0 + 8 * cb;
     const bool ch_ok = dch < (uint32_t)D;
     const bf16_t* pp[NP];
@@ -270,7 +274,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
 
         // ---- (c) 4 x 8 transpose into the ring chunk `cur`
         {
-            bf16_t* ub = u_lds + (8 * cb) * URS + cur * TL + 4 * rb;
+            bf16_t* ub = u_lds + (8 * cb) * URS + cur * TL + ((4 * rb) ^ swz_io);
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
                 u32x2 t2;
@@ -298,7 +302,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             const int c0 = 64 * s + 8 * hh + (cur ^ 1) * TL;     // ring position of the halo chunk's first sample
 #pragma unroll
             for (int mm = MLO; mm < 12; ++mm) {
-                const bf16x8 bf = *(const bf16x8*)(urow + ((c0 + 16 * mm) & (2 * TL - 1)));
+                const bf16x8 bf = *(const bf16x8*)(urow + (((c0 + 16 * mm) & (2 * TL - 1)) ^ swz_mm));
                 if (mm <= 9) acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm <= 9 ? mm - MLO : 0], bf, acc0, 0, 0, 0);
                 if (mm - 2 >= MLO) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm - 2 >= MLO ? mm - 2 - MLO : 0], bf, acc1, 0, 0, 0);
                 if ((mm & 3) == 3) __builtin_amdgcn_sched_barrier(0);    // at most four B fragments in registers at a time
@@ -309,8 +313,8 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                 const f32x16 acc = tau ? acc1 : acc0;
                 u32x4 ua = {0, 0, 0, 0}, ub2 = {0, 0, 0, 0};
                 if (BIAS == HYENA_BIAS_GATED_FP32) {
-                    ua = *(const u32x4*)(urow + cur * TL + tcol);
-                    ub2 = *(const u32x4*)(urow + cur * TL + tcol + 8);
+                    ua = *(const u32x4*)(urow + cur * TL + (tcol ^ swz_mm));
+                    ub2 = *(const u32x4*)(urow + cur * TL + (tcol ^ swz_mm) + 8);
                 }
                 u32x4 z0, z1;
 #pragma unroll
@@ -328,8 +332,8 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                     const uint32_t p = pack_bf2(a0, a1);
                     if (j < 4) z0[j] = p; else z1[j - 4] = p;
                 }
-                *(u32x4*)(z_lds + (16 * w + c) * ZRS + tcol) = z0;
-                *(u32x4*)(z_lds + (16 * w + c) * ZRS + tcol + 8) = z1;
+                *(u32x4*)(z_lds + (16 * w + c) * ZRS + (tcol ^ swz_mm)) = z0;
+                *(u32x4*)(z_lds + (16 * w + c) * ZRS + (tcol ^ swz_mm) + 8) = z1;
             }
         }
         __syncthreads();
@@ -342,7 +346,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
         if (compute && ch_ok) {
             u32x2 zc[8];
 #pragma unroll
-            for (int c = 0; c < 8; ++c) zc[c] = *(const u32x2*)(z_lds + (8 * cb + c) * ZRS + 4 * rb);
+            for (int c = 0; c < 8; ++c) zc[c] = *(const u32x2*)(z_lds + (8 * cb + c) * ZRS + ((4 * rb) ^ swz_io));
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int64_t t = ts + 4 * rb + q;
