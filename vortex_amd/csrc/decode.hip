@@ -102,7 +102,7 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
 
     const int ng = GROUPED ? (512 / dg) : 0;
     float* wl = smem;                       // [W][ng]  taps of the block's groups, transposed
-    float* red = smem + (GROUPED ? W * ng : 0);   // [NSG-1][64][8]
+    float* red = smem + (GROUPED ? W * ng : 0);   // [NSG-1][2][64][4]
     const int gl = GROUPED ? (oc * 8) / dg : 0;
     constexpr int UF = 8;                   // cache slots in flight per lane
     const bf16_t* rb = ring + (b * R) * D + d0;
@@ -183,14 +183,14 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
     }
     if (sg > 0) {
 #pragma unroll
-        for (int c = 0; c < 8; ++c) red[((sg - 1) * 64 + oc) * 8 + c] = acc[c];
+        for (int c = 0; c < 8; ++c) red[(((sg - 1) * 2 + (c >> 2)) * 64 + oc) * 4 + (c & 3)] = acc[c];   // 16 B per lane, lanes contiguous
     }
     __syncthreads();          // also orders every read of slot `pos` before its overwrite below
     if (sg != 0 || !live) return;
 #pragma unroll
     for (int k = 0; k < NSG - 1; ++k)
 #pragma unroll
-        for (int c = 0; c < 8; ++c) acc[c] += red[(k * 64 + oc) * 8 + c];
+        for (int c = 0; c < 8; ++c) acc[c] += red[((k * 2 + (c >> 2)) * 64 + oc) * 4 + (c & 3)];
 
     u32x4 a1, av = {0, 0, 0, 0}, a2 = {0, 0, 0, 0};
     if (FEAT != 0) {
