@@ -228,11 +228,13 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
 }
 
 // ---------------------------------------------------------------- IIR step
-// LPB lanes share one (batch, channel): each holds 16 bytes of its modal state
-// (4 real or 2 complex states), so state traffic is fully coalesced.  The
-// residue-weighted sum is reduced with xor shuffles inside the lane group.
+// LPB lanes share one channel: each holds 16 bytes of its modal state (4 real or 2 complex
+// states), so state traffic is fully coalesced.  A lane walks NB batch elements of that channel
+// with the poles and residues held in registers and the NB state loads issued together, which
+// puts enough bytes in flight to cover HBM latency.  The residue-weighted sum is reduced with
+// xor shuffles inside the lane group.
 // FEAT: lanes 0..2 of a lane group evaluate the fused featurizer step for gates x2, x1, v of their channel.
-template <int S, bool CPLX, bool FEAT>
+template <int S, bool CPLX, bool FEAT, int NB>
 __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict__ x1, const bf16_t* __restrict__ x2,
                                                        const bf16_t* __restrict__ v, int64_t in_bs, ProjArgs pj,
                                                        float* __restrict__ state, const float* __restrict__ poles,
@@ -240,71 +242,82 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
                                                        const float* __restrict__ Dcoef, int d_is_bf16,
                                                        void* __restrict__ out, int out_is_fp32, int64_t out_bs,
                                                        int64_t B, int64_t D, int dg) {
-    constexpr int LPB = CPLX ? S / 2 : S / 4;      // lanes per (b, d)
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int q = (int)(idx % LPB);
-    int64_t bd = idx / LPB;
-    const bool live = bd < B * D;
-    if (!live) bd = 0;
-    const int64_t b = bd / D, d = bd - b * D;
-    const int64_t g = d / dg;
+    constexpr int LPB = CPLX ? S / 2 : S / 4;      // lanes per channel
     constexpr int FPS = CPLX ? 2 : 1;              // floats per state
-    float* sp = state + (bd * S) * FPS + q * 4;
-    const f32x4 st = *(const f32x4*)sp;
-    const f32x4 pp = *(const f32x4*)(poles + (g * S) * FPS + q * 4);
-    const f32x4 rr = *(const f32x4*)(residues + (g * S) * FPS + q * 4);
-    float a, c, gate2 = 0.f;
-    if (FEAT) {
-        static_assert(!FEAT || LPB >= 4, "the fused featurizer needs three lanes per channel");
-        float z = 0.f;
-        if (q < 3) {
-            const uint32_t ch = pj.chan((uint32_t)q, (uint32_t)d);
-            bf16_t* rb = pj.ring + (b * pj.Rf) * pj.C + ch;
-            const bf16_t un = pj.u[b * pj.u_bs + ch];
-            float acc = 0.f;
-            for (int i = 0; i < pj.Rf; ++i) {
-                int s = pj.pos + i;
-                if (s >= pj.Rf) s -= pj.Rf;
-                acc = fmaf(pj.w[(int64_t)i * pj.C + ch], bf_to_f(rb[(int64_t)s * pj.C]), acc);
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;        // (channel, lane of the group)
+    const int q = (int)(idx % LPB);
+    uint32_t d = idx / LPB;
+    const bool chan_live = d < (uint32_t)D;
+    if (!chan_live) d = 0;
+    const int64_t b0 = (int64_t)blockIdx.y * NB;
+    const uint32_t g = d / (uint32_t)dg;
+    f32x4 st[NB];
+    bool live[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        live[j] = chan_live && b0 + j < B;
+        const int64_t bd = live[j] ? (b0 + j) * D + d : 0;
+        st[j] = *(const f32x4*)(state + (bd * S) * FPS + q * 4);
+    }
+    const f32x4 pp = *(const f32x4*)(poles + ((int64_t)g * S) * FPS + q * 4);
+    const f32x4 rr = *(const f32x4*)(residues + ((int64_t)g * S) * FPS + q * 4);
+    const float dco = Dcoef[d];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int64_t b = live[j] ? b0 + j : 0;
+        float a, c, gate2 = 0.f;
+        if (FEAT) {
+            static_assert(!FEAT || LPB >= 4, "the fused featurizer needs three lanes per channel");
+            float z = 0.f;
+            if (q < 3) {
+                const uint32_t ch = pj.chan((uint32_t)q, d);
+                bf16_t* rb = pj.ring + (b * pj.Rf) * pj.C + ch;
+                const bf16_t un = pj.u[b * pj.u_bs + ch];
+                float acc = 0.f;
+                for (int i = 0; i < pj.Rf; ++i) {
+                    int s = pj.pos + i;
+                    if (s >= pj.Rf) s -= pj.Rf;
+                    acc = fmaf(pj.w[(int64_t)i * pj.C + ch], bf_to_f(rb[(int64_t)s * pj.C]), acc);
+                }
+                acc = fmaf(pj.w[(int64_t)pj.Rf * pj.C + ch], bf_to_f(un), acc);
+                if (pj.bias) acc += pj.bias[ch];
+                z = round_bf(acc);
+                if (live[j]) rb[(int64_t)pj.pos * pj.C] = un;
             }
-            acc = fmaf(pj.w[(int64_t)pj.Rf * pj.C + ch], bf_to_f(un), acc);
-            if (pj.bias) acc += pj.bias[ch];
-            z = round_bf(acc);
-            if (live) rb[(int64_t)pj.pos * pj.C] = un;
+            const int base = (threadIdx.x & 63) & ~(LPB - 1);
+            const float g2 = __shfl(z, base, 64), g1 = __shfl(z, base + 1, 64);
+            c = __shfl(z, base + 2, 64);
+            a = pj.flip ? g2 : g1;
+            gate2 = pj.flip ? g1 : g2;
+        } else {
+            a = bf_to_f(x1[b * in_bs + d]);
+            c = bf_to_f(v[b * in_bs + d]);
         }
-        const int base = (threadIdx.x & 63) & ~(LPB - 1);
-        const float g2 = __shfl(z, base, 64), g1 = __shfl(z, base + 1, 64);
-        c = __shfl(z, base + 2, 64);
-        a = pj.flip ? g2 : g1;
-        gate2 = pj.flip ? g1 : g2;
-    } else {
-        a = bf_to_f(x1[b * in_bs + d]);
-        c = bf_to_f(v[b * in_bs + d]);
-    }
-    const float x1v = round_bf(a * c);
-    f32x4 ns;
-    float part;
-    if (CPLX) {
-        // (pr + i pi)(sr + i si) + x1v
-        ns[0] = fmaf(pp[0], st[0], -pp[1] * st[1]) + x1v;
-        ns[1] = fmaf(pp[0], st[1], pp[1] * st[0]);
-        ns[2] = fmaf(pp[2], st[2], -pp[3] * st[3]) + x1v;
-        ns[3] = fmaf(pp[2], st[3], pp[3] * st[2]);
-        part = (rr[0] * ns[0] - rr[1] * ns[1]) + (rr[2] * ns[2] - rr[3] * ns[3]);   // Re(r*s)
-    } else {
+        const float x1v = round_bf(a * c);
+        f32x4 ns;
+        float part;
+        if (CPLX) {
+            // (pr + i pi)(sr + i si) + x1v
+            ns[0] = fmaf(pp[0], st[j][0], -pp[1] * st[j][1]) + x1v;
+            ns[1] = fmaf(pp[0], st[j][1], pp[1] * st[j][0]);
+            ns[2] = fmaf(pp[2], st[j][2], -pp[3] * st[j][3]) + x1v;
+            ns[3] = fmaf(pp[2], st[j][3], pp[3] * st[j][2]);
+            part = (rr[0] * ns[0] - rr[1] * ns[1]) + (rr[2] * ns[2] - rr[3] * ns[3]);   // Re(r*s)
+        } else {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) ns[k] = fmaf(pp[k], st[k], x1v);
-        part = (rr[0] * ns[0] + rr[1] * ns[1]) + (rr[2] * ns[2] + rr[3] * ns[3]);
-    }
-    if (live) *(f32x4*)sp = ns;
+            for (int k = 0; k < 4; ++k) ns[k] = fmaf(pp[k], st[j][k], x1v);
+            part = (rr[0] * ns[0] + rr[1] * ns[1]) + (rr[2] * ns[2] + rr[3] * ns[3]);
+        }
+        if (live[j]) *(f32x4*)(state + (((b0 + j) * D + d) * S) * FPS + q * 4) = ns;
 #pragma unroll
-    for (int m = 1; m < LPB; m <<= 1) part += __shfl_xor(part, m, 64);
-    if (live && q == 0) {
-        float dx = Dcoef[d] * x1v;
-        if (d_is_bf16) dx = round_bf(dx);
-        const float y = (FEAT ? gate2 : bf_to_f(x2[b * in_bs + d])) * (part + dx);
-        if (out_is_fp32) ((float*)out)[b * out_bs + d] = y;
-        else ((bf16_t*)out)[b * out_bs + d] = (bf16_t)f_to_bf_bits(y);
+        for (int m = 1; m < LPB; m <<= 1) part += __shfl_xor(part, m, 64);
+        if (live[j] && q == 0) {
+            float dx = dco * x1v;
+            if (d_is_bf16) dx = round_bf(dx);
+            const float y = (FEAT ? gate2 : bf_to_f(x2[b * in_bs + d])) * (part + dx);
+            if (out_is_fp32) ((float*)out)[b * out_bs + d] = y;
+            else ((bf16_t*)out)[b * out_bs + d] = (bf16_t)f_to_bf_bits(y);
+        }
     }
 }
 
@@ -436,20 +449,26 @@ static int iir_step_launch(const void* x1, const void* x2, const void* v, int64_
     if (B == 0) return 0;
     const int dg = (int)(D / G);
     const int lpb = is_complex ? (int)S / 2 : (int)S / 4;
-    const int64_t nthr = B * D * lpb;
-    dim3 grid((unsigned)((nthr + 255) / 256));
+    if (D * lpb > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: D too large", who);
+    // four batch elements per lane when that still leaves a few wavefronts per SIMD; else one
+    const int nb = (B >= 4 && B * D * lpb >= 4 * 256 * 1024) ? 4 : 1;
+    const int64_t gy = (B + nb - 1) / nb;
+    if (gy > 65535) return hyena_fail(HYENA_EINVAL, "%s: B too large", who);
+    dim3 grid((unsigned)((D * lpb + 255) / 256), (unsigned)gy);
     hipStream_t s = (hipStream_t)stream;
     const bf16_t *p1 = (const bf16_t*)x1, *p2 = (const bf16_t*)x2, *pv = (const bf16_t*)v;
     const bool feat = proj != nullptr;
+#define IIR_GO(SS, C, F, N)                                                                                     \
+    hipLaunchKernelGGL((iir_step_kernel<SS, C, F, N>), grid, dim3(256), 0, s, p1, p2, pv, in_bs, pj, state,     \
+                       poles, residues, Dcoef, d_is_bf16, out, out_is_fp32, out_bs, B, D, dg)
 #define IIR_CASE(SS, C, F)                                                                                      \
-    if (S == SS && (is_complex != 0) == C && feat == F)                                                         \
-        hipLaunchKernelGGL((iir_step_kernel<SS, C, F>), grid, dim3(256), 0, s, p1, p2, pv, in_bs, pj, state,    \
-                           poles, residues, Dcoef, d_is_bf16, out, out_is_fp32, out_bs, B, D, dg);
+    if (S == SS && (is_complex != 0) == C && feat == F) { if (nb == 4) IIR_GO(SS, C, F, 4); else IIR_GO(SS, C, F, 1); }
     IIR_CASE(8, false, false) IIR_CASE(16, false, false) IIR_CASE(32, false, false)
     IIR_CASE(8, true, false) IIR_CASE(16, true, false) IIR_CASE(32, true, false)
     IIR_CASE(16, false, true) IIR_CASE(32, false, true)
     IIR_CASE(8, true, true) IIR_CASE(16, true, true) IIR_CASE(32, true, true)
 #undef IIR_CASE
+#undef IIR_GO
     return hyena_check_launch(who);
 }
 
