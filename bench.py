@@ -211,6 +211,34 @@ def model_prefill(device, L, iters=2):
     return {"workload": f"striped_hyena2_7b_shaped_prefill B=1 L={L}", "tokens_per_s": L / dt, "ms": dt * 1e3}
 
 
+def model_decode(device, L=8192, n=32):
+    """Cached generation with the same Evo 2 7B-shaped stack: one prefill over L tokens (untimed), then n single-token
+    forwards at batch 1 (Hyena layers: one fused layer-step launch each; attention from its key / value cache)."""
+    from vortex_amd.model import StripedHyena2
+    m = StripedHyena2(device=device).to_inference(device)
+    ids = torch.randint(0, 512, (1, L), device=device, generator=torch.Generator(device=device).manual_seed(8))
+    ipd = m.initialize_inference_params(max_seqlen=L + n + 4)
+    x = m(ids, ipd)[:, -1].argmax(-1)[:, None]
+
+    def step(x):
+        for p in ipd.values():
+            p.seqlen_offset = L if p.seqlen_offset == 0 else p.seqlen_offset + 1
+        return m(x, ipd)[:, -1].argmax(-1)[:, None]
+
+    for _ in range(3):
+        x = step(x)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n):
+        x = step(x)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / n
+    del m, ipd
+    torch.cuda.empty_cache()
+    return {"workload": f"striped_hyena2_7b_shaped_decode B=1 prompt={L}", "ms_per_token": dt * 1e3,
+            "tokens_per_s": 1.0 / dt}
+
+
 def cpu_baseline(name):
     """The oracle (a PyTorch port of the reference path) timed on the host cores, on a channel slice."""
     from oracle import hyena_oracle as O
@@ -316,6 +344,7 @@ def main():
         if not args.no_model:
             for L in (8192, 131072):
                 extra[f"model_L{L}"] = model_prefill(device, L)
+            extra["model_decode"] = model_decode(device)
         result["extra"] = extra
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(main_name)

@@ -30,3 +30,21 @@ def test_hyena_blocks_are_batch_invariant_bitwise():
         a, _ = blk.filter(z)
         b, _ = blk.filter(z.repeat(3, 1, 1))
         assert torch.equal(a[0], b[1])
+
+
+@pytest.mark.parametrize("L", [256, 203])
+def test_cached_generation_matches_a_longer_prefill(L):
+    # generation order of vortex/model/generation.py:164-229: prefill, then one token per forward from the caches
+    # (FIR rings, modal states, attention keys / values).  Teacher-forced, so every step's logits can be compared
+    # with one prefill over prompt + continuation.
+    cfg = dict(EVO2_7B, hidden_size=128, num_layers=8, num_attention_heads=4, inner_mlp_size=256,
+               hcs_filter_groups=8, hcm_filter_groups=8, hcl_filter_groups=128)
+    m = StripedHyena2(cfg, seed=5, device="cuda").to_inference("cuda")
+    n = 6
+    ids = torch.randint(0, 512, (2, L + n), device="cuda", generator=torch.Generator(device="cuda").manual_seed(6))
+    full = m(ids).float()                                  # logits at every position of the long sequence
+    toks, scores = m.generate(ids[:, :L], n, forced=ids[:, L:])
+    assert torch.equal(toks, ids[:, L:])
+    want = full[:, L - 1:L + n - 1]                        # step i predicts token L + i from position L + i - 1
+    err = (scores.float() - want).abs().max() / want.abs().max()
+    assert err <= 3e-2, err                                # bf16 GEMM / SDPA paths differ between prefill and decode

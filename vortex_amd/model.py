@@ -69,11 +69,20 @@ def _rotary(x, base, offset=0):
     return torch.cat([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1)
 
 
+class AttentionInferenceParams:
+    """Key / value cache of the attention blocks (the role of vortex/model/cache.py:8-28): per layer two
+    [B, max_seqlen, H, head_dim] tensors, filled up to seqlen_offset."""
+
+    def __init__(self, max_seqlen):
+        self.max_seqlen, self.seqlen_offset = max_seqlen, 0
+        self.key_value_memory_dict = {}
+
+
 class AttentionBlock(nn.Module):
     def __init__(self, cfg, layer_idx):
         super().__init__()
         D, H = cfg["hidden_size"], cfg["num_attention_heads"]
-        self.H, self.base = H, cfg["rotary_emb_base"]
+        self.H, self.base, self.layer_idx = H, cfg["rotary_emb_base"], layer_idx
         self.pre_norm, self.post_norm = RMSNorm(D, cfg["eps"]), RMSNorm(D, cfg["eps"])
         self.Wqkv = nn.Linear(D, 3 * D, bias=False)
         self.out_proj = nn.Linear(D, D, bias=True)
@@ -82,8 +91,19 @@ class AttentionBlock(nn.Module):
     def forward(self, u, inference_params=None):
         B, L, D = u.shape
         qkv = self.Wqkv(self.pre_norm(u)).view(B, L, 3, self.H, D // self.H)
-        q, k, v = _rotary(qkv[:, :, 0], self.base), _rotary(qkv[:, :, 1], self.base), qkv[:, :, 2]
-        o = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True)
+        cached = inference_params is not None and self.layer_idx in inference_params.key_value_memory_dict
+        off = inference_params.seqlen_offset if cached else 0
+        q, k, v = _rotary(qkv[:, :, 0], self.base, off), _rotary(qkv[:, :, 1], self.base, off), qkv[:, :, 2]
+        if inference_params is not None:
+            if not cached:
+                kc = k.new_empty(B, inference_params.max_seqlen, self.H, D // self.H)
+                inference_params.key_value_memory_dict[self.layer_idx] = (kc, torch.empty_like(kc))
+            kc, vc = inference_params.key_value_memory_dict[self.layer_idx]
+            kc[:, off:off + L], vc[:, off:off + L] = k, v
+            if cached:              # decode: the new queries see the whole cache (one token: no mask needed)
+                k, v = kc[:, :off + L], vc[:, :off + L]
+        o = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
+                                           is_causal=not cached)
         u = self.out_proj(o.transpose(1, 2).reshape(B, L, D)) + u
         return self.mlp(self.post_norm(u)) + u, None
 
@@ -152,16 +172,36 @@ class StripedHyena2(nn.Module):
                 p.data = p.data.to(torch.bfloat16)
         return self.eval()
 
-    def initialize_inference_params(self):
+    def initialize_inference_params(self, max_seqlen=8192):
         """vortex/model/model.py:796-830: one cache object per operator family."""
         return {"hcl": HyenaCascadeIIRInferenceParams(), "hcm": HyenaCascadeFIRInferenceParams(),
-                "hcs": HyenaCascadeFIRInferenceParams()}
+                "hcs": HyenaCascadeFIRInferenceParams(), "mha": AttentionInferenceParams(max_seqlen)}
 
     @torch.no_grad()
     def forward(self, input_ids, inference_params_dict=None):
         x = self.embedding(input_ids)
         for kind, block in zip(self.kinds, self.blocks):
-            ip = None if inference_params_dict is None or kind == "attn" else inference_params_dict[kind]
+            ip = None if inference_params_dict is None else inference_params_dict["mha" if kind == "attn" else kind]
             x, _ = block(x, inference_params=ip)
         x = self.norm(x)
         return x @ self.embedding.weight.T
+
+    @torch.no_grad()
+    def generate(self, input_ids, num_tokens, forced=None):
+        """Greedy cached generation in the order of vortex/model/generation.py:164-229: one prefill over the
+        prompt, then one token per forward with the caches' seqlen_offset advanced first.  `forced`
+        [B, num_tokens] replaces the sampled tokens (teacher forcing).  Returns (tokens, logits of every step)."""
+        B, L = input_ids.shape
+        ipd = self.initialize_inference_params(max_seqlen=L + num_tokens)
+        x, toks, scores = input_ids, [], []
+        for i in range(num_tokens):
+            if i > 0:
+                x = x[:, -1:]
+                for p in ipd.values():
+                    p.seqlen_offset = L if p.seqlen_offset == 0 else p.seqlen_offset + 1
+            logits = self.forward(x, ipd)[:, -1]
+            new = logits.argmax(-1) if forced is None else forced[:, i]
+            toks.append(new)
+            scores.append(logits)
+            x = new[:, None]
+        return torch.stack(toks, 1), torch.stack(scores, 1)
