@@ -124,3 +124,68 @@ def test_layer_step_rejects_bad_maps():
         ops.LayerStepper(fring, wf, None, (D, 0, D + 8, 1), inner)(u, y)
     with pytest.raises(NotImplementedError):  # head_dim not a multiple of 8 has no vector kernel
         ops.LayerStepper(fring, wf, None, (4, 12, 4, 1), inner)(u, y)
+
+
+def _random_cases(seed, n):
+    import random
+    rng = random.Random(seed)
+    out = []
+    for _ in range(n):
+        H = rng.choice([1, 2, 4])
+        hd = 8 * rng.randint(1, 6)
+        D = H * hd
+        out.append((rng.randint(1, 5), D, H, rng.choice([2, 3, 4]), rng.choice(["plain", "split", "interleave"]),
+                    rng.random() < 0.5, rng.random() < 0.5, rng.randint(0, 10 ** 6)))
+    return out
+
+
+@pytest.mark.parametrize("B,D,H,Ks,layout,flip,sbias,seed", _random_cases(11, 16))
+def test_layer_steps_random(B, D, H, Ks, layout, flip, sbias, seed):
+    # both fused layer steps on random channel maps, cache depths and group sizes, several tokens in a row
+    import random
+    rng = random.Random(seed)
+    g = torch.Generator().manual_seed(seed)
+    C = 3 * D
+    cs, il = layout == "split", layout == "interleave"
+    wf = torch.randn(C, 1, Ks, generator=g) / Ks ** 0.5
+    bf = torch.randn(C, generator=g) if sbias else None
+    cmap = ops.gate_channel_map(D, interleave=il, head_dim=D // H if cs else None)
+    # FIR layer: per-channel taps or 8-channel groups, short or long cache
+    K = rng.choice([3, 7, 40, 128])
+    G = D if rng.random() < 0.5 else D // 8
+    mr = K == 128
+    w = torch.randn(G, 1, K, generator=g) / K ** 0.5
+    bias = torch.randn(D, generator=g) if mr else None
+    fst, st = torch.randn(B, C, Ks - 1, generator=g).bfloat16(), torch.randn(B, D, K - 1, generator=g).bfloat16()
+    fring, ring = va.FirRing.from_reference(fst.to(DEV)), va.FirRing.from_reference(st.to(DEV))
+    taps = (w.reshape(G, K).flip(-1) if mr else w.reshape(G, K)).contiguous().to(DEV)
+    fir = ops.LayerStepper(fring, wf.reshape(C, Ks).to(DEV), None if bf is None else bf.to(DEV), cmap,
+                           ops.FirStepper(ring, taps, bias=None if bias is None else bias.to(DEV), gated_bias=mr),
+                           flip_x1x2=flip)
+    # IIR layer on the same projections
+    S = rng.choice([16, 32])
+    cplx = rng.random() < 0.5
+    lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(D, S, seed=seed % 1000)
+    Dc = torch.randn(D, generator=g).bfloat16()
+    s0 = torch.randn(B, D, S, generator=g)
+    s0 = torch.complex(s0, torch.randn(B, D, S, generator=g)) if cplx else s0
+    state, fring2 = s0.clone().to(DEV), va.FirRing.from_reference(fst.to(DEV))
+    iir = ops.LayerStepper(fring2, wf.reshape(C, Ks).to(DEV), None if bf is None else bf.to(DEV), cmap,
+                           ops.IirStepper(state, torch.exp(lp)[..., 0].contiguous().to(DEV), r.to(DEV), Dc.to(DEV)),
+                           flip_x1x2=flip)
+    wD = w.repeat_interleave(D // G, 0)
+    ref_f, ref_s, ref_m = fst, st, s0
+    for i in range(4):
+        u = torch.randn(B, C, generator=g).bfloat16()
+        z, ref_f = O.step_fir(u, ref_f, wf, bias=bf)
+        x2, x1, v = oracle_gates(z, D, H, cs, il, flip)
+        y_ref, ref_s = O.step_fir(x1 * v, ref_s, wD, bias=bias, gated_bias=mr, flip_filter=mr)
+        y = torch.empty(B, D, dtype=torch.bfloat16, device=DEV)
+        fir(u.to(DEV), y)
+        assert rel_err(y, y_ref * x2) <= 2e-2, ("fir", i, K, G)
+        y2_ref, ref_m = O.step_iir(x2, x1, v, Dc, r, lp, ref_m)
+        y2 = torch.empty(B, D, dtype=torch.bfloat16, device=DEV)
+        iir(u.to(DEV), y2)
+        assert rel_err(y2, y2_ref.real if cplx else y2_ref) <= 2e-2, ("iir", i, S, cplx)
+    assert rel_err(ring.reference_order(), ref_s) <= 1e-2
+    assert rel_err(torch.view_as_real(state) if cplx else state, torch.view_as_real(ref_m) if cplx else ref_m) <= 1e-2
