@@ -26,7 +26,7 @@ struct ProjArgs {
 };
 
 // z[j] = bf16( sum_i w[i][c0+j]*slot_i[c0+j] + w[Rf][c0+j]*u[c0+j] (+ bias) ) for 8 consecutive channels
-__device__ __forceinline__ void proj_step8(const ProjArgs& pj, int64_t b, uint32_t c0, float* z) {
+__device__ __forceinline__ u32x4 proj_step8(const ProjArgs& pj, int64_t b, uint32_t c0, float* z) {
     const u32x4 un = *(const u32x4*)(pj.u + b * pj.u_bs + c0);
     float acc[8];
 #pragma unroll
@@ -58,24 +58,35 @@ __device__ __forceinline__ void proj_step8(const ProjArgs& pj, int64_t b, uint32
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) z[j] = round_bf(acc[j]);
-    *(u32x4*)(rb + (int64_t)pj.pos * pj.C) = un;        // the oldest slot takes the new sample
+    return un;                                          // the caller stores it into the oldest slot
+}
+
+__device__ __forceinline__ void proj_store8(const ProjArgs& pj, int64_t b, uint32_t c0, u32x4 un) {
+    *(u32x4*)(pj.ring + ((b * pj.Rf) + pj.pos) * pj.C + c0) = un;
 }
 
 // the three gates of 8 consecutive operator channels d0..d0+7: g[0] = x2, g[1] = x1, g[2] = v (before any flip)
 template <int FEAT>
 __device__ __forceinline__ void proj_gates8(const ProjArgs& pj, int64_t b, uint32_t d0, float (*g)[8]) {
     if (FEAT == 3) {            // interleaved: channels 3*d0 .. 3*d0+23, gate = channel % 3
+        // all reads of the three pieces first, the ring-slot stores last: no store sits between dependent loads
         float z[24];
-        proj_step8(pj, b, 3 * d0, z);
-        proj_step8(pj, b, 3 * d0 + 8, z + 8);
-        proj_step8(pj, b, 3 * d0 + 16, z + 16);
+        u32x4 un[3];
+#pragma unroll
+        for (int i = 0; i < 3; ++i) un[i] = proj_step8(pj, b, 3 * d0 + 8 * i, z + 8 * i);
+#pragma unroll
+        for (int i = 0; i < 3; ++i) proj_store8(pj, b, 3 * d0 + 8 * i, un[i]);
 #pragma unroll
         for (int j = 0; j < 8; ++j)
 #pragma unroll
             for (int i = 0; i < 3; ++i) g[i][j] = z[3 * j + i];
     } else {
+        u32x4 un[3];
+        uint32_t ch[3];
 #pragma unroll
-        for (int i = 0; i < 3; ++i) proj_step8(pj, b, pj.chan(i, d0), g[i]);
+        for (int i = 0; i < 3; ++i) { ch[i] = pj.chan(i, d0); un[i] = proj_step8(pj, b, ch[i], g[i]); }
+#pragma unroll
+        for (int i = 0; i < 3; ++i) proj_store8(pj, b, ch[i], un[i]);
     }
 }
 
@@ -262,31 +273,46 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
     const f32x4 pp = *(const f32x4*)(poles + ((int64_t)g * S) * FPS + q * 4);
     const f32x4 rr = *(const f32x4*)(residues + ((int64_t)g * S) * FPS + q * 4);
     const float dco = Dcoef[d];
+    // fused featurizer: lanes 0..2 of the group evaluate gates x2, x1, v of every batch element first (their
+    // loads overlap), the ring-slot stores follow, and only then the state updates start
+    float zf[NB];
+    if (FEAT) {
+        static_assert(!FEAT || LPB >= 4, "the fused featurizer needs three lanes per channel");
+        bf16_t un[NB];
 #pragma unroll
-    for (int j = 0; j < NB; ++j) {
-        const int64_t b = live[j] ? b0 + j : 0;
-        float a, c, gate2 = 0.f;
-        if (FEAT) {
-            static_assert(!FEAT || LPB >= 4, "the fused featurizer needs three lanes per channel");
-            float z = 0.f;
+        for (int j = 0; j < NB; ++j) {
+            zf[j] = 0.f;
+            un[j] = 0;
             if (q < 3) {
+                const int64_t b = live[j] ? b0 + j : 0;
                 const uint32_t ch = pj.chan((uint32_t)q, d);
-                bf16_t* rb = pj.ring + (b * pj.Rf) * pj.C + ch;
-                const bf16_t un = pj.u[b * pj.u_bs + ch];
+                const bf16_t* rb = pj.ring + (b * pj.Rf) * pj.C + ch;
+                un[j] = pj.u[b * pj.u_bs + ch];
                 float acc = 0.f;
                 for (int i = 0; i < pj.Rf; ++i) {
                     int s = pj.pos + i;
                     if (s >= pj.Rf) s -= pj.Rf;
                     acc = fmaf(pj.w[(int64_t)i * pj.C + ch], bf_to_f(rb[(int64_t)s * pj.C]), acc);
                 }
-                acc = fmaf(pj.w[(int64_t)pj.Rf * pj.C + ch], bf_to_f(un), acc);
+                acc = fmaf(pj.w[(int64_t)pj.Rf * pj.C + ch], bf_to_f(un[j]), acc);
                 if (pj.bias) acc += pj.bias[ch];
-                z = round_bf(acc);
-                if (live[j]) rb[(int64_t)pj.pos * pj.C] = un;
+                zf[j] = round_bf(acc);
             }
+        }
+        if (q < 3) {
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+                if (live[j]) pj.ring[(((b0 + j) * pj.Rf) + pj.pos) * pj.C + pj.chan((uint32_t)q, d)] = un[j];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int64_t b = live[j] ? b0 + j : 0;
+        float a, c, gate2 = 0.f;
+        if (FEAT) {
             const int base = (threadIdx.x & 63) & ~(LPB - 1);
-            const float g2 = __shfl(z, base, 64), g1 = __shfl(z, base + 1, 64);
-            c = __shfl(z, base + 2, 64);
+            const float g2 = __shfl(zf[j], base, 64), g1 = __shfl(zf[j], base + 1, 64);
+            c = __shfl(zf[j], base + 2, 64);
             a = pj.flip ? g2 : g1;
             gate2 = pj.flip ? g1 : g2;
         } else {
