@@ -71,6 +71,8 @@ def test_fir_layer_step_sequence_vs_oracle(B, D, H, G, K, Ks, cs, il, flip, sbia
     (2, 256, 4, 16, 16, True, False, True, False, False),     # complex poles, grouped
     (2, 96, 4, 96, 16, True, True, False, True, False),       # column split (head_dim 24), flipped
     (2, 200, 5, 200, 32, False, False, False, False, True),   # plain split, 32 states
+    (3, 48, 4, 48, 16, False, True, False, False, True),      # head_dim 12: no 16-byte pieces, scalar featurizer form
+    (5, 72, 6, 72, 16, True, True, False, True, False),
     (1, 64, 4, 64, 8, True, True, True, False, False),        # interleave + column split has no fused map
 ])
 def test_iir_layer_step_sequence_vs_oracle(B, D, H, G, S, cplx, cs, il, flip, d_bf16):

@@ -244,8 +244,10 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
 // with the poles and residues held in registers and the NB state loads issued together, which
 // puts enough bytes in flight to cover HBM latency.  The residue-weighted sum is reduced with
 // xor shuffles inside the lane group.
-// FEAT: lanes 0..2 of a lane group evaluate the fused featurizer step for gates x2, x1, v of their channel.
-template <int S, bool CPLX, bool FEAT, int NB>
+// FEAT (fused featurizer step): 0 none; 2 lanes 0..2 of a lane group evaluate gates x2, x1, v of their channel
+// with scalar loads (any channel map); 1 / 3 the block's first wavefronts evaluate the gates of all its
+// channels with 16-byte loads (unit-stride / interleaved map, as in the FIR step) and hand them over in LDS.
+template <int S, bool CPLX, int FEAT, int NB>
 __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict__ x1, const bf16_t* __restrict__ x2,
                                                        const bf16_t* __restrict__ v, int64_t in_bs, ProjArgs pj,
                                                        float* __restrict__ state, const float* __restrict__ poles,
@@ -255,6 +257,8 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
                                                        int64_t B, int64_t D, int dg) {
     constexpr int LPB = CPLX ? S / 2 : S / 4;      // lanes per channel
     constexpr int FPS = CPLX ? 2 : 1;              // floats per state
+    constexpr int ND = 256 / LPB;                  // channels per block
+    __shared__ float zs[(FEAT == 1 || FEAT == 3) ? NB * 3 * ND : 1];     // [j][gate-major or interleaved][channel]
     const uint32_t idx = blockIdx.x * 256 + threadIdx.x;        // (channel, lane of the group)
     const int q = (int)(idx % LPB);
     uint32_t d = idx / LPB;
@@ -276,8 +280,28 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
     // fused featurizer: lanes 0..2 of the group evaluate gates x2, x1, v of every batch element first (their
     // loads overlap), the ring-slot stores follow, and only then the state updates start
     float zf[NB];
-    if (FEAT) {
-        static_assert(!FEAT || LPB >= 4, "the fused featurizer needs three lanes per channel");
+    if (FEAT == 1 || FEAT == 3) {
+        static_assert(ND % 8 == 0, "whole 8-channel pieces per block");
+        constexpr int PPB = 3 * ND / 8;            // 8-channel pieces per batch element
+        const uint32_t dblk = blockIdx.x * ND;
+        const int e = threadIdx.x;
+        if (e < NB * PPB) {
+            const int j = e / PPB, r = e - j * PPB;
+            // piece r covers zs columns 8r..8r+7: interleaved order (column = 3*dl + gate) or gate-major (gate*ND + dl)
+            const uint32_t dl0 = FEAT == 3 ? 0 : (uint32_t)(8 * r) % ND;
+            const uint32_t ch = FEAT == 3 ? 3 * dblk + 8 * r : pj.chan((uint32_t)(8 * r) / ND, dblk + dl0);
+            const bool ok = b0 + j < B && (FEAT == 3 ? 3 * dblk + 8 * r < 3 * (uint32_t)D : dblk + dl0 < (uint32_t)D);
+            if (ok) {
+                float z[8];
+                const u32x4 un = proj_step8(pj, b0 + j, ch, z);
+                proj_store8(pj, b0 + j, ch, un);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) zs[(j * 3 * ND) + 8 * r + k] = z[k];
+            }
+        }
+        __syncthreads();
+    } else if (FEAT == 2) {
+        static_assert(FEAT != 2 || LPB >= 4, "the scalar fused featurizer needs three lanes per channel");
         bf16_t un[NB];
 #pragma unroll
         for (int j = 0; j < NB; ++j) {
@@ -309,7 +333,14 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
     for (int j = 0; j < NB; ++j) {
         const int64_t b = live[j] ? b0 + j : 0;
         float a, c, gate2 = 0.f;
-        if (FEAT) {
+        if (FEAT == 1 || FEAT == 3) {
+            const int dl = threadIdx.x / LPB;
+            const float* zj = zs + j * 3 * ND;
+            const float g2 = FEAT == 3 ? zj[3 * dl] : zj[dl], g1 = FEAT == 3 ? zj[3 * dl + 1] : zj[ND + dl];
+            c = FEAT == 3 ? zj[3 * dl + 2] : zj[2 * ND + dl];
+            a = pj.flip ? g2 : g1;
+            gate2 = pj.flip ? g1 : g2;
+        } else if (FEAT == 2) {
             const int base = (threadIdx.x & 63) & ~(LPB - 1);
             const float g2 = __shfl(zf[j], base, 64), g1 = __shfl(zf[j], base + 1, 64);
             c = __shfl(zf[j], base + 2, 64);
@@ -340,7 +371,7 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
         if (live[j] && q == 0) {
             float dx = dco * x1v;
             if (d_is_bf16) dx = round_bf(dx);
-            const float y = (FEAT ? gate2 : bf_to_f(x2[b * in_bs + d])) * (part + dx);
+            const float y = (FEAT != 0 ? gate2 : bf_to_f(x2[b * in_bs + d])) * (part + dx);
             if (out_is_fp32) ((float*)out)[b * out_bs + d] = y;
             else ((bf16_t*)out)[b * out_bs + d] = (bf16_t)f_to_bf_bits(y);
         }
@@ -483,16 +514,18 @@ static int iir_step_launch(const void* x1, const void* x2, const void* v, int64_
     dim3 grid((unsigned)((D * lpb + 255) / 256), (unsigned)gy);
     hipStream_t s = (hipStream_t)stream;
     const bf16_t *p1 = (const bf16_t*)x1, *p2 = (const bf16_t*)x2, *pv = (const bf16_t*)v;
-    const bool feat = proj != nullptr;
+    // fused featurizer: vector form where the channel map and alignment allow it, scalar form otherwise
+    const int feat = !proj ? 0 : (proj_vector_mode(proj, D) ? proj_vector_mode(proj, D) : 2);
 #define IIR_GO(SS, C, F, N)                                                                                     \
     hipLaunchKernelGGL((iir_step_kernel<SS, C, F, N>), grid, dim3(256), 0, s, p1, p2, pv, in_bs, pj, state,     \
                        poles, residues, Dcoef, d_is_bf16, out, out_is_fp32, out_bs, B, D, dg)
 #define IIR_CASE(SS, C, F)                                                                                      \
     if (S == SS && (is_complex != 0) == C && feat == F) { if (nb == 4) IIR_GO(SS, C, F, 4); else IIR_GO(SS, C, F, 1); }
-    IIR_CASE(8, false, false) IIR_CASE(16, false, false) IIR_CASE(32, false, false)
-    IIR_CASE(8, true, false) IIR_CASE(16, true, false) IIR_CASE(32, true, false)
-    IIR_CASE(16, false, true) IIR_CASE(32, false, true)
-    IIR_CASE(8, true, true) IIR_CASE(16, true, true) IIR_CASE(32, true, true)
+#define IIR_FEATS(SS, C) IIR_CASE(SS, C, 1) IIR_CASE(SS, C, 2) IIR_CASE(SS, C, 3)
+    IIR_CASE(8, false, 0) IIR_CASE(16, false, 0) IIR_CASE(32, false, 0)
+    IIR_CASE(8, true, 0) IIR_CASE(16, true, 0) IIR_CASE(32, true, 0)
+    IIR_FEATS(16, false) IIR_FEATS(32, false) IIR_FEATS(8, true) IIR_FEATS(16, true) IIR_FEATS(32, true)
+#undef IIR_FEATS
 #undef IIR_CASE
 #undef IIR_GO
     return hyena_check_launch(who);
