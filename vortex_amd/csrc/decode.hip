@@ -65,31 +65,6 @@ __device__ __forceinline__ void proj_store8(const ProjArgs& pj, int64_t b, uint3
     *(u32x4*)(pj.ring + ((b * pj.Rf) + pj.pos) * pj.C + c0) = un;
 }
 
-// the three gates of 8 consecutive operator channels d0..d0+7: g[0] = x2, g[1] = x1, g[2] = v (before any flip)
-template <int FEAT>
-__device__ __forceinline__ void proj_gates8(const ProjArgs& pj, int64_t b, uint32_t d0, float (*g)[8]) {
-    if (FEAT == 3) {            // interleaved: channels 3*d0 .. 3*d0+23, gate = channel % 3
-        // all reads of the three pieces first, the ring-slot stores last: no store sits between dependent loads
-        float z[24];
-        u32x4 un[3];
-#pragma unroll
-        for (int i = 0; i < 3; ++i) un[i] = proj_step8(pj, b, 3 * d0 + 8 * i, z + 8 * i);
-#pragma unroll
-        for (int i = 0; i < 3; ++i) proj_store8(pj, b, 3 * d0 + 8 * i, un[i]);
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-#pragma unroll
-            for (int i = 0; i < 3; ++i) g[i][j] = z[3 * j + i];
-    } else {
-        u32x4 un[3];
-        uint32_t ch[3];
-#pragma unroll
-        for (int i = 0; i < 3; ++i) { ch[i] = pj.chan(i, d0); un[i] = proj_step8(pj, b, ch[i], g[i]); }
-#pragma unroll
-        for (int i = 0; i < 3; ++i) proj_store8(pj, b, ch[i], un[i]);
-    }
-}
-
 // ---------------------------------------------------------------- FIR step
 // Block = NSG wavefronts over the same 512 channels; wavefront sg handles cache
 // slots sg, sg+NSG, ... so every load instruction reads 1 KiB of one slot row.
@@ -114,6 +89,7 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
     const int ng = GROUPED ? (512 / dg) : 0;
     float* wl = smem;                       // [W][ng]  taps of the block's groups, transposed
     float* red = smem + (GROUPED ? W * ng : 0);   // [NSG-1][2][64][4]
+    float* zs = red + (NSG - 1) * 512;            // [3][512] gates of the block's channels (fused featurizer only)
     const int gl = GROUPED ? (oc * 8) / dg : 0;
     constexpr int UF = 8;                   // cache slots in flight per lane
     const bf16_t* rb = ring + (b * R) * D + d0;
@@ -156,15 +132,21 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
     // the first batch of cache reads goes out before the tap table is staged, so HBM is busy from the start
     u32x4 q0[UF];
     load_batch(sg, q0);
-    uint32_t f1[4], f2[4], fv[4];           // packed gates from the fused featurizer
-    if (FEAT != 0 && sg == 0 && live) {
-        float g[3][8];
-        proj_gates8<FEAT>(pj, b, (uint32_t)d0, g);
+    // Fused featurizer: the block's 3 x 512 projection channels are 192 pieces of 8; thread p evaluates piece p
+    // (its loads overlap the cache reads above) and leaves the gates in LDS for the wavefront that writes the output.
+    if (FEAT != 0) {
+        for (int p = tid; p < 192; p += 64 * NSG) {
+            // FEAT 3: columns in projection order (3*dl + gate); FEAT 1: gate-major (gate*512 + dl)
+            const uint32_t dl0 = FEAT == 3 ? 0 : (uint32_t)(8 * p) & 511;
+            const uint32_t ch = FEAT == 3 ? 3 * (uint32_t)dblk + 8 * p : pj.chan((uint32_t)(8 * p) >> 9, (uint32_t)dblk + dl0);
+            const bool ok = FEAT == 3 ? 3 * (uint32_t)dblk + 8 * p < 3 * (uint32_t)D : (uint32_t)dblk + dl0 < (uint32_t)D;
+            if (ok) {
+                float z[8];
+                const u32x4 un = proj_step8(pj, b, ch, z);
+                proj_store8(pj, b, ch, un);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            f1[j] = pack_bf2(pj.flip ? g[0][2 * j] : g[1][2 * j], pj.flip ? g[0][2 * j + 1] : g[1][2 * j + 1]);
-            f2[j] = pack_bf2(pj.flip ? g[1][2 * j] : g[0][2 * j], pj.flip ? g[1][2 * j + 1] : g[0][2 * j + 1]);
-            fv[j] = pack_bf2(g[2][2 * j], g[2][2 * j + 1]);
+                for (int k = 0; k < 8; ++k) zs[8 * p + k] = z[k];
+            }
         }
     }
     if (GROUPED) {
@@ -206,7 +188,19 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
     u32x4 a1, av = {0, 0, 0, 0}, a2 = {0, 0, 0, 0};
     if (FEAT != 0) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) { a1[j] = f1[j]; av[j] = fv[j]; a2[j] = f2[j]; }
+        for (int j = 0; j < 4; ++j) {
+            float g2[2], g1[2], gv[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int dl = oc * 8 + 2 * j + e;
+                g2[e] = FEAT == 3 ? zs[3 * dl] : zs[dl];
+                g1[e] = FEAT == 3 ? zs[3 * dl + 1] : zs[512 + dl];
+                gv[e] = FEAT == 3 ? zs[3 * dl + 2] : zs[1024 + dl];
+            }
+            a1[j] = pj.flip ? pack_bf2(g2[0], g2[1]) : pack_bf2(g1[0], g1[1]);
+            a2[j] = pj.flip ? pack_bf2(g1[0], g1[1]) : pack_bf2(g2[0], g2[1]);
+            av[j] = pack_bf2(gv[0], gv[1]);
+        }
     } else {
         a1 = *(const u32x4*)(x1 + b * in_bs + d0);
         if (PRE) av = *(const u32x4*)(v + b * in_bs + d0);
@@ -438,7 +432,8 @@ static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_
     const bool pre = proj || v != nullptr, post = proj || x2 != nullptr;
     dim3 grid((unsigned)((D + 511) / 512), (unsigned)B);
     const int nsg = R >= 32 ? 8 : 2;
-    size_t sh = (size_t)(nsg - 1) * 64 * 8 * sizeof(float) + (grouped ? (size_t)(R + 1) * (512 / dg) * sizeof(float) : 0);
+    size_t sh = (size_t)(nsg - 1) * 64 * 8 * sizeof(float) + (grouped ? (size_t)(R + 1) * (512 / dg) * sizeof(float) : 0) +
+                (proj ? 3 * 512 * sizeof(float) : 0);
     if (sh > 160 * 1024) return hyena_fail(HYENA_ENOSUP, "%s: R too large for the LDS tap table", who);
     hipStream_t s = (hipStream_t)stream;
     const bf16_t *p1 = (const bf16_t*)x1, *p2 = (const bf16_t*)x2, *pv = (const bf16_t*)v;
