@@ -71,3 +71,12 @@ def test_new_entry_points_validate_before_touching_the_device():
     ps = _lib.ProjStep(P, 192, P, 2, 0, P, None, 4, 12, 4, 1, 0)
     assert L.hyena_fir_layer_step(ref(ps), P, 6, 0, P, None, 0, P, 64, 1, 64, 4, None) == -3          # head_dim 4
     assert L.hyena_iir_layer_step(None, P, P, P, 0, P, 0, P, 0, 64, 1, 64, 64, 16, None) == -1
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    # no CPU or PyTorch fallback: without the built library every operator raises
+    from vortex_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libhyena_mi355x.so")
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        _lib.lib()
