@@ -49,6 +49,32 @@ def gates(B, D, L, seed, device):
                  for _ in range(3))
 
 
+class _Synthetic:
+    """Seeded synthetic filters and poles of the benchmark configurations (generated on the CPU, as the parity
+    tests generate theirs, so every run sees the same values)."""
+
+    @staticmethod
+    def make_se_filter(G, K=7, seed=100):
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        return torch.randn(G, 1, K, generator=g) / math.sqrt(K)
+
+    @staticmethod
+    def make_mr_filter(G, K=128, seed=200):
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        w = torch.randn(G, 1, K, generator=g) / math.sqrt(K)
+        a = 0.01 + 0.09 * torch.rand(G, 1, 1, generator=g)
+        return w * torch.exp(-a * torch.arange(K)[None, None])
+
+    @staticmethod
+    def make_modal_complex(G, S=16, seed=300, pmin=0.9, pmax=0.9999):
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        mag = pmin + (pmax - pmin) * torch.rand(G, S, generator=g, dtype=torch.float64)
+        ang = math.pi * torch.rand(G, S, generator=g, dtype=torch.float64)
+        log_poles = torch.complex(mag.log(), ang).to(torch.complex64)[..., None]
+        res = torch.complex(torch.randn(G, S, generator=g), torch.randn(G, S, generator=g)) / math.sqrt(2.0)
+        return log_poles, res.to(torch.complex64)
+
+
 def time_steps(fn, steps, warmup):
     """(wall seconds for `steps` calls, average kernel-side ms per call from HIP events on the launch stream)."""
     for _ in range(warmup):
@@ -69,7 +95,7 @@ def time_steps(fn, steps, warmup):
 def build_workload(name, device):
     """Returns (callable, description dict) for one configuration."""
     import vortex_amd as va
-    from oracle import hyena_oracle as O          # input generators only (filters, poles)
+    O = _Synthetic
     from vortex_amd import ops
 
     if name == "se":
@@ -132,7 +158,7 @@ def build_workload(name, device):
 def decode_layer_set(D, device, steps, warmup):
     """One [SE, MR, LI] layer set of cached decode at batch 64: three fused launches per token."""
     import vortex_amd as va
-    from oracle import hyena_oracle as O
+    O = _Synthetic
     B, S = 64, 16
     g = torch.Generator(device=device).manual_seed(6)
     rnd = lambda *s: torch.randn(*s, generator=g, device=device, dtype=torch.float32)
@@ -164,7 +190,7 @@ def decode_layers_from_projection(D, device, steps, warmup):
     gates, K=3 featurizer): featurizer step, split, gates and inner step in one launch per layer."""
     import vortex_amd as va
     from vortex_amd import ops
-    from oracle import hyena_oracle as O
+    O = _Synthetic
     B, S, C = 64, 16, 3 * D
     g = torch.Generator(device=device).manual_seed(7)
     rnd = lambda *s: torch.randn(*s, generator=g, device=device, dtype=torch.float32)
