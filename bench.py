@@ -270,7 +270,7 @@ def cpu_baseline(name):
     from oracle import hyena_oracle as O
     threads = torch.get_num_threads()
     if name == "mr":
-        B, D, L, G, K, Ds = 2, 4096, 32768, 256, 128, 256
+        B, D, L, G, K, Ds = 2, 4096, 32768, 256, 128, 1024
         x2, x1, v = O.make_gates(B, Ds, L, seed=2)
         h = O.make_mr_filter(Ds // 16, K)
         Db = torch.randn(Ds)
@@ -291,7 +291,7 @@ def cpu_baseline(name):
     f()
     ts = []
     t_all = time.perf_counter()
-    while len(ts) < 3 or (time.perf_counter() - t_all < 10 and len(ts) < 20):
+    while len(ts) < 3 or (time.perf_counter() - t_all < 12 and len(ts) < 40):      # about 10 s of CPU work
         t0 = time.perf_counter()
         f()
         ts.append(time.perf_counter() - t0)
