@@ -94,8 +94,9 @@ int hyena_featurizer_fwd(const void* u, int64_t u_batch_stride, int64_t u_time_s
  *   u = bf16(x1*v);  y[t] = sum_k h[g][k] * u[t-k]   (true convolution, h[g][0] on the current sample)
  *   z = bias rule;   out = bf16(x2*z)
  * With taps_reversed != 0 the filter is read in the SE orientation instead
- * (h[g][K-1] on the current sample).  Requires D/G to be a multiple of 16 and
- * L, strides multiples of 8.  out: [B][D][L] bf16. */
+ * (h[g][K-1] on the current sample).  L and strides must be multiples of 8.  The 16 channels of an MFMA
+ * tile share one filter, so groups of D/G = 16, 32, ... channels use the matrix cores fully; other group
+ * sizes run with partly filled tiles (D/G = 15: 94 %, one filter per channel: 6 %).  out: [B][D][L] bf16. */
 int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v,
                  const float* h, int taps_reversed, const float* bias, int bias_mode,
                  void* out, int64_t B, int64_t D, int64_t L, int64_t G, int K,

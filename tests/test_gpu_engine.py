@@ -215,6 +215,40 @@ def test_operator_module_prefill_then_decode(kind, cs, il, fused):
         assert (mod._decode["layer"] is not None) == (not (cs and il))
 
 
+@pytest.mark.parametrize("kind", ["se", "mr", "li_real"])
+def test_operator_module_groups_of_15_channels(kind):
+    # Evo 2 1B geometry in small: hidden = 16 groups x 15 channels (1920 = 128 x 15 there), 15 heads, interleaved gates
+    B, L, H, G, n_dec = 2, 400, 15, 16, 3
+    D = 15 * G
+    K = {"se": 7, "mr": 128}.get(kind)
+    p = make_params(kind, D, G if K else D, seed=41)
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=False, interleave=True, short_filter_length=3,
+               short_filter_bias=False, state_size=16)
+    mod = HyenaCascade(cfg, 0, hyena_filter_groups=G if K else D, fir_inner_filter_length=K)
+    with torch.no_grad():
+        mod.short_filter_weight.copy_(p["short_filter_weight"])
+        if K:
+            mod.h.copy_(p["h"])
+        else:
+            mod.log_poles.copy_(p["log_poles"])
+            mod.residues.copy_(p["residues"])
+        if mod.D is not None:
+            mod.D.data = p["D"].clone()
+    mod = mod.to(DEV)
+    ref = O.OracleCascade(O.OracleEngine(), p, D, H, G if K else D, fir_inner_filter_length=K, interleave=True)
+    u_all = torch.randn(B, L + n_dec, 3 * D, generator=torch.Generator().manual_seed(7)).bfloat16()
+    ip_ref = O.OracleCache()
+    ip_hip = HyenaCascadeFIRInferenceParams() if K else HyenaCascadeIIRInferenceParams()
+    y_ref, _ = ref.forward(u_all[:, :L], ip_ref)
+    y_hip, _ = mod(u_all[:, :L].to(DEV), ip_hip)
+    assert rel_err(y_hip, y_ref) <= 2e-2
+    for i in range(n_dec):
+        tok = u_all[:, L + i: L + i + 1]
+        y_ref, _ = ref.forward(tok, ip_ref)
+        y_hip, _ = mod(tok.to(DEV), ip_hip)
+        assert rel_err(y_hip, y_ref) <= 2e-2, i
+
+
 def test_hyena_ops_interface_layouts():
     import hyena_ops
     from hyena_ops import interface as I

@@ -154,6 +154,24 @@ def test_mr_full_size_rows():
     assert rel_err(out[:, rows], ref) <= TOL
 
 
+@pytest.mark.parametrize("B,D,G,L,K", [
+    (1, 1920 // 8, 16, 1024, 128),     # 15 channels per group (Evo 2 1B: hidden 1920, 128 groups)
+    (2, 96, 4, 520, 128),              # 24 = one full slab of 16 and one of 8
+    (1, 40, 5, 300, 33),               # 8 per group
+    (2, 24, 24, 200, 128),             # one filter per channel
+    (1, 7 * 8, 8, 96, 16),             # 7 per group
+])
+def test_mr_any_group_size(B, D, G, L, K):
+    # groups that are not multiples of the 16-channel MFMA slab run with partly filled slabs
+    g = torch.Generator().manual_seed(D + K)
+    x2, x1, v = (torch.randn(B, D, L, generator=g).bfloat16() for _ in range(3))
+    h = O.make_mr_filter(G, K, seed=D)
+    Db = torch.randn(D, generator=g)
+    ref, _ = O.mr_fir(x2, x1, v, h, Db)
+    out = va.hyena_mr_fwd(x1.cuda(), x2.cuda(), v.cuda(), h.cuda(), Db.cuda())
+    assert rel_err(out, ref) <= TOL
+
+
 def test_se_nontemporal_variant_matches(monkeypatch):
     # large activations take the non-temporal (streaming) code path; force it on a small case
     B, D, L, G, K = 2, 64, 2048, 4, 7
@@ -177,8 +195,6 @@ def test_argument_errors():
     r = ops.rows_of(x)
     with pytest.raises(ValueError):
         ops.fir_fwd_rows(r, r, r, torch.zeros(2, 7, device="cuda"), 1, 32, 60, 7, device=x.device)
-    with pytest.raises(NotImplementedError):              # 8 channels per group: no MFMA tiling
-        va.hyena_mr_fwd(x, x, x, torch.zeros(4, 1, 128, device="cuda"))
     with pytest.raises(NotImplementedError):              # K > 128
         va.hyena_mr_fwd(x, x, x, torch.zeros(2, 1, 200, device="cuda"))
     with pytest.raises(TypeError):

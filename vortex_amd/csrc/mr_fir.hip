@@ -52,7 +52,7 @@ __device__ __forceinline__ u32x4 gate_mul(u32x4 a, u32x4 b) {
 }
 
 template <bool PRE, bool POST, int BIAS, bool NT, bool FULL>
-__global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, RowMap v, const float* __restrict__ h,
+__global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, RowMap v, const float* __restrict__ h,
                                                         int K, int reversed, const float* __restrict__ bias,
                                                         bf16_t* __restrict__ out, int64_t D, int64_t L, int dg,
                                                         int64_t seg_len, int nseg) {
@@ -61,13 +61,18 @@ __global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t nslab = (uint32_t)(D / 16);
+    // A slab is 16 channels of one filter group.  Groups whose size is not a multiple of 16 get a last slab
+    // with fewer live channels (their rows are read as zeros and never stored).
+    const uint32_t spg = ((uint32_t)dg + 15) / 16;              // slabs per group
+    const uint32_t nslab = (uint32_t)(D / dg) * spg;
     const uint32_t bid = blockIdx.x;
     const int seg = (int)(bid % (uint32_t)nseg);
     const uint32_t slab = (bid / (uint32_t)nseg) % nslab;
     const int64_t b = bid / ((uint32_t)nseg * nslab);
-    const int64_t d0 = (int64_t)slab * 16;
-    const int g = (int)((uint32_t)d0 / (uint32_t)dg);
+    const int g = (int)(slab / spg);
+    const int c_base = 16 * (int)(slab % spg);                 // first channel of the slab inside its group
+    const int64_t d0 = (int64_t)g * dg + c_base;
+    const int c_live = dg - c_base < 16 ? dg - c_base : 16;    // live channels of this slab
 
     // ---- Toeplitz fragments of this group's filter (A operand, 32 x 16 each)
     const int n = lane & 31, hh = lane >> 5;
@@ -98,9 +103,11 @@ __global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
     // ---- coalesced layout: this thread moves 16 B of rows 4*r4 + w, r4 = 0..3
     const bf16_t *p1[4], *pv[4], *p2[4];
     bf16_t* po[4];
+    bool rlive[4];
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
-        const int64_t d = d0 + 4 * r4 + w;
+        rlive[r4] = 4 * r4 + w < c_live;
+        const int64_t d = rlive[r4] ? d0 + 4 * r4 + w : d0;
         p1[r4] = x1.row(b, d) + lane * 8;
         pv[r4] = PRE ? v.row(b, d) + lane * 8 : nullptr;
         p2[r4] = POST ? x2.row(b, d) + lane * 8 : nullptr;
@@ -114,7 +121,7 @@ __global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
     {
         const int ch = tid >> 4, tt = (tid & 15) * 8;
         u32x4 hu = {0, 0, 0, 0};
-        if (t_begin > 0) {
+        if (t_begin > 0 && ch < c_live) {
             const u32x4 a = *(const u32x4*)(x1.row(b, d0 + ch) + t_begin - HALO + tt);
             u32x4 c = {0, 0, 0, 0};
             if (PRE) c = *(const u32x4*)(v.row(b, d0 + ch) + t_begin - HALO + tt);
@@ -127,14 +134,14 @@ __global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
     const u32x4 zero4 = {0, 0, 0, 0};
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
-        const bool ok = t_begin + lane * 8 < L;
+        const bool ok = rlive[r4] && t_begin + lane * 8 < L;
         c1[r4] = ok ? ld16<NT>(p1[r4] + t_begin) : zero4;
         cv[r4] = (PRE && ok) ? ld16<NT>(pv[r4] + t_begin) : zero4;
         c2n[r4] = (POST && ok) ? ld16<NT>(p2[r4] + t_begin) : zero4;
     }
 
     float bz = 0.f;
-    if (BIAS != HYENA_BIAS_NONE) bz = bias[d0 + (n & 15)];
+    if (BIAS != HYENA_BIAS_NONE && (n & 15) < c_live) bz = bias[d0 + (n & 15)];
 
     for (int64_t ts = t_begin; ts < t_end; ts += TL) {
         // u of this step -> LDS
@@ -147,9 +154,10 @@ __global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
         u32x4 c2[4];
         {
             const int64_t tn = ts + TL;
-            const bool okn = (tn < t_end) && (tn + lane * 8 < L);
+            const bool okt = (tn < t_end) && (tn + lane * 8 < L);
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
+                const bool okn = okt && rlive[r4];
                 c2[r4] = c2n[r4];
                 c1[r4] = okn ? ld16<NT>(p1[r4] + tn) : zero4;
                 cv[r4] = (PRE && okn) ? ld16<NT>(pv[r4] + tn) : zero4;
@@ -207,6 +215,7 @@ __global__ __launch_bounds__(256, 2) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
         if (ts + lane * 8 < t_end) {
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
+                if (!rlive[r4]) continue;
                 const u32x4 zz = *(const u32x4*)(z_lds + (4 * r4 + w) * ZRS + lane * 8);
                 u32x4 o = zz;
                 if (POST) {
@@ -230,8 +239,6 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
         return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: bad sizes B=%lld D=%lld L=%lld G=%lld", (long long)B,
                           (long long)D, (long long)L, (long long)G);
     if (K < 1 || K > 128) return hyena_fail(HYENA_ENOSUP, "hyena_mr_fwd: K=%d outside 1..128", K);
-    if ((D / G) % 16 != 0)
-        return hyena_fail(HYENA_ENOSUP, "hyena_mr_fwd: D/G=%lld must be a multiple of 16", (long long)(D / G));
     if (bias_mode < 0 || bias_mode > 2 || (bias_mode != HYENA_BIAS_NONE && !bias))
         return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: bias_mode %d needs a bias pointer", bias_mode);
     if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15))
@@ -240,7 +247,7 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
 
     // segments along L: >= 4096 blocks (256 CUs x 3 resident blocks, several rounds), segments >= 2048 samples
-    const int64_t rows = B * (D / 16);
+    const int64_t rows = B * G * ((D / G + 15) / 16);          // (batch, slab) pairs
     int64_t nseg = (4096 + rows - 1) / rows;
     const int64_t max_seg = (L + 2047) / 2048;
     if (nseg > max_seg) nseg = max_seg;

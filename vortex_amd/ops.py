@@ -345,7 +345,7 @@ def fir_step(x1, ring, w, *, x2=None, v=None, bias=None, gated_bias=False):
     _need_cuda(x1, ring.buf, w)
     B, D = x1.shape
     R = ring.buf.shape[1]
-    w = _f32(w)
+    w = _step_taps(w, D)
     G = w.shape[0]
     if w.shape[1] != R + 1:
         raise ValueError(f"taps have {w.shape[1]} columns, cache depth {R} needs {R + 1}")
@@ -396,13 +396,25 @@ def iir_step(x1, x2, v, state, poles, residues, Dcoef, *, out_dtype=torch.bfloat
     return out
 
 
+def _step_taps(w, D):
+    """Taps [G, R+1] in the form hyena_fir_step takes: shared by groups of 8, 16, ... 512 channels (a divisor of
+    512), or one row per channel; other group sizes are expanded to per-channel rows here."""
+    w = _f32(w)
+    G = w.shape[0]
+    dg = D // G
+    if G != D and not (dg % 8 == 0 and 512 % dg == 0):
+        w = w.repeat_interleave(dg, 0).contiguous()
+    return w
+
+
 class FirStepper:
     """A decode FIR step with every argument except the gates bound once (low host overhead)."""
 
     def __init__(self, ring, w, bias=None, gated_bias=False, gated=True):
         _need_cuda(ring.buf, w)
-        self.ring, self.w, self.bias = ring, _f32(w), _f32(bias)
+        self.ring, self.bias = ring, _f32(bias)
         self.R, self.D = ring.buf.shape[1], ring.buf.shape[2]
+        self.w = _step_taps(w, self.D)
         self.G = self.w.shape[0]
         if self.w.shape[1] != self.R + 1:
             raise ValueError(f"taps have {self.w.shape[1]} columns, cache depth {self.R} needs {self.R + 1}")
