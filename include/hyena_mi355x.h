@@ -116,9 +116,9 @@ int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v
  * Each wavefront of hyena_li_fwd expands its group's table once into the MFMA operand fragments it keeps in
  * registers.  log_poles and residues are [G][S][2] float32 (re, im) pairs; real poles have im = 0.  The caller
  * owns the workspace: hyena_li_plan_bytes(G, S) bytes of device memory, reusable until the parameters change.
- * S must be 16.
+ * S is 1..16 (fewer than 16 modes are filled up with poles of residue zero inside the table).
  *
- * hyena_li_fwd: D/G must be a multiple of 16, L and strides multiples of 8.
+ * hyena_li_fwd: L and strides must be multiples of 8; any D/G (groups of a multiple of 4 channels are fastest).
  * y_conv_fp32 (optional, [B][D][L]) receives the fp32 convolution before any rounding;
  * state_out (optional, [B][D][S][2] float32) the modal state after the last sample.
  * d_is_bf16 selects the rounding of z = y + Dcoef*x1v: 1 = bf16(bf16(y) + bf16(Dcoef*x1v)), what
@@ -156,7 +156,7 @@ int hyena_fir_step(const void* x1, const void* x2, const void* v, int64_t in_bat
  * state: [B][D][S] float32 (is_complex == 0) or [B][D][S][2] (re, im) float32, updated in place.
  * poles (already exponentiated) and residues: [G][S] or [G][S][2] float32.
  * Dcoef: [D] float32; d_is_bf16 != 0 rounds Dcoef*x1v to bf16 as a bf16 parameter does.
- * out: [B][D] bf16 (out_is_fp32 == 0) or float32. */
+ * out: [B][D] bf16 (out_is_fp32 == 0) or float32.  S is a power of two up to 32. */
 int hyena_iir_step(const void* x1, const void* x2, const void* v, int64_t in_batch_stride,
                    float* state, const float* poles, const float* residues, int is_complex,
                    const float* Dcoef, int d_is_bf16,
@@ -188,8 +188,8 @@ typedef struct hyena_proj_step {
  * Hyena layer and token.  Same arithmetic as the featurizer's hyena_fir_step (bias rule ADD) followed by
  * the gated step; the featurizer cache slot and the inner cache / state are both updated.
  * hyena_fir_layer_step needs one of the three channel maps listed above, 16-byte aligned pointers and
- * head_dim % 8 == 0; it takes bias_mode NONE or GATED_FP32.  hyena_iir_layer_step takes any map; not
- * available for 8 real states. */
+ * head_dim % 8 == 0; it takes bias_mode NONE or GATED_FP32.  hyena_iir_layer_step takes any map; it
+ * needs at least 16 real or 8 complex states. */
 int hyena_fir_layer_step(const hyena_proj_step* proj,
                          void* ring, int64_t R, int64_t pos,
                          const float* w, const float* bias, int bias_mode,

@@ -80,9 +80,11 @@ def test_iir_step_golden(name):
     assert (state.cpu() - se).abs().max() <= 1e-5 * se.abs().max()
 
 
-@pytest.mark.parametrize("cplx,G", [(False, 256), (True, 256), (True, 16), (False, 1)])
-def test_iir_step_sequence_vs_oracle(cplx, G):
-    B, D, S = 5, 256, 16
+@pytest.mark.parametrize("cplx,G,S", [(False, 256, 16), (True, 256, 16), (True, 16, 16), (False, 1, 16),
+                                      (False, 256, 8), (True, 16, 8), (False, 1, 2), (True, 256, 2), (False, 16, 1),
+                                      (True, 1, 1), (False, 256, 4), (True, 16, 4), (False, 16, 32), (True, 256, 32)])
+def test_iir_step_sequence_vs_oracle(cplx, G, S):
+    B, D = 5, 256
     g = torch.Generator().manual_seed(3)
     lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(G, S, seed=4)
     Dp = torch.randn(D, generator=g).bfloat16()

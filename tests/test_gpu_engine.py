@@ -168,6 +168,43 @@ def test_operator_module_any_prompt_length(kind, L):
             assert rel_err(y_hip, y_ref) <= 2e-2, (fused, i)
 
 
+@pytest.mark.parametrize("S,bias,L", [(8, False, 512), (2, True, 512), (2, True, 37), (4, False, 200)])
+def test_operator_module_small_state_sizes(S, bias, L):
+    # the long-filter layers of the older configurations: state_size 8 (shc-evo2-7b-8k-2T-v1.yml) and 2
+    # (7b-sh-32k-v1.yml), one filter per channel, head-blocked column split, featurizer bias
+    B, D, H, n_dec = 2, 64, 4, 5
+    g = torch.Generator().manual_seed(S)
+    lp, r = O.make_modal_real(D, S, seed=S, pmax=0.999)
+    p = {"short_filter_weight": torch.randn(3 * D, 1, 3, generator=g) / 3 ** 0.5,
+         "short_filter_bias": torch.randn(3 * D, generator=g).bfloat16() if bias else None,
+         "log_poles": lp, "residues": r, "D": torch.randn(D, generator=g).bfloat16()}
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=True, interleave=False, short_filter_length=3,
+               short_filter_bias=bias, state_size=S)
+    ref = O.OracleCascade(O.OracleEngine(), p, D, H, D, column_split_hyena=True, interleave=False)
+    u_all = torch.randn(B, L + n_dec, 3 * D, generator=g).bfloat16()
+    for fused in (True, False):
+        mod = HyenaCascade(cfg, 0)
+        with torch.no_grad():
+            mod.short_filter_weight.copy_(p["short_filter_weight"])
+            if bias:
+                mod.short_filter_bias.copy_(p["short_filter_bias"])
+            mod.log_poles.copy_(lp)
+            mod.residues.copy_(r)
+            mod.D.data = p["D"].clone()
+        mod = mod.to(DEV)
+        mod.fuse_prefill = mod.fuse_decode = fused
+        ip_ref, ip_hip = O.OracleCache(), HyenaCascadeIIRInferenceParams()
+        y_ref, _ = ref.forward(u_all[:, :L], ip_ref)
+        y_hip, _ = mod(u_all[:, :L].to(DEV), ip_hip)
+        assert rel_err(y_hip, y_ref) <= 2e-2
+        assert ip_hip.state_dict[0].shape == (B, D, S)
+        for i in range(n_dec):
+            tok = u_all[:, L + i: L + i + 1]
+            y_ref, _ = ref.forward(tok, ip_ref)
+            y_hip, _ = mod(tok.to(DEV), ip_hip)
+            assert rel_err(y_hip, y_ref) <= 2e-2, (fused, i)
+
+
 @pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("kind,cs,il", [("se", False, True), ("mr", False, True), ("mr", True, False),
                                          ("li_cplx", False, True), ("li_real", True, False), ("se", False, False),

@@ -41,6 +41,24 @@ def test_li_vs_oracle(B, D, L, G, cplx):
     assert rel_err(torch.view_as_real(st) if cplx else st, torch.view_as_real(st_ref) if cplx else st_ref) <= 1e-4
 
 
+@pytest.mark.parametrize("S,cplx,G", [(8, False, 64), (2, False, 1), (2, True, 4), (1, False, 64), (5, True, 2),
+                                      (12, False, 64)])
+def test_li_fewer_than_16_modes(S, cplx, G):
+    # state sizes of the older model configurations (8 and 2); odd sizes ride on the same fill-up
+    B, D, L = 2, 64, 1032
+    x2, x1, v = O.make_gates(B, D, L, seed=S)
+    lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(G, S, seed=7 + S)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(1)).bfloat16()
+    ref, y32_ref, st_ref = O.li_prefill(x2, x1, v, lp, r, Db)
+    out, y32, st = va.hyena_li_fwd(x1.cuda(), x2.cuda(), v.cuda(), lp.cuda(), r.cuda(), Db.cuda(),
+                                   want_state=True, want_fp32=True)
+    torch.cuda.synchronize()
+    assert rel_err(y32, y32_ref) <= 1e-4
+    assert rel_err(out, ref) <= 2e-2
+    assert st.dtype == st_ref.dtype and st.shape == st_ref.shape == (B, D, S)
+    assert rel_err(torch.view_as_real(st) if cplx else st, torch.view_as_real(st_ref) if cplx else st_ref) <= 1e-4
+
+
 def test_li_state_feeds_decode():
     # prefill on L tokens, then decode steps from the emitted state reproduce a longer prefill
     B, D, L, G, n_dec = 2, 32, 1024, 2, 4

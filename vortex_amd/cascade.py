@@ -309,7 +309,7 @@ class HyenaCascade(nn.Module):
             return None
         if fir and (inner.mode == HYENA_BIAS_ADD or (self.column_split_hyena and hd % 8)):
             return None
-        if not fir and inner.S == 8 and not inner.cplx:
+        if not fir and inner.S * (2 if inner.cplx else 1) < 16:      # the fused kernel needs three lanes per channel
             return None
         return ops.LayerStepper(ring, self.short_filter_weight.detach().reshape(3 * self.hidden_size, Ks),
                                 self.short_filter_bias, cmap, inner, flip_x1x2=self.hyena_flip_x1x2)

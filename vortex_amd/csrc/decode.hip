@@ -233,9 +233,17 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
 }
 
 // ---------------------------------------------------------------- IIR step
+// The floats of modal state that one lane owns, loaded and stored as one vector.
+template <int N>
+struct alignas(4 * N) StateVec {
+    float f[N];
+    __device__ __forceinline__ float& operator[](int i) { return f[i]; }
+    __device__ __forceinline__ float operator[](int i) const { return f[i]; }
+};
+
 // LPB lanes share one channel: each holds 16 bytes of its modal state (4 real or 2 complex
-// states), so state traffic is fully coalesced.  A lane walks NB batch elements of that channel
-// with the poles and residues held in registers and the NB state loads issued together, which
+// states; a channel with fewer than 16 bytes of state has one lane), so state traffic is fully
+// coalesced.  A lane walks NB batch elements of that channel with the poles and residues held in registers and the NB state loads issued together, which
 // puts enough bytes in flight to cover HBM latency.  The residue-weighted sum is reduced with
 // xor shuffles inside the lane group.
 // FEAT (fused featurizer step): 0 none; 2 lanes 0..2 of a lane group evaluate gates x2, x1, v of their channel
@@ -249,8 +257,10 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
                                                        const float* __restrict__ Dcoef, int d_is_bf16,
                                                        void* __restrict__ out, int out_is_fp32, int64_t out_bs,
                                                        int64_t B, int64_t D, int dg) {
-    constexpr int LPB = CPLX ? S / 2 : S / 4;      // lanes per channel
     constexpr int FPS = CPLX ? 2 : 1;              // floats per state
+    constexpr int VEC = S * FPS >= 4 ? 4 : S * FPS; // floats of state per lane (1 and 2 only where a channel has no more)
+    constexpr int LPB = S * FPS / VEC;             // lanes per channel
+    using fvec = StateVec<VEC>;
     constexpr int ND = 256 / LPB;                  // channels per block
     __shared__ float zs[(FEAT == 1 || FEAT == 3) ? NB * 3 * ND : 1];     // [j][gate-major or interleaved][channel]
     const uint32_t idx = blockIdx.x * 256 + threadIdx.x;        // (channel, lane of the group)
@@ -260,16 +270,16 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
     if (!chan_live) d = 0;
     const int64_t b0 = (int64_t)blockIdx.y * NB;
     const uint32_t g = d / (uint32_t)dg;
-    f32x4 st[NB];
+    fvec st[NB];
     bool live[NB];
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         live[j] = chan_live && b0 + j < B;
         const int64_t bd = live[j] ? (b0 + j) * D + d : 0;
-        st[j] = *(const f32x4*)(state + (bd * S) * FPS + q * 4);
+        st[j] = *(const fvec*)(state + (bd * S) * FPS + q * VEC);
     }
-    const f32x4 pp = *(const f32x4*)(poles + ((int64_t)g * S) * FPS + q * 4);
-    const f32x4 rr = *(const f32x4*)(residues + ((int64_t)g * S) * FPS + q * 4);
+    const fvec pp = *(const fvec*)(poles + ((int64_t)g * S) * FPS + q * VEC);
+    const fvec rr = *(const fvec*)(residues + ((int64_t)g * S) * FPS + q * VEC);
     const float dco = Dcoef[d];
     // fused featurizer: lanes 0..2 of the group evaluate gates x2, x1, v of every batch element first (their
     // loads overlap), the ring-slot stores follow, and only then the state updates start
@@ -345,21 +355,25 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
             c = bf_to_f(v[b * in_bs + d]);
         }
         const float x1v = round_bf(a * c);
-        f32x4 ns;
-        float part;
+        fvec ns;
+        float part = 0.f;
         if (CPLX) {
-            // (pr + i pi)(sr + i si) + x1v
-            ns[0] = fmaf(pp[0], st[j][0], -pp[1] * st[j][1]) + x1v;
-            ns[1] = fmaf(pp[0], st[j][1], pp[1] * st[j][0]);
-            ns[2] = fmaf(pp[2], st[j][2], -pp[3] * st[j][3]) + x1v;
-            ns[3] = fmaf(pp[2], st[j][3], pp[3] * st[j][2]);
-            part = (rr[0] * ns[0] - rr[1] * ns[1]) + (rr[2] * ns[2] - rr[3] * ns[3]);   // Re(r*s)
+            // (pr + i pi)(sr + i si) + x1v, then Re(r*s)
+#pragma unroll
+            for (int k = 0; k < VEC; k += 2) {
+                ns[k] = fmaf(pp[k], st[j][k], -pp[k + 1] * st[j][k + 1]) + x1v;
+                ns[k + 1] = fmaf(pp[k], st[j][k + 1], pp[k + 1] * st[j][k]);
+            }
+            if (VEC == 4) part = (rr[0] * ns[0] - rr[1] * ns[1]) + (rr[2] * ns[2] - rr[3] * ns[3]);
+            else part = rr[0] * ns[0] - rr[1] * ns[1];
         } else {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) ns[k] = fmaf(pp[k], st[j][k], x1v);
-            part = (rr[0] * ns[0] + rr[1] * ns[1]) + (rr[2] * ns[2] + rr[3] * ns[3]);
+            for (int k = 0; k < VEC; ++k) ns[k] = fmaf(pp[k], st[j][k], x1v);
+            if (VEC == 4) part = (rr[0] * ns[0] + rr[1] * ns[1]) + (rr[2] * ns[2] + rr[3] * ns[3]);
+            else if (VEC == 2) part = rr[0] * ns[0] + rr[1] * ns[1];
+            else part = rr[0] * ns[0];
         }
-        if (live[j]) *(f32x4*)(state + (((b0 + j) * D + d) * S) * FPS + q * 4) = ns;
+        if (live[j]) *(fvec*)(state + (((b0 + j) * D + d) * S) * FPS + q * VEC) = ns;
 #pragma unroll
         for (int m = 1; m < LPB; m <<= 1) part += __shfl_xor(part, m, 64);
         if (live[j] && q == 0) {
@@ -489,18 +503,19 @@ static int iir_step_launch(const void* x1, const void* x2, const void* v, int64_
     if (B < 0 || D <= 0 || G <= 0 || D % G != 0)
         return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld G=%lld", who, (long long)B, (long long)D,
                           (long long)G);
-    if (S != 16 && S != 8 && S != 32)
-        return hyena_fail(HYENA_ENOSUP, "%s: state size %lld (8, 16 or 32 supported)", who, (long long)S);
+    if (S < 1 || S > 32 || (S & (S - 1)))
+        return hyena_fail(HYENA_ENOSUP, "%s: state size %lld (powers of two up to 32 supported)", who, (long long)S);
     if (((uintptr_t)state & 15) || ((uintptr_t)poles & 15) || ((uintptr_t)residues & 15))
         return hyena_fail(HYENA_EALIGN, "%s: state, poles, residues must be 16-byte aligned", who);
     ProjArgs pj = {};
     if (proj) {
         if (int rc = make_proj(proj, D, who, &pj)) return rc;
-        if (!is_complex && S == 8) return hyena_fail(HYENA_ENOSUP, "%s: fused featurizer with 8 real states", who);
+        if (S * (is_complex ? 2 : 1) < 16)
+            return hyena_fail(HYENA_ENOSUP, "%s: fused featurizer with fewer than 16 real / 8 complex states", who);
     }
     if (B == 0) return 0;
     const int dg = (int)(D / G);
-    const int lpb = is_complex ? (int)S / 2 : (int)S / 4;
+    const int lpb = (int)(S * (is_complex ? 2 : 1) >= 4 ? S * (is_complex ? 2 : 1) / 4 : 1);
     if (D * lpb > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: D too large", who);
     // four batch elements per lane when that still leaves a few wavefronts per SIMD; else one
     const int nb = (B >= 4 && B * D * lpb >= 4 * 256 * 1024) ? 4 : 1;
@@ -517,6 +532,8 @@ static int iir_step_launch(const void* x1, const void* x2, const void* v, int64_
 #define IIR_CASE(SS, C, F)                                                                                      \
     if (S == SS && (is_complex != 0) == C && feat == F) { if (nb == 4) IIR_GO(SS, C, F, 4); else IIR_GO(SS, C, F, 1); }
 #define IIR_FEATS(SS, C) IIR_CASE(SS, C, 1) IIR_CASE(SS, C, 2) IIR_CASE(SS, C, 3)
+    IIR_CASE(1, false, 0) IIR_CASE(2, false, 0) IIR_CASE(4, false, 0)
+    IIR_CASE(1, true, 0) IIR_CASE(2, true, 0) IIR_CASE(4, true, 0)
     IIR_CASE(8, false, 0) IIR_CASE(16, false, 0) IIR_CASE(32, false, 0)
     IIR_CASE(8, true, 0) IIR_CASE(16, true, 0) IIR_CASE(32, true, 0)
     IIR_FEATS(16, false) IIR_FEATS(32, false) IIR_FEATS(8, true) IIR_FEATS(16, true) IIR_FEATS(32, true)

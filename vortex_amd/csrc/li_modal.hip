@@ -96,13 +96,15 @@ __device__ __forceinline__ int li_sample(int ib, int m) { return 8 * (m >> 2) + 
 // One block per group; coefficients evaluated in double from the fp32 parameters.
 __global__ __launch_bounds__(256) void li_plan_kernel(const float* __restrict__ log_poles,   // [G][S][2]
                                                       const float* __restrict__ residues,    // [G][S][2]
-                                                      float* __restrict__ ws) {
+                                                      float* __restrict__ ws,
+                                                      int sr) {                              // modes given, <= S
     const int g = blockIdx.x, tid = threadIdx.x;
     float* w = ws + (size_t)g * WS_GROUP;
-    const float* lp = log_poles + (size_t)g * S * 2;
-    const float* rs = residues + (size_t)g * S * 2;
-    // p^k = exp(k*lr) * (cos(k*th), sin(k*th))
+    const float* lp = log_poles + (size_t)g * sr * 2;
+    const float* rs = residues + (size_t)g * sr * 2;
+    // p^k = exp(k*lr) * (cos(k*th), sin(k*th)); the modes past sr are p = 1 with residue 0, which add nothing
     auto ppow = [&](int s, int k, double& re, double& im) {
+        if (s >= sr) { re = 1.0; im = 0.0; return; }
         const double m = exp((double)k * (double)lp[2 * s]);
         const double a = (double)k * (double)lp[2 * s + 1];
         re = m * cos(a);
@@ -110,7 +112,7 @@ __global__ __launch_bounds__(256) void li_plan_kernel(const float* __restrict__ 
     };
     if (tid < C) {                                  // filter head h[0..127]
         double acc = 0.0;
-        for (int s = 0; s < S; ++s) {
+        for (int s = 0; s < sr; ++s) {
             double re, im;
             ppow(s, tid, re, im);
             acc += (double)rs[2 * s] * re - (double)rs[2 * s + 1] * im;
@@ -130,7 +132,7 @@ __global__ __launch_bounds__(256) void li_plan_kernel(const float* __restrict__ 
         ppow(s, b, re, im);
         w[WS_P1 + 2 * tid] = (float)re;
         w[WS_P1 + 2 * tid + 1] = (float)im;
-        const double rr = rs[2 * s], ri = rs[2 * s + 1];
+        const double rr = s < sr ? rs[2 * s] : 0.f, ri = s < sr ? rs[2 * s + 1] : 0.f;
         w[WS_R1 + 2 * tid] = (float)(rr * re - ri * im);
         w[WS_R1 + 2 * tid + 1] = (float)(rr * im + ri * re);
     }
@@ -161,7 +163,8 @@ struct LiArgs {
     const float* Dcoef;       // [D] or null
     bf16_t* out;              // [B][D][L]
     float* y32;               // optional [B][D][L] fp32 convolution output (before any rounding)
-    float* state_out;         // optional [B][D][S][2]
+    float* state_out;         // optional [B][D][sr][2]
+    int sr;                   // modes the caller has (<= S)
     int64_t D, L;
     int dg;
     int d_is_bf16;
@@ -499,8 +502,8 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
         }
         Xr = Xfr;
         Xi = Xfi;
-        if (CPW == 4 || lane < 16) {
-            float* sp_ = a.state_out + ((b * a.D + d0 + sc) * S + sp) * 2;
+        if ((CPW == 4 || lane < 16) && sp < a.sr) {
+            float* sp_ = a.state_out + ((b * a.D + d0 + sc) * a.sr + sp) * 2;
             sp_[0] = Xr * fr_ - Xi * fi;
             sp_[1] = Xr * fi + Xi * fr_;
         }
@@ -510,7 +513,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
 }  // namespace
 
 extern "C" int64_t hyena_li_plan_bytes(int64_t G, int64_t S_) {
-    if (G <= 0 || S_ != S) return 0;
+    if (G <= 0 || S_ < 1 || S_ > S) return 0;
     return (int64_t)G * WS_GROUP * (int64_t)sizeof(float);
 }
 
@@ -518,10 +521,10 @@ extern "C" int hyena_li_plan(const float* log_poles, const float* residues, int6
                              void* stream) {
     if (!log_poles || !residues || !workspace) return hyena_fail(HYENA_EINVAL, "hyena_li_plan: null pointer");
     if (G <= 0 || G > 0x7fffffff) return hyena_fail(HYENA_EINVAL, "hyena_li_plan: bad G=%lld", (long long)G);
-    if (S_ != S) return hyena_fail(HYENA_ENOSUP, "hyena_li_plan: state size %lld (only 16)", (long long)S_);
+    if (S_ < 1 || S_ > S) return hyena_fail(HYENA_ENOSUP, "hyena_li_plan: state size %lld (1..16)", (long long)S_);
     if (((uintptr_t)workspace) & 15) return hyena_fail(HYENA_EALIGN, "hyena_li_plan: workspace must be 16-byte aligned");
     hipLaunchKernelGGL(li_plan_kernel, dim3((unsigned)G), dim3(256), 0, (hipStream_t)stream, log_poles, residues,
-                       (float*)workspace);
+                       (float*)workspace, (int)S_);
     return hyena_check_launch("hyena_li_plan");
 }
 
@@ -533,7 +536,7 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     if (B < 0 || D <= 0 || L < 0 || G <= 0 || D % G != 0)
         return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: bad sizes B=%lld D=%lld L=%lld G=%lld", (long long)B,
                           (long long)D, (long long)L, (long long)G);
-    if (S_ != S) return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: state size %lld (only 16)", (long long)S_);
+    if (S_ < 1 || S_ > S) return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: state size %lld (1..16)", (long long)S_);
     if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15) ||
         (((uintptr_t)y_conv_fp32) & 15) || (((uintptr_t)workspace) & 15))
         return hyena_fail(HYENA_EALIGN, "hyena_li_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
@@ -554,6 +557,7 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     a.out = (bf16_t*)out;
     a.y32 = y_conv_fp32;
     a.state_out = state_out;
+    a.sr = (int)S_;
     a.D = D;
     a.L = L;
     a.dg = (int)(D / G);

@@ -260,7 +260,7 @@ class ModalPlan:
         self._lp, self._rs = pairs(lp), pairs(rs)
         nbytes = _lib.lib().hyena_li_plan_bytes(self.G, self.S)
         if nbytes <= 0:
-            raise NotImplementedError(f"modal state size {self.S} is not supported (16 only)")
+            raise NotImplementedError(f"modal state size {self.S} is not supported (1..16)")
         self.workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=lp.device)
         rc = _lib.lib().hyena_li_plan(_ptr(self._lp), _ptr(self._rs), self.G, self.S, _ptr(self.workspace), _stream())
         _lib.check(rc, "hyena_li_plan")
