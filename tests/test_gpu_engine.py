@@ -168,6 +168,42 @@ def test_operator_module_any_prompt_length(kind, L):
             assert rel_err(y_hip, y_ref) <= 2e-2, (fused, i)
 
 
+@pytest.mark.parametrize("D,H,G", [(640, 10, 64), (768, 12, 64), (1920, 15, 128)])
+@pytest.mark.parametrize("kind", ["se", "mr", "li_real"])
+def test_operator_module_reference_model_geometries(kind, D, H, G):
+    # hidden size / heads / filter groups of shc-evo2-50m-8k-1T.yml, shc-evo2-100m-8k-1T.yml and evo2-1b-8k.yml:
+    # groups of 10, 12 and 15 channels; the long-filter layers have one filter per channel
+    B, L, n_dec = 1, 264, 3
+    K = {"se": 7, "mr": 128}.get(kind)
+    Gk = G if K else D
+    p = make_params(kind, D, Gk, seed=D)
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=False, interleave=True, short_filter_length=3,
+               short_filter_bias=False, state_size=16)
+    ref = O.OracleCascade(O.OracleEngine(), p, D, H, Gk, fir_inner_filter_length=K, interleave=True)
+    u_all = torch.randn(B, L + n_dec, 3 * D, generator=torch.Generator().manual_seed(D)).bfloat16()
+    mod = HyenaCascade(cfg, 0, hyena_filter_groups=Gk, fir_inner_filter_length=K)
+    with torch.no_grad():
+        mod.short_filter_weight.copy_(p["short_filter_weight"])
+        if K:
+            mod.h.copy_(p["h"])
+        else:
+            mod.log_poles.copy_(p["log_poles"])
+            mod.residues.copy_(p["residues"])
+        if mod.D is not None:
+            mod.D.data = p["D"].clone()
+    mod = mod.to(DEV)
+    ip_ref = O.OracleCache()
+    ip_hip = HyenaCascadeFIRInferenceParams() if K else HyenaCascadeIIRInferenceParams()
+    y_ref, _ = ref.forward(u_all[:, :L], ip_ref)
+    y_hip, _ = mod(u_all[:, :L].to(DEV), ip_hip)
+    assert rel_err(y_hip, y_ref) <= 2e-2
+    for i in range(n_dec):
+        tok = u_all[:, L + i: L + i + 1]
+        y_ref, _ = ref.forward(tok, ip_ref)
+        y_hip, _ = mod(tok.to(DEV), ip_hip)
+        assert rel_err(y_hip, y_ref) <= 2e-2, i
+
+
 @pytest.mark.parametrize("S,bias,L", [(8, False, 512), (2, True, 512), (2, True, 37), (4, False, 200)])
 def test_operator_module_small_state_sizes(S, bias, L):
     # the long-filter layers of the older configurations: state_size 8 (shc-evo2-7b-8k-2T-v1.yml) and 2
