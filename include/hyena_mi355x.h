@@ -182,6 +182,7 @@ typedef struct hyena_proj_step {
     const float* bias;        /* [3D] float32 or NULL                                              */
     int64_t ch_inner, ch_outer, gate_stride, ch_stride;
     int flip_x1x2;
+    const int32_t* pos_dev;   /* NULL, or the ring position in device memory (then pos is ignored)  */
 } hyena_proj_step;
 
 /* hyena_fir_step / hyena_iir_step with the featurizer step of the same layer fused in: one launch per
@@ -200,6 +201,24 @@ int hyena_iir_layer_step(const hyena_proj_step* proj,
                          const float* Dcoef, int d_is_bf16,
                          void* out, int out_is_fp32, int64_t out_batch_stride,
                          int64_t B, int64_t D, int64_t G, int64_t S, void* stream);
+
+/* Ring positions in device memory, for callers that replay a recorded token step (a HIP graph) and so cannot
+ * change a scalar argument between tokens.  No counterpart in the reference, whose caches have no position
+ * (vortex/model/engine.py:443-447 shifts the whole cache each token).  The _dpos forms read the position of the
+ * inner cache from *pos_dev (reduced mod R); hyena_proj_step.pos_dev does the same for the featurizer cache in
+ * every layer step.  hyena_ring_advance moves n positions on by one slot, pos[i] = (pos[i] + 1) % depth[i]:
+ * one launch per token for all the rings of a model, after the layer steps of that token. */
+int hyena_fir_step_dpos(const void* x1, const void* x2, const void* v, int64_t in_batch_stride,
+                        void* ring, int64_t R, const int32_t* pos_dev,
+                        const float* w, const float* bias, int bias_mode,
+                        void* out, int64_t out_batch_stride,
+                        int64_t B, int64_t D, int64_t G, void* stream);
+int hyena_fir_layer_step_dpos(const hyena_proj_step* proj,
+                              void* ring, int64_t R, const int32_t* pos_dev,
+                              const float* w, const float* bias, int bias_mode,
+                              void* out, int64_t out_batch_stride,
+                              int64_t B, int64_t D, int64_t G, void* stream);
+int hyena_ring_advance(int32_t* pos, const int32_t* depth, int64_t n, void* stream);
 
 /* Channel-last operand [B][L][D]: element (b, t, d) at ptr + b*batch_stride + t*time_stride + d (elements).
  * This is the (batch, seqlen, groups, group_dim) layout of vortex/ops/hyena_se/fwd.py:17-43 with D = groups*group_dim. */

@@ -191,3 +191,41 @@ def test_layer_steps_random(B, D, H, Ks, layout, flip, sbias, seed):
         assert rel_err(y2, y2_ref.real if cplx else y2_ref) <= 2e-2, ("iir", i, S, cplx)
     assert rel_err(ring.reference_order(), ref_s) <= 1e-2
     assert rel_err(torch.view_as_real(state) if cplx else state, torch.view_as_real(ref_m) if cplx else ref_m) <= 1e-2
+
+
+def test_ring_positions_on_the_device():
+    # hyena_fir_step_dpos / hyena_fir_layer_step_dpos / hyena_ring_advance: the same steps with the ring positions
+    # kept in device memory give bit-identical outputs and caches
+    B, D, G, K, Ks = 3, 512, 32, 7, 3
+    g = torch.Generator().manual_seed(5)
+    w = torch.randn(G, K, generator=g).cuda()
+    fw = torch.randn(3 * D, Ks, generator=g).cuda()
+    cmap = ops.gate_channel_map(D, interleave=True)
+
+    def fresh():
+        gg = torch.Generator().manual_seed(6)
+        fr = ops.FirRing(torch.randn(B, Ks - 1, 3 * D, generator=gg).bfloat16().cuda(), 1)
+        ir = ops.FirRing(torch.randn(B, K - 1, D, generator=gg).bfloat16().cuda(), 4)
+        return fr, ir, ops.LayerStepper(fr, fw, None, cmap, ops.FirStepper(ir, w))
+
+    fr_h, ir_h, step_h = fresh()
+    fr_d, ir_d, step_d = fresh()
+    clock = ops.RingClock([fr_d, ir_d])
+    for t in range(15):
+        u = torch.randn(B, 3 * D, generator=g).bfloat16().cuda()
+        y_h = step_h(u, torch.empty(B, D, dtype=torch.bfloat16, device="cuda"))
+        y_d = step_d(u, torch.empty(B, D, dtype=torch.bfloat16, device="cuda"))
+        clock.advance()
+        assert torch.equal(y_h, y_d), t
+    assert clock.pos.tolist() == [fr_h.pos, ir_h.pos]
+    assert torch.equal(fr_h.reference_order(), fr_d.reference_order())
+    assert torch.equal(ir_h.reference_order(), ir_d.reference_order())
+    # the plain (unfused) step through the same clock
+    x1, x2, v = (torch.randn(B, D, generator=g).bfloat16().cuda() for _ in range(3))
+    y_d = va.fir_step(x1, ir_d, w, x2=x2, v=v)
+    y_h = va.fir_step(x1, ir_h, w, x2=x2, v=v)
+    clock.advance()
+    assert torch.equal(y_h, y_d)
+    clock.release()
+    assert ir_d.pos == ir_h.pos and ir_d.pos_dev is None
+    assert fr_d.pos == (fr_h.pos + 1) % (Ks - 1)          # the clock moved this ring too; no step used it

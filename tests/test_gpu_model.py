@@ -48,3 +48,59 @@ def test_cached_generation_matches_a_longer_prefill(L):
     want = full[:, L - 1:L + n - 1]                        # step i predicts token L + i from position L + i - 1
     err = (scores.float() - want).abs().max() / want.abs().max()
     assert err <= 3e-2, err                                # bf16 GEMM / SDPA paths differ between prefill and decode
+
+
+@pytest.mark.parametrize("L,attn", [(256, True), (203, True), (256, False), (203, False)])
+def test_recorded_token_step_matches_eager_generation(L, attn):
+    # the token step replayed as a HIP graph (ring positions and the attention position in device memory) against
+    # the eager loop, teacher-forced over enough tokens for every ring to wrap (the featurizer ring every 2 tokens,
+    # the Hyena-SE ring every 6), with the host reading results and synchronising between replays
+    cfg = dict(EVO2_7B, hidden_size=128, num_layers=8, num_attention_heads=4, inner_mlp_size=256,
+               hcs_filter_groups=8, hcm_filter_groups=8, hcl_filter_groups=128,
+               pattern=("hcs", "hcm", "hcl", "attn") if attn else ("hcs", "hcm", "hcl"))
+    m = StripedHyena2(cfg, seed=5, device="cuda").to_inference("cuda")
+    n = 20
+    ids = torch.randint(0, 512, (2, L + n), device="cuda", generator=torch.Generator(device="cuda").manual_seed(8))
+    toks_e, scores_e = m.generate(ids[:, :L], n, forced=ids[:, L:])
+    toks_g, scores_g = m.generate(ids[:, :L], n, forced=ids[:, L:], graph=True)
+    torch.cuda.synchronize()
+    assert torch.equal(toks_e, toks_g)
+    for i in range(n):
+        want, got = scores_e[:, i].float(), scores_g[:, i].float()
+        if attn:        # the recorded attention step (masked full-length cache) is another SDPA path: bf16 noise
+            err = (got - want).abs().max() / want.abs().max()
+            assert err <= 3e-2, (i, err.item())
+        else:           # Hyena blocks only: the same kernels on the same data
+            assert torch.equal(got, want), i
+    # a second generation on the same model records a fresh step and still agrees
+    toks_g2, scores_g2 = m.generate(ids[:, :L], n, forced=ids[:, L:], graph=True)
+    assert torch.equal(scores_g2, scores_g)
+
+
+def test_recorded_step_then_eager_steps():
+    # release() hands ring positions back to the host: eager steps after recorded ones continue the same sequence
+    from vortex_amd.model import RecordedDecodeStep
+    cfg = dict(EVO2_7B, hidden_size=128, num_layers=4, num_attention_heads=4, inner_mlp_size=256,
+               hcs_filter_groups=8, hcm_filter_groups=8, hcl_filter_groups=128)
+    m = StripedHyena2(cfg, seed=7, device="cuda").to_inference("cuda")
+    L, n = 200, 9
+    ids = torch.randint(0, 512, (1, L + n), device="cuda", generator=torch.Generator(device="cuda").manual_seed(9))
+    _, want = m.generate(ids[:, :L], n, forced=ids[:, L:])
+
+    with torch.no_grad():
+        ipd = m.initialize_inference_params(max_seqlen=L + n)
+        got = [m(ids[:, :L], ipd)[:, -1]]
+        rec = None
+        for i in range(1, n):
+            for p in ipd.values():
+                p.seqlen_offset = L if p.seqlen_offset == 0 else p.seqlen_offset + 1
+            x = ids[:, L + i - 1:L + i]
+            if i == 2:
+                rec = RecordedDecodeStep(m, ipd, 1)
+            if i == 6:
+                rec.release()
+                rec = None
+            got.append((m(x, ipd) if rec is None else rec(x))[:, -1])
+    got = torch.stack(got, 1).float()
+    err = (got - want.float()).abs().max() / want.float().abs().max()
+    assert err <= 3e-2, err

@@ -109,9 +109,9 @@ def test_gate_channel_map_matches_reference_split(cs, il):
 
 def test_proj_structs_match_header():
     from vortex_amd import _lib
-    # hyena_proj_step: 7 pointer/int64 fields, 4 int64 map fields, one int (padded to 8)
-    assert ctypes.sizeof(_lib.ProjStep) == 12 * 8
-    assert _lib.ProjStep.flip_x1x2.offset == 11 * 8
+    # hyena_proj_step: 7 pointer/int64 fields, 4 int64 map fields, one int (padded to 8), one pointer
+    assert ctypes.sizeof(_lib.ProjStep) == 13 * 8
+    assert _lib.ProjStep.flip_x1x2.offset == 11 * 8 and _lib.ProjStep.pos_dev.offset == 12 * 8
     # hyena_proj_fwd: 5 pointer/int64 fields, two ints, 4 int64 map fields
     assert ctypes.sizeof(_lib.ProjFwd) == 10 * 8
     assert _lib.ProjFwd.Ks.offset == 5 * 8 and _lib.ProjFwd.flip_x1x2.offset == 5 * 8 + 4

@@ -15,6 +15,7 @@ EXPORTS = [
     "hyena_version", "hyena_last_error_string", "hyena_se_fwd", "hyena_mr_fwd",
     "hyena_fir_step", "hyena_iir_step", "hyena_li_plan_bytes", "hyena_li_plan", "hyena_li_fwd", "hyena_featurizer_fwd", "hyena_copy_probe",
     "hyena_fir_layer_step", "hyena_iir_layer_step", "hyena_fir_cl_fwd", "hyena_fir_layer_fwd",
+    "hyena_fir_step_dpos", "hyena_fir_layer_step_dpos", "hyena_ring_advance",
 ]
 
 
@@ -27,7 +28,7 @@ class ProjStep(Structure):
     """hyena_proj_step: the featurizer decode step a layer step evaluates on the fly."""
     _fields_ = [("u", c_void_p), ("u_batch_stride", c_int64), ("ring", c_void_p), ("Rf", c_int64), ("pos", c_int64),
                 ("w", c_void_p), ("bias", c_void_p), ("ch_inner", c_int64), ("ch_outer", c_int64),
-                ("gate_stride", c_int64), ("ch_stride", c_int64), ("flip_x1x2", c_int)]
+                ("gate_stride", c_int64), ("ch_stride", c_int64), ("flip_x1x2", c_int), ("pos_dev", c_void_p)]
 
 
 class Cl(Structure):
@@ -78,6 +79,11 @@ def lib():
                                        c_int64, c_int64, c_int64, c_void_p]
     L.hyena_iir_layer_step.argtypes = [P, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                                        c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p]
+    L.hyena_fir_step_dpos.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p,
+                                      c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p]
+    L.hyena_fir_layer_step_dpos.argtypes = [P, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                            c_int64, c_int64, c_int64, c_int64, c_void_p]
+    L.hyena_ring_advance.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
     C = POINTER(Cl)
     L.hyena_fir_cl_fwd.argtypes = [C, C, C, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64,
                                    c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]

@@ -16,12 +16,17 @@ struct ProjArgs {
     int64_t u_bs;
     bf16_t* ring;
     int Rf, pos, C;
+    const int* pos_dev;    // when set, the ring position lives in device memory and pos is ignored
     const float* w;        // [Rf+1][C], tap-major
     const float* bias;     // [C] or null
     uint32_t ch_inner, ch_outer, gate_stride, ch_stride;
     int flip;
     __device__ __forceinline__ uint32_t chan(uint32_t gate, uint32_t d) const {
         return (d / ch_inner) * ch_outer + gate * gate_stride + (d % ch_inner) * ch_stride;
+    }
+    // a device-resident position is reduced mod Rf so that a stale or foreign counter cannot index past the ring
+    __device__ __forceinline__ void resolve_pos() {
+        if (pos_dev) pos = (int)((uint32_t)*pos_dev % (uint32_t)Rf);
     }
 };
 
@@ -76,9 +81,12 @@ template <bool PRE, bool POST, int BIAS, bool GROUPED, int NSG, int FEAT>
 __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __restrict__ x1, const bf16_t* __restrict__ x2,
                                                        const bf16_t* __restrict__ v, int64_t in_bs, ProjArgs pj,
                                                        bf16_t* __restrict__ ring, int R, int pos,
+                                                       const int* __restrict__ pos_dev,
                                                        const float* __restrict__ w, const float* __restrict__ bias,
                                                        bf16_t* __restrict__ out, int64_t out_bs, int64_t D, int dg) {
     extern __shared__ float smem[];
+    if (pos_dev) pos = (int)((uint32_t)*pos_dev % (uint32_t)R);
+    if (FEAT != 0) pj.resolve_pos();
     const int tid = threadIdx.x, oc = tid & 63, sg = tid >> 6;
     const int64_t dblk = (int64_t)blockIdx.x * 512;
     const int64_t d0 = dblk + oc * 8;
@@ -263,6 +271,7 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
     using fvec = StateVec<VEC>;
     constexpr int ND = 256 / LPB;                  // channels per block
     __shared__ float zs[(FEAT == 1 || FEAT == 3) ? NB * 3 * ND : 1];     // [j][gate-major or interleaved][channel]
+    if (FEAT != 0) pj.resolve_pos();
     const uint32_t idx = blockIdx.x * 256 + threadIdx.x;        // (channel, lane of the group)
     const int q = (int)(idx % LPB);
     uint32_t d = idx / LPB;
@@ -391,7 +400,7 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
 // Validates a fused-featurizer descriptor and converts it; returns 0 or an error code.
 static int make_proj(const hyena_proj_step* p, int64_t D, const char* who, ProjArgs* out) {
     if (!p->u || !p->ring || !p->w) return hyena_fail(HYENA_EINVAL, "%s: proj u, ring, w are required", who);
-    if (p->Rf < 1 || p->Rf > 7 || p->pos < 0 || p->pos >= p->Rf)
+    if (p->Rf < 1 || p->Rf > 7 || (!p->pos_dev && (p->pos < 0 || p->pos >= p->Rf)))
         return hyena_fail(HYENA_EINVAL, "%s: featurizer cache depth %lld / position %lld", who, (long long)p->Rf,
                           (long long)p->pos);
     const int64_t C = 3 * D;
@@ -401,7 +410,7 @@ static int make_proj(const hyena_proj_step* p, int64_t D, const char* who, ProjA
     if (last >= C) return hyena_fail(HYENA_EINVAL, "%s: featurizer channel map reaches channel %lld of %lld", who,
                                      (long long)last, (long long)C);
     out->u = (const bf16_t*)p->u; out->u_bs = p->u_batch_stride; out->ring = (bf16_t*)p->ring;
-    out->Rf = (int)p->Rf; out->pos = (int)p->pos; out->C = (int)C; out->w = p->w; out->bias = p->bias;
+    out->Rf = (int)p->Rf; out->pos = p->pos_dev ? 0 : (int)p->pos; out->pos_dev = (const int*)p->pos_dev; out->C = (int)C; out->w = p->w; out->bias = p->bias;
     out->ch_inner = (uint32_t)(p->ch_inner > D ? D : p->ch_inner); out->ch_outer = (uint32_t)p->ch_outer;
     out->gate_stride = (uint32_t)p->gate_stride; out->ch_stride = (uint32_t)p->ch_stride; out->flip = p->flip_x1x2 != 0;
     return 0;
@@ -418,9 +427,11 @@ static int proj_vector_mode(const hyena_proj_step* p, int64_t D) {
 }
 
 static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_t in_bs, const hyena_proj_step* proj,
-                           void* ring, int64_t R, int64_t pos, const float* w, const float* bias, int bias_mode,
-                           void* out, int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream, const char* who) {
+                           void* ring, int64_t R, int64_t pos, const int32_t* pos_dev, const float* w, const float* bias,
+                           int bias_mode, void* out, int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream,
+                           const char* who) {
     if ((!proj && !x1) || !ring || !w || !out) return hyena_fail(HYENA_EINVAL, "%s: x1, ring, w, out are required", who);
+    if (pos_dev) pos = 0;
     if (B < 0 || D <= 0 || G <= 0 || D % G != 0 || R < 1 || R > 4096 || pos < 0 || pos >= R)
         return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld G=%lld R=%lld pos=%lld", who, (long long)B,
                           (long long)D, (long long)G, (long long)R, (long long)pos);
@@ -454,7 +465,7 @@ static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_
     bool ok = false;
 #define FS_GO(P, Q, M, GR, N, F)                                                                              \
     hipLaunchKernelGGL((fir_step_kernel<P, Q, M, GR, N, F>), grid, dim3(64 * N), sh, s, p1, p2, pv, in_bs, pj, \
-                       (bf16_t*)ring, (int)R, (int)pos, w, bias, (bf16_t*)out, out_bs, D, dg)
+                       (bf16_t*)ring, (int)R, (int)pos, (const int*)pos_dev, w, bias, (bf16_t*)out, out_bs, D, dg)
 #define FS_CASE(P, Q, M, F)                                                                                   \
     if (!ok && pre == P && post == Q && bias_mode == M && feat == F) {                                        \
         if (grouped && nsg == 8) FS_GO(P, Q, M, true, 8, F);                                                  \
@@ -482,16 +493,51 @@ static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_
 extern "C" int hyena_fir_step(const void* x1, const void* x2, const void* v, int64_t in_bs, void* ring, int64_t R,
                               int64_t pos, const float* w, const float* bias, int bias_mode, void* out,
                               int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream) {
-    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, pos, w, bias, bias_mode, out, out_bs, B, D, G, stream,
-                           "hyena_fir_step");
+    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, pos, nullptr, w, bias, bias_mode, out, out_bs, B, D, G,
+                           stream, "hyena_fir_step");
+}
+
+extern "C" int hyena_fir_step_dpos(const void* x1, const void* x2, const void* v, int64_t in_bs, void* ring, int64_t R,
+                                   const int32_t* pos_dev, const float* w, const float* bias, int bias_mode,
+                                   void* out, int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream) {
+    if (!pos_dev) return hyena_fail(HYENA_EINVAL, "hyena_fir_step_dpos: pos_dev is required");
+    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, 0, pos_dev, w, bias, bias_mode, out, out_bs, B, D, G,
+                           stream, "hyena_fir_step_dpos");
 }
 
 extern "C" int hyena_fir_layer_step(const hyena_proj_step* proj, void* ring, int64_t R, int64_t pos, const float* w,
                                     const float* bias, int bias_mode, void* out, int64_t out_bs, int64_t B,
                                     int64_t D, int64_t G, void* stream) {
     if (!proj) return hyena_fail(HYENA_EINVAL, "hyena_fir_layer_step: proj is required");
-    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, pos, w, bias, bias_mode, out, out_bs, B, D, G,
-                           stream, "hyena_fir_layer_step");
+    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, pos, nullptr, w, bias, bias_mode, out, out_bs, B,
+                           D, G, stream, "hyena_fir_layer_step");
+}
+
+extern "C" int hyena_fir_layer_step_dpos(const hyena_proj_step* proj, void* ring, int64_t R, const int32_t* pos_dev,
+                                         const float* w, const float* bias, int bias_mode, void* out, int64_t out_bs,
+                                         int64_t B, int64_t D, int64_t G, void* stream) {
+    if (!proj || !pos_dev) return hyena_fail(HYENA_EINVAL, "hyena_fir_layer_step_dpos: proj and pos_dev are required");
+    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, 0, pos_dev, w, bias, bias_mode, out, out_bs, B, D,
+                           G, stream, "hyena_fir_layer_step_dpos");
+}
+
+namespace {
+__global__ void ring_advance_kernel(int* __restrict__ pos, const int* __restrict__ depth, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const int p = pos[i] + 1;
+        pos[i] = p >= depth[i] ? 0 : p;
+    }
+}
+}  // namespace
+
+extern "C" int hyena_ring_advance(int32_t* pos, const int32_t* depth, int64_t n, void* stream) {
+    if (!pos || !depth) return hyena_fail(HYENA_EINVAL, "hyena_ring_advance: null pointer");
+    if (n < 0 || n > (1 << 24)) return hyena_fail(HYENA_EINVAL, "hyena_ring_advance: bad n=%lld", (long long)n);
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(ring_advance_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, pos,
+                       depth, (int)n);
+    return hyena_check_launch("hyena_ring_advance");
 }
 
 static int iir_step_launch(const void* x1, const void* x2, const void* v, int64_t in_bs, const hyena_proj_step* proj,

@@ -16,6 +16,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import ops
 from .cascade import HyenaCascade, HyenaCascadeFIRInferenceParams, HyenaCascadeIIRInferenceParams
 
 EVO2_7B = dict(
@@ -62,7 +63,10 @@ def _rotary(x, base, offset=0):
     """x [B, L, H, hd]; non-interleaved rotary embedding over the whole head dimension."""
     B, L, H, hd = x.shape
     inv = 1.0 / (base ** (torch.arange(0, hd, 2, device=x.device, dtype=torch.float32) / hd))
-    t = torch.arange(offset, offset + L, device=x.device, dtype=torch.float32)
+    if isinstance(offset, torch.Tensor):            # position kept on the device (recorded token step)
+        t = offset.to(torch.float32) + torch.arange(L, device=x.device, dtype=torch.float32)
+    else:
+        t = torch.arange(offset, offset + L, device=x.device, dtype=torch.float32)
     f = torch.outer(t, inv)
     cos, sin = f.cos()[None, :, None].to(x.dtype), f.sin()[None, :, None].to(x.dtype)
     x1, x2 = x[..., : hd // 2], x[..., hd // 2:]
@@ -71,11 +75,12 @@ def _rotary(x, base, offset=0):
 
 class AttentionInferenceParams:
     """Key / value cache of the attention blocks (the role of vortex/model/cache.py:8-28): per layer two
-    [B, max_seqlen, H, head_dim] tensors, filled up to seqlen_offset."""
+    [B, H, max_seqlen, head_dim] tensors, filled up to seqlen_offset."""
 
     def __init__(self, max_seqlen):
         self.max_seqlen, self.seqlen_offset = max_seqlen, 0
         self.key_value_memory_dict = {}
+        self.offset_dev = None      # int64 [1] device tensor while a recorded token step owns the position
 
 
 class AttentionBlock(nn.Module):
@@ -90,20 +95,40 @@ class AttentionBlock(nn.Module):
 
     def forward(self, u, inference_params=None):
         B, L, D = u.shape
-        qkv = self.Wqkv(self.pre_norm(u)).view(B, L, 3, self.H, D // self.H)
+        hd = D // self.H
+        qkv = self.Wqkv(self.pre_norm(u)).view(B, L, 3, self.H, hd)
         cached = inference_params is not None and self.layer_idx in inference_params.key_value_memory_dict
-        off = inference_params.seqlen_offset if cached else 0
-        q, k, v = _rotary(qkv[:, :, 0], self.base, off), _rotary(qkv[:, :, 1], self.base, off), qkv[:, :, 2]
+        on_device = cached and inference_params.offset_dev is not None
+        off = inference_params.offset_dev if on_device else (inference_params.seqlen_offset if cached else 0)
+        q, k = _rotary(qkv[:, :, 0], self.base, off).transpose(1, 2), _rotary(qkv[:, :, 1], self.base, off).transpose(1, 2)
+        v = qkv[:, :, 2].transpose(1, 2)                                    # [B, H, L, hd]
+        if inference_params is not None and not cached:
+            # zero-filled: the recorded token step reads every row (masked), and 0 * garbage could be NaN
+            kc = k.new_zeros(B, self.H, inference_params.max_seqlen, hd)
+            inference_params.key_value_memory_dict[self.layer_idx] = (kc, torch.zeros_like(kc))
         if inference_params is not None:
-            if not cached:
-                kc = k.new_empty(B, inference_params.max_seqlen, self.H, D // self.H)
-                inference_params.key_value_memory_dict[self.layer_idx] = (kc, torch.empty_like(kc))
             kc, vc = inference_params.key_value_memory_dict[self.layer_idx]
-            kc[:, off:off + L], vc[:, off:off + L] = k, v
-            if cached:              # decode: the new queries see the whole cache (one token: no mask needed)
-                k, v = kc[:, :off + L], vc[:, :off + L]
-        o = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
-                                           is_causal=not cached)
+            if on_device:
+                kc.index_copy_(2, off, k)
+                vc.index_copy_(2, off, v)
+            else:
+                kc[:, :, off:off + L], vc[:, :, off:off + L] = k, v
+        if cached and L == 1:
+            # one query per head: two batched matrix-vector products over the cache rows seen so far.  A recorded
+            # step has fixed shapes, so it reads the whole cache and masks the rows past the position.
+            if not on_device:
+                kc, vc = kc[:, :, :off + 1], vc[:, :, :off + 1]
+            s = torch.matmul(q, kc.transpose(2, 3)).float() * hd ** -0.5         # [B, H, 1, S]
+            if on_device:
+                s = s.masked_fill(torch.arange(kc.shape[2], device=u.device) > off, float("-inf"))
+            o = torch.matmul(torch.softmax(s, dim=-1).to(vc.dtype), vc)
+        else:
+            if cached:                  # a longer continuation: its queries see the cache and, causally, themselves
+                kk, vv = kc[:, :, :off + L], vc[:, :, :off + L]
+                mask = torch.ones(L, off + L, dtype=torch.bool, device=u.device).tril(off)
+                o = F.scaled_dot_product_attention(q, kk, vv, attn_mask=mask)
+            else:
+                o = F.scaled_dot_product_attention(q, k, v, is_causal=True)
         u = self.out_proj(o.transpose(1, 2).reshape(B, L, D)) + u
         return self.mlp(self.post_norm(u)) + u, None
 
@@ -187,21 +212,73 @@ class StripedHyena2(nn.Module):
         return x @ self.embedding.weight.T
 
     @torch.no_grad()
-    def generate(self, input_ids, num_tokens, forced=None):
+    def generate(self, input_ids, num_tokens, forced=None, graph=False):
         """Greedy cached generation in the order of vortex/model/generation.py:164-229: one prefill over the
         prompt, then one token per forward with the caches' seqlen_offset advanced first.  `forced`
-        [B, num_tokens] replaces the sampled tokens (teacher forcing).  Returns (tokens, logits of every step)."""
+        [B, num_tokens] replaces the sampled tokens (teacher forcing).  graph=True replays the token step as a
+        recorded HIP graph from the third token on (RecordedDecodeStep).  Returns (tokens, logits of every step)."""
         B, L = input_ids.shape
         ipd = self.initialize_inference_params(max_seqlen=L + num_tokens)
-        x, toks, scores = input_ids, [], []
+        x, toks, scores, rec = input_ids, [], [], None
         for i in range(num_tokens):
             if i > 0:
                 x = x[:, -1:]
                 for p in ipd.values():
                     p.seqlen_offset = L if p.seqlen_offset == 0 else p.seqlen_offset + 1
-            logits = self.forward(x, ipd)[:, -1]
+            if graph and i == 2:                    # one eager token step has bound the decode kernels by now
+                rec = RecordedDecodeStep(self, ipd, B)
+            logits = (self.forward(x, ipd) if rec is None else rec(x))[:, -1]
             new = logits.argmax(-1) if forced is None else forced[:, i]
             toks.append(new)
             scores.append(logits)
             x = new[:, None]
+        if rec is not None:
+            rec.release()
         return torch.stack(toks, 1), torch.stack(scores, 1)
+
+
+class RecordedDecodeStep:
+    """The cached one-token forward of a StripedHyena2 recorded once as a HIP graph and replayed per token.
+
+    A replay cannot change scalar kernel arguments, so everything that moves from token to token lives in device
+    memory while this object is in use: the ring positions of the FIR caches (ops.RingClock, read by the step
+    kernels, advanced by one launch at the end of the step) and the attention position (an int64 tensor the
+    recorded step increments).  Needs caches that are full (prompt at least as long as the longest FIR filter)
+    and one eager token step beforehand, which binds the decode kernels to the caches.  release() hands the
+    positions back to the host-side fields so that eager steps can follow."""
+
+    def __init__(self, model, ipd, batch):
+        self.model, self.ipd = model, ipd
+        dev = model.embedding.weight.device
+        rings = []
+        for kind, block in zip(model.kinds, model.blocks):
+            if kind == "attn":
+                continue
+            ip, i = ipd[kind], block.filter.layer_idx
+            if i not in ip.fir_state_dict:
+                raise RuntimeError("run the prefill and one token step before recording")
+            rings.append(ip.fir_state_dict[i])
+            if block.filter.fir_inner_filter_length:
+                rings.append(ip.fir_inner_state_dict[i])
+        if any(getattr(r, "valid", r.buf.shape[1]) < r.buf.shape[1] for r in rings):
+            raise NotImplementedError("a cache is still filling up (prompt shorter than a filter): step eagerly")
+        mha = ipd["mha"]
+        self.clock = ops.RingClock(rings)
+        mha.offset_dev = torch.tensor([mha.seqlen_offset], dtype=torch.int64, device=dev)
+        self.tokens = torch.zeros(batch, 1, dtype=torch.int64, device=dev)
+        self.steps = 0
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = model.forward(self.tokens, ipd)
+            self.clock.advance()
+            mha.offset_dev.add_(1)
+
+    def __call__(self, tokens):
+        self.tokens.copy_(tokens)
+        self.graph.replay()
+        self.steps += 1
+        return self.logits.clone()                  # the recorded step writes the same buffer every time
+
+    def release(self):
+        self.clock.release()
+        self.ipd["mha"].offset_dev = None

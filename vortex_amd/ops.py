@@ -319,6 +319,7 @@ class FirRing:
 
     def __init__(self, buf, pos=0):
         self.buf, self.pos = buf, pos
+        self.pos_dev = None         # int32 [1] device tensor once a RingClock owns the position (then pos is stale)
 
     @classmethod
     def from_reference(cls, fir_state):
@@ -332,7 +333,8 @@ class FirRing:
 
     def reference_order(self, dtype=torch.float32):
         R = self.buf.shape[1]
-        idx = (torch.arange(R, device=self.buf.device) + self.pos) % R
+        pos = self.pos if self.pos_dev is None else int(self.pos_dev.item())
+        idx = (torch.arange(R, device=self.buf.device) + pos) % R
         return self.buf.index_select(1, idx).permute(0, 2, 1).to(dtype)
 
 
@@ -355,6 +357,12 @@ def fir_step(x1, ring, w, *, x2=None, v=None, bias=None, gated_bias=False):
     out = torch.empty((B, D), dtype=torch.bfloat16, device=x1.device)
     b = _f32(bias)
     mode = HYENA_BIAS_NONE if b is None else (HYENA_BIAS_GATED_FP32 if gated_bias else HYENA_BIAS_ADD)
+    if ring.pos_dev is not None:                # the position is on a RingClock, which also advances it
+        rc = _lib.lib().hyena_fir_step_dpos(_ptr(x1), _ptr(x2), _ptr(v), x1.stride(0), _ptr(ring.buf), R,
+                                            _ptr(ring.pos_dev), _ptr(w), _ptr(b), mode, _ptr(out), out.stride(0),
+                                            B, D, G, _stream())
+        _lib.check(rc, "hyena_fir_step_dpos")
+        return out
     rc = _lib.lib().hyena_fir_step(_ptr(x1), _ptr(x2), _ptr(v), x1.stride(0), _ptr(ring.buf), R, ring.pos,
                                    _ptr(w), _ptr(b), mode, _ptr(out), out.stride(0), B, D, G, _stream())
     _lib.check(rc, "hyena_fir_step")
@@ -420,17 +428,21 @@ class FirStepper:
             raise ValueError(f"taps have {self.w.shape[1]} columns, cache depth {self.R} needs {self.R + 1}")
         self.mode = HYENA_BIAS_NONE if bias is None else (HYENA_BIAS_GATED_FP32 if gated_bias else HYENA_BIAS_ADD)
         self.gated = gated
-        self._fn = _lib.lib().hyena_fir_step
+        self._fn, self._fn_dpos = _lib.lib().hyena_fir_step, _lib.lib().hyena_fir_step_dpos
 
     def __call__(self, x1, x2, v, out):
         B = x1.shape[0]
-        rc = self._fn(x1.data_ptr(), x2.data_ptr() if self.gated else None, v.data_ptr() if self.gated else None,
-                      x1.stride(0), self.ring.buf.data_ptr(), self.R, self.ring.pos, self.w.data_ptr(),
-                      self.bias.data_ptr() if self.bias is not None else None, self.mode, out.data_ptr(),
-                      out.stride(0), B, self.D, self.G, torch.cuda.current_stream().cuda_stream)
+        ring = self.ring
+        dpos = ring.pos_dev is not None
+        rc = (self._fn_dpos if dpos else self._fn)(
+            x1.data_ptr(), x2.data_ptr() if self.gated else None, v.data_ptr() if self.gated else None,
+            x1.stride(0), ring.buf.data_ptr(), self.R, ring.pos_dev.data_ptr() if dpos else ring.pos, self.w.data_ptr(),
+            self.bias.data_ptr() if self.bias is not None else None, self.mode, out.data_ptr(),
+            out.stride(0), B, self.D, self.G, torch.cuda.current_stream().cuda_stream)
         if rc:
             _lib.check(rc, "hyena_fir_step")
-        self.ring.pos = (self.ring.pos + 1) % self.R
+        if not dpos:
+            ring.pos = (ring.pos + 1) % self.R
         return out
 
 
@@ -495,14 +507,23 @@ class LayerStepper:
         self._pref = ctypes.byref(self.proj)
         self.is_fir = isinstance(inner, FirStepper)
         self._fn = _lib.lib().hyena_fir_layer_step if self.is_fir else _lib.lib().hyena_iir_layer_step
+        self._fn_dpos = _lib.lib().hyena_fir_layer_step_dpos
 
     def __call__(self, u, out):
         """u: [B, 3D] bf16 with contiguous channels; out: [B, D] bf16 (float32 allowed for the IIR step)."""
         B = u.shape[0]
         p, n = self.proj, self.inner
-        p.u, p.u_batch_stride, p.pos = u.data_ptr(), u.stride(0), self.ring.pos
+        dpos = self.ring.pos_dev is not None
+        if self.is_fir and (n.ring.pos_dev is not None) != dpos:
+            raise RuntimeError("the featurizer cache and the inner cache must both be on a RingClock, or neither")
+        p.u, p.u_batch_stride = u.data_ptr(), u.stride(0)
+        p.pos, p.pos_dev = (0, self.ring.pos_dev.data_ptr()) if dpos else (self.ring.pos, None)
         stream = torch.cuda.current_stream().cuda_stream
-        if self.is_fir:
+        if self.is_fir and dpos:
+            rc = self._fn_dpos(self._pref, n.ring.buf.data_ptr(), n.R, n.ring.pos_dev.data_ptr(), n.w.data_ptr(),
+                               n.bias.data_ptr() if n.bias is not None else None, n.mode, out.data_ptr(),
+                               out.stride(0), B, n.D, n.G, stream)
+        elif self.is_fir:
             rc = self._fn(self._pref, n.ring.buf.data_ptr(), n.R, n.ring.pos, n.w.data_ptr(),
                           n.bias.data_ptr() if n.bias is not None else None, n.mode, out.data_ptr(), out.stride(0),
                           B, n.D, n.G, stream)
@@ -512,10 +533,39 @@ class LayerStepper:
                           n.S, stream)
         if rc:
             _lib.check(rc, "hyena_fir_layer_step" if self.is_fir else "hyena_iir_layer_step")
-        self.ring.pos = (self.ring.pos + 1) % self.Rf
-        if self.is_fir:
-            n.ring.pos = (n.ring.pos + 1) % n.R
+        if not dpos:
+            self.ring.pos = (self.ring.pos + 1) % self.Rf
+            if self.is_fir:
+                n.ring.pos = (n.ring.pos + 1) % n.R
         return out
+
+
+class RingClock:
+    """Keeps the positions of a set of FirRing caches in device memory and moves them all on with one launch per
+    token (hyena_ring_advance), so that a recorded token step (a HIP graph) can be replayed: the step kernels then
+    read their ring positions from the device instead of taking them as scalar arguments.
+
+    While a ring is on the clock its host-side `pos` is stale; release() writes the positions back."""
+
+    def __init__(self, rings):
+        self.rings = list(rings)
+        if not self.rings:
+            raise ValueError("no rings")
+        dev = self.rings[0].buf.device
+        if any(r.pos_dev is not None for r in self.rings):
+            raise RuntimeError("a ring is already on a clock")
+        self.pos = torch.tensor([r.pos for r in self.rings], dtype=torch.int32, device=dev)
+        self.depth = torch.tensor([r.buf.shape[1] for r in self.rings], dtype=torch.int32, device=dev)
+        for i, r in enumerate(self.rings):
+            r.pos_dev = self.pos[i:i + 1]
+
+    def advance(self):
+        rc = _lib.lib().hyena_ring_advance(self.pos.data_ptr(), self.depth.data_ptr(), len(self.rings), _stream())
+        _lib.check(rc, "hyena_ring_advance")
+
+    def release(self):
+        for r, p in zip(self.rings, self.pos.tolist()):
+            r.pos, r.pos_dev = p, None
 
 
 class DecodeLayerSet:
