@@ -71,6 +71,20 @@ def test_new_entry_points_validate_before_touching_the_device():
     ps = _lib.ProjStep(P, 192, P, 2, 0, P, None, 4, 12, 4, 1, 0)
     assert L.hyena_fir_layer_step(ref(ps), P, 6, 0, P, None, 0, P, 64, 1, 64, 4, None) == -3          # head_dim 4
     assert L.hyena_iir_layer_step(None, P, P, P, 0, P, 0, P, 0, 64, 1, 64, 64, 16, None) == -1
+    # ring positions in device memory: the pointer is required, and a position on the device lifts the host range check
+    assert L.hyena_fir_step_dpos(P, None, None, 64, P, 6, None, P, None, 0, P, 64, 1, 64, 4, None) == -1
+    assert L.hyena_fir_layer_step_dpos(ref(ps), P, 6, None, P, None, 0, P, 64, 1, 64, 4, None) == -1
+    assert L.hyena_ring_advance(None, P, 4, None) == -1 and L.hyena_ring_advance(P, P, -1, None) == -1
+    assert L.hyena_ring_advance(P, P, 0, None) == 0
+    ps = _lib.ProjStep(P, 192, P, 2, 5, P, None, 64, 0, 64, 1, 0, None)
+    assert L.hyena_fir_layer_step(ref(ps), P, 6, 0, P, None, 0, P, 64, 0, 64, 4, None) == -1           # pos 5 of 2
+    ps = _lib.ProjStep(P, 192, P, 2, 5, P, None, 64, 0, 64, 1, 0, P)
+    assert L.hyena_fir_layer_step(ref(ps), P, 6, 0, P, None, 0, P, 64, 0, 64, 4, None) == 0            # B = 0: no launch
+    # modal state sizes
+    assert L.hyena_li_plan_bytes(4, 16) == L.hyena_li_plan_bytes(4, 2) == 4 * 1536 * 4
+    assert L.hyena_li_plan_bytes(4, 17) == 0 and L.hyena_li_plan_bytes(4, 0) == 0
+    assert L.hyena_iir_step(P, P, P, 64, P, P, P, 0, P, 0, P, 0, 64, 1, 64, 64, 12, None) == -3          # not a power of two
+    assert L.hyena_iir_step(P, P, P, 64, P, P, P, 0, P, 0, P, 0, 64, 0, 64, 64, 2, None) == 0            # B = 0
 
 
 def test_missing_library_fails_loudly(monkeypatch):
