@@ -141,3 +141,29 @@ def test_li_full_size_sampled_groups():
         assert rel_err(y32[:, rows], y32_ref) <= 1e-4 + floor, (g, floor)
         assert rel_err(out[:, rows], ref) <= 2e-2, g
         assert rel_err(torch.view_as_real(st[:, rows]), torch.view_as_real(st_ref)) <= 1e-4, g
+
+
+def test_million_token_rows():
+    # the context length of the 1M configurations (evo2-7b-1m.yml, evo2-40b-1m.yml: max_seqlen 1048576): all three
+    # operators on rows of 2^20 samples against the oracle, and the fused / channel-last layer forms of SE and MR
+    # against the sequence-major kernels
+    B, D, L = 1, 32, 1 << 20
+    x2, x1, v = O.make_gates(B, D, L, seed=77)
+    dx1, dx2, dv = x1.cuda(), x2.cuda(), v.cuda()
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(1)).bfloat16()
+    lp, r = O.make_modal_real(D, 16, seed=78)                      # one filter per channel, real poles
+    ref, y32_ref, st_ref = O.li_prefill(x2, x1, v, lp, r, Db)
+    out, y32, st = va.hyena_li_fwd(dx1, dx2, dv, lp.cuda(), r.cuda(), Db.cuda(), want_state=True, want_fp32=True)
+    assert rel_err(y32, y32_ref) <= 1e-4
+    assert rel_err(out, ref) <= 2e-2
+    assert rel_err(st, st_ref) <= 1e-4
+    del y32, y32_ref
+    h7, h128 = O.make_se_filter(2, 7, seed=79), O.make_mr_filter(2, 128, seed=80)
+    se = va.hyena_se_fwd(dx1, dx2, dv, h7.cuda())
+    assert rel_err(se, O.se_fir(x2, x1, v, h7)[0]) <= 2e-2
+    mr = va.hyena_mr_fwd(dx1, dx2, dv, h128.cuda(), Db.cuda())
+    assert rel_err(mr, O.mr_fir(x2, x1, v, h128, Db)[0]) <= 2e-2
+    cl = lambda t: t.transpose(1, 2).contiguous()
+    mr_cl = va.ops.fir_cl_fwd(cl(dx1), cl(dx2), cl(dv), h128.cuda().reshape(2, 128), bias=Db.cuda(),
+                              bias_mode=va.ops.HYENA_BIAS_GATED_FP32)
+    assert rel_err(mr_cl.transpose(1, 2), mr) <= 1e-2
