@@ -188,3 +188,40 @@ def test_featurizer_front_pad(L, bias):
     ref, _ = O.parallel_fir(u, w, b, fir_length=K, dim_last=True, gate=False)
     assert z.shape == (B, C, L + pad) and not z[..., :pad].any()
     assert rel_err(z[..., pad:], O.interleave(ref)) <= 2e-2
+
+
+def test_kernels_follow_the_current_stream():
+    # every entry point enqueues on the stream it is given (the wrappers pass torch's current stream): work issued
+    # on a side stream is ordered after that stream's earlier work and gives the default-stream result bit for bit
+    import vortex_amd as va
+    B, D, L, G = 2, 64, 4096, 4
+    g = torch.Generator().manual_seed(12)
+    x1, x2, v = (torch.randn(B, D, L, generator=g).bfloat16().cuda() for _ in range(3))
+    h7, h128 = torch.randn(G, 1, 7, generator=g).cuda(), (torch.randn(G, 1, 128, generator=g) / 11).cuda()
+    Db = torch.randn(D, generator=g).bfloat16().cuda()
+    lp = (-(0.01 + torch.rand(G, 16, 1, generator=g))).cuda()
+    r = torch.randn(G, 16, generator=g).cuda()
+
+    def run():
+        se = va.hyena_se_fwd(x1, x2, v, h7)
+        mr = va.hyena_mr_fwd(x1, x2, v, h128, Db)
+        li, _, st = va.hyena_li_fwd(x1, x2, v, lp, r, Db, want_state=True)
+        cl = va.ops.fir_cl_fwd(x1.transpose(1, 2).contiguous(), x2.transpose(1, 2).contiguous(),
+                               v.transpose(1, 2).contiguous(), h128.reshape(G, 128), bias=Db,
+                               bias_mode=va.ops.HYENA_BIAS_GATED_FP32)
+        y = va.iir_step(x1[..., 0].contiguous(), x2[..., 0].contiguous(), v[..., 0].contiguous(), st,
+                        torch.exp(lp[..., 0]), r, Db)
+        return se, mr, li, cl, y, st
+
+    want = run()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        big = torch.randn(64, 1 << 20, device="cuda")
+        for _ in range(20):                      # keep the side stream busy ahead of the kernels under test
+            big = big * 1.0001
+        got = run()
+    side.synchronize()
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
