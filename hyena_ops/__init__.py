@@ -6,6 +6,6 @@ gfx950 kernels of vortex_amd.
 """
 from vortex_amd.ops import hyena_li_fwd, hyena_mr_fwd, hyena_se_fwd  # noqa: F401
 
-from . import interface  # noqa: F401
+from . import interface, kernel_utils, utils  # noqa: F401
 
-__all__ = ["hyena_se_fwd", "hyena_mr_fwd", "hyena_li_fwd", "interface"]
+__all__ = ["hyena_se_fwd", "hyena_mr_fwd", "hyena_li_fwd", "interface", "kernel_utils", "utils"]

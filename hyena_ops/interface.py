@@ -13,6 +13,8 @@ import torch
 from vortex_amd import ops
 from vortex_amd._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE
 
+from .utils import correction_toeplitz, toeplitz
+
 
 @dataclass(eq=False)
 class FwdKernelConfig:
@@ -147,17 +149,10 @@ def two_pass_chunked_gate_conv_gate(x, B, C, h, return_toeplitz=True, schedule="
 
 
 def _toeplitz_pair(h, chunk, dtype):
-    """T[g, i, j] = hf[g, i-j] (0 <= i-j < K) and T_hat[g, i, j] = hf[g, i+chunk-j] (i+chunk-j < K) with
-    hf = h.flip(-1): the within-chunk and previous-chunk Toeplitz factors of
-    vortex/ops/hyena_se/utils.py:5-25, :38-51."""
-    g, K = h.shape[0], h.shape[-1]
-    hf = h.reshape(g, K).flip(-1)
-    idx = torch.arange(chunk, device=h.device)
-    lag = idx[:, None] - idx[None, :]
-    def gather(l):
-        ok = (l >= 0) & (l < K)
-        return torch.where(ok[None], hf[:, l.clamp(0, K - 1)], torch.zeros((), device=h.device, dtype=hf.dtype)).to(dtype)
-    return gather(lag), gather(lag + chunk)
+    """(T, T_hat) of the operator weights h (g, 1, K): the Toeplitz factors of hyena_ops.utils on hf = h.flip(-1),
+    as vortex/ops/hyena_se/ref_fwd.py:216-266 builds them."""
+    hf = h.reshape(h.shape[0], h.shape[-1]).flip(-1)
+    return toeplitz(hf, chunk, dtype=dtype), correction_toeplitz(hf, chunk, dtype=dtype)
 
 
 def two_pass_fwd_grouped(x, B, C, h, y=None, return_y2=False, return_toeplitz=False, return_bx_lag=False,

@@ -144,3 +144,35 @@ def test_from_vortex_shares_parameters_and_config():
     model = types.SimpleNamespace(blocks=blocks)
     assert use_hip_filters(model) == 2 and use_hip_filters(model) == 0
     assert isinstance(blocks[2].filter, HyenaCascade) and blocks[2].filter.log_poles is modal.log_poles
+
+
+def test_hyena_ops_utils_toeplitz_factors():
+    # `from hyena_ops.utils import toeplitz, correction_toeplitz` (vortex/ops/hyena_se/ref_fwd.py:24): the definition
+    # by brute force on the arange filter of vortex/ops/hyena_se/tests/test_toeplitz.py:33-66, the in-place forms, and the
+    # two-pass identity y_c = T x_c + T_hat x_{c-1} against a direct causal convolution
+    from hyena_ops.utils import correction_toeplitz, correction_toeplitz_from_empty, toeplitz, toeplitz_from_empty
+    from hyena_ops.kernel_utils import BwdKernelConfig, FwdKernelConfig
+    assert FwdKernelConfig() is not None and BwdKernelConfig() is not None
+    for g, K, C in [(1, 4, 16), (2, 4, 32), (3, 7, 8), (2, 32, 32)]:
+        h = torch.arange(1, g * K + 1).reshape(g, 1, K)
+        hf = h[:, 0].flip(-1)
+        T, Th = toeplitz(hf, C), correction_toeplitz(hf, C)
+        assert T.shape == Th.shape == (g, C, C) and T.dtype == hf.dtype
+        for gi in range(g):
+            for i in range(C):
+                for j in range(C):
+                    assert int(T[gi, i, j]) == (int(hf[gi, i - j]) if 0 <= i - j < K else 0)
+                    assert int(Th[gi, i, j]) == (int(hf[gi, i + C - j]) if (j >= i and i + C - j < K) else 0)
+        assert torch.equal(toeplitz_from_empty(torch.empty(g, C, C), hf), T.float())
+        assert torch.equal(correction_toeplitz_from_empty(torch.empty(g, C, C), hf), Th.float())
+    gen = torch.Generator().manual_seed(3)
+    g, K, C, n = 2, 5, 8, 4
+    hf = torch.randn(g, K, generator=gen, dtype=torch.float64)
+    x = torch.randn(g, n * C, generator=gen, dtype=torch.float64)
+    T, Th = toeplitz(hf, C), correction_toeplitz(hf, C, dtype=torch.float64)
+    xc = x.reshape(g, n, C)
+    prev = torch.cat([torch.zeros(g, 1, C, dtype=torch.float64), xc[:, :-1]], 1)
+    y = (torch.einsum("gij,gnj->gni", T, xc) + torch.einsum("gij,gnj->gni", Th, prev)).reshape(g, n * C)
+    direct = torch.stack([sum(hf[gi, k] * torch.cat([torch.zeros(k, dtype=torch.float64), x[gi, :n * C - k]])
+                              for k in range(K)) for gi in range(g)])
+    assert torch.allclose(y, direct, atol=1e-12)
