@@ -203,3 +203,32 @@ def test_layer_full_size_config2():
     ref, _ = oracle_layer(us, wf.cpu()[ch][:, None, :], None, h.repeat_interleave(D // G, 0)[ds], Db[ds], n, 1, False,
                           True, False)
     assert rel_err(y[:, :, ds.to(DEV)].permute(0, 2, 1), ref) <= 2e-2
+
+
+def test_layer_projection_beyond_32_bit_offsets():
+    # a projection of more than 2^32 elements (L = 360448 rows of 3 x 4096 channels, 8.9 GB): the last rows are
+    # only right with 64-bit element offsets.  The one-launch layer and the featurizer kernel against the oracle on
+    # sampled channels, compared over the last 4096 samples (the filters reach back 130 samples at most).
+    B, L, D, G, K, Ks = 1, 360448, 4096, 256, 128, 3
+    C = 3 * D
+    assert L * C > 1 << 32
+    g = torch.Generator(device=DEV).manual_seed(14)
+    u = torch.randn(B, L, C, generator=g, device=DEV, dtype=torch.bfloat16)
+    wf = (torch.randn(C, Ks, generator=g, device=DEV) / Ks ** 0.5)
+    h = O.make_mr_filter(G, K)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(13))
+    cmap = ops.gate_channel_map(D, interleave=True)
+    y = ops.fir_layer_fwd(u, wf.t().contiguous(), None, cmap, h.reshape(G, K).to(DEV), bias=Db.to(DEV),
+                          bias_mode=HYENA_BIAS_GATED_FP32)
+    ds = torch.tensor([0, 1777, 4095])
+    ch = (3 * ds[:, None] + torch.arange(3)[None]).reshape(-1)
+    T = 4096 + 256
+    us = u[:, L - T:, ch.to(DEV)].cpu()
+    ref, _ = oracle_layer(us, wf.cpu()[ch][:, None, :], None, h.repeat_interleave(D // G, 0)[ds], Db[ds], len(ds), 1,
+                          False, True, False)
+    assert rel_err(y[:, L - 4096:, ds.to(DEV)].permute(0, 2, 1), ref[..., 256:]) <= 2e-2
+    del y
+    z = ops.featurizer_fwd(u, wf, None, interleave=True)           # [B, 3D, L]: rows of the three gates
+    zs = torch.stack([z[0, i * D + d, L - 4096:] for d in ds.tolist() for i in range(3)]).cpu()
+    zr, _ = O.parallel_fir(us, wf.cpu()[ch][:, None, :], None, fir_length=Ks, dim_last=True, gate=False)
+    assert rel_err(zs, zr[0][:, 256:]) <= 1e-2

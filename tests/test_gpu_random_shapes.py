@@ -225,3 +225,44 @@ def test_kernels_follow_the_current_stream():
     side.synchronize()
     for a, b in zip(got, want):
         assert torch.equal(a, b)
+
+
+def test_offsets_beyond_32_bits():
+    # tensors of more than 2^32 elements (B=2, D=4096, L=2^19+4096: 8.1 GiB each): the rows at the far end are only
+    # right if every element offset is computed in 64 bits.  Sampled rows against the oracle.
+    import vortex_amd as va
+    from oracle import hyena_oracle as O
+    B, D, L, G = 2, 4096, (1 << 19) + 4096, 256
+    assert B * D * L > 1 << 32
+    gen = torch.Generator(device="cuda").manual_seed(21)
+    x1, x2, v = (torch.randn(B, D, L, generator=gen, device="cuda", dtype=torch.bfloat16) for _ in range(3))
+    h7, h128 = O.make_se_filter(G, 7, seed=1), O.make_mr_filter(G, 128, seed=2)
+    lp, r = O.make_modal_real(G, 16, seed=3)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(4)).bfloat16()
+    groups = (0, 131, 255)
+
+    def check(out, ref_fn, b=1):
+        for g in groups:
+            rows = slice(16 * g, 16 * g + 16)
+            a1, a2, av = x1[b:b + 1, rows].cpu(), x2[b:b + 1, rows].cpu(), v[b:b + 1, rows].cpu()
+            ref = ref_fn(a2, a1, av, g, rows)
+            err = (out[b:b + 1, rows].float().cpu() - ref.float()).abs().max() / ref.float().abs().max()
+            assert err <= 2e-2, (g, err.item())
+
+    out = va.hyena_se_fwd(x1, x2, v, h7.cuda())
+    check(out, lambda a2, a1, av, g, rows: O.se_fir(a2, a1, av, h7[g:g + 1])[0])
+    out = va.hyena_mr_fwd(x1, x2, v, h128.cuda(), Db.cuda())
+    check(out, lambda a2, a1, av, g, rows: O.mr_fir(a2, a1, av, h128[g:g + 1], Db[rows])[0])
+    out, _, st = va.hyena_li_fwd(x1, x2, v, lp.cuda(), r.cuda(), Db.cuda(), want_state=True)
+    check(out, lambda a2, a1, av, g, rows: O.li_prefill(a2, a1, av, lp[g:g + 1], r[g:g + 1], Db[rows])[0])
+    del out
+    # channel-last: the same samples as [B, L, D]; the last batch element's rows lie past 2^32 elements
+    c1, c2, cv = (t.transpose(1, 2).contiguous() for t in (x1, x2, v))
+    del x1, x2, v
+    out = va.ops.fir_cl_fwd(c1, c2, cv, h128.reshape(G, 128).cuda(), bias=Db.cuda(), bias_mode=va.ops.HYENA_BIAS_GATED_FP32)
+    for g in groups:
+        rows = slice(16 * g, 16 * g + 16)
+        a1, a2, av = (t[1:2, :, rows].transpose(1, 2).contiguous().cpu() for t in (c1, c2, cv))
+        ref = O.mr_fir(a2, a1, av, h128[g:g + 1], Db[rows])[0]
+        err = (out[1:2, :, rows].transpose(1, 2).float().cpu() - ref.float()).abs().max() / ref.float().abs().max()
+        assert err <= 2e-2, (g, err.item())
