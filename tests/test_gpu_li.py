@@ -167,3 +167,30 @@ def test_million_token_rows():
     mr_cl = va.ops.fir_cl_fwd(cl(dx1), cl(dx2), cl(dv), h128.cuda().reshape(2, 128), bias=Db.cuda(),
                               bias_mode=va.ops.HYENA_BIAS_GATED_FP32)
     assert rel_err(mr_cl.transpose(1, 2), mr) <= 1e-2
+
+
+@pytest.mark.parametrize("L", [65536 + 520, 2048 * 5 + 8, 2048 * 3, 1544, 8])
+@pytest.mark.parametrize("cplx", [True, False])
+def test_li_cooperative_form(L, cplx, monkeypatch):
+    # rows of 65536 samples and more in shared-filter groups run with the four wavefronts of a block on consecutive
+    # pieces of the same channels and the modal state handed across through LDS.  Forced on here for short and ragged
+    # rows too (last steps with idle wavefronts, the final state in any of the four pieces): against the oracle,
+    # and against the one-wavefront form for the same inputs.
+    B, D, G = 2, 16, 2
+    x2, x1, v = O.make_gates(B, D, L, seed=L)
+    lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(G, 16, seed=5)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(1)).bfloat16()
+    ref, y32_ref, st_ref = O.li_prefill(x2, x1, v, lp, r, Db)
+    res = {}
+    for coop in ("1", "0"):
+        monkeypatch.setenv("HYENA_LI_COOP", coop)
+        res[coop] = va.hyena_li_fwd(x1.cuda(), x2.cuda(), v.cuda(), lp.cuda(), r.cuda(), Db.cuda(),
+                                    want_state=True, want_fp32=True)
+        out, y32, st = res[coop]
+        assert rel_err(y32, y32_ref) <= 1e-4, coop
+        assert rel_err(out, ref) <= 2e-2, coop
+        assert rel_err(torch.view_as_real(st) if cplx else st, torch.view_as_real(st_ref) if cplx else st_ref) <= 1e-4, coop
+    assert rel_err(res["1"][1], res["0"][1]) <= 1e-5          # the same sums, grouped differently across the state hand-off
+    monkeypatch.setenv("HYENA_LI_COOP", "1")
+    out_nt, _, _ = va.hyena_li_fwd(x1.cuda(), x2.cuda(), v.cuda(), lp.cuda(), r.cuda(), Db.cuda())   # the bf16-only variant
+    assert torch.equal(out_nt, res["1"][0])
