@@ -211,6 +211,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     // table for the block, build a quarter of the fragments each and read the rest from LDS.
     // 16x16x32 A operand: lane holds row m = lane & 15, k = 8*(lane >> 4) + e, e = 0..7.
     bf16x8 Th[8], Tl[8], Poh[8], Pol[8], Pih[8], Pil[8];
+    float pcr, pci, pinv_r, pinv_i;                            // p^128 and 1/p of this lane's pole (lane & 15)
     {
         float* tb = COOP ? (float*)lds_all : (float*)lds;
         u32x4* fb = (u32x4*)(lds_all + WS_GROUP * 4);           // COOP: [48 fragments][64 lanes]
@@ -226,6 +227,10 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
             wave_sync();
         }
         const int m = lane & 15, qa = lane >> 4;
+        pcr = tb[WS_P16 + 2 * (9 * m + 8)];
+        pci = tb[WS_P16 + 2 * (9 * m + 8) + 1];
+        pinv_r = tb[WS_PINV + 2 * m];
+        pinv_i = tb[WS_PINV + 2 * m + 1];
         const float2* t16 = (const float2*)(tb + WS_P16);
         const float2* t1 = (const float2*)(tb + WS_P1);
         const float2* tr = (const float2*)(tb + WS_R1);
@@ -305,15 +310,14 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     float Xr = 0.f, Xi = 0.f;
     float Xfr = 0.f, Xfi = 0.f;                                // state after the chunk that holds sample L-1
     bool have_final = !COOP;                                   // COOP: only the wavefront whose piece holds sample L-1
-    const float pcr = ws[WS_P16 + 2 * (9 * sp + 8)], pci = ws[WS_P16 + 2 * (9 * sp + 8) + 1];   // p^128
+    float dco = 0.f;
+    if (a.Dcoef) dco = a.Dcoef[d0 + (CPW == 4 ? c : 0)];
     float X0r = 0.f, X0i = 0.f;                                // COOP: state at the start of the block's step
     float ppr = pcr, ppi = pci;                                // COOP: p^TLW, one wavefront's piece
     if (COOP) {
 #pragma unroll
         for (int k = 1; k < 16 / CPW; ++k) { const float t = ppr * pcr - ppi * pci; ppi = ppr * pci + ppi * pcr; ppr = t; }
     }
-    float dco = 0.f;
-    if (a.Dcoef) dco = a.Dcoef[d0 + (CPW == 4 ? c : 0)];
 
     // ---- coalesced layout: lane moves samples 8*lane..8*lane+7 of each of the 4 rows
     const int lofs = lane * 8 + 32 * (lane >> 4);              // position inside a padded LDS row
@@ -562,7 +566,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     if (a.state_out && have_final) {
         // the captured chunk ends (-L) % 128 samples past L with zero inputs: undo that, X *= p^-pad
         int pad = (int)((C - L % C) % C);
-        float qr = ws[WS_PINV + 2 * sp], qi = ws[WS_PINV + 2 * sp + 1];
+        float qr = pinv_r, qi = pinv_i;
         float fr_ = 1.f, fi = 0.f;
         while (pad) {
             if (pad & 1) { const float t = fr_ * qr - fi * qi; fi = fr_ * qi + fi * qr; fr_ = t; }
