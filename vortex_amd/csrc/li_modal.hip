@@ -48,12 +48,13 @@ constexpr int WAVE_LDS_BYTES = 2 * 4 * URS * 2 + 16 * LRS * 4 + 2 * 16 * XRS * 2
 constexpr int FR_T = 0, FR_PO = 16, FR_PI = 32, N_FRAG = 48;
 // Workspace per group (floats), evaluated in double by the plan kernel.  Every power of a pole the fragments
 // need is one fp32 complex product of a coarse and a fine table entry, p^(16a+b) = P16[a] * P1[b]:
-constexpr int WS_HEAD = 0;                         // [128]        filter head h[0..127]
+constexpr int WS_ZPAD = 32;                        // zeros ahead of the head: lags -31..-1 read as 0 without a test
+constexpr int WS_HEAD = WS_ZPAD;                   // [128]        filter head h[0..127]
 constexpr int WS_P16 = WS_HEAD + C;                // [16][9][2]   p^(16a), a = 0..8  (a = 8: the chunk factor p^128)
 constexpr int WS_P1 = WS_P16 + S * 9 * 2;          // [16][16][2]  p^b
 constexpr int WS_R1 = WS_P1 + S * 16 * 2;          // [16][16][2]  r * p^b
 constexpr int WS_PINV = WS_R1 + S * 16 * 2;        // [16][2]      1/p
-constexpr int WS_GROUP = 1536;                     // 1472 used; 6 KB, a whole number of 16-byte lane loads
+constexpr int WS_GROUP = 1536;                     // 1504 used; 6 KB, a whole number of 16-byte lane loads
 static_assert(WS_PINV + 2 * S <= WS_GROUP, "workspace layout");
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) {
@@ -110,6 +111,7 @@ __global__ __launch_bounds__(256) void li_plan_kernel(const float* __restrict__ 
         re = m * cos(a);
         im = m * sin(a);
     };
+    if (tid < WS_ZPAD) w[tid] = 0.f;
     if (tid < C) {                                  // filter head h[0..127]
         double acc = 0.0;
         for (int s = 0; s < sr; ++s) {
@@ -282,41 +284,63 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
         for (int f = 0; f < 8; ++f) {               // Toeplitz: rows of (superblock Sigma, half ib) x inputs of block J
             if (!mine(f)) continue;
             const int delta = f >> 1, ib = f & 1;   // delta = Sigma - J
+            // lag = 32*delta + sample - (8*qa + k) lies in -31..127; the zeros ahead of the head stand for lag < 0
+            const float* hp = tb + WS_HEAD + 32 * delta + li_sample(ib, m) - 8 * qa;
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const int lag = 32 * delta + li_sample(ib, m) - (8 * qa + k);
-                const float hv = tb[WS_HEAD + (lag < 0 ? 0 : (lag >= C ? C - 1 : lag))];
-                val[k] = (lag >= 0 && lag < C) ? hv : 0.f;
-            }
+            for (int k = 0; k < 8; ++k) val[k] = hp[-k];
             li_split(val, th[FR_T + f], th[FR_T + 8 + f]);
         }
+        // Pout: output sample i of (Sigma, ib) x state rows 8*qa + k hold Re / -Im of r * p^(i+1).  The exponent is
+        // e = 32*Sigma + 4*ib + eb with eb = 1..28 per lane, so its table indices are (e >> 4) = 2*Sigma + hi and
+        // (e & 15) = lo with hi, lo fixed per (lane, ib): one address per lane, the rest are immediate offsets.
+        {
+            const int eb = li_sample(0, m) + 1;
 #pragma unroll
-        for (int f = 0; f < 8; ++f) {               // Pout: output sample i of (Sigma, ib) x state rows 8*qa + k
-            if (!mine(f)) continue;
-            const int Sg = f >> 1, ib = f & 1;
-            const int e = 32 * Sg + li_sample(ib, m) + 1;          // Re / -Im of r * p^(i+1)
+            for (int ib = 0; ib < 2; ++ib) {
+                const int hi = (eb + 4 * ib) >> 4, lo = (eb + 4 * ib) & 15;
+                const float2* pa0 = t16 + (4 * qa) * 9 + hi;
+                float2 rb[4];
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-                const int s = 4 * qa + kk;
-                const float2 pa = t16[s * 9 + (e >> 4)], pb = tr[s * 16 + (e & 15)];
-                val[2 * kk] = pa.x * pb.x - pa.y * pb.y;
-                val[2 * kk + 1] = -(pa.x * pb.y + pa.y * pb.x);
+                for (int kk = 0; kk < 4; ++kk) rb[kk] = tr[(4 * qa + kk) * 16 + lo];
+#pragma unroll
+                for (int Sg = 0; Sg < 4; ++Sg) {
+                    const int f = 2 * Sg + ib;
+                    if (!mine(f)) continue;
+#pragma unroll
+                    for (int kk = 0; kk < 4; ++kk) {
+                        const float2 pa = pa0[kk * 9 + 2 * Sg];
+                        val[2 * kk] = pa.x * rb[kk].x - pa.y * rb[kk].y;
+                        val[2 * kk + 1] = -(pa.x * rb[kk].y + pa.y * rb[kk].x);
+                    }
+                    li_split(val, th[FR_PO + f], th[FR_PO + 8 + f]);
+                }
             }
-            li_split(val, th[FR_PO + f], th[FR_PO + 8 + f]);
         }
+        // Pin: state row 16*mu + m x inputs 32*kappa + 8*qa + k hold Re or Im (row parity) of p^(127 - j).  With
+        // e = 127 - 32*kappa - 8*qa - k the coarse index (e >> 4) = 7 - (qa >> 1) - 2*kappa does not depend on k and the
+        // fine one (e & 15) = 15 - 8*(qa & 1) - k not on kappa (no borrow for k = 0..7).
+        {
+            const bool im_row = m & 1;
 #pragma unroll
-        for (int f = 0; f < 8; ++f) {               // Pin: state row 16*mu + m x inputs 32*kappa + 8*qa + k
-            if (!mine(f)) continue;
-            const int mu = f >> 2, kp = f & 3;
-            const int s = 8 * mu + (m >> 1);
+            for (int mu = 0; mu < 2; ++mu) {
+                const int s = 8 * mu + (m >> 1);
+                const float2* pb0 = t1 + s * 16 + 15 - 8 * (qa & 1);
+                const float2* pa0 = t16 + s * 9 + 7 - (qa >> 1);
+                float2 pb[8];
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const int e = C - 1 - (32 * kp + 8 * qa + k);      // p^(127 - j)
-                const float2 pa = t16[s * 9 + (e >> 4)], pb = t1[s * 16 + (e & 15)];
-                const float re = pa.x * pb.x - pa.y * pb.y, im = pa.x * pb.y + pa.y * pb.x;
-                val[k] = (m & 1) ? im : re;
+                for (int k = 0; k < 8; ++k) pb[k] = pb0[-k];
+#pragma unroll
+                for (int kp = 0; kp < 4; ++kp) {
+                    const int f = 4 * mu + kp;
+                    if (!mine(f)) continue;
+                    const float2 pa = pa0[-2 * kp];
+                    // Re = pa.x*pb.x - pa.y*pb.y, Im = pa.y*pb.x + pa.x*pb.y
+                    const float ca = im_row ? pa.y : pa.x, cb = im_row ? pa.x : -pa.y;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) val[k] = ca * pb[k].x + cb * pb[k].y;
+                    li_split(val, th[FR_PI + f], th[FR_PI + 8 + f]);
+                }
             }
-            li_split(val, th[FR_PI + f], th[FR_PI + 8 + f]);
         }
         if (COOP) {
 #pragma unroll
