@@ -156,6 +156,9 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     const int64_t t_end = (t_begin + seg_len < L) ? t_begin + seg_len : L;
     if (t_begin >= t_end) return;
     const int64_t ts0 = t_begin > 0 ? t_begin - TL : 0;      // one extra step rebuilds the halo of a later segment
+    // a short filter (MLO = 7: K <= 17) only reaches 16 samples back, the featurizer at most 3 more: of the halo
+    // step only the last 24 rows are read, the rest stay zero and feed no output of this segment
+    const int64_t t_lo = MLO == 7 ? t_begin - 24 : ts0;
 
     // zero halo at the sequence start
     if (t_begin == 0) {
@@ -171,7 +174,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
             const int64_t t = ts + 4 * rb + r - RF;
-            const bool ok = ch_ok && t >= 0 && t < t_end;
+            const bool ok = ch_ok && t >= t_lo && t >= 0 && t < t_end;
 #pragma unroll
             for (int i = 0; i < NP; ++i) raw[i][r] = ok ? *(const u32x4*)(pp[i] + t * pstr[i]) : zero4;
         }
@@ -396,7 +399,11 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     if (B == 0 || L == 0) return 0;
 
     // Segments along L.  512 blocks are resident at a time (2 per CU); pick the segment count whose block
-    // count fills whole rounds of 512 best, charging each segment its extra 128-sample halo step.
+    // count fills whole rounds of 512 best, charging each segment its extra halo step: 128 samples, or about a
+    // third of that for the short-filter variant, which reads only the last 24 rows of it.
+    const bool aux = y2_out || bx_out;
+    const bool shortk = K <= 17 && a.pre && bias_mode == HYENA_BIAS_NONE && !aux;
+    const double halo_cost = shortk ? 40.0 : (double)TL;
     const int64_t ndb = (D + CB - 1) / CB;
     const int64_t rows = B * ndb;
     int64_t nseg = 1;
@@ -407,7 +414,7 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
             const int64_t sl = ((L + c - 1) / c + TL - 1) / TL * TL;
             const int64_t nb = rows * ((L + sl - 1) / sl);
             const double fill = (double)nb / (double)((nb + 511) / 512 * 512);
-            const double score = fill * (double)sl / (double)(sl + TL);
+            const double score = fill * (double)sl / ((double)sl + halo_cost);
             if (score > best + 1e-9) { best = score; nseg = c; }
         }
     }
@@ -421,8 +428,6 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)nblk);
     const int dg = (int)(D / G);
-    const bool aux = y2_out || bx_out;
-    const bool shortk = K <= 17;
     bool ok = false;
 #define CL_GO(P, Q, M, F, KSV, AX, ML)                                                                            \
     hipLaunchKernelGGL((fir_cl_kernel<P, Q, M, F, KSV, AX, ML>), grid, dim3(256), 0, s, a.x1, a.x2, a.v, a.pj, h, \
@@ -431,7 +436,7 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
 #define CL_CASE(P, Q, M, F, KSV)                                                                                  \
     if (!ok && a.pre == P && a.post == Q && bias_mode == M && a.feat == F && (F == 0 || a.ks == KSV)) {           \
         if (aux) CL_GO(P, Q, M, F, KSV, true, 0);                                                                 \
-        else if (shortk && P && M == HYENA_BIAS_NONE) CL_GO(P, Q, M, F, KSV, false, (P && M == HYENA_BIAS_NONE) ? 7 : 0); \
+        else if (shortk) CL_GO(P, Q, M, F, KSV, false, (P && M == HYENA_BIAS_NONE) ? 7 : 0);                      \
         else CL_GO(P, Q, M, F, KSV, false, 0);                                                                    \
         ok = true;                                                                                                \
     }
