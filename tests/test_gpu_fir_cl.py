@@ -232,3 +232,22 @@ def test_layer_projection_beyond_32_bit_offsets():
     zs = torch.stack([z[0, i * D + d, L - 4096:] for d in ds.tolist() for i in range(3)]).cpu()
     zr, _ = O.parallel_fir(us, wf.cpu()[ch][:, None, :], None, fir_length=Ks, dim_last=True, gate=False)
     assert rel_err(zs, zr[0][:, 256:]) <= 1e-2
+
+
+@pytest.mark.parametrize("K", [7, 128])
+def test_cl_nontemporal_variants_match(K, monkeypatch):
+    # tensors larger than the last-level cache use non-temporal accesses (another instantiation of the kernel):
+    # forced on at a small size, it must give the same bits, for the gated form and the fused layer
+    B, L, D, G, Ks = 2, 1000, 128, 8, 3
+    g = torch.Generator().manual_seed(K)
+    x1, x2, v = (torch.randn(B, L, D, generator=g).bfloat16().to(DEV) for _ in range(3))
+    u = torch.randn(B, L, 3 * D, generator=g).bfloat16().to(DEV)
+    wf = (torch.randn(Ks, 3 * D, generator=g) / Ks ** 0.5).to(DEV)
+    h = (O.make_mr_filter(G, K) if K == 128 else O.make_se_filter(G, K)).reshape(G, K).to(DEV)
+    cmap = ops.gate_channel_map(D, interleave=True)
+    res = {}
+    for nt in ("0", "1"):
+        monkeypatch.setenv("HYENA_CL_NT", nt)
+        res[nt] = (ops.fir_cl_fwd(x1, x2, v, h, taps_reversed=K < 128),
+                   ops.fir_layer_fwd(u, wf, None, cmap, h, taps_reversed=K < 128))
+    assert torch.equal(res["0"][0], res["1"][0]) and torch.equal(res["0"][1], res["1"][1])

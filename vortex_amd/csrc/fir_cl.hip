@@ -63,7 +63,9 @@ __device__ __forceinline__ float el(const u32x4& r, int e) { return (e & 1) ? bf
 // KS = featurizer taps (FEAT != 0).  AUX = also store y2 (z before the x2 gate) and / or bx = bf16(x1*v).
 // MLO = first Toeplitz block that can be non-zero: 0 for any K <= 128, 7 for K <= 17 (lags 0..16 touch only
 // blocks 7..9), which leaves three A fragments in registers and five B reads / six MFMAs per step.
-template <bool PRE, bool POST, int BIAS, int FEAT, int KS, bool AUX, int MLO>
+// NT = non-temporal accesses for tensors that stream through the last-level cache: the output rows always, the
+// input rows only without the fused featurizer (its lanes re-read their neighbours' rows, which must stay cached).
+template <bool PRE, bool POST, int BIAS, int FEAT, int KS, bool AUX, int MLO, bool NT>
 __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMap v, ProjFwd pj,
                                                         const float* __restrict__ h, int K, int reversed,
                                                         const float* __restrict__ bias, bf16_t* __restrict__ out,
@@ -176,7 +178,8 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             const int64_t t = ts + 4 * rb + r - RF;
             const bool ok = ch_ok && t >= t_lo && t >= 0 && t < t_end;
 #pragma unroll
-            for (int i = 0; i < NP; ++i) raw[i][r] = ok ? *(const u32x4*)(pp[i] + t * pstr[i]) : zero4;
+            for (int i = 0; i < NP; ++i) raw[i][r] = ok ? ((NT && !FEAT) ? __builtin_nontemporal_load((const u32x4*)(pp[i] + t * pstr[i]))
+                                                                 : *(const u32x4*)(pp[i] + t * pstr[i])) : zero4;
         }
     };
     load_step(ts0);
@@ -366,7 +369,8 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                         for (int j = 0; j < 4; ++j)
                             o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(g2[q][j]), bf_hi(zz[j]) * bf_hi(g2[q][j]));
                     }
-                    *(u32x4*)(out + (b * L + t) * D + dch) = o;
+                    if (NT) __builtin_nontemporal_store(o, (u32x4*)(out + (b * L + t) * D + dch));
+                    else *(u32x4*)(out + (b * L + t) * D + dch) = o;
                 }
             }
         }
@@ -428,16 +432,21 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)nblk);
     const int dg = (int)(D / G);
+    // tensors larger than the last-level cache stream through it: non-temporal accesses then
+    bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
+    if (const char* e = getenv("HYENA_CL_NT")) nt = atoi(e) != 0;
     bool ok = false;
-#define CL_GO(P, Q, M, F, KSV, AX, ML)                                                                            \
-    hipLaunchKernelGGL((fir_cl_kernel<P, Q, M, F, KSV, AX, ML>), grid, dim3(256), 0, s, a.x1, a.x2, a.v, a.pj, h, \
+#define CL_GO(P, Q, M, F, KSV, AX, ML, N)                                                                         \
+    hipLaunchKernelGGL((fir_cl_kernel<P, Q, M, F, KSV, AX, ML, N>), grid, dim3(256), 0, s, a.x1, a.x2, a.v, a.pj, h, \
                        K, taps_reversed, bias, (bf16_t*)out, (bf16_t*)y2_out, (bf16_t*)bx_out, bx_from, L, D, dg,   \
                        seg_len, (int)nseg, (int)ndb)
 #define CL_CASE(P, Q, M, F, KSV)                                                                                  \
     if (!ok && a.pre == P && a.post == Q && bias_mode == M && a.feat == F && (F == 0 || a.ks == KSV)) {           \
-        if (aux) CL_GO(P, Q, M, F, KSV, true, 0);                                                                 \
-        else if (shortk) CL_GO(P, Q, M, F, KSV, false, (P && M == HYENA_BIAS_NONE) ? 7 : 0);                      \
-        else CL_GO(P, Q, M, F, KSV, false, 0);                                                                    \
+        if (aux) CL_GO(P, Q, M, F, KSV, true, 0, false);                                                          \
+        else if (shortk && nt) CL_GO(P, Q, M, F, KSV, false, (P && M == HYENA_BIAS_NONE) ? 7 : 0, true);          \
+        else if (shortk) CL_GO(P, Q, M, F, KSV, false, (P && M == HYENA_BIAS_NONE) ? 7 : 0, false);               \
+        else if (nt) CL_GO(P, Q, M, F, KSV, false, 0, true);                                                      \
+        else CL_GO(P, Q, M, F, KSV, false, 0, false);                                                             \
         ok = true;                                                                                                \
     }
     CL_CASE(true, true, HYENA_BIAS_NONE, 0, 3)
