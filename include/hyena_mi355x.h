@@ -260,7 +260,9 @@ typedef struct hyena_proj_fwd {
 
 /* A whole Hyena-SE / Hyena-MR layer at prefill in one launch: featurizer FIR, split, x1*v gate, inner FIR,
  * bias rule (NONE or GATED_FP32), x2 gate; u [B][L][3D] in, out [B][L][D], nothing in between touches device
- * memory.  Replaces the two parallel_fir calls of vortex/model/model.py:233-291.  bx_out / bx_from as above. */
+ * memory.  Replaces the two parallel_fir calls of vortex/model/model.py:233-291.  bx_out / bx_from as above, but
+ * here bx is the cache tail only: L - bx_from may not exceed K - 1 (it is copied out of the kernel's LDS ring after
+ * the last step). */
 int hyena_fir_layer_fwd(const hyena_proj_fwd* proj,
                         const float* h, int taps_reversed, const float* bias, int bias_mode,
                         void* out, void* bx_out, int64_t bx_from,

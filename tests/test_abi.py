@@ -94,3 +94,15 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libhyena_mi355x.so")
     with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
         _lib.lib()
+
+
+def test_fused_layer_tail_limit_is_checked_before_launch():
+    # with the featurizer fused in, bx_out is the cache tail: more than K-1 rows is refused
+    from vortex_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built in this tree")
+    L = _lib.lib()
+    P = 4096
+    pj = _lib.ProjFwd(P, 192, 192, P, None, 3, 0, 64, 0, 64, 1)
+    assert L.hyena_fir_layer_fwd(ctypes.byref(pj), P, 0, None, 0, P, P, 100, 1, 200, 64, 4, 7, None) == -3
+    assert b"cache tail" in L.hyena_last_error_string()

@@ -60,7 +60,9 @@ __device__ __forceinline__ float el(const u32x4& r, int e) { return (e & 1) ? bf
 
 // FEAT: 0 = gates given as three channel-last tensors; 1 = gates from the fused featurizer, unit channel
 // stride (plain or head-blocked split); 3 = fused featurizer with interleaved gates (channel 3d+i).
-// KS = featurizer taps (FEAT != 0).  AUX = also store y2 (z before the x2 gate) and / or bx = bf16(x1*v).
+// KS = featurizer taps (FEAT != 0).  AUX = also store y2 (z before the x2 gate) and / or bx = bf16(x1*v).  With the
+// featurizer fused in, bx is the cache tail (at most the last K-1 samples): it is copied out of the LDS ring after
+// the last step, which keeps the step loop free of the extra stores and their registers.
 // MLO = first Toeplitz block that can be non-zero: 0 for any K <= 128, 7 for K <= 17 (lags 0..16 touch only
 // blocks 7..9), which leaves three A fragments in registers and five B reads / six MFMAs per step.
 // NT = non-temporal accesses for tensors that stream through the last-level cache: the output rows always, the
@@ -188,7 +190,9 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     if (BIAS != HYENA_BIAS_NONE && slab_live) bz = bias[d0 + 16 * w + (n & 15)];
 
     int cur = 0;                       // ring chunk the current step writes; the other one is its halo
+    int64_t ts_last = ts0;
     for (int64_t ts = ts0; ts < t_end; ts += TL) {
+        ts_last = ts;
         const bool compute = ts >= t_begin;
         // ---- (a) gates of this lane's 4 x 8 block
         u32x4 bx[4], g2[4];
@@ -289,7 +293,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                 *(u32x2*)(ub + c * URS) = t2;
             }
         }
-        if (AUX && bx_out && compute && ch_ok) {
+        if (AUX && !FEAT && bx_out && compute && ch_ok) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int64_t t = ts + 4 * rb + q;
@@ -362,7 +366,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                     zz[j] = (q & 1) ? pair_hi(zc[2 * j][q >> 1], zc[2 * j + 1][q >> 1])
                                     : pair_lo(zc[2 * j][q >> 1], zc[2 * j + 1][q >> 1]);
                 if (t < t_end) {
-                    if (AUX && y2_out) *(u32x4*)(y2_out + (b * L + t) * D + dch) = zz;
+                    if (AUX && !FEAT && y2_out) *(u32x4*)(y2_out + (b * L + t) * D + dch) = zz;
                     u32x4 o = zz;
                     if (POST) {
 #pragma unroll
@@ -375,6 +379,26 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             }
         }
         cur ^= 1;
+    }
+
+    // ---- cache tail from the ring: chunk cur ^ 1 holds samples ts_last .. ts_last + 127, chunk cur the 128 before
+    if (AUX && FEAT && bx_out && t_end == L) {
+        const int ntail = (int)(L - bx_from);                        // <= K - 1 <= 127 (checked by the launcher)
+        for (int e = tid; e < ntail * (CB / 8); e += 256) {
+            const int ti = e >> 3, oc = e & 7;
+            const int rel = (int)(bx_from + ti - (ts_last - TL));    // 1 .. 255
+            const int chunk = rel >= TL ? (cur ^ 1) : cur, pos = rel & (TL - 1);
+            if (d0 + 8 * oc < (uint32_t)D) {
+                u32x4 o;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int c0 = 8 * oc + 2 * j, c1 = c0 + 1;      // both in slab (8*oc) >> 4
+                    const int p = chunk * TL + (pos ^ (32 * (oc >> 1)));
+                    o[j] = (uint32_t)u_lds[c0 * URS + p] | ((uint32_t)u_lds[c1 * URS + p] << 16);
+                }
+                *(u32x4*)(bx_out + (b * (int64_t)ntail + ti) * D + d0 + 8 * oc) = o;
+            }
+        }
     }
 }
 
@@ -398,6 +422,9 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     if (bias_mode < 0 || bias_mode > 2 || (bias_mode != HYENA_BIAS_NONE && !bias))
         return hyena_fail(HYENA_EINVAL, "%s: bias_mode %d needs a bias pointer", who, bias_mode);
     if (bx_out && (bx_from < 0 || bx_from > L)) return hyena_fail(HYENA_EINVAL, "%s: bx_from outside 0..L", who);
+    if (bx_out && a.feat && L - bx_from > K - 1)
+        return hyena_fail(HYENA_ENOSUP, "%s: with the featurizer fused, bx is the cache tail (at most K-1 = %d samples)",
+                          who, K - 1);
     if ((((uintptr_t)out | (uintptr_t)y2_out | (uintptr_t)bx_out) & 15))
         return hyena_fail(HYENA_EALIGN, "%s: outputs must be 16-byte aligned", who);
     if (B == 0 || L == 0) return 0;
@@ -406,7 +433,7 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     // count fills whole rounds of 512 best, charging each segment its extra halo step: 128 samples, or about a
     // third of that for the short-filter variant, which reads only the last 24 rows of it.
     const bool aux = y2_out || bx_out;
-    const bool shortk = K <= 17 && a.pre && bias_mode == HYENA_BIAS_NONE && !aux;
+    const bool shortk = K <= 17 && a.pre && bias_mode == HYENA_BIAS_NONE;
     const double halo_cost = shortk ? 40.0 : (double)TL;
     const int64_t ndb = (D + CB - 1) / CB;
     const int64_t rows = B * ndb;
@@ -442,7 +469,8 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
                        seg_len, (int)nseg, (int)ndb)
 #define CL_CASE(P, Q, M, F, KSV)                                                                                  \
     if (!ok && a.pre == P && a.post == Q && bias_mode == M && a.feat == F && (F == 0 || a.ks == KSV)) {           \
-        if (aux) CL_GO(P, Q, M, F, KSV, true, 0, false);                                                          \
+        if (aux && shortk) CL_GO(P, Q, M, F, KSV, true, (P && M == HYENA_BIAS_NONE) ? 7 : 0, false);              \
+        else if (aux) CL_GO(P, Q, M, F, KSV, true, 0, false);                                                     \
         else if (shortk && nt) CL_GO(P, Q, M, F, KSV, false, (P && M == HYENA_BIAS_NONE) ? 7 : 0, true);          \
         else if (shortk) CL_GO(P, Q, M, F, KSV, false, (P && M == HYENA_BIAS_NONE) ? 7 : 0, false);               \
         else if (nt) CL_GO(P, Q, M, F, KSV, false, 0, true);                                                      \
