@@ -246,12 +246,24 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     if (B == 0 || L == 0) return 0;
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
 
-    // segments along L: >= 4096 blocks (256 CUs x 3 resident blocks, several rounds), segments >= 2048 samples
+    // Segments along L, chosen by a cost model fitted to measurements on one MI355X: a segment costs its length
+    // plus about 160 samples for the halo and the fragment build; segments longer than 2048 samples stream about
+    // 5 % slower per doubling (with short ones the blocks of a row set work at many offsets at once, which the
+    // memory system serves faster); 768 blocks are resident at a time (3 per CU) and the last round is on average
+    // half empty.
     const int64_t rows = B * G * ((D / G + 15) / 16);          // (batch, slab) pairs
-    int64_t nseg = (4096 + rows - 1) / rows;
-    const int64_t max_seg = (L + 2047) / 2048;
-    if (nseg > max_seg) nseg = max_seg;
-    if (nseg < 1) nseg = 1;
+    int64_t nseg = 1;
+    {
+        double best = 0.0;
+        for (int64_t sl = 1024; ; sl *= 2) {
+            const int64_t c = (L + sl - 1) / sl;
+            const double nb = (double)(rows * c);
+            double cost = ((double)sl + 160.0) * (nb <= 768.0 ? 1.0 : nb / 768.0 + 0.5);
+            for (int64_t x = sl; x > 2048; x /= 2) cost *= 1.05;
+            if (best == 0.0 || cost < best) { best = cost; nseg = c; }
+            if (sl >= L) break;
+        }
+    }
     if (const char* e = getenv("HYENA_MR_NSEG")) { int64_t x = atoll(e); if (x >= 1) nseg = x; }
     int64_t seg_len = (L + nseg - 1) / nseg;
     seg_len = (seg_len + TL - 1) / TL * TL;
