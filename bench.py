@@ -26,7 +26,7 @@ HBM_PEAK_GBS = 8000.0     # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
 # counter reads for the plain copy launch of known size (profiles/bench_default_hbm_traffic.txt).
-MEASURED_TRAFFIC = {"mr": 2178.42e6, "se": 271.75e6, "li": 8603.44e6}
+MEASURED_TRAFFIC = {"mr": 2211.99e6, "se": 271.75e6, "li": 8597.09e6}
 
 
 def parse():
@@ -35,6 +35,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="mr", choices=["mr", "se", "li", "decode", "mr_cl", "mr_layer", "se_layer"])
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="untimed run of each workload before its warm-up steps, until clocks have settled")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-model", action="store_true", help="skip the end-to-end model prefill legs")
@@ -75,8 +77,20 @@ class _Synthetic:
         return log_poles, res.to(torch.complex64)
 
 
+SETTLE_S = 0.15     # set from --settle-ms
+
+
 def time_steps(fn, steps, warmup):
-    """(wall seconds for `steps` calls, average kernel-side ms per call from HIP events on the launch stream)."""
+    """(wall seconds for `steps` calls, average kernel-side ms per call from HIP events on the launch stream).
+
+    Before the `warmup` untimed steps the workload runs for SETTLE_S seconds, also untimed: after lighter work the
+    first tens of launches of a bandwidth-heavy kernel run up to 15 % slower (clock and power management settling),
+    and a short run would measure that transient instead of the sustained rate."""
+    t_end = time.perf_counter() + SETTLE_S
+    while SETTLE_S > 0 and time.perf_counter() < t_end:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -329,6 +343,8 @@ def main():
         sys.exit(1)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    global SETTLE_S
+    SETTLE_S = max(args.settle_ms, 0.0) / 1e3
 
     def run(name, steps, warmup):
         fn, d = build_workload(name, device)
@@ -359,7 +375,7 @@ def main():
         "value": m["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": m["wall_s"] / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16 in/out, fp32 accumulate", "data": "synthetic",
-        "config": {"workload": m["workload"]},
+        "config": {"workload": m["workload"], "settle_ms": args.settle_ms},
         "roofline": {"bound": "hbm", "achieved": m["hbm_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": m["hbm_gbs"] / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(main_name),
                      "kernel": m["kernel"],
@@ -367,9 +383,7 @@ def main():
     }
     if not args.no_extras:
         extra = {}
-        # the heavy kernels take about ten launches to reach steady clocks: the default run warms the extra
-        # workloads up that long; short profiling runs (--warmup below 5) keep their own count
-        extra_warmup = args.warmup if args.warmup < 5 else max(args.warmup, 10)
+        extra_warmup = args.warmup
         for name in ("se", "mr", "li"):
             if name == main_name:
                 continue
