@@ -246,8 +246,8 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
             }
     };
     // With four channels per wavefront the rows are requested before the fragment build and travel during it
-    // (measured 5 % faster at L = 8192..32768).  With one channel per wavefront the same order is 10 % slower on
-    // short rows, so there the rows are requested after the build.
+    // (measured 5 % faster at L = 8192..32768).  With one channel per wavefront the same order measured 1-3 %
+    // slower on rows up to 8192 samples and 1-2 % faster from 131072 on; there the rows are requested after the build.
     constexpr bool ROWS_FIRST = CPW == 4;
     if (ROWS_FIRST) request_rows();
 
