@@ -41,7 +41,7 @@ int main(int argc, char** argv) {
     if (!lib) { printf("dlopen failed: %s\n", dlerror()); return 2; }
 #define SYM(name) auto p_##name = (decltype(&name))dlsym(lib, #name); CHECK(p_##name, "missing symbol " #name);
     SYM(hyena_version) SYM(hyena_last_error_string) SYM(hyena_mr_fwd) SYM(hyena_fir_cl_fwd) SYM(hyena_fir_step)
-    SYM(hyena_iir_step) SYM(hyena_se_fwd)
+    SYM(hyena_iir_step) SYM(hyena_se_fwd) SYM(hyena_fir_step_dpos) SYM(hyena_ring_advance)
     printf("%s\n", p_hyena_version());
     hipStream_t stream; HIP_OK(hipStreamCreate(&stream));
 
@@ -114,6 +114,33 @@ int main(int argc, char** argv) {
             CHECK(rr == hist, "hyena_fir_step ring contents after step %d", step);
         }
         printf("hyena_fir_step on a ring cache: ok\n");
+
+        // the same ring continued with its position in device memory: seven more steps, so the ring wraps
+        std::vector<int32_t> pos_h = {2, 0}, depth_h = {(int32_t)R, 5};     // a second, unused ring of depth 5
+        int32_t *d_pos = dev(pos_h), *d_depth = dev(depth_h);
+        for (int step = 2; step < 9; ++step) {
+            const int64_t p = step % R;
+            for (size_t i = 0; i < u.size(); ++i) u[i] = to_bf16((float)((int)((i + 3 * step) % 9) - 4) / 2.f);
+            HIP_OK(hipMemcpy(d_u, u.data(), u.size() * 2, hipMemcpyHostToDevice));
+            int rc = p_hyena_fir_step_dpos(d_u, d_1, d_1, Ds, d_ring, R, d_pos, d_w, nullptr, HYENA_BIAS_NONE, d_y, Ds, Bs, Ds, Ds, stream);
+            CHECK(rc == 0, "hyena_fir_step_dpos rc=%d: %s", rc, p_hyena_last_error_string());
+            rc = p_hyena_ring_advance(d_pos, d_depth, 2, stream);
+            CHECK(rc == 0, "hyena_ring_advance rc=%d: %s", rc, p_hyena_last_error_string());
+            HIP_OK(hipStreamSynchronize(stream));
+            auto y = host(d_y, (size_t)(Bs * Ds));
+            for (int b = 0; b < Bs; ++b) for (int d = 0; d < Ds; ++d) {
+                float acc = 0.f;
+                for (int i = 0; i < R; ++i) acc += w[d * (R + 1) + i] * from_bf16(hist[(b * R + (p + i) % R) * Ds + d]);
+                acc += w[d * (R + 1) + R] * from_bf16(u[b * Ds + d]);
+                CHECK(from_bf16(y[b * Ds + d]) == from_bf16(to_bf16(acc)), "hyena_fir_step_dpos step %d b=%d d=%d got %g want %g",
+                      step, b, d, from_bf16(y[b * Ds + d]), acc);
+            }
+            for (int b = 0; b < Bs; ++b) for (int d = 0; d < Ds; ++d) hist[(b * R + p) * Ds + d] = u[b * Ds + d];
+            CHECK(host(d_ring, ring.size()) == hist, "hyena_fir_step_dpos ring contents after step %d", step);
+            auto ph = host(d_pos, 2);
+            CHECK(ph[0] == (step + 1) % R && ph[1] == (step - 1) % 5, "hyena_ring_advance positions after step %d: %d %d", step, ph[0], ph[1]);
+        }
+        printf("hyena_fir_step_dpos / hyena_ring_advance (positions in device memory): ok\n");
     }
 
     // ---- decode IIR step, real poles: state = p*state + x1v ; y = x2 * (sum r*state + D*x1v)
