@@ -57,10 +57,14 @@ def test_mr_random(B, L, seed):
     assert rel_err(out, ref) <= 2e-2, (B, D, L, G, K)
 
 
+@pytest.mark.parametrize("coop", ["0", "1"])
 @pytest.mark.parametrize("B,L,seed", cases(3, 10))
-def test_li_random(B, L, seed):
+def test_li_random(B, L, seed, coop, monkeypatch):
+    # coop = "1" forces the cooperative form (four wavefronts per set of channels) wherever groups have four channels
+    monkeypatch.setenv("HYENA_LI_COOP", coop)
     rng = random.Random(seed)
     cplx = rng.random() < 0.5
+    S = rng.choice([16, 16, 8, 3])
     dg = rng.choice([1, 2, 4, 8, 16])
     G = rng.randint(1, 3)
     D = G * dg
@@ -68,12 +72,12 @@ def test_li_random(B, L, seed):
         k = 8 // (D & -D) if (D & -D) < 8 else 1
         D, G = D * k, G * k
     x2, x1, v = O.make_gates(B, D, L, seed=seed)
-    lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(G, 16, seed=seed + 1)
+    lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(G, S, seed=seed + 1)
     Db = torch.randn(D, generator=torch.Generator().manual_seed(seed)).bfloat16()
     ref, y32_ref, st_ref = O.li_prefill(x2, x1, v, lp, r, Db)
     out, y32, st = va.hyena_li_fwd(x1.cuda(), x2.cuda(), v.cuda(), lp.cuda(), r.cuda(), Db.cuda(),
                                    want_state=True, want_fp32=True)
-    assert rel_err(y32, y32_ref) <= 1e-4, (B, D, L, G, cplx)
+    assert rel_err(y32, y32_ref) <= 1e-4, (B, D, L, G, cplx, S)
     assert rel_err(out, ref) <= 2e-2
     sr = torch.view_as_real(st) if cplx else st
     assert rel_err(sr, torch.view_as_real(st_ref) if cplx else st_ref) <= 1e-4
