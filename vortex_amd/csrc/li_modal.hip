@@ -395,11 +395,21 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
 
         // u = bf16(x1*v) of this step -> LDS; refill the stage with step ts + PF*TLW
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const bool okn = !GUARD || (tn + roff(r) + lane * 8 < Lw);
-            *(u32x4*)(u_w + r * URS + lofs) = gate_mul<PRE>(c1[p][r], cv[p][r]);
-            c1[p][r] = okn ? ld16<NT>(p1[r] + tn) : zero4;
-            cv[p][r] = (PRE && okn) ? ld16<NT>(pv[r] + tn) : zero4;
+        for (int r = 0; r < 4; ++r) *(u32x4*)(u_w + r * URS + lofs) = gate_mul<PRE>(c1[p][r], cv[p][r]);
+        // whole pieces inside the row (a wave-uniform test) are requested without per-lane predicates
+        if (tn + TLW <= Lw) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                c1[p][r] = ld16<NT>(p1[r] + tn);
+                if (PRE) cv[p][r] = ld16<NT>(pv[r] + tn);
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const bool okn = tn + roff(r) + lane * 8 < Lw;
+                c1[p][r] = okn ? ld16<NT>(p1[r] + tn) : zero4;
+                cv[p][r] = (PRE && okn) ? ld16<NT>(pv[r] + tn) : zero4;
+            }
         }
         wave_sync();
 
@@ -445,18 +455,30 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
         // ---- deferred output of the previous step: gate with x2, store, refill its x2 stage
         {
             const int64_t ts_out = ts - STEP, t_refill = ts - STEP + (int64_t)PF * STEP;
+            u32x4 o[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const bool okc = !GUARD || (ts_out >= 0 && ts_out + roff(r) + lane * 8 < Lw);
-                const bool okr = !GUARD || (ts_out >= 0 && t_refill + roff(r) + lane * 8 < Lw);
-                u32x4 o = zz[r];
+                o[r] = zz[r];
                 if (POST) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        o[j] = pack_bf2(bf_lo(zz[r][j]) * bf_lo(c2[pp][r][j]), bf_hi(zz[r][j]) * bf_hi(c2[pp][r][j]));
+                        o[r][j] = pack_bf2(bf_lo(zz[r][j]) * bf_lo(c2[pp][r][j]), bf_hi(zz[r][j]) * bf_hi(c2[pp][r][j]));
                 }
-                if (okc) st16<NT>(po[r] + ts_out, o);
-                if (!GUARD || ts_out >= 0) c2[pp][r] = (POST && okr) ? ld16<NT>(p2[r] + t_refill) : zero4;
+            }
+            if (ts_out >= 0 && t_refill + TLW <= Lw) {             // wave-uniform: store and refill whole pieces
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    st16<NT>(po[r] + ts_out, o[r]);
+                    if (POST) c2[pp][r] = ld16<NT>(p2[r] + t_refill);
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const bool okc = ts_out >= 0 && ts_out + roff(r) + lane * 8 < Lw;
+                    const bool okr = ts_out >= 0 && t_refill + roff(r) + lane * 8 < Lw;
+                    if (okc) st16<NT>(po[r] + ts_out, o[r]);
+                    if (ts_out >= 0) c2[pp][r] = (POST && okr) ? ld16<NT>(p2[r] + t_refill) : zero4;
+                }
             }
         }
         wave_sync();
