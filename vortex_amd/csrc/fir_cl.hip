@@ -74,7 +74,6 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                                                         bf16_t* __restrict__ y2_out, bf16_t* __restrict__ bx_out,
                                                         int64_t bx_from, int64_t L, int64_t D, int dg,
                                                         int64_t seg_len, int nseg, int ndb) {
-    constexpr bool EARLY = !FEAT;                  // next step's rows requested before (true) or after the MFMA phase
     constexpr int RF = FEAT ? KS - 1 : 0;          // extra rows a lane reads before its own four
     constexpr int NR = 4 + RF;                     // rows per lane and load piece
     constexpr int NP = (FEAT || (PRE && POST)) ? 3 : (PRE ? 2 : 1);   // load pieces per row
@@ -174,16 +173,22 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
 
     u32x4 raw[NP][NR];
     const u32x4 zero4 = {0, 0, 0, 0};
-    auto load_step = [&](int64_t ts) {
+    auto load_pieces = [&](int64_t ts, int i0, int i1) {
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
             const int64_t t = ts + 4 * rb + r - RF;
             const bool ok = ch_ok && t >= t_lo && t >= 0 && t < t_end;
 #pragma unroll
-            for (int i = 0; i < NP; ++i) raw[i][r] = ok ? ((NT && !FEAT) ? __builtin_nontemporal_load((const u32x4*)(pp[i] + t * pstr[i]))
+            for (int i = 0; i < NP; ++i) if (i >= i0 && i < i1) raw[i][r] = ok ? ((NT && !FEAT) ? __builtin_nontemporal_load((const u32x4*)(pp[i] + t * pstr[i]))
                                                                  : *(const u32x4*)(pp[i] + t * pstr[i])) : zero4;
         }
     };
+    auto load_step = [&](int64_t ts) { load_pieces(ts, 0, NP); };
+    // Pieces of the next step requested before the MFMA phase (the rest after it).  Without the featurizer all
+    // of them travel during the MFMA phase.  With it a lane holds 18 row pieces, which next to all ten A fragments
+    // do not fit the register budget of two blocks per CU: one piece goes out early (measured 4 % faster for the
+    // medium filter than none, two spill), none for the short-filter form.
+    constexpr int NEARLY = FEAT ? (MLO == 0 ? 1 : 0) : NP;
     load_step(ts0);
 
     float bz = 0.f;
@@ -275,12 +280,9 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                 if (POST) g2[q] = raw[NP - 1][q];
             }
         }
-        // ---- (b) next step's rows are requested now and arrive during the MFMA phase
-        // With the featurizer fused in, a lane holds 18 row pieces; next to all ten A fragments, keeping them in
-        // flight across the MFMA phase does not fit the register budget of two blocks per CU, so they are
-        // requested after it instead (measured: no slower than the early request where both fit).
+        // ---- (b) next step's rows (NEARLY pieces of them) are requested now and arrive during the MFMA phase
         __builtin_amdgcn_sched_barrier(0);
-        if (EARLY && ts + TL < t_end) load_step(ts + TL);
+        if (ts + TL < t_end) load_pieces(ts + TL, 0, NEARLY);
 
         // ---- (c) 4 x 8 transpose into the ring chunk `cur`
         {
@@ -347,9 +349,9 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             }
         }
         __syncthreads();
-        if (!EARLY) {
+        if (NEARLY < NP) {
             __builtin_amdgcn_sched_barrier(0);
-            if (ts + TL < t_end) load_step(ts + TL);
+            if (ts + TL < t_end) load_pieces(ts + TL, NEARLY, NP);
         }
 
         // ---- 8 x 4 transpose back, gate with x2, store rows
