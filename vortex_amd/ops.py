@@ -159,7 +159,8 @@ def fir_layer_fwd(u, feat_w, feat_bias, channel_map, taps, *, bias=None, bias_mo
     """A whole Hyena-SE / MR layer at prefill in one launch: u [B, L, 3D] bf16 -> out [B, L, D] bf16.
 
     feat_w [Ks, 3D] float32 (tap-major, last row on the current sample), feat_bias [3D] or None, channel_map from
-    gate_channel_map().  bx_from: also return rows bx_from.. of bf16(x1*v) (the inner FIR cache of a decode step).
+    gate_channel_map().  bx_from: also return rows bx_from.. of bf16(x1*v), the inner FIR cache of a decode step
+    (at most the last K-1 rows: L - bx_from <= K - 1).
     """
     _need_cuda(u, feat_w, taps)
     if u.dtype != torch.bfloat16 or u.dim() != 3 or u.stride(2) != 1:
