@@ -261,19 +261,37 @@ def modal_state_closed_form(x1v, log_poles, dtype=torch.float64):
     return torch.einsum("dsl,bdl->bds", w, x1v.to(cdt))
 
 
+def truncated_fir(x1v, h, threshold):
+    """The long_fir_threshold branch of parallel_iir (engine.py:339-349): the first `threshold` samples of the
+    materialised filter h [1, D, L], cast to the activations' dtype, applied with F.conv1d and padding
+    threshold-1.  conv1d is a cross-correlation, so tap h[threshold-1] lands on the current sample and h[0] on
+    the oldest one: y[t] = sum_j h[threshold-1-j] * x1v[t-j], computed in the activations' dtype."""
+    assert h.shape[0] == 1, "batch size must be 1 for long_fir_threshold"
+    w = h[0][:, None][..., :threshold]
+    L = x1v.shape[-1]
+    return F.conv1d(x1v, w.to(dtype=x1v.dtype), stride=1, groups=x1v.shape[1], padding=w.shape[-1] - 1)[..., :L]
+
+
 def parallel_iir(
     z_pre, h, D, L, poles, residues, dims, column_split_hyena=False,
     flip_x1x2=False, want_state=False, keep_complex_state=False, return_fp32_conv=False,
+    long_fir_threshold=None,
 ):
-    """Restatement of HyenaInferenceEngine.parallel_iir, default FFT branch.
+    """Restatement of HyenaInferenceEngine.parallel_iir: the default FFT branch and the truncated-FIR branch.
 
     engine.py:283-353 and :379-404.  Returns (y [B, L, D], state or None[,
     y_conv_fp32]).  Cast order: y = bf16(conv); out = (y + x1v*D)*x2 in the
-    tensors' own dtypes.
+    tensors' own dtypes.  With long_fir_threshold the reference has no spectrum to prefill the state from
+    (engine.py:380-392 reads X_s, which that branch never assigns), so the branch only exists without a cache.
     """
     hidden, _, _, state_size, groups = dims
     x2, x1, v = split_gates(z_pre, dims, column_split_hyena, flip_x1x2)
     x1v = x1 * v
+    if long_fir_threshold is not None:
+        assert not want_state, "the reference cannot prefill the modal state on this branch"
+        y = truncated_fir(x1v, h, long_fir_threshold).to(x1v.dtype)
+        y = (y + x1v * D.unsqueeze(-1)) * x2
+        return (y.permute(0, 2, 1), None)
     y32, X_s = long_conv_fp32(x1v, h)
     y = y32.to(x1v.dtype)
     y = (y + x1v * D.unsqueeze(-1)) * x2
@@ -494,7 +512,7 @@ class OracleEngine:
                      long_fir_threshold=None):
         y, state = parallel_iir(z_pre, h, D, L, poles, residues, dims, column_split_hyena,
                                 self.hyena_flip_x1x2, inference_params is not None,
-                                keep_complex_state=poles.is_complex())
+                                keep_complex_state=poles.is_complex(), long_fir_threshold=long_fir_threshold)
         if inference_params is not None:
             inference_params.state_dict[layer_idx] = state
         return y
@@ -560,7 +578,8 @@ class OracleCascade:
     """
 
     def __init__(self, engine, params, hidden, n_heads, groups, layer_idx=0, fir_inner_filter_length=None,
-                 column_split_hyena=False, interleave=False, state_size=16):
+                 column_split_hyena=False, interleave=False, state_size=16, long_fir_threshold=None):
+        self.long_fir_threshold = long_fir_threshold            # model.py:185
         self.engine, self.p = engine, params
         self.hidden, self.n_heads, self.groups = hidden, n_heads, groups
         self.layer_idx, self.K = layer_idx, fir_inner_filter_length
@@ -605,7 +624,7 @@ class OracleCascade:
                 z_pre, h, p["D"], L, t=None, poles=p["log_poles"], residues=p["residues"], dims=dims,
                 inference_params=inference_params, layer_idx=self.layer_idx, prefill_style="fft",
                 use_flashfft=False, fftconv_fn=None, column_split_hyena=self.column_split_hyena,
-                long_fir_threshold=None, padding_mask=padding_mask)
+                long_fir_threshold=self.long_fir_threshold, padding_mask=padding_mask)
         return y, inference_params
 
     def sequential_forward(self, u, inference_params):

@@ -422,3 +422,52 @@ def test_operator_module_padding_mask(kind):
     y_ref, _ = ref.forward(u, None, padding_mask=mask)
     y_hip, _ = mod(u.to(DEV), None, padding_mask=mask.to(DEV))
     assert rel_err(y_hip, y_ref) <= 2e-2
+
+
+@pytest.mark.parametrize("T,L,cs", [(128, 1024, False), (32, 520, True), (7, 333, False)])
+def test_engine_parallel_iir_truncated_fir_branch(T, L, cs):
+    # long_fir_threshold (vortex/model/engine.py:339-349): the first T samples of the materialised modal filter as a
+    # bf16 depthwise FIR, in the orientation F.conv1d gives them.  Engine against the oracle's restatement.
+    B, D, H = 1, 32, 4
+    g = torch.Generator().manual_seed(T)
+    lp, r = O.make_modal_real(D, 16, seed=T, pmax=0.99)
+    h = O.modal_filter(lp, r, L)                                   # [1, D, L]
+    z_pre = torch.randn(B, 3 * D, L, generator=g).bfloat16()
+    Db = torch.randn(D, generator=g).bfloat16()
+    dims = (D, H, D // H, 16, D)
+    y_ref, _ = O.parallel_iir(z_pre, h, Db, L, lp, r, dims, column_split_hyena=cs, long_fir_threshold=T)
+    eng = HyenaInferenceEngine()
+    y = eng.parallel_iir(z_pre.to(DEV), h.to(DEV), Db.to(DEV), L, lp.to(DEV), r.to(DEV), None, dims, 0,
+                         column_split_hyena=cs, long_fir_threshold=T)
+    assert y.shape == (B, L, D) and rel_err(y, y_ref) <= 2e-2
+    with pytest.raises(NotImplementedError):                        # the reference cannot prefill a cache on this branch
+        eng.parallel_iir(z_pre.to(DEV), h.to(DEV), Db.to(DEV), L, lp.to(DEV), r.to(DEV), None, dims, 0,
+                         inference_params=HyenaCascadeIIRInferenceParams(), long_fir_threshold=T)
+    with pytest.raises(NotImplementedError):
+        eng.parallel_iir(z_pre.to(DEV), h.to(DEV), Db.to(DEV), L, lp.to(DEV), r.to(DEV), None, dims, 0,
+                         long_fir_threshold=200)
+
+
+@pytest.mark.parametrize("T,G", [(128, 4), (16, 64)])
+def test_operator_module_truncated_fir_config(T, G):
+    # `long_fir_threshold` in the model configuration (vortex/model/model.py:185, :310): the operator module builds
+    # the T filter samples itself and runs them as a grouped FIR; against the oracle call sequence
+    B, L, D, H = 2, 700, 64, 4
+    p = make_params("li_real", D, G, seed=T)
+    pr = dict(p, log_poles=p["log_poles"].repeat_interleave(D // G, 0), residues=p["residues"].repeat_interleave(D // G, 0))
+    ref = O.OracleCascade(O.OracleEngine(), pr, D, H, D, interleave=True, long_fir_threshold=T)
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=False, interleave=True, short_filter_length=3,
+               short_filter_bias=False, state_size=16, long_fir_threshold=T)
+    mod = HyenaCascade(cfg, 0, hyena_filter_groups=G)
+    with torch.no_grad():
+        mod.short_filter_weight.copy_(p["short_filter_weight"])
+        mod.log_poles.copy_(p["log_poles"])
+        mod.residues.copy_(p["residues"])
+        mod.D.data = p["D"].clone()
+    mod = mod.to(DEV)
+    u = torch.randn(B, L, 3 * D, generator=torch.Generator().manual_seed(3)).bfloat16()
+    y_ref, _ = ref.forward(u)
+    y, _ = mod(u.to(DEV))
+    assert rel_err(y, y_ref) <= 2e-2
+    with pytest.raises(NotImplementedError):
+        mod(u.to(DEV), HyenaCascadeIIRInferenceParams())

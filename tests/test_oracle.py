@@ -312,3 +312,35 @@ def test_step_iir_consistent_with_prefill(cplx):
         assert (yr.float() - exp).abs().max() <= 2e-2 * exp.abs().max()
     s_ref = O.modal_state_closed_form(x1 * v, lp)
     assert (state.to(s_ref.dtype) - s_ref).abs().max() <= 1e-4 * s_ref.abs().max()
+
+
+@pytest.mark.parametrize("T", [1, 5, 32])
+def test_truncated_fir_branch_of_parallel_iir(T):
+    # long_fir_threshold (vortex/model/engine.py:339-349): F.conv1d correlates, so the truncated filter is applied
+    # with h[T-1] on the current sample.  Impulse response and a float64 brute force pin the orientation; the
+    # whole branch follows with the usual gating.
+    B, D, L = 1, 4, 48
+    g = torch.Generator().manual_seed(50 + T)
+    h = torch.randn(1, D, L, generator=g)
+    hb = h[0, :, :T].bfloat16().double()
+    x = torch.zeros(B, D, L).bfloat16()
+    x[:, :, 7] = 1.0
+    y = O.truncated_fir(x, h, T)
+    for j in range(T):
+        assert torch.equal(y[0, :, 7 + j].double(), hb[:, T - 1 - j])           # y[t0 + j] = h[T-1-j]
+    assert y[0, :, :7].abs().max() == 0 and y[0, :, 7 + T:].abs().max() == 0
+    x = torch.randn(B, D, L, generator=g).bfloat16()
+    y = O.truncated_fir(x, h, T).double()
+    want = torch.zeros(B, D, L, dtype=torch.float64)
+    for t in range(L):
+        for j in range(min(T, t + 1)):
+            want[0, :, t] += hb[:, T - 1 - j] * x[0, :, t - j].double()
+    assert (y - want).abs().max() <= 2 ** -8 * want.abs().max()                 # one bf16 rounding of the sum
+    z_pre = torch.randn(B, 3 * D, L, generator=g).bfloat16()
+    Db = torch.randn(D, generator=g).bfloat16()
+    dims = (D, 2, D // 2, 16, D)
+    out, st = O.parallel_iir(z_pre, h, Db, L, None, None, dims, long_fir_threshold=T)
+    x2, x1, v = z_pre.split(D, 1)
+    x1v = x1 * v
+    assert st is None
+    assert torch.equal(out, ((O.truncated_fir(x1v, h, T) + x1v * Db[:, None]) * x2).permute(0, 2, 1))

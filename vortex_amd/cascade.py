@@ -110,6 +110,7 @@ class HyenaCascade(nn.Module):
         self.hyena_flip_x1x2 = _cfg(config, "hyena_flip_x1x2", False)
         self.interleave = _cfg(config, "interleave", False)
         self.short_filter_length = _cfg(config, "short_filter_length", 3)
+        self.long_fir_threshold = _cfg(config, "long_fir_threshold", None)      # vortex/model/model.py:185
         self.fir_inner_filter_length = fir_inner_filter_length
         self.short_filter_weight = nn.Parameter(torch.randn(3 * D, 1, self.short_filter_length))
         self.short_filter_bias = nn.Parameter(torch.randn(3 * D)) if _cfg(config, "short_filter_bias", False) else None
@@ -216,6 +217,20 @@ class HyenaCascade(nn.Module):
                 y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, K, device=u.device, taps_reversed=True)
             if masked:
                 y = y * mask     # a 0/1 mask on the convolution commutes with the x2 gate
+        elif self.long_fir_threshold is not None:
+            # vortex/model/engine.py:339-349: the first `threshold` samples of the modal filter as a bf16 FIR, with
+            # the last of them on the current sample (F.conv1d correlates); the reference cannot prefill a cache here
+            if caching:
+                raise NotImplementedError("long_fir_threshold with a cache: the reference has no state prefill on "
+                                          "this branch (vortex/model/engine.py:380-392 reads an unassigned X_s)")
+            T = min(int(self.long_fir_threshold), L_true)
+            if T > 128:
+                raise NotImplementedError("long_fir_threshold above 128 taps has no kernel")
+            t = torch.arange(T, device=u.device)[None, None]
+            h = (self.residues.detach()[..., None] * torch.exp(self.log_poles.detach() * t)).sum(1)
+            taps = (h.real if h.is_complex() else h).to(torch.bfloat16).to(torch.float32).contiguous()   # [G, T]
+            y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, T, device=u.device, bias=self._f32_param("D"),
+                                 bias_mode=HYENA_BIAS_GATED_FP32, taps_reversed=True, force_mfma=True)
         else:
             y, _, state = ops.li_fwd_rows(r1, r2, rv, self.modal_plan(), self.D, B, D, L, device=u.device,
                                           want_state=caching)

@@ -131,9 +131,10 @@ class HyenaInferenceEngine:
                      column_split_hyena=False, long_fir_threshold=None):
         """vortex/model/engine.py:262-404.  `h` (the materialised filter) is not read: the kernel works
         from `poles` (log-poles) and `residues` directly.  Returns y [B, L, D]; writes the modal state
-        into inference_params.state_dict[layer_idx]."""
-        if long_fir_threshold is not None:
-            raise NotImplementedError("long_fir_threshold (truncated bf16 FIR) is not supported")
+        into inference_params.state_dict[layer_idx].  With long_fir_threshold (engine.py:339-349) the first
+        `threshold` samples of `h`, rounded to bf16, run as a per-channel FIR in the orientation F.conv1d gives
+        them there (h[threshold-1] on the current sample); up to 128 taps, and, as in the reference, without a
+        cache to prefill."""
         if z_pre.dtype != torch.bfloat16:
             raise TypeError(f"the gfx950 Hyena kernels take bfloat16 activations, got {z_pre.dtype}")
         hidden, n_heads, head_dim = dims[0], dims[1], dims[2]
@@ -143,6 +144,20 @@ class HyenaInferenceEngine:
         r2, r1, rv = (ops.rows_of_projection(zp, hidden, i, hd) for i in range(3))
         if self.hyena_flip_x1x2:
             r1, r2 = r2, r1
+        if long_fir_threshold is not None:
+            if inference_params is not None:
+                raise NotImplementedError("long_fir_threshold with a cache: the reference has no state prefill on "
+                                          "this branch (vortex/model/engine.py:380-392 reads an unassigned X_s)")
+            T = min(int(long_fir_threshold), h.shape[-1])
+            if T > 128:
+                raise NotImplementedError("long_fir_threshold above 128 taps has no kernel")
+            assert h.shape[0] == 1, "batch size must be 1 for long_fir_threshold"
+            taps = h[0][:, :T].to(torch.bfloat16).to(torch.float32).contiguous()       # [D, T], bf16-rounded
+            out = ops.fir_fwd_rows(r1, r2, rv, taps, B, hidden, L + pad, T, device=z_pre.device, bias=ops._f32(D),
+                                   bias_mode=HYENA_BIAS_GATED_FP32, taps_reversed=True, force_mfma=True)
+            if pad:
+                out = out[..., pad:]
+            return out.permute(0, 2, 1)
         plan = self._plan(poles, residues)
         want_state = inference_params is not None
         out, _, state = ops.li_fwd_rows(r1, r2, rv, plan, D, B, hidden, L + pad, device=z_pre.device,
