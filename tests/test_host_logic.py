@@ -176,3 +176,19 @@ def test_hyena_ops_utils_toeplitz_factors():
     direct = torch.stack([sum(hf[gi, k] * torch.cat([torch.zeros(k, dtype=torch.float64), x[gi, :n * C - k]])
                               for k in range(K)) for gi in range(g)])
     assert torch.allclose(y, direct, atol=1e-12)
+
+
+def test_operator_module_compute_filter_matches_the_closed_form():
+    # HyenaCascade.compute_filter / update_time (vortex/model/model.py:377-398) on the CPU: h[g, t] = sum_s r e^(lp t)
+    from vortex_amd.cascade import HyenaCascade
+    cfg = dict(hidden_size=16, num_attention_heads=2, state_size=4, short_filter_length=3, short_filter_bias=False)
+    mod = HyenaCascade(cfg, 0, hyena_filter_groups=2)
+    with torch.no_grad():
+        mod.log_poles.copy_(-torch.rand(2, 4, 1))
+    h, dt, lp, r = mod.compute_filter(10, "cpu")
+    assert h.shape == (1, 2, 10) and dt == torch.float32 and mod.t.shape == (1, 1, 10)
+    want = torch.stack([sum(r[g, s] * torch.exp(lp[g, s, 0] * torch.arange(10)) for s in range(4)) for g in range(2)])
+    assert torch.allclose(h[0], want, atol=1e-6)
+    assert torch.allclose(h[0, :, 0], r.sum(1), atol=1e-6)          # h[0] = sum of the residues
+    mod.update_time(6, "cpu")
+    assert mod.t.shape == (1, 1, 6)

@@ -124,6 +124,7 @@ class HyenaCascade(nn.Module):
             self.residues = nn.Parameter(torch.randn(G, self.state_size, dtype=dt))
             self.D = nn.Parameter(torch.zeros(D))
             self.h = None
+        self.t = None
         self._plan = None
         self._decode = None
         self.fuse_decode = True        # one launch per decode step where the fused layer-step kernels apply
@@ -183,6 +184,25 @@ class HyenaCascade(nn.Module):
             self._f32_cache[name] = hit
         return hit[1]
 
+    def update_time(self, L, device):
+        """vortex/model/model.py:377-388: the cached time vector [1, 1, L]."""
+        t = getattr(self, "t", None)
+        if t is None or t.shape[-1] < L or t.device != torch.device(device):
+            self.t = torch.arange(L, device=device)[None, None]
+        else:
+            self.t = t[..., :L]
+
+    def compute_filter(self, L, device):
+        """vortex/model/model.py:390-398: the materialised modal filter h [1, G, L] in float32 (the real part for
+        complex parameters) with the float32 parameters.  The kernels never need it (they work from the poles and
+        residues); it is here for callers that inspect or export the filter."""
+        self.update_time(L, device)
+        filter_dtype = torch.float32
+        cdt = torch.complex64 if self.log_poles.is_complex() else filter_dtype
+        residues, log_poles = self.residues.to(cdt), self.log_poles.to(cdt)
+        h = (residues[..., None] * (log_poles * self.t).exp()).sum(1)[None]
+        return (h.real if h.is_complex() else h), filter_dtype, log_poles, residues
+
     def modal_plan(self):
         key = (self.log_poles._version, self.residues._version, self.log_poles.data_ptr())
         if self._plan is None or self._plan[0] != key:
@@ -226,9 +246,9 @@ class HyenaCascade(nn.Module):
             T = min(int(self.long_fir_threshold), L_true)
             if T > 128:
                 raise NotImplementedError("long_fir_threshold above 128 taps has no kernel")
-            t = torch.arange(T, device=u.device)[None, None]
-            h = (self.residues.detach()[..., None] * torch.exp(self.log_poles.detach() * t)).sum(1)
-            taps = (h.real if h.is_complex() else h).to(torch.bfloat16).to(torch.float32).contiguous()   # [G, T]
+            with torch.no_grad():
+                h = self.compute_filter(T, u.device)[0][0]
+            taps = h.to(torch.bfloat16).to(torch.float32).contiguous()                     # [G, T]
             y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, T, device=u.device, bias=self._f32_param("D"),
                                  bias_mode=HYENA_BIAS_GATED_FP32, taps_reversed=True, force_mfma=True)
         else:
