@@ -361,8 +361,8 @@ def main():
         from vortex_amd import _lib
         stream = torch.cuda.current_stream().cuda_stream
         nbytes = a.numel() * 2
-        wall, ms = time_steps(lambda: _lib.check(_lib.lib().hyena_copy_probe(a.data_ptr(), b.data_ptr(), nbytes,
-                                                                             stream), "copy"), 5, 2)
+        probe = _lib.copy_probe()
+        wall, ms = time_steps(lambda: _lib.check(probe(a.data_ptr(), b.data_ptr(), nbytes, stream), "copy"), 5, 2)
         print(f"copy probe (copy_probe_kernel, 16 B/lane): 1 GiB read + 1 GiB written per launch, "
               f"{ms * 1e3:.1f} us, {2 * nbytes / (ms * 1e-3) / 1e9:.0f} GB/s", file=sys.stderr)
         del a, b

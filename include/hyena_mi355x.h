@@ -49,10 +49,15 @@ enum hyena_bias_mode {
 const char* hyena_version(void);
 const char* hyena_last_error_string(void);
 
-/* Plain device-to-device copy of nbytes (multiple of 16) with the kernels' own access shape,
- * 16 bytes per lane.  No counterpart in the reference: it is the calibration launch for
- * hardware traffic counters and the bandwidth yardstick printed by bench.py. */
-int hyena_copy_probe(const void* src, void* dst, int64_t nbytes, void* stream);
+/* Launch-shape override, for tests and tuning sweeps; no counterpart in the reference.  The launchers choose
+ * segment counts, cached / non-temporal accesses and work decompositions from the problem size; this pins one of
+ * those choices process-wide until it is reset with a negative value.  Nothing is read from the environment.
+ *   "mr_nseg", "cl_nseg", "li_nseg"            segments along L of hyena_mr_fwd, hyena_fir_cl_fwd / layer_fwd, hyena_li_fwd
+ *   "se_nt", "mr_nt", "li_nt", "cl_nt"         0 = cached, 1 = non-temporal global accesses
+ *   "li_cpw"                                    1 = one channel per wavefront in hyena_li_fwd
+ *   "li_coop"                                   0 / 1 = lone / cooperating wavefronts in hyena_li_fwd
+ * Returns 0, or HYENA_EINVAL for an unknown name. */
+int hyena_set_launch_override(const char* name, int64_t value);
 
 /* Hyena-SE: gated causal depthwise short FIR (2 <= K <= 8), direct form.
  * Replaces HyenaInferenceEngine.parallel_fir, K < 128 branch
@@ -112,7 +117,7 @@ int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v
  *   state_out[b][d][s] = sum_j p^(L-1-j) x1v[b][d][j]          (complex, (re, im) pairs)
  *
  * hyena_li_plan turns the modal parameters into a 6 KB per-group coefficient table, evaluated in double on
- * the device: the filter head h[0..127], coarse and fine powers of every pole (p^(16a), p^b, r*p^b) and 1/p.
+ * the device: the filter head h[0..127] and coarse and fine powers of every pole (p^(16a), p^b, r*p^b).
  * Each wavefront of hyena_li_fwd expands its group's table once into the MFMA operand fragments it keeps in
  * registers.  log_poles and residues are [G][S][2] float32 (re, im) pairs; real poles have im = 0.  The caller
  * owns the workspace: hyena_li_plan_bytes(G, S) bytes of device memory, reusable until the parameters change.

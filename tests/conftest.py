@@ -21,3 +21,20 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture
+def override():
+    """override(mr_nseg=4, li_coop=1, ...): pins launch-shape choices of the library (hyena_set_launch_override) so
+    that small inputs exercise the multi-segment, non-temporal or cooperative code paths; reset after the test."""
+    from vortex_amd import _lib
+    used = set()
+
+    def set_(**kv):
+        for k, v in kv.items():
+            _lib.check(_lib.lib().hyena_set_launch_override(k.encode(), int(v)), "hyena_set_launch_override")
+            used.add(k)
+
+    yield set_
+    for k in used:
+        _lib.lib().hyena_set_launch_override(k.encode(), -1)

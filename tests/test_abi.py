@@ -106,3 +106,38 @@ def test_fused_layer_tail_limit_is_checked_before_launch():
     pj = _lib.ProjFwd(P, 192, 192, P, None, 3, 0, 64, 0, 64, 1)
     assert L.hyena_fir_layer_fwd(ctypes.byref(pj), P, 0, None, 0, P, P, 100, 1, 200, 64, 4, 7, None) == -3
     assert b"cache tail" in L.hyena_last_error_string()
+
+
+def test_bad_row_descriptors_are_rejected_by_every_prefill_entry_point():
+    # a channel map that would divide by zero or wrap in the kernels' 32-bit arithmetic is an argument error
+    # (no launch): ch_inner = 0, ch_inner >= 2^31, negative ch_outer, B*D >= 2^31
+    from vortex_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built in this tree")
+    L = _lib.lib()
+    P = 4096
+    ref = ctypes.byref
+    good = _lib.Rows(P, 64 * 16, 64, 16, 16)
+    bad = [_lib.Rows(P, 64 * 16, 64, 0, 16), _lib.Rows(P, 64 * 16, 64, 1 << 32, 16), _lib.Rows(P, 64 * 16, 64, 16, -3)]
+    for r in bad:
+        for args in ((r, good, good), (good, r, good), (good, good, r)):
+            x1, x2, v = (ref(a) for a in args)
+            assert L.hyena_se_fwd(x1, x2, v, P, None, 0, P, 1, 16, 64, 1, 7, None) == -1
+            assert L.hyena_mr_fwd(x1, x2, v, P, 0, None, 0, P, 1, 16, 64, 1, 128, None) == -1
+            assert b"channel map" in L.hyena_last_error_string()
+            assert L.hyena_li_fwd(x1, x2, v, P, None, 1, P, None, None, 1, 16, 64, 1, 16, None) == -1
+            assert b"channel map" in L.hyena_last_error_string()
+    g = ref(good)
+    assert L.hyena_mr_fwd(g, g, g, P, 0, None, 0, P, 1 << 20, 1 << 12, 64, 1, 128, None) == -1
+    assert L.hyena_li_fwd(g, g, g, P, None, 1, P, None, None, 1 << 20, 1 << 12, 64, 1, 16, None) == -1
+
+
+def test_launch_override_names():
+    from vortex_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built in this tree")
+    L = _lib.lib()
+    for n in (b"mr_nseg", b"cl_nseg", b"li_nseg", b"se_nt", b"mr_nt", b"li_nt", b"cl_nt", b"li_cpw", b"li_coop"):
+        assert L.hyena_set_launch_override(n, 1) == 0 and L.hyena_set_launch_override(n, -1) == 0
+    assert L.hyena_set_launch_override(b"HYENA_MR_NSEG", 1) == -1
+    assert L.hyena_set_launch_override(None, 1) == -1

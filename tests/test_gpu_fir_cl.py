@@ -26,13 +26,9 @@ def cl(t):
 @pytest.fixture
 def segments(request):
     """Forces a number of segments along L so that short sequences exercise the halo rebuild."""
-    old = os.environ.get("HYENA_CL_NSEG")
-    os.environ["HYENA_CL_NSEG"] = str(request.param)
-    yield request.param
-    if old is None:
-        del os.environ["HYENA_CL_NSEG"]
-    else:
-        os.environ["HYENA_CL_NSEG"] = old
+    from vortex_amd._lib import launch_override
+    with launch_override(cl_nseg=request.param):
+        yield request.param
 
 
 @pytest.mark.parametrize("segments", [1, 3], indirect=True)
@@ -162,11 +158,9 @@ def test_cl_impulse_response_across_steps_and_segments():
     for p in pos:
         x1[:, p] = 1
     one = torch.ones(B, L, D, dtype=torch.bfloat16)
-    os.environ["HYENA_CL_NSEG"] = "4"
-    try:
+    from vortex_amd._lib import launch_override
+    with launch_override(cl_nseg=4):
         out = ops.fir_cl_fwd(x1.to(DEV), one.to(DEV), one.to(DEV), h.reshape(G, K).to(DEV)).cpu().float()
-    finally:
-        del os.environ["HYENA_CL_NSEG"]
     hw = h.repeat_interleave(D // G, 0)[:, 0]            # [D, K]
     exp = torch.zeros(B, L, D)
     for p in pos:
@@ -235,7 +229,7 @@ def test_layer_projection_beyond_32_bit_offsets():
 
 
 @pytest.mark.parametrize("K", [7, 128])
-def test_cl_nontemporal_variants_match(K, monkeypatch):
+def test_cl_nontemporal_variants_match(K, override):
     # tensors larger than the last-level cache use non-temporal accesses (another instantiation of the kernel):
     # forced on at a small size, it must give the same bits, for the gated form and the fused layer
     B, L, D, G, Ks = 2, 1000, 128, 8, 3
@@ -247,7 +241,7 @@ def test_cl_nontemporal_variants_match(K, monkeypatch):
     cmap = ops.gate_channel_map(D, interleave=True)
     res = {}
     for nt in ("0", "1"):
-        monkeypatch.setenv("HYENA_CL_NT", nt)
+        override(cl_nt=int(nt))
         res[nt] = (ops.fir_cl_fwd(x1, x2, v, h, taps_reversed=K < 128),
                    ops.fir_layer_fwd(u, wf, None, cmap, h, taps_reversed=K < 128))
     assert torch.equal(res["0"][0], res["1"][0]) and torch.equal(res["0"][1], res["1"][1])

@@ -171,7 +171,7 @@ def test_million_token_rows():
 
 @pytest.mark.parametrize("L", [65536 + 520, 2048 * 5 + 8, 2048 * 3, 1544, 8])
 @pytest.mark.parametrize("cplx", [True, False])
-def test_li_cooperative_form(L, cplx, monkeypatch):
+def test_li_cooperative_form(L, cplx, override):
     # rows of 65536 samples and more in shared-filter groups run with the four wavefronts of a block on consecutive
     # pieces of the same channels and the modal state handed across through LDS.  Forced on here for short and ragged
     # rows too (last steps with idle wavefronts, the final state in any of the four pieces): against the oracle,
@@ -183,7 +183,7 @@ def test_li_cooperative_form(L, cplx, monkeypatch):
     ref, y32_ref, st_ref = O.li_prefill(x2, x1, v, lp, r, Db)
     res = {}
     for coop in ("1", "0"):
-        monkeypatch.setenv("HYENA_LI_COOP", coop)
+        override(li_coop=int(coop))
         res[coop] = va.hyena_li_fwd(x1.cuda(), x2.cuda(), v.cuda(), lp.cuda(), r.cuda(), Db.cuda(),
                                     want_state=True, want_fp32=True)
         out, y32, st = res[coop]
@@ -191,6 +191,58 @@ def test_li_cooperative_form(L, cplx, monkeypatch):
         assert rel_err(out, ref) <= 2e-2, coop
         assert rel_err(torch.view_as_real(st) if cplx else st, torch.view_as_real(st_ref) if cplx else st_ref) <= 1e-4, coop
     assert rel_err(res["1"][1], res["0"][1]) <= 1e-5          # the same sums, grouped differently across the state hand-off
-    monkeypatch.setenv("HYENA_LI_COOP", "1")
+    override(li_coop=1)
     out_nt, _, _ = va.hyena_li_fwd(x1.cuda(), x2.cuda(), v.cuda(), lp.cuda(), r.cuda(), Db.cuda())   # the bf16-only variant
     assert torch.equal(out_nt, res["1"][0])
+
+
+def _fast_modal(G, S, cplx, seed, pmin=0.05, pmax=0.9):
+    """Poles with log-uniform |p| in [pmin, pmax]: the fast-decaying range a trained or randn-initialised
+    log_poles parameter (vortex/model/model.py:202) also covers."""
+    g = torch.Generator().manual_seed(seed)
+    import math
+    lm = math.log(pmin) + (math.log(pmax) - math.log(pmin)) * torch.rand(G, S, generator=g, dtype=torch.float64)
+    if cplx:
+        ang = math.pi * torch.rand(G, S, generator=g, dtype=torch.float64)
+        lp = torch.complex(lm, ang).to(torch.complex64)[..., None]
+        r = (torch.complex(torch.randn(G, S, generator=g), torch.randn(G, S, generator=g)) / 2 ** 0.5).to(torch.complex64)
+    else:
+        lp, r = lm.to(torch.float32)[..., None], torch.randn(G, S, generator=g)
+    return lp, r
+
+
+@pytest.mark.parametrize("form", ["lone", "coop", "cpw1"])
+@pytest.mark.parametrize("cplx", [True, False])
+@pytest.mark.parametrize("tail", [8, 64, 120, 0])
+def test_li_state_with_fast_poles_and_ragged_length(tail, cplx, form, override):
+    # L % 128 = 128 - tail: the last chunk is mostly padding.  The emitted state must stay finite and match
+    # the closed form sum_j p^(L-1-j) u_j (float64) for poles whose 120th power underflows float32, on the
+    # one-wavefront, cooperative and one-channel-per-wavefront forms; one decode step then continues from it.
+    B, G, S = 2, 2, 16
+    D = 16 if form != "cpw1" else 8
+    L = 2048 + 512 + (128 - tail) % 128 + (0 if tail else 128)
+    if form == "coop":
+        override(li_coop=1)
+    elif form == "lone":
+        override(li_coop=0)
+    else:
+        override(li_cpw=1)
+    x2, x1, v = O.make_gates(B, D, L + 1, seed=tail + 1)
+    lp, r = _fast_modal(G, S, cplx, seed=40 + tail)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(1)).bfloat16()
+    c = lambda t: t[..., :L].contiguous()
+    ref, y32_ref, _ = O.li_prefill(c(x2), c(x1), c(v), lp, r, Db)
+    out, y32, st = va.hyena_li_fwd(c(x1).cuda(), c(x2).cuda(), c(v).cuda(), lp.cuda(), r.cuda(), Db.cuda(),
+                                   want_state=True, want_fp32=True)
+    assert torch.isfinite(torch.view_as_real(st) if cplx else st).all()
+    st64 = O.modal_state_closed_form(c(x1) * c(v), lp)
+    got = torch.view_as_real(st.cpu()) if cplx else st.cpu()
+    exp = torch.view_as_real(st64) if cplx else st64
+    assert rel_err(got, exp) <= 1e-4, (tail, cplx, form)
+    assert rel_err(y32, y32_ref) <= 1e-4
+    assert rel_err(out, ref) <= 2e-2
+    # one decode token from that state equals position L of a longer prefill
+    full, _, _ = O.li_prefill(x2, x1, v, lp, r, Db, want_state=False)
+    y = va.iir_step(x1[..., L].contiguous().cuda(), x2[..., L].contiguous().cuda(), v[..., L].contiguous().cuda(),
+                    st, torch.exp(lp[..., 0]).cuda(), r.cuda(), Db.cuda())
+    assert rel_err(y, full[..., L]) <= 2e-2

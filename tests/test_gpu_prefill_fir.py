@@ -172,19 +172,19 @@ def test_mr_any_group_size(B, D, G, L, K):
     assert rel_err(out, ref) <= TOL
 
 
-def test_se_nontemporal_variant_matches(monkeypatch):
+def test_se_nontemporal_variant_matches(override):
     # large activations take the non-temporal (streaming) code path; force it on a small case
     B, D, L, G, K = 2, 64, 2048, 4, 7
     x2, x1, v = O.make_gates(B, D, L, seed=13)
     h = O.make_se_filter(G, K)
     a = va.hyena_se_fwd(x1.cuda(), x2.cuda(), v.cuda(), h.cuda())
-    monkeypatch.setenv("HYENA_SE_NT", "1")
+    override(se_nt=1)
     b = va.hyena_se_fwd(x1.cuda(), x2.cuda(), v.cuda(), h.cuda())
     assert torch.equal(a, b)
-    monkeypatch.setenv("HYENA_MR_NT", "1")
+    override(mr_nt=1)
     hm = O.make_mr_filter(G, 128)
     c = va.hyena_mr_fwd(x1.cuda(), x2.cuda(), v.cuda(), hm.cuda())
-    monkeypatch.setenv("HYENA_MR_NT", "0")
+    override(mr_nt=0)
     d = va.hyena_mr_fwd(x1.cuda(), x2.cuda(), v.cuda(), hm.cuda())
     assert torch.equal(c, d)
 

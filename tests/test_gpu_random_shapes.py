@@ -59,9 +59,9 @@ def test_mr_random(B, L, seed):
 
 @pytest.mark.parametrize("coop", ["0", "1"])
 @pytest.mark.parametrize("B,L,seed", cases(3, 10))
-def test_li_random(B, L, seed, coop, monkeypatch):
+def test_li_random(B, L, seed, coop, override):
     # coop = "1" forces the cooperative form (four wavefronts per set of channels) wherever groups have four channels
-    monkeypatch.setenv("HYENA_LI_COOP", coop)
+    override(li_coop=int(coop))
     rng = random.Random(seed)
     cplx = rng.random() < 0.5
     S = rng.choice([16, 16, 8, 3])
@@ -105,14 +105,14 @@ def cl_cases(seed, n):
 
 
 @pytest.mark.parametrize("B,L,seed", cl_cases(7, 14))
-def test_channel_last_fir_random(B, L, seed, monkeypatch):
+def test_channel_last_fir_random(B, L, seed, override):
     # channel-last kernel: any L (rows are independent), channel counts that leave partial 64-channel blocks,
     # every filter length class, forced segment counts
     rng = random.Random(seed)
     K = rng.choice([1, 2, 7, 16, 17, 18, 33, 64, 97, 98, 99, 127, 128])
     G = rng.randint(1, 5)
     D = G * 16 * rng.randint(1, 3)
-    monkeypatch.setenv("HYENA_CL_NSEG", str(rng.randint(1, 5)))
+    override(cl_nseg=rng.randint(1, 5))
     x2, x1, v = O.make_gates(B, D, L, seed=seed)
     h = O.make_mr_filter(G, K, seed=seed + 1)
     Db = torch.randn(D, generator=torch.Generator().manual_seed(seed))
@@ -129,7 +129,7 @@ def test_channel_last_fir_random(B, L, seed, monkeypatch):
 
 
 @pytest.mark.parametrize("B,L,seed", cl_cases(8, 12))
-def test_fused_layer_random(B, L, seed, monkeypatch):
+def test_fused_layer_random(B, L, seed, override):
     rng = random.Random(seed)
     K = rng.choice([2, 4, 7, 17, 18, 64, 128])
     Ks = rng.choice([3, 4])
@@ -139,7 +139,7 @@ def test_fused_layer_random(B, L, seed, monkeypatch):
     cs, il = rng.choice([(False, False), (True, False), (False, True)])
     flip, sbias = rng.random() < 0.5, rng.random() < 0.5
     L = max(L, K)
-    monkeypatch.setenv("HYENA_CL_NSEG", str(rng.randint(1, 4)))
+    override(cl_nseg=rng.randint(1, 4))
     g = torch.Generator().manual_seed(seed)
     C = 3 * D
     u = torch.randn(B, L, C, generator=g).bfloat16()

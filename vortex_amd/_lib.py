@@ -13,7 +13,7 @@ HYENA_BIAS_NONE, HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32 = 0, 1, 2
 
 EXPORTS = [
     "hyena_version", "hyena_last_error_string", "hyena_se_fwd", "hyena_mr_fwd",
-    "hyena_fir_step", "hyena_iir_step", "hyena_li_plan_bytes", "hyena_li_plan", "hyena_li_fwd", "hyena_featurizer_fwd", "hyena_copy_probe",
+    "hyena_fir_step", "hyena_iir_step", "hyena_li_plan_bytes", "hyena_li_plan", "hyena_li_fwd", "hyena_featurizer_fwd", "hyena_set_launch_override",
     "hyena_fir_layer_step", "hyena_iir_layer_step", "hyena_fir_cl_fwd", "hyena_fir_layer_fwd",
     "hyena_fir_step_dpos", "hyena_fir_layer_step_dpos", "hyena_ring_advance",
 ]
@@ -73,7 +73,7 @@ def lib():
                                c_int64, c_int64, c_int64, c_void_p]
     L.hyena_featurizer_fwd.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int64,
                                        c_int64, c_int64, c_int64, c_int, c_int, c_void_p]
-    L.hyena_copy_probe.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
+    L.hyena_set_launch_override.argtypes = [c_char_p, c_int64]
     P = POINTER(ProjStep)
     L.hyena_fir_layer_step.argtypes = [P, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int64,
                                        c_int64, c_int64, c_int64, c_void_p]
@@ -95,6 +95,43 @@ def lib():
             fn.restype = c_int64 if name == "hyena_li_plan_bytes" else c_int
     _lib = L
     return L
+
+
+class launch_override:
+    """Context manager pinning one launch-shape choice of the library (hyena_set_launch_override) for its body.
+
+    Tests use it to force the multi-segment, non-temporal or cooperative code paths on small inputs."""
+
+    def __init__(self, **kv):
+        self.kv = kv
+
+    def __enter__(self):
+        for k, v in self.kv.items():
+            check(lib().hyena_set_launch_override(k.encode(), int(v)), "hyena_set_launch_override")
+        return self
+
+    def __exit__(self, *exc):
+        for k in self.kv:
+            lib().hyena_set_launch_override(k.encode(), -1)
+        return False
+
+
+_probe = None
+PROBE_PATH = os.path.join(_HERE, "libhyena_probe.so")
+
+
+def copy_probe():
+    """hyena_copy_probe(src, dst, nbytes, stream) of libhyena_probe.so: a plain 16-bytes-per-lane device copy, the
+    calibration launch for traffic counters and the bandwidth yardstick of the benchmark (not an operator)."""
+    global _probe
+    if _probe is None:
+        if not os.path.exists(PROBE_PATH):
+            raise RuntimeError(f"{PROBE_PATH} is not built; run `python -m vortex_amd.build`")
+        P = ctypes.CDLL(PROBE_PATH)
+        P.hyena_copy_probe.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
+        P.hyena_copy_probe.restype = c_int
+        _probe = P.hyena_copy_probe
+    return _probe
 
 
 def check(rc, what):

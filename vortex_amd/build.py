@@ -10,6 +10,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libhyena_mi355x.so")
+PROBE = os.path.join(HERE, "libhyena_probe.so")          # copy kernel for counter calibration; not part of the ABI
 SELFTEST = os.path.join(HERE, "abi_selftest")          # plain C++ program that exercises the C ABI without torch
 SOURCES = ["api.hip", "se_fir.hip", "mr_fir.hip", "li_modal.hip", "decode.hip", "featurizer.hip", "fir_cl.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -43,6 +44,7 @@ def build(verbose=True, jobs=4):
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(compile_one, srcs))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+    _run([HIPCC] + FLAGS + ["-shared", os.path.join(CSRC, "copy_probe.hip"), "-o", PROBE])
     _run([HIPCC, "-O2", "-std=c++17", os.path.join(CSRC, "abi_selftest.cpp"), "-o", SELFTEST, "-ldl"])
     if verbose:
         print("built", LIB)

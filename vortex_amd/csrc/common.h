@@ -56,10 +56,15 @@ static inline RowMap make_rowmap(const hyena_rows* r) {
 int hyena_fail(int code, const char* fmt, ...);
 int hyena_check_launch(const char* what);
 
+// launch-shape overrides set through hyena_set_launch_override (api.hip); -1 = the launcher's own choice
+enum { HYENA_OV_MR_NSEG, HYENA_OV_CL_NSEG, HYENA_OV_SE_NT, HYENA_OV_MR_NT, HYENA_OV_LI_NT, HYENA_OV_CL_NT,
+       HYENA_OV_LI_CPW, HYENA_OV_LI_COOP, HYENA_OV_LI_NSEG, HYENA_OV_COUNT };
+int64_t hyena_override(int id);
+
 static inline bool rows_aligned8(const hyena_rows* r) {
     return r == nullptr || ((((uintptr_t)r->ptr) & 15) == 0 && r->batch_stride % 8 == 0 && r->row_stride % 8 == 0);
 }
 static inline bool rows_valid(const hyena_rows* r) {
-    return r == nullptr || (r->ptr != nullptr && r->ch_inner > 0 && r->ch_inner < (1LL << 31) && r->ch_outer >= 0 &&
+    return r == nullptr || r->ptr == nullptr || (r->ch_inner > 0 && r->ch_inner < (1LL << 31) && r->ch_outer >= 0 &&
                             r->ch_outer < (1LL << 31));
 }

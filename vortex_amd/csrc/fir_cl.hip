@@ -451,7 +451,7 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
             if (score > best + 1e-9) { best = score; nseg = c; }
         }
     }
-    if (const char* e = getenv("HYENA_CL_NSEG")) { int64_t x = atoll(e); if (x >= 1) nseg = x; }
+    { const int64_t x = hyena_override(HYENA_OV_CL_NSEG); if (x >= 1) nseg = x; }
     int64_t seg_len = (L + nseg - 1) / nseg;
     seg_len = (seg_len + TL - 1) / TL * TL;
     nseg = (L + seg_len - 1) / seg_len;
@@ -463,7 +463,7 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     const int dg = (int)(D / G);
     // tensors larger than the last-level cache stream through it: non-temporal accesses then
     bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
-    if (const char* e = getenv("HYENA_CL_NT")) nt = atoi(e) != 0;
+    { const int64_t x = hyena_override(HYENA_OV_CL_NT); if (x >= 0) nt = x != 0; }
     bool ok = false;
 #define CL_GO(P, Q, M, F, KSV, AX, ML, N)                                                                         \
     hipLaunchKernelGGL((fir_cl_kernel<P, Q, M, F, KSV, AX, ML, N>), grid, dim3(256), 0, s, a.x1, a.x2, a.v, a.pj, h, \

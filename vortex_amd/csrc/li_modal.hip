@@ -53,9 +53,9 @@ constexpr int WS_HEAD = WS_ZPAD;                   // [128]        filter head h
 constexpr int WS_P16 = WS_HEAD + C;                // [16][9][2]   p^(16a), a = 0..8  (a = 8: the chunk factor p^128)
 constexpr int WS_P1 = WS_P16 + S * 9 * 2;          // [16][16][2]  p^b
 constexpr int WS_R1 = WS_P1 + S * 16 * 2;          // [16][16][2]  r * p^b
-constexpr int WS_PINV = WS_R1 + S * 16 * 2;        // [16][2]      1/p
-constexpr int WS_GROUP = 1536;                     // 1504 used; 6 KB, a whole number of 16-byte lane loads
-static_assert(WS_PINV + 2 * S <= WS_GROUP, "workspace layout");
+constexpr int WS_END = WS_R1 + S * 16 * 2;
+constexpr int WS_GROUP = 1536;                     // 1472 used; 6 KB, a whole number of 16-byte lane loads
+static_assert(WS_END <= WS_GROUP, "workspace layout");
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) {
     union { u32x4 u; bf16x8 b; } c;
@@ -138,13 +138,7 @@ __global__ __launch_bounds__(256) void li_plan_kernel(const float* __restrict__ 
         w[WS_R1 + 2 * tid] = (float)(rr * re - ri * im);
         w[WS_R1 + 2 * tid + 1] = (float)(rr * im + ri * re);
     }
-    if (tid < S) {
-        double re, im;
-        ppow(tid, -1, re, im);
-        w[WS_PINV + 2 * tid] = (float)re;
-        w[WS_PINV + 2 * tid + 1] = (float)im;
-    }
-    for (int e = WS_PINV + 2 * S + tid; e < WS_GROUP; e += 256) w[e] = 0.f;
+    for (int e = WS_END + tid; e < WS_GROUP; e += 256) w[e] = 0.f;
 }
 
 // (hi, lo) bf16 split of eight fp32 coefficients into two A-operand fragments
@@ -196,9 +190,15 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     const int64_t d0 = (int64_t)((uint32_t)quad % qpb) * CPW;
     const int g = (int)((uint32_t)d0 / (uint32_t)a.dg);
     const float* ws = a.ws + (size_t)g * WS_GROUP;
+    // The kernel walks a virtual row of Lv = L + pad samples, a whole number of chunks, whose first pad samples
+    // are zeros ahead of the real row: zero history in front of a causal filter changes no output, and the last
+    // chunk then ends exactly on sample L-1, so the scan's state after it is the decode state as it stands.
     const int64_t L = a.L;
+    const int pad = (int)((C - L % C) % C);                    // multiple of 8 (L is), < 128
+    const int64_t Lv = L + pad;
     const int64_t woff = COOP ? (int64_t)w * TLW : 0;          // this wavefront's piece inside a step
-    const int64_t Lw = L - woff;                               // the row as this wavefront sees it (may be <= 0)
+    const int64_t Lw = Lv - woff;                              // the virtual row as this wavefront sees it (may be <= 0)
+    const int64_t lo = pad - woff;                             // positions below lo (first wavefront, first chunk) are padding
 
     unsigned char* lds = lds_all + w * WAVE_LDS_BYTES;
     bf16_t* u_w = (bf16_t*)lds;                                // [4][URS]
@@ -226,10 +226,11 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int64_t d = d0 + (CPW == 4 ? r : 0);
-        p1[r] = a.x1.row(b, d) + woff + roff(r) + lane * 8;
-        pv[r] = PRE ? a.v.row(b, d) + woff + roff(r) + lane * 8 : nullptr;
-        p2[r] = POST ? a.x2.row(b, d) + woff + roff(r) + lane * 8 : nullptr;
-        po[r] = a.out + (b * a.D + d) * L + woff + roff(r) + lane * 8;
+        const int64_t o = woff + roff(r) + lane * 8 - pad;     // pointers are in virtual positions; never used below lo
+        p1[r] = a.x1.row(b, d) + o;
+        pv[r] = PRE ? a.v.row(b, d) + o : nullptr;
+        p2[r] = POST ? a.x2.row(b, d) + o : nullptr;
+        po[r] = a.out + (b * a.D + d) * L + o;
     }
     const u32x4 zero4 = {0, 0, 0, 0};
     u32x4 c1[PF][4], cv[PF][4], c2[PF][4];
@@ -239,7 +240,8 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int64_t t = (int64_t)p * STEP;
-                const bool ok = t + roff(r) + lane * 8 < Lw;
+                const int64_t pos = t + roff(r) + lane * 8;
+                const bool ok = pos < Lw && pos >= lo;
                 c1[p][r] = ok ? ld16<NT>(p1[r] + t) : zero4;
                 cv[p][r] = (PRE && ok) ? ld16<NT>(pv[r] + t) : zero4;
                 c2[p][r] = (POST && ok) ? ld16<NT>(p2[r] + t) : zero4;
@@ -257,7 +259,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     // table for the block, build a quarter of the fragments each and read the rest from LDS.
     // 16x16x32 A operand: lane holds row m = lane & 15, k = 8*(lane >> 4) + e, e = 0..7.
     bf16x8 Th[8], Tl[8], Poh[8], Pol[8], Pih[8], Pil[8];
-    float pcr, pci, pinv_r, pinv_i;                            // p^128 and 1/p of this lane's pole (lane & 15)
+    float pcr, pci;                                            // p^128 of this lane's pole (lane & 15)
     {
         float* tb = COOP ? (float*)lds_all : (float*)lds;
         u32x4* fb = (u32x4*)(lds_all + WS_GROUP * 4);           // COOP: [48 fragments][64 lanes]
@@ -272,8 +274,6 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
         const int m = lane & 15, qa = lane >> 4;
         pcr = tb[WS_P16 + 2 * (9 * m + 8)];
         pci = tb[WS_P16 + 2 * (9 * m + 8) + 1];
-        pinv_r = tb[WS_PINV + 2 * m];
-        pinv_i = tb[WS_PINV + 2 * m + 1];
         const float2* t16 = (const float2*)(tb + WS_P16);
         const float2* t1 = (const float2*)(tb + WS_P1);
         const float2* tr = (const float2*)(tb + WS_R1);
@@ -465,7 +465,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                         o[r][j] = pack_bf2(bf_lo(zz[r][j]) * bf_lo(c2[pp][r][j]), bf_hi(zz[r][j]) * bf_hi(c2[pp][r][j]));
                 }
             }
-            if (ts_out >= 0 && t_refill + TLW <= Lw) {             // wave-uniform: store and refill whole pieces
+            if (ts_out >= 0 && (ts_out > 0 || lo <= 0) && t_refill + TLW <= Lw) {   // wave-uniform: store and refill whole pieces
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     st16<NT>(po[r] + ts_out, o[r]);
@@ -474,7 +474,8 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const bool okc = ts_out >= 0 && ts_out + roff(r) + lane * 8 < Lw;
+                    const int64_t pos = ts_out + roff(r) + lane * 8;
+                    const bool okc = ts_out >= 0 && pos < Lw && pos >= lo;
                     const bool okr = ts_out >= 0 && t_refill + roff(r) + lane * 8 < Lw;
                     if (okc) st16<NT>(po[r] + ts_out, o[r]);
                     if (ts_out >= 0) c2[pp][r] = (POST && okr) ? ld16<NT>(p2[r] + t_refill) : zero4;
@@ -565,8 +566,8 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
             const int tl = 32 * Sg + 8 * q;                     // inside the chunk
             if (Y32) {
                 const int64_t t0 = ts + roff(c) + C * s + tl;
-                if (t0 < Lw) {
-                    float* yp = a.y32 + (b * a.D + d0 + (CPW == 4 ? c : 0)) * L + woff + t0;
+                if (t0 < Lw && t0 >= lo) {
+                    float* yp = a.y32 + (b * a.D + d0 + (CPW == 4 ? c : 0)) * L + woff + t0 - pad;
                     *(f32x4*)yp = acc[Sg][0];
                     *(f32x4*)(yp + 4) = acc[Sg][1];
                 }
@@ -596,19 +597,20 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     };
 
     const std::integral_constant<bool, true> guarded;
-    // the bounds are the block's (L, not Lw): with COOP every wavefront runs every step and meets every barrier
-    for (int64_t ts = 0; ts < L; ts += (int64_t)PF * STEP) {
+    // the bounds are the block's (Lv, not Lw): with COOP every wavefront runs every step and meets every barrier
+    for (int64_t ts = 0; ts < Lv; ts += (int64_t)PF * STEP) {
 #pragma unroll
         for (int p = 0; p < PF; ++p)
-            if (ts + (int64_t)p * STEP < L) step(guarded, p, ts + (int64_t)p * STEP);
+            if (ts + (int64_t)p * STEP < Lv) step(guarded, p, ts + (int64_t)p * STEP);
     }
     {   // output of the last step
-        const int64_t ts_last = ((L + STEP - 1) / STEP - 1) * STEP;
+        const int64_t ts_last = ((Lv + STEP - 1) / STEP - 1) * STEP;
         wave_sync();
         const int pl = (int)((ts_last / STEP) % PF);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const bool okc = ts_last + roff(r) + lane * 8 < Lw;
+            const int64_t pos = ts_last + roff(r) + lane * 8;
+            const bool okc = pos < Lw && pos >= lo;
             const u32x4 zz = *(const u32x4*)(z_w + r * URS + lofs);
             u32x4 x2v = c2[0][r];
 #pragma unroll
@@ -625,21 +627,11 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     }
 
     if (a.state_out && have_final) {
-        // the captured chunk ends (-L) % 128 samples past L with zero inputs: undo that, X *= p^-pad
-        int pad = (int)((C - L % C) % C);
-        float qr = pinv_r, qi = pinv_i;
-        float fr_ = 1.f, fi = 0.f;
-        while (pad) {
-            if (pad & 1) { const float t = fr_ * qr - fi * qi; fi = fr_ * qi + fi * qr; fr_ = t; }
-            const float t = qr * qr - qi * qi; qi = 2.f * qr * qi; qr = t;
-            pad >>= 1;
-        }
-        Xr = Xfr;
-        Xi = Xfi;
+        // the last chunk of the virtual row ends on sample L-1: the scan's state after it is the decode state
         if ((CPW == 4 || lane < 16) && sp < a.sr) {
             float* sp_ = a.state_out + ((b * a.D + d0 + sc) * a.sr + sp) * 2;
-            sp_[0] = Xr * fr_ - Xi * fi;
-            sp_[1] = Xr * fi + Xi * fr_;
+            sp_[0] = Xfr;
+            sp_[1] = Xfi;
         }
     }
 }
@@ -675,16 +667,19 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
         (((uintptr_t)y_conv_fp32) & 15) || (((uintptr_t)workspace) & 15))
         return hyena_fail(HYENA_EALIGN, "hyena_li_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
     if (d_is_bf16 < 0 || d_is_bf16 > 2) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: d_is_bf16 must be 0, 1 or 2");
+    // the kernel does the channel arithmetic in 32 bits: reject maps and sizes that would wrap or divide by zero
+    if (!rows_valid(x1) || !rows_valid(x2) || !rows_valid(v) || B * D >= (1LL << 31) || L >= (1LL << 40))
+        return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: B*D and the channel map must fit 31 bits");
     if (B == 0 || L == 0) return 0;
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
     int cpw = ((D / G) % 4 == 0) ? 4 : 1;                    // channels per wavefront (they share one filter)
-    if (const char* e = getenv("HYENA_LI_CPW")) { if (atoi(e) == 1) cpw = 1; }
+    if (hyena_override(HYENA_OV_LI_CPW) == 1) cpw = 1;
     const int64_t nquads = B * (D / cpw);
     // Long rows of shared-filter channels go to the cooperative form (one block per work item): measured 6 %, 14 %
     // and 2 % faster at L = 65536, 131072 and 262144, slower below (the block's waves start and end together).
     // One channel per wavefront gains nothing from it: there the per-step scan, not the row pattern, sets the pace.
     bool coop = cpw == 4 && L >= 65536;
-    if (const char* e = getenv("HYENA_LI_COOP")) coop = cpw == 4 && atoi(e) != 0;
+    { const int64_t x = hyena_override(HYENA_OV_LI_COOP); if (x >= 0) coop = cpw == 4 && x != 0; }
     const int64_t nblk = coop ? nquads : (nquads + 3) / 4;
     if (nquads > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: problem too large for one launch");
     LiArgs a;
@@ -705,7 +700,7 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)nblk);
     bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
-    if (const char* e = getenv("HYENA_LI_NT")) nt = atoi(e) != 0;
+    { const int64_t x = hyena_override(HYENA_OV_LI_NT); if (x >= 0) nt = x != 0; }
     // DMODE and Y32 are compile-time so that the hot loop carries no uniform branches.  The fp32
     // side output is a verification path: it always uses cached accesses.
     const int dmode = d_is_bf16;

@@ -243,6 +243,9 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
         return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: bias_mode %d needs a bias pointer", bias_mode);
     if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15))
         return hyena_fail(HYENA_EALIGN, "hyena_mr_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
+    // the kernels do the channel arithmetic in 32 bits: reject maps and sizes that would wrap or divide by zero
+    if (!rows_valid(x1) || !rows_valid(x2) || !rows_valid(v) || B * D >= (1LL << 31) || L / 8 >= (1LL << 31))
+        return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: B*D, L/8 and the channel map must fit 31 bits");
     if (B == 0 || L == 0) return 0;
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
 
@@ -264,7 +267,7 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
             if (sl >= L) break;
         }
     }
-    if (const char* e = getenv("HYENA_MR_NSEG")) { int64_t x = atoll(e); if (x >= 1) nseg = x; }
+    { const int64_t x = hyena_override(HYENA_OV_MR_NSEG); if (x >= 1) nseg = x; }
     int64_t seg_len = (L + nseg - 1) / nseg;
     seg_len = (seg_len + TL - 1) / TL * TL;
     nseg = (L + seg_len - 1) / seg_len;
@@ -278,7 +281,7 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     bool ok = false;
     // activations larger than the last-level cache stream through it: use non-temporal accesses then
     bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
-    if (const char* e = getenv("HYENA_MR_NT")) nt = atoi(e) != 0;
+    { const int64_t x = hyena_override(HYENA_OV_MR_NT); if (x >= 0) nt = x != 0; }
     const bool full = K > 98;
 #define MR_LAUNCH(P, Q, M, N, F)                                                                              \
     hipLaunchKernelGGL((mr_fir_kernel<P, Q, M, N, F>), grid, dim3(256), 0, s, m1, m2, mv, h, K, taps_reversed, \

@@ -181,7 +181,7 @@ extern "C" int hyena_se_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     const bool rowu = (opr % 256 == 0) && D <= 65535 && B <= 65535;
     // activations larger than the last-level cache stream through it: non-temporal accesses then
     bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
-    if (const char* e = getenv("HYENA_SE_NT")) nt = atoi(e) != 0;
+    { const int64_t x = hyena_override(HYENA_OV_SE_NT); if (x >= 0) nt = x != 0; }
     const int64_t nblk = (tot + 255) / 256;
     if (nblk > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "hyena_se_fwd: problem too large for one launch");
     dim3 grid((unsigned)nblk);
