@@ -137,6 +137,19 @@ int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v
                  void* out, float* y_conv_fp32, float* state_out,
                  int64_t B, int64_t D, int64_t L, int64_t G, int64_t S, void* stream);
 
+/* hyena_li_plan + hyena_li_fwd in a form that allocates nothing and takes no workspace.  No counterpart in the
+ * reference: it is for callers that cannot allocate device memory or keep a workspace alive -- code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The coefficient tables go into a static device
+ * array inside the library (6 KB per filter group; at most 4096 groups = 24 MiB, which each GPU the library runs
+ * on holds until the process ends); more groups are refused with HYENA_ENOSUP.  The tables are rebuilt from
+ * log_poles / residues ([G][S][2] float32) on every call, on `stream`, ahead of the main launch.  Same arguments,
+ * arithmetic and results as hyena_li_fwd otherwise.  Every call on a GPU shares that GPU's array: calls that
+ * overlap on one GPU (different streams, or threads) race; calls on one stream are ordered and safe. */
+int hyena_li_fwd_static(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v,
+                        const float* log_poles, const float* residues, const float* Dcoef, int d_is_bf16,
+                        void* out, float* y_conv_fp32, float* state_out,
+                        int64_t B, int64_t D, int64_t L, int64_t G, int64_t S, void* stream);
+
 /* Decode FIR step on a ring-buffer cache.  Replaces HyenaInferenceEngine.step_fir
  * (vortex/model/engine.py:406-449; native precedent vortex/ops/conv/csrc/step_fir.cu:13-109)
  * fused with the caller's gates (vortex/model/model.py:352, :359):

@@ -23,6 +23,7 @@
 // block barrier anywhere, only the in-order LDS pipe of the wavefront itself, and the four
 // wavefronts of a CU drift apart and cover each other's memory latency.  Global traffic is
 // coalesced 16 B per lane (1 KiB per row and instruction), prefetched PF steps ahead in registers.
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
@@ -654,24 +655,97 @@ extern "C" int hyena_li_plan(const float* log_poles, const float* residues, int6
     return hyena_check_launch("hyena_li_plan");
 }
 
+namespace {
+int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const void* workspace,
+                const float* Dcoef, int d_is_bf16, void* out, float* y_conv_fp32, float* state_out,
+                int64_t B, int64_t D, int64_t L, int64_t G, int64_t S_, void* stream, bool check_only);
+}
+
 extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const void* workspace,
                             const float* Dcoef, int d_is_bf16, void* out, float* y_conv_fp32, float* state_out,
                             int64_t B, int64_t D, int64_t L, int64_t G, int64_t S_, void* stream) {
+    return li_fwd_impl("hyena_li_fwd", x1, x2, v, workspace, Dcoef, d_is_bf16, out, y_conv_fp32, state_out, B, D, L, G,
+                       S_, stream, false);
+}
+
+// ------------------------------------------------------------------ the form that allocates nothing
+// The coefficient tables live in a file-scope device array instead of a caller-owned workspace.  Host code
+// must not use the array's name as an address: each device holds its own copy, whose address is looked up
+// once per device (hipGetSymbolAddress with that device current) and kept.
+namespace {
+constexpr int64_t LI_STATIC_MAX_GROUPS = 4096;                 // 24 MiB per device, held until the process ends
+constexpr int LI_STATIC_MAX_DEVICES = 64;
+static __device__ __align__(256) float scratch[LI_STATIC_MAX_GROUPS * WS_GROUP];
+std::mutex g_scratch_mu;
+float* g_scratch_ptr[LI_STATIC_MAX_DEVICES] = {};
+
+int li_scratch_for_current_device(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hyena_fail((int)e, "hyena_li_fwd_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= LI_STATIC_MAX_DEVICES)
+        return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd_static: device index %d (0..%d)", dev, LI_STATIC_MAX_DEVICES - 1);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        float* p = nullptr;
+        e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return hyena_fail(e != hipSuccess ? (int)e : HYENA_EINVAL, "hyena_li_fwd_static: hipGetSymbolAddress: %s",
+                              hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+}  // namespace
+
+extern "C" int hyena_li_fwd_static(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v,
+                                   const float* log_poles, const float* residues, const float* Dcoef, int d_is_bf16,
+                                   void* out, float* y_conv_fp32, float* state_out, int64_t B, int64_t D, int64_t L,
+                                   int64_t G, int64_t S_, void* stream) {
+    if (!log_poles || !residues) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd_static: log_poles and residues are required");
+    if (G <= 0) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd_static: bad G=%lld", (long long)G);
+    if (G > LI_STATIC_MAX_GROUPS)
+        return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd_static: %lld filter groups exceed the static table of %lld; use "
+                          "hyena_li_plan + hyena_li_fwd with a caller-owned workspace", (long long)G,
+                          (long long)LI_STATIC_MAX_GROUPS);
+    if (S_ < 1 || S_ > S) return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd_static: state size %lld (1..16)", (long long)S_);
+    float* ws = nullptr;
+    if (int rc = li_scratch_for_current_device(&ws)) return rc;
+    // every argument check of the main launch runs before anything is enqueued
+    if (int rc = li_fwd_impl("hyena_li_fwd_static", x1, x2, v, ws, Dcoef, d_is_bf16, out, y_conv_fp32, state_out, B, D,
+                             L, G, S_, stream, true))
+        return rc;
+    if (B == 0 || L == 0) return 0;
+    // the plan kernel rewrites the whole table of each of the G groups, so nothing of an earlier call survives in
+    // the part this call reads
+    hipLaunchKernelGGL(li_plan_kernel, dim3((unsigned)G), dim3(256), 0, (hipStream_t)stream, log_poles, residues, ws,
+                       (int)S_);
+    if (int rc = hyena_check_launch("hyena_li_fwd_static (tables)")) return rc;
+    return li_fwd_impl("hyena_li_fwd_static", x1, x2, v, ws, Dcoef, d_is_bf16, out, y_conv_fp32, state_out, B, D, L, G,
+                       S_, stream, false);
+}
+
+namespace {
+int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const void* workspace,
+                const float* Dcoef, int d_is_bf16, void* out, float* y_conv_fp32, float* state_out,
+                int64_t B, int64_t D, int64_t L, int64_t G, int64_t S_, void* stream, bool check_only) {
     if (!x1 || !x1->ptr || !workspace || !out)
-        return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: x1, workspace and out are required");
+        return hyena_fail(HYENA_EINVAL, "%s: x1, workspace and out are required", who);
     if (B < 0 || D <= 0 || L < 0 || G <= 0 || D % G != 0)
-        return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: bad sizes B=%lld D=%lld L=%lld G=%lld", (long long)B,
+        return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld L=%lld G=%lld", who, (long long)B,
                           (long long)D, (long long)L, (long long)G);
-    if (S_ < 1 || S_ > S) return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: state size %lld (1..16)", (long long)S_);
+    if (S_ < 1 || S_ > S) return hyena_fail(HYENA_ENOSUP, "%s: state size %lld (1..16)", who, (long long)S_);
     if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15) ||
         (((uintptr_t)y_conv_fp32) & 15) || (((uintptr_t)workspace) & 15))
-        return hyena_fail(HYENA_EALIGN, "hyena_li_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
-    if (d_is_bf16 < 0 || d_is_bf16 > 2) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: d_is_bf16 must be 0, 1 or 2");
+        return hyena_fail(HYENA_EALIGN, "%s: L and strides must be multiples of 8, pointers 16-byte aligned", who);
+    if (d_is_bf16 < 0 || d_is_bf16 > 2) return hyena_fail(HYENA_EINVAL, "%s: d_is_bf16 must be 0, 1 or 2", who);
     // the kernel does the channel arithmetic in 32 bits: reject maps and sizes that would wrap or divide by zero
     if (!rows_valid(x1) || !rows_valid(x2) || !rows_valid(v) || B * D >= (1LL << 31) || L >= (1LL << 40))
-        return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: B*D and the channel map must fit 31 bits");
-    if (B == 0 || L == 0) return 0;
+        return hyena_fail(HYENA_EINVAL, "%s: B*D and the channel map must fit 31 bits", who);
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
+    if (pre != post) return hyena_fail(HYENA_ENOSUP, "%s: pass both v and x2 or neither", who);
+    if (B == 0 || L == 0) return 0;
     int cpw = ((D / G) % 4 == 0) ? 4 : 1;                    // channels per wavefront (they share one filter)
     if (hyena_override(HYENA_OV_LI_CPW) == 1) cpw = 1;
     const int64_t nquads = B * (D / cpw);
@@ -681,7 +755,8 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     bool coop = cpw == 4 && L >= 65536;
     { const int64_t x = hyena_override(HYENA_OV_LI_COOP); if (x >= 0) coop = cpw == 4 && x != 0; }
     const int64_t nblk = coop ? nquads : (nquads + 3) / 4;
-    if (nquads > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "hyena_li_fwd: problem too large for one launch");
+    if (nquads > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: problem too large for one launch", who);
+    if (check_only) return 0;
     LiArgs a;
     a.x1 = make_rowmap(x1);
     a.x2 = make_rowmap(post ? x2 : nullptr);
@@ -717,10 +792,10 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
 #define LI_M(P, Q, N, Y) do { if (dmode == 1) LI_LAUNCH(P, Q, N, 1, Y); else if (dmode == 2) LI_LAUNCH(P, Q, N, 2, Y); else LI_LAUNCH(P, Q, N, 0, Y); } while (0)
 #define LI_N(P, Q) do { if (y32) LI_M(P, Q, false, true); else if (nt) LI_M(P, Q, true, false); else LI_M(P, Q, false, false); } while (0)
     if (pre && post) LI_N(true, true);
-    else if (!pre && !post) LI_N(false, false);
-    else return hyena_fail(HYENA_ENOSUP, "hyena_li_fwd: pass both v and x2 or neither");
+    else LI_N(false, false);
 #undef LI_N
 #undef LI_M
 #undef LI_LAUNCH
-    return hyena_check_launch("hyena_li_fwd");
+    return hyena_check_launch(who);
 }
+}  // namespace
