@@ -6,36 +6,15 @@ k*x rounded to bf16, fp32 accumulation, the convolution rounded to bf16, then th
 output gate (vortex/model/engine.py:159, :197-208, :232).  Forward only.
 """
 import warnings
-from dataclasses import dataclass
 
 import torch
 
 from vortex_amd import ops
-from vortex_amd._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE
+from vortex_amd._lib import (HYENA_BIAS_ADD, HYENA_BIAS_ADD_FP32, HYENA_BIAS_GATED_BF16, HYENA_BIAS_GATED_FP32,
+                             HYENA_BIAS_NONE)
 
+from .kernel_utils import BwdKernelConfig, FwdKernelConfig  # noqa: F401
 from .utils import correction_toeplitz, toeplitz
-
-
-@dataclass(eq=False)
-class FwdKernelConfig:
-    """Accepted for signature compatibility (vortex/ops/hyena_se/kernel_utils.py:326-335); the HIP
-    kernels have fixed tiles, so every field is ignored."""
-    schedule: str = "default"
-    autotune: bool = False
-    CHUNK_SIZE: int = 128
-    BLOCK_D: int = 32
-    THREADBLOCK_SWIZZLE: str = "row"
-    RETURN_TOEPLITZ: bool = False
-
-
-@dataclass(eq=False)
-class BwdKernelConfig:
-    """vortex/ops/hyena_se/kernel_utils.py:337-343; unused (forward only)."""
-    schedule: str = "default"
-    autotune: bool = False
-    CHUNK_SIZE: int = 128
-    BLOCK_D: int = 32
-    LOAD_TOEPLITZ: bool = False
 
 
 def _to_bdl(t, layout):
@@ -116,29 +95,88 @@ def inner_hyena_se(x, k, q, h, bias=None, input_layout="bdl", output_layout="bdl
     return _from_bdl(y, output_layout, G)
 
 
-inner_hyena_se_ref = inner_hyena_se
+def _fir_per_channel(x, taps, q, k, bias, mode):
+    """out = [q *] bias_rule(corr(taps, [k *] x)) on [B, D, L] bf16 with a tap table [G', K], G' in {1, D} or any
+    divisor of D in the blocked map; the short kernel up to 8 taps, the MFMA kernel above."""
+    B, D, L = x.shape
+    K = taps.shape[1]
+    if K > 128:
+        raise NotImplementedError("filters longer than 128 taps have no FIR kernel")
+    (x, pad), (k, _), (q, _) = ops.front_pad8(x), (ops.front_pad8(k) if k is not None else (None, 0)), \
+        (ops.front_pad8(q) if q is not None else (None, 0))
+    y = ops.fir_fwd_rows(ops.rows_of(x), ops.rows_of(q), ops.rows_of(k), taps, B, D, L + pad, K, device=x.device,
+                         bias=bias, bias_mode=mode, taps_reversed=True, force_mfma=K > 8)
+    return y[..., pad:] if pad else y
+
+
+def _bias_rule(weight_dtype, bias, apply_gated_bias, D):
+    """(bias [D] float32 or None, bias mode) for causal_conv1d_ref semantics (interface.py:228-243): the arithmetic
+    runs in weight.dtype.  float32 weights: conv + bias, or conv + x*bias, formed in float32 and rounded once;
+    bf16 weights: F.conv1d adds its bias before its single rounding, the gated bias is bf16 tensor arithmetic."""
+    if bias is None:
+        return None, HYENA_BIAS_NONE
+    b = ops._f32(bias.reshape(-1))
+    if b.numel() != D:
+        raise ValueError(f"bias must have {D} elements ([D], or [D, 1] for a gated bias)")
+    if not apply_gated_bias:
+        return b, HYENA_BIAS_ADD_FP32
+    return b, (HYENA_BIAS_GATED_BF16 if weight_dtype == torch.bfloat16 else HYENA_BIAS_GATED_FP32)
 
 
 def causal_conv1d_ref(x, weight, bias=None, apply_gated_bias=False, return_final_states=False, final_states_out=None,
                       activation=None, *args, **kwargs):
-    """Depthwise causal FIR without gates (vortex/ops/hyena_se/interface.py:207-244).
+    """Depthwise causal FIR without gates (vortex/ops/hyena_se/interface.py:207-244), any 1 <= K <= 128.
 
-    x [B, D, L] bf16, weight [D, K]; bias added after the bf16 rounding, or `+ x*bias` in fp32
-    when apply_gated_bias.
+    x [B, D, L] bf16, weight [D, K] float32 or bf16 (weight[:, K-1] on the current sample); the result is rounded
+    to bf16 once, after the bias: out = bf16(conv + bias[d]), or with apply_gated_bias bf16(conv + x*bias[d])
+    (bf16 weights: bf16(bf16(conv) + bf16(x*bias[d])), the reference's bf16 tensor arithmetic).  A gated bias is
+    [D, 1] in the reference (it multiplies x by plain broadcasting, interface.py:240); [D] is taken as the same
+    per-channel coefficient here.  Other input dtypes and the silu activation have no kernel.
     """
     if activation is not None:
         raise NotImplementedError("activation is not supported")
+    ops._need_cuda(x, weight)
     B, D, L = x.shape
-    K = weight.shape[-1]
-    mode = HYENA_BIAS_NONE if bias is None else (HYENA_BIAS_GATED_FP32 if apply_gated_bias else HYENA_BIAS_ADD)
-    if mode == HYENA_BIAS_GATED_FP32 or K > 8:
-        raise NotImplementedError("ungated FIR with per-channel taps is limited to K <= 8 without gated bias")
-    xp, pad = ops.front_pad8(x)
-    out = ops.fir_fwd_rows(ops.rows_of(xp), None, None, ops._f32(weight).reshape(D, K), B, D, L + pad, K,
-                           device=x.device, bias=ops._f32(bias), bias_mode=mode, taps_reversed=True)
-    if pad:
-        out = out[..., pad:]
+    if weight.dim() != 2 or weight.shape[0] != D:
+        raise ValueError("weight must be [D, K]")
+    b, mode = _bias_rule(weight.dtype, bias, apply_gated_bias, D)
+    out = _fir_per_channel(x, ops._f32(weight), None, None, b, mode)
     return out if not return_final_states else (out, final_states_out)
+
+
+def inner_hyena_se_ref(x, k, q, h, bias=None, input_layout="bdl", output_layout="bdl", inner_layout="bdl",
+                       apply_gated_bias=False, schedule="default", autotune=False, fwd_kernel_cfg=None,
+                       bwd_kernel_cfg=None, use_fast_causal_conv1d=False, kernel_path="unfused_gcg_fast"):
+    """y = q * causal_conv1d_ref(k * x) with the reference function's own filter-to-channel map
+    (vortex/ops/hyena_se/interface.py:342-397).
+
+    h: [G, 1, K].  Unlike inner_hyena_se (and the model path), this function assigns filters with
+    `h.squeeze(1).repeat(d // G, 1)` (interface.py:375-376): channel c is filtered by h[c % G] -- striped, not
+    blocked.  The kernels run it with one tap row per channel (a single shared row when G == 1).  Rounding
+    follows causal_conv1d_ref (in h.dtype); up to 4 taps on the default kernel_path the reference calls the
+    causal_conv1d extension, which accumulates conv + bias in float32 and takes no gated bias.
+    """
+    if inner_layout != "bdl":
+        raise AssertionError("unfused_gcg only supports bdl inner layout")
+    if kernel_path not in ("unfused_gcg", "unfused_gcg_fast"):
+        raise NotImplementedError("Reference cgcg kernel path not integrated in hyena_se_ref")
+    ops._need_cuda(x, k, q, h)
+    G = h.shape[0]
+    xb, kb, qb = (_to_bdl(t, input_layout) for t in (x, k, q))
+    assert kb.shape == qb.shape == xb.shape, "feature groups must have the same shape"
+    B, D, L = xb.shape
+    if apply_gated_bias and kernel_path == "unfused_gcg_fast":
+        warnings.warn("Gated bias not supported for unfused_gcg_fast kernel")
+    taps = ops._f32(h).reshape(G, -1)
+    K = taps.shape[1]
+    if G not in (1, D):
+        taps = taps.repeat(D // G, 1)                    # row c = h[c % G]
+    if kernel_path == "unfused_gcg_fast" and K <= 4:
+        b, mode = _bias_rule(torch.float32, bias, False, D)
+    else:
+        b, mode = _bias_rule(h.dtype, bias, apply_gated_bias, D)
+    y = _fir_per_channel(xb, taps, qb, kb, b, mode)
+    return _from_bdl(y, output_layout, G)
 
 
 def two_pass_chunked_gate_conv_gate(x, B, C, h, return_toeplitz=True, schedule="default", autotune=False,

@@ -43,7 +43,12 @@ typedef struct hyena_rows {
 enum hyena_bias_mode {
     HYENA_BIAS_NONE = 0,
     HYENA_BIAS_ADD = 1,         /* z = bf16(bf16(conv) + bias[d])      vortex/model/engine.py:222-223 */
-    HYENA_BIAS_GATED_FP32 = 2   /* z = bf16(conv + bias[d]*u) in fp32  vortex/model/engine.py:78      */
+    HYENA_BIAS_GATED_FP32 = 2,  /* z = bf16(conv + bias[d]*u) in fp32  vortex/model/engine.py:78      */
+    /* the two below: hyena_se_fwd and hyena_mr_fwd only */
+    HYENA_BIAS_ADD_FP32 = 3,    /* z = bf16(conv + bias[d]), one rounding: F.conv1d with float32 weights and its
+                                   own bias argument, vortex/ops/hyena_se/interface.py:236-243 */
+    HYENA_BIAS_GATED_BF16 = 4   /* z = bf16(bf16(conv) + bf16(bias[d]*u)): bf16 tensor arithmetic after the
+                                   convolution was cast, vortex/model/engine.py:208-221, :352-353 */
 };
 
 const char* hyena_version(void);

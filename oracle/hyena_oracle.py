@@ -25,6 +25,11 @@ How each function is pinned (see tests/test_oracle_*.py):
                                  test/test_prefill.py:85-229)
   toeplitz / correction        : known-answer arange filter of
                                  vortex/ops/hyena_se/tests/test_toeplitz.py
+  causal_conv1d_ref /
+  inner_hyena_se_ref           : float64 brute-force loops (bias inside the single
+                                 rounding, gated bias), a hand-computed rounding
+                                 known answer, and the impulse response, which
+                                 shows the striped filter-to-channel map
   step_fir / step_iir          : no reference test touches these ("parity
                                  unpinned" by the reference's own tests); they
                                  are pinned here by prefill-vs-decode
@@ -477,6 +482,64 @@ def causal_conv1d_ref(x, weight, bias=None, apply_gated_bias=False):
     if apply_gated_bias:
         out = out + x * gb
     return out.to(dt)
+
+
+def reshape_inputs(x, k, q, num_groups, input_layout):
+    """vortex/ops/hyena_se/interface.py:272-319 for inner_layout == "bdl" (the only inner layout the
+    reference's inner_hyena_se_ref accepts, interface.py:370): to [B, D, L], channel d = g*dg + j."""
+    def one(t):
+        if input_layout == "bdl":
+            return t
+        if input_layout == "blgdg":                       # rearrange "b l g dg -> b (g dg) l"
+            b, l, g, dg = t.shape
+            assert g == num_groups, "number of groups in feature groups and filter must match"
+            return t.permute(0, 2, 3, 1).reshape(b, g * dg, l)
+        if input_layout == "bgdgl":                       # rearrange "b g d l -> b (g d) l"
+            b, g, dg, l = t.shape
+            assert g == num_groups, "number of groups in feature groups and filter must match"
+            return t.reshape(b, g * dg, l)
+        raise NotImplementedError("input_layout must be bdl, blgdg or bgdgl")
+    return one(x), one(k), one(q)
+
+
+def reshape_outputs(y, num_groups, output_layout):
+    """vortex/ops/hyena_se/interface.py:322-339 for inner_layout == "bdl"."""
+    b, d, l = y.shape
+    if output_layout == "bdl":
+        return y
+    if output_layout == "bld":
+        return y.permute(0, 2, 1)
+    if output_layout == "blgdg":                          # rearrange "b (g dg) l -> b l g dg"
+        return y.reshape(b, num_groups, d // num_groups, l).permute(0, 3, 1, 2)
+    raise NotImplementedError("output_layout must be bld, bdl or blgdg")
+
+
+def inner_hyena_se_ref(x, k, q, h, bias=None, input_layout="bdl", output_layout="bdl", apply_gated_bias=False,
+                       kernel_path="unfused_gcg_fast"):
+    """vortex/ops/hyena_se/interface.py:342-397: y = q * causal_conv1d(k * x) with h (g, 1, K).
+
+    Filters are assigned to channels with `h.squeeze(1).repeat(d // g, 1)` (interface.py:375-376): channel c
+    uses filter c % g -- striped, unlike the repeat_interleave (blocked) map of the model path and of
+    gcg_fwd_ref.  With g == d the reference leaves h as [d, 1, K], which its own causal_conv1d_ref cannot
+    unpack (`dim, width = weight.shape`, interface.py:231); the squeeze is the evident intent and is done here.
+    The K <= 4 shortcut of kernel_path "unfused_gcg_fast" (interface.py:380-381) calls the causal_conv1d CUDA
+    extension, which is not part of this oracle: it accumulates conv + bias in float32 and rounds once
+    (vortex/ops/conv/csrc/causal_conv1d_fwd.cu:108-120), i.e. causal_conv1d_ref with float32 weights, which is
+    what runs here for it.  It takes no gated bias.
+    """
+    num_groups = h.shape[0]
+    x, k, q = reshape_inputs(x, k, q, num_groups, input_layout)
+    assert k.shape == q.shape == x.shape, "feature groups must have the same shape"
+    b, d, l = x.shape
+    h = h.squeeze(1)
+    if num_groups != d:
+        h = h.repeat(d // num_groups, 1)
+    kx = k * x
+    if kernel_path == "unfused_gcg_fast" and h.shape[-1] <= 4:
+        y = causal_conv1d_ref(kx, h.float(), bias=None if bias is None else bias.float())
+    else:
+        y = causal_conv1d_ref(kx, h, bias=bias, apply_gated_bias=apply_gated_bias)
+    return reshape_outputs(q * y, num_groups, output_layout)
 
 
 # --------------------------------------------------------------------------

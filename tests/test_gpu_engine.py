@@ -334,8 +334,9 @@ def test_hyena_ops_interface_layouts():
                                           fwd_kernel_cfg=I.FwdKernelConfig(), bwd_kernel_cfg=I.BwdKernelConfig())
     assert y.shape == ref.shape and rel_err(y, ref) <= 2e-2
     xb, kb, qb = (t.reshape(B, L, G * dg).transpose(1, 2).contiguous() for t in (x, k, q))
-    y2 = I.inner_hyena_se_ref(xb.to(DEV), kb.to(DEV), qb.to(DEV), h.to(DEV), output_layout="bld")
+    y2 = I.inner_hyena_se(xb.to(DEV), kb.to(DEV), qb.to(DEV), h.to(DEV), output_layout="bld")   # blocked groups
     assert rel_err(y2, ref.reshape(B, L, G * dg)) <= 2e-2
+    # inner_hyena_se_ref stripes the filters instead (tests/test_gpu_hyena_ops.py)
     # package-level names of vortex/model/layers.py:19
     out = hyena_ops.hyena_se_fwd(kb.to(DEV), qb.to(DEV), xb.to(DEV), h.to(DEV))
     assert rel_err(out.transpose(1, 2), ref.reshape(B, L, G * dg)) <= 2e-2

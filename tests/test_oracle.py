@@ -344,3 +344,112 @@ def test_truncated_fir_branch_of_parallel_iir(T):
     x1v = x1 * v
     assert st is None
     assert torch.equal(out, ((O.truncated_fir(x1v, h, T) + x1v * Db[:, None]) * x2).permute(0, 2, 1))
+
+
+# ---------------------------------------------------------------- hyena_ops.interface references (a12)
+
+def _bf16_ulp(x):
+    """Spacing of bfloat16 at |x| (float64 tensor in, float64 out)."""
+    e = torch.floor(torch.log2(x.abs().clamp_min(2.0 ** -126)))
+    return torch.pow(2.0, e - 7)
+
+
+@pytest.mark.parametrize("K,bias_kind", [(3, "none"), (7, "add"), (7, "gated"), (33, "add"), (128, "gated")])
+def test_causal_conv1d_ref_vs_bruteforce_fp32_weights(K, bias_kind):
+    # interface.py:207-244 with float32 weights: x is upcast, conv + bias (or conv + x*gated_bias) is formed in
+    # float32 and rounded ONCE to the input dtype
+    g = torch.Generator().manual_seed(K)
+    B, D, L = 2, 5, 150
+    x = torch.randn(B, D, L, generator=g).bfloat16()
+    w = torch.randn(D, K, generator=g) / math.sqrt(K)
+    bias = torch.randn(D, generator=g) if bias_kind != "none" else None
+    # the gated bias multiplies x [B, D, L] by plain broadcasting (interface.py:240), so a per-channel one is [D, 1]
+    out = O.causal_conv1d_ref(x, w, bias[:, None] if bias_kind == "gated" else bias, apply_gated_bias=bias_kind == "gated")
+    assert out.dtype == torch.bfloat16 and out.shape == (B, D, L)
+    xn, wn = x.double().numpy(), w.double().numpy()
+    for b in range(B):
+        z = torch.from_numpy(brute_corr(xn[b], wn))
+        if bias_kind == "add":
+            z = z + bias.double()[:, None]
+        if bias_kind == "gated":
+            z = z + x[b].double() * bias.double()[:, None]
+        # one rounding of the exact value, up to float32 accumulation error: never off by more than half an ulp + eps
+        err = (out[b].double() - z).abs()
+        assert (err <= 0.5 * _bf16_ulp(z) * 1.02 + 1e-6).all(), (K, bias_kind, err.max())
+
+
+def test_causal_conv1d_ref_single_rounding_known_answer():
+    # conv = 1 + 2^-8 (a bf16 tie that rounds down to 1), bias = 2^-8: one rounding of the sum gives 1 + 2^-7,
+    # rounding the convolution first would give bf16(1 + 2^-8) = 1
+    x = torch.tensor([[[1.0, 1.0]]]).bfloat16()
+    w = torch.tensor([[2.0 ** -8, 1.0]])                     # w[K-1] on the current sample
+    b = torch.tensor([2.0 ** -8])
+    out = O.causal_conv1d_ref(x, w, b)
+    assert out.flatten().tolist() == [1.0, 1.0 + 2.0 ** -7]
+    gated = O.causal_conv1d_ref(x, w, b[:, None], apply_gated_bias=True)  # + x * 2^-8 in float32, same sums
+    assert gated.flatten().tolist() == [1.0, 1.0 + 2.0 ** -7]
+    # float32 in: nothing is rounded to bf16 at all
+    out32 = O.causal_conv1d_ref(x.float(), w, b)
+    assert out32.dtype == torch.float32 and out32.flatten().tolist() == [1.0 + 2.0 ** -8, 1.0 + 2.0 ** -7]
+
+
+def test_causal_conv1d_ref_bf16_weights_compute_in_bf16():
+    # weight.dtype decides the arithmetic (interface.py:228): with bf16 weights F.conv1d runs in bf16 and the gated
+    # bias is bf16 tensor arithmetic, out + x*bias with both roundings.  Pinned to the exact value within 2 ulps.
+    g = torch.Generator().manual_seed(5)
+    B, D, L, K = 1, 4, 64, 7
+    x = torch.randn(B, D, L, generator=g).bfloat16()
+    w = (torch.randn(D, K, generator=g) / math.sqrt(K)).bfloat16()
+    bias = torch.randn(D, generator=g).bfloat16()
+    out = O.causal_conv1d_ref(x, w, bias[:, None], apply_gated_bias=True)
+    assert out.dtype == torch.bfloat16
+    z = torch.from_numpy(brute_corr(x[0].double().numpy(), w.double().numpy()))
+    exact = z + x[0].double() * bias.double()[:, None]
+    scale = torch.maximum(z.abs(), (x[0].double() * bias.double()[:, None]).abs())
+    assert ((out[0].double() - exact).abs() <= 2.0 * _bf16_ulp(torch.maximum(scale, exact.abs()))).all()
+
+
+@pytest.mark.parametrize("G", [1, 2, 4, 8])
+def test_inner_hyena_se_ref_stripes_filters_over_channels(G):
+    # interface.py:375-376: h.squeeze(1).repeat(d // g, 1) -> channel c is filtered by h[c % g].  Impulse input,
+    # unit gates: the output rows are the filters themselves, read back in cross-correlation order.
+    D, L, K = 8, 16, 5
+    h = torch.arange(G * K, dtype=torch.float32).reshape(G, 1, K) + 1
+    x = torch.zeros(1, D, L, dtype=torch.bfloat16)
+    x[..., 0] = 1
+    one = torch.ones_like(x)
+    y = O.inner_hyena_se_ref(x, one, one, h, kernel_path="unfused_gcg")
+    for c in range(D):
+        assert y[0, c, :K].tolist() == h[c % G, 0].flip(-1).tolist(), c
+        assert y[0, c, K:].abs().max() == 0
+    if 1 < G < D:      # and it is NOT the blocked map of the model path
+        blocked = O.gcg_fwd_ref(x.permute(0, 2, 1).reshape(1, L, G, D // G), one.permute(0, 2, 1).reshape(1, L, G, D // G),
+                                one.permute(0, 2, 1).reshape(1, L, G, D // G), h.bfloat16())
+        assert not torch.equal(blocked.reshape(1, L, D).permute(0, 2, 1).float(), y.float())
+
+
+@pytest.mark.parametrize("K,path", [(4, "unfused_gcg_fast"), (4, "unfused_gcg"), (7, "unfused_gcg_fast")])
+def test_inner_hyena_se_ref_vs_bruteforce_and_layouts(K, path):
+    g = torch.Generator().manual_seed(K)
+    B, G, dg, L = 2, 3, 4, 40
+    D = G * dg
+    x, k, q = (torch.randn(B, D, L, generator=g).bfloat16() for _ in range(3))
+    h = torch.randn(G, 1, K, generator=g) / math.sqrt(K)
+    bias = torch.randn(D, generator=g)
+    y = O.inner_hyena_se_ref(x, k, q, h, bias=bias, kernel_path=path)
+    kx = (k * x)
+    w = h[:, 0].repeat(D // G, 1).double().numpy()
+    for b in range(B):
+        z = torch.from_numpy(brute_corr(kx[b].double().numpy(), w)) + bias.double()[:, None]
+        zb = z.float().bfloat16()                 # one rounding of conv + bias (float32 accumulation: allow one ulp)
+        ref = (q[b] * zb).double()
+        err = (y[b].double() - ref).abs()
+        assert (err <= 1.01 * _bf16_ulp(z) * q[b].double().abs() + _bf16_ulp(ref)).all()
+    # layouts: (b, l, g, dg) and (b, g, dg, l) in, "bld" / "blgdg" out are pure re-indexings of the same numbers
+    to_blgdg = lambda t: t.permute(0, 2, 1).reshape(B, L, G, dg)
+    y2 = O.inner_hyena_se_ref(to_blgdg(x), to_blgdg(k), to_blgdg(q), h, bias=bias, input_layout="blgdg",
+                              output_layout="blgdg", kernel_path=path)
+    assert torch.equal(y2, to_blgdg(y))
+    y3 = O.inner_hyena_se_ref(x.reshape(B, G, dg, L), k.reshape(B, G, dg, L), q.reshape(B, G, dg, L), h, bias=bias,
+                              input_layout="bgdgl", output_layout="bld", kernel_path=path)
+    assert torch.equal(y3, y.permute(0, 2, 1))

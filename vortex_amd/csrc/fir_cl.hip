@@ -421,8 +421,10 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     if (K < 1 || K > 128) return hyena_fail(HYENA_ENOSUP, "%s: K=%d outside 1..128", who, K);
     if ((D / G) % 16 != 0)
         return hyena_fail(HYENA_ENOSUP, "%s: D/G=%lld must be a multiple of 16", who, (long long)(D / G));
-    if (bias_mode < 0 || bias_mode > 2 || (bias_mode != HYENA_BIAS_NONE && !bias))
+    if (bias_mode < 0 || bias_mode > 4 || (bias_mode != HYENA_BIAS_NONE && !bias))
         return hyena_fail(HYENA_EINVAL, "%s: bias_mode %d needs a bias pointer", who, bias_mode);
+    if (bias_mode > HYENA_BIAS_GATED_FP32)
+        return hyena_fail(HYENA_ENOSUP, "%s: bias_mode %d is built for the sequence-major kernels only", who, bias_mode);
     if (bx_out && (bx_from < 0 || bx_from > L)) return hyena_fail(HYENA_EINVAL, "%s: bx_from outside 0..L", who);
     if (bx_out && a.feat && L - bx_from > K - 1)
         return hyena_fail(HYENA_ENOSUP, "%s: with the featurizer fused, bx is the cache tail (at most K-1 = %d samples)",

@@ -185,7 +185,7 @@ __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
             const int tcol = 64 * w + 32 * tau + 256 * s + 16 * hh;
             const f32x16 acc = tau ? acc1 : acc0;
             u32x4 ua = {0, 0, 0, 0}, ub2 = {0, 0, 0, 0};
-            if (BIAS == HYENA_BIAS_GATED_FP32) {
+            if (BIAS == HYENA_BIAS_GATED_FP32 || BIAS == HYENA_BIAS_GATED_BF16) {
                 ua = *(const u32x4*)(u_lds + c * URS + HALO + tcol);
                 ub2 = *(const u32x4*)(u_lds + c * URS + HALO + tcol + 8);
             }
@@ -201,6 +201,16 @@ __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
                 if (BIAS == HYENA_BIAS_ADD) {
                     a0 = round_bf(a0) + bz;
                     a1 = round_bf(a1) + bz;
+                }
+                if (BIAS == HYENA_BIAS_ADD_FP32) {
+                    a0 += bz;
+                    a1 += bz;
+                }
+                if (BIAS == HYENA_BIAS_GATED_BF16) {             // bf16 tensor arithmetic: every product and sum rounded
+                    const uint32_t uw = j < 4 ? ua[j] : ub2[j - 4];
+                    const uint32_t yp = pack_bf2(a0, a1), tp = pack_bf2(bz * bf_lo(uw), bz * bf_hi(uw));
+                    a0 = bf_lo(yp) + bf_lo(tp);
+                    a1 = bf_hi(yp) + bf_hi(tp);
                 }
                 const uint32_t p = pack_bf2(a0, a1);
                 if (j < 4) z0[j] = p; else z1[j - 4] = p;
@@ -239,7 +249,7 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
         return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: bad sizes B=%lld D=%lld L=%lld G=%lld", (long long)B,
                           (long long)D, (long long)L, (long long)G);
     if (K < 1 || K > 128) return hyena_fail(HYENA_ENOSUP, "hyena_mr_fwd: K=%d outside 1..128", K);
-    if (bias_mode < 0 || bias_mode > 2 || (bias_mode != HYENA_BIAS_NONE && !bias))
+    if (bias_mode < 0 || bias_mode > 4 || (bias_mode != HYENA_BIAS_NONE && !bias))
         return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: bias_mode %d needs a bias pointer", bias_mode);
     if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15))
         return hyena_fail(HYENA_EALIGN, "hyena_mr_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
@@ -300,6 +310,10 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     MR_CASE(false, false, HYENA_BIAS_NONE)
     MR_CASE(false, false, HYENA_BIAS_ADD)
     MR_CASE(false, false, HYENA_BIAS_GATED_FP32)
+    MR_CASE(true, true, HYENA_BIAS_ADD_FP32)
+    MR_CASE(false, false, HYENA_BIAS_ADD_FP32)
+    MR_CASE(true, true, HYENA_BIAS_GATED_BF16)
+    MR_CASE(false, false, HYENA_BIAS_GATED_BF16)
 #undef MR_CASE
 #undef MR_LAUNCH
     if (!ok) return hyena_fail(HYENA_ENOSUP, "hyena_mr_fwd: this gate/bias combination has no kernel");

@@ -111,10 +111,15 @@ __global__ __launch_bounds__(256) void se_fir_kernel(RowMap x1, RowMap x2, RowMa
 #pragma unroll
             for (int k = 0; k < K; ++k) acc = fmaf(w[k], ext[i + k], acc);
             if (BIAS == HYENA_BIAS_GATED_FP32) acc = fmaf(bz, u[i], acc);
+            if (BIAS == HYENA_BIAS_ADD_FP32) acc += bz;
             z[e] = acc;
         }
         uint32_t zp = pack_bf2(z[0], z[1]);                      // z = bf16(conv), one conversion per pair
         if (BIAS == HYENA_BIAS_ADD) zp = pack_bf2(bf_lo(zp) + bz, bf_hi(zp) + bz);
+        if (BIAS == HYENA_BIAS_GATED_BF16) {                     // bf16 tensor arithmetic: every product and sum rounded
+            const uint32_t tp = pack_bf2(bz * u[2 * j], bz * u[2 * j + 1]);
+            zp = pack_bf2(bf_lo(zp) + bf_lo(tp), bf_hi(zp) + bf_hi(tp));
+        }
         o[j] = POST ? pack_bf2(bf_lo(zp) * bf_lo(a2[j]), bf_hi(zp) * bf_hi(a2[j])) : zp;
     }
     if (active) {
@@ -155,6 +160,10 @@ bool launch_gates(bool pre, bool post, int bias_mode, bool rowu, bool nt, dim3 g
     SE_CASE(true, false, HYENA_BIAS_NONE)
     SE_CASE(false, true, HYENA_BIAS_NONE)
     SE_CASE(false, false, HYENA_BIAS_GATED_FP32)
+    SE_CASE(true, true, HYENA_BIAS_ADD_FP32)
+    SE_CASE(false, false, HYENA_BIAS_ADD_FP32)
+    SE_CASE(true, true, HYENA_BIAS_GATED_BF16)
+    SE_CASE(false, false, HYENA_BIAS_GATED_BF16)
 #undef SE_CASE
     return false;
 }
@@ -169,7 +178,7 @@ extern "C" int hyena_se_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
         return hyena_fail(HYENA_EINVAL, "hyena_se_fwd: bad sizes B=%lld D=%lld L=%lld G=%lld", (long long)B,
                           (long long)D, (long long)L, (long long)G);
     if (K < 2 || K > 8) return hyena_fail(HYENA_ENOSUP, "hyena_se_fwd: K=%d outside 2..8 (use hyena_mr_fwd)", K);
-    if (bias_mode < 0 || bias_mode > 2 || (bias_mode != HYENA_BIAS_NONE && !bias))
+    if (bias_mode < 0 || bias_mode > 4 || (bias_mode != HYENA_BIAS_NONE && !bias))
         return hyena_fail(HYENA_EINVAL, "hyena_se_fwd: bias_mode %d needs a bias pointer", bias_mode);
     if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15))
         return hyena_fail(HYENA_EALIGN, "hyena_se_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
