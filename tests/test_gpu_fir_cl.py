@@ -245,3 +245,31 @@ def test_cl_nontemporal_variants_match(K, override):
         res[nt] = (ops.fir_cl_fwd(x1, x2, v, h, taps_reversed=K < 128),
                    ops.fir_layer_fwd(u, wf, None, cmap, h, taps_reversed=K < 128))
     assert torch.equal(res["0"][0], res["1"][0]) and torch.equal(res["0"][1], res["1"][1])
+
+
+@pytest.mark.parametrize("Ks,nseg", [(3, 3), (4, 2), (3, 1)])
+def test_layer_fwd_oldest_tap_across_segments(Ks, nseg, override):
+    # Taps that do not decay: the oldest one (lag 127) weighs as much as the newest, so an output at the first
+    # sample of a later segment that read a wrong halo sample is off by a whole term.  Checked per element:
+    # the first halo samples of a segment are featurizer outputs and need the Ks-1 rows before the halo step.
+    from parity import abs_scale, assert_gated_close
+    B, L, D, H, G, K = 1, 1024 + 384, 64, 4, 4, 128
+    override(cl_nseg=nseg)
+    g = torch.Generator().manual_seed(Ks)
+    C = 3 * D
+    u = torch.randn(B, L, C, generator=g).bfloat16()
+    wf = torch.randn(C, 1, Ks, generator=g) / Ks ** 0.5
+    h = (torch.randn(G, 1, K, generator=g) / K ** 0.5).bfloat16().float()           # bf16-exact: the MFMA operand is exact
+    ref, _ = oracle_layer(u, wf, None, h, torch.zeros(D), D, H, False, True, False)
+    z, _ = O.parallel_fir(u, wf, None, fir_length=Ks, dim_last=True, gate=False)
+    x2, x1, v = O.interleave(z).split([D, D, D], dim=1)
+    bx = x1 * v
+    zr = O.fft_causal_conv_fp32(bx.float(), h.repeat_interleave(D // G, 0)[:, 0]).bfloat16()     # pre-gate value
+    y = ops.fir_layer_fwd(u.to(DEV), wf.reshape(C, Ks).t().contiguous().to(DEV), None, ops.gate_channel_map(D, interleave=True),
+                          h.reshape(G, K).to(DEV))
+    y = y.permute(0, 2, 1)
+    assert rel_err(y, ref) <= 2e-2
+    S = abs_scale(bx, h.repeat_interleave(D // G, 0)[:, 0])
+    # the gates themselves carry the featurizer's own rounding boundary (one bf16 ulp of x1, v or x2 now and then),
+    # which moves bx by up to 2^-7 relatively: 2^-6 * S covers it, a wrong halo sample is off by ~S / 11
+    assert_gated_close(y, ref, zr, x2, S, 2.0 ** -6, ulps_z=2.0, gate_ulps=1.0, what=f"fused MR layer Ks={Ks} nseg={nseg}")

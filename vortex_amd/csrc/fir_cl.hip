@@ -160,8 +160,10 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     if (t_begin >= t_end) return;
     const int64_t ts0 = t_begin > 0 ? t_begin - TL : 0;      // one extra step rebuilds the halo of a later segment
     // a short filter (MLO = 7: K <= 17) only reaches 16 samples back, the featurizer at most 3 more: of the halo
-    // step only the last 24 rows are read, the rest stay zero and feed no output of this segment
-    const int64_t t_lo = MLO == 7 ? t_begin - 24 : ts0;
+    // step only the last 24 rows are read, the rest stay zero and feed no output of this segment.  Otherwise the
+    // whole halo step is read, and with the featurizer fused in also the RF rows ahead of it: the first halo
+    // samples are featurizer outputs themselves and need their own history (lag K-1 = 127 reaches sample ts0 + 1).
+    const int64_t t_lo = MLO == 7 ? t_begin - 24 : ts0 - RF;
 
     // zero halo at the sequence start
     if (t_begin == 0) {
