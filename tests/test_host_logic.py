@@ -192,3 +192,34 @@ def test_operator_module_compute_filter_matches_the_closed_form():
     assert torch.allclose(h[0, :, 0], r.sum(1), atol=1e-6)          # h[0] = sum of the residues
     mod.update_time(6, "cpu")
     assert mod.t.shape == (1, 1, 6)
+
+
+def test_per_element_bound_catches_a_single_wrong_halo_sample():
+    # the error statement of tests/parity.py, exercised on the CPU: an output that read one wrong input sample at a
+    # segment start fails it even where the sample is small, while one-ulp roundings of the pre-gate value pass
+    import pytest
+    from parity import abs_scale, assert_gated_close, rel_err
+    g = torch.Generator().manual_seed(0)
+    B, D, L, K = 1, 4, 512, 128
+    x2, x1, v = O.make_gates(B, D, L, seed=1)
+    h = torch.randn(D, K, generator=g) / K ** 0.5 * torch.exp(-0.08 * torch.arange(K))     # decaying: lag 127 is tiny
+    u = x1 * v
+    z32 = O.fft_causal_conv_fp32(u.float(), h)
+    z_ref = z32.bfloat16()
+    ref = x2 * z_ref
+    S = abs_scale(u, h)
+    # legitimate: sums that land on the other side of a rounding boundary
+    nudged = (z32 * (1 + 2.0 ** -10)).bfloat16()
+    assert_gated_close(x2 * nudged, ref, z_ref, x2, S, 2.0 ** -8, fft_floor=4e-6)
+    # a slip: output t = 256 misses input t - 127 (what a halo sample lost at a segment start does)
+    bad32 = z32.clone()
+    bad32[..., 256] -= h[:, 127] * u[..., 256 - 127].float()
+    bad = x2 * bad32.bfloat16()
+    assert rel_err(bad, ref) < 2e-2                     # invisible to the normalised maximum ...
+    hflat = torch.randn(D, K, generator=g) / K ** 0.5   # ... unless the oldest tap carries weight
+    z32f = O.fft_causal_conv_fp32(u.float(), hflat)
+    badf = z32f.clone()
+    badf[..., 256] -= hflat[:, 127] * u[..., 256 - 127].float()
+    with pytest.raises(AssertionError):
+        assert_gated_close(x2 * badf.bfloat16(), x2 * z32f.bfloat16(), z32f.bfloat16(), x2, abs_scale(u, hflat),
+                           2.0 ** -8, fft_floor=4e-6)
