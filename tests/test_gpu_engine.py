@@ -472,3 +472,82 @@ def test_operator_module_truncated_fir_config(T, G):
     assert rel_err(y, y_ref) <= 2e-2
     with pytest.raises(NotImplementedError):
         mod(u.to(DEV), HyenaCascadeIIRInferenceParams())
+
+
+@pytest.mark.parametrize("cplx,L", [(False, 1032), (True, 520)])
+def test_engine_parallel_iir_recurrence_prefill_seam(cplx, L):
+    # prefill_style="recurrence" (vortex/model/engine.py:314-321, :473-504): poles themselves and residues arrive as
+    # [D, S, 1, 2] (re, im) lanes, one filter per channel; the state comes back as [B, D, S, 2] float32.  Checked
+    # against the explicit recurrence in float64 (what that branch evaluates, without its bf16 state rounding).
+    B, D, H, S = 2, 16, 2, 16
+    g = torch.Generator().manual_seed(L)
+    lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(D, S, seed=L, pmax=0.99)
+    p = torch.exp(lp[..., 0].to(torch.complex64))
+    poles = torch.view_as_real(p)[:, :, None, :].contiguous()                            # [D, S, 1, 2]
+    res_re = (r.real if cplx else r).float()
+    residues = torch.stack([res_re, torch.zeros_like(res_re)], -1)[:, :, None, :].contiguous()
+    z_pre = torch.randn(B, 3 * D, L, generator=g).bfloat16()
+    Db = torch.randn(D, generator=g).bfloat16()
+    dims = (D, H, D // H, S, D)
+    x2, x1, v = z_pre.split([D, D, D], dim=1)
+    x1v = x1 * v
+    # y = sum_s r_re * s_re is what engine.py:500 forms: residues with a zero imaginary lane in the exact recurrence
+    y64, s64 = O.prefill_direct_recurrence(x1v, lp.to(torch.complex64) if cplx else lp, res_re.to(torch.complex64) if cplx else res_re)
+    y_ref = ((y64.float().bfloat16() + x1v * Db[:, None]) * x2).permute(0, 2, 1)
+    ip = HyenaCascadeIIRInferenceParams()
+    eng = HyenaInferenceEngine()
+    y = eng.parallel_iir(z_pre.to(DEV), None, Db.to(DEV), L, poles.to(DEV), residues.to(DEV), None, dims, 3,
+                         inference_params=ip, prefill_style="recurrence")
+    assert y.shape == (B, L, D) and rel_err(y, y_ref) <= 2e-2
+    st = ip.state_dict[3]
+    assert st.shape == (B, D, S, 2) and st.dtype == torch.float32
+    s_ref = torch.view_as_real(s64.to(torch.complex128)) if cplx else torch.stack([s64, torch.zeros_like(s64)], -1)
+    assert rel_err(st, s_ref) <= 1e-4
+    with pytest.raises(ValueError):
+        eng.parallel_iir(z_pre.to(DEV), None, Db.to(DEV), L, lp.to(DEV), r.to(DEV), None, dims, 3,
+                         inference_params=HyenaCascadeIIRInferenceParams(), prefill_style="recurrence")
+    with pytest.raises(NotImplementedError):
+        eng.parallel_iir(z_pre.to(DEV), None, Db.to(DEV), L, lp.to(DEV), r.to(DEV), None, dims, 3,
+                         inference_params=HyenaCascadeIIRInferenceParams(), prefill_style="modal-scan")
+
+
+def test_engine_per_channel_weight_with_groups_argument():
+    # vortex's conv1d filters per channel whatever `groups` says (engine.py:203).  A weight whose rows differ inside a
+    # group must therefore run per channel; one that was expanded with repeat_interleave may be folded back.
+    B, D, H, G, K, L = 1, 32, 2, 4, 7, 256
+    g = torch.Generator().manual_seed(0)
+    u = torch.randn(B, 3 * D, L, generator=g).bfloat16()
+    dims = (D, H, D // H, 16, G)
+    eng = HyenaInferenceEngine()
+    w_distinct = torch.randn(D, 1, K, generator=g) / K ** 0.5
+    w_grouped = (torch.randn(G, 1, K, generator=g) / K ** 0.5).repeat_interleave(D // G, 0)
+    for w in (w_distinct, w_grouped):
+        ref, _ = O.parallel_fir(u, w, None, L, dims, groups=G, dim_last=False, fir_length=K, gate=True)
+        wd = w.to(DEV)
+        for _ in range(2):                                          # second call: the cached verdict
+            z, _ = eng.parallel_fir(torch.nn.functional.conv1d, u.to(DEV), wd, None, L, dims, groups=G, dim_last=False,
+                                    fir_length=K, gate=True)
+            assert rel_err(z, ref) <= 2e-2
+    # an in-place update of the same tensor object is seen (version counter)
+    wd = w_grouped.clone().to(DEV)
+    eng.parallel_fir(torch.nn.functional.conv1d, u.to(DEV), wd, None, L, dims, groups=G, dim_last=False, fir_length=K, gate=True)
+    wd.copy_(w_distinct)
+    ref, _ = O.parallel_fir(u, w_distinct, None, L, dims, groups=G, dim_last=False, fir_length=K, gate=True)
+    z, _ = eng.parallel_fir(torch.nn.functional.conv1d, u.to(DEV), wd, None, L, dims, groups=G, dim_last=False,
+                            fir_length=K, gate=True)
+    assert rel_err(z, ref) <= 2e-2
+
+
+def test_engine_short_fir_gated_bias_in_bf16():
+    # K < 128 with gated_bias (engine.py:218-221): z = bf16(conv), then z + bias*u in bf16 tensor arithmetic
+    B, D, H, G, K, L = 2, 32, 2, 2, 7, 264
+    g = torch.Generator().manual_seed(1)
+    u = torch.randn(B, 3 * D, L, generator=g).bfloat16()
+    w = (torch.randn(G, 1, K, generator=g) / K ** 0.5).repeat_interleave(D // G, 0)
+    bias = torch.randn(D, generator=g).bfloat16()
+    dims = (D, H, D // H, 16, G)
+    ref, _ = O.parallel_fir(u, w, bias, L, dims, groups=G, gated_bias=True, dim_last=False, fir_length=K, gate=True)
+    z, _ = HyenaInferenceEngine().parallel_fir(torch.nn.functional.conv1d, u.to(DEV), w.to(DEV), bias.to(DEV), L, dims,
+                                               groups=G, gated_bias=True, dim_last=False, fir_length=K, gate=True)
+    assert rel_err(z, ref) <= 2e-2
+    assert (z.cpu() == ref).float().mean() > 0.97

@@ -13,7 +13,7 @@ import torch
 import torch.nn as nn
 
 from . import ops
-from ._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE
+from ._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_BF16, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE
 
 
 @dataclass
@@ -176,7 +176,7 @@ class HyenaCascade(nn.Module):
         p = getattr(self, name)
         if p is None:
             return None
-        key = (p.data_ptr(), p._version, p.dtype)
+        key = (id(p), p.data_ptr(), p._version, p.dtype)
         hit = self._f32_cache.get(name)
         if hit is None or hit[0] != key:
             t = p.detach().to(torch.float32)
@@ -204,7 +204,8 @@ class HyenaCascade(nn.Module):
         return (h.real if h.is_complex() else h), filter_dtype, log_poles, residues
 
     def modal_plan(self):
-        key = (self.log_poles._version, self.residues._version, self.log_poles.data_ptr())
+        key = (id(self.log_poles), id(self.residues), self.log_poles._version, self.residues._version,
+               self.log_poles.data_ptr(), self.residues.data_ptr())
         if self._plan is None or self._plan[0] != key:
             self._plan = (key, ops.ModalPlan(self.log_poles, self.residues))
         return self._plan[1]
@@ -249,8 +250,10 @@ class HyenaCascade(nn.Module):
             with torch.no_grad():
                 h = self.compute_filter(T, u.device)[0][0]
             taps = h.to(torch.bfloat16).to(torch.float32).contiguous()                     # [G, T]
+            # (bf16(y) + x1v*D) in the tensors' own dtype (engine.py:351-353): bf16 arithmetic with a bf16 D
+            mode = HYENA_BIAS_GATED_BF16 if self.D.dtype == torch.bfloat16 else HYENA_BIAS_GATED_FP32
             y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, T, device=u.device, bias=self._f32_param("D"),
-                                 bias_mode=HYENA_BIAS_GATED_FP32, taps_reversed=True, force_mfma=True)
+                                 bias_mode=mode, taps_reversed=True, force_mfma=True)
         else:
             y, _, state = ops.li_fwd_rows(r1, r2, rv, self.modal_plan(), self.D, B, D, L, device=u.device,
                                           want_state=caching)
@@ -286,7 +289,8 @@ class HyenaCascade(nn.Module):
         """u [B, L, 3D] -> y [B, L, D] in one launch; with a cache object also the two FIR caches."""
         B, L, C = u.shape
         K, Ks = self.fir_inner_filter_length, self.short_filter_length
-        key = ("short_filter_weight_t", self.short_filter_weight.data_ptr(), self.short_filter_weight._version)
+        key = ("short_filter_weight_t", id(self.short_filter_weight), self.short_filter_weight.data_ptr(),
+               self.short_filter_weight._version)
         hit = self._f32_cache.get("wf_t")
         if hit is None or hit[0] != key:
             hit = (key, self._f32_param("short_filter_weight", (C, Ks)).t().contiguous())

@@ -6,23 +6,50 @@ switches a vortex HyenaCascade to the HIP path with no other source change.
 Everything here runs on the GPU through the C ABI; there is no PyTorch fallback
 for the convolutions, and CPU tensors are rejected.
 """
+import weakref
+
 import torch
 
 from . import ops
-from ._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE
+from ._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_BF16, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE
 
 IIR_PREFILL_MODES = ["recurrence", "modal-fft", "hybrid-modal-recurrence", "modal-scan", "canonical-fft",
                      "iir-fir-caching"]
 
 
+_GROUPED_OK = {}     # id(weight) -> (weakref, version, groups, verdict): the row-equality check runs once per parameter version
+
+
+def _rows_constant_in_groups(weight, w, D, groups):
+    """Whether a [D, K] tap table repeats each row D/groups times (what repeat_interleave of a [G, 1, K] filter bank
+    gives, vortex/model/model.py:261-262).  One device reduction and host read per parameter version, cached."""
+    hit = _GROUPED_OK.get(id(weight))
+    if hit is not None and hit[0]() is weight and hit[1] == weight._version and hit[2] == groups:
+        return hit[3]
+    ok = bool((w.reshape(groups, D // groups, -1) == w.reshape(groups, D // groups, -1)[:, :1]).all())
+    if len(_GROUPED_OK) > 256:
+        _GROUPED_OK.clear()
+    _GROUPED_OK[id(weight)] = (weakref.ref(weight), weight._version, groups, ok)
+    return ok
+
+
 def _group_taps(weight, D, groups):
-    """[D, 1, K] (a [G, 1, K] filter bank expanded with repeat_interleave, vortex/model/model.py:261-262)
-    or [G, 1, K] -> ([G', K] float32, G')."""
+    """[D, 1, K] or [G, 1, K] -> [G', K] float32 taps for the kernels.
+
+    vortex hands the engine a [G, 1, K] filter bank expanded with repeat_interleave to [D, 1, K] together with
+    `groups` (vortex/model/model.py:261-286); its own conv1d ignores `groups` and filters per channel
+    (vortex/model/engine.py:203).  The expanded table is folded back to [G, K] only when its rows really are
+    constant inside each group (checked once per parameter version); distinct per-channel rows run per channel."""
     w = weight.detach().reshape(weight.shape[0], -1)
     rows = w.shape[0]
-    if groups is not None and rows == D and groups < D and D % groups == 0:
+    if groups is not None and rows == D and groups < D and D % groups == 0 and _rows_constant_in_groups(weight, w, D, groups):
         w = w[:: D // groups]
     return w.to(torch.float32).contiguous()
+
+
+def _same_tensor(hit, t):
+    """Cache guard: the cached entry was built from this very tensor object at this version."""
+    return hit is not None and hit[0]() is t and hit[1] == t._version
 
 
 class HyenaInferenceEngine:
@@ -36,8 +63,8 @@ class HyenaInferenceEngine:
         self.ground_truth_activations_path = ground_truth_activations_path
         self.print_activations = print_activations
         self.hyena_flip_x1x2 = hyena_flip_x1x2
-        self._plans = {}
-        self._poles = {}
+        self._plan_hit = None        # (weakref poles, version, weakref residues, version, kind, ModalPlan)
+        self._poles_hit = None       # (weakref log-poles, version, exponentiated poles)
 
     # ------------------------------------------------------------------ prefill FIR
     def parallel_fir(self, fir_fn, u, weight, bias, L, dims, groups=None, gated_bias=False,
@@ -68,9 +95,11 @@ class HyenaInferenceEngine:
                 z = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, taps.shape[1], device=u.device,
                                      bias=ops._f32(bias), bias_mode=mode, taps_reversed=False, force_mfma=True)
             else:
-                if bias is not None and gated_bias:
-                    raise NotImplementedError("gated bias on the short-FIR branch has no kernel")
-                mode = HYENA_BIAS_NONE if bias is None else HYENA_BIAS_ADD
+                if bias is not None and bias.dtype != torch.bfloat16:
+                    raise NotImplementedError("a float32 bias promotes the short-FIR output to float32 in vortex; "
+                                              "only bfloat16 (or no) bias is supported")
+                # after the cast of the convolution: z + bias*u or z + bias in bf16 tensor arithmetic (engine.py:218-223)
+                mode = HYENA_BIAS_NONE if bias is None else (HYENA_BIAS_GATED_BF16 if gated_bias else HYENA_BIAS_ADD)
                 z = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, taps.shape[1], device=u.device,
                                      bias=ops._f32(bias), bias_mode=mode, taps_reversed=True)
             if pad:
@@ -118,13 +147,16 @@ class HyenaInferenceEngine:
         return x1, v
 
     # ------------------------------------------------------------------ prefill IIR
-    def _plan(self, poles, residues):
-        key = (poles.data_ptr(), poles._version, residues.data_ptr(), residues._version)
-        p = self._plans.get(key)
-        if p is None:
-            self._plans.clear()
-            p = self._plans[key] = ops.ModalPlan(poles, residues)
-        return p
+    def _plan(self, poles, residues, kind="log", build=None):
+        """ModalPlan of (poles, residues), rebuilt when either tensor object or its version changes.  Keyed on the
+        objects themselves (weak references), not on addresses, which the allocator reuses."""
+        h = self._plan_hit
+        if h is not None and h[0]() is poles and h[1] == poles._version and h[2]() is residues \
+                and h[3] == residues._version and h[4] == kind:
+            return h[5]
+        plan = build() if build is not None else ops.ModalPlan(poles, residues)
+        self._plan_hit = (weakref.ref(poles), poles._version, weakref.ref(residues), residues._version, kind, plan)
+        return plan
 
     def parallel_iir(self, z_pre, h, D, L, poles, residues, t, dims, layer_idx, inference_params=None,
                      prefill_style="fft", fftconv_fn=None, padding_mask=None, use_flashfft=False,
@@ -153,17 +185,51 @@ class HyenaInferenceEngine:
                 raise NotImplementedError("long_fir_threshold above 128 taps has no kernel")
             assert h.shape[0] == 1, "batch size must be 1 for long_fir_threshold"
             taps = h[0][:, :T].to(torch.bfloat16).to(torch.float32).contiguous()       # [D, T], bf16-rounded
+            # (bf16(y) + x1v*D) in the tensors' own dtype (engine.py:351-353): bf16 arithmetic with a bf16 D
+            mode = HYENA_BIAS_GATED_BF16 if D.dtype == torch.bfloat16 else HYENA_BIAS_GATED_FP32
             out = ops.fir_fwd_rows(r1, r2, rv, taps, B, hidden, L + pad, T, device=z_pre.device, bias=ops._f32(D),
-                                   bias_mode=HYENA_BIAS_GATED_FP32, taps_reversed=True, force_mfma=True)
+                                   bias_mode=mode, taps_reversed=True, force_mfma=True)
             if pad:
                 out = out[..., pad:]
             return out.permute(0, 2, 1)
-        plan = self._plan(poles, residues)
         want_state = inference_params is not None
+        if want_state and prefill_style == "recurrence":
+            return self._prefill_recurrence(r1, r2, rv, D, poles, residues, B, hidden, L, pad, z_pre.device,
+                                            inference_params, layer_idx)
+        if want_state and prefill_style != "fft":
+            raise NotImplementedError(f"prefill_style {prefill_style!r}")          # engine.py:395-396
+        plan = self._plan(poles, residues)
         out, _, state = ops.li_fwd_rows(r1, r2, rv, plan, D, B, hidden, L + pad, device=z_pre.device,
                                         want_state=want_state)
         if want_state:
             inference_params.state_dict[layer_idx] = state
+        if pad:
+            out = out[..., pad:]
+        return out.permute(0, 2, 1)
+
+    def _prefill_recurrence(self, r1, r2, rv, D, poles, residues, B, hidden, L, pad, device, inference_params,
+                            layer_idx):
+        """prefill_style == "recurrence" (vortex/model/engine.py:314-321, :473-504).  On this branch the reference
+        takes the poles themselves (not their logarithms) and the residues as [D, S, 1, 2] tensors of (re, im)
+        lanes, one filter per channel, and leaves the state as [B, D, S, 2] float32.  The same chunked scan runs it:
+        the recurrence s_t = p s_{t-1} + u_t is what the kernel evaluates anyway.  Deviations, all on the side of
+        the mathematics: the state is carried in float32 (the reference's `0 * x1v_` makes it bf16 and rounds it
+        every step), the complex product is the true one (the reference's in-place lane update feeds the new real
+        lane into the imaginary one), and y = sum_s r_re * s_re as the reference forms it (its `[..., 0]` of the
+        lane-wise product drops r_im * s_im).  With real poles -- the only kind vortex's own parameters give --
+        these coincide with the FFT prefill."""
+        if poles.dim() != 4 or poles.shape[-1] != 2 or residues.shape != poles.shape or poles.shape[0] != hidden:
+            raise ValueError("prefill_style='recurrence' takes poles and residues of shape [D, state, 1, 2] (re, im)")
+        def build():
+            p = torch.view_as_complex(poles.detach()[:, :, 0].to(torch.float32).contiguous())        # [D, S]
+            # log p; a pole of exactly zero gets e^-100, which is zero in float32 from the first power on
+            logp = torch.complex(p.abs().clamp_min(1e-43).log().clamp_min(-100.0), torch.angle(p))
+            res = torch.complex(residues.detach()[:, :, 0, 0].to(torch.float32), torch.zeros_like(p.real))
+            return ops.ModalPlan(logp, res)
+
+        plan = self._plan(poles, residues, "rec", build)
+        out, _, state = ops.li_fwd_rows(r1, r2, rv, plan, D, B, hidden, L + pad, device=device, want_state=True)
+        inference_params.state_dict[layer_idx] = torch.view_as_real(state).contiguous()               # [B, D, S, 2]
         if pad:
             out = out[..., pad:]
         return out.permute(0, 2, 1)
@@ -193,11 +259,11 @@ class HyenaInferenceEngine:
         as torch promotion makes it in the reference."""
         if iir_groups > 1:
             raise NotImplementedError
-        key = (poles.data_ptr(), poles._version)
-        p = self._poles.get(key)
-        if p is None:
-            self._poles.clear()
-            p = self._poles[key] = torch.exp(poles.detach())[..., 0].contiguous()
+        if _same_tensor(self._poles_hit, poles):
+            p = self._poles_hit[2]
+        else:
+            p = torch.exp(poles.detach())[..., 0].contiguous()
+            self._poles_hit = (weakref.ref(poles), poles._version, p)
         if not iir_state.is_contiguous():
             iir_state = iir_state.contiguous()
         y = ops.iir_step(x1, x2, v, iir_state, p, residues.detach(), D, out_dtype=torch.float32)
