@@ -357,7 +357,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
             for (int i = 0; i < N_FRAG; ++i) th[i] = fb[i * 64 + lane];
         }
 #pragma unroll
-        for (int i = 0; i < N_FRAG; ++i) asm volatile("" : "+v"(th[i]));
+        for (int i = 0; i < N_FRAG; ++i) asm volatile("" : "+a"(th[i]));     // fragments live in accumulation registers: only the MFMAs read them
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
             Th[q] = as_bf16x8(th[FR_T + q]);   Tl[q] = as_bf16x8(th[FR_T + 8 + q]);
