@@ -25,8 +25,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0     # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
-# counter reads for the plain copy launch of known size (profiles/bench_default_hbm_traffic.txt).
+# counter reads for the plain copy launch of known size.  These are constants of the committed profile, not
+# measurements of this run: `roofline.traffic_source` names the file they were read from.
 MEASURED_TRAFFIC = {"mr": 2211.99e6, "se": 271.75e6, "li": 8597.09e6}
+TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; copy-probe calibrated)"
 
 
 def parse():
@@ -34,7 +36,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="mr", choices=["mr", "se", "li", "decode", "mr_cl", "mr_layer", "se_layer"])
+    ap.add_argument("--workload", default="mr", choices=["mr", "se", "se_b8", "li", "li_g4096", "decode", "mr_cl", "mr_layer",
+                                                         "se_layer"])
     ap.add_argument("--settle-ms", type=float, default=150.0,
                     help="untimed run of each workload before its warm-up steps, until clocks have settled")
     ap.add_argument("--no-extras", action="store_true")
@@ -80,14 +83,15 @@ class _Synthetic:
 SETTLE_S = 0.15     # set from --settle-ms
 
 
-def time_steps(fn, steps, warmup):
+def time_steps(fn, steps, warmup, settle=None):
     """(wall seconds for `steps` calls, average kernel-side ms per call from HIP events on the launch stream).
 
     Before the `warmup` untimed steps the workload runs for SETTLE_S seconds, also untimed: after lighter work the
     first tens of launches of a bandwidth-heavy kernel run up to 15 % slower (clock and power management settling),
     and a short run would measure that transient instead of the sustained rate."""
-    t_end = time.perf_counter() + SETTLE_S
-    while SETTLE_S > 0 and time.perf_counter() < t_end:
+    settle = SETTLE_S if settle is None else settle
+    t_end = time.perf_counter() + settle
+    while settle > 0 and time.perf_counter() < t_end:
         for _ in range(10):
             fn()
         torch.cuda.synchronize()
@@ -112,8 +116,9 @@ def build_workload(name, device):
     O = _Synthetic
     from vortex_amd import ops
 
-    if name == "se":
-        B, D, L, G, K = 1, 4096, 8192, 256, 7
+    if name in ("se", "se_b8"):
+        # config 1 (268 MB working set: close to the 256 MB last-level cache) and the same rows at batch 8 (2.1 GB)
+        B, D, L, G, K = (1 if name == "se" else 8), 4096, 8192, 256, 7
         x2, x1, v = gates(B, D, L, 1, device)
         h = O.make_se_filter(G, K).reshape(G, K).to(device)
         r1, r2, rv = ops.rows_of(x1), ops.rows_of(x2), ops.rows_of(v)
@@ -132,8 +137,9 @@ def build_workload(name, device):
                                       bias_mode=ops.HYENA_BIAS_GATED_FP32, force_mfma=True, out=out)
         return fn, dict(workload=f"hyena_mr_prefill B={B} L={L} D={D} groups={G} K={K}", tokens=B * L,
                         bytes=8 * B * D * L, kernel="mr_fir_kernel", keep=(x1, x2, v, h, Db, out))
-    if name == "li":
-        B, D, L, G, S = 1, 4096, 262144, 256, 16
+    if name in ("li", "li_g4096"):
+        # config 3, and the same rows with one filter per channel (vortex's own hcl_filter_groups == hidden_size)
+        B, D, L, G, S = 1, 4096, 262144, (256 if name == "li" else 4096), 16
         x2, x1, v = gates(B, D, L, 4, device)
         lp, r = O.make_modal_complex(G, S)
         Db = torch.randn(D, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).to(device)
@@ -194,9 +200,20 @@ def decode_layer_set(D, device, steps, warmup):
     wall, ms = time_steps(fn, steps, warmup)
     # algorithmic bytes: caches read once, one ring slot written per FIR, modal state read+written,
     # 3 gate vectors in and 1 output vector out per operator
-    byts = B * D * 2 * (6 + 127) + 2 * B * D * 2 + 2 * state.numel() * 8 + 3 * 4 * B * D * 2
+    gates_io = 4 * B * D * 2
+    b_se, b_mr, b_li = B * D * 2 * 6 + B * D * 2 + gates_io, B * D * 2 * 127 + B * D * 2 + gates_io, \
+        2 * state.numel() * 8 + gates_io
+    byts = b_se + b_mr + b_li
+    # each step alone, launched back to back: kernels shorter than a launch (about 6 us from Python) read as the
+    # launch rate, so `launch_bound` marks figures that are an upper bound of the kernel's own duration
+    per = {}
+    for nm, st, xx, bb in (("se_step", step.se, x[0], b_se), ("mr_step", step.mr, x[1], b_mr), ("iir_step", step.li, x[2], b_li)):
+        o = step.out[0]
+        _, kms = time_steps(lambda: st(xx[1], xx[0], xx[2], o), max(steps, 100), warmup)
+        per[nm] = dict(us=kms * 1e3, bytes=bb, hbm_gbs=bb / (kms * 1e-3) / 1e9, frac=bb / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                       launch_bound=kms * 1e3 < 10.0)
     return dict(us_per_step=ms * 1e3, wall_us_per_step=wall / steps * 1e6, bytes=byts,
-                hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
+                hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, kernels=per)
 
 
 def decode_layers_from_projection(D, device, steps, warmup):
@@ -348,10 +365,14 @@ def main():
 
     def run(name, steps, warmup):
         fn, d = build_workload(name, device)
+        # cold: the first `steps` launches after `warmup`, with no settle phase (what a short run of this workload
+        # after other work sees); then the settled, sustained figure
+        _, cold_ms = time_steps(fn, steps, warmup, settle=0.0)
         wall, ms = time_steps(fn, steps, warmup)
         d.pop("keep")
         d.update(wall_s=wall, kernel_ms=ms, tokens_per_s=d["tokens"] * steps / wall,
-                 hbm_gbs=d["bytes"] / (ms * 1e-3) / 1e9)
+                 hbm_gbs=d["bytes"] / (ms * 1e-3) / 1e9, cold_kernel_ms=cold_ms,
+                 cold_frac=d["bytes"] / (cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
         torch.cuda.empty_cache()
         return d
 
@@ -378,25 +399,27 @@ def main():
         "config": {"workload": m["workload"], "settle_ms": args.settle_ms},
         "roofline": {"bound": "hbm", "achieved": m["hbm_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": m["hbm_gbs"] / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(main_name),
+                     "traffic_source": TRAFFIC_SOURCE if MEASURED_TRAFFIC.get(main_name) else None,
                      "kernel": m["kernel"],
-                     "algorithmic_bytes_per_launch": m["bytes"], "kernel_ms": m["kernel_ms"]},
+                     "algorithmic_bytes_per_launch": m["bytes"], "kernel_ms": m["kernel_ms"],
+                     "cold": {"kernel_ms": m["cold_kernel_ms"], "frac": m["cold_frac"],
+                              "what": f"first {args.steps} launches after {args.warmup} warm-up launches, no settle phase"}},
     }
     if not args.no_extras:
         extra = {}
         extra_warmup = args.warmup
-        for name in ("se", "mr", "li"):
+        def entry(e):
+            return {"workload": e["workload"], "tokens_per_s": e["tokens_per_s"], "kernel_us": e["kernel_ms"] * 1e3,
+                    "hbm_gbs": e["hbm_gbs"], "roofline_frac": e["hbm_gbs"] / HBM_PEAK_GBS,
+                    "cold_kernel_us": e["cold_kernel_ms"] * 1e3, "cold_roofline_frac": e["cold_frac"]}
+
+        for name in ("se", "se_b8", "mr", "li", "li_g4096"):
             if name == main_name:
                 continue
-            steps = max(3, min(args.steps, 20 if name == "li" else args.steps))
-            e = run(name, steps, extra_warmup)
-            extra[name] = {"workload": e["workload"], "tokens_per_s": e["tokens_per_s"],
-                           "kernel_us": e["kernel_ms"] * 1e3, "hbm_gbs": e["hbm_gbs"],
-                           "roofline_frac": e["hbm_gbs"] / HBM_PEAK_GBS}
+            steps = max(3, min(args.steps, 20 if name.startswith("li") else args.steps))
+            extra[name] = entry(run(name, steps, extra_warmup))
         for name in ("mr_cl", "mr_layer", "se_layer"):
-            e = run(name, max(3, min(args.steps, 20)), extra_warmup)
-            extra[name] = {"workload": e["workload"], "tokens_per_s": e["tokens_per_s"],
-                           "kernel_us": e["kernel_ms"] * 1e3, "hbm_gbs": e["hbm_gbs"],
-                           "roofline_frac": e["hbm_gbs"] / HBM_PEAK_GBS}
+            extra[name] = entry(run(name, max(3, min(args.steps, 20)), extra_warmup))
         for D in (4096, 8192):
             extra[f"decode_D{D}"] = decode_layer_set(D, device, max(args.steps, 50), max(args.warmup, 5))
         extra["decode_from_projection_D4096"] = decode_layers_from_projection(4096, device, max(args.steps, 50),
