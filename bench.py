@@ -45,6 +45,9 @@ def parse():
     ap.add_argument("--no-model", action="store_true", help="skip the end-to-end model prefill legs")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 1 GiB device copy (calibration of FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--pattern-probes", action="store_true",
+                    help="also stream the bytes of the Hyena-LI configuration with no arithmetic in several access "
+                         "orders (whole rows, independent segments) and print what each delivers to stderr")
     return ap.parse_args()
 
 
@@ -387,6 +390,23 @@ def main():
         print(f"copy probe (copy_probe_kernel, 16 B/lane): 1 GiB read + 1 GiB written per launch, "
               f"{ms * 1e3:.1f} us, {2 * nbytes / (ms * 1e-3) / 1e9:.0f} GB/s", file=sys.stderr)
         del a, b
+        torch.cuda.empty_cache()
+
+    if args.pattern_probes:
+        from vortex_amd import _lib
+        D, L = 4096, 262144
+        t = [torch.empty(D, L, dtype=torch.bfloat16, device=device).normal_() for _ in range(3)]
+        o = torch.empty(D, L, dtype=torch.bfloat16, device=device)
+        probe, stream = _lib.stream_probe(), torch.cuda.current_stream().cuda_stream
+        print(f"access-pattern probes: {D} rows of {L} bf16 samples, 3 reads + 1 write, no arithmetic", file=sys.stderr)
+        cases = [("whole rows, one block per 4 rows (a one-pass scan)", 0, 0)]
+        cases += [(f"independent segments of {s} samples, row sets in order", 1, s) for s in (65536, 16384, 8192, 4096, 2048)]
+        for what, pat, seg in cases:
+            fn = lambda: _lib.check(probe(t[0].data_ptr(), t[1].data_ptr(), t[2].data_ptr(), o.data_ptr(), D, L, pat, seg,
+                                          stream), "stream probe")
+            _, ms = time_steps(fn, 5, 2)
+            print(f"  {what:75s} {ms * 1e3:8.1f} us {8 * D * L / (ms * 1e-3) / 1e9:7.0f} GB/s", file=sys.stderr)
+        del t, o
         torch.cuda.empty_cache()
 
     main_name = args.workload if args.workload != "decode" else "mr"
