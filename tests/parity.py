@@ -65,3 +65,18 @@ def assert_gated_close(got, ref, z_ref, x2, S, eps_acc, ulps_z=1.0, gate_ulps=0.
                         f"{ratio:.2f} at {tuple(int(i) for i in (err / bound).argmax().unsqueeze(0))}; "
                         f"{off2} elements differ by more than 2 bf16 ulps of the pre-gate value")
     return ratio
+
+
+def log_uniform_modal(G, S, cplx, seed, pmin=0.05, pmax=0.9999):
+    """Modal parameters with log-uniform |p| in [pmin, pmax]: slow poles as in the benchmark configurations and the
+    fast-decaying ones a trained or randn-initialised log_poles parameter (vortex/model/model.py:202) also holds.
+    Returns (log_poles [G, S, 1], residues [G, S]), complex64 or float32."""
+    import math
+    g = torch.Generator().manual_seed(seed)
+    lm = math.log(pmin) + (math.log(pmax) - math.log(pmin)) * torch.rand(G, S, generator=g, dtype=torch.float64)
+    if cplx:
+        ang = math.pi * torch.rand(G, S, generator=g, dtype=torch.float64)
+        lp = torch.complex(lm, ang).to(torch.complex64)[..., None]
+        r = (torch.complex(torch.randn(G, S, generator=g), torch.randn(G, S, generator=g)) / 2 ** 0.5).to(torch.complex64)
+        return lp, r
+    return lm.to(torch.float32)[..., None], torch.randn(G, S, generator=g)

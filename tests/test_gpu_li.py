@@ -197,18 +197,8 @@ def test_li_cooperative_form(L, cplx, override):
 
 
 def _fast_modal(G, S, cplx, seed, pmin=0.05, pmax=0.9):
-    """Poles with log-uniform |p| in [pmin, pmax]: the fast-decaying range a trained or randn-initialised
-    log_poles parameter (vortex/model/model.py:202) also covers."""
-    g = torch.Generator().manual_seed(seed)
-    import math
-    lm = math.log(pmin) + (math.log(pmax) - math.log(pmin)) * torch.rand(G, S, generator=g, dtype=torch.float64)
-    if cplx:
-        ang = math.pi * torch.rand(G, S, generator=g, dtype=torch.float64)
-        lp = torch.complex(lm, ang).to(torch.complex64)[..., None]
-        r = (torch.complex(torch.randn(G, S, generator=g), torch.randn(G, S, generator=g)) / 2 ** 0.5).to(torch.complex64)
-    else:
-        lp, r = lm.to(torch.float32)[..., None], torch.randn(G, S, generator=g)
-    return lp, r
+    from parity import log_uniform_modal
+    return log_uniform_modal(G, S, cplx, seed, pmin, pmax)
 
 
 @pytest.mark.parametrize("form", ["lone", "coop", "cpw1"])

@@ -72,15 +72,24 @@ def test_li_random(B, L, seed, coop, override):
         k = 8 // (D & -D) if (D & -D) < 8 else 1
         D, G = D * k, G * k
     x2, x1, v = O.make_gates(B, D, L, seed=seed)
-    lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(G, S, seed=seed + 1)
+    # poles from the whole range a checkpoint can hold: log-uniform |p| in [0.05, 0.9999]
+    from parity import log_uniform_modal
+    lp, r = log_uniform_modal(G, S, cplx, seed + 1)
     Db = torch.randn(D, generator=torch.Generator().manual_seed(seed)).bfloat16()
+    x2n, x1n, vn = (torch.randn(B, D, generator=torch.Generator().manual_seed(seed + 2 + i)).bfloat16() for i in range(3))
+    cat = lambda t, n: torch.cat([t, n[..., None]], -1)
+    full, _, _ = O.li_prefill(cat(x2, x2n), cat(x1, x1n), cat(v, vn), lp, r, Db, want_state=False)
     ref, y32_ref, st_ref = O.li_prefill(x2, x1, v, lp, r, Db)
     out, y32, st = va.hyena_li_fwd(x1.cuda(), x2.cuda(), v.cuda(), lp.cuda(), r.cuda(), Db.cuda(),
                                    want_state=True, want_fp32=True)
     assert rel_err(y32, y32_ref) <= 1e-4, (B, D, L, G, cplx, S)
     assert rel_err(out, ref) <= 2e-2
     sr = torch.view_as_real(st) if cplx else st
+    assert torch.isfinite(sr).all()
     assert rel_err(sr, torch.view_as_real(st_ref) if cplx else st_ref) <= 1e-4
+    if S & (S - 1) == 0:          # one decode token from the emitted state = position L of a longer prefill
+        y = va.iir_step(x1n.cuda(), x2n.cuda(), vn.cuda(), st, torch.exp(lp[..., 0]).cuda(), r.cuda(), Db.cuda())
+        assert rel_err(y, full[..., L]) <= 2e-2
 
 
 @pytest.mark.parametrize("B,L,seed", cases(4, 8))
