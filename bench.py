@@ -45,6 +45,8 @@ def parse():
     ap.add_argument("--no-model", action="store_true", help="skip the end-to-end model prefill legs")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 1 GiB device copy (calibration of FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--li-cached-inputs", action="store_true",
+                    help="also time Hyena-LI at config 3 with its reads served from cache (the kernel's own pace)")
     ap.add_argument("--pattern-probes", action="store_true",
                     help="also stream the bytes of the Hyena-LI configuration with no arithmetic in several access "
                          "orders (whole rows, independent segments) and print what each delivers to stderr")
@@ -407,6 +409,27 @@ def main():
             _, ms = time_steps(fn, 5, 2)
             print(f"  {what:75s} {ms * 1e3:8.1f} us {8 * D * L / (ms * 1e-3) / 1e9:7.0f} GB/s", file=sys.stderr)
         del t, o
+        torch.cuda.empty_cache()
+
+    if args.li_cached_inputs:
+        # Hyena-LI at config 3 with every channel reading the same 16 rows (a row descriptor with row stride L and
+        # batch stride 0 over a 16-row tensor): the reads are served from cache, the 2.1 GB of output is still written.
+        # What is left is the kernel's own pace plus the write stream.
+        import vortex_amd as va
+        from vortex_amd import ops
+        from vortex_amd._lib import Rows
+        B, D, L, G = 1, 4096, 262144, 256
+        small = [torch.randn(16, L, device=device).to(torch.bfloat16) for _ in range(3)]
+        lp, r = _Synthetic.make_modal_complex(G, 16)
+        plan = va.ModalPlan(lp.to(device), r.to(device))
+        Db = torch.randn(D).to(torch.bfloat16).to(device)
+        out = torch.empty(B, D, L, dtype=torch.bfloat16, device=device)
+        rows = [Rows(t.data_ptr(), 0, L, 16, 0) for t in small]            # channel d -> row d % 16
+        full = gates(B, D, L, 4, device)
+        for what, rr in (("inputs from HBM", [ops.rows_of(t) for t in (full[1], full[0], full[2])]), ("inputs cached", rows)):
+            _, ms = time_steps(lambda: ops.li_fwd_rows(rr[0], rr[1], rr[2], plan, Db, B, D, L, device=device, out=out), 10, 3)
+            print(f"hyena_li_fwd config 3, {what}: {ms * 1e3:.1f} us", file=sys.stderr)
+        del small, full, out
         torch.cuda.empty_cache()
 
     main_name = args.workload if args.workload != "decode" else "mr"
