@@ -59,7 +59,7 @@ const char* hyena_last_error_string(void);
  * those choices process-wide until it is reset with a negative value.  Nothing is read from the environment.
  *   "mr_nseg", "cl_nseg", "li_nseg"            segments along L of hyena_mr_fwd, hyena_fir_cl_fwd / layer_fwd, hyena_li_fwd
  *   "se_nt", "mr_nt", "li_nt", "cl_nt"         0 = cached, 1 = non-temporal global accesses
- *   "li_cpw"                                    1 = one channel per wavefront in hyena_li_fwd
+ *   "li_cpw"                                    1 / 4 = channels per wavefront in hyena_li_fwd (4 needs D/G % 4 == 0)
  *   "li_coop"                                   0 / 1 = lone / cooperating wavefronts in hyena_li_fwd
  * Returns 0, or HYENA_EINVAL for an unknown name. */
 int hyena_set_launch_override(const char* name, int64_t value);

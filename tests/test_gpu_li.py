@@ -27,7 +27,12 @@ def rel_err(a, b):
     (1, 6, 2600, 6, True),         # one filter per channel, complex poles, ragged length
     (1, 8, 1024, 4, True),         # two channels per group
 ])
-def test_li_vs_oracle(B, D, L, G, cplx):
+@pytest.mark.parametrize("form", ["auto", "lone4", "coop4", "cpw1"])
+def test_li_vs_oracle(B, D, L, G, cplx, form, override):
+    # the launcher picks the work decomposition from the shape (auto); the other cases pin each of the three forms
+    if form in ("lone4", "coop4") and (D // G) % 4:
+        pytest.skip("four channels per wavefront need groups of a multiple of four channels")
+    override(**{"auto": {}, "lone4": dict(li_cpw=4, li_coop=0), "coop4": dict(li_cpw=4, li_coop=1), "cpw1": dict(li_cpw=1)}[form])
     x2, x1, v = O.make_gates(B, D, L, seed=L + D)
     lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(G, 16, seed=L)
     Db = torch.randn(D, generator=torch.Generator().manual_seed(1)).bfloat16()
@@ -172,9 +177,9 @@ def test_million_token_rows():
 @pytest.mark.parametrize("L", [65536 + 520, 2048 * 5 + 8, 2048 * 3, 1544, 8])
 @pytest.mark.parametrize("cplx", [True, False])
 def test_li_cooperative_form(L, cplx, override):
-    # rows of 65536 samples and more in shared-filter groups run with the four wavefronts of a block on consecutive
-    # pieces of the same channels and the modal state handed across through LDS.  Forced on here for short and ragged
-    # rows too (last steps with idle wavefronts, the final state in any of the four pieces): against the oracle,
+    # problems with too few channels to fill the chip run with the four wavefronts of a block on consecutive
+    # pieces of the same channels and the modal state handed across through LDS.  Forced on here for long, short and
+    # ragged rows (last steps with idle wavefronts, the final state in any of the four pieces): against the oracle,
     # and against the one-wavefront form for the same inputs.
     B, D, G = 2, 16, 2
     x2, x1, v = O.make_gates(B, D, L, seed=L)
@@ -183,7 +188,7 @@ def test_li_cooperative_form(L, cplx, override):
     ref, y32_ref, st_ref = O.li_prefill(x2, x1, v, lp, r, Db)
     res = {}
     for coop in ("1", "0"):
-        override(li_coop=int(coop))
+        override(li_cpw=4, li_coop=int(coop))
         res[coop] = va.hyena_li_fwd(x1.cuda(), x2.cuda(), v.cuda(), lp.cuda(), r.cuda(), Db.cuda(),
                                     want_state=True, want_fp32=True)
         out, y32, st = res[coop]
@@ -212,9 +217,9 @@ def test_li_state_with_fast_poles_and_ragged_length(tail, cplx, form, override):
     D = 16 if form != "cpw1" else 8
     L = 2048 + 512 + (128 - tail) % 128 + (0 if tail else 128)
     if form == "coop":
-        override(li_coop=1)
+        override(li_cpw=4, li_coop=1)
     elif form == "lone":
-        override(li_coop=0)
+        override(li_cpw=4, li_coop=0)
     else:
         override(li_cpw=1)
     x2, x1, v = O.make_gates(B, D, L + 1, seed=tail + 1)

@@ -746,13 +746,17 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
     if (pre != post) return hyena_fail(HYENA_ENOSUP, "%s: pass both v and x2 or neither", who);
     if (B == 0 || L == 0) return 0;
-    int cpw = ((D / G) % 4 == 0) ? 4 : 1;                    // channels per wavefront (they share one filter)
-    if (hyena_override(HYENA_OV_LI_CPW) == 1) cpw = 1;
+    // Work decomposition (measured on B*D = 1024 .. 8192 rows, L = 8192 .. 524288):
+    //  * rows of 65536 samples or more: one channel per wavefront, 2048 samples per step.  A wavefront then reads
+    //    4 KiB of its row in one go, which the memory system serves 4-9 % faster than four rows 1 KiB at a time.
+    //  * shorter rows: four channels of one filter per wavefront, 512 samples per step (a quarter of the scan
+    //    links and fragment builds) - as lone wavefronts when there are enough of them to fill the chip, in the
+    //    cooperative form (one block per four channels, four times as many blocks) when there are not.
+    const bool can4 = (D / G) % 4 == 0;
+    int cpw = (can4 && L < 65536) ? 4 : 1;                   // channels per wavefront (they share one filter)
+    { const int64_t x = hyena_override(HYENA_OV_LI_CPW); if (x == 1) cpw = 1; else if (x == 4 && can4) cpw = 4; }
     const int64_t nquads = B * (D / cpw);
-    // Long rows of shared-filter channels go to the cooperative form (one block per work item): measured 6 %, 14 %
-    // and 2 % faster at L = 65536, 131072 and 262144, slower below (the block's waves start and end together).
-    // One channel per wavefront gains nothing from it: there the per-step scan, not the row pattern, sets the pace.
-    bool coop = cpw == 4 && L >= 65536;
+    bool coop = cpw == 4 && nquads <= 512;
     { const int64_t x = hyena_override(HYENA_OV_LI_COOP); if (x >= 0) coop = cpw == 4 && x != 0; }
     const int64_t nblk = coop ? nquads : (nquads + 3) / 4;
     if (nquads > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: problem too large for one launch", who);
