@@ -67,19 +67,23 @@ def test_new_entry_points_validate_before_touching_the_device():
     pj = _lib.ProjFwd(P, 192, 192, P, None, 3, 0, 64, 0, 80, 1)
     assert L.hyena_fir_layer_fwd(ref(pj), P, 0, None, 0, P, None, 0, 1, 8, 64, 4, 7, None) == -1      # map past 3D
     ps = _lib.ProjStep(P, 192, P, 0, 0, P, None, 64, 0, 64, 1, 0)
-    assert L.hyena_fir_layer_step(ref(ps), P, 6, 0, P, None, 0, P, 64, 1, 64, 4, None) == -1          # empty cache
+    assert L.hyena_fir_layer_step(ref(ps), P, 6, 64, 0, P, None, 0, P, 64, 1, 64, 4, None) == -1          # empty cache
     ps = _lib.ProjStep(P, 192, P, 2, 0, P, None, 4, 12, 4, 1, 0)
-    assert L.hyena_fir_layer_step(ref(ps), P, 6, 0, P, None, 0, P, 64, 1, 64, 4, None) == -3          # head_dim 4
+    assert L.hyena_fir_layer_step(ref(ps), P, 6, 64, 0, P, None, 0, P, 64, 1, 64, 4, None) == -3          # head_dim 4
     assert L.hyena_iir_layer_step(None, P, P, P, 0, P, 0, P, 0, 64, 1, 64, 64, 16, None) == -1
     # ring positions in device memory: the pointer is required, and a position on the device lifts the host range check
-    assert L.hyena_fir_step_dpos(P, None, None, 64, P, 6, None, P, None, 0, P, 64, 1, 64, 4, None) == -1
-    assert L.hyena_fir_layer_step_dpos(ref(ps), P, 6, None, P, None, 0, P, 64, 1, 64, 4, None) == -1
+    assert L.hyena_fir_step_dpos(P, None, None, 64, P, 6, 64, None, P, None, 0, P, 64, 1, 64, 4, None) == -1
+    assert L.hyena_fir_layer_step_dpos(ref(ps), P, 6, 64, None, P, None, 0, P, 64, 1, 64, 4, None) == -1
+    # cache layout: the channel block is D or a multiple of 512 that divides D
+    assert L.hyena_fir_step_dpos(P, None, None, 1024, P, 6, 256, P, P, None, 0, P, 1024, 1, 1024, 64, None) == -1
+    assert L.hyena_fir_step_dpos(P, None, None, 1536, P, 6, 1024, P, P, None, 0, P, 1536, 1, 1536, 96, None) == -1
+    assert L.hyena_fir_step_dpos(P, None, None, 1536, P, 6, 512, P, P, None, 0, P, 1536, 0, 1536, 96, None) == 0
     assert L.hyena_ring_advance(None, P, 4, None) == -1 and L.hyena_ring_advance(P, P, -1, None) == -1
     assert L.hyena_ring_advance(P, P, 0, None) == 0
     ps = _lib.ProjStep(P, 192, P, 2, 5, P, None, 64, 0, 64, 1, 0, None)
-    assert L.hyena_fir_layer_step(ref(ps), P, 6, 0, P, None, 0, P, 64, 0, 64, 4, None) == -1           # pos 5 of 2
+    assert L.hyena_fir_layer_step(ref(ps), P, 6, 64, 0, P, None, 0, P, 64, 0, 64, 4, None) == -1           # pos 5 of 2
     ps = _lib.ProjStep(P, 192, P, 2, 5, P, None, 64, 0, 64, 1, 0, P)
-    assert L.hyena_fir_layer_step(ref(ps), P, 6, 0, P, None, 0, P, 64, 0, 64, 4, None) == 0            # B = 0: no launch
+    assert L.hyena_fir_layer_step(ref(ps), P, 6, 64, 0, P, None, 0, P, 64, 0, 64, 4, None) == 0            # B = 0: no launch
     # modal state sizes
     assert L.hyena_li_plan_bytes(4, 16) == L.hyena_li_plan_bytes(4, 2) == 4 * 1536 * 4
     assert L.hyena_li_plan_bytes(4, 17) == 0 and L.hyena_li_plan_bytes(4, 0) == 0

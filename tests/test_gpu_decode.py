@@ -64,6 +64,36 @@ def test_fir_step_sequence_vs_oracle(B, D, G, K, flip, gated):
             assert torch.equal(ring.reference_order().cpu(), ref_state)
 
 
+@pytest.mark.parametrize("D,blocks", [(1536, (1536, 512)), (2048, (2048, 512, 1024)), (4096, (4096, None))])
+def test_fir_step_channel_blocked_cache(D, blocks):
+    """The cache layouts [B, D/block, R, block] hold the same ring: outputs and contents are bit-equal to the plain
+    [B, R, D] cache (block = D) over more steps than the ring has slots, and the plain one matches the oracle."""
+    B, G, K = 3, D // 16, 128
+    R = K - 1
+    g = torch.Generator().manual_seed(D)
+    w = torch.randn(G, 1, K, generator=g) / K ** 0.5
+    bias = torch.randn(D, generator=g)
+    st = torch.randn(B, D, R, generator=g).bfloat16()
+    rings = [va.FirRing.from_reference(st.cuda(), block=b) for b in blocks]
+    assert rings[0].block == D and all(r.block == 512 for r in rings[1:2])
+    assert all(torch.equal(r.reference_order().cpu(), st.float()) for r in rings)
+    taps = eff_taps(w, R, True).cuda()
+    ref_state = st
+    for step in range(R + 4):
+        x1, x2, v = (torch.randn(B, D, generator=g).bfloat16() for _ in range(3))
+        ys = [va.fir_step(x1.cuda(), r, taps, x2=x2.cuda(), v=v.cuda(), bias=bias.cuda(), gated_bias=True) for r in rings]
+        assert all(torch.equal(ys[0], y) for y in ys[1:]), step
+        if step in (0, 5, R - 1, R + 3):
+            y_ref, ref_state = O.step_fir(x1 * v, ref_state, w.repeat_interleave(16, 0), bias=bias, gated_bias=True,
+                                          flip_filter=True)
+            y_ref = (y_ref * x2).float()
+            assert (ys[0].float().cpu() - y_ref).abs().max() <= 2e-2 * y_ref.abs().max()
+            assert all(torch.equal(r.reference_order().cpu(), ref_state) for r in rings), step
+        else:
+            _, ref_state = O.step_fir(x1 * v, ref_state, w.repeat_interleave(16, 0), bias=bias, gated_bias=True,
+                                      flip_filter=True)
+
+
 @pytest.mark.parametrize("name", ["real_bf16D", "real_f32D", "cplx_f32D"])
 def test_iir_step_golden(name):
     x2, x1, v = (torch.from_numpy(GOLD[f"iir_{name}_{k}"]).bfloat16().cuda() for k in ("x2", "x1", "v"))

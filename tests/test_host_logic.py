@@ -55,7 +55,7 @@ def test_fir_ring_reference_order_and_rotation():
     # emulate two steps: the oldest slot is overwritten, then the oldest moves on
     for step in range(2):
         new = torch.full((B, D), 100.0 + step)
-        ring.buf[:, ring.pos] = new.bfloat16()
+        ring.slots()[:, ring.pos] = new.bfloat16()        # block = D: slots() is a view of the cache
         ring.pos = (ring.pos + 1) % R
         st = torch.cat([st[..., 1:], new[..., None]], dim=-1)
         assert torch.equal(ring.reference_order(), st)

@@ -62,7 +62,7 @@ def lib():
                                c_int, c_void_p]
     L.hyena_mr_fwd.argtypes = [R, R, R, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64,
                                c_int64, c_int, c_void_p]
-    L.hyena_fir_step.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p,
+    L.hyena_fir_step.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p,
                                  c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p]
     L.hyena_iir_step.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int,
                                  c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int64,
@@ -77,13 +77,13 @@ def lib():
                                        c_int64, c_int64, c_int64, c_int, c_int, c_void_p]
     L.hyena_set_launch_override.argtypes = [c_char_p, c_int64]
     P = POINTER(ProjStep)
-    L.hyena_fir_layer_step.argtypes = [P, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int64,
+    L.hyena_fir_layer_step.argtypes = [P, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int64,
                                        c_int64, c_int64, c_int64, c_void_p]
     L.hyena_iir_layer_step.argtypes = [P, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                                        c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p]
-    L.hyena_fir_step_dpos.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p,
+    L.hyena_fir_step_dpos.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p,
                                       c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p]
-    L.hyena_fir_layer_step_dpos.argtypes = [P, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+    L.hyena_fir_layer_step_dpos.argtypes = [P, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                             c_int64, c_int64, c_int64, c_int64, c_void_p]
     L.hyena_ring_advance.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
     C = POINTER(Cl)

@@ -389,7 +389,7 @@ class HyenaCascade(nn.Module):
         d = self._decode_plan(inference_params)
         B = u.shape[0]
         rings = [d["ring"]] + ([d["inner"].ring] if self.fir_inner_filter_length else [])
-        if any(getattr(r, "valid", r.buf.shape[1]) < r.buf.shape[1] for r in rings):
+        if any(getattr(r, "valid", r.R) < r.R for r in rings):
             return self._growing_step(u, d), inference_params
         if self.fuse_decode and d["layer"] is not None and u.stride(1) == 1 and u.stride(0) % 8 == 0 and u.data_ptr() % 16 == 0:
             y = torch.empty(B, self.hidden_size, dtype=torch.bfloat16, device=u.device)

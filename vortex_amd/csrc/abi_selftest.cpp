@@ -98,7 +98,7 @@ int main(int argc, char** argv) {
         std::vector<uint16_t> hist = ring;      // host model of the ring contents
         for (int step = 0; step < 2; ++step) {
             const int64_t p = step;             // oldest slot
-            int rc = p_hyena_fir_step(d_u, d_1, d_1, Ds, d_ring, R, p, d_w, nullptr, HYENA_BIAS_NONE, d_y, Ds, Bs, Ds, Ds, stream);
+            int rc = p_hyena_fir_step(d_u, d_1, d_1, Ds, d_ring, R, Ds, p, d_w, nullptr, HYENA_BIAS_NONE, d_y, Ds, Bs, Ds, Ds, stream);
             CHECK(rc == 0, "hyena_fir_step rc=%d: %s", rc, p_hyena_last_error_string());
             HIP_OK(hipStreamSynchronize(stream));
             auto y = host(d_y, (size_t)(Bs * Ds));
@@ -122,7 +122,7 @@ int main(int argc, char** argv) {
             const int64_t p = step % R;
             for (size_t i = 0; i < u.size(); ++i) u[i] = to_bf16((float)((int)((i + 3 * step) % 9) - 4) / 2.f);
             HIP_OK(hipMemcpy(d_u, u.data(), u.size() * 2, hipMemcpyHostToDevice));
-            int rc = p_hyena_fir_step_dpos(d_u, d_1, d_1, Ds, d_ring, R, d_pos, d_w, nullptr, HYENA_BIAS_NONE, d_y, Ds, Bs, Ds, Ds, stream);
+            int rc = p_hyena_fir_step_dpos(d_u, d_1, d_1, Ds, d_ring, R, Ds, d_pos, d_w, nullptr, HYENA_BIAS_NONE, d_y, Ds, Bs, Ds, Ds, stream);
             CHECK(rc == 0, "hyena_fir_step_dpos rc=%d: %s", rc, p_hyena_last_error_string());
             rc = p_hyena_ring_advance(d_pos, d_depth, 2, stream);
             CHECK(rc == 0, "hyena_ring_advance rc=%d: %s", rc, p_hyena_last_error_string());

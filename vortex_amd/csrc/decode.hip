@@ -74,13 +74,14 @@ __device__ __forceinline__ void proj_store8(const ProjArgs& pj, int64_t b, uint3
 // Block = NSG wavefronts over the same 512 channels; wavefront sg handles cache
 // slots sg, sg+NSG, ... so every load instruction reads 1 KiB of one slot row.
 // NSG = 8 for deep caches (enough loads in flight to cover HBM latency), 2 for shallow ones.
-// Ring layout [B][R][D]: channels contiguous, so the slot written back is one
-// coalesced row per batch element.
+// Ring layout [B][D/cb][R][cb] with cb = D (plain [B][R][D]) or a multiple of 512: channels contiguous, so the
+// slot written back is one coalesced row per batch element and channel block.  With cb = 512 the R slots a block
+// reads are one contiguous run of R KiB instead of 1 KiB pieces 2*D bytes apart, which deep caches stream faster.
 // FEAT != 0: the gates come from the fused featurizer step (ProjArgs) instead of x1, x2, v.
 template <bool PRE, bool POST, int BIAS, bool GROUPED, int NSG, int FEAT>
 __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __restrict__ x1, const bf16_t* __restrict__ x2,
                                                        const bf16_t* __restrict__ v, int64_t in_bs, ProjArgs pj,
-                                                       bf16_t* __restrict__ ring, int R, int pos,
+                                                       bf16_t* __restrict__ ring, int R, int cb, int pos,
                                                        const int* __restrict__ pos_dev,
                                                        const float* __restrict__ w, const float* __restrict__ bias,
                                                        bf16_t* __restrict__ out, int64_t out_bs, int64_t D, int dg) {
@@ -100,7 +101,10 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
     float* zs = red + (NSG - 1) * 512;            // [3][512] gates of the block's channels (fused featurizer only)
     const int gl = GROUPED ? (oc * 8) / dg : 0;
     constexpr int UF = 8;                   // cache slots in flight per lane
-    const bf16_t* rb = ring + (b * R) * D + d0;
+    // ring [B][D/cb][R][cb]: the block's 512 channels lie inside one channel block (cb = D is the plain [B][R][D])
+    const uint32_t cblk = (uint32_t)d0 / (uint32_t)cb;
+    const int64_t roff = ((b * (int64_t)((uint32_t)D / (uint32_t)cb) + cblk) * R) * cb + (d0 - (int64_t)cblk * cb);
+    const bf16_t* rb = ring + roff;
     const u32x4 zero4 = {0, 0, 0, 0};
 
     auto load_batch = [&](int i, u32x4* q) {
@@ -109,7 +113,7 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
             const int ii = i + NSG * k;
             int s = pos + ii;
             if (s >= R) s -= R;
-            q[k] = (live && ii < R) ? *(const u32x4*)(rb + (int64_t)s * D) : zero4;
+            q[k] = (live && ii < R) ? *(const u32x4*)(rb + (int64_t)s * cb) : zero4;
         }
     };
     float acc[8];
@@ -237,7 +241,7 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
     const u32x4 ov = {o[0], o[1], o[2], o[3]};
     *(u32x4*)(out + b * out_bs + d0) = ov;
     const u32x4 uv = {up[0], up[1], up[2], up[3]};
-    *(u32x4*)(ring + (b * R + pos) * D + d0) = uv;
+    *(u32x4*)(ring + roff + (int64_t)pos * cb) = uv;
 }
 
 // ---------------------------------------------------------------- IIR step
@@ -427,7 +431,7 @@ static int proj_vector_mode(const hyena_proj_step* p, int64_t D) {
 }
 
 static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_t in_bs, const hyena_proj_step* proj,
-                           void* ring, int64_t R, int64_t pos, const int32_t* pos_dev, const float* w, const float* bias,
+                           void* ring, int64_t R, int64_t cb, int64_t pos, const int32_t* pos_dev, const float* w, const float* bias,
                            int bias_mode, void* out, int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream,
                            const char* who) {
     if ((!proj && !x1) || !ring || !w || !out) return hyena_fail(HYENA_EINVAL, "%s: x1, ring, w, out are required", who);
@@ -435,6 +439,10 @@ static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_
     if (B < 0 || D <= 0 || G <= 0 || D % G != 0 || R < 1 || R > 4096 || pos < 0 || pos >= R)
         return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld G=%lld R=%lld pos=%lld", who, (long long)B,
                           (long long)D, (long long)G, (long long)R, (long long)pos);
+    if (cb != D && (cb <= 0 || cb % 512 != 0 || D % cb != 0))
+        return hyena_fail(HYENA_EINVAL, "%s: ring_block %lld must be D or a multiple of 512 that divides D=%lld", who,
+                          (long long)cb, (long long)D);
+    if (D >= (1LL << 31)) return hyena_fail(HYENA_EINVAL, "%s: D too large", who);
     if (bias_mode < 0 || bias_mode > 2 || (bias_mode != HYENA_BIAS_NONE && !bias))
         return hyena_fail(HYENA_EINVAL, "%s: bias_mode %d needs a bias pointer", who, bias_mode);
     if (D % 8 != 0 || in_bs % 8 != 0 || out_bs % 8 != 0 || ((uintptr_t)x1 & 15) || ((uintptr_t)ring & 15) ||
@@ -465,7 +473,7 @@ static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_
     bool ok = false;
 #define FS_GO(P, Q, M, GR, N, F)                                                                              \
     hipLaunchKernelGGL((fir_step_kernel<P, Q, M, GR, N, F>), grid, dim3(64 * N), sh, s, p1, p2, pv, in_bs, pj, \
-                       (bf16_t*)ring, (int)R, (int)pos, (const int*)pos_dev, w, bias, (bf16_t*)out, out_bs, D, dg)
+                       (bf16_t*)ring, (int)R, (int)cb, (int)pos, (const int*)pos_dev, w, bias, (bf16_t*)out, out_bs, D, dg)
 #define FS_CASE(P, Q, M, F)                                                                                   \
     if (!ok && pre == P && post == Q && bias_mode == M && feat == F) {                                        \
         if (grouped && nsg == 8) FS_GO(P, Q, M, true, 8, F);                                                  \
@@ -491,33 +499,33 @@ static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_
 }
 
 extern "C" int hyena_fir_step(const void* x1, const void* x2, const void* v, int64_t in_bs, void* ring, int64_t R,
-                              int64_t pos, const float* w, const float* bias, int bias_mode, void* out,
+                              int64_t cb, int64_t pos, const float* w, const float* bias, int bias_mode, void* out,
                               int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream) {
-    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, pos, nullptr, w, bias, bias_mode, out, out_bs, B, D, G,
+    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, cb, pos, nullptr, w, bias, bias_mode, out, out_bs, B, D, G,
                            stream, "hyena_fir_step");
 }
 
 extern "C" int hyena_fir_step_dpos(const void* x1, const void* x2, const void* v, int64_t in_bs, void* ring, int64_t R,
-                                   const int32_t* pos_dev, const float* w, const float* bias, int bias_mode,
+                                   int64_t cb, const int32_t* pos_dev, const float* w, const float* bias, int bias_mode,
                                    void* out, int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream) {
     if (!pos_dev) return hyena_fail(HYENA_EINVAL, "hyena_fir_step_dpos: pos_dev is required");
-    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, 0, pos_dev, w, bias, bias_mode, out, out_bs, B, D, G,
+    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, cb, 0, pos_dev, w, bias, bias_mode, out, out_bs, B, D, G,
                            stream, "hyena_fir_step_dpos");
 }
 
-extern "C" int hyena_fir_layer_step(const hyena_proj_step* proj, void* ring, int64_t R, int64_t pos, const float* w,
+extern "C" int hyena_fir_layer_step(const hyena_proj_step* proj, void* ring, int64_t R, int64_t cb, int64_t pos, const float* w,
                                     const float* bias, int bias_mode, void* out, int64_t out_bs, int64_t B,
                                     int64_t D, int64_t G, void* stream) {
     if (!proj) return hyena_fail(HYENA_EINVAL, "hyena_fir_layer_step: proj is required");
-    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, pos, nullptr, w, bias, bias_mode, out, out_bs, B,
+    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, cb, pos, nullptr, w, bias, bias_mode, out, out_bs, B,
                            D, G, stream, "hyena_fir_layer_step");
 }
 
-extern "C" int hyena_fir_layer_step_dpos(const hyena_proj_step* proj, void* ring, int64_t R, const int32_t* pos_dev,
+extern "C" int hyena_fir_layer_step_dpos(const hyena_proj_step* proj, void* ring, int64_t R, int64_t cb, const int32_t* pos_dev,
                                          const float* w, const float* bias, int bias_mode, void* out, int64_t out_bs,
                                          int64_t B, int64_t D, int64_t G, void* stream) {
     if (!proj || !pos_dev) return hyena_fail(HYENA_EINVAL, "hyena_fir_layer_step_dpos: proj and pos_dev are required");
-    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, 0, pos_dev, w, bias, bias_mode, out, out_bs, B, D,
+    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, cb, 0, pos_dev, w, bias, bias_mode, out, out_bs, B, D,
                            G, stream, "hyena_fir_layer_step_dpos");
 }
 

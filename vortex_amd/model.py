@@ -260,7 +260,7 @@ class RecordedDecodeStep:
             rings.append(ip.fir_state_dict[i])
             if block.filter.fir_inner_filter_length:
                 rings.append(ip.fir_inner_state_dict[i])
-        if any(getattr(r, "valid", r.buf.shape[1]) < r.buf.shape[1] for r in rings):
+        if any(getattr(r, "valid", r.R) < r.R for r in rings):
             raise NotImplementedError("a cache is still filling up (prompt shorter than a filter): step eagerly")
         mha = ipd["mha"]
         self.clock = ops.RingClock(rings)

@@ -312,31 +312,48 @@ def hyena_li_fwd(x1, x2, v, log_poles, residues, D_bias=None, *, plan=None, want
 
 
 class FirRing:
-    """Ring-buffer FIR cache [B, R, D] bf16 plus the index of its oldest slot.
+    """Ring-buffer FIR cache of R slots over D channels (bf16) plus the index of its oldest slot.
 
     Holds the same samples as the reference's [B, D, R] oldest-first fir_state
     (vortex/model/engine.py:414, :443-447); reference_order() returns that view.
+
+    Built from the slots as a [B, R, D] tensor.  `buf` is the device layout [B, D/block, R, block]: block = D is
+    that tensor itself (a view, so a caller's tensor is updated in place); block = 512 keeps the R slots of 512
+    channels in one contiguous run, which the step kernel streams faster from deep caches.  block=None picks 512
+    for caches of 32 slots and more whose D is a multiple of 512, and D otherwise.
     """
 
-    def __init__(self, buf, pos=0):
-        self.buf, self.pos = buf, pos
+    def __init__(self, slots, pos=0, block=None):
+        B, R, D = slots.shape
+        if block is None:
+            block = 512 if (R >= 32 and D % 512 == 0 and D > 512) else D
+        if block != D and (block % 512 or D % block):
+            raise ValueError(f"block {block} must be D or a multiple of 512 that divides D={D}")
+        self.B, self.R, self.D, self.block = B, R, D, block
+        if block == D:
+            self.buf = slots.contiguous().view(B, 1, R, D)
+        else:
+            self.buf = slots.reshape(B, R, D // block, block).permute(0, 2, 1, 3).contiguous()
+        self.pos = pos
         self.pos_dev = None         # int32 [1] device tensor once a RingClock owns the position (then pos is stale)
 
     @classmethod
-    def from_reference(cls, fir_state):
+    def from_reference(cls, fir_state, block=None):
         """fir_state: [B, D, R] oldest-first (any float dtype holding bf16-exact values)."""
-        return cls(fir_state.to(torch.bfloat16).permute(0, 2, 1).contiguous(), 0)
+        return cls(fir_state.to(torch.bfloat16).permute(0, 2, 1).contiguous(), 0, block)
 
     @property
     def shape(self):   # what engine.step_fir reads as cache size: shape[-1]
-        B, R, D = self.buf.shape
-        return torch.Size((B, D, R))
+        return torch.Size((self.B, self.D, self.R))
+
+    def slots(self):
+        """The slots as [B, R, D] in storage order (slot `pos` is the oldest); a view for block = D."""
+        return self.buf.permute(0, 2, 1, 3).reshape(self.B, self.R, self.D)
 
     def reference_order(self, dtype=torch.float32):
-        R = self.buf.shape[1]
         pos = self.pos if self.pos_dev is None else int(self.pos_dev.item())
-        idx = (torch.arange(R, device=self.buf.device) + pos) % R
-        return self.buf.index_select(1, idx).permute(0, 2, 1).to(dtype)
+        idx = (torch.arange(self.R, device=self.buf.device) + pos) % self.R
+        return self.slots().index_select(1, idx).permute(0, 2, 1).to(dtype)
 
 
 def fir_step(x1, ring, w, *, x2=None, v=None, bias=None, gated_bias=False):
@@ -347,7 +364,9 @@ def fir_step(x1, ring, w, *, x2=None, v=None, bias=None, gated_bias=False):
     """
     _need_cuda(x1, ring.buf, w)
     B, D = x1.shape
-    R = ring.buf.shape[1]
+    R = ring.R
+    if ring.D != D:
+        raise ValueError(f"cache over {ring.D} channels, gates over {D}")
     w = _step_taps(w, D)
     G = w.shape[0]
     if w.shape[1] != R + 1:
@@ -359,12 +378,12 @@ def fir_step(x1, ring, w, *, x2=None, v=None, bias=None, gated_bias=False):
     b = _f32(bias)
     mode = HYENA_BIAS_NONE if b is None else (HYENA_BIAS_GATED_FP32 if gated_bias else HYENA_BIAS_ADD)
     if ring.pos_dev is not None:                # the position is on a RingClock, which also advances it
-        rc = _lib.lib().hyena_fir_step_dpos(_ptr(x1), _ptr(x2), _ptr(v), x1.stride(0), _ptr(ring.buf), R,
+        rc = _lib.lib().hyena_fir_step_dpos(_ptr(x1), _ptr(x2), _ptr(v), x1.stride(0), _ptr(ring.buf), R, ring.block,
                                             _ptr(ring.pos_dev), _ptr(w), _ptr(b), mode, _ptr(out), out.stride(0),
                                             B, D, G, _stream())
         _lib.check(rc, "hyena_fir_step_dpos")
         return out
-    rc = _lib.lib().hyena_fir_step(_ptr(x1), _ptr(x2), _ptr(v), x1.stride(0), _ptr(ring.buf), R, ring.pos,
+    rc = _lib.lib().hyena_fir_step(_ptr(x1), _ptr(x2), _ptr(v), x1.stride(0), _ptr(ring.buf), R, ring.block, ring.pos,
                                    _ptr(w), _ptr(b), mode, _ptr(out), out.stride(0), B, D, G, _stream())
     _lib.check(rc, "hyena_fir_step")
     ring.pos = (ring.pos + 1) % R
@@ -422,7 +441,7 @@ class FirStepper:
     def __init__(self, ring, w, bias=None, gated_bias=False, gated=True):
         _need_cuda(ring.buf, w)
         self.ring, self.bias = ring, _f32(bias)
-        self.R, self.D = ring.buf.shape[1], ring.buf.shape[2]
+        self.R, self.D = ring.R, ring.D
         self.w = _step_taps(w, self.D)
         self.G = self.w.shape[0]
         if self.w.shape[1] != self.R + 1:
@@ -437,7 +456,8 @@ class FirStepper:
         dpos = ring.pos_dev is not None
         rc = (self._fn_dpos if dpos else self._fn)(
             x1.data_ptr(), x2.data_ptr() if self.gated else None, v.data_ptr() if self.gated else None,
-            x1.stride(0), ring.buf.data_ptr(), self.R, ring.pos_dev.data_ptr() if dpos else ring.pos, self.w.data_ptr(),
+            x1.stride(0), ring.buf.data_ptr(), self.R, ring.block, ring.pos_dev.data_ptr() if dpos else ring.pos,
+            self.w.data_ptr(),
             self.bias.data_ptr() if self.bias is not None else None, self.mode, out.data_ptr(),
             out.stride(0), B, self.D, self.G, torch.cuda.current_stream().cuda_stream)
         if rc:
@@ -499,7 +519,9 @@ class LayerStepper:
     def __init__(self, feat_ring, feat_w, feat_bias, channel_map, inner, flip_x1x2=False):
         _need_cuda(feat_ring.buf, feat_w)
         self.ring, self.inner = feat_ring, inner
-        self.Rf, C = feat_ring.buf.shape[1], feat_ring.buf.shape[2]
+        if feat_ring.block != feat_ring.D:
+            raise ValueError("the featurizer cache must use the plain [B, R, 3D] layout (block = D)")
+        self.Rf, C = feat_ring.R, feat_ring.D
         self.w = _f32(feat_w).reshape(C, self.Rf + 1).t().contiguous()        # tap-major [Rf+1, C]
         self.bias = _f32(feat_bias)
         ci, co, gs, cs = channel_map
@@ -521,11 +543,11 @@ class LayerStepper:
         p.pos, p.pos_dev = (0, self.ring.pos_dev.data_ptr()) if dpos else (self.ring.pos, None)
         stream = torch.cuda.current_stream().cuda_stream
         if self.is_fir and dpos:
-            rc = self._fn_dpos(self._pref, n.ring.buf.data_ptr(), n.R, n.ring.pos_dev.data_ptr(), n.w.data_ptr(),
+            rc = self._fn_dpos(self._pref, n.ring.buf.data_ptr(), n.R, n.ring.block, n.ring.pos_dev.data_ptr(), n.w.data_ptr(),
                                n.bias.data_ptr() if n.bias is not None else None, n.mode, out.data_ptr(),
                                out.stride(0), B, n.D, n.G, stream)
         elif self.is_fir:
-            rc = self._fn(self._pref, n.ring.buf.data_ptr(), n.R, n.ring.pos, n.w.data_ptr(),
+            rc = self._fn(self._pref, n.ring.buf.data_ptr(), n.R, n.ring.block, n.ring.pos, n.w.data_ptr(),
                           n.bias.data_ptr() if n.bias is not None else None, n.mode, out.data_ptr(), out.stride(0),
                           B, n.D, n.G, stream)
         else:
@@ -556,7 +578,7 @@ class RingClock:
         if any(r.pos_dev is not None for r in self.rings):
             raise RuntimeError("a ring is already on a clock")
         self.pos = torch.tensor([r.pos for r in self.rings], dtype=torch.int32, device=dev)
-        self.depth = torch.tensor([r.buf.shape[1] for r in self.rings], dtype=torch.int32, device=dev)
+        self.depth = torch.tensor([r.R for r in self.rings], dtype=torch.int32, device=dev)
         for i, r in enumerate(self.rings):
             r.pos_dev = self.pos[i:i + 1]
 
