@@ -402,6 +402,7 @@ def main():
         probe, stream = _lib.stream_probe(), torch.cuda.current_stream().cuda_stream
         print(f"access-pattern probes: {D} rows of {L} bf16 samples, 3 reads + 1 write, no arithmetic", file=sys.stderr)
         cases = [("whole rows, one block per 4 rows (a one-pass scan)", 0, 0)]
+        cases += [(f"whole rows, one block per row (4 wavefronts x 4 KiB per step), {256 * n} rows in flight", 2, n) for n in (8, 4, 2, 1)]
         cases += [(f"independent segments of {s} samples, row sets in order", 1, s) for s in (65536, 16384, 8192, 4096, 2048)]
         for what, pat, seg in cases:
             fn = lambda: _lib.check(probe(t[0].data_ptr(), t[1].data_ptr(), t[2].data_ptr(), o.data_ptr(), D, L, pat, seg,

@@ -8,6 +8,10 @@
 //   pattern 1  segments:    one block per (row set, segment of `seg` samples), segments of a row set on consecutive
 //              blocks -- the order of a kernel whose blocks are independent (Hyena-MR); a carried state would have
 //              to be handed from block to block
+//   pattern 2  one row per block:  the four wavefronts of a block walk ONE row together, 4 KiB each per step
+//              (16 KiB of the row per block step, two steps prefetched); `seg` = blocks resident per CU (1, 2, 4
+//              or 8, enforced with an LDS request), i.e. 256 .. 2048 rows in flight on the chip -- the order of a
+//              scan whose block shares one row and passes the state between its wavefronts
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -62,14 +66,42 @@ __global__ __launch_bounds__(256) void stream_probe_kernel(const bf16_t* a, cons
         }
     }
 }
+// pattern 2: block = one row, wavefront w takes samples [2048 w, 2048 w + 2048) of each 8192-sample block step
+__global__ __launch_bounds__(256) void row_probe_kernel(const bf16_t* a, const bf16_t* b, const bf16_t* c, bf16_t* o, int64_t L) {
+    extern __shared__ char occupancy_limit[];
+    constexpr int K = 4;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int64_t step = 4 * K * 512, nsteps = L / step;
+    const int64_t base = (int64_t)blockIdx.x * L + (int64_t)w * K * 512 + lane * 8;
+    u32x4 x[PF][K], y[PF][K], z[PF][K];
+#pragma unroll
+    for (int p = 0; p < PF; ++p)
+#pragma unroll
+        for (int j = 0; j < K; ++j)
+            if (p < nsteps) { const int64_t t = base + p * step + j * 512; x[p][j] = ldnt(a + t); y[p][j] = ldnt(b + t); z[p][j] = ldnt(c + t); }
+    for (int64_t u0 = 0; u0 < nsteps; u0 += PF) {
+#pragma unroll
+        for (int p = 0; p < PF; ++p) {
+            const int64_t u = u0 + p;
+            if (u >= nsteps) break;
+#pragma unroll
+            for (int j = 0; j < K; ++j) {
+                const int64_t t = base + u * step + j * 512;
+                stnt(o + t, x[p][j] ^ y[p][j] ^ z[p][j]);
+                if (u + PF < nsteps) { const int64_t tn = t + PF * step; x[p][j] = ldnt(a + tn); y[p][j] = ldnt(b + tn); z[p][j] = ldnt(c + tn); }
+            }
+            __syncthreads();      // the wavefronts of a block stay together, as a state passed between them would force
+        }
+    }
+}
 }  // namespace
 
 // a, b, c, o: D rows of L bf16 samples each (contiguous); D % 4 == 0, L % 2048 == 0.
-// pattern 0: seg ignored.  pattern 1: seg a multiple of 2048 dividing L.
+// pattern 0: seg ignored.  pattern 1: seg a multiple of 2048 dividing L.  pattern 2: seg = blocks per CU (1, 2, 4, 8), L % 8192 == 0.
 // 0 on success, -1 for a rejected argument, a positive hipError_t if the launch failed.
 extern "C" int hyena_stream_probe(const void* a, const void* b, const void* c, void* o, int64_t D, int64_t L, int pattern,
                                   int64_t seg, void* stream) {
-    if (!a || !b || !c || !o || D <= 0 || D % R || L <= 0 || L % 2048 || pattern < 0 || pattern > 1) return -1;
+    if (!a || !b || !c || !o || D <= 0 || D % R || L <= 0 || L % 2048 || pattern < 0 || pattern > 2) return -1;
     Walk wk = {};
     wk.L = L; wk.nsets = D / R;
     int64_t grid;
@@ -77,6 +109,13 @@ extern "C" int hyena_stream_probe(const void* a, const void* b, const void* c, v
     else if (pattern == 1) {
         if (seg <= 0 || seg % 2048 || L % seg) return -1;
         wk.seg = seg; wk.nseg = (int)(L / seg); wk.nunits = seg / 2048; grid = wk.nsets * wk.nseg;
+    }
+    else {
+        if (L % 8192 || (seg != 1 && seg != 2 && seg != 4 && seg != 8) || D > 0x7fffffffLL) return -1;
+        const size_t lds = seg == 1 ? 100000 : seg == 2 ? 70000 : seg == 4 ? 36000 : 0;      // of 160 KiB per CU
+        hipLaunchKernelGGL(row_probe_kernel, dim3((unsigned)D), dim3(256), lds, (hipStream_t)stream, (const bf16_t*)a,
+                           (const bf16_t*)b, (const bf16_t*)c, (bf16_t*)o, L);
+        return (int)hipGetLastError();
     }
     if (grid > 0x7fffffffLL) return -1;
 #define GO(P) hipLaunchKernelGGL(stream_probe_kernel<P>, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)a, \
