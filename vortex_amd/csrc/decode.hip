@@ -144,6 +144,21 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
     // the first batch of cache reads goes out before the tap table is staged, so HBM is busy from the start
     u32x4 q0[UF];
     load_batch(sg, q0);
+    // the output wavefront requests its gates and bias now, so that they arrive with the cache instead of costing
+    // a second round trip to memory after the reduction
+    u32x4 a1 = zero4, av = zero4, a2 = zero4;
+    f32x4 bs0 = {0.f, 0.f, 0.f, 0.f}, bs1 = bs0;
+    if (sg == 0 && live) {
+        if (FEAT == 0) {
+            a1 = *(const u32x4*)(x1 + b * in_bs + d0);
+            if (PRE) av = *(const u32x4*)(v + b * in_bs + d0);
+            if (POST) a2 = *(const u32x4*)(x2 + b * in_bs + d0);
+        }
+        if (BIAS != HYENA_BIAS_NONE) {
+            bs0 = *(const f32x4*)(bias + d0);
+            bs1 = *(const f32x4*)(bias + d0 + 4);
+        }
+    }
     // Fused featurizer: the block's 3 x 512 projection channels are 192 pieces of 8; thread p evaluates piece p
     // (its loads overlap the cache reads above) and leaves the gates in LDS for the wavefront that writes the output.
     if (FEAT != 0) {
@@ -197,7 +212,6 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
 #pragma unroll
         for (int c = 0; c < 8; ++c) acc[c] += red[((k * 2 + (c >> 2)) * 64 + oc) * 4 + (c & 3)];
 
-    u32x4 a1, av = {0, 0, 0, 0}, a2 = {0, 0, 0, 0};
     if (FEAT != 0) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -213,10 +227,6 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
             a2[j] = pj.flip ? pack_bf2(g1[0], g1[1]) : pack_bf2(g2[0], g2[1]);
             av[j] = pack_bf2(gv[0], gv[1]);
         }
-    } else {
-        a1 = *(const u32x4*)(x1 + b * in_bs + d0);
-        if (PRE) av = *(const u32x4*)(v + b * in_bs + d0);
-        if (POST) a2 = *(const u32x4*)(x2 + b * in_bs + d0);
     }
     uint32_t up[4], o[4];
 #pragma unroll
@@ -230,8 +240,9 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
             const int c = 2 * j + e;
             const float h0 = GROUPED ? wl[R * ng + gl] : w[(d0 + c) * W + R];
             float yy = fmaf(h0, uu[e], acc[c]);
-            if (BIAS == HYENA_BIAS_GATED_FP32) yy = fmaf(bias[d0 + c], uu[e], yy);
-            if (BIAS == HYENA_BIAS_ADD) yy += bias[d0 + c];
+            const float bc = c < 4 ? bs0[c & 3] : bs1[c & 3];
+            if (BIAS == HYENA_BIAS_GATED_FP32) yy = fmaf(bc, uu[e], yy);
+            if (BIAS == HYENA_BIAS_ADD) yy += bc;
             yy = round_bf(yy);
             if (POST) yy *= (e ? bf_hi(a2[j]) : bf_lo(a2[j]));
             y[e] = yy;
@@ -446,7 +457,7 @@ static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_
     if (bias_mode < 0 || bias_mode > 2 || (bias_mode != HYENA_BIAS_NONE && !bias))
         return hyena_fail(HYENA_EINVAL, "%s: bias_mode %d needs a bias pointer", who, bias_mode);
     if (D % 8 != 0 || in_bs % 8 != 0 || out_bs % 8 != 0 || ((uintptr_t)x1 & 15) || ((uintptr_t)ring & 15) ||
-        ((uintptr_t)out & 15) || (x2 && ((uintptr_t)x2 & 15)) || (v && ((uintptr_t)v & 15)))
+        ((uintptr_t)out & 15) || (x2 && ((uintptr_t)x2 & 15)) || (v && ((uintptr_t)v & 15)) || ((uintptr_t)bias & 15))
         return hyena_fail(HYENA_EALIGN, "%s: D and strides must be multiples of 8, pointers 16-byte aligned", who);
     if (B > 65535) return hyena_fail(HYENA_EINVAL, "%s: B > 65535", who);
     ProjArgs pj = {};
