@@ -113,7 +113,7 @@ def cl_cases(seed, n):
     return [(rng.choice([1, 2, 3]), rng.randint(1, 3000), rng.randint(0, 10 ** 6)) for _ in range(n)]
 
 
-@pytest.mark.parametrize("B,L,seed", cl_cases(7, 14))
+@pytest.mark.parametrize("B,L,seed", cl_cases(7, 14) + [(3, 1, 960982)])      # the last: one time row, permuted view
 def test_channel_last_fir_random(B, L, seed, override):
     # channel-last kernel: any L (rows are independent), channel counts that leave partial 64-channel blocks,
     # every filter length class, forced segment counts

@@ -46,6 +46,19 @@ def test_rows_of_strided_view():
         ops.rows_of(u.float())
 
 
+def test_size_one_dimensions_get_dense_strides():
+    # torch leaves the stride of a size-one dimension arbitrary (here 1 for the time axis of a permuted [B, D, 1]
+    # tensor); the descriptors handed to the C entry points carry the dense value, which passes the alignment checks
+    t = torch.zeros(3, 48, 1, dtype=torch.bfloat16).permute(0, 2, 1)
+    assert t.stride() == (48, 1, 1)
+    assert ops._strides(t) == [48, 48, 1]
+    c = ops._cl_of(t)
+    assert (c.batch_stride, c.time_stride) == (48, 48)
+    r = ops.rows_of(torch.zeros(1, 1, 64, dtype=torch.bfloat16))
+    assert (r.batch_stride, r.row_stride) == (64, 64)
+    assert ops._strides(torch.zeros(4, 6, 16)[:, :3]) == [96, 16, 1]
+
+
 def test_fir_ring_reference_order_and_rotation():
     B, D, R = 2, 3, 5
     st = torch.arange(B * D * R, dtype=torch.float32).reshape(B, D, R)

@@ -25,6 +25,17 @@ def _need_cuda(*ts):
             raise RuntimeError("vortex_amd operators run on the GPU only (got a CPU tensor); there is no CPU fallback")
 
 
+def _strides(t):
+    """Strides of a tensor with those of size-one dimensions (which torch leaves arbitrary) replaced by the dense
+    values, so that the alignment checks of the C entry points see what a larger tensor of that layout would have."""
+    st, dense = list(t.stride()), 1
+    for i in range(t.dim() - 1, -1, -1):
+        if t.shape[i] == 1:
+            st[i] = dense
+        dense = max(dense, st[i] * t.shape[i])
+    return st
+
+
 def rows_of(t):
     """Row descriptor of a [B, D, L] bf16 tensor whose samples are contiguous."""
     if t is None:
@@ -34,7 +45,8 @@ def rows_of(t):
     if t.dim() != 3 or (t.shape[2] > 1 and t.stride(2) != 1):
         raise ValueError("expected a [B, D, L] tensor with contiguous samples")
     B, D, L = t.shape
-    return Rows(t.data_ptr(), t.stride(0), t.stride(1), D, D)
+    bs, rs, _ = _strides(t)
+    return Rows(t.data_ptr(), bs, rs, D, D)
 
 
 def rows_of_projection(u, hidden, which, head_dim=None):
@@ -74,8 +86,8 @@ def front_pad8(t):
     """
     B, D, L = t.shape
     pad = (-L) % 8
-    if pad == 0 and (L <= 1 or t.stride(2) == 1) and t.stride(1) % 8 == 0 and t.stride(0) % 8 == 0 \
-            and t.data_ptr() % 16 == 0:
+    st = _strides(t)
+    if pad == 0 and st[2] == 1 and st[1] % 8 == 0 and st[0] % 8 == 0 and t.data_ptr() % 16 == 0:
         return t, 0
     buf = torch.empty((B, D, L + pad), dtype=t.dtype, device=t.device)
     if pad:
@@ -128,7 +140,8 @@ def _cl_of(t):
         return None
     if t.dtype != torch.bfloat16 or t.dim() != 3 or (t.shape[2] > 1 and t.stride(2) != 1):
         raise ValueError("expected a [B, L, D] bfloat16 tensor with contiguous channels")
-    return Cl(t.data_ptr(), t.stride(0), t.stride(1))
+    bs, ts, _ = _strides(t)
+    return Cl(t.data_ptr(), bs, ts)
 
 
 def fir_cl_fwd(x1, x2, v, taps, *, bias=None, bias_mode=HYENA_BIAS_NONE, taps_reversed=False, want_y2=False,
@@ -177,7 +190,7 @@ def fir_layer_fwd(u, feat_w, feat_bias, channel_map, taps, *, bias=None, bias_mo
         out = torch.empty((B, L, D), dtype=torch.bfloat16, device=u.device)
     bx = torch.empty((B, L - bx_from, D), dtype=torch.bfloat16, device=u.device) if bx_from is not None else None
     if out.numel():
-        pj = ProjFwd(u.data_ptr(), u.stride(0), u.stride(1), feat_w.data_ptr(),
+        pj = ProjFwd(u.data_ptr(), _strides(u)[0], _strides(u)[1], feat_w.data_ptr(),
                      feat_bias.data_ptr() if feat_bias is not None else None, feat_w.shape[0], int(flip_x1x2),
                      ci, co, gs, cs)
         rc = _lib.lib().hyena_fir_layer_fwd(ctypes.byref(pj), _ptr(taps), int(taps_reversed), _ptr(_f32(bias)),
@@ -238,7 +251,7 @@ def featurizer_fwd(u, taps, bias=None, interleave=False, front_pad=0):
     if out.numel() == 0:
         return out
     b = _f32(bias)
-    rc = _lib.lib().hyena_featurizer_fwd(_ptr(u), u.stride(0), u.stride(1), _ptr(taps), _ptr(b), int(interleave), _ptr(out),
+    rc = _lib.lib().hyena_featurizer_fwd(_ptr(u), _strides(u)[0], _strides(u)[1], _ptr(taps), _ptr(b), int(interleave), _ptr(out),
                                          B, L, C, taps.shape[0], taps.shape[1], front_pad, _stream())
     _lib.check(rc, "hyena_featurizer_fwd")
     return out
