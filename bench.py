@@ -318,7 +318,7 @@ def model_decode(device, L=8192, n=32):
             "recorded_step_tokens_per_s": 1.0 / dt_rec}
 
 
-def cpu_baseline(name):
+def cpu_baseline(name, budget_s=12.0):
     """The oracle (a PyTorch port of the reference path) timed on the host cores, on a channel slice."""
     from oracle import hyena_oracle as O
     threads = torch.get_num_threads()
@@ -339,12 +339,39 @@ def cpu_baseline(name):
         lp, r = O.make_modal_complex(Ds // 16, 16)
         Db = torch.randn(Ds).bfloat16()
         f = lambda: O.li_prefill(x2, x1, v, lp, r, Db, want_state=False)
+    elif name == "decode":
+        # one [SE, MR, LI] layer set at config 4, D = 4096, full shape: the reference's own step functions
+        B, D, S = 64, 4096, 16
+        g = torch.Generator().manual_seed(6)
+        gates3 = [[torch.randn(B, D, generator=g).bfloat16() for _ in range(3)] for _ in range(3)]
+        st_se, st_mr = torch.randn(B, D, 6, generator=g), torch.randn(B, D, 127, generator=g)
+        w_se, w_mr = torch.randn(D, 1, 7, generator=g), torch.randn(D, 1, 128, generator=g)
+        Dm, Dl = torch.randn(D, generator=g), torch.randn(D, generator=g).bfloat16()
+        lp, r = O.make_modal_complex(D, S)
+        st_li = torch.zeros(B, D, S, dtype=torch.complex64)
+
+        def f():
+            (a2, a1, av), (b2, b1, bv), (c2, c1, cv) = gates3
+            y0, _ = O.step_fir(a1 * av, st_se, w_se)
+            y1, _ = O.step_fir(b1 * bv, st_mr, w_mr, bias=Dm, gated_bias=True, flip_filter=True)
+            y2, _ = O.step_iir(c2, c1, cv, Dl, r, lp, st_li)
+            return y0 * a2, y1 * b2, y2
+        f()
+        ts, t_all = [], time.perf_counter()
+        while len(ts) < 3 or (time.perf_counter() - t_all < budget_s and len(ts) < 40):
+            t0 = time.perf_counter()
+            f()
+            ts.append(time.perf_counter() - t0)
+        t = sorted(ts)[len(ts) // 2]
+        return dict(value=t * 1e6, unit="us per layer-set step", cores=threads, kind="port",
+                    sample=f"oracle step_fir / step_iir (vortex/model/engine.py:406-467 restated) at the full shape "
+                           f"B={B} D={D}, caches of 6 and 127, {S} complex states; median of {len(ts)} steps")
     else:
         return None
     f()
     ts = []
     t_all = time.perf_counter()
-    while len(ts) < 3 or (time.perf_counter() - t_all < 12 and len(ts) < 40):      # about 10 s of CPU work
+    while len(ts) < 3 or (time.perf_counter() - t_all < budget_s and len(ts) < 40):      # about 10 s of CPU work
         t0 = time.perf_counter()
         f()
         ts.append(time.perf_counter() - t0)
@@ -475,6 +502,10 @@ def main():
         result["extra"] = extra
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(main_name)
+        if "extra" in result:                      # shorter samples of the other workloads' CPU path beside their GPU figures
+            for name, key in (("se", "se"), ("li", "li"), ("decode", "decode_D4096")):
+                if name != main_name and key in result["extra"]:
+                    result["extra"][key]["cpu_baseline"] = cpu_baseline(name, 3.0)
     print(json.dumps(result))
 
 
