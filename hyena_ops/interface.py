@@ -6,6 +6,7 @@ k*x rounded to bf16, fp32 accumulation, the convolution rounded to bf16, then th
 output gate (vortex/model/engine.py:159, :197-208, :232).  Forward only.
 """
 import warnings
+from dataclasses import dataclass
 
 import torch
 
@@ -15,6 +16,89 @@ from vortex_amd._lib import (HYENA_BIAS_ADD, HYENA_BIAS_ADD_FP32, HYENA_BIAS_GAT
 
 from .kernel_utils import BwdKernelConfig, FwdKernelConfig  # noqa: F401
 from .utils import correction_toeplitz, toeplitz
+
+
+@dataclass(eq=False)
+class DefaultTwoPassChunkedGateConvGateFwdConfig(FwdKernelConfig):
+    """vortex/ops/hyena_se/interface.py:27-34: the forward record `two_pass_chunked_gate_conv_gate` falls back to."""
+    schedule: str = "default"
+    autotune: bool = True
+    CHUNK_SIZE: int = 128
+    BLOCK_D: int = 32
+    THREADBLOCK_SWIZZLE: str = "row"
+
+
+@dataclass(eq=False)
+class DefaultTwoPassChunkedGateConvGateBwdConfig(BwdKernelConfig):
+    """vortex/ops/hyena_se/interface.py:36-44 (carried for callers that name it; this build is forward only)."""
+    schedule: str = "default"
+    autotune: bool = True
+    CHUNK_SIZE: int = 128
+    BLOCK_D: int = 32
+    THREADBLOCK_SWIZZLE: str = "row"
+    LOAD_TOEPLITZ: bool = False
+    LOAD_BX_LAG: bool = False
+
+
+def reshape_inputs(x, k, q, num_groups, input_layout, inner_layout):
+    """The three feature groups from `input_layout` to `inner_layout` (vortex/ops/hyena_se/interface.py:272-319).
+
+    Layouts: "bdl" [B, D, L], "blgdg" [B, L, G, dg], "bgdgl" [B, G, dg, L], channel d = g*dg + j.  The pairs the
+    reference takes: bdl -> bdl | blgdg, blgdg -> bdl | bgdgl, bgdgl -> bdl | bgdgl (its bgdgl -> bdl branch names
+    undefined variables, interface.py:309-311; the rearrangement it spells is done here).  Views where torch allows."""
+    def one(t):
+        if input_layout == "bdl":
+            b, d, l = t.shape
+            if inner_layout == "bdl":
+                return t
+            if inner_layout == "blgdg":
+                return t.transpose(1, 2).reshape(b, l, num_groups, d // num_groups)
+            raise NotImplementedError("inner_layout must be bdl or blgdg")
+        if input_layout == "blgdg":
+            b, l, g, dg = t.shape
+            assert g == num_groups, "number of groups in feature groups and filter must match"
+            if inner_layout == "bdl":
+                return t.permute(0, 2, 3, 1).reshape(b, g * dg, l)
+            if inner_layout == "bgdgl":
+                return t.permute(0, 2, 3, 1)
+            raise NotImplementedError("inner_layout must be bdl or bgdgl")
+        if input_layout == "bgdgl":
+            b, g, dg, l = t.shape
+            assert g == num_groups, "number of groups in feature groups and filter must match"
+            if inner_layout == "bdl":
+                return t.reshape(b, g * dg, l)
+            if inner_layout == "bgdgl":
+                return t
+            raise NotImplementedError("inner_layout must be bdl or bgdgl")
+        raise NotImplementedError("input_layout must be bdl, blgdg or bgdgl")
+    return one(x), one(k), one(q)
+
+
+def reshape_outputs(y, num_groups, output_layout, inner_layout):
+    """The operator output from `inner_layout` ("bdl" or "blgdg") to `output_layout` ("bld", "bdl", "blgdg")
+    (vortex/ops/hyena_se/interface.py:322-339)."""
+    if inner_layout == "bdl":
+        b, d, l = y.shape
+        if output_layout == "bld":
+            return y.transpose(1, 2)
+        if output_layout == "blgdg":
+            return y.reshape(b, num_groups, d // num_groups, l).permute(0, 3, 1, 2)
+        if output_layout == "bdl":
+            return y
+        raise NotImplementedError("output_layout must be bld, bdl or blgdg")
+    if inner_layout == "blgdg":
+        b, l, g, dg = y.shape
+        if output_layout == "bld":
+            return y.reshape(b, l, g * dg)
+        if output_layout == "blgdg":
+            return y
+        raise NotImplementedError("output_layout must be bld or blgdg")
+    raise NotImplementedError("inner_layout must be bdl or blgdg")
+
+
+def gate_gate(x, k, q):
+    """vortex/ops/hyena_se/interface.py:771-773: the operator with the convolution left out."""
+    return x * k * q
 
 
 def _to_bdl(t, layout):

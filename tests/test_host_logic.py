@@ -236,3 +236,45 @@ def test_per_element_bound_catches_a_single_wrong_halo_sample():
     with pytest.raises(AssertionError):
         assert_gated_close(x2 * badf.bfloat16(), x2 * z32f.bfloat16(), z32f.bfloat16(), x2, abs_scale(u, hflat),
                            2.0 ** -8, fft_floor=4e-6)
+
+
+def test_hyena_ops_reshape_helpers_follow_the_index_definitions():
+    # vortex/ops/hyena_se/interface.py:272-339: every layout is a re-indexing of channel d = g*dg + j; checked
+    # element by element against that definition, and against the oracle's restatement for the bdl inner layout
+    from hyena_ops.interface import (DefaultTwoPassChunkedGateConvGateBwdConfig, DefaultTwoPassChunkedGateConvGateFwdConfig,
+                                     gate_gate, reshape_inputs, reshape_outputs)
+    from oracle import hyena_oracle as O
+    B, G, dg, Ls = 2, 3, 4, 5
+    D = G * dg
+    bdl = torch.arange(B * D * Ls, dtype=torch.float32).reshape(B, D, Ls)
+    blgdg = torch.empty(B, Ls, G, dg)
+    bgdgl = torch.empty(B, G, dg, Ls)
+    for b in range(B):
+        for g in range(G):
+            for j in range(dg):
+                for t in range(Ls):
+                    blgdg[b, t, g, j] = bgdgl[b, g, j, t] = bdl[b, g * dg + j, t]
+    forms = {"bdl": bdl, "blgdg": blgdg, "bgdgl": bgdgl}
+    for src, dst in [("bdl", "bdl"), ("bdl", "blgdg"), ("blgdg", "bdl"), ("blgdg", "bgdgl"), ("bgdgl", "bdl"),
+                     ("bgdgl", "bgdgl")]:
+        for got in reshape_inputs(forms[src], forms[src], forms[src], G, src, dst):
+            assert torch.equal(got, forms[dst]), (src, dst)
+        if dst == "bdl":
+            assert all(torch.equal(a, b_) for a, b_ in zip(reshape_inputs(forms[src], forms[src], forms[src], G, src, dst),
+                                                           O.reshape_inputs(forms[src], forms[src], forms[src], G, src)))
+    with pytest.raises(NotImplementedError):
+        reshape_inputs(bdl, bdl, bdl, G, "bdl", "bgdgl")
+    with pytest.raises(AssertionError):
+        reshape_inputs(blgdg, blgdg, blgdg, G + 1, "blgdg", "bdl")
+    bld = bdl.permute(0, 2, 1)
+    for out_layout, want in (("bdl", bdl), ("bld", bld), ("blgdg", blgdg)):
+        assert torch.equal(reshape_outputs(bdl, G, out_layout, "bdl"), want)
+        assert torch.equal(reshape_outputs(bdl, G, out_layout, "bdl"), O.reshape_outputs(bdl, G, out_layout))
+    assert torch.equal(reshape_outputs(blgdg, G, "bld", "blgdg"), bld)
+    assert torch.equal(reshape_outputs(blgdg, G, "blgdg", "blgdg"), blgdg)
+    with pytest.raises(NotImplementedError):
+        reshape_outputs(blgdg, G, "bdl", "blgdg")
+    assert torch.equal(gate_gate(bdl, 2 * bdl, 3 * bdl), 6 * bdl ** 3)
+    f, w = DefaultTwoPassChunkedGateConvGateFwdConfig(), DefaultTwoPassChunkedGateConvGateBwdConfig()
+    assert (f.autotune, f.CHUNK_SIZE, f.BLOCK_D, f.RETURN_Y2) == (True, 128, 32, True)
+    assert (w.LOAD_TOEPLITZ, w.LOAD_BX_LAG, w.name) == (False, False, "bwd")
