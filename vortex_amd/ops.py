@@ -337,7 +337,11 @@ class FirRing:
     """
 
     def __init__(self, slots, pos=0, block=None):
+        if slots.dtype != torch.bfloat16 or slots.dim() != 3:
+            raise TypeError(f"the cache slots must be a [B, R, D] bfloat16 tensor, got {tuple(slots.shape)} {slots.dtype}")
         B, R, D = slots.shape
+        if not 0 <= pos < max(R, 1):
+            raise ValueError(f"oldest-slot index {pos} outside 0..{R - 1}")
         if block is None:
             block = 512 if (R >= 32 and D % 512 == 0 and D > 512) else D
         if block != D and (block % 512 or D % block):
