@@ -212,11 +212,25 @@ def decode_layer_set(D, device, steps, warmup):
     # each step alone, launched back to back: kernels shorter than a launch (about 6 us from Python) read as the
     # launch rate, so `launch_bound` marks figures that are an upper bound of the kernel's own duration
     per = {}
-    for nm, st, xx, bb in (("se_step", step.se, x[0], b_se), ("mr_step", step.mr, x[1], b_mr), ("iir_step", step.li, x[2], b_li)):
+    # the Hyena-MR step as the reference's algorithm has it (the whole cache read every token), on a cache of its own
+    from vortex_amd import ops
+    mr_plain = ops.FirStepper(va.FirRing(rnd(B, 127, D).to(torch.bfloat16)), w_mr, bias=Dmr, gated_bias=True, far_sums=False)
+    for nm, st, xx, bb in (("se_step", step.se, x[0], b_se), ("mr_step", step.mr, x[1], b_mr),
+                           ("mr_step_whole_cache", mr_plain, x[1], b_mr), ("iir_step", step.li, x[2], b_li)):
         o = step.out[0]
         _, kms = time_steps(lambda: st(xx[1], xx[0], xx[2], o), max(steps, 100), warmup)
         per[nm] = dict(us=kms * 1e3, bytes=bb, hbm_gbs=bb / (kms * 1e-3) / 1e9, frac=bb / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                        launch_bound=kms * 1e3 < 10.0)
+    if step.mr.far is not None:
+        # The shipped Hyena-MR step keeps far sums and reads its whole cache only every n-th token: per token about
+        # (127 / n + (n - 1) / 2) slots, the far buffer (n - 1 rows written per window, one read on n - 1 of n tokens)
+        # and the gates.  Its `bytes`, `hbm_gbs` and `frac` above stay those of the reference's algorithm (what a token
+        # costs a kernel that reads the cache whole), so they are a rate of algorithmic bytes, not a bandwidth.
+        n = step.mr.far.numel() // (B * D)
+        moved = B * D * 2 * (127 / n + (n - 1) / 2) + B * D * 4 * 2 * (n - 1) / n + B * D * 2 + gates_io
+        per["mr_step"].update(bytes_moved_per_token=moved, moved_gbs=moved / (per["mr_step"]["us"] * 1e-6) / 1e9,
+                              window_tokens=n, note="bytes / hbm_gbs / frac are algorithmic (whole cache per token); "
+                              "the kernel moves bytes_moved_per_token on average")
     return dict(us_per_step=ms * 1e3, wall_us_per_step=wall / steps * 1e6, bytes=byts,
                 hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, kernels=per)
 

@@ -245,6 +245,32 @@ int hyena_fir_layer_step_dpos(const hyena_proj_step* proj,
                               int64_t B, int64_t D, int64_t G, void* stream);
 int hyena_ring_advance(int32_t* pos, const int32_t* depth, int64_t n, void* stream);
 
+/* FIR step on a deep cache (R >= 32) that reads about a third of the cache per token.  No counterpart in the
+ * reference, which reads (and rewrites) the whole cache every token (vortex/model/engine.py:427-447); same result up
+ * to the order of the float32 sums.  The part of a later token's sum that the cache already determines is formed
+ * three tokens at a time and kept in `far` ([B][3][D] float32, hyena_fir_far_bytes(B, D) bytes, contents owned by
+ * these calls): a block of 512 channels reads its whole cache on every third token (staggered over the blocks) and
+ * far[j] plus the j newest slots on the others.  `far` depends on the taps: one buffer per (cache, w) pair.
+ * cnt: token counter in [0, hyena_fir_far_period(R)) (the ring slot is cnt % R; the caller moves on to
+ * (cnt + 1) % period), or cnt_dev != NULL: the counter in device memory (hyena_ring_advance with depth = period).
+ * rebuild != 0: every block rebuilds its far sums from the cache as it stands; pass it on the first step and
+ * after anything else (hyena_fir_step, a prefill) has written to the cache.  Other arguments as hyena_fir_step /
+ * hyena_fir_layer_step. */
+int64_t hyena_fir_far_period(int64_t R);
+int64_t hyena_fir_far_bytes(int64_t B, int64_t D);
+int hyena_fir_step_far(const void* x1, const void* x2, const void* v, int64_t in_batch_stride,
+                       void* ring, int64_t R, int64_t ring_block, int64_t cnt, const int32_t* cnt_dev,
+                       float* far, int rebuild,
+                       const float* w, const float* bias, int bias_mode,
+                       void* out, int64_t out_batch_stride,
+                       int64_t B, int64_t D, int64_t G, void* stream);
+int hyena_fir_layer_step_far(const hyena_proj_step* proj,
+                             void* ring, int64_t R, int64_t ring_block, int64_t cnt, const int32_t* cnt_dev,
+                             float* far, int rebuild,
+                             const float* w, const float* bias, int bias_mode,
+                             void* out, int64_t out_batch_stride,
+                             int64_t B, int64_t D, int64_t G, void* stream);
+
 /* Channel-last operand [B][L][D]: element (b, t, d) at ptr + b*batch_stride + t*time_stride + d (elements).
  * This is the (batch, seqlen, groups, group_dim) layout of vortex/ops/hyena_se/fwd.py:17-43 with D = groups*group_dim. */
 typedef struct hyena_cl {

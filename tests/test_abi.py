@@ -78,6 +78,15 @@ def test_new_entry_points_validate_before_touching_the_device():
     assert L.hyena_fir_step_dpos(P, None, None, 1024, P, 6, 256, P, P, None, 0, P, 1024, 1, 1024, 64, None) == -1
     assert L.hyena_fir_step_dpos(P, None, None, 1536, P, 6, 1024, P, P, None, 0, P, 1536, 1, 1536, 96, None) == -1
     assert L.hyena_fir_step_dpos(P, None, None, 1536, P, 6, 512, P, P, None, 0, P, 1536, 0, 1536, 96, None) == 0
+    # far-sum FIR step: deep caches only, the far buffer is required, the counter runs to lcm(window, R)
+    per = L.hyena_fir_far_period(127)
+    assert per % 127 == 0 and per // 127 == L.hyena_fir_far_period(1) and L.hyena_fir_far_period(0) == 0
+    assert L.hyena_fir_far_bytes(64, 4096) == 64 * L.hyena_fir_far_period(1) * 4096 * 4
+    assert L.hyena_fir_step_far(P, None, None, 512, P, 127, 512, 0, None, None, 0, P, None, 0, P, 512, 1, 512, 32, None) == -1
+    assert L.hyena_fir_step_far(P, None, None, 512, P, 6, 512, 0, None, P, 0, P, None, 0, P, 512, 1, 512, 32, None) == -3
+    assert L.hyena_fir_step_far(P, None, None, 512, P, 127, 512, per, None, P, 0, P, None, 0, P, 512, 1, 512, 32, None) == -1
+    assert L.hyena_fir_step_far(P, None, None, 512, P, 127, 512, per - 1, None, P, 1, P, None, 0, P, 512, 0, 512, 32, None) == 0
+    assert L.hyena_fir_layer_step_far(None, P, 127, 512, 0, None, P, 0, P, None, 0, P, 512, 1, 512, 32, None) == -1
     assert L.hyena_ring_advance(None, P, 4, None) == -1 and L.hyena_ring_advance(P, P, -1, None) == -1
     assert L.hyena_ring_advance(P, P, 0, None) == 0
     ps = _lib.ProjStep(P, 192, P, 2, 5, P, None, 64, 0, 64, 1, 0, None)

@@ -94,6 +94,62 @@ def test_fir_step_channel_blocked_cache(D, blocks):
                                       flip_filter=True)
 
 
+@pytest.mark.parametrize("B,D,G,R,gated,on_clock", [
+    (3, 1024, 64, 127, True, False),      # Hyena-MR cache, grouped taps
+    (2, 1536, 1536, 127, True, False),    # one tap row per channel
+    (5, 520, 65, 127, False, False),      # D not a multiple of the 512-channel block
+    (1, 512, 32, 40, True, False),        # a shorter deep cache (counter period lcm(3, 40))
+    (4, 2048, 128, 127, True, True),      # counter in device memory (what a recorded token step uses)
+])
+def test_fir_step_far_sums(B, D, G, R, gated, on_clock):
+    """The stepper that keeps far sums (it reads its whole cache only every third token, staggered over the blocks)
+    against the oracle and against the plain step on a copy of the cache, for more tokens than two ring periods, with
+    a plain step on the same cache in between (the stepper then rebuilds its far sums)."""
+    from vortex_amd import _lib, ops
+    g = torch.Generator().manual_seed(D + R)
+    K = R + 1
+    w = torch.randn(G, 1, K, generator=g) / K ** 0.5
+    wD = w.repeat_interleave(D // G, 0)
+    bias = torch.randn(D, generator=g) if gated else None
+    st = torch.randn(B, D, R, generator=g).bfloat16()
+    taps = eff_taps(w, R, True).cuda()
+    rings = [va.FirRing.from_reference(st.cuda()) for _ in range(2)]
+    bias_d = None if bias is None else bias.cuda()
+    far = ops.FirStepper(rings[0], taps, bias=bias_d, gated_bias=gated)
+    plain = ops.FirStepper(rings[1], taps, bias=bias_d, gated_bias=gated, far_sums=False)
+    assert far.far is not None and plain.far is None and rings[0].period == _lib.lib().hyena_fir_far_period(R)
+    clock = ops.RingClock([rings[0]]) if on_clock else None
+    ref_state = st
+    ya, yb = (torch.empty(B, D, dtype=torch.bfloat16, device="cuda") for _ in range(2))
+    worst = 0.0
+    for step in range(2 * R + 7):
+        x1, x2, v = (torch.randn(B, D, generator=g).bfloat16() for _ in range(3))
+        y_ref, ref_state = O.step_fir(x1 * v, ref_state, wD, bias=bias, gated_bias=gated, flip_filter=True)
+        y_ref = (y_ref * x2).float()
+        if step in (5, R + 1) and not on_clock:      # something else steps the cache: the far sums are rebuilt afterwards
+            ya = va.fir_step(x1.cuda(), rings[0], taps, x2=x2.cuda(), v=v.cuda(), bias=bias_d, gated_bias=gated)
+            assert rings[0].far_owner is None
+        else:
+            far(x1.cuda(), x2.cuda(), v.cuda(), ya)
+            if clock is not None:
+                clock.advance()
+        plain(x1.cuda(), x2.cuda(), v.cuda(), yb)
+        assert (ya.float().cpu() - y_ref).abs().max() <= 2e-2 * y_ref.abs().max(), step
+        # against the plain step: the same products summed in another order, so at most the last bf16 digit moves
+        d = (ya.float() - yb.float()).abs()
+        tol = yb.float().abs() * 2.0 ** -7 + 2e-3 * x2.cuda().float().abs()
+        assert (d <= tol).all(), (step, (d / tol).max().item())
+        worst = max(worst, (d > 0).float().mean().item())
+        if step in (0, 6, R, 2 * R + 6):
+            if clock is not None:
+                torch.cuda.synchronize()
+            assert torch.equal(rings[0].reference_order().cpu(), ref_state), step
+    assert worst < 0.2, worst          # nearly every output is bit-identical
+    if clock is not None:
+        clock.release()
+        assert rings[0].pos == (2 * R + 7) % rings[0].period
+
+
 @pytest.mark.parametrize("name", ["real_bf16D", "real_f32D", "cplx_f32D"])
 def test_iir_step_golden(name):
     x2, x1, v = (torch.from_numpy(GOLD[f"iir_{name}_{k}"]).bfloat16().cuda() for k in ("x2", "x1", "v"))

@@ -16,6 +16,7 @@ EXPORTS = [
     "hyena_fir_step", "hyena_iir_step", "hyena_li_plan_bytes", "hyena_li_plan", "hyena_li_fwd", "hyena_li_fwd_static", "hyena_featurizer_fwd", "hyena_set_launch_override",
     "hyena_fir_layer_step", "hyena_iir_layer_step", "hyena_fir_cl_fwd", "hyena_fir_layer_fwd",
     "hyena_fir_step_dpos", "hyena_fir_layer_step_dpos", "hyena_ring_advance",
+    "hyena_fir_far_period", "hyena_fir_far_bytes", "hyena_fir_step_far", "hyena_fir_layer_step_far",
 ]
 
 
@@ -86,6 +87,13 @@ def lib():
     L.hyena_fir_layer_step_dpos.argtypes = [P, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                             c_int64, c_int64, c_int64, c_int64, c_void_p]
     L.hyena_ring_advance.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
+    L.hyena_fir_far_period.argtypes = [c_int64]
+    L.hyena_fir_far_bytes.argtypes = [c_int64, c_int64]
+    L.hyena_fir_step_far.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p,
+                                     c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64,
+                                     c_int64, c_void_p]
+    L.hyena_fir_layer_step_far.argtypes = [P, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p,
+                                           c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p]
     C = POINTER(Cl)
     L.hyena_fir_cl_fwd.argtypes = [C, C, C, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64,
                                    c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]
@@ -94,7 +102,7 @@ def lib():
     for name in EXPORTS:
         fn = getattr(L, name)
         if name not in ("hyena_version", "hyena_last_error_string"):
-            fn.restype = c_int64 if name == "hyena_li_plan_bytes" else c_int
+            fn.restype = c_int64 if name in ("hyena_li_plan_bytes", "hyena_fir_far_period", "hyena_fir_far_bytes") else c_int
     _lib = L
     return L
 

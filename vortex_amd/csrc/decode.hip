@@ -78,15 +78,30 @@ __device__ __forceinline__ void proj_store8(const ProjArgs& pj, int64_t b, uint3
 // slot written back is one coalesced row per batch element and channel block.  With cb = 512 the R slots a block
 // reads are one contiguous run of R KiB instead of 1 KiB pieces 2*D bytes apart, which deep caches stream faster.
 // FEAT != 0: the gates come from the fused featurizer step (ProjArgs) instead of x1, x2, v.
-template <bool PRE, bool POST, int BIAS, bool GROUPED, int NSG, int FEAT>
+//
+// NBT > 1 (deep caches with a `far` buffer [B][NBT][D] float32): the part of the sum that the cache already
+// determines is formed for NBT tokens at a time.  Token counter cnt (ring slot cnt % R); a block's window starts
+// when j = (cnt + blockIdx.x + blockIdx.y) % NBT is 0.  Then the block reads its whole cache once and forms, beside
+// this token's sum, far[j'] = sum_{i >= j'} w[i - j'] * state_i for j' = 1 .. NBT-1: what the samples cached NOW
+// will add to the outputs j' tokens later (i counts from the oldest slot; the j' oldest have dropped out by then).
+// The other NBT-1 tokens of the window read far[j] and only the j newest slots: y = far[j] + sum_{k=1..j}
+// w[R-k] * (k-th newest) + w[R] * u.  Windows are staggered over the blocks, so every launch moves about 1/NBT of
+// the cache.  all_heavy != 0 makes every block rebuild its window from the cache as it stands (the first step on a
+// cache, or after anything else wrote to it): a block at position j then forms far[j'] for j' > j over the slots
+// that were cached when its window began, sum_{i = j'-j}^{R-1-j} w[i + j - j'] * state_i.
+template <bool PRE, bool POST, int BIAS, bool GROUPED, int NSG, int FEAT, int NBT>
 __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __restrict__ x1, const bf16_t* __restrict__ x2,
                                                        const bf16_t* __restrict__ v, int64_t in_bs, ProjArgs pj,
                                                        bf16_t* __restrict__ ring, int R, int cb, int pos,
-                                                       const int* __restrict__ pos_dev,
+                                                       const int* __restrict__ pos_dev, int period,
+                                                       float* __restrict__ far, int all_heavy,
                                                        const float* __restrict__ w, const float* __restrict__ bias,
                                                        bf16_t* __restrict__ out, int64_t out_bs, int64_t D, int dg) {
     extern __shared__ float smem[];
-    if (pos_dev) pos = (int)((uint32_t)*pos_dev % (uint32_t)R);
+    if (pos_dev) pos = (int)((uint32_t)*pos_dev % (uint32_t)period);      // period = R, or lcm(NBT, R) with a far buffer
+    const int jw = NBT > 1 ? (int)((uint32_t)(pos + blockIdx.x + blockIdx.y) % (uint32_t)NBT) : 0;   // place in the window
+    const bool heavy = NBT == 1 || all_heavy != 0 || jw == 0;
+    if (NBT > 1) pos = (int)((uint32_t)pos % (uint32_t)R);
     if (FEAT != 0) pj.resolve_pos();
     const int tid = threadIdx.x, oc = tid & 63, sg = tid >> 6;
     const int64_t dblk = (int64_t)blockIdx.x * 512;
@@ -96,9 +111,9 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
     const int W = R + 1;
 
     const int ng = GROUPED ? (512 / dg) : 0;
-    float* wl = smem;                       // [W][ng]  taps of the block's groups, transposed
-    float* red = smem + (GROUPED ? W * ng : 0);   // [NSG-1][2][64][4]
-    float* zs = red + (NSG - 1) * 512;            // [3][512] gates of the block's channels (fused featurizer only)
+    float* wl = smem + (NBT - 1) * ng;      // [W][ng]  taps of the block's groups, transposed, behind NBT-1 rows of zeros
+    float* red = smem + (GROUPED ? (W + NBT - 1) * ng : 0);   // [NSG-1][NBT][2][64][4]
+    float* zs = red + (NSG - 1) * NBT * 512;      // [3][512] gates of the block's channels (fused featurizer only)
     const int gl = GROUPED ? (oc * 8) / dg : 0;
     constexpr int UF = 8;                   // cache slots in flight per lane
     // ring [B][D/cb][R][cb]: the block's 512 channels lie inside one channel block (cb = D is the plain [B][R][D])
@@ -107,35 +122,45 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
     const bf16_t* rb = ring + roff;
     const u32x4 zero4 = {0, 0, 0, 0};
 
+    // The main loop covers the slots that were cached when the block's window began: all R of them, except in a
+    // rebuild at place jw of a window, where the jw newest belong to the near part below.
+    const int Rl = R - (NBT > 1 ? jw : 0);
     auto load_batch = [&](int i, u32x4* q) {
 #pragma unroll
         for (int k = 0; k < UF; ++k) {
             const int ii = i + NSG * k;
             int s = pos + ii;
             if (s >= R) s -= R;
-            q[k] = (live && ii < R) ? *(const u32x4*)(rb + (int64_t)s * cb) : zero4;
+            q[k] = (live && ii < Rl) ? *(const u32x4*)(rb + (int64_t)s * cb) : zero4;
         }
     };
-    float acc[8];
+    float acc[NBT][8];
 #pragma unroll
-    for (int c = 0; c < 8; ++c) acc[c] = 0.f;
+    for (int jj = 0; jj < NBT; ++jj)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) acc[jj][c] = 0.f;
+    // tap of slot ii for the output jj tokens ahead (jj = 0: this token) is w[ii - jj]; the rows of zeros ahead of the
+    // LDS table stand for ii < jj (a slot that has dropped out of the cache by then)
     auto fma_batch = [&](int i, const u32x4* q) {
 #pragma unroll
         for (int k = 0; k < UF; ++k) {
             int ii = i + NSG * k;
             if (ii >= R) ii = R - 1;        // the slot was loaded as zeros; any finite tap will do
-            if (GROUPED) {
-                const float t = wl[ii * ng + gl];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    acc[2 * j] = fmaf(t, bf_lo(q[k][j]), acc[2 * j]);
-                    acc[2 * j + 1] = fmaf(t, bf_hi(q[k][j]), acc[2 * j + 1]);
-                }
-            } else if (live) {
+            for (int jj = 0; jj < NBT; ++jj) {
+                if (GROUPED) {
+                    const float t = wl[(ii - jj) * ng + gl];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    acc[2 * j] = fmaf(w[(d0 + 2 * j) * W + ii], bf_lo(q[k][j]), acc[2 * j]);
-                    acc[2 * j + 1] = fmaf(w[(d0 + 2 * j + 1) * W + ii], bf_hi(q[k][j]), acc[2 * j + 1]);
+                    for (int j = 0; j < 4; ++j) {
+                        acc[jj][2 * j] = fmaf(t, bf_lo(q[k][j]), acc[jj][2 * j]);
+                        acc[jj][2 * j + 1] = fmaf(t, bf_hi(q[k][j]), acc[jj][2 * j + 1]);
+                    }
+                } else if (live && ii >= jj) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        acc[jj][2 * j] = fmaf(w[(d0 + 2 * j) * W + ii - jj], bf_lo(q[k][j]), acc[jj][2 * j]);
+                        acc[jj][2 * j + 1] = fmaf(w[(d0 + 2 * j + 1) * W + ii - jj], bf_hi(q[k][j]), acc[jj][2 * j + 1]);
+                    }
                 }
             }
         }
@@ -143,7 +168,7 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
 
     // the first batch of cache reads goes out before the tap table is staged, so HBM is busy from the start
     u32x4 q0[UF];
-    load_batch(sg, q0);
+    if (heavy) load_batch(sg, q0);
     // the output wavefront requests its gates and bias now, so that they arrive with the cache instead of costing
     // a second round trip to memory after the reduction
     u32x4 a1 = zero4, av = zero4, a2 = zero4;
@@ -176,41 +201,96 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
             }
         }
     }
-    if (GROUPED) {
-        const int64_t g0 = dblk / dg;
-        const int64_t gmax = (D + dg - 1) / dg;
-        if ((W & 3) == 0) {
-            for (int e = tid; e < (W / 4) * ng; e += 64 * NSG) {      // groups fastest: conflict-free LDS stores
-                const int i4 = (e / ng) * 4, gl2 = e - (e / ng) * ng;
-                f32x4 t = {0.f, 0.f, 0.f, 0.f};
-                if (g0 + gl2 < gmax) t = *(const f32x4*)(w + (g0 + gl2) * W + i4);
+    float h0[8];                            // taps on the new sample
+    if (NBT > 1 && !heavy) {
+        // ---- inside a window: far[jw] plus the jw newest slots, all on the output wavefront
+        if (FEAT != 0) __syncthreads();     // the gates are in LDS
+        if (sg != 0 || !live) return;
+        const f32x4 f0 = *(const f32x4*)(far + ((b * NBT + jw) * D + d0));
+        const f32x4 f1 = *(const f32x4*)(far + ((b * NBT + jw) * D + d0 + 4));
 #pragma unroll
-                for (int k = 0; k < 4; ++k) wl[(i4 + k) * ng + gl2] = t[k];
+        for (int c = 0; c < 8; ++c) acc[0][c] = c < 4 ? f0[c & 3] : f1[c & 3];
+    } else {
+        if (GROUPED) {
+            const int64_t g0 = dblk / dg;
+            const int64_t gmax = (D + dg - 1) / dg;
+            for (int e = tid; e < (NBT - 1) * ng; e += 64 * NSG) smem[e] = 0.f;
+            if ((W & 3) == 0) {
+                for (int e = tid; e < (W / 4) * ng; e += 64 * NSG) {      // groups fastest: conflict-free LDS stores
+                    const int i4 = (e / ng) * 4, gl2 = e - (e / ng) * ng;
+                    f32x4 t = {0.f, 0.f, 0.f, 0.f};
+                    if (g0 + gl2 < gmax) t = *(const f32x4*)(w + (g0 + gl2) * W + i4);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) wl[(i4 + k) * ng + gl2] = t[k];
+                }
+            } else {
+                for (int e = tid; e < W * ng; e += 64 * NSG) {
+                    const int i = e / ng, gl2 = e - i * ng;
+                    wl[i * ng + gl2] = (g0 + gl2 < gmax) ? w[(g0 + gl2) * W + i] : 0.f;
+                }
             }
-        } else {
-            for (int e = tid; e < W * ng; e += 64 * NSG) {
-                const int i = e / ng, gl2 = e - i * ng;
-                wl[i * ng + gl2] = (g0 + gl2 < gmax) ? w[(g0 + gl2) * W + i] : 0.f;
+            __syncthreads();
+        }
+        fma_batch(sg, q0);
+        for (int i = sg + UF * NSG; i < R; i += UF * NSG) {
+            u32x4 q[UF];
+            load_batch(i, q);
+            fma_batch(i, q);
+        }
+        if (sg > 0) {
+#pragma unroll
+            for (int jj = 0; jj < NBT; ++jj)
+#pragma unroll
+                for (int c = 0; c < 8; ++c)          // 16 B per lane, lanes contiguous
+                    red[((((sg - 1) * NBT + jj) * 2 + (c >> 2)) * 64 + oc) * 4 + (c & 3)] = acc[jj][c];
+        }
+        __syncthreads();          // also orders every read of slot `pos` before its overwrite below
+        if (sg != 0 || !live) return;
+#pragma unroll(NBT > 1 ? 1 : NSG - 1)
+        for (int k = 0; k < NSG - 1; ++k) {
+#pragma unroll
+            for (int jj = 0; jj < NBT; ++jj)
+#pragma unroll
+                for (int c = 0; c < 8; ++c) acc[jj][c] += red[(((k * NBT + jj) * 2 + (c >> 2)) * 64 + oc) * 4 + (c & 3)];
+        }
+        if (NBT > 1) {
+            // what the cache adds to the later tokens of this window
+#pragma unroll
+            for (int jj = 1; jj < NBT; ++jj) {
+                if (jw + jj >= NBT) break;
+                float* fp = far + ((b * NBT + jw + jj) * D + d0);
+                *(f32x4*)fp = f32x4{acc[jj][0], acc[jj][1], acc[jj][2], acc[jj][3]};
+                *(f32x4*)(fp + 4) = f32x4{acc[jj][4], acc[jj][5], acc[jj][6], acc[jj][7]};
             }
         }
-        __syncthreads();
     }
-    fma_batch(sg, q0);
-    for (int i = sg + UF * NSG; i < R; i += UF * NSG) {
-        u32x4 q[UF];
-        load_batch(i, q);
-        fma_batch(i, q);
+    {
+        // taps on the new sample, and (with far sums) the near part: the jw newest slots, which entered the cache
+        // after the window's far sums were formed
+        const int64_t gw = GROUPED ? (dblk / dg + gl) * W : 0;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) h0[c] = GROUPED ? w[gw + R] : w[(d0 + c) * W + R];
+        if (NBT > 1) {
+            u32x4 qn[NBT > 1 ? NBT - 1 : 1];
+#pragma unroll
+            for (int k = 1; k < NBT; ++k) {
+                int sl = pos - k;
+                if (sl < 0) sl += R;
+                qn[k - 1] = k <= jw ? *(const u32x4*)(rb + (int64_t)sl * cb) : zero4;
+            }
+#pragma unroll
+            for (int k = 1; k < NBT; ++k) {
+                if (k > jw) break;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float t0 = GROUPED ? w[gw + R - k] : w[(d0 + 2 * j) * W + R - k];
+                    const float t1 = GROUPED ? t0 : w[(d0 + 2 * j + 1) * W + R - k];
+                    acc[0][2 * j] = fmaf(t0, bf_lo(qn[k - 1][j]), acc[0][2 * j]);
+                    acc[0][2 * j + 1] = fmaf(t1, bf_hi(qn[k - 1][j]), acc[0][2 * j + 1]);
+                }
+            }
+        }
     }
-    if (sg > 0) {
-#pragma unroll
-        for (int c = 0; c < 8; ++c) red[(((sg - 1) * 2 + (c >> 2)) * 64 + oc) * 4 + (c & 3)] = acc[c];   // 16 B per lane, lanes contiguous
-    }
-    __syncthreads();          // also orders every read of slot `pos` before its overwrite below
-    if (sg != 0 || !live) return;
-#pragma unroll
-    for (int k = 0; k < NSG - 1; ++k)
-#pragma unroll
-        for (int c = 0; c < 8; ++c) acc[c] += red[((k * 2 + (c >> 2)) * 64 + oc) * 4 + (c & 3)];
 
     if (FEAT != 0) {
 #pragma unroll
@@ -238,8 +318,7 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int c = 2 * j + e;
-            const float h0 = GROUPED ? wl[R * ng + gl] : w[(d0 + c) * W + R];
-            float yy = fmaf(h0, uu[e], acc[c]);
+            float yy = fmaf(h0[c], uu[e], acc[0][c]);
             const float bc = c < 4 ? bs0[c & 3] : bs1[c & 3];
             if (BIAS == HYENA_BIAS_GATED_FP32) yy = fmaf(bc, uu[e], yy);
             if (BIAS == HYENA_BIAS_ADD) yy += bc;
@@ -441,15 +520,26 @@ static int proj_vector_mode(const hyena_proj_step* p, int64_t D) {
     return 0;
 }
 
+constexpr int FAR_NBT = 3;          // tokens per window of the far sums
+
+static int64_t far_period(int64_t R) {      // lcm(FAR_NBT, R): one counter gives the ring slot (cnt % R) and the window phase (cnt % NBT)
+    int64_t a = R, b = FAR_NBT;
+    while (b) { const int64_t t = a % b; a = b; b = t; }
+    return R / a * FAR_NBT;
+}
+
 static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_t in_bs, const hyena_proj_step* proj,
-                           void* ring, int64_t R, int64_t cb, int64_t pos, const int32_t* pos_dev, const float* w, const float* bias,
+                           void* ring, int64_t R, int64_t cb, int64_t pos, const int32_t* pos_dev, float* far, int rebuild,
+                           const float* w, const float* bias,
                            int bias_mode, void* out, int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream,
                            const char* who) {
     if ((!proj && !x1) || !ring || !w || !out) return hyena_fail(HYENA_EINVAL, "%s: x1, ring, w, out are required", who);
     if (pos_dev) pos = 0;
-    if (B < 0 || D <= 0 || G <= 0 || D % G != 0 || R < 1 || R > 4096 || pos < 0 || pos >= R)
+    const int64_t period = far ? far_period(R) : R;
+    if (B < 0 || D <= 0 || G <= 0 || D % G != 0 || R < 1 || R > 4096 || pos < 0 || pos >= period)
         return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld G=%lld R=%lld pos=%lld", who, (long long)B,
                           (long long)D, (long long)G, (long long)R, (long long)pos);
+    if (far && R < 32) return hyena_fail(HYENA_ENOSUP, "%s: the far-sum form is for caches of 32 slots and more", who);
     if (cb != D && (cb <= 0 || cb % 512 != 0 || D % cb != 0))
         return hyena_fail(HYENA_EINVAL, "%s: ring_block %lld must be D or a multiple of 512 that divides D=%lld", who,
                           (long long)cb, (long long)D);
@@ -457,7 +547,8 @@ static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_
     if (bias_mode < 0 || bias_mode > 2 || (bias_mode != HYENA_BIAS_NONE && !bias))
         return hyena_fail(HYENA_EINVAL, "%s: bias_mode %d needs a bias pointer", who, bias_mode);
     if (D % 8 != 0 || in_bs % 8 != 0 || out_bs % 8 != 0 || ((uintptr_t)x1 & 15) || ((uintptr_t)ring & 15) ||
-        ((uintptr_t)out & 15) || (x2 && ((uintptr_t)x2 & 15)) || (v && ((uintptr_t)v & 15)) || ((uintptr_t)bias & 15))
+        ((uintptr_t)out & 15) || (x2 && ((uintptr_t)x2 & 15)) || (v && ((uintptr_t)v & 15)) || ((uintptr_t)bias & 15) ||
+        ((uintptr_t)far & 15))
         return hyena_fail(HYENA_EALIGN, "%s: D and strides must be multiples of 8, pointers 16-byte aligned", who);
     if (B > 65535) return hyena_fail(HYENA_EINVAL, "%s: B > 65535", who);
     ProjArgs pj = {};
@@ -476,21 +567,25 @@ static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_
     const bool pre = proj || v != nullptr, post = proj || x2 != nullptr;
     dim3 grid((unsigned)((D + 511) / 512), (unsigned)B);
     const int nsg = R >= 32 ? 8 : 2;
-    size_t sh = (size_t)(nsg - 1) * 64 * 8 * sizeof(float) + (grouped ? (size_t)(R + 1) * (512 / dg) * sizeof(float) : 0) +
+    const int nbt = far ? FAR_NBT : 1;
+    size_t sh = (size_t)(nsg - 1) * nbt * 64 * 8 * sizeof(float) + (grouped ? (size_t)(R + nbt) * (512 / dg) * sizeof(float) : 0) +
                 (proj ? 3 * 512 * sizeof(float) : 0);
     if (sh > 160 * 1024) return hyena_fail(HYENA_ENOSUP, "%s: R too large for the LDS tap table", who);
     hipStream_t s = (hipStream_t)stream;
     const bf16_t *p1 = (const bf16_t*)x1, *p2 = (const bf16_t*)x2, *pv = (const bf16_t*)v;
     bool ok = false;
-#define FS_GO(P, Q, M, GR, N, F)                                                                              \
-    hipLaunchKernelGGL((fir_step_kernel<P, Q, M, GR, N, F>), grid, dim3(64 * N), sh, s, p1, p2, pv, in_bs, pj, \
-                       (bf16_t*)ring, (int)R, (int)cb, (int)pos, (const int*)pos_dev, w, bias, (bf16_t*)out, out_bs, D, dg)
+#define FS_GO(P, Q, M, GR, N, F, T)                                                                              \
+    hipLaunchKernelGGL((fir_step_kernel<P, Q, M, GR, N, F, T>), grid, dim3(64 * N), sh, s, p1, p2, pv, in_bs, pj, \
+                       (bf16_t*)ring, (int)R, (int)cb, (int)pos, (const int*)pos_dev, (int)period, far, rebuild, \
+                       w, bias, (bf16_t*)out, out_bs, D, dg)
 #define FS_CASE(P, Q, M, F)                                                                                   \
     if (!ok && pre == P && post == Q && bias_mode == M && feat == F) {                                        \
-        if (grouped && nsg == 8) FS_GO(P, Q, M, true, 8, F);                                                  \
-        else if (grouped) FS_GO(P, Q, M, true, 2, F);                                                         \
-        else if (nsg == 8) FS_GO(P, Q, M, false, 8, F);                                                       \
-        else FS_GO(P, Q, M, false, 2, F);                                                                     \
+        if (far && grouped) FS_GO(P, Q, M, true, 8, F, FAR_NBT);                                              \
+        else if (far) FS_GO(P, Q, M, false, 8, F, FAR_NBT);                                                   \
+        else if (grouped && nsg == 8) FS_GO(P, Q, M, true, 8, F, 1);                                          \
+        else if (grouped) FS_GO(P, Q, M, true, 2, F, 1);                                                      \
+        else if (nsg == 8) FS_GO(P, Q, M, false, 8, F, 1);                                                    \
+        else FS_GO(P, Q, M, false, 2, F, 1);                                                                  \
         ok = true;                                                                                            \
     }
     FS_CASE(true, true, HYENA_BIAS_NONE, 0)
@@ -512,32 +607,55 @@ static int fir_step_launch(const void* x1, const void* x2, const void* v, int64_
 extern "C" int hyena_fir_step(const void* x1, const void* x2, const void* v, int64_t in_bs, void* ring, int64_t R,
                               int64_t cb, int64_t pos, const float* w, const float* bias, int bias_mode, void* out,
                               int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream) {
-    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, cb, pos, nullptr, w, bias, bias_mode, out, out_bs, B, D, G,
-                           stream, "hyena_fir_step");
+    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, cb, pos, nullptr, nullptr, 0, w, bias, bias_mode, out, out_bs,
+                           B, D, G, stream, "hyena_fir_step");
 }
 
 extern "C" int hyena_fir_step_dpos(const void* x1, const void* x2, const void* v, int64_t in_bs, void* ring, int64_t R,
                                    int64_t cb, const int32_t* pos_dev, const float* w, const float* bias, int bias_mode,
                                    void* out, int64_t out_bs, int64_t B, int64_t D, int64_t G, void* stream) {
     if (!pos_dev) return hyena_fail(HYENA_EINVAL, "hyena_fir_step_dpos: pos_dev is required");
-    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, cb, 0, pos_dev, w, bias, bias_mode, out, out_bs, B, D, G,
-                           stream, "hyena_fir_step_dpos");
+    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, cb, 0, pos_dev, nullptr, 0, w, bias, bias_mode, out, out_bs,
+                           B, D, G, stream, "hyena_fir_step_dpos");
 }
 
 extern "C" int hyena_fir_layer_step(const hyena_proj_step* proj, void* ring, int64_t R, int64_t cb, int64_t pos, const float* w,
                                     const float* bias, int bias_mode, void* out, int64_t out_bs, int64_t B,
                                     int64_t D, int64_t G, void* stream) {
     if (!proj) return hyena_fail(HYENA_EINVAL, "hyena_fir_layer_step: proj is required");
-    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, cb, pos, nullptr, w, bias, bias_mode, out, out_bs, B,
-                           D, G, stream, "hyena_fir_layer_step");
+    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, cb, pos, nullptr, nullptr, 0, w, bias, bias_mode, out,
+                           out_bs, B, D, G, stream, "hyena_fir_layer_step");
 }
 
 extern "C" int hyena_fir_layer_step_dpos(const hyena_proj_step* proj, void* ring, int64_t R, int64_t cb, const int32_t* pos_dev,
                                          const float* w, const float* bias, int bias_mode, void* out, int64_t out_bs,
                                          int64_t B, int64_t D, int64_t G, void* stream) {
     if (!proj || !pos_dev) return hyena_fail(HYENA_EINVAL, "hyena_fir_layer_step_dpos: proj and pos_dev are required");
-    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, cb, 0, pos_dev, w, bias, bias_mode, out, out_bs, B, D,
-                           G, stream, "hyena_fir_layer_step_dpos");
+    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, cb, 0, pos_dev, nullptr, 0, w, bias, bias_mode, out,
+                           out_bs, B, D, G, stream, "hyena_fir_layer_step_dpos");
+}
+
+extern "C" int64_t hyena_fir_far_period(int64_t R) { return R >= 1 ? far_period(R) : 0; }
+extern "C" int64_t hyena_fir_far_bytes(int64_t B, int64_t D) {
+    return B >= 0 && D > 0 ? B * FAR_NBT * D * (int64_t)sizeof(float) : 0;
+}
+
+extern "C" int hyena_fir_step_far(const void* x1, const void* x2, const void* v, int64_t in_bs, void* ring, int64_t R,
+                                  int64_t cb, int64_t cnt, const int32_t* cnt_dev, float* far, int rebuild, const float* w,
+                                  const float* bias, int bias_mode, void* out, int64_t out_bs, int64_t B, int64_t D,
+                                  int64_t G, void* stream) {
+    if (!far) return hyena_fail(HYENA_EINVAL, "hyena_fir_step_far: far is required");
+    return fir_step_launch(x1, x2, v, in_bs, nullptr, ring, R, cb, cnt, cnt_dev, far, rebuild != 0, w, bias, bias_mode, out,
+                           out_bs, B, D, G, stream, "hyena_fir_step_far");
+}
+
+extern "C" int hyena_fir_layer_step_far(const hyena_proj_step* proj, void* ring, int64_t R, int64_t cb, int64_t cnt,
+                                        const int32_t* cnt_dev, float* far, int rebuild, const float* w, const float* bias,
+                                        int bias_mode, void* out, int64_t out_bs, int64_t B, int64_t D, int64_t G,
+                                        void* stream) {
+    if (!proj || !far) return hyena_fail(HYENA_EINVAL, "hyena_fir_layer_step_far: proj and far are required");
+    return fir_step_launch(nullptr, nullptr, nullptr, 0, proj, ring, R, cb, cnt, cnt_dev, far, rebuild != 0, w, bias, bias_mode,
+                           out, out_bs, B, D, G, stream, "hyena_fir_layer_step_far");
 }
 
 namespace {

@@ -351,7 +351,9 @@ class FirRing:
             self.buf = slots.contiguous().view(B, 1, R, D)
         else:
             self.buf = slots.reshape(B, R, D // block, block).permute(0, 2, 1, 3).contiguous()
-        self.pos = pos
+        self.pos = pos              # oldest slot; with a far-sum stepper bound, a token counter modulo `period`
+        self.period = R             # (then the oldest slot is pos % R)
+        self.far_owner = None       # the FirStepper whose far sums are in step with this cache, if any
         self.pos_dev = None         # int32 [1] device tensor once a RingClock owns the position (then pos is stale)
 
     @classmethod
@@ -395,15 +397,17 @@ def fir_step(x1, ring, w, *, x2=None, v=None, bias=None, gated_bias=False):
     b = _f32(bias)
     mode = HYENA_BIAS_NONE if b is None else (HYENA_BIAS_GATED_FP32 if gated_bias else HYENA_BIAS_ADD)
     if ring.pos_dev is not None:                # the position is on a RingClock, which also advances it
+        ring.far_owner = None
         rc = _lib.lib().hyena_fir_step_dpos(_ptr(x1), _ptr(x2), _ptr(v), x1.stride(0), _ptr(ring.buf), R, ring.block,
                                             _ptr(ring.pos_dev), _ptr(w), _ptr(b), mode, _ptr(out), out.stride(0),
                                             B, D, G, _stream())
         _lib.check(rc, "hyena_fir_step_dpos")
         return out
-    rc = _lib.lib().hyena_fir_step(_ptr(x1), _ptr(x2), _ptr(v), x1.stride(0), _ptr(ring.buf), R, ring.block, ring.pos,
-                                   _ptr(w), _ptr(b), mode, _ptr(out), out.stride(0), B, D, G, _stream())
+    rc = _lib.lib().hyena_fir_step(_ptr(x1), _ptr(x2), _ptr(v), x1.stride(0), _ptr(ring.buf), R, ring.block,
+                                   ring.pos % R, _ptr(w), _ptr(b), mode, _ptr(out), out.stride(0), B, D, G, _stream())
     _lib.check(rc, "hyena_fir_step")
-    ring.pos = (ring.pos + 1) % R
+    ring.pos = (ring.pos + 1) % ring.period
+    ring.far_owner = None           # a stepper with far sums bound to this cache has to rebuild them
     return out
 
 
@@ -453,9 +457,14 @@ def _step_taps(w, D):
 
 
 class FirStepper:
-    """A decode FIR step with every argument except the gates bound once (low host overhead)."""
+    """A decode FIR step with every argument except the gates bound once (low host overhead).
 
-    def __init__(self, ring, w, bias=None, gated_bias=False, gated=True):
+    far_sums (default: caches of 32 slots and more): the step reads about a third of the cache per token by
+    forming, three tokens at a time, what the cached samples add to the next outputs (hyena_fir_step_far; same result up
+    to the order of the float32 sums).  The stepper owns the far-sum buffer, which belongs to this (cache, taps) pair;
+    if anything else steps the cache in between, the next call rebuilds it."""
+
+    def __init__(self, ring, w, bias=None, gated_bias=False, gated=True, far_sums=None):
         _need_cuda(ring.buf, w)
         self.ring, self.bias = ring, _f32(bias)
         self.R, self.D = ring.R, ring.D
@@ -465,22 +474,49 @@ class FirStepper:
             raise ValueError(f"taps have {self.w.shape[1]} columns, cache depth {self.R} needs {self.R + 1}")
         self.mode = HYENA_BIAS_NONE if bias is None else (HYENA_BIAS_GATED_FP32 if gated_bias else HYENA_BIAS_ADD)
         self.gated = gated
-        self._fn, self._fn_dpos = _lib.lib().hyena_fir_step, _lib.lib().hyena_fir_step_dpos
+        L = _lib.lib()
+        self._fn, self._fn_dpos, self._fn_far = L.hyena_fir_step, L.hyena_fir_step_dpos, L.hyena_fir_step_far
+        if far_sums is None:
+            far_sums = self.R >= 32
+        self.far = None
+        if far_sums:
+            if self.R < 32:
+                raise ValueError("far sums are for caches of 32 slots and more")
+            if ring.pos_dev is not None:
+                raise RuntimeError("bind the stepper before the cache goes on a RingClock")
+            self.far = torch.empty(L.hyena_fir_far_bytes(ring.B, self.D) // 4, dtype=torch.float32, device=ring.buf.device)
+            ring.period = L.hyena_fir_far_period(self.R)
+
+    def far_rebuild(self):
+        """1 when this call has to rebuild the far sums (first step, or something else stepped the cache); claims the cache."""
+        if self.ring.far_owner is self:
+            return 0
+        self.ring.far_owner = self
+        return 1
 
     def __call__(self, x1, x2, v, out):
         B = x1.shape[0]
         ring = self.ring
         dpos = ring.pos_dev is not None
-        rc = (self._fn_dpos if dpos else self._fn)(
-            x1.data_ptr(), x2.data_ptr() if self.gated else None, v.data_ptr() if self.gated else None,
-            x1.stride(0), ring.buf.data_ptr(), self.R, ring.block, ring.pos_dev.data_ptr() if dpos else ring.pos,
-            self.w.data_ptr(),
-            self.bias.data_ptr() if self.bias is not None else None, self.mode, out.data_ptr(),
-            out.stride(0), B, self.D, self.G, torch.cuda.current_stream().cuda_stream)
+        if self.far is not None:
+            rc = self._fn_far(
+                x1.data_ptr(), x2.data_ptr() if self.gated else None, v.data_ptr() if self.gated else None,
+                x1.stride(0), ring.buf.data_ptr(), self.R, ring.block, 0 if dpos else ring.pos,
+                ring.pos_dev.data_ptr() if dpos else None, self.far.data_ptr(), self.far_rebuild(), self.w.data_ptr(),
+                self.bias.data_ptr() if self.bias is not None else None, self.mode, out.data_ptr(),
+                out.stride(0), B, self.D, self.G, torch.cuda.current_stream().cuda_stream)
+        else:
+            ring.far_owner = None
+            rc = (self._fn_dpos if dpos else self._fn)(
+                x1.data_ptr(), x2.data_ptr() if self.gated else None, v.data_ptr() if self.gated else None,
+                x1.stride(0), ring.buf.data_ptr(), self.R, ring.block,
+                ring.pos_dev.data_ptr() if dpos else ring.pos % self.R,
+                self.w.data_ptr(), self.bias.data_ptr() if self.bias is not None else None, self.mode, out.data_ptr(),
+                out.stride(0), B, self.D, self.G, torch.cuda.current_stream().cuda_stream)
         if rc:
             _lib.check(rc, "hyena_fir_step")
         if not dpos:
-            ring.pos = (ring.pos + 1) % self.R
+            ring.pos = (ring.pos + 1) % ring.period
         return out
 
 
@@ -548,6 +584,7 @@ class LayerStepper:
         self.is_fir = isinstance(inner, FirStepper)
         self._fn = _lib.lib().hyena_fir_layer_step if self.is_fir else _lib.lib().hyena_iir_layer_step
         self._fn_dpos = _lib.lib().hyena_fir_layer_step_dpos
+        self._fn_far = _lib.lib().hyena_fir_layer_step_far
 
     def __call__(self, u, out):
         """u: [B, 3D] bf16 with contiguous channels; out: [B, D] bf16 (float32 allowed for the IIR step)."""
@@ -559,12 +596,19 @@ class LayerStepper:
         p.u, p.u_batch_stride = u.data_ptr(), u.stride(0)
         p.pos, p.pos_dev = (0, self.ring.pos_dev.data_ptr()) if dpos else (self.ring.pos, None)
         stream = torch.cuda.current_stream().cuda_stream
-        if self.is_fir and dpos:
+        if self.is_fir and n.far is not None:
+            rc = self._fn_far(self._pref, n.ring.buf.data_ptr(), n.R, n.ring.block, 0 if dpos else n.ring.pos,
+                              n.ring.pos_dev.data_ptr() if dpos else None, n.far.data_ptr(), n.far_rebuild(),
+                              n.w.data_ptr(), n.bias.data_ptr() if n.bias is not None else None, n.mode,
+                              out.data_ptr(), out.stride(0), B, n.D, n.G, stream)
+        elif self.is_fir and dpos:
+            n.ring.far_owner = None
             rc = self._fn_dpos(self._pref, n.ring.buf.data_ptr(), n.R, n.ring.block, n.ring.pos_dev.data_ptr(), n.w.data_ptr(),
                                n.bias.data_ptr() if n.bias is not None else None, n.mode, out.data_ptr(),
                                out.stride(0), B, n.D, n.G, stream)
         elif self.is_fir:
-            rc = self._fn(self._pref, n.ring.buf.data_ptr(), n.R, n.ring.block, n.ring.pos, n.w.data_ptr(),
+            n.ring.far_owner = None
+            rc = self._fn(self._pref, n.ring.buf.data_ptr(), n.R, n.ring.block, n.ring.pos % n.R, n.w.data_ptr(),
                           n.bias.data_ptr() if n.bias is not None else None, n.mode, out.data_ptr(), out.stride(0),
                           B, n.D, n.G, stream)
         else:
@@ -576,7 +620,7 @@ class LayerStepper:
         if not dpos:
             self.ring.pos = (self.ring.pos + 1) % self.Rf
             if self.is_fir:
-                n.ring.pos = (n.ring.pos + 1) % n.R
+                n.ring.pos = (n.ring.pos + 1) % n.ring.period
         return out
 
 
@@ -595,7 +639,7 @@ class RingClock:
         if any(r.pos_dev is not None for r in self.rings):
             raise RuntimeError("a ring is already on a clock")
         self.pos = torch.tensor([r.pos for r in self.rings], dtype=torch.int32, device=dev)
-        self.depth = torch.tensor([r.R for r in self.rings], dtype=torch.int32, device=dev)
+        self.depth = torch.tensor([r.period for r in self.rings], dtype=torch.int32, device=dev)
         for i, r in enumerate(self.rings):
             r.pos_dev = self.pos[i:i + 1]
 
