@@ -2,6 +2,7 @@
 // on the command line, allocates with hipMalloc, and verifies known answers bit for bit:
 //   hyena_mr_fwd / hyena_fir_cl_fwd   impulse response with bf16-exact taps equals the filter
 //   hyena_fir_step                    dot product over a ring cache, slot rotation
+//   hyena_fir_step_far                the same step on a deep cache read whole only every third token, 3 ring periods
 //   hyena_iir_step                    one modal update against the closed form
 //   argument errors                   negative return codes and a message
 // Usage: abi_selftest /path/to/libhyena_mi355x.so
@@ -42,6 +43,7 @@ int main(int argc, char** argv) {
 #define SYM(name) auto p_##name = (decltype(&name))dlsym(lib, #name); CHECK(p_##name, "missing symbol " #name);
     SYM(hyena_version) SYM(hyena_last_error_string) SYM(hyena_mr_fwd) SYM(hyena_fir_cl_fwd) SYM(hyena_fir_step)
     SYM(hyena_iir_step) SYM(hyena_se_fwd) SYM(hyena_fir_step_dpos) SYM(hyena_ring_advance)
+    SYM(hyena_fir_step_far) SYM(hyena_fir_far_period) SYM(hyena_fir_far_bytes)
     printf("%s\n", p_hyena_version());
     hipStream_t stream; HIP_OK(hipStreamCreate(&stream));
 
@@ -141,6 +143,54 @@ int main(int argc, char** argv) {
             CHECK(ph[0] == (step + 1) % R && ph[1] == (step - 1) % 5, "hyena_ring_advance positions after step %d: %d %d", step, ph[0], ph[1]);
         }
         printf("hyena_fir_step_dpos / hyena_ring_advance (positions in device memory): ok\n");
+    }
+
+    // ---- decode FIR step with far sums: ring [B=3][D/512=2][R=40][512] in channel blocks, taps shared by groups of
+    // 16 channels; small dyadic values, so every float32 sum is exact whatever its order and the outputs must be equal
+    // bit for bit to the host model for three periods of the ring
+    {
+        const int64_t Bs = 3, Ds = 1024, R = 40, Gs = Ds / 16, cb = 512;
+        const int64_t period = p_hyena_fir_far_period(R);
+        CHECK(period % R == 0 && period / R == p_hyena_fir_far_period(1) && period / R >= 2, "far period %lld", (long long)period);
+        std::vector<uint16_t> ring(Bs * R * Ds), u(Bs * Ds), one_s(Bs * Ds, to_bf16(1.f));
+        std::vector<float> w(Gs * (R + 1));
+        auto slot = [&](int64_t b, int64_t s, int64_t d) { return ((b * (Ds / cb) + d / cb) * R + s) * cb + d % cb; };
+        std::vector<float> hist(Bs * R * Ds);                       // hist[(b*R + i)*Ds + d]: i-th oldest sample
+        for (int64_t b = 0; b < Bs; ++b) for (int64_t i = 0; i < R; ++i) for (int64_t d = 0; d < Ds; ++d) {
+            const float val = (float)((int)((b * 7 + i * 3 + d) % 9) - 4) / 4.f;
+            hist[(b * R + i) * Ds + d] = val;
+            ring[slot(b, i, d)] = to_bf16(val);                     // counter 0: slot i is the i-th oldest
+        }
+        for (size_t i = 0; i < w.size(); ++i) w[i] = (float)((int)(i % 7) - 3) / 8.f;
+        uint16_t *d_ring = dev(ring), *d_u = dev(u), *d_1 = dev(one_s), *d_y; float *d_w = dev(w), *d_far;
+        HIP_OK(hipMalloc(&d_y, Bs * Ds * 2));
+        HIP_OK(hipMalloc(&d_far, (size_t)p_hyena_fir_far_bytes(Bs, Ds)));
+        for (int step = 0; step < 3 * R + 2; ++step) {
+            for (size_t i = 0; i < u.size(); ++i) u[i] = to_bf16((float)((int)((i + 5 * step) % 9) - 4) / 2.f);
+            HIP_OK(hipMemcpy(d_u, u.data(), u.size() * 2, hipMemcpyHostToDevice));
+            const int64_t cnt = step % period;
+            int rc = p_hyena_fir_step_far(d_u, d_1, d_1, Ds, d_ring, R, cb, cnt, nullptr, d_far, step == 0, d_w, nullptr,
+                                          HYENA_BIAS_NONE, d_y, Ds, Bs, Ds, Gs, stream);
+            CHECK(rc == 0, "hyena_fir_step_far rc=%d: %s", rc, p_hyena_last_error_string());
+            HIP_OK(hipStreamSynchronize(stream));
+            auto y = host(d_y, (size_t)(Bs * Ds));
+            for (int64_t b = 0; b < Bs; ++b) for (int64_t d = 0; d < Ds; ++d) {
+                float acc = 0.f;
+                for (int64_t i = 0; i < R; ++i) acc += w[(d / 16) * (R + 1) + i] * hist[(b * R + i) * Ds + d];
+                acc += w[(d / 16) * (R + 1) + R] * from_bf16(u[b * Ds + d]);
+                CHECK(from_bf16(y[b * Ds + d]) == from_bf16(to_bf16(acc)), "hyena_fir_step_far step %d b=%lld d=%lld got %g want %g",
+                      step, (long long)b, (long long)d, from_bf16(y[b * Ds + d]), acc);
+            }
+            for (int64_t b = 0; b < Bs; ++b) for (int64_t d = 0; d < Ds; ++d) {          // the window moves on by one sample
+                for (int64_t i = 0; i + 1 < R; ++i) hist[(b * R + i) * Ds + d] = hist[(b * R + i + 1) * Ds + d];
+                hist[(b * R + R - 1) * Ds + d] = from_bf16(u[b * Ds + d]);
+            }
+        }
+        auto rr = host(d_ring, ring.size());
+        const int64_t pos_end = (3 * R + 2) % R;
+        for (int64_t b = 0; b < Bs; ++b) for (int64_t i = 0; i < R; ++i) for (int64_t d = 0; d < Ds; d += 37)
+            CHECK(from_bf16(rr[slot(b, (pos_end + i) % R, d)]) == hist[(b * R + i) * Ds + d], "hyena_fir_step_far ring contents");
+        printf("hyena_fir_step_far (channel-blocked cache, windows of %lld tokens): ok\n", (long long)(period / R));
     }
 
     // ---- decode IIR step, real poles: state = p*state + x1v ; y = x2 * (sum r*state + D*x1v)

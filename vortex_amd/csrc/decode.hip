@@ -246,7 +246,8 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
         }
         __syncthreads();          // also orders every read of slot `pos` before its overwrite below
         if (sg != 0 || !live) return;
-#pragma unroll(NBT > 1 ? 1 : NSG - 1)
+        constexpr int RED_UNROLL = NBT > 1 ? 1 : NSG - 1;      // with far sums: one wavefront's partial sums at a time
+#pragma unroll RED_UNROLL
         for (int k = 0; k < NSG - 1; ++k) {
 #pragma unroll
             for (int jj = 0; jj < NBT; ++jj)
@@ -257,10 +258,11 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
             // what the cache adds to the later tokens of this window
 #pragma unroll
             for (int jj = 1; jj < NBT; ++jj) {
-                if (jw + jj >= NBT) break;
-                float* fp = far + ((b * NBT + jw + jj) * D + d0);
-                *(f32x4*)fp = f32x4{acc[jj][0], acc[jj][1], acc[jj][2], acc[jj][3]};
-                *(f32x4*)(fp + 4) = f32x4{acc[jj][4], acc[jj][5], acc[jj][6], acc[jj][7]};
+                if (jw + jj < NBT) {
+                    float* fp = far + ((b * NBT + jw + jj) * D + d0);
+                    *(f32x4*)fp = f32x4{acc[jj][0], acc[jj][1], acc[jj][2], acc[jj][3]};
+                    *(f32x4*)(fp + 4) = f32x4{acc[jj][4], acc[jj][5], acc[jj][6], acc[jj][7]};
+                }
             }
         }
     }
@@ -280,13 +282,14 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
             }
 #pragma unroll
             for (int k = 1; k < NBT; ++k) {
-                if (k > jw) break;
+                if (k <= jw) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float t0 = GROUPED ? w[gw + R - k] : w[(d0 + 2 * j) * W + R - k];
-                    const float t1 = GROUPED ? t0 : w[(d0 + 2 * j + 1) * W + R - k];
-                    acc[0][2 * j] = fmaf(t0, bf_lo(qn[k - 1][j]), acc[0][2 * j]);
-                    acc[0][2 * j + 1] = fmaf(t1, bf_hi(qn[k - 1][j]), acc[0][2 * j + 1]);
+                    for (int j = 0; j < 4; ++j) {
+                        const float t0 = GROUPED ? w[gw + R - k] : w[(d0 + 2 * j) * W + R - k];
+                        const float t1 = GROUPED ? t0 : w[(d0 + 2 * j + 1) * W + R - k];
+                        acc[0][2 * j] = fmaf(t0, bf_lo(qn[k - 1][j]), acc[0][2 * j]);
+                        acc[0][2 * j + 1] = fmaf(t1, bf_hi(qn[k - 1][j]), acc[0][2 * j + 1]);
+                    }
                 }
             }
         }
