@@ -271,6 +271,44 @@ int hyena_fir_layer_step_far(const hyena_proj_step* proj,
                              void* out, int64_t out_batch_stride,
                              int64_t B, int64_t D, int64_t G, void* stream);
 
+/* Modal IIR step that reads and writes the state once per window of hyena_iir_window_tokens() (4) tokens instead of
+ * every token.  No counterpart in the reference (vortex/model/engine.py:451-467 updates the state per token); same
+ * outputs up to float32 rounding.  With S the state before a window's first token t0,
+ *   Re sum_s r s_{t0+j} = far[j] + sum_{k<=j} g[k] u_{t0+j-k},  far[j] = Re sum_s r p^(j+1) S,  g[k] = Re sum_s r p^k:
+ * on the first token of a window the kernel folds the window before into the stored state and forms far[]; on the
+ * other tokens it reads neither state nor poles.  Windows are staggered over the batch elements.  The caller owns
+ *   hist [B][W][D] bf16 (the last W inputs x1*v; contents owned by these calls), far [B][W][D] float32,
+ *   g [G][W] float32 (from the caller: g[k] = Re sum_s residues * poles^k), W = hyena_iir_window_tokens(),
+ * counts tokens in cnt = token % W (or cnt_dev: the counter in device memory, advanced with hyena_ring_advance,
+ * depth W) and passes warm = the number of tokens stepped with these calls since `state` was last exact (0 on the
+ * first call; anything >= W means "W or more").  Between two windows the `state` tensor lags the tokens by up to W
+ * inputs; hyena_iir_window_flush folds them in (then restart with warm = 0), e.g. before anything else reads the
+ * state.  Available for 16 states, 16-byte aligned gates with D % 8 == 0, and (in the layer step) the featurizer
+ * maps that have a vector form (hyena_iir_window_supported); other cases return HYENA_ENOSUP: use hyena_iir_step. */
+typedef struct hyena_iir_window {
+    void* hist;
+    float* far;
+    const float* g;
+    int64_t cnt;
+    const int32_t* cnt_dev;
+    int warm;
+    int reserved;                /* 0 */
+} hyena_iir_window;
+int64_t hyena_iir_window_tokens(void);
+int hyena_iir_window_supported(int64_t B, int64_t D, int64_t S, int is_complex);
+int hyena_iir_step_win(const void* x1, const void* x2, const void* v, int64_t in_batch_stride,
+                       float* state, const float* poles, const float* residues, int is_complex,
+                       const float* Dcoef, int d_is_bf16,
+                       void* out, int out_is_fp32, int64_t out_batch_stride,
+                       int64_t B, int64_t D, int64_t G, int64_t S, const hyena_iir_window* win, void* stream);
+int hyena_iir_layer_step_win(const hyena_proj_step* proj,
+                             float* state, const float* poles, const float* residues, int is_complex,
+                             const float* Dcoef, int d_is_bf16,
+                             void* out, int out_is_fp32, int64_t out_batch_stride,
+                             int64_t B, int64_t D, int64_t G, int64_t S, const hyena_iir_window* win, void* stream);
+int hyena_iir_window_flush(float* state, const float* poles, const float* residues, int is_complex,
+                           int64_t B, int64_t D, int64_t G, int64_t S, const hyena_iir_window* win, void* stream);
+
 /* Channel-last operand [B][L][D]: element (b, t, d) at ptr + b*batch_stride + t*time_stride + d (elements).
  * This is the (batch, seqlen, groups, group_dim) layout of vortex/ops/hyena_se/fwd.py:17-43 with D = groups*group_dim. */
 typedef struct hyena_cl {

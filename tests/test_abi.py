@@ -87,6 +87,23 @@ def test_new_entry_points_validate_before_touching_the_device():
     assert L.hyena_fir_step_far(P, None, None, 512, P, 127, 512, per, None, P, 0, P, None, 0, P, 512, 1, 512, 32, None) == -1
     assert L.hyena_fir_step_far(P, None, None, 512, P, 127, 512, per - 1, None, P, 1, P, None, 0, P, 512, 0, 512, 32, None) == 0
     assert L.hyena_fir_layer_step_far(None, P, 127, 512, 0, None, P, 0, P, None, 0, P, 512, 1, 512, 32, None) == -1
+    # windowed modal step: 16 states and B*D of 65536 and more, all three window buffers, the counter inside the window
+    W = L.hyena_iir_window_tokens()
+    assert W >= 2 and L.hyena_iir_window_supported(64, 4096, 16, 0) == 1 and L.hyena_iir_window_supported(64, 4096, 16, 1) == 1
+    assert L.hyena_iir_window_supported(64, 4096, 8, 0) == 0 and L.hyena_iir_window_supported(8, 4096, 16, 0) == 0
+    assert L.hyena_iir_window_supported(64, 4100, 16, 0) == 0
+    iw = lambda *a: ref(_lib.IirWindow(*a))
+    win_args = lambda w, B=64, D=4096, S=16: (P, P, P, D, P, P, P, 0, P, 0, P, 0, D, B, D, D, S, w, None)
+    assert L.hyena_iir_step_win(*win_args(None)) == -1
+    assert L.hyena_iir_step_win(*win_args(iw(P, None, P, 0, None, 0, 0))) == -1          # no far buffer
+    assert L.hyena_iir_step_win(*win_args(iw(P, P, P, W, None, 0, 0))) == -1             # counter past the window
+    assert L.hyena_iir_step_win(*win_args(iw(P, P, P, 0, None, -1, 0))) == -1            # warm below zero
+    assert L.hyena_iir_step_win(*win_args(iw(P, P, P, 0, None, 0, 0), S=8)) == -3
+    assert L.hyena_iir_step_win(*win_args(iw(P, P, P, 0, None, 0, 0), B=4)) == -3
+    assert L.hyena_iir_layer_step_win(None, P, P, P, 0, P, 0, P, 0, 64, 64, 4096, 4096, 16, iw(P, P, P, 0, None, 0, 0),
+                                      None) == -1
+    assert L.hyena_iir_window_flush(P, P, P, 0, 64, 4096, 4096, 16, None, None) == -1
+    assert L.hyena_iir_window_flush(P, P, P, 0, 64, 4096, 4096, 16, iw(None, None, None, 0, None, 1, 0), None) == -1
     assert L.hyena_ring_advance(None, P, 4, None) == -1 and L.hyena_ring_advance(P, P, -1, None) == -1
     assert L.hyena_ring_advance(P, P, 0, None) == 0
     ps = _lib.ProjStep(P, 192, P, 2, 5, P, None, 64, 0, 64, 1, 0, None)

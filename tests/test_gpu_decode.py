@@ -185,3 +185,74 @@ def test_iir_step_sequence_vs_oracle(cplx, G, S):
         y = va.iir_step(x1.cuda(), x2.cuda(), v.cuda(), state, poles, r.cuda(), Dp.cuda())
         assert (y.float().cpu() - y_ref.float()).abs().max() <= 2e-2 * y_ref.float().abs().max()
     assert (state.cpu() - st_ref).abs().max() <= 1e-4 * st_ref.abs().max()
+
+
+@pytest.mark.parametrize("cplx,B,D,G,fused,on_clock", [
+    (True, 64, 2048, 128, False, False),     # complex poles, grouped
+    (False, 64, 4096, 4096, False, False),   # vortex's own: real poles, one filter per channel
+    (True, 50, 2048, 2048, True, False),     # layer step from the projection (interleaved gates)
+    (False, 37, 2056, 257, True, True),      # counter in device memory; D not a multiple of 256
+    (True, 70, 1000, 125, False, False),     # D a multiple of 8 only
+])
+def test_iir_step_windowed_state(cplx, B, D, G, fused, on_clock):
+    """The stepper that reads and writes the modal state once per window of four tokens (windows staggered over the
+    batch elements): outputs against the oracle on every token, the state after flush() against the oracle's, a flush
+    in the middle of the run (windows restart), and the plain stepper on a copy of the state for comparison."""
+    from vortex_amd import _lib, ops
+    S, W = 16, _lib.lib().hyena_iir_window_tokens()
+    assert _lib.lib().hyena_iir_window_supported(B, D, S, int(cplx))
+    g = torch.Generator().manual_seed(D + cplx)
+    lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(G, S, seed=9)
+    Dp = torch.randn(D, generator=g).bfloat16()
+    lpD, rD = lp.repeat_interleave(D // G, 0), r.repeat_interleave(D // G, 0)
+    dt = torch.complex64 if cplx else torch.float32
+    st_ref = (torch.randn(B, D, S, generator=g) * 0.5).to(dt)
+    states = [st_ref.clone().cuda() for _ in range(2)]
+    poles = torch.exp(lp[..., 0]).cuda()
+    win = ops.IirStepper(states[0], poles, r.cuda(), Dp.cuda(), windowed=True)
+    plain = ops.IirStepper(states[1], poles, r.cuda(), Dp.cuda())
+    assert win.win is not None and plain.win is None
+    C = 3 * D
+    if fused:
+        wf = torch.randn(C, 1, 3, generator=g) / 3 ** 0.5
+        fst = torch.randn(B, C, 2, generator=g).bfloat16()
+        frings = [va.FirRing.from_reference(fst.cuda()) for _ in range(2)]
+        cmap = ops.gate_channel_map(D, interleave=True)
+        steps = [ops.LayerStepper(fr, wf.reshape(C, 3).cuda(), None, cmap, n) for fr, n in zip(frings, (win, plain))]
+        assert win.win is not None
+        ref_f = fst
+    clock = None
+    ya, yb = (torch.empty(B, D, dtype=torch.bfloat16, device="cuda") for _ in range(2))
+    as_real = lambda t: torch.view_as_real(t) if cplx else t
+    for step in range(4 * W + 2):
+        if on_clock and step == W + 1:              # from here on the counters live in device memory
+            clock = ops.RingClock([win] + ([frings[0]] if fused else []))
+        if fused:
+            u = torch.randn(B, C, generator=g).bfloat16()
+            z, ref_f = O.step_fir(u, ref_f, wf)
+            x2, x1, v = O.interleave(z).split([D] * 3, dim=1)
+            steps[0](u.cuda(), ya)
+            steps[1](u.cuda(), yb)
+        else:
+            x1, x2, v = (torch.randn(B, D, generator=g).bfloat16() for _ in range(3))
+            win(x1.cuda(), x2.cuda(), v.cuda(), ya)
+            plain(x1.cuda(), x2.cuda(), v.cuda(), yb)
+        if clock is not None:
+            clock.advance()
+        y_ref, st_ref = O.step_iir(x2, x1, v, Dp, rD, lpD, st_ref)
+        y_ref = (y_ref.real if cplx else y_ref).float()
+        assert (ya.float().cpu() - y_ref).abs().max() <= 2e-2 * y_ref.abs().max(), step
+        d = (ya.float() - yb.float()).abs().max().item()
+        assert d <= 2e-2 * y_ref.abs().max().item(), (step, d)
+        if step in (W - 1, 2 * W):                  # the state as anyone else may read it
+            win.flush()
+            sr = as_real(st_ref)
+            assert (as_real(states[0]).cpu() - sr).abs().max() <= (2e-3 if fused else 1e-4) * sr.abs().max(), step
+            assert win.warm == 0
+    assert not torch.equal(as_real(states[0]).cpu(), as_real(states[1]).cpu())      # the state lags until the flush
+    win.flush()
+    sr = as_real(st_ref)
+    assert (as_real(states[0]).cpu() - sr).abs().max() <= (2e-3 if fused else 1e-4) * sr.abs().max()
+    assert (as_real(states[0]) - as_real(states[1])).abs().max() <= 1e-4 * sr.abs().max()
+    if clock is not None:
+        clock.release()

@@ -77,6 +77,32 @@ def test_recorded_token_step_matches_eager_generation(L, attn):
     assert torch.equal(scores_g2, scores_g)
 
 
+def test_windowed_modal_state_in_generation():
+    # at batch x width of 65536 and more the Hyena-LI decode step keeps its modal state in windows of several tokens:
+    # the recorded step replays the same kernels as the eager loop bit for bit, both agree with a longer prefill, and
+    # the plain per-token state update gives the same logits up to bf16 rounding
+    from vortex_amd import ops
+    cfg = dict(EVO2_7B, hidden_size=1024, num_layers=3, num_attention_heads=8, inner_mlp_size=1024,
+               hcs_filter_groups=8, hcm_filter_groups=8, hcl_filter_groups=1024, pattern=("hcs", "hcm", "hcl"))
+    m = StripedHyena2(cfg, seed=11, device="cuda").to_inference("cuda")
+    B, L, n = 64, 160, 15
+    ids = torch.randint(0, 512, (B, L + n), device="cuda", generator=torch.Generator(device="cuda").manual_seed(12))
+    toks_e, scores_e = m.generate(ids[:, :L], n, forced=ids[:, L:])
+    inner = m.blocks[2].filter._decode["inner"]
+    assert isinstance(inner, ops.IirStepper) and inner.win is not None
+    toks_g, scores_g = m.generate(ids[:, :L], n, forced=ids[:, L:], graph=True)
+    assert torch.equal(scores_g, scores_e)
+    want = m(ids).float()[:, L - 1:L + n - 1]
+    err = (scores_e.float() - want).abs().max() / want.abs().max()
+    assert err <= 3e-2, err
+    for blk in m.blocks:
+        blk.filter.window_decode_state = False
+    _, scores_p = m.generate(ids[:, :L], n, forced=ids[:, L:])
+    assert m.blocks[2].filter._decode["inner"].win is None
+    err = (scores_e.float() - scores_p.float()).abs().max() / want.abs().max()
+    assert err <= 2e-2, err
+
+
 def test_recorded_step_then_eager_steps():
     # release() hands ring positions back to the host: eager steps after recorded ones continue the same sequence
     from vortex_amd.model import RecordedDecodeStep

@@ -17,6 +17,8 @@ EXPORTS = [
     "hyena_fir_layer_step", "hyena_iir_layer_step", "hyena_fir_cl_fwd", "hyena_fir_layer_fwd",
     "hyena_fir_step_dpos", "hyena_fir_layer_step_dpos", "hyena_ring_advance",
     "hyena_fir_far_period", "hyena_fir_far_bytes", "hyena_fir_step_far", "hyena_fir_layer_step_far",
+    "hyena_iir_window_tokens", "hyena_iir_window_supported", "hyena_iir_step_win", "hyena_iir_layer_step_win",
+    "hyena_iir_window_flush",
 ]
 
 
@@ -30,6 +32,12 @@ class ProjStep(Structure):
     _fields_ = [("u", c_void_p), ("u_batch_stride", c_int64), ("ring", c_void_p), ("Rf", c_int64), ("pos", c_int64),
                 ("w", c_void_p), ("bias", c_void_p), ("ch_inner", c_int64), ("ch_outer", c_int64),
                 ("gate_stride", c_int64), ("ch_stride", c_int64), ("flip_x1x2", c_int), ("pos_dev", c_void_p)]
+
+
+class IirWindow(Structure):
+    """hyena_iir_window: the buffers and counters of the windowed modal step."""
+    _fields_ = [("hist", c_void_p), ("far", c_void_p), ("g", c_void_p), ("cnt", c_int64), ("cnt_dev", c_void_p),
+                ("warm", c_int), ("reserved", c_int)]
 
 
 class Cl(Structure):
@@ -87,6 +95,16 @@ def lib():
     L.hyena_fir_layer_step_dpos.argtypes = [P, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                             c_int64, c_int64, c_int64, c_int64, c_void_p]
     L.hyena_ring_advance.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
+    WN = POINTER(IirWindow)
+    L.hyena_iir_window_tokens.argtypes = []
+    L.hyena_iir_window_supported.argtypes = [c_int64, c_int64, c_int64, c_int]
+    L.hyena_iir_step_win.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int,
+                                     c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                     WN, c_void_p]
+    L.hyena_iir_layer_step_win.argtypes = [P, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+                                           c_int64, c_int64, c_int64, c_int64, c_int64, WN, c_void_p]
+    L.hyena_iir_window_flush.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, WN,
+                                         c_void_p]
     L.hyena_fir_far_period.argtypes = [c_int64]
     L.hyena_fir_far_bytes.argtypes = [c_int64, c_int64]
     L.hyena_fir_step_far.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p,
@@ -102,7 +120,7 @@ def lib():
     for name in EXPORTS:
         fn = getattr(L, name)
         if name not in ("hyena_version", "hyena_last_error_string"):
-            fn.restype = c_int64 if name in ("hyena_li_plan_bytes", "hyena_fir_far_period", "hyena_fir_far_bytes") else c_int
+            fn.restype = c_int64 if name in ("hyena_li_plan_bytes", "hyena_fir_far_period", "hyena_fir_far_bytes", "hyena_iir_window_tokens") else c_int
     _lib = L
     return L
 

@@ -128,6 +128,9 @@ class HyenaCascade(nn.Module):
         self._plan = None
         self._decode = None
         self.fuse_decode = True        # one launch per decode step where the fused layer-step kernels apply
+        # decode: the modal state is read and written once per four tokens (ops.IirStepper windowed);
+        # inference_params.state_dict then lags the tokens by up to four inputs until flush_decode_state()
+        self.window_decode_state = True
         self.fuse_prefill = True       # one launch per SE / MR prefill where the fused layer kernel applies
         self._f32_cache = {}
 
@@ -334,7 +337,8 @@ class HyenaCascade(nn.Module):
         else:
             st = inference_params.state_dict[i]
             poles = torch.exp(self.log_poles.detach())[..., 0].contiguous()
-            d["inner"] = ops.IirStepper(st, poles, self.residues.detach(), self.D.detach())
+            d["inner"] = ops.IirStepper(st, poles, self.residues.detach(), self.D.detach(),
+                                        windowed=self.window_decode_state)
         d["layer"] = self._fused_step(ring, d["inner"])
         self._decode = d
         return d
@@ -352,6 +356,13 @@ class HyenaCascade(nn.Module):
             return None
         return ops.LayerStepper(ring, self.short_filter_weight.detach().reshape(3 * self.hidden_size, Ks),
                                 self.short_filter_bias, cmap, inner, flip_x1x2=self.hyena_flip_x1x2)
+
+    def flush_decode_state(self):
+        """Brings inference_params.state_dict[layer_idx] up to the last token (the windowed modal step lets it lag by up
+        to four inputs); call it before reading or saving the state during decode.  No-op otherwise."""
+        inner = (self._decode or {}).get("inner")
+        if isinstance(inner, ops.IirStepper):
+            inner.flush()
 
     def _growing_step(self, u, d):
         """Decode step while a cache still holds fewer samples than its filter needs (prompt shorter than the

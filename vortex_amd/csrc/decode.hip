@@ -354,96 +354,229 @@ struct alignas(4 * N) StateVec {
 // FEAT (fused featurizer step): 0 none; 2 lanes 0..2 of a lane group evaluate gates x2, x1, v of their channel
 // with scalar loads (any channel map); 1 / 3 the block's first wavefronts evaluate the gates of all its
 // channels with 16-byte loads (unit-stride / interleaved map, as in the FIR step) and hand them over in LDS.
-template <int S, bool CPLX, int FEAT, int NB>
+//
+// WIN > 1: the state is read and written once per window of WIN tokens instead of every token.  With S the
+// state before the window's first token t0,  s_{t0+j} = p^(j+1) S + sum_{k<=j} p^k u_{t0+j-k},  so
+//   Re sum_s r s_{t0+j} = far[j] + sum_{k<=j} g[k] u_{t0+j-k},   far[j] = Re sum_s r p^(j+1) S,   g[k] = Re sum_s r p^k.
+// Windows are staggered over the batch elements, place jw = (cnt + b) % WIN; a block row takes NB batch elements of
+// one residue class b % WIN, so that they are at the same place of their windows.  On the first token of its window
+// (mode 1) a batch element's blocks fold the inputs of the window before (kept in `hist`, [B][WIN][D] bf16, slot =
+// token % WIN) into the stored state, S = p^WIN S' + sum_k p^k u_{t0-1-k}, write it back and form far[0..WIN-1]
+// ([B][WIN][D] float32).  On the other tokens (mode 2) nothing of the state or the poles is touched: the work is one
+// lane per channel, 256 channels per block, and the rest of the batch element's blocks leave at once.
+// `warm` = tokens stepped this way since the stored state was last exact (saturating at WIN): a batch element steps
+// the plain way (mode 0) until its first window begins (warm >= jw fails), and a window's first token folds WIN
+// pending inputs only if the window before it existed (warm >= WIN).  flush != 0 (mode 3): no token is processed; the
+// pending inputs are folded into the state, which is exact afterwards.
+struct WinArgs {
+    bf16_t* hist;          // [B][WIN][D]
+    float* far;            // [B][WIN][D]
+    const float* g;        // [G][WIN]
+    int cnt;               // token index modulo WIN
+    const int* cnt_dev;    // when set, the counter lives in device memory
+    int warm, flush;
+};
+
+template <int S, bool CPLX, int FEAT, int NB, int WIN>
 __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict__ x1, const bf16_t* __restrict__ x2,
                                                        const bf16_t* __restrict__ v, int64_t in_bs, ProjArgs pj,
                                                        float* __restrict__ state, const float* __restrict__ poles,
                                                        const float* __restrict__ residues,
                                                        const float* __restrict__ Dcoef, int d_is_bf16,
                                                        void* __restrict__ out, int out_is_fp32, int64_t out_bs,
-                                                       int64_t B, int64_t D, int dg) {
+                                                       int64_t B, int64_t D, int dg, WinArgs wa) {
     constexpr int FPS = CPLX ? 2 : 1;              // floats per state
     constexpr int VEC = S * FPS >= 4 ? 4 : S * FPS; // floats of state per lane (1 and 2 only where a channel has no more)
     constexpr int LPB = S * FPS / VEC;             // lanes per channel
     using fvec = StateVec<VEC>;
     constexpr int ND = 256 / LPB;                  // channels per block
-    __shared__ float zs[(FEAT == 1 || FEAT == 3) ? NB * 3 * ND : 1];     // [j][gate-major or interleaved][channel]
+    constexpr bool VFEAT = FEAT == 1 || FEAT == 3;
+    static_assert(WIN <= 1 || (VEC == 4 && FEAT != 2), "windows: 16-byte state pieces, vector featurizer");
+    __shared__ float zs[VFEAT ? (WIN > 1 && 3 * 256 > NB * 3 * ND ? 3 * 256 : NB * 3 * ND) : 1];  // [j][gate-major or interleaved][channel]
     if (FEAT != 0) pj.resolve_pos();
+    // ---- what this batch element does with this token: 0 plain step, 1 first token of a window, 2 inside a window, 3 flush
+    int mode = 0, jw = 0, cnt = 0, npend = 0;
+    if (WIN > 1) {
+        cnt = wa.cnt_dev ? (int)((uint32_t)*wa.cnt_dev % (uint32_t)WIN) : wa.cnt;
+        jw = (int)((uint32_t)(cnt + blockIdx.y) % (uint32_t)WIN);          // blockIdx.y % WIN is the row's residue class
+        if (wa.flush) {
+            mode = 3;                              // inputs since the window began: jw of them, or a whole window
+            npend = jw > 0 ? (wa.warm >= jw ? jw : 0) : (wa.warm >= WIN ? WIN : 0);
+            if (npend == 0) return;                // the stored state is exact already
+        } else if (wa.warm >= jw) {
+            mode = jw == 0 ? 1 : 2;
+            npend = wa.warm >= WIN ? WIN : 0;
+        }
+    }
+    // batch element j of this block row: NB consecutive ones, or (windows) NB of one residue class b % WIN
+    auto bj = [&](int j) -> int64_t {
+        if (WIN > 1) return (int64_t)WIN * ((int64_t)NB * (blockIdx.y / WIN) + j) + blockIdx.y % WIN;
+        return (int64_t)blockIdx.y * NB + j;
+    };
+    if (WIN > 1 && mode == 2) {
+        // ---- inside a window: far[jw] and the inputs since the window began; one lane per channel
+        const uint32_t dblk = blockIdx.x * 256;
+        if (dblk >= (uint32_t)D) return;
+        const uint32_t dch = dblk + threadIdx.x;
+        const bool ok = dch < (uint32_t)D;
+        const uint32_t dc = ok ? dch : 0;
+      for (int jb = 0; jb < NB; ++jb) {
+        const int64_t b = bj(jb);
+        if (b >= B) break;                         // uniform: the rest of the class is beyond the batch
+        float a, c, gate2;
+        if (VFEAT) {
+            if (jb > 0) __syncthreads();           // the gates of the batch element before have been picked up
+            const int r = threadIdx.x;             // piece r covers zs columns 8r..8r+7 (96 pieces for 3 x 256 channels)
+            if (r < 96) {
+                const uint32_t dl0 = FEAT == 3 ? 0 : (uint32_t)(8 * r) % 256;
+                const uint32_t ch = FEAT == 3 ? 3 * dblk + 8 * r : pj.chan((uint32_t)(8 * r) / 256, dblk + dl0);
+                const bool okp = FEAT == 3 ? 3 * dblk + 8 * r < 3 * (uint32_t)D : dblk + dl0 < (uint32_t)D;
+                if (okp) {
+                    float z[8];
+                    const u32x4 un = proj_step8(pj, b, ch, z);
+                    proj_store8(pj, b, ch, un);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) zs[8 * r + k] = z[k];
+                }
+            }
+            __syncthreads();
+            const int dl = threadIdx.x;
+            const float g2 = FEAT == 3 ? zs[3 * dl] : zs[dl], g1 = FEAT == 3 ? zs[3 * dl + 1] : zs[256 + dl];
+            c = FEAT == 3 ? zs[3 * dl + 2] : zs[512 + dl];
+            a = pj.flip ? g2 : g1;
+            gate2 = pj.flip ? g1 : g2;
+        } else {
+            a = bf_to_f(x1[b * in_bs + dc]);
+            c = bf_to_f(v[b * in_bs + dc]);
+            gate2 = bf_to_f(x2[b * in_bs + dc]);
+        }
+        if (!ok) continue;
+        const float x1v = round_bf(a * c);
+        const float* gp = wa.g + (int64_t)(dc / (uint32_t)dg) * WIN;
+        float part = wa.far[(b * WIN + jw) * D + dc] + gp[0] * x1v;
+#pragma unroll
+        for (int k = 1; k < WIN; ++k) {
+            int sl = cnt - k;
+            if (sl < 0) sl += WIN;
+            if (k <= jw) part = fmaf(gp[k], bf_to_f(wa.hist[(b * WIN + sl) * D + dc]), part);
+        }
+        float dx = Dcoef[dc] * x1v;
+        if (d_is_bf16) dx = round_bf(dx);
+        const float y = gate2 * (part + dx);
+        if (out_is_fp32) ((float*)out)[b * out_bs + dc] = y;
+        else ((bf16_t*)out)[b * out_bs + dc] = (bf16_t)f_to_bf_bits(y);
+        wa.hist[(b * WIN + cnt) * D + dc] = (bf16_t)f_to_bf_bits(x1v);
+      }
+        return;
+    }
     const uint32_t idx = blockIdx.x * 256 + threadIdx.x;        // (channel, lane of the group)
     const int q = (int)(idx % LPB);
     uint32_t d = idx / LPB;
     const bool chan_live = d < (uint32_t)D;
     if (!chan_live) d = 0;
-    const int64_t b0 = (int64_t)blockIdx.y * NB;
     const uint32_t g = d / (uint32_t)dg;
     fvec st[NB];
     bool live[NB];
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
-        live[j] = chan_live && b0 + j < B;
-        const int64_t bd = live[j] ? (b0 + j) * D + d : 0;
+        live[j] = chan_live && bj(j) < B;
+        const int64_t bd = live[j] ? bj(j) * D + d : 0;
         st[j] = *(const fvec*)(state + (bd * S) * FPS + q * VEC);
+    }
+    // the inputs a window's first token (or a flush) folds into the state, newest first: u_{t-1-k}
+    float pend[NB][WIN > 1 ? WIN : 1];
+    if (WIN > 1 && (mode == 1 || mode == 3)) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+            for (int k = 0; k < WIN; ++k) {
+                int sl = cnt - 1 - k;
+                if (sl < 0) sl += WIN;
+                const int64_t bb = live[j] ? bj(j) : 0;
+                pend[j][k] = k < npend ? bf_to_f(wa.hist[(bb * WIN + sl) * D + d]) : 0.f;
+            }
     }
     const fvec pp = *(const fvec*)(poles + ((int64_t)g * S) * FPS + q * VEC);
     const fvec rr = *(const fvec*)(residues + ((int64_t)g * S) * FPS + q * VEC);
-    const float dco = Dcoef[d];
+    const float dco = mode != 3 ? Dcoef[d] : 0.f;      // a flush has no token: no gates, no output, no Dcoef
     // fused featurizer: lanes 0..2 of the group evaluate gates x2, x1, v of every batch element first (their
     // loads overlap), the ring-slot stores follow, and only then the state updates start
     float zf[NB];
-    if (FEAT == 1 || FEAT == 3) {
-        static_assert(ND % 8 == 0, "whole 8-channel pieces per block");
-        constexpr int PPB = 3 * ND / 8;            // 8-channel pieces per batch element
-        const uint32_t dblk = blockIdx.x * ND;
-        const int e = threadIdx.x;
-        if (e < NB * PPB) {
-            const int j = e / PPB, r = e - j * PPB;
-            // piece r covers zs columns 8r..8r+7: interleaved order (column = 3*dl + gate) or gate-major (gate*ND + dl)
-            const uint32_t dl0 = FEAT == 3 ? 0 : (uint32_t)(8 * r) % ND;
-            const uint32_t ch = FEAT == 3 ? 3 * dblk + 8 * r : pj.chan((uint32_t)(8 * r) / ND, dblk + dl0);
-            const bool ok = b0 + j < B && (FEAT == 3 ? 3 * dblk + 8 * r < 3 * (uint32_t)D : dblk + dl0 < (uint32_t)D);
-            if (ok) {
-                float z[8];
-                const u32x4 un = proj_step8(pj, b0 + j, ch, z);
-                proj_store8(pj, b0 + j, ch, un);
+    if (mode != 3) {
+        if (VFEAT) {
+            static_assert(ND % 8 == 0, "whole 8-channel pieces per block");
+            constexpr int PPB = 3 * ND / 8;            // 8-channel pieces per batch element
+            const uint32_t dblk = blockIdx.x * ND;
+            const int e = threadIdx.x;
+            if (e < NB * PPB) {
+                const int j = e / PPB, r = e - j * PPB;
+                // piece r covers zs columns 8r..8r+7: interleaved order (column = 3*dl + gate) or gate-major (gate*ND + dl)
+                const uint32_t dl0 = FEAT == 3 ? 0 : (uint32_t)(8 * r) % ND;
+                const uint32_t ch = FEAT == 3 ? 3 * dblk + 8 * r : pj.chan((uint32_t)(8 * r) / ND, dblk + dl0);
+                const bool ok = bj(j) < B && (FEAT == 3 ? 3 * dblk + 8 * r < 3 * (uint32_t)D : dblk + dl0 < (uint32_t)D);
+                if (ok) {
+                    float z[8];
+                    const u32x4 un = proj_step8(pj, bj(j), ch, z);
+                    proj_store8(pj, bj(j), ch, un);
 #pragma unroll
-                for (int k = 0; k < 8; ++k) zs[(j * 3 * ND) + 8 * r + k] = z[k];
-            }
-        }
-        __syncthreads();
-    } else if (FEAT == 2) {
-        static_assert(FEAT != 2 || LPB >= 4, "the scalar fused featurizer needs three lanes per channel");
-        bf16_t un[NB];
-#pragma unroll
-        for (int j = 0; j < NB; ++j) {
-            zf[j] = 0.f;
-            un[j] = 0;
-            if (q < 3) {
-                const int64_t b = live[j] ? b0 + j : 0;
-                const uint32_t ch = pj.chan((uint32_t)q, d);
-                const bf16_t* rb = pj.ring + (b * pj.Rf) * pj.C + ch;
-                un[j] = pj.u[b * pj.u_bs + ch];
-                float acc = 0.f;
-                for (int i = 0; i < pj.Rf; ++i) {
-                    int s = pj.pos + i;
-                    if (s >= pj.Rf) s -= pj.Rf;
-                    acc = fmaf(pj.w[(int64_t)i * pj.C + ch], bf_to_f(rb[(int64_t)s * pj.C]), acc);
+                    for (int k = 0; k < 8; ++k) zs[(j * 3 * ND) + 8 * r + k] = z[k];
                 }
-                acc = fmaf(pj.w[(int64_t)pj.Rf * pj.C + ch], bf_to_f(un[j]), acc);
-                if (pj.bias) acc += pj.bias[ch];
-                zf[j] = round_bf(acc);
+            }
+            __syncthreads();
+        } else if (FEAT == 2) {
+            static_assert(FEAT != 2 || LPB >= 4, "the scalar fused featurizer needs three lanes per channel");
+            bf16_t un[NB];
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                zf[j] = 0.f;
+                un[j] = 0;
+                if (q < 3) {
+                    const int64_t b = live[j] ? bj(j) : 0;
+                    const uint32_t ch = pj.chan((uint32_t)q, d);
+                    const bf16_t* rb = pj.ring + (b * pj.Rf) * pj.C + ch;
+                    un[j] = pj.u[b * pj.u_bs + ch];
+                    float acc = 0.f;
+                    for (int i = 0; i < pj.Rf; ++i) {
+                        int s = pj.pos + i;
+                        if (s >= pj.Rf) s -= pj.Rf;
+                        acc = fmaf(pj.w[(int64_t)i * pj.C + ch], bf_to_f(rb[(int64_t)s * pj.C]), acc);
+                    }
+                    acc = fmaf(pj.w[(int64_t)pj.Rf * pj.C + ch], bf_to_f(un[j]), acc);
+                    if (pj.bias) acc += pj.bias[ch];
+                    zf[j] = round_bf(acc);
+                }
+            }
+            if (q < 3) {
+#pragma unroll
+                for (int j = 0; j < NB; ++j)
+                    if (live[j]) pj.ring[((bj(j) * pj.Rf) + pj.pos) * pj.C + pj.chan((uint32_t)q, d)] = un[j];
             }
         }
-        if (q < 3) {
+    }
+    // powers of the poles a window needs: pw[m] = p^(m+1), m = 0 .. WIN-1 (state-wise; complex pairs or 4 reals)
+    fvec pw[WIN > 1 ? WIN : 1];
+    if (WIN > 1 && (mode == 1 || mode == 3)) {
+        pw[0] = pp;
 #pragma unroll
-            for (int j = 0; j < NB; ++j)
-                if (live[j]) pj.ring[(((b0 + j) * pj.Rf) + pj.pos) * pj.C + pj.chan((uint32_t)q, d)] = un[j];
+        for (int m = 1; m < WIN; ++m) {
+            if (CPLX) {
+#pragma unroll
+                for (int k = 0; k < VEC; k += 2) {
+                    pw[m][k] = pw[m - 1][k] * pp[k] - pw[m - 1][k + 1] * pp[k + 1];
+                    pw[m][k + 1] = pw[m - 1][k] * pp[k + 1] + pw[m - 1][k + 1] * pp[k];
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) pw[m][k] = pw[m - 1][k] * pp[k];
+            }
         }
     }
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
-        const int64_t b = live[j] ? b0 + j : 0;
-        float a, c, gate2 = 0.f;
-        if (FEAT == 1 || FEAT == 3) {
+        const int64_t b = live[j] ? bj(j) : 0;
+        float a = 0.f, c = 0.f, gate2 = 0.f;
+        if (mode == 3) {
+        } else if (VFEAT) {
             const int dl = threadIdx.x / LPB;
             const float* zj = zs + j * 3 * ND;
             const float g2 = FEAT == 3 ? zj[3 * dl] : zj[dl], g1 = FEAT == 3 ? zj[3 * dl + 1] : zj[ND + dl];
@@ -461,33 +594,91 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
             c = bf_to_f(v[b * in_bs + d]);
         }
         const float x1v = round_bf(a * c);
-        fvec ns;
         float part = 0.f;
-        if (CPLX) {
-            // (pr + i pi)(sr + i si) + x1v, then Re(r*s)
+        if (WIN > 1 && mode != 0) {
+            // first token of a window (or a flush): fold the pending inputs, S = p^n S' + sum_k p^k u_{t-1-k}
+            fvec ns = st[j];
+            if (npend > 0) {
 #pragma unroll
-            for (int k = 0; k < VEC; k += 2) {
-                ns[k] = fmaf(pp[k], st[j][k], -pp[k + 1] * st[j][k + 1]) + x1v;
-                ns[k + 1] = fmaf(pp[k], st[j][k + 1], pp[k + 1] * st[j][k]);
+                for (int m = 0; m < WIN; ++m) {          // p^npend, picked without indexing registers
+                    if (m + 1 == npend) {
+                        if (CPLX) {
+#pragma unroll
+                            for (int k = 0; k < VEC; k += 2) {
+                                ns[k] = pw[m][k] * st[j][k] - pw[m][k + 1] * st[j][k + 1];
+                                ns[k + 1] = pw[m][k] * st[j][k + 1] + pw[m][k + 1] * st[j][k];
+                            }
+                        } else {
+#pragma unroll
+                            for (int k = 0; k < VEC; ++k) ns[k] = pw[m][k] * st[j][k];
+                        }
+                    }
+                }
+                // + u_{t-1} (p^0) + p u_{t-2} + ...   (pend[j][k] is zero from k = npend on)
+#pragma unroll
+                for (int k = 0; k < VEC; k += (CPLX ? 2 : 1)) ns[k] += pend[j][0];
+#pragma unroll
+                for (int m = 1; m < WIN; ++m)
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) ns[k] = fmaf(pw[m - 1][k], pend[j][m], ns[k]);
+                if (live[j]) *(fvec*)(state + ((b * D + d) * S) * FPS + q * VEC) = ns;
             }
-            if (VEC == 4) part = (rr[0] * ns[0] - rr[1] * ns[1]) + (rr[2] * ns[2] - rr[3] * ns[3]);
-            else part = rr[0] * ns[0] - rr[1] * ns[1];
+            if (mode == 1) {
+                // far[m] = Re sum_s r p^(m+1) S: this lane's states, then the lane group
+                float fm[WIN > 1 ? WIN : 1];
+#pragma unroll
+                for (int m = 0; m < WIN; ++m) {
+                    if (CPLX) {
+                        float t = 0.f;
+#pragma unroll
+                        for (int k = 0; k < VEC; k += 2) {
+                            const float zr = pw[m][k] * ns[k] - pw[m][k + 1] * ns[k + 1];
+                            const float zi = pw[m][k] * ns[k + 1] + pw[m][k + 1] * ns[k];
+                            t += rr[k] * zr - rr[k + 1] * zi;
+                        }
+                        fm[m] = t;
+                    } else {
+                        fm[m] = (rr[0] * pw[m][0] * ns[0] + rr[1] * pw[m][1] * ns[1]) + (rr[2 % VEC] * pw[m][2 % VEC] * ns[2 % VEC] + rr[3 % VEC] * pw[m][3 % VEC] * ns[3 % VEC]);
+                    }
+#pragma unroll
+                    for (int sh = 1; sh < LPB; sh <<= 1) fm[m] += __shfl_xor(fm[m], sh, 64);
+                }
+                if (live[j] && q == 0) {
+#pragma unroll
+                    for (int m = 1; m < WIN; ++m) wa.far[(b * WIN + m) * D + d] = fm[m];
+                }
+                part = fm[0] + wa.g[(int64_t)g * WIN] * x1v;
+            }
         } else {
+            fvec ns;
+            if (CPLX) {
+                // (pr + i pi)(sr + i si) + x1v, then Re(r*s)
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) ns[k] = fmaf(pp[k], st[j][k], x1v);
-            if (VEC == 4) part = (rr[0] * ns[0] + rr[1] * ns[1]) + (rr[2] * ns[2] + rr[3] * ns[3]);
-            else if (VEC == 2) part = rr[0] * ns[0] + rr[1] * ns[1];
-            else part = rr[0] * ns[0];
+                for (int k = 0; k < VEC; k += 2) {
+                    ns[k] = fmaf(pp[k], st[j][k], -pp[k + 1] * st[j][k + 1]) + x1v;
+                    ns[k + 1] = fmaf(pp[k], st[j][k + 1], pp[k + 1] * st[j][k]);
+                }
+                if (VEC == 4) part = (rr[0] * ns[0] - rr[1] * ns[1]) + (rr[2] * ns[2] - rr[3] * ns[3]);
+                else part = rr[0] * ns[0] - rr[1] * ns[1];
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) ns[k] = fmaf(pp[k], st[j][k], x1v);
+                if (VEC == 4) part = (rr[0] * ns[0] + rr[1] * ns[1]) + (rr[2] * ns[2] + rr[3] * ns[3]);
+                else if (VEC == 2) part = rr[0] * ns[0] + rr[1] * ns[1];
+                else part = rr[0] * ns[0];
+            }
+            if (live[j]) *(fvec*)(state + ((b * D + d) * S) * FPS + q * VEC) = ns;
+#pragma unroll
+            for (int m = 1; m < LPB; m <<= 1) part += __shfl_xor(part, m, 64);
         }
-        if (live[j]) *(fvec*)(state + (((b0 + j) * D + d) * S) * FPS + q * VEC) = ns;
-#pragma unroll
-        for (int m = 1; m < LPB; m <<= 1) part += __shfl_xor(part, m, 64);
-        if (live[j] && q == 0) {
+        if (mode != 3 && live[j] && q == 0) {
             float dx = dco * x1v;
             if (d_is_bf16) dx = round_bf(dx);
             const float y = (FEAT != 0 ? gate2 : bf_to_f(x2[b * in_bs + d])) * (part + dx);
             if (out_is_fp32) ((float*)out)[b * out_bs + d] = y;
             else ((bf16_t*)out)[b * out_bs + d] = (bf16_t)f_to_bf_bits(y);
+            // this token's input joins the window's inputs (after every read of the slot it replaces, above)
+            if (WIN > 1) wa.hist[(b * WIN + cnt) * D + d] = (bf16_t)f_to_bf_bits(x1v);
         }
     }
 }
@@ -680,11 +871,23 @@ extern "C" int hyena_ring_advance(int32_t* pos, const int32_t* depth, int64_t n,
     return hyena_check_launch("hyena_ring_advance");
 }
 
+constexpr int IIR_WIN = 4;          // tokens per window of the windowed modal step
+
+struct hyena_iir_window_c {         // hyena_iir_window as the launcher takes it, with the flush flag in its reserved field
+    void* hist; float* far; const float* g; int64_t cnt; const int32_t* cnt_dev; int warm; int flush;
+};
+
+static bool iir_win_geometry(int64_t B, int64_t D, int64_t S) {
+    // built for 16 states (vortex's and the benchmark's size); small problems are launch-bound either way
+    return S == 16 && B >= 1 && D % 8 == 0 && B * D >= 65536;
+}
+
 static int iir_step_launch(const void* x1, const void* x2, const void* v, int64_t in_bs, const hyena_proj_step* proj,
                            float* state, const float* poles, const float* residues, int is_complex,
                            const float* Dcoef, int d_is_bf16, void* out, int out_is_fp32, int64_t out_bs, int64_t B,
-                           int64_t D, int64_t G, int64_t S, void* stream, const char* who) {
-    if ((!proj && (!x1 || !x2 || !v)) || !state || !poles || !residues || !Dcoef || !out)
+                           int64_t D, int64_t G, int64_t S, const hyena_iir_window_c* win, void* stream, const char* who) {
+    const bool flush = win && win->flush;
+    if ((!flush && ((!proj && (!x1 || !x2 || !v)) || !Dcoef || !out)) || !state || !poles || !residues)
         return hyena_fail(HYENA_EINVAL, "%s: all pointers are required", who);
     if (B < 0 || D <= 0 || G <= 0 || D % G != 0)
         return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld G=%lld", who, (long long)B, (long long)D,
@@ -693,6 +896,18 @@ static int iir_step_launch(const void* x1, const void* x2, const void* v, int64_
         return hyena_fail(HYENA_ENOSUP, "%s: state size %lld (powers of two up to 32 supported)", who, (long long)S);
     if (((uintptr_t)state & 15) || ((uintptr_t)poles & 15) || ((uintptr_t)residues & 15))
         return hyena_fail(HYENA_EALIGN, "%s: state, poles, residues must be 16-byte aligned", who);
+    WinArgs wa = {};
+    if (win) {
+        if (!win->hist || (!flush && (!win->far || !win->g)))
+            return hyena_fail(HYENA_EINVAL, "%s: the window needs its hist, far and g buffers", who);
+        if (!iir_win_geometry(B, D, S))
+            return hyena_fail(HYENA_ENOSUP, "%s: the windowed step takes 16 states, D %% 8 == 0 and B*D of 65536 and more; "
+                              "use the plain step", who);
+        if ((!win->cnt_dev && (win->cnt < 0 || win->cnt >= IIR_WIN)) || win->warm < 0)
+            return hyena_fail(HYENA_EINVAL, "%s: window counter %lld / warm %d", who, (long long)win->cnt, win->warm);
+        wa.hist = (bf16_t*)win->hist; wa.far = win->far; wa.g = win->g; wa.cnt = win->cnt_dev ? 0 : (int)win->cnt;
+        wa.cnt_dev = (const int*)win->cnt_dev; wa.warm = win->warm > IIR_WIN ? IIR_WIN : win->warm; wa.flush = flush;
+    }
     ProjArgs pj = {};
     if (proj) {
         if (int rc = make_proj(proj, D, who, &pj)) return rc;
@@ -703,20 +918,31 @@ static int iir_step_launch(const void* x1, const void* x2, const void* v, int64_
     const int dg = (int)(D / G);
     const int lpb = (int)(S * (is_complex ? 2 : 1) >= 4 ? S * (is_complex ? 2 : 1) / 4 : 1);
     if (D * lpb > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: D too large", who);
-    // four batch elements per lane when that still leaves a few wavefronts per SIMD; else one
-    const int nb = (B >= 4 && B * D * lpb >= 4 * 256 * 1024) ? 4 : 1;
-    const int64_t gy = (B + nb - 1) / nb;
+    // four batch elements per lane when that still leaves a few wavefronts per SIMD; else one.  Windowed form: one
+    // (measured: 11.3 / 17.5 us at D = 4096 / 8192 against 15.4 / 19.4 us with four of one residue class b % WIN);
+    // its block rows come in groups of WIN, one per residue class
+    const int nb = (!win && B >= 4 && B * D * lpb >= 4 * 256 * 1024) ? 4 : 1;
+    const int64_t gy = win ? IIR_WIN * (((B + IIR_WIN - 1) / IIR_WIN + nb - 1) / nb) : (B + nb - 1) / nb;
     if (gy > 65535) return hyena_fail(HYENA_EINVAL, "%s: B too large", who);
     dim3 grid((unsigned)((D * lpb + 255) / 256), (unsigned)gy);
     hipStream_t s = (hipStream_t)stream;
     const bf16_t *p1 = (const bf16_t*)x1, *p2 = (const bf16_t*)x2, *pv = (const bf16_t*)v;
     // fused featurizer: vector form where the channel map and alignment allow it, scalar form otherwise
     const int feat = !proj ? 0 : (proj_vector_mode(proj, D) ? proj_vector_mode(proj, D) : 2);
-#define IIR_GO(SS, C, F, N)                                                                                     \
-    hipLaunchKernelGGL((iir_step_kernel<SS, C, F, N>), grid, dim3(256), 0, s, p1, p2, pv, in_bs, pj, state,     \
-                       poles, residues, Dcoef, d_is_bf16, out, out_is_fp32, out_bs, B, D, dg)
+#define IIR_GO(SS, C, F, N, WN)                                                                                 \
+    hipLaunchKernelGGL((iir_step_kernel<SS, C, F, N, WN>), grid, dim3(256), 0, s, p1, p2, pv, in_bs, pj, state, \
+                       poles, residues, Dcoef, d_is_bf16, out, out_is_fp32, out_bs, B, D, dg, wa)
+    if (win) {
+        if (feat == 2)
+            return hyena_fail(HYENA_ENOSUP, "%s: the windowed step needs a featurizer channel map with 16-byte pieces", who);
+#define IIR_WCASE(C, F) if ((is_complex != 0) == C && feat == F) IIR_GO(16, C, F, 1, IIR_WIN);
+        IIR_WCASE(false, 0) IIR_WCASE(false, 1) IIR_WCASE(false, 3)
+        IIR_WCASE(true, 0) IIR_WCASE(true, 1) IIR_WCASE(true, 3)
+#undef IIR_WCASE
+        return hyena_check_launch(who);
+    }
 #define IIR_CASE(SS, C, F)                                                                                      \
-    if (S == SS && (is_complex != 0) == C && feat == F) { if (nb == 4) IIR_GO(SS, C, F, 4); else IIR_GO(SS, C, F, 1); }
+    if (S == SS && (is_complex != 0) == C && feat == F) { if (nb == 4) IIR_GO(SS, C, F, 4, 1); else IIR_GO(SS, C, F, 1, 1); }
 #define IIR_FEATS(SS, C) IIR_CASE(SS, C, 1) IIR_CASE(SS, C, 2) IIR_CASE(SS, C, 3)
     IIR_CASE(1, false, 0) IIR_CASE(2, false, 0) IIR_CASE(4, false, 0)
     IIR_CASE(1, true, 0) IIR_CASE(2, true, 0) IIR_CASE(4, true, 0)
@@ -734,7 +960,7 @@ extern "C" int hyena_iir_step(const void* x1, const void* x2, const void* v, int
                               int d_is_bf16, void* out, int out_is_fp32, int64_t out_bs, int64_t B, int64_t D,
                               int64_t G, int64_t S, void* stream) {
     return iir_step_launch(x1, x2, v, in_bs, nullptr, state, poles, residues, is_complex, Dcoef, d_is_bf16, out,
-                           out_is_fp32, out_bs, B, D, G, S, stream, "hyena_iir_step");
+                           out_is_fp32, out_bs, B, D, G, S, nullptr, stream, "hyena_iir_step");
 }
 
 extern "C" int hyena_iir_layer_step(const hyena_proj_step* proj, float* state, const float* poles,
@@ -743,5 +969,43 @@ extern "C" int hyena_iir_layer_step(const hyena_proj_step* proj, float* state, c
                                     int64_t S, void* stream) {
     if (!proj) return hyena_fail(HYENA_EINVAL, "hyena_iir_layer_step: proj is required");
     return iir_step_launch(nullptr, nullptr, nullptr, 0, proj, state, poles, residues, is_complex, Dcoef, d_is_bf16,
-                           out, out_is_fp32, out_bs, B, D, G, S, stream, "hyena_iir_layer_step");
+                           out, out_is_fp32, out_bs, B, D, G, S, nullptr, stream, "hyena_iir_layer_step");
+}
+
+// ---- the windowed modal step (see iir_step_kernel)
+static_assert(sizeof(hyena_iir_window) == sizeof(hyena_iir_window_c), "hyena_iir_window layout");
+
+extern "C" int64_t hyena_iir_window_tokens(void) { return IIR_WIN; }
+extern "C" int hyena_iir_window_supported(int64_t B, int64_t D, int64_t S, int is_complex) {
+    (void)is_complex;
+    return D > 0 && iir_win_geometry(B, D, S) ? 1 : 0;
+}
+
+extern "C" int hyena_iir_step_win(const void* x1, const void* x2, const void* v, int64_t in_bs, float* state,
+                                  const float* poles, const float* residues, int is_complex, const float* Dcoef,
+                                  int d_is_bf16, void* out, int out_is_fp32, int64_t out_bs, int64_t B, int64_t D,
+                                  int64_t G, int64_t S, const hyena_iir_window* win, void* stream) {
+    if (!win) return hyena_fail(HYENA_EINVAL, "hyena_iir_step_win: win is required");
+    hyena_iir_window_c w = {win->hist, win->far, win->g, win->cnt, win->cnt_dev, win->warm, 0};
+    return iir_step_launch(x1, x2, v, in_bs, nullptr, state, poles, residues, is_complex, Dcoef, d_is_bf16, out,
+                           out_is_fp32, out_bs, B, D, G, S, &w, stream, "hyena_iir_step_win");
+}
+
+extern "C" int hyena_iir_layer_step_win(const hyena_proj_step* proj, float* state, const float* poles,
+                                        const float* residues, int is_complex, const float* Dcoef, int d_is_bf16,
+                                        void* out, int out_is_fp32, int64_t out_bs, int64_t B, int64_t D, int64_t G,
+                                        int64_t S, const hyena_iir_window* win, void* stream) {
+    if (!proj || !win) return hyena_fail(HYENA_EINVAL, "hyena_iir_layer_step_win: proj and win are required");
+    hyena_iir_window_c w = {win->hist, win->far, win->g, win->cnt, win->cnt_dev, win->warm, 0};
+    return iir_step_launch(nullptr, nullptr, nullptr, 0, proj, state, poles, residues, is_complex, Dcoef, d_is_bf16,
+                           out, out_is_fp32, out_bs, B, D, G, S, &w, stream, "hyena_iir_layer_step_win");
+}
+
+extern "C" int hyena_iir_window_flush(float* state, const float* poles, const float* residues, int is_complex,
+                                      int64_t B, int64_t D, int64_t G, int64_t S, const hyena_iir_window* win,
+                                      void* stream) {
+    if (!win) return hyena_fail(HYENA_EINVAL, "hyena_iir_window_flush: win is required");
+    hyena_iir_window_c w = {win->hist, win->far, win->g, win->cnt, win->cnt_dev, win->warm, 1};
+    return iir_step_launch(nullptr, nullptr, nullptr, 0, nullptr, state, poles, residues, is_complex, nullptr, 0, nullptr,
+                           0, 0, B, D, G, S, &w, stream, "hyena_iir_window_flush");
 }

@@ -216,7 +216,7 @@ class StripedHyena2(nn.Module):
         """Greedy cached generation in the order of vortex/model/generation.py:164-229: one prefill over the
         prompt, then one token per forward with the caches' seqlen_offset advanced first.  `forced`
         [B, num_tokens] replaces the sampled tokens (teacher forcing).  graph=True replays the token step as a
-        recorded HIP graph from the third token on (RecordedDecodeStep).  Returns (tokens, logits of every step)."""
+        recorded HIP graph from the fifth token on (RecordedDecodeStep).  Returns (tokens, logits of every step)."""
         B, L = input_ids.shape
         ipd = self.initialize_inference_params(max_seqlen=L + num_tokens)
         x, toks, scores, rec = input_ids, [], [], None
@@ -225,8 +225,8 @@ class StripedHyena2(nn.Module):
                 x = x[:, -1:]
                 for p in ipd.values():
                     p.seqlen_offset = L if p.seqlen_offset == 0 else p.seqlen_offset + 1
-            if graph and i == 2:                    # one eager token step has bound the decode kernels by now
-                rec = RecordedDecodeStep(self, ipd, B)
+            if graph and i == 5:                    # four eager token steps have bound the decode kernels and opened
+                rec = RecordedDecodeStep(self, ipd, B)   # every window of the windowed modal steps by now
             logits = (self.forward(x, ipd) if rec is None else rec(x))[:, -1]
             new = logits.argmax(-1) if forced is None else forced[:, i]
             toks.append(new)
@@ -260,7 +260,12 @@ class RecordedDecodeStep:
             rings.append(ip.fir_state_dict[i])
             if block.filter.fir_inner_filter_length:
                 rings.append(ip.fir_inner_state_dict[i])
-        if any(getattr(r, "valid", r.R) < r.R for r in rings):
+            inner = (block.filter._decode or {}).get("inner")
+            if isinstance(inner, ops.IirStepper) and inner.win is not None:     # a windowed modal step counts tokens too
+                if inner.warm < inner.period:
+                    raise RuntimeError(f"step {inner.period} tokens eagerly before recording (windowed modal state)")
+                rings.append(inner)
+        if any(getattr(r, "valid", r.R) < r.R for r in rings if isinstance(r, ops.FirRing)):
             raise NotImplementedError("a cache is still filling up (prompt shorter than a filter): step eagerly")
         mha = ipd["mha"]
         self.clock = ops.RingClock(rings)

@@ -521,9 +521,14 @@ class FirStepper:
 
 
 class IirStepper:
-    """A decode modal-IIR step with the state and modal parameters bound once."""
+    """A decode modal-IIR step with the state and modal parameters bound once.
 
-    def __init__(self, state, poles, residues, Dcoef):
+    windowed=True (16 states; otherwise ignored): the state tensor is read and written once per window of four tokens
+    instead of every token (hyena_iir_step_win; same outputs up to float32 rounding).  Between windows the state
+    tensor lags the tokens by up to four inputs: call flush() before anything else reads it.  The stepper then also
+    counts tokens (`pos`, `period`, `pos_dev`), so it can go on a RingClock like a cache."""
+
+    def __init__(self, state, poles, residues, Dcoef, windowed=False):
         _need_cuda(state, poles, residues, Dcoef)
         self.cplx = state.is_complex()
         flat = (lambda t: _f32(torch.view_as_real(t.detach().to(torch.complex64).contiguous()))) if self.cplx \
@@ -534,17 +539,72 @@ class IirStepper:
         self.dco, self.d_is_bf16 = _f32(Dcoef), int(Dcoef.dtype == torch.bfloat16)
         self.G, self.S = poles.shape[0], state.shape[-1]
         self.D = state.shape[1]
-        self._fn = _lib.lib().hyena_iir_step
+        L = _lib.lib()
+        self._fn = L.hyena_iir_step
+        self.win = None
+        B = state.shape[0]
+        if windowed and L.hyena_iir_window_supported(B, self.D, self.S, int(self.cplx)):
+            W = L.hyena_iir_window_tokens()
+            dev = state.device
+            pk = poles.detach().to(torch.complex128 if self.cplx else torch.float64)
+            rk = residues.detach().to(pk.dtype)
+            g = torch.stack([(rk * pk ** k).real.sum(-1) if self.cplx else (rk * pk ** k).sum(-1) for k in range(W)], -1)
+            self._g = g.to(torch.float32).contiguous()
+            self._hist = torch.zeros(B, W, self.D, dtype=torch.bfloat16, device=dev)
+            self._far = torch.zeros(B, W, self.D, dtype=torch.float32, device=dev)
+            self.win = _lib.IirWindow(self._hist.data_ptr(), self._far.data_ptr(), self._g.data_ptr(), 0, None, 0, 0)
+            self._wref = ctypes.byref(self.win)
+            self._fn_win, self._fn_flush = L.hyena_iir_step_win, L.hyena_iir_window_flush
+            self.pos, self.period, self.pos_dev, self.warm = 0, W, None, 0
+
+    def _window(self):
+        """The window descriptor for this call; advances the host-side counters."""
+        w = self.win
+        if self.pos_dev is not None:
+            # a recorded step replays this call with `warm` frozen: every window has to be open by then
+            if self.warm < self.period and torch.cuda.is_current_stream_capturing():
+                raise RuntimeError(f"step {self.period} tokens eagerly before recording the windowed modal step")
+            w.cnt, w.cnt_dev = 0, self.pos_dev.data_ptr()
+        else:
+            w.cnt, w.cnt_dev = self.pos, None
+            self.pos = (self.pos + 1) % self.period
+        w.warm = self.warm
+        self.warm = min(self.warm + 1, self.period)
+        return self._wref
 
     def __call__(self, x1, x2, v, out):
         B = x1.shape[0]
-        rc = self._fn(x1.data_ptr(), x2.data_ptr(), v.data_ptr(), x1.stride(0), self.st.data_ptr(), self.p.data_ptr(),
-                      self.r.data_ptr(), int(self.cplx), self.dco.data_ptr(), self.d_is_bf16, out.data_ptr(),
-                      int(out.dtype == torch.float32), out.stride(0), B, self.D, self.G, self.S,
-                      torch.cuda.current_stream().cuda_stream)
+        stream = torch.cuda.current_stream().cuda_stream
+        if self.win is not None:
+            rc = self._fn_win(x1.data_ptr(), x2.data_ptr(), v.data_ptr(), x1.stride(0), self.st.data_ptr(),
+                              self.p.data_ptr(), self.r.data_ptr(), int(self.cplx), self.dco.data_ptr(), self.d_is_bf16,
+                              out.data_ptr(), int(out.dtype == torch.float32), out.stride(0), B, self.D, self.G, self.S,
+                              self._window(), stream)
+        else:
+            rc = self._fn(x1.data_ptr(), x2.data_ptr(), v.data_ptr(), x1.stride(0), self.st.data_ptr(), self.p.data_ptr(),
+                          self.r.data_ptr(), int(self.cplx), self.dco.data_ptr(), self.d_is_bf16, out.data_ptr(),
+                          int(out.dtype == torch.float32), out.stride(0), B, self.D, self.G, self.S, stream)
         if rc:
             _lib.check(rc, "hyena_iir_step")
         return out
+
+    def flush(self):
+        """Folds the inputs of the open windows into the state tensor, which is exact afterwards (no-op for the plain
+        stepper).  The next steps start new windows."""
+        if self.win is None or self.warm == 0:
+            return
+        w = self.win
+        w.cnt, w.cnt_dev = (0, self.pos_dev.data_ptr()) if self.pos_dev is not None else (self.pos, None)
+        w.warm = self.warm
+        rc = self._fn_flush(self.st.data_ptr(), self.p.data_ptr(), self.r.data_ptr(), int(self.cplx), self.state.shape[0],
+                            self.D, self.G, self.S, self._wref, torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "hyena_iir_window_flush")
+        self.warm = 0
+
+    def unwindow(self):
+        """Back to the plain step (after a flush): for callers whose launch has no windowed form."""
+        self.flush()
+        self.win = None
 
 
 def gate_channel_map(hidden, *, interleave=False, head_dim=None):
@@ -585,14 +645,23 @@ class LayerStepper:
         self._fn = _lib.lib().hyena_fir_layer_step if self.is_fir else _lib.lib().hyena_iir_layer_step
         self._fn_dpos = _lib.lib().hyena_fir_layer_step_dpos
         self._fn_far = _lib.lib().hyena_fir_layer_step_far
+        self._fn_win = _lib.lib().hyena_iir_layer_step_win
+        if not self.is_fir and inner.win is not None:
+            # the windowed modal step needs a featurizer map with 16-byte pieces (unit-stride or interleaved)
+            D = inner.D
+            vec = (cs == 1 and ci % 8 == 0 and co % 8 == 0 and gs % 8 == 0) or (cs == 3 and gs == 1 and ci >= D)
+            if not vec or D % 8 or feat_ring.buf.data_ptr() % 16 or self.w.data_ptr() % 16:
+                inner.unwindow()
 
     def __call__(self, u, out):
         """u: [B, 3D] bf16 with contiguous channels; out: [B, D] bf16 (float32 allowed for the IIR step)."""
         B = u.shape[0]
         p, n = self.proj, self.inner
         dpos = self.ring.pos_dev is not None
-        if self.is_fir and (n.ring.pos_dev is not None) != dpos:
-            raise RuntimeError("the featurizer cache and the inner cache must both be on a RingClock, or neither")
+        if (self.is_fir and (n.ring.pos_dev is not None) != dpos) or \
+                (not self.is_fir and n.win is not None and (n.pos_dev is not None) != dpos):
+            raise RuntimeError("the featurizer cache and the inner cache / windowed state must both be on a RingClock, "
+                               "or neither")
         p.u, p.u_batch_stride = u.data_ptr(), u.stride(0)
         p.pos, p.pos_dev = (0, self.ring.pos_dev.data_ptr()) if dpos else (self.ring.pos, None)
         stream = torch.cuda.current_stream().cuda_stream
@@ -611,6 +680,10 @@ class LayerStepper:
             rc = self._fn(self._pref, n.ring.buf.data_ptr(), n.R, n.ring.block, n.ring.pos % n.R, n.w.data_ptr(),
                           n.bias.data_ptr() if n.bias is not None else None, n.mode, out.data_ptr(), out.stride(0),
                           B, n.D, n.G, stream)
+        elif n.win is not None:
+            rc = self._fn_win(self._pref, n.st.data_ptr(), n.p.data_ptr(), n.r.data_ptr(), int(n.cplx), n.dco.data_ptr(),
+                              n.d_is_bf16, out.data_ptr(), int(out.dtype == torch.float32), out.stride(0), B, n.D, n.G,
+                              n.S, n._window(), stream)
         else:
             rc = self._fn(self._pref, n.st.data_ptr(), n.p.data_ptr(), n.r.data_ptr(), int(n.cplx), n.dco.data_ptr(),
                           n.d_is_bf16, out.data_ptr(), int(out.dtype == torch.float32), out.stride(0), B, n.D, n.G,
@@ -635,7 +708,7 @@ class RingClock:
         self.rings = list(rings)
         if not self.rings:
             raise ValueError("no rings")
-        dev = self.rings[0].buf.device
+        dev = self.rings[0].buf.device if hasattr(self.rings[0], "buf") else self.rings[0].state.device
         if any(r.pos_dev is not None for r in self.rings):
             raise RuntimeError("a ring is already on a clock")
         self.pos = torch.tensor([r.pos for r in self.rings], dtype=torch.int32, device=dev)
