@@ -215,8 +215,11 @@ def decode_layer_set(D, device, steps, warmup):
     # the Hyena-MR step as the reference's algorithm has it (the whole cache read every token), on a cache of its own
     from vortex_amd import ops
     mr_plain = ops.FirStepper(va.FirRing(rnd(B, 127, D).to(torch.bfloat16)), w_mr, bias=Dmr, gated_bias=True, far_sums=False)
+    # and the Hyena-LI step that reads and writes the modal state on every token, on a state of its own
+    li_plain = ops.IirStepper(torch.zeros_like(state), poles, res, Dli)
     for nm, st, xx, bb in (("se_step", step.se, x[0], b_se), ("mr_step", step.mr, x[1], b_mr),
-                           ("mr_step_whole_cache", mr_plain, x[1], b_mr), ("iir_step", step.li, x[2], b_li)):
+                           ("mr_step_whole_cache", mr_plain, x[1], b_mr), ("iir_step", step.li, x[2], b_li),
+                           ("iir_step_state_every_token", li_plain, x[2], b_li)):
         o = step.out[0]
         _, kms = time_steps(lambda: st(xx[1], xx[0], xx[2], o), max(steps, 100), warmup)
         per[nm] = dict(us=kms * 1e3, bytes=bb, hbm_gbs=bb / (kms * 1e-3) / 1e9, frac=bb / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
@@ -231,6 +234,15 @@ def decode_layer_set(D, device, steps, warmup):
         per["mr_step"].update(bytes_moved_per_token=moved, moved_gbs=moved / (per["mr_step"]["us"] * 1e-6) / 1e9,
                               window_tokens=n, note="bytes / hbm_gbs / frac are algorithmic (whole cache per token); "
                               "the kernel moves bytes_moved_per_token on average")
+    if step.li.win is not None:
+        # The shipped Hyena-LI step keeps the state in windows of n tokens: per token 1/n of the state traffic, a far
+        # row (float32) written on n - 1 tokens of n by the window's first token and read once each, and the window's
+        # inputs (bf16: one row written per token, (n + n (n - 1) / 2) / n rows read).  `bytes` stays algorithmic.
+        n = step.li.period
+        moved = 2 * state.numel() * 8 / n + B * D * 4 * 2 * (n - 1) / n + B * D * 2 * (1 + (n + n * (n - 1) / 2) / n) + gates_io
+        per["iir_step"].update(bytes_moved_per_token=moved, moved_gbs=moved / (per["iir_step"]["us"] * 1e-6) / 1e9,
+                               window_tokens=n, note="bytes / hbm_gbs / frac are algorithmic (state read and written per "
+                               "token); the kernel moves bytes_moved_per_token on average")
     return dict(us_per_step=ms * 1e3, wall_us_per_step=wall / steps * 1e6, bytes=byts,
                 hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, kernels=per)
 
@@ -251,7 +263,8 @@ def decode_layers_from_projection(D, device, steps, warmup):
     inner = [ops.FirStepper(va.FirRing(rnd(B, 6, D).to(torch.bfloat16)), rnd(G, 7) * 7 ** -0.5),
              ops.FirStepper(va.FirRing(rnd(B, 127, D).to(torch.bfloat16)), rnd(G, 128) * 128 ** -0.5, bias=rnd(D),
                             gated_bias=True),
-             ops.IirStepper(state, torch.exp(lp[..., 0]).to(device), r.to(device), rnd(D).to(torch.bfloat16))]
+             ops.IirStepper(state, torch.exp(lp[..., 0]).to(device), r.to(device), rnd(D).to(torch.bfloat16),
+                            windowed=True)]
     layers = [ops.LayerStepper(va.FirRing(rnd(B, 2, C).to(torch.bfloat16)), rnd(C, 3) * 3 ** -0.5, None, cmap, n)
               for n in inner]
     u = [rnd(B, C).to(torch.bfloat16) for _ in range(3)]

@@ -193,6 +193,8 @@ def test_iir_step_sequence_vs_oracle(cplx, G, S):
     (True, 50, 2048, 2048, True, False),     # layer step from the projection (interleaved gates)
     (False, 37, 2056, 257, True, True),      # counter in device memory; D not a multiple of 256
     (True, 70, 1000, 125, False, False),     # D a multiple of 8 only
+    (True, 68, 4104, 513, False, False),     # large enough for two batch elements per block at a window's head (17 of them)
+    (False, 130, 4096, 4096, True, True),    # the same from the projection, counters in device memory
 ])
 def test_iir_step_windowed_state(cplx, B, D, G, fused, on_clock):
     """The stepper that reads and writes the modal state once per window of four tokens (windows staggered over the

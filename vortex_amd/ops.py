@@ -726,12 +726,15 @@ class RingClock:
 
 
 class DecodeLayerSet:
-    """Cached decode step of one [Hyena-SE, Hyena-MR, Hyena-LI] layer set: three fused launches."""
+    """Cached decode step of one [Hyena-SE, Hyena-MR, Hyena-LI] layer set: three fused launches.
 
-    def __init__(self, ring_se, w_se, ring_mr, w_mr, D_mr, state_li, poles, residues, D_li):
+    window_state: the Hyena-LI step keeps its modal state in windows of several tokens where the library has that form
+    (IirStepper windowed=True): state_li then lags the tokens until flush()."""
+
+    def __init__(self, ring_se, w_se, ring_mr, w_mr, D_mr, state_li, poles, residues, D_li, window_state=True):
         self.se = FirStepper(ring_se, w_se)
         self.mr = FirStepper(ring_mr, w_mr, bias=D_mr, gated_bias=True)
-        self.li = IirStepper(state_li, poles, residues, D_li)
+        self.li = IirStepper(state_li, poles, residues, D_li, windowed=window_state)
         B, D = state_li.shape[0], state_li.shape[1]
         self.out = [torch.empty(B, D, dtype=torch.bfloat16, device=state_li.device) for _ in range(3)]
 
@@ -741,3 +744,7 @@ class DecodeLayerSet:
         self.mr(g_mr[1], g_mr[0], g_mr[2], self.out[1])
         self.li(g_li[1], g_li[0], g_li[2], self.out[2])
         return self.out
+
+    def flush(self):
+        """Brings state_li up to the last token (no-op without windows)."""
+        self.li.flush()
