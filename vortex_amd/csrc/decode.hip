@@ -382,6 +382,23 @@ struct WinArgs {
     uint32_t nhb, nxh, nxl;
 };
 
+// Sum over the N lanes (a power of two up to 16, aligned) that share a channel, in the order of an xor butterfly: data-
+// parallel-primitive operands of the additions themselves (quad swaps, then the mirrored half row / row, whose lanes
+// hold the other half's partial sum by then).
+template <int CTRL>
+__device__ __forceinline__ float dpp_take(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+template <int N>
+__device__ __forceinline__ float lane_group_sum(float x) {
+    static_assert(N >= 1 && N <= 16 && (N & (N - 1)) == 0, "lane groups of 1, 2, 4, 8 or 16");
+    if (N >= 2) x += dpp_take<0xB1>(x);        // quad_perm [1, 0, 3, 2]
+    if (N >= 4) x += dpp_take<0x4E>(x);        // quad_perm [2, 3, 0, 1]
+    if (N >= 8) x += dpp_take<0x141>(x);       // row_half_mirror
+    if (N >= 16) x += dpp_take<0x140>(x);      // row_mirror
+    return x;
+}
+
 template <int S, bool CPLX, int FEAT, int NB, int WIN>
 __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict__ x1, const bf16_t* __restrict__ x2,
                                                        const bf16_t* __restrict__ v, int64_t in_bs, ProjArgs pj,
@@ -467,26 +484,26 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
             a = pj.flip ? g2 : g1;
             gate2 = pj.flip ? g1 : g2;
         } else {
-            a = bf_to_f(x1[b * in_bs + dc]);
-            c = bf_to_f(v[b * in_bs + dc]);
-            gate2 = bf_to_f(x2[b * in_bs + dc]);
+            a = bf_to_f((x1 + b * in_bs)[dc]);
+            c = bf_to_f((v + b * in_bs)[dc]);
+            gate2 = bf_to_f((x2 + b * in_bs)[dc]);
         }
         if (!ok) return;
         const float x1v = round_bf(a * c);
-        const float* gp = wa.g + (int64_t)(dc / (uint32_t)dg) * WIN;
-        float part = wa.far[(b * WIN + jw) * D + dc] + gp[0] * x1v;
+        const float* gp = wa.g + (dc / (uint32_t)dg) * (uint32_t)WIN;
+        float part = (wa.far + (b * WIN + jw) * D)[dc] + gp[0] * x1v;
 #pragma unroll
         for (int k = 1; k < WIN; ++k) {
             int sl = cnt - k;
             if (sl < 0) sl += WIN;
-            if (k <= jw) part = fmaf(gp[k], bf_to_f(wa.hist[(b * WIN + sl) * D + dc]), part);
+            if (k <= jw) part = fmaf(gp[k], bf_to_f((wa.hist + (b * WIN + sl) * D)[dc]), part);
         }
         float dx = Dcoef[dc] * x1v;
         if (d_is_bf16) dx = round_bf(dx);
         const float y = gate2 * (part + dx);
-        if (out_is_fp32) ((float*)out)[b * out_bs + dc] = y;
-        else ((bf16_t*)out)[b * out_bs + dc] = (bf16_t)f_to_bf_bits(y);
-        wa.hist[(b * WIN + cnt) * D + dc] = (bf16_t)f_to_bf_bits(x1v);
+        if (out_is_fp32) ((float*)out + b * out_bs)[dc] = y;
+        else ((bf16_t*)out + b * out_bs)[dc] = (bf16_t)f_to_bf_bits(y);
+        (wa.hist + (b * WIN + cnt) * D)[dc] = (bf16_t)f_to_bf_bits(x1v);
         return;
     }
     const uint32_t idx = xb * 256 + threadIdx.x;                // (channel, lane of the group)
@@ -495,13 +512,17 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
     const bool chan_live = d < (uint32_t)D;
     if (!chan_live) d = 0;
     const uint32_t g = d / (uint32_t)dg;
+    // Addresses are a block-uniform row base (batch element; 0 for the rows past the batch, whose lanes store nothing)
+    // plus a 32-bit lane offset, so the 64-bit part of the arithmetic is scalar.
+    auto bu = [&](int j) -> int64_t { return bj(j) < B ? bj(j) : 0; };
+    const int64_t row_floats = D * (int64_t)(S * FPS);
+    const uint32_t soff = (d * LPB + q) * VEC;             // this lane's piece of its channel's state inside a row
     fvec st[NB];
     bool live[NB];
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         live[j] = chan_live && bj(j) < B;
-        const int64_t bd = live[j] ? bj(j) * D + d : 0;
-        st[j] = *(const fvec*)(state + (bd * S) * FPS + q * VEC);
+        st[j] = *(const fvec*)(state + bu(j) * row_floats + soff);
     }
     // the inputs a window's first token (or a flush) folds into the state, newest first: u_{t-1-k}
     float pend[NB][WIN > 1 ? WIN : 1];
@@ -512,12 +533,11 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
             for (int k = 0; k < WIN; ++k) {
                 int sl = cnt - 1 - k;
                 if (sl < 0) sl += WIN;
-                const int64_t bb = live[j] ? bj(j) : 0;
-                pend[j][k] = k < npend ? bf_to_f(wa.hist[(bb * WIN + sl) * D + d]) : 0.f;
+                pend[j][k] = k < npend ? bf_to_f((wa.hist + (bu(j) * WIN + sl) * D)[d]) : 0.f;
             }
     }
-    const fvec pp = *(const fvec*)(poles + ((int64_t)g * S) * FPS + q * VEC);
-    const fvec rr = *(const fvec*)(residues + ((int64_t)g * S) * FPS + q * VEC);
+    const fvec pp = *(const fvec*)(poles + (g * (uint32_t)(S * FPS) + q * VEC));
+    const fvec rr = *(const fvec*)(residues + (g * (uint32_t)(S * FPS) + q * VEC));
     const float dco = mode != 3 ? Dcoef[d] : 0.f;      // a flush has no token: no gates, no output, no Dcoef
     // fused featurizer: lanes 0..2 of the group evaluate gates x2, x1, v of every batch element first (their
     // loads overlap), the ring-slot stores follow, and only then the state updates start
@@ -551,7 +571,7 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
                 zf[j] = 0.f;
                 un[j] = 0;
                 if (q < 3) {
-                    const int64_t b = live[j] ? bj(j) : 0;
+                    const int64_t b = bu(j);
                     const uint32_t ch = pj.chan((uint32_t)q, d);
                     const bf16_t* rb = pj.ring + (b * pj.Rf) * pj.C + ch;
                     un[j] = pj.u[b * pj.u_bs + ch];
@@ -593,7 +613,7 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
     }
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
-        const int64_t b = live[j] ? bj(j) : 0;
+        const int64_t b = bu(j);
         float a = 0.f, c = 0.f, gate2 = 0.f;
         if (mode == 3) {
         } else if (VFEAT) {
@@ -610,8 +630,8 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
             a = pj.flip ? g2 : g1;
             gate2 = pj.flip ? g1 : g2;
         } else {
-            a = bf_to_f(x1[b * in_bs + d]);
-            c = bf_to_f(v[b * in_bs + d]);
+            a = bf_to_f((x1 + b * in_bs)[d]);
+            c = bf_to_f((v + b * in_bs)[d]);
         }
         const float x1v = round_bf(a * c);
         float part = 0.f;
@@ -641,7 +661,7 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
                 for (int m = 1; m < WIN; ++m)
 #pragma unroll
                     for (int k = 0; k < VEC; ++k) ns[k] = fmaf(pw[m - 1][k], pend[j][m], ns[k]);
-                if (live[j]) *(fvec*)(state + ((b * D + d) * S) * FPS + q * VEC) = ns;
+                if (live[j]) *(fvec*)(state + b * row_floats + soff) = ns;
             }
             if (mode == 1) {
                 // far[m] = Re sum_s r p^(m+1) S: this lane's states, then the lane group
@@ -660,14 +680,13 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
                     } else {
                         fm[m] = (rr[0] * pw[m][0] * ns[0] + rr[1] * pw[m][1] * ns[1]) + (rr[2 % VEC] * pw[m][2 % VEC] * ns[2 % VEC] + rr[3 % VEC] * pw[m][3 % VEC] * ns[3 % VEC]);
                     }
-#pragma unroll
-                    for (int sh = 1; sh < LPB; sh <<= 1) fm[m] += __shfl_xor(fm[m], sh, 64);
+                    fm[m] = lane_group_sum<LPB>(fm[m]);
                 }
                 if (live[j] && q == 0) {
 #pragma unroll
-                    for (int m = 1; m < WIN; ++m) wa.far[(b * WIN + m) * D + d] = fm[m];
+                    for (int m = 1; m < WIN; ++m) (wa.far + (b * WIN + m) * D)[d] = fm[m];
                 }
-                part = fm[0] + wa.g[(int64_t)g * WIN] * x1v;
+                part = fm[0] + wa.g[g * (uint32_t)WIN] * x1v;
             }
         } else {
             fvec ns;
@@ -687,18 +706,17 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
                 else if (VEC == 2) part = rr[0] * ns[0] + rr[1] * ns[1];
                 else part = rr[0] * ns[0];
             }
-            if (live[j]) *(fvec*)(state + ((b * D + d) * S) * FPS + q * VEC) = ns;
-#pragma unroll
-            for (int m = 1; m < LPB; m <<= 1) part += __shfl_xor(part, m, 64);
+            if (live[j]) *(fvec*)(state + b * row_floats + soff) = ns;
+            part = lane_group_sum<LPB>(part);
         }
         if (mode != 3 && live[j] && q == 0) {
             float dx = dco * x1v;
             if (d_is_bf16) dx = round_bf(dx);
-            const float y = (FEAT != 0 ? gate2 : bf_to_f(x2[b * in_bs + d])) * (part + dx);
-            if (out_is_fp32) ((float*)out)[b * out_bs + d] = y;
-            else ((bf16_t*)out)[b * out_bs + d] = (bf16_t)f_to_bf_bits(y);
+            const float y = (FEAT != 0 ? gate2 : bf_to_f((x2 + b * in_bs)[d])) * (part + dx);
+            if (out_is_fp32) ((float*)out + b * out_bs)[d] = y;
+            else ((bf16_t*)out + b * out_bs)[d] = (bf16_t)f_to_bf_bits(y);
             // this token's input joins the window's inputs (after every read of the slot it replaces, above)
-            if (WIN > 1) wa.hist[(b * WIN + cnt) * D + d] = (bf16_t)f_to_bf_bits(x1v);
+            if (WIN > 1) (wa.hist + (b * WIN + cnt) * D)[d] = (bf16_t)f_to_bf_bits(x1v);
         }
     }
 }
@@ -939,7 +957,7 @@ static int iir_step_launch(const void* x1, const void* x2, const void* v, int64_
     if (B == 0) return 0;
     const int dg = (int)(D / G);
     const int lpb = (int)(S * (is_complex ? 2 : 1) >= 4 ? S * (is_complex ? 2 : 1) / 4 : 1);
-    if (D * lpb > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: D too large", who);
+    if (D * lpb > 0x0fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: D too large", who);   // 32-bit byte offsets inside a row
     // four batch elements per lane when that still leaves a few wavefronts per SIMD; else one.  Windowed form: one
     // (measured: 11.3 / 17.5 us at D = 4096 / 8192 against 15.4 / 19.4 us with four of one residue class b % WIN);
     // its block rows come in groups of WIN, one per residue class
