@@ -288,6 +288,51 @@ def test_operator_module_prefill_then_decode(kind, cs, il, fused):
         assert (mod._decode["layer"] is not None) == (not (cs and il))
 
 
+@pytest.mark.parametrize("kind,cs,il,fused", [("li_cplx", False, True, True), ("li_real", True, False, True),
+                                              ("li_cplx", True, True, True), ("li_real", False, False, False)])
+def test_operator_module_windowed_modal_state(kind, cs, il, fused):
+    # at batch x width of 65536 and more the module's decode step keeps the modal state in windows of four tokens:
+    # outputs against the oracle call sequence on every token, the cached state lagging in between and equal to
+    # the oracle's after flush_decode_state(), and further tokens after the flush
+    from vortex_amd import ops
+    B, L, D, H, G = 64, 8, 1024, 8, 64
+    p = make_params(kind, D, G, seed=13)
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=cs, interleave=il, short_filter_length=3,
+               short_filter_bias=False, state_size=16)
+    mod = HyenaCascade(cfg, 0, hyena_filter_groups=G, complex_modal=(kind == "li_cplx"))
+    with torch.no_grad():
+        mod.short_filter_weight.copy_(p["short_filter_weight"])
+        mod.log_poles.copy_(p["log_poles"])
+        mod.residues.copy_(p["residues"])
+        mod.D.data = p["D"].clone()
+    mod = mod.to(DEV)
+    mod.fuse_decode = mod.fuse_prefill = fused
+    pr = dict(p, log_poles=p["log_poles"].repeat_interleave(D // G, 0), residues=p["residues"].repeat_interleave(D // G, 0))
+    ref = O.OracleCascade(O.OracleEngine(), pr, D, H, D, column_split_hyena=cs, interleave=il)
+    n_dec = 11
+    u_all = torch.randn(B, L + n_dec, 3 * D, generator=torch.Generator().manual_seed(4)).bfloat16()
+    ip_ref, ip_hip = O.OracleCache(), HyenaCascadeIIRInferenceParams()
+    y_ref, _ = ref.forward(u_all[:, :L], ip_ref)
+    y_hip, _ = mod(u_all[:, :L].to(DEV), ip_hip)
+    assert rel_err(y_hip, y_ref) <= 2e-2
+    as_real = lambda t: torch.view_as_real(t) if t.is_complex() else t
+    for i in range(n_dec):
+        tok = u_all[:, L + i: L + i + 1]
+        y_ref, _ = ref.forward(tok, ip_ref)
+        y_hip, _ = mod(tok.to(DEV), ip_hip)
+        assert rel_err(y_hip, y_ref) <= 2e-2, i
+        if i == 6:
+            inner = mod._decode["inner"]
+            assert isinstance(inner, ops.IirStepper) and inner.win is not None
+            assert rel_err(as_real(ip_hip.state_dict[0]), as_real(ip_ref.state_dict[0])) > 1e-2     # lags the tokens
+            mod.flush_decode_state()
+            assert rel_err(as_real(ip_hip.state_dict[0]), as_real(ip_ref.state_dict[0])) <= 1e-3
+    mod.flush_decode_state()
+    assert rel_err(as_real(ip_hip.state_dict[0]), as_real(ip_ref.state_dict[0])) <= 1e-3
+    mod.flush_decode_state()                               # nothing pending: no launch, same state
+    assert rel_err(as_real(ip_hip.state_dict[0]), as_real(ip_ref.state_dict[0])) <= 1e-3
+
+
 @pytest.mark.parametrize("kind", ["se", "mr", "li_real"])
 def test_operator_module_groups_of_15_channels(kind):
     # Evo 2 1B geometry in small: hidden = 16 groups x 15 channels (1920 = 128 x 15 there), 15 heads, interleaved gates

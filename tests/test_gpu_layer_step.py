@@ -115,6 +115,42 @@ def test_iir_layer_step_sequence_vs_oracle(B, D, H, G, S, cplx, cs, il, flip, d_
         assert rel_err(sh, sr) <= 1e-2, i
 
 
+def test_windowed_modal_stepper_goes_back_to_the_plain_step_for_scalar_maps():
+    # a head-blocked split with heads of 12 channels has no 16-byte pieces, so the fused layer step has no windowed
+    # form: LayerStepper flushes the open windows (the state is exact again) and steps the state on every token
+    B, D, H, S = 64, 1032, 86, 16
+    g = torch.Generator().manual_seed(5)
+    C, Ks = 3 * D, 3
+    wf = torch.randn(C, 1, Ks, generator=g) / Ks ** 0.5
+    lp, r = O.make_modal_real(D, S, seed=3)
+    Dc = torch.randn(D, generator=g).bfloat16()
+    fst = torch.randn(B, C, Ks - 1, generator=g).bfloat16()
+    ref_s = torch.randn(B, D, S, generator=g)
+    state = ref_s.clone().to(DEV)
+    inner = ops.IirStepper(state, torch.exp(lp)[..., 0].contiguous().to(DEV), r.to(DEV), Dc.to(DEV), windowed=True)
+    assert inner.win is not None
+    y = torch.empty(B, D, dtype=torch.bfloat16, device=DEV)
+    for i in range(2):                                      # two tokens inside open windows
+        x1, x2, v = (torch.randn(B, D, generator=g).bfloat16() for _ in range(3))
+        y_ref, ref_s = O.step_iir(x2, x1, v, Dc, r, lp, ref_s)
+        inner(x1.to(DEV), x2.to(DEV), v.to(DEV), y)
+        assert rel_err(y, y_ref) <= 2e-2, i
+    assert rel_err(state, ref_s) > 1e-3                     # lagging
+    fring = va.FirRing.from_reference(fst.to(DEV))
+    cmap = ops.gate_channel_map(D, head_dim=D // H)
+    step = ops.LayerStepper(fring, wf.reshape(C, Ks).to(DEV), None, cmap, inner)
+    assert inner.win is None and rel_err(state, ref_s) <= 1e-4
+    ref_f = fst
+    for i in range(3):
+        u = torch.randn(B, C, generator=g).bfloat16()
+        z, ref_f = O.step_fir(u, ref_f, wf)
+        x2, x1, v = oracle_gates(z, D, H, True, False, False)
+        y_ref, ref_s = O.step_iir(x2, x1, v, Dc, r, lp, ref_s)
+        step(u.to(DEV), y)
+        assert rel_err(y, y_ref) <= 2e-2, i
+        assert rel_err(state, ref_s) <= 1e-3, i
+
+
 def test_layer_step_rejects_bad_maps():
     D = 64
     fring = va.FirRing(torch.zeros(1, 2, 3 * D, dtype=torch.bfloat16, device=DEV))
