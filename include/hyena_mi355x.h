@@ -282,8 +282,9 @@ int hyena_fir_layer_step_far(const hyena_proj_step* proj,
  * counts tokens in cnt = token % W (or cnt_dev: the counter in device memory, advanced with hyena_ring_advance,
  * depth W) and passes warm = the number of tokens stepped with these calls since `state` was last exact (0 on the
  * first call; anything >= W means "W or more").  Between two windows the `state` tensor lags the tokens by up to W
- * inputs; hyena_iir_window_flush folds them in (then restart with warm = 0), e.g. before anything else reads the
- * state.  Available for 16 states, 16-byte aligned gates with D % 8 == 0, and (in the layer step) the featurizer
+ * inputs; hyena_iir_window_flush (called with cnt = the counter of the NEXT token, i.e. advanced past the last step, and
+ * the current warm) folds them in; afterwards go on counting cnt as before and restart warm at 0.  Flush before
+ * anything else reads the state.  Available for 16 states, 16-byte aligned gates with D % 8 == 0, and (in the layer step) the featurizer
  * maps that have a vector form (hyena_iir_window_supported); other cases return HYENA_ENOSUP: use hyena_iir_step. */
 typedef struct hyena_iir_window {
     void* hist;

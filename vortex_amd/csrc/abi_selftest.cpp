@@ -4,6 +4,7 @@
 //   hyena_fir_step                    dot product over a ring cache, slot rotation
 //   hyena_fir_step_far                the same step on a deep cache read whole only every third token, 3 ring periods
 //   hyena_iir_step                    one modal update against the closed form
+//   hyena_iir_step_win                the modal step with the state in windows of tokens against hyena_iir_step (float32 rounding)
 //   argument errors                   negative return codes and a message
 // Usage: abi_selftest /path/to/libhyena_mi355x.so
 #include <dlfcn.h>
@@ -44,6 +45,7 @@ int main(int argc, char** argv) {
     SYM(hyena_version) SYM(hyena_last_error_string) SYM(hyena_mr_fwd) SYM(hyena_fir_cl_fwd) SYM(hyena_fir_step)
     SYM(hyena_iir_step) SYM(hyena_se_fwd) SYM(hyena_fir_step_dpos) SYM(hyena_ring_advance)
     SYM(hyena_fir_step_far) SYM(hyena_fir_far_period) SYM(hyena_fir_far_bytes)
+    SYM(hyena_iir_step_win) SYM(hyena_iir_window_flush) SYM(hyena_iir_window_tokens) SYM(hyena_iir_window_supported)
     printf("%s\n", p_hyena_version());
     hipStream_t stream; HIP_OK(hipStreamCreate(&stream));
 
@@ -222,6 +224,68 @@ int main(int argc, char** argv) {
                   y[b * Ds + d], want);
         }
         printf("hyena_iir_step closed form: ok\n");
+    }
+
+    // ---- windowed modal step from C: the caller owns hist / far / g, counts tokens and warm; against hyena_iir_step on a
+    //      copy of the state, outputs on every token and the state after a flush
+    {
+        const int64_t Bs = 16, Ds = 4096, S = 16, W = p_hyena_iir_window_tokens();
+        CHECK(p_hyena_iir_window_supported(Bs, Ds, S, 0) == 1, "windowed step not offered for B=16 D=4096");
+        std::vector<float> st(Bs * Ds * S), poles(Ds * S), res(Ds * S), Dc(Ds), g(Ds * W);
+        uint32_t rng = 12345u;
+        auto rnd = [&]() { rng = rng * 1664525u + 1013904223u; return (float)((rng >> 8) & 0xffff) / 65536.f - 0.5f; };
+        for (auto& x : st) x = rnd();
+        for (auto& x : poles) x = 0.5f + 0.9f * rnd();           // 0.05 .. 0.95
+        for (auto& x : res) x = rnd();
+        for (auto& x : Dc) x = rnd();
+        for (int64_t d = 0; d < Ds; ++d) for (int64_t k = 0; k < W; ++k) {
+            double acc = 0.0;
+            for (int64_t s = 0; s < S; ++s) acc += (double)res[d * S + s] * pow((double)poles[d * S + s], (double)k);
+            g[d * W + k] = (float)acc;
+        }
+        float *d_sa = dev(st), *d_sb = dev(st), *d_p = dev(poles), *d_r = dev(res), *d_D = dev(Dc), *d_g = dev(g), *d_ya, *d_yb, *d_far;
+        uint16_t* d_hist;
+        HIP_OK(hipMalloc(&d_ya, Bs * Ds * 4)); HIP_OK(hipMalloc(&d_yb, Bs * Ds * 4));
+        HIP_OK(hipMalloc(&d_far, Bs * W * Ds * 4)); HIP_OK(hipMalloc(&d_hist, Bs * W * Ds * 2));
+        HIP_OK(hipMemset(d_far, 0, Bs * W * Ds * 4)); HIP_OK(hipMemset(d_hist, 0, Bs * W * Ds * 2));
+        std::vector<uint16_t> x1(Bs * Ds), x2(Bs * Ds), v(Bs * Ds);
+        uint16_t *d1 = dev(x1), *d2 = dev(x2), *dv = dev(v);
+        hyena_iir_window win = {};
+        win.hist = d_hist; win.far = d_far; win.g = d_g;
+        int warm = 0;
+        auto flush_and_compare = [&](int step) {          // step = tokens done so far - 1; the flush takes the next token's counter
+            win.cnt = (step + 1) % W; win.warm = warm;
+            int rc = p_hyena_iir_window_flush(d_sa, d_p, d_r, 0, Bs, Ds, Ds, S, &win, stream);
+            CHECK(rc == 0, "hyena_iir_window_flush rc=%d: %s", rc, p_hyena_last_error_string());
+            warm = 0;
+            HIP_OK(hipStreamSynchronize(stream));
+            auto sa = host(d_sa, st.size()); auto sb = host(d_sb, st.size());
+            for (size_t i = 0; i < sa.size(); ++i)
+                CHECK(fabsf(sa[i] - sb[i]) <= 3e-5f * (1.f + fabsf(sb[i])), "windowed state after flush, step %d i=%zu got %g want %g",
+                      step, i, sa[i], sb[i]);
+        };
+        for (int step = 0; step < 11; ++step) {
+            for (auto& x : x1) x = to_bf16(rnd());
+            for (auto& x : x2) x = to_bf16(1.f + rnd());
+            for (auto& x : v) x = to_bf16(2.f * rnd());
+            HIP_OK(hipMemcpy(d1, x1.data(), x1.size() * 2, hipMemcpyHostToDevice));
+            HIP_OK(hipMemcpy(d2, x2.data(), x2.size() * 2, hipMemcpyHostToDevice));
+            HIP_OK(hipMemcpy(dv, v.data(), v.size() * 2, hipMemcpyHostToDevice));
+            win.cnt = step % W; win.warm = warm;
+            int rc = p_hyena_iir_step_win(d1, d2, dv, Ds, d_sa, d_p, d_r, 0, d_D, 0, d_ya, 1, Ds, Bs, Ds, Ds, S, &win, stream);
+            CHECK(rc == 0, "hyena_iir_step_win rc=%d: %s", rc, p_hyena_last_error_string());
+            warm = warm < W ? warm + 1 : (int)W;
+            rc = p_hyena_iir_step(d1, d2, dv, Ds, d_sb, d_p, d_r, 0, d_D, 0, d_yb, 1, Ds, Bs, Ds, Ds, S, stream);
+            CHECK(rc == 0, "hyena_iir_step rc=%d: %s", rc, p_hyena_last_error_string());
+            HIP_OK(hipStreamSynchronize(stream));
+            auto ya = host(d_ya, (size_t)(Bs * Ds)); auto yb = host(d_yb, (size_t)(Bs * Ds));
+            for (size_t i = 0; i < ya.size(); ++i)
+                CHECK(fabsf(ya[i] - yb[i]) <= 1e-4f * (1.f + fabsf(yb[i])), "hyena_iir_step_win step %d i=%zu got %g want %g", step,
+                      i, ya[i], yb[i]);
+            if (step == 5) flush_and_compare(step);          // in the middle of the windows; they restart
+        }
+        flush_and_compare(10);
+        printf("hyena_iir_step_win / hyena_iir_window_flush (windows of %lld tokens) against hyena_iir_step: ok\n", (long long)W);
     }
 
     // ---- rejected arguments come back as negative codes with a message, before anything is launched
