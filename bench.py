@@ -36,7 +36,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="mr", choices=["mr", "se", "se_b8", "li", "li_g4096", "decode", "mr_cl", "mr_layer",
+    ap.add_argument("--workload", default="mr", choices=["mr", "se", "se_b8", "li", "li_g4096", "decode", "mr_cl", "mr_layer", "li_layer",
                                                          "se_layer"])
     ap.add_argument("--settle-ms", type=float, default=150.0,
                     help="untimed run of each workload before its warm-up steps, until clocks have settled")
@@ -177,6 +177,27 @@ def build_workload(name, device):
             what, keep = ("hyena_mr" if mr else "hyena_se") + "_layer featurizer+operator from the projection", (u, wf, h, Db, out)
         return fn, dict(workload=f"{what} B={B} L={L} D={D} groups={G} K={K}", tokens=B * L, bytes=8 * B * D * L,
                         kernel="fir_cl_kernel", keep=keep)
+    if name == "li_layer":
+        # a whole Hyena-LI layer from the projection at the config-3 shape: featurizer + split + x1*v in one launch
+        # (rows xv, x2), then the modal scan on them; 8 bytes per output element would be a one-pass layer, the two
+        # launches move 16 (10 + 6)
+        B, D, L, G, S = 1, 4096, 262144, 256, 16
+        g = torch.Generator(device=device).manual_seed(10)
+        u = torch.randn(B, L, 3 * D, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+        wf = torch.randn(3, 3 * D, generator=g, device=device, dtype=torch.float32) * 3 ** -0.5
+        cmap = ops.gate_channel_map(D, interleave=True)
+        lp, r = O.make_modal_complex(G, S)
+        Db = torch.randn(D, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).to(device)
+        plan = va.ModalPlan(lp.to(device), r.to(device))
+        out = torch.empty(B, D, L, dtype=torch.bfloat16, device=device)
+
+        def fn():
+            xv, x2 = ops.featurizer_gates_fwd(u, wf, None, cmap)
+            ops.li_fwd_rows(ops.rows_of(xv), ops.rows_of(x2), None, plan, Db, B, D, L, device=device, out=out)
+
+        return fn, dict(workload=f"hyena_li_layer featurizer+gates then modal scan, from the projection B={B} L={L} D={D} "
+                                 f"groups={G} poles={S} complex", tokens=B * L, bytes=8 * B * D * L,
+                        kernel="proj_gates_kernel + li_kernel", keep=(u, wf, plan, Db, out))
     raise ValueError(name)
 
 
@@ -516,8 +537,8 @@ def main():
                 continue
             steps = max(3, min(args.steps, 20 if name.startswith("li") else args.steps))
             extra[name] = entry(run(name, steps, extra_warmup))
-        for name in ("mr_cl", "mr_layer", "se_layer"):
-            extra[name] = entry(run(name, max(3, min(args.steps, 20)), extra_warmup))
+        for name in ("mr_cl", "mr_layer", "se_layer", "li_layer"):
+            extra[name] = entry(run(name, max(3, min(args.steps, 10 if name == "li_layer" else 20)), extra_warmup))
         for D in (4096, 8192):
             extra[f"decode_D{D}"] = decode_layer_set(D, device, max(args.steps, 50), max(args.warmup, 5))
         extra["decode_from_projection_D4096"] = decode_layers_from_projection(4096, device, max(args.steps, 50),

@@ -58,6 +58,7 @@ const char* hyena_last_error_string(void);
  * segment counts, cached / non-temporal accesses and work decompositions from the problem size; this pins one of
  * those choices process-wide until it is reset with a negative value.  Nothing is read from the environment.
  *   "mr_nseg", "cl_nseg", "li_nseg"            segments along L of hyena_mr_fwd, hyena_fir_cl_fwd / layer_fwd, hyena_li_fwd
+ *                                               (cl_nseg also: blocks along L per channel strip in hyena_featurizer_gates_fwd)
  *   "se_nt", "mr_nt", "li_nt", "cl_nt"         0 = cached, 1 = non-temporal global accesses
  *   "li_cpw"                                    1 / 4 = channels per wavefront in hyena_li_fwd (4 needs D/G % 4 == 0)
  *   "li_coop"                                   0 / 1 = lone / cooperating wavefronts in hyena_li_fwd
@@ -133,7 +134,9 @@ int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v
  * state_out (optional, [B][D][S][2] float32) the modal state after the last sample.
  * d_is_bf16 selects the rounding of z = y + Dcoef*x1v: 1 = bf16(bf16(y) + bf16(Dcoef*x1v)), what
  * bf16 tensors give in vortex/model/engine.py:352-353; 0 = bf16(bf16(y) + Dcoef*x1v), a float32
- * Dcoef; 2 = bf16(y + Dcoef*x1v), a single rounding (cheaper, within one bf16 ulp of mode 1). */
+ * Dcoef; 2 = bf16(y + Dcoef*x1v), a single rounding (cheaper, within one bf16 ulp of mode 1).
+ * v == NULL with x2 given: x1 already holds x1v = bf16(x1*v) (what hyena_featurizer_gates_fwd writes), 6 instead of 8
+ * bytes per sample; v == x2 == NULL: the ungated convolution of x1. */
 int64_t hyena_li_plan_bytes(int64_t G, int64_t S);
 int hyena_li_plan(const float* log_poles, const float* residues, int64_t G, int64_t S,
                   void* workspace, void* stream);
@@ -347,6 +350,16 @@ typedef struct hyena_proj_fwd {
     int flip_x1x2;
     int64_t ch_inner, ch_outer, gate_stride, ch_stride;
 } hyena_proj_fwd;
+
+/* Featurizer and gates of a Hyena-LI layer at prefill in one launch: the featurizer FIR over the projection
+ * u [B][L][3D] (vortex/model/engine.py:188-223), interleave / split (vortex/model/model.py:251-252,
+ * engine.py:300-310) and x1v = x1*v (engine.py:312), written as the two row tensors hyena_li_fwd reads:
+ *   xv_out [B][D][L + front_pad] = bf16(x1*v),  x2_out [B][D][L + front_pad] = x2   (bf16; the first front_pad
+ * columns are zero: front_pad = -L % 8 makes any L usable).  The three gate tensors [B][3D][L] of
+ * hyena_featurizer_fwd are never written: 10 instead of 12 bytes per (channel, sample) here and 6 instead of 8 in
+ * hyena_li_fwd (v = NULL).  Channel maps and Ks as hyena_fir_layer_fwd; others return HYENA_ENOSUP. */
+int hyena_featurizer_gates_fwd(const hyena_proj_fwd* proj, void* xv_out, void* x2_out,
+                               int64_t B, int64_t L, int64_t D, int front_pad, void* stream);
 
 /* A whole Hyena-SE / Hyena-MR layer at prefill in one launch: featurizer FIR, split, x1*v gate, inner FIR,
  * bias rule (NONE or GATED_FP32), x2 gate; u [B][L][3D] in, out [B][L][D], nothing in between touches device

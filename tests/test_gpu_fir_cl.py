@@ -273,3 +273,60 @@ def test_layer_fwd_oldest_tap_across_segments(Ks, nseg, override):
     # the gates themselves carry the featurizer's own rounding boundary (one bf16 ulp of x1, v or x2 now and then),
     # which moves bx by up to 2^-7 relatively: 2^-6 * S covers it, a wrong halo sample is off by ~S / 11
     assert_gated_close(y, ref, zr, x2, S, 2.0 ** -6, ulps_z=2.0, gate_ulps=1.0, what=f"fused MR layer Ks={Ks} nseg={nseg}")
+
+
+@pytest.mark.parametrize("segments", [1, 2], indirect=True)      # blocks that walk all tiles of a row / half of them
+@pytest.mark.parametrize("B,L,D,H,Ks,cs,il,flip,sbias", [
+    (2, 512, 64, 4, 3, False, True, False, False),        # Evo 2 layout: interleaved gates
+    (1, 1000, 128, 4, 3, False, True, True, True),        # L % 256 != 0, flipped gates, featurizer bias
+    (2, 333, 96, 4, 3, True, False, False, True),         # head-blocked split (head_dim 24), L % 8 != 0, D % 64 != 0
+    (1, 700, 200, 5, 4, False, False, False, False),      # plain split, 4-tap featurizer
+    (1, 261, 64, 2, 4, False, True, False, True),
+    (3, 5, 64, 4, 3, False, True, False, True),           # shorter than one pass
+])
+def test_featurizer_gates_fwd_vs_oracle_and_unfused_path(B, L, D, H, Ks, cs, il, flip, sbias, segments):
+    # the gate-fused featurizer against the oracle's featurizer / interleave / split / x1*v, and bit for bit
+    # against the three-tensor featurizer kernel followed by the same split
+    g = torch.Generator().manual_seed(L + D + Ks)
+    C = 3 * D
+    u = torch.randn(B, L, C, generator=g).bfloat16()
+    wf = torch.randn(C, 1, Ks, generator=g) / Ks ** 0.5
+    bf = torch.randn(C, generator=g).bfloat16() if sbias else None
+    z, _ = O.parallel_fir(u, wf, bf, fir_length=Ks, dim_last=True, gate=False)
+    if il:
+        z = O.interleave(z)
+    x2, x1, v = O.split_gates(z, (D, H, D // H, 16, D), cs, flip)
+    pad = (-L) % 8
+    cmap = ops.gate_channel_map(D, interleave=il, head_dim=D // H if cs else None)
+    xv, g2 = ops.featurizer_gates_fwd(u.to(DEV), wf.reshape(C, Ks).t().contiguous().to(DEV),
+                                      None if bf is None else bf.to(DEV), cmap, flip_x1x2=flip, front_pad=pad)
+    assert xv.shape == g2.shape == (B, D, L + pad)
+    assert not xv[..., :pad].any() and not g2[..., :pad].any()
+    assert rel_err(xv[..., pad:], (x1 * v)) <= 1e-2 and rel_err(g2[..., pad:], x2) <= 1e-2
+    zk = ops.featurizer_fwd(u.to(DEV), wf.reshape(C, Ks).to(DEV), None if bf is None else bf.to(DEV), interleave=il,
+                            front_pad=pad)
+    hd = D // H if cs else None
+    k2, k1, kv = (zk.reshape(B, H, 3, D // H, -1)[:, :, i].reshape(B, D, -1) for i in range(3)) if cs else zk.split(D, 1)
+    if flip:
+        k1, k2 = k2, k1
+    assert torch.equal(xv, k1 * kv) and torch.equal(g2, k2.contiguous())
+
+
+@pytest.mark.parametrize("cplx,G", [(True, 8), (False, 128)])
+def test_li_fwd_on_premultiplied_rows(cplx, G):
+    # hyena_li_fwd with v = NULL: x1 holds bf16(x1*v) already; same output and state as the three-gate call
+    B, D, L, S = 2, 128, 4096, 16
+    g = torch.Generator().manual_seed(21)
+    x1, x2, v = (torch.randn(B, D, L, generator=g).bfloat16().to(DEV) for _ in range(3))
+    lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(G, S, seed=4)
+    Dc = torch.randn(D, generator=g).bfloat16().to(DEV)
+    plan = ops.ModalPlan(lp.to(DEV), r.to(DEV))
+    want, _, st_want = ops.li_fwd_rows(ops.rows_of(x1), ops.rows_of(x2), ops.rows_of(v), plan, Dc, B, D, L, device=DEV,
+                                       want_state=True)
+    xv = x1 * v
+    got, _, st_got = ops.li_fwd_rows(ops.rows_of(xv), ops.rows_of(x2), None, plan, Dc, B, D, L, device=DEV,
+                                     want_state=True)
+    assert torch.equal(got, want) and torch.equal(torch.view_as_real(st_got) if cplx else st_got,
+                                                  torch.view_as_real(st_want) if cplx else st_want)
+    with pytest.raises(NotImplementedError):      # v without x2 has no meaning
+        ops.li_fwd_rows(ops.rows_of(x1), None, ops.rows_of(v), plan, Dc, B, D, L, device=DEV)

@@ -221,6 +221,8 @@ class HyenaCascade(nn.Module):
         caching = inference_params is not None
         if not masked and self.fuse_prefill and self._can_fuse_prefill(u, L, caching):
             return self._fused_prefill(u, inference_params), inference_params
+        if not masked and self.fuse_prefill and self._can_fuse_gates(u):
+            return self._modal_prefill_from_projection(u, inference_params), inference_params
         w = self._f32_param("short_filter_weight", (C, Ks))
         # the sequence-major kernels take multiples of 8 samples: other lengths run behind -L % 8 zero samples
         pad, L_true = (-L) % 8, L
@@ -288,20 +290,54 @@ class HyenaCascade(nn.Module):
             return False
         return u.stride(2) == 1 and u.stride(1) % 8 == 0 and u.stride(0) % 8 == 0 and u.data_ptr() % 16 == 0
 
-    def _fused_prefill(self, u, inference_params):
-        """u [B, L, 3D] -> y [B, L, D] in one launch; with a cache object also the two FIR caches."""
-        B, L, C = u.shape
-        K, Ks = self.fir_inner_filter_length, self.short_filter_length
+    def _can_fuse_gates(self, u):
+        """Whether hyena_featurizer_gates_fwd covers this layer: a Hyena-LI layer (modal filter, no truncated-FIR
+        branch) with a 3- or 4-tap featurizer, a closed channel map and an aligned projection."""
+        D, hd = self.hidden_size, self.hidden_size_per_attention_head
+        if self.fir_inner_filter_length or self.long_fir_threshold is not None:
+            return False
+        if self.short_filter_length not in (3, 4) or self._channel_map() is None:
+            return False
+        if D % 8 or (self.column_split_hyena and hd % 8):
+            return False
+        return u.stride(2) == 1 and u.stride(1) % 8 == 0 and u.stride(0) % 8 == 0 and u.data_ptr() % 16 == 0
+
+    def _featurizer_taps_t(self, C, Ks):
         key = ("short_filter_weight_t", id(self.short_filter_weight), self.short_filter_weight.data_ptr(),
                self.short_filter_weight._version)
         hit = self._f32_cache.get("wf_t")
         if hit is None or hit[0] != key:
             hit = (key, self._f32_param("short_filter_weight", (C, Ks)).t().contiguous())
             self._f32_cache["wf_t"] = hit
+        return hit[1]
+
+    def _modal_prefill_from_projection(self, u, inference_params):
+        """Hyena-LI prefill in two launches: featurizer + split + x1*v (rows xv, x2), then the modal scan."""
+        B, L, C = u.shape
+        D, Ks = self.hidden_size, self.short_filter_length
+        caching = inference_params is not None
+        pad = (-L) % 8
+        xv, x2 = ops.featurizer_gates_fwd(u, self._featurizer_taps_t(C, Ks), self._f32_param("short_filter_bias"),
+                                          self._channel_map(), flip_x1x2=self.hyena_flip_x1x2, front_pad=pad)
+        y, _, state = ops.li_fwd_rows(ops.rows_of(xv), ops.rows_of(x2), None, self.modal_plan(), self.D, B, D, L + pad,
+                                      device=u.device, want_state=caching)
+        if caching:
+            inference_params.state_dict[self.layer_idx] = state
+            inference_params.fir_state_dict[self.layer_idx] = _ring(u[:, max(L - (Ks - 1), 0):], Ks - 1)
+            self._decode = None
+        if pad:
+            y = y[..., pad:]
+        return y.permute(0, 2, 1)
+
+    def _fused_prefill(self, u, inference_params):
+        """u [B, L, 3D] -> y [B, L, D] in one launch; with a cache object also the two FIR caches."""
+        B, L, C = u.shape
+        K, Ks = self.fir_inner_filter_length, self.short_filter_length
+        wf_t = self._featurizer_taps_t(C, Ks)
         mr = K >= 128
         taps = self._f32_param("h", (self.h.shape[0], K))
         caching = inference_params is not None
-        res = ops.fir_layer_fwd(u, hit[1], self._f32_param("short_filter_bias"), self._channel_map(), taps,
+        res = ops.fir_layer_fwd(u, wf_t, self._f32_param("short_filter_bias"), self._channel_map(), taps,
                                 bias=self._f32_param("D") if mr else None,
                                 bias_mode=HYENA_BIAS_GATED_FP32 if mr else HYENA_BIAS_NONE, taps_reversed=not mr,
                                 flip_x1x2=self.hyena_flip_x1x2, bx_from=max(L - (K - 1), 0) if caching else None)

@@ -58,6 +58,78 @@ __device__ __forceinline__ uint32_t pair_hi(uint32_t first, uint32_t second) {
 // element e (0..7) of a packed row of 8 bf16, as float
 __device__ __forceinline__ float el(const u32x4& r, int e) { return (e & 1) ? bf_hi(r[e >> 1]) : bf_lo(r[e >> 1]); }
 
+// Featurizer FIR and gates of one lane's 4 rows x 8 operator channels from its three row pieces (raw[i][r]: piece i,
+// row r - (KS - 1) relative to the lane's first row; w_lds: the block's taps and bias in lane-piece order):
+// bx = bf16(x1*v) and g2 = x2, each as 4 rows of 8 packed channels.
+template <int FEAT, int KS>
+__device__ __forceinline__ void lane_gates(const u32x4 (&raw)[3][KS + 3], const float* w_lds, int cb, const ProjFwd& pj,
+                                           u32x4 (&bx)[4], u32x4 (&g2)[4]) {
+    u32x4 zq[3][4];
+    int woff = 8 * cb;
+    asm volatile("" : "+v"(woff));      // re-read the tap table every step instead of pinning 96 registers
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        float tw[KS][8], bb[8];
+#pragma unroll
+        for (int k = 0; k <= KS; ++k) {
+            const f32x4 t0 = *(const f32x4*)(w_lds + (k * 3 + i) * CB + woff);
+            const f32x4 t1 = *(const f32x4*)(w_lds + (k * 3 + i) * CB + woff + 4);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (k < KS) { tw[k][j] = t0[j]; tw[k][4 + j] = t1[j]; }
+                else { bb[j] = t0[j]; bb[4 + j] = t1[j]; }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float acc[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+#pragma unroll
+            for (int k = 0; k < KS; ++k) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[j] = fmaf(tw[k][j], el(raw[i][q + k], j), acc[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) zq[i][q][j] = pack_bf2(acc[2 * j], acc[2 * j + 1]);
+        }
+        if (pj.bias) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    zq[i][q][j] = pack_bf2(bf_lo(zq[i][q][j]) + bb[2 * j], bf_hi(zq[i][q][j]) + bb[2 * j + 1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);      // one piece at a time: its rows are dead before the next starts
+    }
+    // rows past the end of the sequence hold bias-only values; they are never stored and never feed a
+    // valid output (causality), so they need no masking.  Rows before t = 0 do not exist (ts0 >= 0).
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float a1[2], a2[2], av[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int jd = 2 * j + e;
+                if (FEAT == 3) {        // channel 3*jd + gate of the lane's 24
+                    const int e0 = 3 * jd, e1 = 3 * jd + 1, e2 = 3 * jd + 2;
+                    a2[e] = el(zq[e0 >> 3][q], e0 & 7);
+                    a1[e] = el(zq[e1 >> 3][q], e1 & 7);
+                    av[e] = el(zq[e2 >> 3][q], e2 & 7);
+                } else {
+                    a2[e] = el(zq[0][q], jd);
+                    a1[e] = el(zq[1][q], jd);
+                    av[e] = el(zq[2][q], jd);
+                }
+                if (pj.flip) { const float t = a1[e]; a1[e] = a2[e]; a2[e] = t; }
+            }
+            bx[q][j] = pack_bf2(a1[0] * av[0], a1[1] * av[1]);
+            g2[q][j] = pack_bf2(a2[0], a2[1]);
+        }
+    }
+}
+
 // FEAT: 0 = gates given as three channel-last tensors; 1 = gates from the fused featurizer, unit channel
 // stride (plain or head-blocked split); 3 = fused featurizer with interleaved gates (channel 3d+i).
 // KS = featurizer taps (FEAT != 0).  AUX = also store y2 (z before the x2 gate) and / or bx = bf16(x1*v).  With the
@@ -203,71 +275,8 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
         const bool compute = ts >= t_begin;
         // ---- (a) gates of this lane's 4 x 8 block
         u32x4 bx[4], g2[4];
-        if (FEAT) {
-            u32x4 zq[3][4];
-            int woff = 8 * cb;
-            asm volatile("" : "+v"(woff));      // re-read the tap table every step instead of pinning 96 registers
-#pragma unroll
-            for (int i = 0; i < 3; ++i) {
-                float tw[KS][8], bb[8];
-#pragma unroll
-                for (int k = 0; k <= KS; ++k) {
-                    const f32x4 t0 = *(const f32x4*)(w_lds + (k * 3 + i) * CB + woff);
-                    const f32x4 t1 = *(const f32x4*)(w_lds + (k * 3 + i) * CB + woff + 4);
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        if (k < KS) { tw[k][j] = t0[j]; tw[k][4 + j] = t1[j]; }
-                        else { bb[j] = t0[j]; bb[4 + j] = t1[j]; }
-                    }
-                }
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    float acc[8];
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-#pragma unroll
-                    for (int k = 0; k < KS; ++k) {
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) acc[j] = fmaf(tw[k][j], el(raw[i][q + k], j), acc[j]);
-                    }
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) zq[i][q][j] = pack_bf2(acc[2 * j], acc[2 * j + 1]);
-                }
-                if (pj.bias) {
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-#pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            zq[i][q][j] = pack_bf2(bf_lo(zq[i][q][j]) + bb[2 * j], bf_hi(zq[i][q][j]) + bb[2 * j + 1]);
-                }
-                __builtin_amdgcn_sched_barrier(0);      // one piece at a time: its rows are dead before the next starts
-            }
-            // rows past the end of the sequence hold bias-only values; they are never stored and never feed a
-            // valid output (causality), so they need no masking.  Rows before t = 0 do not exist (ts0 >= 0).
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float a1[2], a2[2], av[2];
-#pragma unroll
-                    for (int e = 0; e < 2; ++e) {
-                        const int jd = 2 * j + e;
-                        if (FEAT == 3) {        // channel 3*jd + gate of the lane's 24
-                            const int e0 = 3 * jd, e1 = 3 * jd + 1, e2 = 3 * jd + 2;
-                            a2[e] = el(zq[e0 >> 3][q], e0 & 7);
-                            a1[e] = el(zq[e1 >> 3][q], e1 & 7);
-                            av[e] = el(zq[e2 >> 3][q], e2 & 7);
-                        } else {
-                            a2[e] = el(zq[0][q], jd);
-                            a1[e] = el(zq[1][q], jd);
-                            av[e] = el(zq[2][q], jd);
-                        }
-                        if (pj.flip) { const float t = a1[e]; a1[e] = a2[e]; a2[e] = t; }
-                    }
-                    bx[q][j] = pack_bf2(a1[0] * av[0], a1[1] * av[1]);
-                    g2[q][j] = pack_bf2(a2[0], a2[1]);
-                }
-            }
+        if constexpr (FEAT != 0) {
+            lane_gates<FEAT, KS>(raw, w_lds, cb, pj, bx, g2);
         } else {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -406,6 +415,124 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     }
 }
 
+// Featurizer and gates for the sequence-major operators (Hyena-LI): u [B][L][3D] in, xv = bf16(x1*v) and x2 out as
+// [B][D][Lout] rows (Lout = L + pad, the first `pad` columns zero).  One block takes 64 operator channels x 256
+// output columns: the lanes evaluate the featurizer on their 4 rows x 8 channels as in fir_cl_kernel (two passes of
+// 128 rows), transpose into two LDS tiles [64 ch][256 columns] and the block stores 512-byte runs of each channel
+// row; a block walks several consecutive tiles, the first row pieces of the next one requested before the stores.
+// Blocks with neighbouring ids take neighbouring channel strips of the same rows.  Plain (cached) stores: the
+// neighbouring runs of a row written by the next tiles merge in the cache (measured 3-8 % faster than streaming stores).
+constexpr int GT = 256;        // output columns per block
+constexpr int GRS = 264;       // row stride (elements) of the transposed tiles: 528 B = 16 * 33
+
+template <int FEAT, int KS>
+__global__ __launch_bounds__(256, 2) void proj_gates_kernel(ProjFwd pj, bf16_t* __restrict__ xv_out,
+                                                            bf16_t* __restrict__ x2_out, int64_t L, int64_t Lout,
+                                                            int pad, int64_t D, int ndb, int nchunk, int ntpb) {
+    constexpr int RF = KS - 1, NR = 4 + RF;
+    __shared__ __attribute__((aligned(16))) bf16_t xv_t[CB * GRS];
+    __shared__ __attribute__((aligned(16))) bf16_t x2_t[CB * GRS];
+    __shared__ __attribute__((aligned(16))) float w_lds[(KS + 1) * 3 * CB];
+    const int tid = threadIdx.x;
+    const uint32_t bid = blockIdx.x;
+    const uint32_t db = bid % (uint32_t)ndb;
+    const uint32_t chunk = (bid / (uint32_t)ndb) % (uint32_t)nchunk;      // ntpb consecutive tiles along the columns
+    const int64_t b = bid / ((uint32_t)ndb * (uint32_t)nchunk);
+    const uint32_t d0 = db * CB;
+    const int64_t c_begin = (int64_t)chunk * ntpb * GT;
+    const int64_t c_end = c_begin + (int64_t)ntpb * GT < Lout ? c_begin + (int64_t)ntpb * GT : Lout;
+    if (c_begin >= c_end) return;
+
+    const int cb = tid & 7, rb = tid >> 3;
+    const int swz_io = 32 * (cb >> 1);                     // as in fir_cl_kernel: keeps the 8-byte transposed writes off each other's banks
+    const uint32_t dch = d0 + 8 * cb;
+    const bool ch_ok = dch < (uint32_t)D;
+    const bf16_t* pp[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+        pp[i] = FEAT == 3 ? pj.u + b * pj.bs + 3 * (int64_t)dch + 8 * i : pj.u + b * pj.bs + pj.chan(i, ch_ok ? dch : 0);
+
+    const u32x4 zero4 = {0, 0, 0, 0};
+    // the 18 (21) row pieces of one pass of 128 columns starting at column cs; rows past either end read as zero
+    auto load_pass = [&](int64_t cs, u32x4 (&raw)[3][NR]) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int64_t t = cs + 4 * rb + r - RF - pad;  // input sample of this row
+            const bool ok = ch_ok && t >= 0 && t < L;
+#pragma unroll
+            for (int i = 0; i < 3; ++i) raw[i][r] = ok ? *(const u32x4*)(pp[i] + t * pj.ts) : zero4;
+        }
+    };
+    u32x4 raw[3][NR];
+    load_pass(c_begin, raw);                               // travels while the tap table is staged
+
+    for (int e = tid; e < (KS + 1) * 3 * CB; e += 256) {   // taps / bias of the block's channels in lane-piece order
+        const int k = e / (3 * CB), r = e - k * 3 * CB, i = r / CB, dl = r - i * CB;
+        const uint32_t dd = d0 + dl;
+        float val = 0.f;
+        if (dd < (uint32_t)D) {
+            const uint32_t ch = FEAT == 3 ? 3 * (d0 + (dl & ~7)) + 8 * i + (dl & 7) : pj.chan(i, dd);
+            if (k < KS) val = pj.w[(int64_t)k * 3 * D + ch];
+            else if (pj.bias) val = pj.bias[ch];
+        }
+        w_lds[e] = val;
+    }
+    __syncthreads();
+
+    // featurizer, gates and the 4 x 8 transposes of one pass into half `half` of the two tiles
+    auto gate_pass = [&](int64_t cs, int half, const u32x4 (&raw)[3][NR]) {
+        u32x4 bx[4], g2[4];
+        lane_gates<FEAT, KS>(raw, w_lds, cb, pj, bx, g2);
+        if (cs < pad) {                                    // the padding columns stay zero, bias or not
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (cs + 4 * rb + q < pad) { bx[q] = zero4; g2[q] = zero4; }
+        }
+        bf16_t* xb = xv_t + (8 * cb) * GRS + half * TL + ((4 * rb) ^ swz_io);
+        bf16_t* gb = x2_t + (8 * cb) * GRS + half * TL + ((4 * rb) ^ swz_io);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            u32x2 t2, t3;
+            if (c & 1) {
+                t2[0] = pair_hi(bx[0][c >> 1], bx[1][c >> 1]); t2[1] = pair_hi(bx[2][c >> 1], bx[3][c >> 1]);
+                t3[0] = pair_hi(g2[0][c >> 1], g2[1][c >> 1]); t3[1] = pair_hi(g2[2][c >> 1], g2[3][c >> 1]);
+            } else {
+                t2[0] = pair_lo(bx[0][c >> 1], bx[1][c >> 1]); t2[1] = pair_lo(bx[2][c >> 1], bx[3][c >> 1]);
+                t3[0] = pair_lo(g2[0][c >> 1], g2[1][c >> 1]); t3[1] = pair_lo(g2[2][c >> 1], g2[3][c >> 1]);
+            }
+            *(u32x2*)(xb + c * GRS) = t2;
+            *(u32x2*)(gb + c * GRS) = t3;
+        }
+    };
+
+    const int l32 = tid & 31, r8 = tid >> 5;
+    const int tcol = 8 * l32;
+#pragma unroll 1
+    for (int64_t c0 = c_begin; c0 < c_end; c0 += GT) {
+        const bool second = c0 + TL < c_end, next = c0 + GT < c_end;
+        gate_pass(c0, 0, raw);
+        if (second) {
+            load_pass(c0 + TL, raw);
+            gate_pass(c0 + TL, 1, raw);
+        }
+        if (next) load_pass(c0 + GT, raw);                 // travels during the stores
+        __syncthreads();
+        // ---- stores: 32 lanes cover the 512 bytes of one channel row, 8 rows per round, xv then x2
+        const int64_t col = c0 + tcol;
+        if (col < Lout) {
+#pragma unroll 4
+            for (int rnd = 0; rnd < 2 * CB / 8; ++rnd) {
+                const int rr = rnd * 8 + r8, ch = rr & (CB - 1);
+                if (d0 + ch >= (uint32_t)D) continue;
+                const bf16_t* tile = rr < CB ? xv_t : x2_t;
+                const u32x4 o = *(const u32x4*)(tile + ch * GRS + (tcol & TL) + ((tcol & (TL - 1)) ^ (32 * (ch >> 4))));
+                *(u32x4*)((rr < CB ? xv_out : x2_out) + (b * D + d0 + ch) * Lout + col) = o;
+            }
+        }
+        if (next) __syncthreads();                         // the tiles are free again
+    }
+}
+
 struct LaunchArgs {
     ClMap x1, x2, v;
     ProjFwd pj;
@@ -503,6 +630,31 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     return hyena_check_launch(who);
 }
 
+// Validates a prefill featurizer descriptor and fills the launch arguments (feat = 1: unit channel stride, 3: interleaved)
+static int make_proj_fwd(const hyena_proj_fwd* proj, int64_t D, const char* who, LaunchArgs& a) {
+    if (!proj || !proj->u || !proj->w) return hyena_fail(HYENA_EINVAL, "%s: proj, proj->u, proj->w are required", who);
+    if (proj->Ks != 3 && proj->Ks != 4)
+        return hyena_fail(HYENA_ENOSUP, "%s: featurizer length %d (3 or 4 supported)", who, proj->Ks);
+    if (D <= 0 || D % 8 != 0 || ((uintptr_t)proj->u & 15) || proj->u_batch_stride % 8 != 0 ||
+        proj->u_time_stride % 8 != 0)
+        return hyena_fail(HYENA_EALIGN, "%s: D and strides must be multiples of 8, u 16-byte aligned", who);
+    if (proj->ch_inner <= 0 || proj->ch_outer < 0 || proj->gate_stride <= 0)
+        return hyena_fail(HYENA_EINVAL, "%s: bad featurizer channel map", who);
+    a.pj.u = (const bf16_t*)proj->u; a.pj.bs = proj->u_batch_stride; a.pj.ts = proj->u_time_stride;
+    a.pj.w = proj->w; a.pj.bias = proj->bias;
+    a.pj.ch_inner = (uint32_t)(proj->ch_inner > D ? D : proj->ch_inner); a.pj.ch_outer = (uint32_t)proj->ch_outer;
+    a.pj.gate_stride = (uint32_t)proj->gate_stride; a.pj.flip = proj->flip_x1x2 != 0;
+    if (proj->ch_stride == 3 && proj->gate_stride == 1 && proj->ch_inner >= D) a.feat = 3;
+    else if (proj->ch_stride == 1 && proj->ch_inner % 8 == 0 && proj->ch_outer % 8 == 0 && proj->gate_stride % 8 == 0) {
+        a.feat = 1;
+        const int64_t last = ((D - 1) / proj->ch_inner) * proj->ch_outer + 2 * proj->gate_stride + (D - 1) % proj->ch_inner;
+        if (last >= 3 * D) return hyena_fail(HYENA_EINVAL, "%s: featurizer channel map reaches channel %lld of %lld", who,
+                                             (long long)last, (long long)(3 * D));
+    } else return hyena_fail(HYENA_ENOSUP, "%s: this featurizer channel map has no fused kernel", who);
+    a.ks = proj->Ks; a.pre = true; a.post = true;
+    return 0;
+}
+
 static bool cl_ok(const hyena_cl* c) {
     return c && c->ptr && !((uintptr_t)c->ptr & 15) && c->batch_stride % 8 == 0 && c->time_stride % 8 == 0;
 }
@@ -533,27 +685,42 @@ extern "C" int hyena_fir_layer_fwd(const hyena_proj_fwd* proj, const float* h, i
                                    int bias_mode, void* out, void* bx_out, int64_t bx_from, int64_t B, int64_t L,
                                    int64_t D, int64_t G, int K, void* stream) {
     const char* who = "hyena_fir_layer_fwd";
-    if (!proj || !proj->u || !proj->w) return hyena_fail(HYENA_EINVAL, "%s: proj, proj->u, proj->w are required", who);
-    if (proj->Ks != 3 && proj->Ks != 4)
-        return hyena_fail(HYENA_ENOSUP, "%s: featurizer length %d (3 or 4 supported)", who, proj->Ks);
-    if (D <= 0 || D % 8 != 0 || ((uintptr_t)proj->u & 15) || proj->u_batch_stride % 8 != 0 ||
-        proj->u_time_stride % 8 != 0)
-        return hyena_fail(HYENA_EALIGN, "%s: D and strides must be multiples of 8, u 16-byte aligned", who);
-    if (proj->ch_inner <= 0 || proj->ch_outer < 0 || proj->gate_stride <= 0)
-        return hyena_fail(HYENA_EINVAL, "%s: bad featurizer channel map", who);
     LaunchArgs a = {};
-    a.pj.u = (const bf16_t*)proj->u; a.pj.bs = proj->u_batch_stride; a.pj.ts = proj->u_time_stride;
-    a.pj.w = proj->w; a.pj.bias = proj->bias;
-    a.pj.ch_inner = (uint32_t)(proj->ch_inner > D ? D : proj->ch_inner); a.pj.ch_outer = (uint32_t)proj->ch_outer;
-    a.pj.gate_stride = (uint32_t)proj->gate_stride; a.pj.flip = proj->flip_x1x2 != 0;
-    if (proj->ch_stride == 3 && proj->gate_stride == 1 && proj->ch_inner >= D) a.feat = 3;
-    else if (proj->ch_stride == 1 && proj->ch_inner % 8 == 0 && proj->ch_outer % 8 == 0 && proj->gate_stride % 8 == 0) {
-        a.feat = 1;
-        const int64_t last = ((D - 1) / proj->ch_inner) * proj->ch_outer + 2 * proj->gate_stride + (D - 1) % proj->ch_inner;
-        if (last >= 3 * D) return hyena_fail(HYENA_EINVAL, "%s: featurizer channel map reaches channel %lld of %lld", who,
-                                             (long long)last, (long long)(3 * D));
-    } else return hyena_fail(HYENA_ENOSUP, "%s: this featurizer channel map has no fused kernel", who);
-    a.ks = proj->Ks; a.pre = true; a.post = true;
+    if (int rc = make_proj_fwd(proj, D, who, a)) return rc;
     if (bias_mode == HYENA_BIAS_ADD) return hyena_fail(HYENA_ENOSUP, "%s: additive inner bias", who);
     return fir_cl_launch(a, h, taps_reversed, bias, bias_mode, out, nullptr, bx_out, bx_from, B, L, D, G, K, stream, who);
+}
+
+extern "C" int hyena_featurizer_gates_fwd(const hyena_proj_fwd* proj, void* xv_out, void* x2_out, int64_t B, int64_t L,
+                                          int64_t D, int front_pad, void* stream) {
+    const char* who = "hyena_featurizer_gates_fwd";
+    if (!xv_out || !x2_out) return hyena_fail(HYENA_EINVAL, "%s: both outputs are required", who);
+    if (B < 0 || L < 0 || D >= (1LL << 30)) return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld L=%lld D=%lld", who,
+                                                               (long long)B, (long long)L, (long long)D);
+    if (front_pad < 0 || front_pad > 7) return hyena_fail(HYENA_EINVAL, "%s: front_pad %d outside 0..7", who, front_pad);
+    LaunchArgs a = {};
+    if (int rc = make_proj_fwd(proj, D, who, a)) return rc;
+    const int64_t Lout = L > 0 ? L + front_pad : 0;
+    if (Lout % 8 != 0 || (((uintptr_t)xv_out | (uintptr_t)x2_out) & 15))
+        return hyena_fail(HYENA_EALIGN, "%s: L + front_pad must be a multiple of 8, outputs 16-byte aligned", who);
+    if (B == 0 || L == 0) return 0;
+    const int64_t ndb = (D + CB - 1) / CB, ntt = (Lout + GT - 1) / GT;
+    // consecutive tiles per block (the tap table is staged once, the next tile's rows travel during the stores): as
+    // many as leave about four rounds of resident blocks (512 at a time), at most 4 (measured flat from 2 to 8)
+    int64_t ntpb = B * ndb * ntt / 2048;
+    ntpb = ntpb < 1 ? 1 : (ntpb > 4 ? 4 : ntpb);
+    { const int64_t x = hyena_override(HYENA_OV_CL_NSEG); if (x >= 1) ntpb = (ntt + x - 1) / x; }
+    const int64_t nchunk = (ntt + ntpb - 1) / ntpb;
+    if (B * ndb * nchunk > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: problem too large for one launch", who);
+    dim3 grid((unsigned)(B * ndb * nchunk));
+    hipStream_t s = (hipStream_t)stream;
+#define PG_GO(F, KSV)                                                                                              \
+    hipLaunchKernelGGL((proj_gates_kernel<F, KSV>), grid, dim3(256), 0, s, a.pj, (bf16_t*)xv_out, (bf16_t*)x2_out, L, \
+                       Lout, front_pad, D, (int)ndb, (int)nchunk, (int)ntpb)
+    if (a.feat == 3 && a.ks == 3) PG_GO(3, 3);
+    else if (a.feat == 3) PG_GO(3, 4);
+    else if (a.ks == 3) PG_GO(1, 3);
+    else PG_GO(1, 4);
+#undef PG_GO
+    return hyena_check_launch(who);
 }

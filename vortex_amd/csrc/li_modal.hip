@@ -744,7 +744,7 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
     if (!rows_valid(x1) || !rows_valid(x2) || !rows_valid(v) || B * D >= (1LL << 31) || L >= (1LL << 40))
         return hyena_fail(HYENA_EINVAL, "%s: B*D and the channel map must fit 31 bits", who);
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
-    if (pre != post) return hyena_fail(HYENA_ENOSUP, "%s: pass both v and x2 or neither", who);
+    if (pre && !post) return hyena_fail(HYENA_ENOSUP, "%s: v without x2 (pass both, x2 alone with x1 holding x1*v, or neither)", who);
     if (B == 0 || L == 0) return 0;
     // Work decomposition (measured on B*D = 1024 .. 8192 rows, L = 8192 .. 524288):
     //  * rows of 65536 samples or more: one channel per wavefront, 2048 samples per step.  A wavefront then reads
@@ -796,6 +796,7 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
 #define LI_M(P, Q, N, Y) do { if (dmode == 1) LI_LAUNCH(P, Q, N, 1, Y); else if (dmode == 2) LI_LAUNCH(P, Q, N, 2, Y); else LI_LAUNCH(P, Q, N, 0, Y); } while (0)
 #define LI_N(P, Q) do { if (y32) LI_M(P, Q, false, true); else if (nt) LI_M(P, Q, true, false); else LI_M(P, Q, false, false); } while (0)
     if (pre && post) LI_N(true, true);
+    else if (post) LI_N(false, true);          // x1 already holds bf16(x1*v) (hyena_featurizer_gates_fwd)
     else LI_N(false, false);
 #undef LI_N
 #undef LI_M
