@@ -222,12 +222,17 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     const int lofs = lane * 8 + 32 * (lane >> 4);              // position inside a padded LDS row
     const bf16_t *p1[4], *pv[4], *p2[4];
     bf16_t* po[4];
+    // uniform 64-bit row addresses plus one 32-bit lane offset keep the sixteen row pointers out of the vector registers
+    const uint32_t lane_b = (uint32_t)lane * 16u;
+    auto lane_at = [&](const bf16_t* p) -> const bf16_t* { return (const bf16_t*)((const char*)p + lane_b); };
+    auto lane_to = [&](bf16_t* p) -> bf16_t* { return (bf16_t*)((char*)p + lane_b); };
     // LDS row r is channel d0 + r (CPW = 4) or the r-th 512-sample piece of channel d0 (CPW = 1)
     auto roff = [](int r) -> int64_t { return CPW == 4 ? 0 : (int64_t)TL * r; };
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int64_t d = d0 + (CPW == 4 ? r : 0);
-        const int64_t o = woff + roff(r) + lane * 8 - pad;     // pointers are in virtual positions; never used below lo
+        const int64_t o = woff + roff(r) - pad;                // virtual positions, never used below lo; wave-uniform: the
+                                                               // lane's 16 bytes are added at each access (lane_at)
         p1[r] = a.x1.row(b, d) + o;
         pv[r] = PRE ? a.v.row(b, d) + o : nullptr;
         p2[r] = POST ? a.x2.row(b, d) + o : nullptr;
@@ -243,9 +248,9 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                 const int64_t t = (int64_t)p * STEP;
                 const int64_t pos = t + roff(r) + lane * 8;
                 const bool ok = pos < Lw && pos >= lo;
-                c1[p][r] = ok ? ld16<NT>(p1[r] + t) : zero4;
-                cv[p][r] = (PRE && ok) ? ld16<NT>(pv[r] + t) : zero4;
-                c2[p][r] = (POST && ok) ? ld16<NT>(p2[r] + t) : zero4;
+                c1[p][r] = ok ? ld16<NT>(lane_at(p1[r] + t)) : zero4;
+                cv[p][r] = (PRE && ok) ? ld16<NT>(lane_at(pv[r] + t)) : zero4;
+                c2[p][r] = (POST && ok) ? ld16<NT>(lane_at(p2[r] + t)) : zero4;
             }
     };
     // With four channels per wavefront the rows are requested before the fragment build and travel during it
@@ -386,9 +391,11 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
         for (int k = 1; k < 16 / CPW; ++k) { const float t = ppr * pcr - ppi * pci; ppi = ppr * pci + ppi * pcr; ppr = t; }
     }
 
-    // One 512-sample step.  GUARD = true predicates every access on the sequence bounds.  The
-    // unguarded form exists, but straight-line code lets the compiler hoist so many loads that it
-    // spills registers, so every step runs guarded.
+    // One step.  GUARD = true tests every access against the row's bounds (a wave-uniform test for whole pieces, per-lane
+    // predicates otherwise); GUARD = false is for steps whose loads, stores and refills are all whole pieces inside the
+    // row: no branch surrounds a memory instruction there, which is what lets the compiler count exactly how many
+    // younger requests may still be in flight when a register stage is consumed (with branches around them it has to
+    // wait for everything outstanding, the prefetched stages included).
     auto step = [&](auto guard_tag, const int p, const int64_t ts) {
         constexpr bool GUARD = decltype(guard_tag)::value;
         const int pp = (p + PF - 1) % PF;                      // register stage of the previous step
@@ -398,18 +405,22 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) *(u32x4*)(u_w + r * URS + lofs) = gate_mul<PRE>(c1[p][r], cv[p][r]);
         // whole pieces inside the row (a wave-uniform test) are requested without per-lane predicates
-        if (tn + TLW <= Lw) {
+        if (!GUARD || tn + TLW <= Lw) {
+            // (without branches around them the scheduler would move these requests, and what waits on the registers
+            // they overwrite, far from here and run out of registers: pin the group where the branches used to hold it)
+            if (!GUARD) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                c1[p][r] = ld16<NT>(p1[r] + tn);
-                if (PRE) cv[p][r] = ld16<NT>(pv[r] + tn);
+                c1[p][r] = ld16<NT>(lane_at(p1[r] + tn));
+                if (PRE) cv[p][r] = ld16<NT>(lane_at(pv[r] + tn));
             }
+            if (!GUARD) __builtin_amdgcn_sched_barrier(0);
         } else {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const bool okn = tn + roff(r) + lane * 8 < Lw;
-                c1[p][r] = okn ? ld16<NT>(p1[r] + tn) : zero4;
-                cv[p][r] = (PRE && okn) ? ld16<NT>(pv[r] + tn) : zero4;
+                c1[p][r] = okn ? ld16<NT>(lane_at(p1[r] + tn)) : zero4;
+                cv[p][r] = (PRE && okn) ? ld16<NT>(lane_at(pv[r] + tn)) : zero4;
             }
         }
         wave_sync();
@@ -466,20 +477,22 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                         o[r][j] = pack_bf2(bf_lo(zz[r][j]) * bf_lo(c2[pp][r][j]), bf_hi(zz[r][j]) * bf_hi(c2[pp][r][j]));
                 }
             }
-            if (ts_out >= 0 && (ts_out > 0 || lo <= 0) && t_refill + TLW <= Lw) {   // wave-uniform: store and refill whole pieces
+            if (!GUARD || (ts_out >= 0 && (ts_out > 0 || lo <= 0) && t_refill + TLW <= Lw)) {   // wave-uniform: store and refill whole pieces
+                if (!GUARD) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    st16<NT>(po[r] + ts_out, o[r]);
-                    if (POST) c2[pp][r] = ld16<NT>(p2[r] + t_refill);
+                    st16<NT>(lane_to(po[r] + ts_out), o[r]);
+                    if (POST) c2[pp][r] = ld16<NT>(lane_at(p2[r] + t_refill));
                 }
+                if (!GUARD) __builtin_amdgcn_sched_barrier(0);
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int64_t pos = ts_out + roff(r) + lane * 8;
                     const bool okc = ts_out >= 0 && pos < Lw && pos >= lo;
                     const bool okr = ts_out >= 0 && t_refill + roff(r) + lane * 8 < Lw;
-                    if (okc) st16<NT>(po[r] + ts_out, o[r]);
-                    if (ts_out >= 0) c2[pp][r] = (POST && okr) ? ld16<NT>(p2[r] + t_refill) : zero4;
+                    if (okc) st16<NT>(lane_to(po[r] + ts_out), o[r]);
+                    if (ts_out >= 0) c2[pp][r] = (POST && okr) ? ld16<NT>(lane_at(p2[r] + t_refill)) : zero4;
                 }
             }
         }
@@ -598,11 +611,26 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     };
 
     const std::integral_constant<bool, true> guarded;
-    // the bounds are the block's (Lv, not Lw): with COOP every wavefront runs every step and meets every barrier
+    const std::integral_constant<bool, false> whole;
+    // Rotations of PF steps.  A rotation is `whole` when every access of its steps is a whole piece inside the row: not
+    // the first one (its stores start at sample 0, behind the padding), and the refill of its last step, PF steps ahead,
+    // still ends inside the row of every wavefront of the block (the last one starts 3 pieces further on with COOP).
+    // Every guarded rotation, and the prologue, ends with a wait for all outstanding requests, so that the whole
+    // rotations start from a known state; they are the first and the last two of a row.
+    // The bounds are the block's (Lv, not Lw): with COOP every wavefront runs every step and meets every barrier.
+    constexpr int VMCNT0 = 0x0F70;                             // s_waitcnt vmcnt(0), other counters unconstrained
+    const int64_t whole_until = Lv - (COOP ? 3 * TLW : 0) - TLW - (int64_t)(2 * PF - 1) * STEP;
+    __builtin_amdgcn_s_waitcnt(VMCNT0);
     for (int64_t ts = 0; ts < Lv; ts += (int64_t)PF * STEP) {
+        if (ts > 0 && ts <= whole_until) {
 #pragma unroll
-        for (int p = 0; p < PF; ++p)
-            if (ts + (int64_t)p * STEP < Lv) step(guarded, p, ts + (int64_t)p * STEP);
+            for (int p = 0; p < PF; ++p) step(whole, p, ts + (int64_t)p * STEP);
+        } else {
+#pragma unroll
+            for (int p = 0; p < PF; ++p)
+                if (ts + (int64_t)p * STEP < Lv) step(guarded, p, ts + (int64_t)p * STEP);
+            __builtin_amdgcn_s_waitcnt(VMCNT0);
+        }
     }
     {   // output of the last step
         const int64_t ts_last = ((Lv + STEP - 1) / STEP - 1) * STEP;
@@ -623,7 +651,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                 for (int j = 0; j < 4; ++j)
                     o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(x2v[j]), bf_hi(zz[j]) * bf_hi(x2v[j]));
             }
-            if (okc) st16<NT>(po[r] + ts_last, o);
+            if (okc) st16<NT>(lane_to(po[r] + ts_last), o);
         }
     }
 
@@ -786,12 +814,14 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
     const bool y32 = y_conv_fp32 != nullptr;
     if (y32) nt = false;
 // prefetch depth in steps: two with four channels per wavefront (measured 1-3 % faster than three, which in turn
-// beats four, whose registers spill), three with one channel per wavefront (two is 30 % slower there)
+// beats four, whose registers spill).  One channel per wavefront: two for the gated forms (three stages of three or two
+// input streams leave the whole-piece steps short of registers: 75-110 spilled dwords and 1.63 against 1.52 ms on
+// x1*v rows at L = 262144), three for the ungated one (1.28 against 1.36 ms)
 #define LI_LAUNCH(P, Q, N, M, Y)                                                                           \
     do {                                                                                                   \
         if (cpw == 4 && coop) hipLaunchKernelGGL((li_kernel<P, Q, N, 2, M, Y, 4, true>), grid, dim3(256), 0, s, a);   \
         else if (cpw == 4) hipLaunchKernelGGL((li_kernel<P, Q, N, 2, M, Y, 4, false>), grid, dim3(256), 0, s, a);     \
-        else hipLaunchKernelGGL((li_kernel<P, Q, N, 3, M, Y, 1, false>), grid, dim3(256), 0, s, a);                   \
+        else hipLaunchKernelGGL((li_kernel<P, Q, N, (P || Q) ? 2 : 3, M, Y, 1, false>), grid, dim3(256), 0, s, a);    \
     } while (0)
 #define LI_M(P, Q, N, Y) do { if (dmode == 1) LI_LAUNCH(P, Q, N, 1, Y); else if (dmode == 2) LI_LAUNCH(P, Q, N, 2, Y); else LI_LAUNCH(P, Q, N, 0, Y); } while (0)
 #define LI_N(P, Q) do { if (y32) LI_M(P, Q, false, true); else if (nt) LI_M(P, Q, true, false); else LI_M(P, Q, false, false); } while (0)
