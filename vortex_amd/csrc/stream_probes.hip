@@ -50,7 +50,27 @@ __global__ __launch_bounds__(256) void stream_probe_kernel(const bf16_t* a, cons
         for (int r = 0; r < R; ++r)
             if (cur[p] >= 0) { const int64_t t = cur[p] + r * wk.L; x[p][r] = ldnt(a + t); y[p][r] = ldnt(b + t); z[p][r] = ldnt(c + t); }
     }
-    for (int64_t u0 = 0; u0 < wk.nunits; u0 += PF) {
+    // Rotations in which every unit and every refill exists run without a branch around any memory instruction: only
+    // then can the compiler count the younger requests that may still be in flight when a stage is consumed; with the
+    // tests of the loop below around them it waits for all outstanding requests at every step, which makes the
+    // prefetch depth meaningless.  (One wait for everything first: the prologue's requests were conditional.)
+    int64_t u0 = 0;
+    __builtin_amdgcn_s_waitcnt(0x0F70);                            // vmcnt(0)
+    for (; u0 + 2 * PF <= wk.nunits; u0 += PF) {
+#pragma unroll
+        for (int p = 0; p < PF; ++p) {
+            const int64_t t0 = cur[p], tn0 = wk.at<PATTERN>(u0 + p + PF, w, lane);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                stnt(o + t0 + r * wk.L, x[p][r] ^ y[p][r] ^ z[p][r]);
+                const int64_t tn = tn0 + r * wk.L;
+                x[p][r] = ldnt(a + tn); y[p][r] = ldnt(b + tn); z[p][r] = ldnt(c + tn);
+            }
+            cur[p] = tn0;
+            __syncthreads();
+        }
+    }
+    for (; u0 < wk.nunits; u0 += PF) {
 #pragma unroll
         for (int p = 0; p < PF; ++p) {
             const int64_t u = u0 + p;
@@ -79,7 +99,21 @@ __global__ __launch_bounds__(256) void row_probe_kernel(const bf16_t* a, const b
 #pragma unroll
         for (int j = 0; j < K; ++j)
             if (p < nsteps) { const int64_t t = base + p * step + j * 512; x[p][j] = ldnt(a + t); y[p][j] = ldnt(b + t); z[p][j] = ldnt(c + t); }
-    for (int64_t u0 = 0; u0 < nsteps; u0 += PF) {
+    int64_t u0 = 0;
+    __builtin_amdgcn_s_waitcnt(0x0F70);                            // vmcnt(0); whole rotations as in stream_probe_kernel
+    for (; u0 + 2 * PF <= nsteps; u0 += PF) {
+#pragma unroll
+        for (int p = 0; p < PF; ++p) {
+#pragma unroll
+            for (int j = 0; j < K; ++j) {
+                const int64_t t = base + (u0 + p) * step + j * 512, tn = t + PF * step;
+                stnt(o + t, x[p][j] ^ y[p][j] ^ z[p][j]);
+                x[p][j] = ldnt(a + tn); y[p][j] = ldnt(b + tn); z[p][j] = ldnt(c + tn);
+            }
+            __syncthreads();
+        }
+    }
+    for (; u0 < nsteps; u0 += PF) {
 #pragma unroll
         for (int p = 0; p < PF; ++p) {
             const int64_t u = u0 + p;
