@@ -505,7 +505,14 @@ def main():
         for what, rr in (("inputs from HBM", [ops.rows_of(t) for t in (full[1], full[0], full[2])]), ("inputs cached", rows)):
             _, ms = time_steps(lambda: ops.li_fwd_rows(rr[0], rr[1], rr[2], plan, Db, B, D, L, device=device, out=out), 10, 3)
             print(f"hyena_li_fwd config 3, {what}: {ms * 1e3:.1f} us", file=sys.stderr)
-        del small, full, out
+        # the same rows with x1 holding x1*v already (two input streams, what hyena_featurizer_gates_fwd hands over) and
+        # ungated (one input stream)
+        x1v = full[1] * full[2]
+        rx, r2 = ops.rows_of(x1v), ops.rows_of(full[0])
+        for what, a2 in (("x1*v rows and x2 (6 bytes per sample)", r2), ("ungated, one input stream (4 bytes per sample)", None)):
+            _, ms = time_steps(lambda: ops.li_fwd_rows(rx, a2, None, plan, Db, B, D, L, device=device, out=out), 10, 3)
+            print(f"hyena_li_fwd config 3, {what}: {ms * 1e3:.1f} us", file=sys.stderr)
+        del small, full, out, x1v
         torch.cuda.empty_cache()
 
     main_name = args.workload if args.workload != "decode" else "mr"
