@@ -618,18 +618,24 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     // Every guarded rotation, and the prologue, ends with a wait for all outstanding requests, so that the whole
     // rotations start from a known state; they are the first and the last two of a row.
     // The bounds are the block's (Lv, not Lw): with COOP every wavefront runs every step and meets every barrier.
+    // The one-channel form with all three gate streams keeps guarded steps throughout: it runs at the ceiling of its
+    // access order either way, and three register stages under guarded steps measured 2 % faster there (1.628 against
+    // 1.659 ms at L = 262144) than the two stages that fit whole-piece steps.
+    constexpr bool WHOLE_ROTATIONS = !(CPW == 1 && PRE && POST);
     constexpr int VMCNT0 = 0x0F70;                             // s_waitcnt vmcnt(0), other counters unconstrained
     const int64_t whole_until = Lv - (COOP ? 3 * TLW : 0) - TLW - (int64_t)(2 * PF - 1) * STEP;
-    __builtin_amdgcn_s_waitcnt(VMCNT0);
+    if (WHOLE_ROTATIONS) __builtin_amdgcn_s_waitcnt(VMCNT0);
     for (int64_t ts = 0; ts < Lv; ts += (int64_t)PF * STEP) {
-        if (ts > 0 && ts <= whole_until) {
+        if (WHOLE_ROTATIONS && ts > 0 && ts <= whole_until) {
+            if constexpr (WHOLE_ROTATIONS) {
 #pragma unroll
-            for (int p = 0; p < PF; ++p) step(whole, p, ts + (int64_t)p * STEP);
+                for (int p = 0; p < PF; ++p) step(whole, p, ts + (int64_t)p * STEP);
+            }
         } else {
 #pragma unroll
             for (int p = 0; p < PF; ++p)
                 if (ts + (int64_t)p * STEP < Lv) step(guarded, p, ts + (int64_t)p * STEP);
-            __builtin_amdgcn_s_waitcnt(VMCNT0);
+            if (WHOLE_ROTATIONS) __builtin_amdgcn_s_waitcnt(VMCNT0);
         }
     }
     {   // output of the last step
@@ -814,14 +820,14 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
     const bool y32 = y_conv_fp32 != nullptr;
     if (y32) nt = false;
 // prefetch depth in steps: two with four channels per wavefront (measured 1-3 % faster than three, which in turn
-// beats four, whose registers spill).  One channel per wavefront: two for the gated forms (three stages of three or two
-// input streams leave the whole-piece steps short of registers: 75-110 spilled dwords and 1.63 against 1.52 ms on
-// x1*v rows at L = 262144), three for the ungated one (1.28 against 1.36 ms)
+// beats four, whose registers spill).  One channel per wavefront: three, except on x1*v rows (three stages of two
+// input streams leave the whole-piece steps short of registers: 110 spilled dwords and 1.63 against 1.52 ms at
+// L = 262144); the three-gate form runs its three stages under guarded steps (see the step loop)
 #define LI_LAUNCH(P, Q, N, M, Y)                                                                           \
     do {                                                                                                   \
         if (cpw == 4 && coop) hipLaunchKernelGGL((li_kernel<P, Q, N, 2, M, Y, 4, true>), grid, dim3(256), 0, s, a);   \
         else if (cpw == 4) hipLaunchKernelGGL((li_kernel<P, Q, N, 2, M, Y, 4, false>), grid, dim3(256), 0, s, a);     \
-        else hipLaunchKernelGGL((li_kernel<P, Q, N, (P || Q) ? 2 : 3, M, Y, 1, false>), grid, dim3(256), 0, s, a);    \
+        else hipLaunchKernelGGL((li_kernel<P, Q, N, (P != Q) ? 2 : 3, M, Y, 1, false>), grid, dim3(256), 0, s, a);    \
     } while (0)
 #define LI_M(P, Q, N, Y) do { if (dmode == 1) LI_LAUNCH(P, Q, N, 1, Y); else if (dmode == 2) LI_LAUNCH(P, Q, N, 2, Y); else LI_LAUNCH(P, Q, N, 0, Y); } while (0)
 #define LI_N(P, Q) do { if (y32) LI_M(P, Q, false, true); else if (nt) LI_M(P, Q, true, false); else LI_M(P, Q, false, false); } while (0)
