@@ -226,6 +226,11 @@ def test_layer_projection_beyond_32_bit_offsets():
     zs = torch.stack([z[0, i * D + d, L - 4096:] for d in ds.tolist() for i in range(3)]).cpu()
     zr, _ = O.parallel_fir(us, wf.cpu()[ch][:, None, :], None, fir_length=Ks, dim_last=True, gate=False)
     assert rel_err(zs, zr[0][:, 256:]) <= 1e-2
+    # and the gate-fused featurizer at the far end of the same projection: bit for bit what the three gate rows give
+    xv, g2 = ops.featurizer_gates_fwd(u, wf.t().contiguous(), None, cmap)
+    for d in ds.tolist():
+        assert torch.equal(xv[0, d, L - 4096:], z[0, D + d, L - 4096:] * z[0, 2 * D + d, L - 4096:])
+        assert torch.equal(g2[0, d, L - 4096:], z[0, d, L - 4096:])
 
 
 @pytest.mark.parametrize("K", [7, 128])

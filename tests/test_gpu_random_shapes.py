@@ -168,6 +168,43 @@ def test_fused_layer_random(B, L, seed, override):
         assert rel_err(bx.permute(0, 2, 1), (x1 * v)[..., L - (K - 1):]) <= 1e-2
 
 
+@pytest.mark.parametrize("B,L,seed", cl_cases(9, 14))
+def test_featurizer_gates_random(B, L, seed, override):
+    # the gate-fused featurizer (rows xv = x1*v and x2 for Hyena-LI): any L behind its front padding, channel counts
+    # that leave partial 64-channel blocks, both featurizer lengths, every layout with 16-byte pieces, forced numbers
+    # of tiles per block; then the modal scan on those rows against the oracle's Hyena-LI on the oracle's gates
+    rng = random.Random(seed)
+    Ks = rng.choice([3, 4])
+    H = rng.choice([1, 2, 3])
+    hd = 8 * rng.randint(1, 5)
+    D = H * hd
+    cs, il = rng.choice([(False, False), (True, False), (False, True)])
+    flip, sbias = rng.random() < 0.5, rng.random() < 0.5
+    override(cl_nseg=rng.randint(1, 4))
+    g = torch.Generator().manual_seed(seed)
+    C = 3 * D
+    u = torch.randn(B, L, C, generator=g).bfloat16()
+    wf = torch.randn(C, 1, Ks, generator=g) / Ks ** 0.5
+    bf = torch.randn(C, generator=g).bfloat16() if sbias else None
+    z, _ = O.parallel_fir(u, wf, bf, fir_length=Ks, dim_last=True, gate=False)
+    if il:
+        z = O.interleave(z)
+    x2, x1, v = O.split_gates(z, (D, H, hd), cs, flip)
+    pad = (-L) % 8
+    cmap = ops.gate_channel_map(D, interleave=il, head_dim=hd if cs else None)
+    xv, g2 = ops.featurizer_gates_fwd(u.cuda(), wf.reshape(C, Ks).t().contiguous().cuda(),
+                                      None if bf is None else bf.cuda(), cmap, flip_x1x2=flip, front_pad=pad)
+    what = (B, D, L, Ks, cs, il, flip, sbias)
+    assert not xv[..., :pad].any() and not g2[..., :pad].any(), what
+    assert rel_err(xv[..., pad:], x1 * v) <= 1e-2 and rel_err(g2[..., pad:], x2) <= 1e-2, what
+    lp, r = O.make_modal_real(D, 16, seed=seed)
+    Dc = torch.randn(D, generator=g).bfloat16()
+    ref, _, _ = O.li_prefill(x2, x1, v, lp, r, Dc, want_state=False)
+    plan = ops.ModalPlan(lp.cuda(), r.cuda())
+    y, _, _ = ops.li_fwd_rows(ops.rows_of(xv), ops.rows_of(g2), None, plan, Dc.cuda(), B, D, L + pad, device="cuda")
+    assert rel_err(y[..., pad:], ref) <= 2e-2, what
+
+
 @pytest.mark.parametrize("L", [1, 5, 63, 1001, 2049])
 def test_lengths_that_are_not_multiples_of_8(L):
     # the tensor-level operators accept any length: they run behind -L % 8 zero samples (ops.front_pad8)
