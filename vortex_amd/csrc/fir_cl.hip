@@ -261,7 +261,8 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     // Pieces of the next step requested before the MFMA phase (the rest after it).  Without the featurizer all
     // of them travel during the MFMA phase.  With it a lane holds 18 row pieces, which next to all ten A fragments
     // do not fit the register budget of two blocks per CU: one piece goes out early (measured 4 % faster for the
-    // medium filter than none, two spill), none for the short-filter form.
+    // medium filter than none; two fit since the output addresses stopped taking registers but measured 7 % slower),
+    // none for the short-filter form (one measured the same).
     constexpr int NEARLY = FEAT ? (MLO == 0 ? 1 : 0) : NP;
     load_step(ts0);
 
@@ -370,6 +371,13 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             u32x2 zc[8];
 #pragma unroll
             for (int c = 0; c < 8; ++c) zc[c] = *(const u32x2*)(z_lds + (8 * cb + c) * ZRS + ((4 * rb) ^ swz_io));
+            // the step's first output row as a block-uniform address, the lane's row and channels as a 32-bit byte offset
+            // (the launcher bounds 128 rows of D channels to 2^32 bytes): no 64-bit address per lane and row
+            bf16_t* const out_step = out + (b * L + ts) * D;
+            bf16_t* const y2_step = (AUX && !FEAT && y2_out) ? y2_out + (b * L + ts) * D : nullptr;
+            uint32_t lane_row_b = ((uint32_t)(4 * rb) * (uint32_t)D + dch) * 2u;
+            const uint32_t row_b = (uint32_t)D * 2u;
+            asm volatile("" : "+v"(lane_row_b));      // keeps the compiler from folding it into four per-lane row pointers held (and spilled) across the loop
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int64_t t = ts + 4 * rb + q;
@@ -379,15 +387,16 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                     zz[j] = (q & 1) ? pair_hi(zc[2 * j][q >> 1], zc[2 * j + 1][q >> 1])
                                     : pair_lo(zc[2 * j][q >> 1], zc[2 * j + 1][q >> 1]);
                 if (t < t_end) {
-                    if (AUX && !FEAT && y2_out) *(u32x4*)(y2_out + (b * L + t) * D + dch) = zz;
+                    if (AUX && !FEAT && y2_out) *(u32x4*)((char*)y2_step + (lane_row_b + q * row_b)) = zz;
                     u32x4 o = zz;
                     if (POST) {
 #pragma unroll
                         for (int j = 0; j < 4; ++j)
                             o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(g2[q][j]), bf_hi(zz[j]) * bf_hi(g2[q][j]));
                     }
-                    if (NT) __builtin_nontemporal_store(o, (u32x4*)(out + (b * L + t) * D + dch));
-                    else *(u32x4*)(out + (b * L + t) * D + dch) = o;
+                    u32x4* const dst = (u32x4*)((char*)out_step + (lane_row_b + q * row_b));
+                    if (NT) __builtin_nontemporal_store(o, dst);
+                    else *dst = o;
                 }
             }
         }
@@ -544,7 +553,7 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
                          void* out, void* y2_out, void* bx_out, int64_t bx_from, int64_t B, int64_t L, int64_t D,
                          int64_t G, int K, void* stream, const char* who) {
     if (!h || !out) return hyena_fail(HYENA_EINVAL, "%s: h and out are required", who);
-    if (B < 0 || D <= 0 || L < 0 || G <= 0 || D % G != 0 || D >= (1LL << 30))
+    if (B < 0 || D <= 0 || L < 0 || G <= 0 || D % G != 0 || D >= (1LL << 24))
         return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld L=%lld G=%lld", who, (long long)B, (long long)D,
                           (long long)L, (long long)G);
     if (K < 1 || K > 128) return hyena_fail(HYENA_ENOSUP, "%s: K=%d outside 1..128", who, K);
