@@ -786,11 +786,15 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
     //  * shorter rows: four channels of one filter per wavefront, 512 samples per step (a quarter of the scan
     //    links and fragment builds) - as lone wavefronts when there are enough of them to fill the chip, in the
     //    cooperative form (one block per four channels, four times as many blocks) when there are not.
+    //  * long rows with all three gate streams and four channels per filter: the cooperative form again (its four
+    //    wavefronts read consecutive pieces of the same four rows; 2-4 % faster than one channel per wavefront from
+    //    65536 samples on, e.g. 1.61 against 1.64-1.65 ms at L = 262144; on x1*v rows it is 1-4 % slower).
     const bool can4 = (D / G) % 4 == 0;
-    int cpw = (can4 && L < 65536) ? 4 : 1;                   // channels per wavefront (they share one filter)
+    const bool long_coop = can4 && L >= 65536 && pre && post;
+    int cpw = (can4 && (L < 65536 || long_coop)) ? 4 : 1;    // channels per wavefront (they share one filter)
     { const int64_t x = hyena_override(HYENA_OV_LI_CPW); if (x == 1) cpw = 1; else if (x == 4 && can4) cpw = 4; }
     const int64_t nquads = B * (D / cpw);
-    bool coop = cpw == 4 && nquads <= 512;
+    bool coop = cpw == 4 && (nquads <= 512 || long_coop);
     { const int64_t x = hyena_override(HYENA_OV_LI_COOP); if (x >= 0) coop = cpw == 4 && x != 0; }
     const int64_t nblk = coop ? nquads : (nquads + 3) / 4;
     if (nquads > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: problem too large for one launch", who);
