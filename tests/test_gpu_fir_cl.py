@@ -317,10 +317,12 @@ def test_featurizer_gates_fwd_vs_oracle_and_unfused_path(B, L, D, H, Ks, cs, il,
     assert torch.equal(xv, k1 * kv) and torch.equal(g2, k2.contiguous())
 
 
-@pytest.mark.parametrize("cplx,G", [(True, 8), (False, 128)])
-def test_li_fwd_on_premultiplied_rows(cplx, G):
+@pytest.mark.parametrize("cplx,G,D,L", [(True, 8, 128, 4096), (False, 128, 128, 4096),
+                                        (True, 32, 32, 65536 + 520),      # one channel per wavefront, whole-piece steps
+                                        (False, 2, 32, 2048 * 9 + 8)])    # four channels per wavefront, long enough for them
+def test_li_fwd_on_premultiplied_rows(cplx, G, D, L):
     # hyena_li_fwd with v = NULL: x1 holds bf16(x1*v) already; same output and state as the three-gate call
-    B, D, L, S = 2, 128, 4096, 16
+    B, S = 2, 16
     g = torch.Generator().manual_seed(21)
     x1, x2, v = (torch.randn(B, D, L, generator=g).bfloat16().to(DEV) for _ in range(3))
     lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(G, S, seed=4)
