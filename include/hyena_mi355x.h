@@ -355,10 +355,12 @@ typedef struct hyena_proj_fwd {
  * u [B][L][3D] (vortex/model/engine.py:188-223), interleave / split (vortex/model/model.py:251-252,
  * engine.py:300-310) and x1v = x1*v (engine.py:312), written as the two row tensors hyena_li_fwd reads:
  *   xv_out [B][D][L + front_pad] = bf16(x1*v),  x2_out [B][D][L + front_pad] = x2   (bf16; the first front_pad
- * columns are zero: front_pad = -L % 8 makes any L usable).  The three gate tensors [B][3D][L] of
+ * columns are zero: front_pad = -L % 8 makes any L usable).  Rows are out_row_stride elements apart (a multiple of 8,
+ * at least L + front_pad; the columns beyond are not written): rows a power of two apart stream more slowly in the
+ * scan that follows, a stride a few KB off one avoids that.  The three gate tensors [B][3D][L] of
  * hyena_featurizer_fwd are never written: 10 instead of 12 bytes per (channel, sample) here and 6 instead of 8 in
  * hyena_li_fwd (v = NULL).  Channel maps and Ks as hyena_fir_layer_fwd; others return HYENA_ENOSUP. */
-int hyena_featurizer_gates_fwd(const hyena_proj_fwd* proj, void* xv_out, void* x2_out,
+int hyena_featurizer_gates_fwd(const hyena_proj_fwd* proj, void* xv_out, void* x2_out, int64_t out_row_stride,
                                int64_t B, int64_t L, int64_t D, int front_pad, void* stream);
 
 /* A whole Hyena-SE / Hyena-MR layer at prefill in one launch: featurizer FIR, split, x1*v gate, inner FIR,

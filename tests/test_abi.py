@@ -89,15 +89,17 @@ def test_new_entry_points_validate_before_touching_the_device():
     assert L.hyena_fir_layer_step_far(None, P, 127, 512, 0, None, P, 0, P, None, 0, P, 512, 1, 512, 32, None) == -1
     # gate-fused featurizer: descriptor checks as in the layer call, both outputs, column count a multiple of 8
     pj = _lib.ProjFwd(P, 192, 192, P, None, 3, 0, 64, 0, 64, 1)
-    assert L.hyena_featurizer_gates_fwd(None, P, P, 1, 8, 64, 0, None) == -1
-    assert L.hyena_featurizer_gates_fwd(ref(pj), P, None, 1, 8, 64, 0, None) == -1
-    assert L.hyena_featurizer_gates_fwd(ref(pj), P, P, 1, 5, 64, 0, None) == -2        # 5 columns
-    assert L.hyena_featurizer_gates_fwd(ref(pj), P, P, 1, 5, 64, 8, None) == -1        # front_pad above 7
-    assert L.hyena_featurizer_gates_fwd(ref(pj), P, P, 0, 5, 64, 3, None) == 0         # B = 0: no launch
+    assert L.hyena_featurizer_gates_fwd(None, P, P, 8, 1, 8, 64, 0, None) == -1
+    assert L.hyena_featurizer_gates_fwd(ref(pj), P, None, 8, 1, 8, 64, 0, None) == -1
+    assert L.hyena_featurizer_gates_fwd(ref(pj), P, P, 8, 1, 5, 64, 0, None) == -2     # 5 columns
+    assert L.hyena_featurizer_gates_fwd(ref(pj), P, P, 16, 1, 5, 64, 8, None) == -1    # front_pad above 7
+    assert L.hyena_featurizer_gates_fwd(ref(pj), P, P, 8, 0, 5, 64, 3, None) == 0      # B = 0: no launch
+    assert L.hyena_featurizer_gates_fwd(ref(pj), P, P, 8, 1, 16, 64, 0, None) == -1    # rows 8 apart for 16 columns
+    assert L.hyena_featurizer_gates_fwd(ref(pj), P, P, 20, 1, 16, 64, 0, None) == -2   # row stride not a multiple of 8
     pj5 = _lib.ProjFwd(P, 192, 192, P, None, 5, 0, 64, 0, 64, 1)
-    assert L.hyena_featurizer_gates_fwd(ref(pj5), P, P, 1, 8, 64, 0, None) == -3       # 5-tap featurizer
+    assert L.hyena_featurizer_gates_fwd(ref(pj5), P, P, 8, 1, 8, 64, 0, None) == -3    # 5-tap featurizer
     pjs = _lib.ProjFwd(P, 192, 192, P, None, 3, 0, 4, 12, 4, 1)
-    assert L.hyena_featurizer_gates_fwd(ref(pjs), P, P, 1, 8, 64, 0, None) == -3       # heads of 4 channels: no 16-byte pieces
+    assert L.hyena_featurizer_gates_fwd(ref(pjs), P, P, 8, 1, 8, 64, 0, None) == -3    # heads of 4 channels: no 16-byte pieces
     # windowed modal step: 16 states and B*D of 65536 and more, all three window buffers, the counter inside the window
     W = L.hyena_iir_window_tokens()
     assert W >= 2 and L.hyena_iir_window_supported(64, 4096, 16, 0) == 1 and L.hyena_iir_window_supported(64, 4096, 16, 1) == 1

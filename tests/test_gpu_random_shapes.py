@@ -192,9 +192,12 @@ def test_featurizer_gates_random(B, L, seed, override):
     x2, x1, v = O.split_gates(z, (D, H, hd), cs, flip)
     pad = (-L) % 8
     cmap = ops.gate_channel_map(D, interleave=il, head_dim=hd if cs else None)
+    row_pad = rng.choice([0, 0, 8, 2048])                 # rows of the results further apart than their length
     xv, g2 = ops.featurizer_gates_fwd(u.cuda(), wf.reshape(C, Ks).t().contiguous().cuda(),
-                                      None if bf is None else bf.cuda(), cmap, flip_x1x2=flip, front_pad=pad)
-    what = (B, D, L, Ks, cs, il, flip, sbias)
+                                      None if bf is None else bf.cuda(), cmap, flip_x1x2=flip, front_pad=pad,
+                                      row_pad=row_pad)
+    assert xv.stride(1) == L + pad + row_pad
+    what = (B, D, L, Ks, cs, il, flip, sbias, row_pad)
     assert not xv[..., :pad].any() and not g2[..., :pad].any(), what
     assert rel_err(xv[..., pad:], x1 * v) <= 1e-2 and rel_err(g2[..., pad:], x2) <= 1e-2, what
     lp, r = O.make_modal_real(D, 16, seed=seed)

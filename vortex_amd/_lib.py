@@ -116,7 +116,7 @@ def lib():
     C = POINTER(Cl)
     L.hyena_fir_cl_fwd.argtypes = [C, C, C, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64,
                                    c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]
-    L.hyena_featurizer_gates_fwd.argtypes = [POINTER(ProjFwd), c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]
+    L.hyena_featurizer_gates_fwd.argtypes = [POINTER(ProjFwd), c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]
     L.hyena_fir_layer_fwd.argtypes = [POINTER(ProjFwd), c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int64,
                                       c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]
     for name in EXPORTS:

@@ -437,7 +437,8 @@ constexpr int GRS = 264;       // row stride (elements) of the transposed tiles:
 template <int FEAT, int KS>
 __global__ __launch_bounds__(256, 2) void proj_gates_kernel(ProjFwd pj, bf16_t* __restrict__ xv_out,
                                                             bf16_t* __restrict__ x2_out, int64_t L, int64_t Lout,
-                                                            int pad, int64_t D, int ndb, int nchunk, int ntpb) {
+                                                            int64_t out_rs, int pad, int64_t D, int ndb, int nchunk,
+                                                            int ntpb) {
     constexpr int RF = KS - 1, NR = 4 + RF;
     __shared__ __attribute__((aligned(16))) bf16_t xv_t[CB * GRS];
     __shared__ __attribute__((aligned(16))) bf16_t x2_t[CB * GRS];
@@ -535,7 +536,7 @@ __global__ __launch_bounds__(256, 2) void proj_gates_kernel(ProjFwd pj, bf16_t* 
                 if (d0 + ch >= (uint32_t)D) continue;
                 const bf16_t* tile = rr < CB ? xv_t : x2_t;
                 const u32x4 o = *(const u32x4*)(tile + ch * GRS + (tcol & TL) + ((tcol & (TL - 1)) ^ (32 * (ch >> 4))));
-                *(u32x4*)((rr < CB ? xv_out : x2_out) + (b * D + d0 + ch) * Lout + col) = o;
+                *(u32x4*)((rr < CB ? xv_out : x2_out) + (b * D + d0 + ch) * out_rs + col) = o;
             }
         }
         if (next) __syncthreads();                         // the tiles are free again
@@ -700,8 +701,8 @@ extern "C" int hyena_fir_layer_fwd(const hyena_proj_fwd* proj, const float* h, i
     return fir_cl_launch(a, h, taps_reversed, bias, bias_mode, out, nullptr, bx_out, bx_from, B, L, D, G, K, stream, who);
 }
 
-extern "C" int hyena_featurizer_gates_fwd(const hyena_proj_fwd* proj, void* xv_out, void* x2_out, int64_t B, int64_t L,
-                                          int64_t D, int front_pad, void* stream) {
+extern "C" int hyena_featurizer_gates_fwd(const hyena_proj_fwd* proj, void* xv_out, void* x2_out, int64_t out_row_stride,
+                                          int64_t B, int64_t L, int64_t D, int front_pad, void* stream) {
     const char* who = "hyena_featurizer_gates_fwd";
     if (!xv_out || !x2_out) return hyena_fail(HYENA_EINVAL, "%s: both outputs are required", who);
     if (B < 0 || L < 0 || D >= (1LL << 30)) return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld L=%lld D=%lld", who,
@@ -710,8 +711,10 @@ extern "C" int hyena_featurizer_gates_fwd(const hyena_proj_fwd* proj, void* xv_o
     LaunchArgs a = {};
     if (int rc = make_proj_fwd(proj, D, who, a)) return rc;
     const int64_t Lout = L > 0 ? L + front_pad : 0;
-    if (Lout % 8 != 0 || (((uintptr_t)xv_out | (uintptr_t)x2_out) & 15))
-        return hyena_fail(HYENA_EALIGN, "%s: L + front_pad must be a multiple of 8, outputs 16-byte aligned", who);
+    if (Lout % 8 != 0 || out_row_stride % 8 != 0 || (((uintptr_t)xv_out | (uintptr_t)x2_out) & 15))
+        return hyena_fail(HYENA_EALIGN, "%s: L + front_pad and out_row_stride must be multiples of 8, outputs 16-byte aligned", who);
+    if (out_row_stride < Lout) return hyena_fail(HYENA_EINVAL, "%s: out_row_stride %lld below the %lld columns of a row", who,
+                                                 (long long)out_row_stride, (long long)Lout);
     if (B == 0 || L == 0) return 0;
     const int64_t ndb = (D + CB - 1) / CB, ntt = (Lout + GT - 1) / GT;
     // consecutive tiles per block (the tap table is staged once, the next tile's rows travel during the stores): as
@@ -725,7 +728,7 @@ extern "C" int hyena_featurizer_gates_fwd(const hyena_proj_fwd* proj, void* xv_o
     hipStream_t s = (hipStream_t)stream;
 #define PG_GO(F, KSV)                                                                                              \
     hipLaunchKernelGGL((proj_gates_kernel<F, KSV>), grid, dim3(256), 0, s, a.pj, (bf16_t*)xv_out, (bf16_t*)x2_out, L, \
-                       Lout, front_pad, D, (int)ndb, (int)nchunk, (int)ntpb)
+                       Lout, out_row_stride, front_pad, D, (int)ndb, (int)nchunk, (int)ntpb)
     if (a.feat == 3 && a.ks == 3) PG_GO(3, 3);
     else if (a.feat == 3) PG_GO(3, 4);
     else if (a.ks == 3) PG_GO(1, 3);

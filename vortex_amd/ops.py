@@ -199,10 +199,12 @@ def fir_layer_fwd(u, feat_w, feat_bias, channel_map, taps, *, bias=None, bias_mo
     return out if bx_from is None else (out, bx)
 
 
-def featurizer_gates_fwd(u, feat_w, feat_bias, channel_map, *, flip_x1x2=False, front_pad=0):
+def featurizer_gates_fwd(u, feat_w, feat_bias, channel_map, *, flip_x1x2=False, front_pad=0, row_pad=0):
     """Featurizer, split and x1*v of a Hyena-LI layer in one launch: u [B, L, 3D] bf16 -> (xv, x2), each
     [B, D, L + front_pad] bf16 with xv = bf16(x1*v): the rows li_fwd_rows reads as (x1r=rows_of(xv), x2r=rows_of(x2),
-    vr=None).  feat_w [Ks, 3D] float32 tap-major, feat_bias [3D] or None, channel_map from gate_channel_map()."""
+    vr=None).  feat_w [Ks, 3D] float32 tap-major, feat_bias [3D] or None, channel_map from gate_channel_map().
+    row_pad (a multiple of 8): the rows of the two results are L + front_pad + row_pad elements apart (views of wider
+    buffers), e.g. to keep long rows from lying a power of two apart."""
     _need_cuda(u, feat_w)
     if u.dtype != torch.bfloat16 or u.dim() != 3 or u.stride(2) != 1:
         raise ValueError("expected a [B, L, 3D] bfloat16 projection with contiguous channels")
@@ -213,13 +215,14 @@ def featurizer_gates_fwd(u, feat_w, feat_bias, channel_map, *, flip_x1x2=False, 
         raise ValueError("feat_w must be [Ks, 3D] (tap-major)")
     ci, co, gs, cs = channel_map
     Lout = L + front_pad if L else 0
-    xv = torch.empty((B, D, Lout), dtype=torch.bfloat16, device=u.device)
-    x2 = torch.empty((B, D, Lout), dtype=torch.bfloat16, device=u.device)
+    xv = torch.empty((B, D, Lout + row_pad), dtype=torch.bfloat16, device=u.device)[..., :Lout]
+    x2 = torch.empty((B, D, Lout + row_pad), dtype=torch.bfloat16, device=u.device)[..., :Lout]
     if xv.numel():
         pj = ProjFwd(u.data_ptr(), _strides(u)[0], _strides(u)[1], feat_w.data_ptr(),
                      feat_bias.data_ptr() if feat_bias is not None else None, feat_w.shape[0], int(flip_x1x2),
                      ci, co, gs, cs)
-        rc = _lib.lib().hyena_featurizer_gates_fwd(ctypes.byref(pj), _ptr(xv), _ptr(x2), B, L, D, front_pad, _stream())
+        rc = _lib.lib().hyena_featurizer_gates_fwd(ctypes.byref(pj), _ptr(xv), _ptr(x2), Lout + row_pad, B, L, D,
+                                                   front_pad, _stream())
         _lib.check(rc, "hyena_featurizer_gates_fwd")
     return xv, x2
 
