@@ -194,20 +194,31 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     const int swz_io = 32 * (cb >> 1), swz_mm = 32 * w;
     const uint32_t dch = d0 + 8 * cb;
     const bool ch_ok = dch < (uint32_t)D;
+    // Row pieces are addressed as a block-uniform base (tensor, batch element, piece; the time row is added per step)
+    // plus a 32-bit byte offset of the lane (its first row and channels): no 64-bit pointer per lane and piece.  The
+    // launcher bounds 128 rows of any operand to 2^32 bytes.
     const bf16_t* pp[NP];
+    uint32_t loff[NP];
     int64_t pts;
     if (FEAT == 3) {
 #pragma unroll
-        for (int i = 0; i < NP; ++i) pp[i] = pj.u + b * pj.bs + 3 * (int64_t)dch + 8 * i;
+        for (int i = 0; i < NP; ++i) {
+            pp[i] = pj.u + b * pj.bs + 8 * i;
+            loff[i] = ((uint32_t)(4 * rb) * (uint32_t)pj.ts + 3u * dch) * 2u;
+        }
         pts = pj.ts;
     } else if (FEAT == 1) {
 #pragma unroll
-        for (int i = 0; i < NP; ++i) pp[i] = pj.u + b * pj.bs + pj.chan(i, ch_ok ? dch : 0);
+        for (int i = 0; i < NP; ++i) {
+            pp[i] = pj.u + b * pj.bs + (int64_t)i * pj.gate_stride;
+            loff[i] = ((uint32_t)(4 * rb) * (uint32_t)pj.ts + pj.chan(0, ch_ok ? dch : 0)) * 2u;
+        }
         pts = pj.ts;
     } else {
-        pp[0] = x1.ptr + b * x1.bs + dch;
-        if (NP >= 2) pp[1] = v.ptr + b * v.bs + dch;
-        if (NP >= 3) pp[2] = x2.ptr + b * x2.bs + dch;
+        pp[0] = x1.ptr + b * x1.bs;
+        loff[0] = ((uint32_t)(4 * rb) * (uint32_t)x1.ts + dch) * 2u;
+        if (NP >= 2) { pp[1] = v.ptr + b * v.bs; loff[1] = ((uint32_t)(4 * rb) * (uint32_t)v.ts + dch) * 2u; }
+        if (NP >= 3) { pp[2] = x2.ptr + b * x2.bs; loff[2] = ((uint32_t)(4 * rb) * (uint32_t)x2.ts + dch) * 2u; }
         pts = 0;
     }
     const int64_t pstr[3] = {FEAT ? pts : x1.ts, FEAT ? pts : v.ts, FEAT ? pts : x2.ts};
@@ -248,13 +259,22 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     u32x4 raw[NP][NR];
     const u32x4 zero4 = {0, 0, 0, 0};
     auto load_pieces = [&](int64_t ts, int i0, int i1) {
+        uint32_t lo[NP];                          // (with the featurizer the pieces share one offset)
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            if (FEAT && i > 0) { lo[i] = lo[0]; continue; }
+            lo[i] = loff[i];
+            asm volatile("" : "+v"(lo[i]));       // keeps the compiler from folding it into per-lane row pointers held across the loop
+        }
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
             const int64_t t = ts + 4 * rb + r - RF;
             const bool ok = ch_ok && t >= t_lo && t >= 0 && t < t_end;
 #pragma unroll
-            for (int i = 0; i < NP; ++i) if (i >= i0 && i < i1) raw[i][r] = ok ? ((NT && !FEAT) ? __builtin_nontemporal_load((const u32x4*)(pp[i] + t * pstr[i]))
-                                                                 : *(const u32x4*)(pp[i] + t * pstr[i])) : zero4;
+            for (int i = 0; i < NP; ++i) if (i >= i0 && i < i1) {
+                const u32x4* src = (const u32x4*)((const char*)(pp[i] + (ts + r - RF) * pstr[i]) + lo[i]);
+                raw[i][r] = ok ? ((NT && !FEAT) ? __builtin_nontemporal_load(src) : *src) : zero4;
+            }
         }
     };
     auto load_step = [&](int64_t ts) { load_pieces(ts, 0, NP); };
@@ -650,6 +670,8 @@ static int make_proj_fwd(const hyena_proj_fwd* proj, int64_t D, const char* who,
         return hyena_fail(HYENA_EALIGN, "%s: D and strides must be multiples of 8, u 16-byte aligned", who);
     if (proj->ch_inner <= 0 || proj->ch_outer < 0 || proj->gate_stride <= 0)
         return hyena_fail(HYENA_EINVAL, "%s: bad featurizer channel map", who);
+    if (proj->u_time_stride < 0 || proj->u_time_stride >= (1LL << 24) || D >= (1LL << 24))
+        return hyena_fail(HYENA_EINVAL, "%s: u_time_stride and D must lie below 2^24 (32-bit byte offsets inside a step)", who);
     a.pj.u = (const bf16_t*)proj->u; a.pj.bs = proj->u_batch_stride; a.pj.ts = proj->u_time_stride;
     a.pj.w = proj->w; a.pj.bias = proj->bias;
     a.pj.ch_inner = (uint32_t)(proj->ch_inner > D ? D : proj->ch_inner); a.pj.ch_outer = (uint32_t)proj->ch_outer;
@@ -668,6 +690,8 @@ static int make_proj_fwd(const hyena_proj_fwd* proj, int64_t D, const char* who,
 static bool cl_ok(const hyena_cl* c) {
     return c && c->ptr && !((uintptr_t)c->ptr & 15) && c->batch_stride % 8 == 0 && c->time_stride % 8 == 0;
 }
+// the kernels address a lane's rows with 32-bit byte offsets inside a 128-row step
+static bool cl_stride_ok(const hyena_cl* c) { return c->time_stride >= 0 && c->time_stride < (1LL << 24); }
 
 }  // namespace
 
@@ -681,6 +705,8 @@ extern "C" int hyena_fir_cl_fwd(const hyena_cl* x1, const hyena_cl* x2, const hy
     if (pre != post) return hyena_fail(HYENA_ENOSUP, "%s: pass both gates v and x2, or neither", who);
     if (!cl_ok(x1) || (pre && (!cl_ok(v) || !cl_ok(x2))) || D % 8 != 0)
         return hyena_fail(HYENA_EALIGN, "%s: D and strides must be multiples of 8, pointers 16-byte aligned", who);
+    if (!cl_stride_ok(x1) || (pre && (!cl_stride_ok(v) || !cl_stride_ok(x2))))
+        return hyena_fail(HYENA_EINVAL, "%s: time strides must lie in 0 .. 2^24 - 1 elements", who);
     LaunchArgs a = {};
     a.x1 = {(const bf16_t*)x1->ptr, x1->batch_stride, x1->time_stride};
     if (pre) {
