@@ -336,13 +336,13 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
         }
         __syncthreads();
 
+        // ---- MFMA phase: this wavefront's 16 channels x 128 samples
+        const int c = n & 15, s = n >> 4;
+        f32x16 acc0, acc1;
+        const bf16_t* urow = u_lds + (16 * w + c) * URS;
         if (compute && slab_live) {
-            // ---- MFMA phase: this wavefront's 16 channels x 128 samples
-            const int c = n & 15, s = n >> 4;
-            f32x16 acc0, acc1;
 #pragma unroll
             for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
-            const bf16_t* urow = u_lds + (16 * w + c) * URS;
             const int c0 = 64 * s + 8 * hh + (cur ^ 1) * TL;     // ring position of the halo chunk's first sample
 #pragma unroll
             for (int mm = MLO; mm < 12; ++mm) {
@@ -351,6 +351,15 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                 if (mm - 2 >= MLO) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm - 2 >= MLO ? mm - 2 - MLO : 0], bf, acc1, 0, 0, 0);
                 if ((mm & 3) == 3) __builtin_amdgcn_sched_barrier(0);    // at most four B fragments in registers at a time
             }
+        }
+        // the rest of the next step's rows go out here, behind the MFMAs and ahead of the epilogue, the barrier and the
+        // output stage, which they overlap (the B fragments are dead by now)
+        if (NEARLY < NP) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (ts + TL < t_end) load_pieces(ts + TL, NEARLY, NP);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (compute && slab_live) {
 #pragma unroll
             for (int tau = 0; tau < 2; ++tau) {
                 const int tcol = 32 * tau + 64 * s + 16 * hh;
@@ -381,10 +390,6 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             }
         }
         __syncthreads();
-        if (NEARLY < NP) {
-            __builtin_amdgcn_sched_barrier(0);
-            if (ts + TL < t_end) load_pieces(ts + TL, NEARLY, NP);
-        }
 
         // ---- 8 x 4 transpose back, gate with x2, store rows
         if (compute && ch_ok) {
