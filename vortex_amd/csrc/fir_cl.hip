@@ -353,8 +353,10 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             }
         }
         // the rest of the next step's rows go out here, behind the MFMAs and ahead of the epilogue, the barrier and the
-        // output stage, which they overlap (the B fragments are dead by now)
-        if (NEARLY < NP) {
+        // output stage, which they overlap (the B fragments are dead by now); the short-filter form, with six MFMAs
+        // to hide behind, measured 1-2 % better with them behind the barrier
+        constexpr bool LATE_BEFORE_EPILOGUE = MLO == 0;
+        if (NEARLY < NP && LATE_BEFORE_EPILOGUE) {
             __builtin_amdgcn_sched_barrier(0);
             if (ts + TL < t_end) load_pieces(ts + TL, NEARLY, NP);
             __builtin_amdgcn_sched_barrier(0);
@@ -390,6 +392,10 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             }
         }
         __syncthreads();
+        if (NEARLY < NP && !LATE_BEFORE_EPILOGUE) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (ts + TL < t_end) load_pieces(ts + TL, NEARLY, NP);
+        }
 
         // ---- 8 x 4 transpose back, gate with x2, store rows
         if (compute && ch_ok) {
