@@ -239,7 +239,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
         po[r] = a.out + (b * a.D + d) * L + o;
     }
     const u32x4 zero4 = {0, 0, 0, 0};
-    u32x4 c1[PF][4], cv[PF][4], c2[PF][4];
+    u32x4 c1[PF][4], cv[PRE ? PF : 1][4], c2[POST ? PF : 1][4];      // register stages (absent gates take none)
     auto request_rows = [&]() {
 #pragma unroll
         for (int p = 0; p < PF; ++p)
@@ -249,8 +249,8 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                 const int64_t pos = t + roff(r) + lane * 8;
                 const bool ok = pos < Lw && pos >= lo;
                 c1[p][r] = ok ? ld16<NT>(lane_at(p1[r] + t)) : zero4;
-                cv[p][r] = (PRE && ok) ? ld16<NT>(lane_at(pv[r] + t)) : zero4;
-                c2[p][r] = (POST && ok) ? ld16<NT>(lane_at(p2[r] + t)) : zero4;
+                if constexpr (PRE) cv[p][r] = ok ? ld16<NT>(lane_at(pv[r] + t)) : zero4;
+                if constexpr (POST) c2[p][r] = ok ? ld16<NT>(lane_at(p2[r] + t)) : zero4;
             }
     };
     // With four channels per wavefront the rows are requested before the fragment build and travel during it
@@ -396,14 +396,17 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     // row: no branch surrounds a memory instruction there, which is what lets the compiler count exactly how many
     // younger requests may still be in flight when a register stage is consumed (with branches around them it has to
     // wait for everything outstanding, the prefetched stages included).
-    auto step = [&](auto guard_tag, const int p, const int64_t ts) {
+    auto step = [&](auto guard_tag, const int p, const int64_t ts) __attribute__((always_inline)) {
         constexpr bool GUARD = decltype(guard_tag)::value;
         const int pp = (p + PF - 1) % PF;                      // register stage of the previous step
         const int64_t tn = ts + (int64_t)PF * STEP;            // step that reuses this register stage
 
         // u = bf16(x1*v) of this step -> LDS; refill the stage with step ts + PF*TLW
 #pragma unroll
-        for (int r = 0; r < 4; ++r) *(u32x4*)(u_w + r * URS + lofs) = gate_mul<PRE>(c1[p][r], cv[p][r]);
+        for (int r = 0; r < 4; ++r) {
+            if constexpr (PRE) *(u32x4*)(u_w + r * URS + lofs) = gate_mul<true>(c1[p][r], cv[p][r]);
+            else *(u32x4*)(u_w + r * URS + lofs) = c1[p][r];
+        }
         // whole pieces inside the row (a wave-uniform test) are requested without per-lane predicates
         if (!GUARD || tn + TLW <= Lw) {
             // (without branches around them the scheduler would move these requests, and what waits on the registers
@@ -412,7 +415,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 c1[p][r] = ld16<NT>(lane_at(p1[r] + tn));
-                if (PRE) cv[p][r] = ld16<NT>(lane_at(pv[r] + tn));
+                if constexpr (PRE) cv[p][r] = ld16<NT>(lane_at(pv[r] + tn));
             }
             if (!GUARD) __builtin_amdgcn_sched_barrier(0);
         } else {
@@ -420,7 +423,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
             for (int r = 0; r < 4; ++r) {
                 const bool okn = tn + roff(r) + lane * 8 < Lw;
                 c1[p][r] = okn ? ld16<NT>(lane_at(p1[r] + tn)) : zero4;
-                cv[p][r] = (PRE && okn) ? ld16<NT>(lane_at(pv[r] + tn)) : zero4;
+                if constexpr (PRE) cv[p][r] = okn ? ld16<NT>(lane_at(pv[r] + tn)) : zero4;
             }
         }
         wave_sync();
@@ -471,7 +474,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 o[r] = zz[r];
-                if (POST) {
+                if constexpr (POST) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
                         o[r][j] = pack_bf2(bf_lo(zz[r][j]) * bf_lo(c2[pp][r][j]), bf_hi(zz[r][j]) * bf_hi(c2[pp][r][j]));
@@ -482,7 +485,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     st16<NT>(lane_to(po[r] + ts_out), o[r]);
-                    if (POST) c2[pp][r] = ld16<NT>(lane_at(p2[r] + t_refill));
+                    if constexpr (POST) c2[pp][r] = ld16<NT>(lane_at(p2[r] + t_refill));
                 }
                 if (!GUARD) __builtin_amdgcn_sched_barrier(0);
             } else {
@@ -492,7 +495,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                     const bool okc = ts_out >= 0 && pos < Lw && pos >= lo;
                     const bool okr = ts_out >= 0 && t_refill + roff(r) + lane * 8 < Lw;
                     if (okc) st16<NT>(lane_to(po[r] + ts_out), o[r]);
-                    if (ts_out >= 0) c2[pp][r] = (POST && okr) ? ld16<NT>(lane_at(p2[r] + t_refill)) : zero4;
+                    if constexpr (POST) { if (ts_out >= 0) c2[pp][r] = okr ? ld16<NT>(lane_at(p2[r] + t_refill)) : zero4; }
                 }
             }
         }
@@ -647,12 +650,12 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
             const int64_t pos = ts_last + roff(r) + lane * 8;
             const bool okc = pos < Lw && pos >= lo;
             const u32x4 zz = *(const u32x4*)(z_w + r * URS + lofs);
-            u32x4 x2v = c2[0][r];
-#pragma unroll
-            for (int p = 1; p < PF; ++p)
-                if (p == pl) x2v = c2[p][r];
             u32x4 o = zz;
-            if (POST) {
+            if constexpr (POST) {
+                u32x4 x2v = c2[0][r];
+#pragma unroll
+                for (int p = 1; p < PF; ++p)
+                    if (p == pl) x2v = c2[p][r];
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                     o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(x2v[j]), bf_hi(zz[j]) * bf_hi(x2v[j]));
@@ -786,11 +789,11 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
     //  * shorter rows: four channels of one filter per wavefront, 512 samples per step (a quarter of the scan
     //    links and fragment builds) - as lone wavefronts when there are enough of them to fill the chip, in the
     //    cooperative form (one block per four channels, four times as many blocks) when there are not.
-    //  * long rows with all three gate streams and four channels per filter: the cooperative form again (its four
-    //    wavefronts read consecutive pieces of the same four rows; 2-4 % faster than one channel per wavefront from
-    //    65536 samples on, e.g. 1.61 against 1.64-1.65 ms at L = 262144; on x1*v rows it is 1-4 % slower).
+    //  * long gated rows with four channels per filter: the cooperative form again (its four wavefronts read
+    //    consecutive pieces of the same four rows; 1-4 % faster than one channel per wavefront from 65536 samples
+    //    on, e.g. 1.61 against 1.64-1.65 ms with three gate streams and 1.25 against 1.29 ms on x1*v rows at L = 262144).
     const bool can4 = (D / G) % 4 == 0;
-    const bool long_coop = can4 && L >= 65536 && pre && post;
+    const bool long_coop = can4 && L >= 65536 && post;
     int cpw = (can4 && (L < 65536 || long_coop)) ? 4 : 1;    // channels per wavefront (they share one filter)
     { const int64_t x = hyena_override(HYENA_OV_LI_CPW); if (x == 1) cpw = 1; else if (x == 4 && can4) cpw = 4; }
     const int64_t nquads = B * (D / cpw);
