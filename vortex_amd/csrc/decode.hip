@@ -462,6 +462,23 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
         const uint32_t dc = ok ? dch : 0;
         const int64_t b = brow;
         if (b >= B) return;
+        // everything this token reads besides the gates is requested first, unconditionally (the slots of the window's
+        // inputs that are not in use yet are read as well and multiplied away): one round trip for the lot instead of
+        // one per term
+        const float far_j = (wa.far + (b * WIN + jw) * D)[dc];
+        const float dcoef = Dcoef[dc];
+        float gk[WIN], hk[WIN];
+        {
+            const float* gp = wa.g + (dc / (uint32_t)dg) * (uint32_t)WIN;
+#pragma unroll
+            for (int k = 0; k < WIN; ++k) gk[k] = gp[k];
+#pragma unroll
+            for (int k = 1; k < WIN; ++k) {
+                int sl = cnt - k;
+                if (sl < 0) sl += WIN;
+                hk[k] = bf_to_f((wa.hist + (b * WIN + sl) * D)[dc]);
+            }
+        }
         float a, c, gate2;
         if (VFEAT) {
             const int r = threadIdx.x;             // piece r covers zs columns 8r..8r+7 (96 pieces for 3 x 256 channels)
@@ -490,15 +507,11 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
         }
         if (!ok) return;
         const float x1v = round_bf(a * c);
-        const float* gp = wa.g + (dc / (uint32_t)dg) * (uint32_t)WIN;
-        float part = (wa.far + (b * WIN + jw) * D)[dc] + gp[0] * x1v;
+        float part = far_j + gk[0] * x1v;
 #pragma unroll
-        for (int k = 1; k < WIN; ++k) {
-            int sl = cnt - k;
-            if (sl < 0) sl += WIN;
-            if (k <= jw) part = fmaf(gp[k], bf_to_f((wa.hist + (b * WIN + sl) * D)[dc]), part);
-        }
-        float dx = Dcoef[dc] * x1v;
+        for (int k = 1; k < WIN; ++k)
+            if (k <= jw) part = fmaf(gk[k], hk[k], part);
+        float dx = dcoef * x1v;
         if (d_is_bf16) dx = round_bf(dx);
         const float y = gate2 * (part + dx);
         if (out_is_fp32) ((float*)out + b * out_bs)[dc] = y;
@@ -533,12 +546,32 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
             for (int k = 0; k < WIN; ++k) {
                 int sl = cnt - 1 - k;
                 if (sl < 0) sl += WIN;
-                pend[j][k] = k < npend ? bf_to_f((wa.hist + (bu(j) * WIN + sl) * D)[d]) : 0.f;
-            }
+                pend[j][k] = bf_to_f((wa.hist + (bu(j) * WIN + sl) * D)[d]);     // every slot is requested; the unused
+            }                                                                            // ones are dropped further down
     }
     const fvec pp = *(const fvec*)(poles + (g * (uint32_t)(S * FPS) + q * VEC));
     const fvec rr = *(const fvec*)(residues + (g * (uint32_t)(S * FPS) + q * VEC));
     const float dco = mode != 3 ? Dcoef[d] : 0.f;      // a flush has no token: no gates, no output, no Dcoef
+    // gates given as vectors, and the window's first filter sample, are requested here with everything above: one
+    // round trip for all of a token's operands instead of one per use
+    float ga[NB], gc[NB], gg[NB], g0 = 0.f;
+    if (FEAT == 0 && mode != 3) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const int64_t b = bu(j);
+            ga[j] = bf_to_f((x1 + b * in_bs)[d]);
+            gc[j] = bf_to_f((v + b * in_bs)[d]);
+            gg[j] = bf_to_f((x2 + b * in_bs)[d]);
+        }
+    }
+    if (WIN > 1 && mode == 1) g0 = wa.g[g * (uint32_t)WIN];
+    if (WIN > 1 && (mode == 1 || mode == 3)) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+            for (int k = 0; k < WIN; ++k)
+                if (k >= npend) pend[j][k] = 0.f;
+    }
     // fused featurizer: lanes 0..2 of the group evaluate gates x2, x1, v of every batch element first (their
     // loads overlap), the ring-slot stores follow, and only then the state updates start
     float zf[NB];
@@ -630,8 +663,8 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
             a = pj.flip ? g2 : g1;
             gate2 = pj.flip ? g1 : g2;
         } else {
-            a = bf_to_f((x1 + b * in_bs)[d]);
-            c = bf_to_f((v + b * in_bs)[d]);
+            a = ga[j];
+            c = gc[j];
         }
         const float x1v = round_bf(a * c);
         float part = 0.f;
@@ -686,7 +719,7 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
 #pragma unroll
                     for (int m = 1; m < WIN; ++m) (wa.far + (b * WIN + m) * D)[d] = fm[m];
                 }
-                part = fm[0] + wa.g[g * (uint32_t)WIN] * x1v;
+                part = fm[0] + g0 * x1v;
             }
         } else {
             fvec ns;
@@ -712,7 +745,7 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
         if (mode != 3 && live[j] && q == 0) {
             float dx = dco * x1v;
             if (d_is_bf16) dx = round_bf(dx);
-            const float y = (FEAT != 0 ? gate2 : bf_to_f((x2 + b * in_bs)[d])) * (part + dx);
+            const float y = (FEAT != 0 ? gate2 : gg[j]) * (part + dx);
             if (out_is_fp32) ((float*)out + b * out_bs)[d] = y;
             else ((bf16_t*)out + b * out_bs)[d] = (bf16_t)f_to_bf_bits(y);
             // this token's input joins the window's inputs (after every read of the slot it replaces, above)
