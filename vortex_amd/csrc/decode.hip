@@ -30,40 +30,75 @@ struct ProjArgs {
     }
 };
 
-// z[j] = bf16( sum_i w[i][c0+j]*slot_i[c0+j] + w[Rf][c0+j]*u[c0+j] (+ bias) ) for 8 consecutive channels
-__device__ __forceinline__ u32x4 proj_step8(const ProjArgs& pj, int64_t b, uint32_t c0, float* z) {
+// z[j] = bf16( sum_i w[i][c0+j]*slot_i[c0+j] + w[Rf][c0+j]*u[c0+j] (+ bias) ) for 8 consecutive channels.
+// RF > 0: the cache depth is known at compile time and every operand (projection row, RF slots, RF+1 tap rows, bias)
+// is requested before the first one is used, one memory round trip instead of one per slot.  RF == 0: any depth, one
+// slot after the other.  Both add the terms in the same order.
+template <int RF>
+__device__ __forceinline__ u32x4 proj_step8_n(const ProjArgs& pj, int64_t b, uint32_t c0, float* z) {
     const u32x4 un = *(const u32x4*)(pj.u + b * pj.u_bs + c0);
     float acc[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-    bf16_t* rb = pj.ring + (b * pj.Rf) * pj.C + c0;
-    for (int i = 0; i < pj.Rf; ++i) {
-        int s = pj.pos + i;
-        if (s >= pj.Rf) s -= pj.Rf;
-        const u32x4 q = *(const u32x4*)(rb + (int64_t)s * pj.C);
-        const f32x4 t0 = *(const f32x4*)(pj.w + (int64_t)i * pj.C + c0);
-        const f32x4 t1 = *(const f32x4*)(pj.w + (int64_t)i * pj.C + c0 + 4);
+    const bf16_t* rb = pj.ring + (b * pj.Rf) * pj.C + c0;
+    auto add = [&](const f32x4& t0, const f32x4& t1, const u32x4& q) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             acc[2 * j] = fmaf(j < 2 ? t0[2 * j] : t1[2 * j - 4], bf_lo(q[j]), acc[2 * j]);
             acc[2 * j + 1] = fmaf(j < 2 ? t0[2 * j + 1] : t1[2 * j - 3], bf_hi(q[j]), acc[2 * j + 1]);
         }
-    }
-    const f32x4 h0 = *(const f32x4*)(pj.w + (int64_t)pj.Rf * pj.C + c0);
-    const f32x4 h1 = *(const f32x4*)(pj.w + (int64_t)pj.Rf * pj.C + c0 + 4);
+    };
+    f32x4 b0 = {0.f, 0.f, 0.f, 0.f}, b1 = {0.f, 0.f, 0.f, 0.f};
+    if (RF > 0) {
+        constexpr int N = RF > 0 ? RF : 1;
+        u32x4 q[N];
+        f32x4 t0[N + 1], t1[N + 1];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        acc[2 * j] = fmaf(j < 2 ? h0[2 * j] : h1[2 * j - 4], bf_lo(un[j]), acc[2 * j]);
-        acc[2 * j + 1] = fmaf(j < 2 ? h0[2 * j + 1] : h1[2 * j - 3], bf_hi(un[j]), acc[2 * j + 1]);
-    }
-    if (pj.bias) {
-        const f32x4 b0 = *(const f32x4*)(pj.bias + c0), b1 = *(const f32x4*)(pj.bias + c0 + 4);
+        for (int i = 0; i < N; ++i) {
+            int s = pj.pos + i;
+            if (s >= N) s -= N;
+            q[i] = *(const u32x4*)(rb + (int64_t)s * pj.C);
+        }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] += j < 4 ? b0[j] : b1[j - 4];
+        for (int i = 0; i <= N; ++i) {
+            t0[i] = *(const f32x4*)(pj.w + (int64_t)i * pj.C + c0);
+            t1[i] = *(const f32x4*)(pj.w + (int64_t)i * pj.C + c0 + 4);
+        }
+        if (pj.bias) {
+            b0 = *(const f32x4*)(pj.bias + c0);
+            b1 = *(const f32x4*)(pj.bias + c0 + 4);
+        }
+#pragma unroll
+        for (int i = 0; i < N; ++i) add(t0[i], t1[i], q[i]);
+        add(t0[N], t1[N], un);
+    } else {
+        for (int i = 0; i < pj.Rf; ++i) {
+            int s = pj.pos + i;
+            if (s >= pj.Rf) s -= pj.Rf;
+            const u32x4 q = *(const u32x4*)(rb + (int64_t)s * pj.C);
+            const f32x4 t0 = *(const f32x4*)(pj.w + (int64_t)i * pj.C + c0);
+            const f32x4 t1 = *(const f32x4*)(pj.w + (int64_t)i * pj.C + c0 + 4);
+            add(t0, t1, q);
+        }
+        const f32x4 h0 = *(const f32x4*)(pj.w + (int64_t)pj.Rf * pj.C + c0);
+        const f32x4 h1 = *(const f32x4*)(pj.w + (int64_t)pj.Rf * pj.C + c0 + 4);
+        add(h0, h1, un);
+        if (pj.bias) {
+            b0 = *(const f32x4*)(pj.bias + c0);
+            b1 = *(const f32x4*)(pj.bias + c0 + 4);
+        }
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) z[j] = round_bf(acc[j]);
+    for (int j = 0; j < 8; ++j) z[j] = round_bf(acc[j] + (j < 4 ? b0[j & 3] : b1[j & 3]));
     return un;                                          // the caller stores it into the oldest slot
+}
+
+// The depths short featurizers have (2, 3 and 4 taps) take the one-round-trip form.
+__device__ __forceinline__ u32x4 proj_step8(const ProjArgs& pj, int64_t b, uint32_t c0, float* z) {
+    if (pj.Rf == 2) return proj_step8_n<2>(pj, b, c0, z);
+    if (pj.Rf == 1) return proj_step8_n<1>(pj, b, c0, z);
+    if (pj.Rf == 3) return proj_step8_n<3>(pj, b, c0, z);
+    return proj_step8_n<0>(pj, b, c0, z);
 }
 
 __device__ __forceinline__ void proj_store8(const ProjArgs& pj, int64_t b, uint32_t c0, u32x4 un) {
@@ -184,6 +219,36 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
             bs1 = *(const f32x4*)(bias + d0 + 4);
         }
     }
+    // and, for the same reason, what the end of the step reads: the taps on the new sample (k = 0) and on the k-th
+    // newest slot, those slots (the near part of a window), and inside a window its far sums
+    float tk[NBT][GROUPED ? 1 : 8];
+    u32x4 qn[NBT > 1 ? NBT - 1 : 1];
+    f32x4 f0 = {0.f, 0.f, 0.f, 0.f}, f1 = f0;
+#pragma unroll
+    for (int k = 0; k < NBT; ++k)
+#pragma unroll
+        for (int c = 0; c < (GROUPED ? 1 : 8); ++c) tk[k][c] = 0.f;
+#pragma unroll
+    for (int k = 1; k < NBT; ++k) qn[k - 1] = zero4;
+    if (sg == 0 && live) {
+        const int64_t gw = GROUPED ? (dblk / dg + gl) * W : 0;
+#pragma unroll
+        for (int k = 0; k < NBT; ++k) {
+            if (k <= jw) {
+#pragma unroll
+                for (int c = 0; c < (GROUPED ? 1 : 8); ++c) tk[k][c] = GROUPED ? w[gw + R - k] : w[(d0 + c) * W + R - k];
+                if (k > 0) {
+                    int sl = pos - k;
+                    if (sl < 0) sl += R;
+                    qn[k - 1] = *(const u32x4*)(rb + (int64_t)sl * cb);
+                }
+            }
+        }
+        if (NBT > 1 && !heavy) {
+            f0 = *(const f32x4*)(far + ((b * NBT + jw) * D + d0));
+            f1 = *(const f32x4*)(far + ((b * NBT + jw) * D + d0 + 4));
+        }
+    }
     // Fused featurizer: the block's 3 x 512 projection channels are 192 pieces of 8; thread p evaluates piece p
     // (its loads overlap the cache reads above) and leaves the gates in LDS for the wavefront that writes the output.
     if (FEAT != 0) {
@@ -206,8 +271,6 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
         // ---- inside a window: far[jw] plus the jw newest slots, all on the output wavefront
         if (FEAT != 0) __syncthreads();     // the gates are in LDS
         if (sg != 0 || !live) return;
-        const f32x4 f0 = *(const f32x4*)(far + ((b * NBT + jw) * D + d0));
-        const f32x4 f1 = *(const f32x4*)(far + ((b * NBT + jw) * D + d0 + 4));
 #pragma unroll
         for (int c = 0; c < 8; ++c) acc[0][c] = c < 4 ? f0[c & 3] : f1[c & 3];
     } else {
@@ -269,27 +332,17 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
     {
         // taps on the new sample, and (with far sums) the near part: the jw newest slots, which entered the cache
         // after the window's far sums were formed
-        const int64_t gw = GROUPED ? (dblk / dg + gl) * W : 0;
 #pragma unroll
-        for (int c = 0; c < 8; ++c) h0[c] = GROUPED ? w[gw + R] : w[(d0 + c) * W + R];
-        if (NBT > 1) {
-            u32x4 qn[NBT > 1 ? NBT - 1 : 1];
+        for (int c = 0; c < 8; ++c) h0[c] = tk[0][GROUPED ? 0 : c];
 #pragma unroll
-            for (int k = 1; k < NBT; ++k) {
-                int sl = pos - k;
-                if (sl < 0) sl += R;
-                qn[k - 1] = k <= jw ? *(const u32x4*)(rb + (int64_t)sl * cb) : zero4;
-            }
+        for (int k = 1; k < NBT; ++k) {
+            if (k <= jw) {
 #pragma unroll
-            for (int k = 1; k < NBT; ++k) {
-                if (k <= jw) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const float t0 = GROUPED ? w[gw + R - k] : w[(d0 + 2 * j) * W + R - k];
-                        const float t1 = GROUPED ? t0 : w[(d0 + 2 * j + 1) * W + R - k];
-                        acc[0][2 * j] = fmaf(t0, bf_lo(qn[k - 1][j]), acc[0][2 * j]);
-                        acc[0][2 * j + 1] = fmaf(t1, bf_hi(qn[k - 1][j]), acc[0][2 * j + 1]);
-                    }
+                for (int j = 0; j < 4; ++j) {
+                    const float t0 = tk[k][GROUPED ? 0 : 2 * j];
+                    const float t1 = tk[k][GROUPED ? 0 : 2 * j + 1];
+                    acc[0][2 * j] = fmaf(t0, bf_lo(qn[k - 1][j]), acc[0][2 * j]);
+                    acc[0][2 * j + 1] = fmaf(t1, bf_hi(qn[k - 1][j]), acc[0][2 * j + 1]);
                 }
             }
         }
@@ -467,7 +520,8 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
         // one per term
         const float far_j = (wa.far + (b * WIN + jw) * D)[dc];
         const float dcoef = Dcoef[dc];
-        float gk[WIN], hk[WIN];
+        float gk[WIN];
+        uint32_t hk[WIN];                          // as loaded; converted at their use, behind the featurizer's requests
         {
             const float* gp = wa.g + (dc / (uint32_t)dg) * (uint32_t)WIN;
 #pragma unroll
@@ -476,7 +530,7 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
             for (int k = 1; k < WIN; ++k) {
                 int sl = cnt - k;
                 if (sl < 0) sl += WIN;
-                hk[k] = bf_to_f((wa.hist + (b * WIN + sl) * D)[dc]);
+                hk[k] = (wa.hist + (b * WIN + sl) * D)[dc];
             }
         }
         float a, c, gate2;
@@ -510,7 +564,10 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
         float part = far_j + gk[0] * x1v;
 #pragma unroll
         for (int k = 1; k < WIN; ++k)
-            if (k <= jw) part = fmaf(gk[k], hk[k], part);
+        {
+            asm volatile("" : "+v"(hk[k]));        // keeps the conversion here, behind the featurizer's requests
+            if (k <= jw) part = fmaf(gk[k], __uint_as_float(hk[k] << 16), part);
+        }
         float dx = dcoef * x1v;
         if (d_is_bf16) dx = round_bf(dx);
         const float y = gate2 * (part + dx);
@@ -539,6 +596,7 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
     }
     // the inputs a window's first token (or a flush) folds into the state, newest first: u_{t-1-k}
     float pend[NB][WIN > 1 ? WIN : 1];
+    uint32_t pend_raw[NB][WIN > 1 ? WIN : 1];        // as loaded; converted behind the featurizer's requests
     if (WIN > 1 && (mode == 1 || mode == 3)) {
 #pragma unroll
         for (int j = 0; j < NB; ++j)
@@ -546,8 +604,8 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
             for (int k = 0; k < WIN; ++k) {
                 int sl = cnt - 1 - k;
                 if (sl < 0) sl += WIN;
-                pend[j][k] = bf_to_f((wa.hist + (bu(j) * WIN + sl) * D)[d]);     // every slot is requested; the unused
-            }                                                                            // ones are dropped further down
+                pend_raw[j][k] = (wa.hist + (bu(j) * WIN + sl) * D)[d];          // every slot is requested; the unused
+            }                                                                     // ones are dropped further down
     }
     const fvec pp = *(const fvec*)(poles + (g * (uint32_t)(S * FPS) + q * VEC));
     const fvec rr = *(const fvec*)(residues + (g * (uint32_t)(S * FPS) + q * VEC));
@@ -555,6 +613,7 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
     // gates given as vectors, and the window's first filter sample, are requested here with everything above: one
     // round trip for all of a token's operands instead of one per use
     float ga[NB], gc[NB], gg[NB], g0 = 0.f;
+    if (WIN > 1 && mode == 1) g0 = wa.g[g * (uint32_t)WIN];
     if (FEAT == 0 && mode != 3) {
 #pragma unroll
         for (int j = 0; j < NB; ++j) {
@@ -563,14 +622,6 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
             gc[j] = bf_to_f((v + b * in_bs)[d]);
             gg[j] = bf_to_f((x2 + b * in_bs)[d]);
         }
-    }
-    if (WIN > 1 && mode == 1) g0 = wa.g[g * (uint32_t)WIN];
-    if (WIN > 1 && (mode == 1 || mode == 3)) {
-#pragma unroll
-        for (int j = 0; j < NB; ++j)
-#pragma unroll
-            for (int k = 0; k < WIN; ++k)
-                if (k >= npend) pend[j][k] = 0.f;
     }
     // fused featurizer: lanes 0..2 of the group evaluate gates x2, x1, v of every batch element first (their
     // loads overlap), the ring-slot stores follow, and only then the state updates start
@@ -625,6 +676,19 @@ __global__ __launch_bounds__(256) void iir_step_kernel(const bf16_t* __restrict_
                     if (live[j]) pj.ring[((bj(j) * pj.Rf) + pj.pos) * pj.C + pj.chan((uint32_t)q, d)] = un[j];
             }
         }
+    }
+    // the history slots that hold no pending input were requested with the rest; they are dropped here, behind the
+    // featurizer's requests, so that those do not wait for this round trip
+    if (WIN > 1 && (mode == 1 || mode == 3)) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+            for (int k = 0; k < WIN; ++k)
+            {
+                // (opaque to the optimizer, which would otherwise convert right behind the load and wait there)
+                asm volatile("" : "+v"(pend_raw[j][k]));
+                pend[j][k] = k >= npend ? 0.f : __uint_as_float(pend_raw[j][k] << 16);
+            }
     }
     // powers of the poles a window needs: pw[m] = p^(m+1), m = 0 .. WIN-1 (state-wise; complex pairs or 4 reals)
     fvec pw[WIN > 1 ? WIN : 1];
