@@ -164,7 +164,7 @@ def test_layer_step_rejects_bad_maps():
         ops.LayerStepper(fring, wf, None, (4, 12, 4, 1), inner)(u, y)
 
 
-def _random_cases(seed, n):
+def _random_cases(seed, n, taps=(2, 3, 4)):
     import random
     rng = random.Random(seed)
     out = []
@@ -172,12 +172,14 @@ def _random_cases(seed, n):
         H = rng.choice([1, 2, 4])
         hd = 8 * rng.randint(1, 6)
         D = H * hd
-        out.append((rng.randint(1, 5), D, H, rng.choice([2, 3, 4]), rng.choice(["plain", "split", "interleave"]),
+        out.append((rng.randint(1, 5), D, H, rng.choice(taps), rng.choice(["plain", "split", "interleave"]),
                     rng.random() < 0.5, rng.random() < 0.5, rng.randint(0, 10 ** 6)))
     return out
 
 
-@pytest.mark.parametrize("B,D,H,Ks,layout,flip,sbias,seed", _random_cases(11, 16))
+# featurizers of 2-4 taps take the step that requests all its operands at once, longer ones (up to the 8 taps the
+# library accepts) the slot-by-slot form
+@pytest.mark.parametrize("B,D,H,Ks,layout,flip,sbias,seed", _random_cases(11, 16) + _random_cases(12, 8, (5, 6, 7, 8)))
 def test_layer_steps_random(B, D, H, Ks, layout, flip, sbias, seed):
     # both fused layer steps on random channel maps, cache depths and group sizes, several tokens in a row
     import random
@@ -213,7 +215,7 @@ def test_layer_steps_random(B, D, H, Ks, layout, flip, sbias, seed):
                            flip_x1x2=flip)
     wD = w.repeat_interleave(D // G, 0)
     ref_f, ref_s, ref_m = fst, st, s0
-    for i in range(4):
+    for i in range(max(4, Ks + 1)):              # past one turn of the featurizer's ring
         u = torch.randn(B, C, generator=g).bfloat16()
         z, ref_f = O.step_fir(u, ref_f, wf, bias=bf)
         x2, x1, v = oracle_gates(z, D, H, cs, il, flip)
