@@ -264,8 +264,20 @@ def decode_layer_set(D, device, steps, warmup):
         per["iir_step"].update(bytes_moved_per_token=moved, moved_gbs=moved / (per["iir_step"]["us"] * 1e-6) / 1e9,
                                window_tokens=n, note="bytes / hbm_gbs / frac are algorithmic (state read and written per "
                                "token); the kernel moves bytes_moved_per_token on average")
+    # The same token step (three launches and the counter update) recorded once as a HIP graph and replayed: the ring
+    # positions and the window counter then live in device memory (ops.RingClock).  Every cache is full and more
+    # than a window of tokens has been stepped by now, which is what a recording needs.
+    clock = ops.RingClock([ring_se, ring_mr] + ([step.li] if step.li.win is not None else []))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn()
+        clock.advance()
+    _, gms = time_steps(graph.replay, steps, warmup)
+    clock.release()
     return dict(us_per_step=ms * 1e3, wall_us_per_step=wall / steps * 1e6, bytes=byts,
-                hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, kernels=per)
+                hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                us_per_step_graph_replay=gms * 1e3, frac_graph_replay=byts / (gms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                kernels=per)
 
 
 def decode_layers_from_projection(D, device, steps, warmup):
@@ -286,8 +298,8 @@ def decode_layers_from_projection(D, device, steps, warmup):
                             gated_bias=True),
              ops.IirStepper(state, torch.exp(lp[..., 0]).to(device), r.to(device), rnd(D).to(torch.bfloat16),
                             windowed=True)]
-    layers = [ops.LayerStepper(va.FirRing(rnd(B, 2, C).to(torch.bfloat16)), rnd(C, 3) * 3 ** -0.5, None, cmap, n)
-              for n in inner]
+    frings = [va.FirRing(rnd(B, 2, C).to(torch.bfloat16)) for _ in inner]
+    layers = [ops.LayerStepper(fr, rnd(C, 3) * 3 ** -0.5, None, cmap, n) for fr, n in zip(frings, inner)]
     u = [rnd(B, C).to(torch.bfloat16) for _ in range(3)]
     out = [torch.empty(B, D, dtype=torch.bfloat16, device=device) for _ in range(3)]
 
@@ -299,8 +311,17 @@ def decode_layers_from_projection(D, device, steps, warmup):
     # inner caches / state as in decode_layer_set; per layer the projection row, two featurizer slots read and
     # one written (3D channels each) and one output row
     byts = B * D * 2 * (6 + 127) + 2 * B * D * 2 + 2 * state.numel() * 8 + 3 * (4 * B * C * 2 + B * D * 2)
+    # and replayed as a HIP graph, every ring position and the window counter in device memory
+    clock = ops.RingClock(frings + [inner[0].ring, inner[1].ring] + ([inner[2]] if inner[2].win is not None else []))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn()
+        clock.advance()
+    _, gms = time_steps(graph.replay, steps, warmup)
+    clock.release()
     return dict(us_per_step=ms * 1e3, wall_us_per_step=wall / steps * 1e6, bytes=byts,
-                hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
+                hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                us_per_step_graph_replay=gms * 1e3, frac_graph_replay=byts / (gms * 1e-3) / 1e9 / HBM_PEAK_GBS)
 
 
 def model_prefill(device, L, iters=2):

@@ -150,7 +150,7 @@ __global__ __launch_bounds__(64 * NSG) void fir_step_kernel(const bf16_t* __rest
     float* red = smem + (GROUPED ? (W + NBT - 1) * ng : 0);   // [NSG-1][NBT][2][64][4]
     float* zs = red + (NSG - 1) * NBT * 512;      // [3][512] gates of the block's channels (fused featurizer only)
     const int gl = GROUPED ? (oc * 8) / dg : 0;
-    constexpr int UF = 8;                   // cache slots in flight per lane
+    constexpr int UF = 8;                   // cache slots in flight per lane (16, a 127-slot cache in one batch, needs 165 registers: one block per CU, 8 % slower)
     // ring [B][D/cb][R][cb]: the block's 512 channels lie inside one channel block (cb = D is the plain [B][R][D])
     const uint32_t cblk = (uint32_t)d0 / (uint32_t)cb;
     const int64_t roff = ((b * (int64_t)((uint32_t)D / (uint32_t)cb) + cblk) * R) * cb + (d0 - (int64_t)cblk * cb);
