@@ -15,6 +15,8 @@
 // Wavefront w of a block contracts channels 16w..16w+15 (one filter group per wavefront).
 // The LDS input tile is a two-chunk ring: the chunk written in one step is the
 // 128-sample halo of the next, so nothing is copied between steps.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -258,7 +260,10 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
 
     u32x4 raw[NP][NR];
     const u32x4 zero4 = {0, 0, 0, 0};
-    auto load_pieces = [&](int64_t ts, int i0, int i1) {
+    // whole_tag: every row of the step is inside the segment and every channel of the block exists, so the requests
+    // carry no test (and no branch, which lets the compiler count on them when it places its waits)
+    auto load_pieces = [&](int64_t ts, int i0, int i1, auto whole_tag) __attribute__((always_inline)) {
+        constexpr bool WHOLE = decltype(whole_tag)::value;
         uint32_t lo[NP];                          // (with the featurizer the pieces share one offset)
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
@@ -269,15 +274,16 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
             const int64_t t = ts + 4 * rb + r - RF;
-            const bool ok = ch_ok && t >= t_lo && t >= 0 && t < t_end;
+            const bool ok = WHOLE || (ch_ok && t >= t_lo && t >= 0 && t < t_end);
 #pragma unroll
             for (int i = 0; i < NP; ++i) if (i >= i0 && i < i1) {
                 const u32x4* src = (const u32x4*)((const char*)(pp[i] + (ts + r - RF) * pstr[i]) + lo[i]);
-                raw[i][r] = ok ? ((NT && !FEAT) ? __builtin_nontemporal_load(src) : *src) : zero4;
+                if (WHOLE) raw[i][r] = (NT && !FEAT) ? __builtin_nontemporal_load(src) : *src;
+                else raw[i][r] = ok ? ((NT && !FEAT) ? __builtin_nontemporal_load(src) : *src) : zero4;
             }
         }
     };
-    auto load_step = [&](int64_t ts) { load_pieces(ts, 0, NP); };
+    auto load_step = [&](int64_t ts) { load_pieces(ts, 0, NP, std::false_type{}); };
     // Pieces of the next step requested before the MFMA phase (the rest after it).  Without the featurizer all
     // of them travel during the MFMA phase.  With it a lane holds 18 row pieces, which next to all ten A fragments
     // do not fit the register budget of two blocks per CU: one piece goes out early (measured 4 % faster for the
@@ -291,9 +297,12 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
 
     int cur = 0;                       // ring chunk the current step writes; the other one is its halo
     int64_t ts_last = ts0;
-    for (int64_t ts = ts0; ts < t_end; ts += TL) {
+    // One step.  whole_tag: the step computes, all of its rows and of the next step's are inside the segment and every
+    // channel of the block exists: no test guards a request or a store then.
+    auto step = [&](const int64_t ts, auto whole_tag) __attribute__((always_inline)) {
+        constexpr bool WHOLE = decltype(whole_tag)::value;
         ts_last = ts;
-        const bool compute = ts >= t_begin;
+        const bool compute = WHOLE || ts >= t_begin;
         // ---- (a) gates of this lane's 4 x 8 block
         u32x4 bx[4], g2[4];
         if constexpr (FEAT != 0) {
@@ -314,7 +323,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
         }
         // ---- (b) next step's rows (NEARLY pieces of them) are requested now and arrive during the MFMA phase
         __builtin_amdgcn_sched_barrier(0);
-        if (ts + TL < t_end) load_pieces(ts + TL, 0, NEARLY);
+        if (WHOLE || ts + TL < t_end) load_pieces(ts + TL, 0, NEARLY, whole_tag);
 
         // ---- (c) 4 x 8 transpose into the ring chunk `cur`
         {
@@ -340,7 +349,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
         const int c = n & 15, s = n >> 4;
         f32x16 acc0, acc1;
         const bf16_t* urow = u_lds + (16 * w + c) * URS;
-        if (compute && slab_live) {
+        if (WHOLE || (compute && slab_live)) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
             const int c0 = 64 * s + 8 * hh + (cur ^ 1) * TL;     // ring position of the halo chunk's first sample
@@ -358,10 +367,10 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
         constexpr bool LATE_BEFORE_EPILOGUE = MLO == 0;
         if (NEARLY < NP && LATE_BEFORE_EPILOGUE) {
             __builtin_amdgcn_sched_barrier(0);
-            if (ts + TL < t_end) load_pieces(ts + TL, NEARLY, NP);
+            if (WHOLE || ts + TL < t_end) load_pieces(ts + TL, NEARLY, NP, whole_tag);
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (compute && slab_live) {
+        if (WHOLE || (compute && slab_live)) {
 #pragma unroll
             for (int tau = 0; tau < 2; ++tau) {
                 const int tcol = 32 * tau + 64 * s + 16 * hh;
@@ -394,11 +403,11 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
         __syncthreads();
         if (NEARLY < NP && !LATE_BEFORE_EPILOGUE) {
             __builtin_amdgcn_sched_barrier(0);
-            if (ts + TL < t_end) load_pieces(ts + TL, NEARLY, NP);
+            if (WHOLE || ts + TL < t_end) load_pieces(ts + TL, NEARLY, NP, whole_tag);
         }
 
         // ---- 8 x 4 transpose back, gate with x2, store rows
-        if (compute && ch_ok) {
+        if (WHOLE || (compute && ch_ok)) {
             u32x2 zc[8];
 #pragma unroll
             for (int c = 0; c < 8; ++c) zc[c] = *(const u32x2*)(z_lds + (8 * cb + c) * ZRS + ((4 * rb) ^ swz_io));
@@ -417,7 +426,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                 for (int j = 0; j < 4; ++j)
                     zz[j] = (q & 1) ? pair_hi(zc[2 * j][q >> 1], zc[2 * j + 1][q >> 1])
                                     : pair_lo(zc[2 * j][q >> 1], zc[2 * j + 1][q >> 1]);
-                if (t < t_end) {
+                if (WHOLE || t < t_end) {
                     if (AUX && !FEAT && y2_out) *(u32x4*)((char*)y2_step + (lane_row_b + q * row_b)) = zz;
                     u32x4 o = zz;
                     if (POST) {
@@ -432,7 +441,23 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             }
         }
         cur ^= 1;
+    };
+    // The steps in the middle of a segment take the form without tests: with a branch around a request or a store the
+    // compiler has to assume that nothing younger is in flight and waits for everything at the next use of a row piece,
+    // the stores of the step before included; counted exactly, that wait leaves the four stores outstanding.  The steps
+    // at either end (the halo step, the last two) keep their tests, and the state handed to the first whole step is made
+    // known by an explicit wait for everything.  Measured at the config-2 / config-1 shapes: fused Hyena-MR layer 0.506 ->
+    // 0.488-0.490 ms, fused Hyena-SE layer 55.6 -> 52.5-53.1 us; with the gates given as tensors 0.4546 -> 0.4585 ms
+    // (all of the next step's rows go out at once there, on top of the stores), so that form keeps its tests.
+    int64_t ts = ts0;
+    if (!AUX && FEAT != 0 && d0 + CB <= (uint32_t)D) {
+        for (; ts < t_begin; ts += TL) step(ts, std::false_type{});
+        if (ts + 2 * TL <= t_end) {
+            __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0)
+            for (; ts + 2 * TL <= t_end; ts += TL) step(ts, std::true_type{});
+        }
     }
+    for (; ts < t_end; ts += TL) step(ts, std::false_type{});
 
     // ---- cache tail from the ring: chunk cur ^ 1 holds samples ts_last .. ts_last + 127, chunk cur the 128 before
     if (AUX && FEAT && bx_out && t_end == L) {
@@ -495,17 +520,22 @@ __global__ __launch_bounds__(256, 2) void proj_gates_kernel(ProjFwd pj, bf16_t* 
 
     const u32x4 zero4 = {0, 0, 0, 0};
     // the 18 (21) row pieces of one pass of 128 columns starting at column cs; rows past either end read as zero
-    auto load_pass = [&](int64_t cs, u32x4 (&raw)[3][NR]) {
+    // whole_tag: every row of the pass exists and so does every channel of the block; the requests carry no test then
+    auto load_pass = [&](int64_t cs, u32x4 (&raw)[3][NR], auto whole_tag) __attribute__((always_inline)) {
+        constexpr bool WHOLE = decltype(whole_tag)::value;
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
             const int64_t t = cs + 4 * rb + r - RF - pad;  // input sample of this row
-            const bool ok = ch_ok && t >= 0 && t < L;
+            const bool ok = WHOLE || (ch_ok && t >= 0 && t < L);
 #pragma unroll
-            for (int i = 0; i < 3; ++i) raw[i][r] = ok ? *(const u32x4*)(pp[i] + t * pj.ts) : zero4;
+            for (int i = 0; i < 3; ++i) {
+                if (WHOLE) raw[i][r] = *(const u32x4*)(pp[i] + t * pj.ts);
+                else raw[i][r] = ok ? *(const u32x4*)(pp[i] + t * pj.ts) : zero4;
+            }
         }
     };
     u32x4 raw[3][NR];
-    load_pass(c_begin, raw);                               // travels while the tap table is staged
+    load_pass(c_begin, raw, std::false_type{});            // travels while the tap table is staged
 
     for (int e = tid; e < (KS + 1) * 3 * CB; e += 256) {   // taps / bias of the block's channels in lane-piece order
         const int k = e / (3 * CB), r = e - k * 3 * CB, i = r / CB, dl = r - i * CB;
@@ -521,7 +551,7 @@ __global__ __launch_bounds__(256, 2) void proj_gates_kernel(ProjFwd pj, bf16_t* 
     __syncthreads();
 
     // featurizer, gates and the 4 x 8 transposes of one pass into half `half` of the two tiles
-    auto gate_pass = [&](int64_t cs, int half, const u32x4 (&raw)[3][NR]) {
+    auto gate_pass = [&](int64_t cs, int half, const u32x4 (&raw)[3][NR]) __attribute__((always_inline)) {
         u32x4 bx[4], g2[4];
         lane_gates<FEAT, KS>(raw, w_lds, cb, pj, bx, g2);
         if (cs < pad) {                                    // the padding columns stay zero, bias or not
@@ -548,30 +578,51 @@ __global__ __launch_bounds__(256, 2) void proj_gates_kernel(ProjFwd pj, bf16_t* 
 
     const int l32 = tid & 31, r8 = tid >> 5;
     const int tcol = 8 * l32;
-#pragma unroll 1
-    for (int64_t c0 = c_begin; c0 < c_end; c0 += GT) {
-        const bool second = c0 + TL < c_end, next = c0 + GT < c_end;
+    // One tile.  whole_tag: this tile and the next lie inside the block's columns, all their input rows exist and so does
+    // every channel of the block: no test guards a request or a store then.
+    auto tile_step = [&](const int64_t c0, auto whole_tag) __attribute__((always_inline)) {
+        constexpr bool WHOLE = decltype(whole_tag)::value;
+        const bool second = WHOLE || c0 + TL < c_end, next = WHOLE || c0 + GT < c_end;
         gate_pass(c0, 0, raw);
         if (second) {
-            load_pass(c0 + TL, raw);
+            load_pass(c0 + TL, raw, whole_tag);
             gate_pass(c0 + TL, 1, raw);
         }
-        if (next) load_pass(c0 + GT, raw);                 // travels during the stores
+        if (next) load_pass(c0 + GT, raw, whole_tag);      // travels during the stores
         __syncthreads();
         // ---- stores: 32 lanes cover the 512 bytes of one channel row, 8 rows per round, xv then x2
         const int64_t col = c0 + tcol;
-        if (col < Lout) {
+        auto store_round = [&](int rnd) __attribute__((always_inline)) {
+            const int rr = rnd * 8 + r8, ch = rr & (CB - 1);
+            if (!WHOLE && d0 + ch >= (uint32_t)D) return;
+            const bf16_t* tile = rr < CB ? xv_t : x2_t;
+            const u32x4 o = *(const u32x4*)(tile + ch * GRS + (tcol & TL) + ((tcol & (TL - 1)) ^ (32 * (ch >> 4))));
+            *(u32x4*)((rr < CB ? xv_out : x2_out) + (b * D + d0 + ch) * out_rs + col) = o;
+        };
+        if constexpr (WHOLE) {
+#pragma unroll
+            for (int rnd = 0; rnd < 2 * CB / 8; ++rnd) store_round(rnd);       // straight-line: the sixteen stores are counted
+        } else if (col < Lout) {
 #pragma unroll 4
-            for (int rnd = 0; rnd < 2 * CB / 8; ++rnd) {
-                const int rr = rnd * 8 + r8, ch = rr & (CB - 1);
-                if (d0 + ch >= (uint32_t)D) continue;
-                const bf16_t* tile = rr < CB ? xv_t : x2_t;
-                const u32x4 o = *(const u32x4*)(tile + ch * GRS + (tcol & TL) + ((tcol & (TL - 1)) ^ (32 * (ch >> 4))));
-                *(u32x4*)((rr < CB ? xv_out : x2_out) + (b * D + d0 + ch) * out_rs + col) = o;
-            }
+            for (int rnd = 0; rnd < 2 * CB / 8; ++rnd) store_round(rnd);
         }
         if (next) __syncthreads();                         // the tiles are free again
+    };
+    // Tiles in the middle of the block's run take the form without tests (see fir_cl_kernel: with a branch around a
+    // request or a store the compiler waits for everything in flight, the stores of the tile before included, at the
+    // next use of a row piece); the first tile of the sequence, whose first rows do not exist, and a run's last two keep
+    // their tests.
+    int64_t c0 = c_begin;
+    if (KS <= 3 && d0 + CB <= (uint32_t)D) {              // (with four taps the second copy of the step does not fit the registers)
+        for (; c0 < c_end && c0 < pad + RF; c0 += GT) tile_step(c0, std::false_type{});
+        if (c0 + 2 * GT <= c_end) {
+            __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): a known state for the counted waits
+#pragma unroll 1
+            for (; c0 + 2 * GT <= c_end; c0 += GT) tile_step(c0, std::true_type{});
+        }
     }
+#pragma unroll 1
+    for (; c0 < c_end; c0 += GT) tile_step(c0, std::false_type{});
 }
 
 struct LaunchArgs {

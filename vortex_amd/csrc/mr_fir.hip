@@ -17,6 +17,8 @@
 //   -> coalesced read, * x2, 16 B/lane store.
 // The 128-sample tail of a step stays in LDS as the next step's halo, so each
 // input is read from HBM once per segment.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -108,11 +110,17 @@ __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
     for (int r4 = 0; r4 < 4; ++r4) {
         rlive[r4] = 4 * r4 + w < c_live;
         const int64_t d = rlive[r4] ? d0 + 4 * r4 + w : d0;
-        p1[r4] = x1.row(b, d) + lane * 8;
-        pv[r4] = PRE ? v.row(b, d) + lane * 8 : nullptr;
-        p2[r4] = POST ? x2.row(b, d) + lane * 8 : nullptr;
-        po[r4] = out + (b * D + d) * L + lane * 8;
+        p1[r4] = x1.row(b, d);
+        pv[r4] = PRE ? v.row(b, d) : nullptr;
+        p2[r4] = POST ? x2.row(b, d) : nullptr;
+        po[r4] = out + (b * D + d) * L;
     }
+    // The row bases above are the same for every lane of the wavefront; a lane adds its 32-bit byte offset at each
+    // access (scalar base + vector offset addressing), so no 64-bit address per lane and row is held across the loop.
+    const uint32_t lane_b = (uint32_t)lane * 16u;
+    auto at = [](const bf16_t* base, int64_t t, uint32_t off) __attribute__((always_inline)) {
+        return (const bf16_t*)((const char*)(base + t) + off);
+    };
     const int64_t t_begin = (int64_t)seg * seg_len;
     const int64_t t_end = (t_begin + seg_len < L) ? t_begin + seg_len : L;
     if (t_begin >= t_end) return;
@@ -135,15 +143,18 @@ __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
         const bool ok = rlive[r4] && t_begin + lane * 8 < L;
-        c1[r4] = ok ? ld16<NT>(p1[r4] + t_begin) : zero4;
-        cv[r4] = (PRE && ok) ? ld16<NT>(pv[r4] + t_begin) : zero4;
-        c2n[r4] = (POST && ok) ? ld16<NT>(p2[r4] + t_begin) : zero4;
+        c1[r4] = ok ? ld16<NT>(at(p1[r4], t_begin, lane_b)) : zero4;
+        cv[r4] = (PRE && ok) ? ld16<NT>(at(pv[r4], t_begin, lane_b)) : zero4;
+        c2n[r4] = (POST && ok) ? ld16<NT>(at(p2[r4], t_begin, lane_b)) : zero4;
     }
 
     float bz = 0.f;
     if (BIAS != HYENA_BIAS_NONE && (n & 15) < c_live) bz = bias[d0 + (n & 15)];
 
-    for (int64_t ts = t_begin; ts < t_end; ts += TL) {
+    // One step.  whole_tag: all sixteen channels of the slab exist and this step and the next lie inside the segment, so
+    // no test guards a request or a store.
+    auto step = [&](const int64_t ts, auto whole_tag) __attribute__((always_inline)) {
+        constexpr bool WHOLE = decltype(whole_tag)::value;
         // u of this step -> LDS
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4)
@@ -155,13 +166,21 @@ __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
         {
             const int64_t tn = ts + TL;
             const bool okt = (tn < t_end) && (tn + lane * 8 < L);
+            uint32_t lo = lane_b;
+            asm volatile("" : "+v"(lo));          // keeps the compiler from folding it into per-lane row pointers held across the loop
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
                 const bool okn = okt && rlive[r4];
                 c2[r4] = c2n[r4];
-                c1[r4] = okn ? ld16<NT>(p1[r4] + tn) : zero4;
-                cv[r4] = (PRE && okn) ? ld16<NT>(pv[r4] + tn) : zero4;
-                c2n[r4] = (POST && okn) ? ld16<NT>(p2[r4] + tn) : zero4;
+                if (WHOLE) {
+                    c1[r4] = ld16<NT>(at(p1[r4], tn, lo));
+                    if (PRE) cv[r4] = ld16<NT>(at(pv[r4], tn, lo));
+                    if (POST) c2n[r4] = ld16<NT>(at(p2[r4], tn, lo));
+                } else {
+                    c1[r4] = okn ? ld16<NT>(at(p1[r4], tn, lo)) : zero4;
+                    cv[r4] = (PRE && okn) ? ld16<NT>(at(pv[r4], tn, lo)) : zero4;
+                    c2n[r4] = (POST && okn) ? ld16<NT>(at(p2[r4], tn, lo)) : zero4;
+                }
             }
         }
         // tail of this step = halo of the next one (read now, written after the MFMA phase)
@@ -222,10 +241,12 @@ __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
 
         *(u32x4*)(u_lds + (tid >> 4) * URS + (tid & 15) * 8) = tail;
         // ---- gate with x2 and store, coalesced
-        if (ts + lane * 8 < t_end) {
+        if (WHOLE || ts + lane * 8 < t_end) {
+            uint32_t lo = lane_b;
+            asm volatile("" : "+v"(lo));
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
-                if (!rlive[r4]) continue;
+                if (!WHOLE && !rlive[r4]) continue;
                 const u32x4 zz = *(const u32x4*)(z_lds + (4 * r4 + w) * ZRS + lane * 8);
                 u32x4 o = zz;
                 if (POST) {
@@ -233,10 +254,21 @@ __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
                     for (int j = 0; j < 4; ++j)
                         o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(c2[r4][j]), bf_hi(zz[j]) * bf_hi(c2[r4][j]));
                 }
-                st16<NT>(po[r4] + ts, o);
+                st16<NT>((bf16_t*)((char*)(po[r4] + ts) + lo), o);
             }
         }
+    };
+    // Steps in the middle of a segment take the form without tests.  With a branch around a request or a store the
+    // compiler must assume that nothing younger is in flight, and waits for everything at the next use of a prefetched
+    // row: the stores of the step before included, a write's whole latency per step.  Counted exactly, that wait leaves
+    // the four stores outstanding.  The last step of a segment keeps its tests; the prologue's requests are waited for
+    // in full before the first whole step so that its counts start from a known state.
+    int64_t ts = t_begin;
+    if (c_live == 16 && ts + 2 * TL <= t_end) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0)
+        for (; ts + 2 * TL <= t_end; ts += TL) step(ts, std::true_type{});
     }
+    for (; ts < t_end; ts += TL) step(ts, std::false_type{});
 }
 
 }  // namespace
