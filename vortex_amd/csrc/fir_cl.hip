@@ -287,9 +287,11 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     // Pieces of the next step requested before the MFMA phase (the rest after it).  Without the featurizer all
     // of them travel during the MFMA phase.  With it a lane holds 18 row pieces, which next to all ten A fragments
     // do not fit the register budget of two blocks per CU: one piece goes out early (measured 4 % faster for the
-    // medium filter than none; two fit since the output addresses stopped taking registers but measured 7 % slower),
-    // none for the short-filter form (one measured the same).
-    constexpr int NEARLY = FEAT ? (MLO == 0 ? 1 : 0) : NP;
+    // medium filter than none; two fit since the output addresses stopped taking registers but measured 7 % slower,
+    // and still 1-2 % slower with the steps without tests below).  The short-filter form, with three A fragments, has
+    // room for all three: since its middle steps run without tests (counted waits) that is 1.6-2.4 % faster than none,
+    // from B*L = 8192 to 131072 rows; before, one piece early had measured the same as none.
+    constexpr int NEARLY = FEAT ? (MLO == 0 ? 1 : NP) : NP;
     load_step(ts0);
 
     float bz = 0.f;
@@ -448,7 +450,8 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     // at either end (the halo step, the last two) keep their tests, and the state handed to the first whole step is made
     // known by an explicit wait for everything.  Measured at the config-2 / config-1 shapes: fused Hyena-MR layer 0.506 ->
     // 0.488-0.490 ms, fused Hyena-SE layer 55.6 -> 52.5-53.1 us; with the gates given as tensors 0.4546 -> 0.4585 ms
-    // (all of the next step's rows go out at once there, on top of the stores), so that form keeps its tests.
+    // (all of the next step's rows go out at once there, on top of the stores; 0.4568 ms with them held back behind the
+    // barrier), so that form keeps its tests.
     int64_t ts = ts0;
     if (!AUX && FEAT != 0 && d0 + CB <= (uint32_t)D) {
         for (; ts < t_begin; ts += TL) step(ts, std::false_type{});
