@@ -158,7 +158,10 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t bid = blockIdx.x;
-    // channel blocks fastest: the blocks resident at one time read neighbouring 128-byte pieces of the same rows
+    // channel blocks fastest: the blocks resident at one time read neighbouring 128-byte pieces of the same rows.
+    // Workgroups are dealt to the 8 XCDs in turn (id mod 8), so every XCD takes every eighth channel block of all
+    // row tiles; giving an XCD neighbouring channel blocks (0.457 -> 0.509 ms with the gates given as tensors), whole
+    // row tiles (0.488 ms) or an eighth of the block order (0.487 ms) all measured slower.
     const uint32_t db = bid % (uint32_t)ndb;
     const int seg = (int)((bid / (uint32_t)ndb) % (uint32_t)nseg);
     const int64_t b = bid / ((uint32_t)nseg * (uint32_t)ndb);
@@ -504,7 +507,12 @@ __global__ __launch_bounds__(256, 2) void proj_gates_kernel(ProjFwd pj, bf16_t* 
     __shared__ __attribute__((aligned(16))) float w_lds[(KS + 1) * 3 * CB];
     const int tid = threadIdx.x;
     const uint32_t bid = blockIdx.x;
-    const uint32_t db = bid % (uint32_t)ndb;
+    // Workgroups are dealt to the 8 XCDs in turn (id mod 8): XCD x takes the x-th eighth of the channel blocks of a row
+    // tile, neighbouring strips, so that its L2 fetches 3 KB runs of each row (D = 4096) instead of every eighth 384-byte
+    // piece: 2.27 -> 2.18 ms at the config-3 shape.  (The same order made fir_cl_kernel slower: 0.457 -> 0.509 ms with
+    // the gates given as tensors.)
+    uint32_t db = bid % (uint32_t)ndb;
+    if ((ndb & 7) == 0) db = (db & 7u) * ((uint32_t)ndb >> 3) + (db >> 3);
     const uint32_t chunk = (bid / (uint32_t)ndb) % (uint32_t)nchunk;      // ntpb consecutive tiles along the columns
     const int64_t b = bid / ((uint32_t)ndb * (uint32_t)nchunk);
     const uint32_t d0 = db * CB;

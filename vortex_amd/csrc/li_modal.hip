@@ -184,7 +184,12 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     __shared__ float2 e_sh[COOP ? 2 * 4 * 64 : 1];             // [step parity][wavefront][lane] piece end states
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int64_t quad = COOP ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + w;   // CPW channels of one batch element
+    // Workgroups are dealt to the 8 XCDs in turn (id mod 8).  XCD x takes the x-th eighth of the rows, so that each XCD
+    // walks one contiguous part of the tensors instead of every eighth row group of all of them: 1.64 -> 1.52 ms at
+    // B = 1, L = 262144, D = 4096 with 256 filter groups, 1.62 -> 1.58 ms with one filter per channel.
+    uint32_t xbid = blockIdx.x;
+    if ((gridDim.x & 7u) == 0) xbid = (xbid & 7u) * (gridDim.x >> 3) + (xbid >> 3);
+    const int64_t quad = COOP ? (int64_t)xbid : (int64_t)xbid * 4 + w;   // CPW channels of one batch element
     if (quad >= a.nquads) return;                              // whole wavefront leaves (never with COOP: no barrier is skipped)
     const uint32_t qpb = (uint32_t)(a.D / CPW);
     const int64_t b = (uint32_t)quad / qpb;

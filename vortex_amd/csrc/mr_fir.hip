@@ -67,7 +67,12 @@ __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
     // with fewer live channels (their rows are read as zeros and never stored).
     const uint32_t spg = ((uint32_t)dg + 15) / 16;              // slabs per group
     const uint32_t nslab = (uint32_t)(D / dg) * spg;
-    const uint32_t bid = blockIdx.x;
+    // Workgroups are dealt to the 8 XCDs in turn (id mod 8).  For tensors that stream through the caches XCD x takes
+    // the x-th eighth of the (batch, slab, segment) order, so that each XCD (and its L2) walks one contiguous part of
+    // the tensors instead of every eighth piece of all of them: 340 -> 334 us at the config-2 shape.  Cache-resident
+    // shapes measured 4-5 % slower that way and keep the plain order.
+    uint32_t bid = blockIdx.x;
+    if (NT && (gridDim.x & 7u) == 0) bid = (bid & 7u) * (gridDim.x >> 3) + (bid >> 3);
     const int seg = (int)(bid % (uint32_t)nseg);
     const uint32_t slab = (bid / (uint32_t)nseg) % nslab;
     const int64_t b = bid / ((uint32_t)nseg * nslab);

@@ -27,13 +27,27 @@ __global__ __launch_bounds__(256) void se_fir_kernel(RowMap x1, RowMap x2, RowMa
     // all index arithmetic in 32 bits: the host checks that B*D and L/8 fit
     uint32_t row, oct;
     uint32_t b, d;
+    // Workgroups are dealt to the 8 XCDs in turn (linear id mod 8).  For tensors that stream through the caches XCD x
+    // takes the x-th eighth of the blocks in memory order, so that each XCD walks one contiguous part of the tensors.
+    uint32_t gx = blockIdx.x, gy = blockIdx.y, gz = blockIdx.z;
+    if (NT) {
+        const uint32_t nb = gridDim.x * gridDim.y * gridDim.z;         // the host bounds the block count to 2^31
+        if ((nb & 7u) == 0) {
+            uint32_t lid = gx + gridDim.x * (gy + gridDim.y * gz);
+            lid = (lid & 7u) * (nb >> 3) + (lid >> 3);
+            gx = lid % gridDim.x;
+            lid /= gridDim.x;
+            gy = lid % gridDim.y;
+            gz = lid / gridDim.y;
+        }
+    }
     if (ROWU) {                              // a block never straddles rows: grid = (blocks per row, D, B)
-        d = blockIdx.y;
-        b = blockIdx.z;
+        d = gy;
+        b = gz;
         row = b * (uint32_t)D + d;
-        oct = blockIdx.x * 256u + threadIdx.x;
+        oct = gx * 256u + threadIdx.x;
     } else {
-        const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+        const uint64_t idx = (uint64_t)gx * 256u + threadIdx.x;
         row = (uint32_t)(idx / (uint32_t)octs_per_row);
         oct = (uint32_t)(idx - (uint64_t)row * (uint32_t)octs_per_row);
     }
