@@ -500,11 +500,16 @@ def main():
         cases = [("whole rows, one block per 4 rows (a one-pass scan)", 0, 0)]
         cases += [(f"whole rows, one block per row (4 wavefronts x 4 KiB per step), {256 * n} rows in flight", 2, n) for n in (8, 4, 2, 1)]
         cases += [(f"independent segments of {s} samples, row sets in order", 1, s) for s in (65536, 16384, 8192, 4096, 2048)]
+        # each order twice: blocks dealt to the 8 XCDs in turn (every XCD touches every eighth block's memory), and XCD x
+        # taking the x-th eighth of the block order (pattern + 8), which is what the row kernels do for streaming shapes
         for what, pat, seg in cases:
-            fn = lambda: _lib.check(probe(t[0].data_ptr(), t[1].data_ptr(), t[2].data_ptr(), o.data_ptr(), D, L, pat, seg,
-                                          stream), "stream probe")
-            _, ms = time_steps(fn, 5, 2)
-            print(f"  {what:75s} {ms * 1e3:8.1f} us {8 * D * L / (ms * 1e-3) / 1e9:7.0f} GB/s", file=sys.stderr)
+            res = []
+            for xcd in (0, 8):
+                fn = lambda: _lib.check(probe(t[0].data_ptr(), t[1].data_ptr(), t[2].data_ptr(), o.data_ptr(), D, L,
+                                              pat + xcd, seg, stream), "stream probe")
+                _, ms = time_steps(fn, 5, 2)
+                res.append(f"{ms * 1e3:8.1f} us {8 * D * L / (ms * 1e-3) / 1e9:6.0f} GB/s")
+            print(f"  {what:75s} {res[0]}   XCD-contiguous: {res[1]}", file=sys.stderr)
         del t, o
         torch.cuda.empty_cache()
 

@@ -57,8 +57,10 @@ const char* hyena_last_error_string(void);
 /* Launch-shape override, for tests and tuning sweeps; no counterpart in the reference.  The launchers choose
  * segment counts, cached / non-temporal accesses and work decompositions from the problem size; this pins one of
  * those choices process-wide until it is reset with a negative value.  Nothing is read from the environment.
- *   "mr_nseg", "cl_nseg", "li_nseg"            segments along L of hyena_mr_fwd, hyena_fir_cl_fwd / layer_fwd, hyena_li_fwd
+ *   "mr_nseg", "cl_nseg"                       segments along L of hyena_mr_fwd, hyena_fir_cl_fwd / layer_fwd
  *                                               (cl_nseg also: blocks along L per channel strip in hyena_featurizer_gates_fwd)
+ *   "li_xcd"                                    hyena_li_fwd: consecutive row groups an XCD takes in one run (0 = blocks in
+ *                                               plain order, every eighth to one XCD; default a whole eighth of the rows)
  *   "se_nt", "mr_nt", "li_nt", "cl_nt"         0 = cached, 1 = non-temporal global accesses
  *   "li_cpw"                                    1 / 4 = channels per wavefront in hyena_li_fwd (4 needs D/G % 4 == 0)
  *   "li_coop"                                   0 / 1 = lone / cooperating wavefronts in hyena_li_fwd

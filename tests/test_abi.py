@@ -180,7 +180,7 @@ def test_launch_override_names():
     if not os.path.exists(_lib.LIB_PATH):
         pytest.skip("library not built in this tree")
     L = _lib.lib()
-    for n in (b"mr_nseg", b"cl_nseg", b"li_nseg", b"se_nt", b"mr_nt", b"li_nt", b"cl_nt", b"li_cpw", b"li_coop"):
+    for n in (b"mr_nseg", b"cl_nseg", b"li_xcd", b"se_nt", b"mr_nt", b"li_nt", b"cl_nt", b"li_cpw", b"li_coop"):
         assert L.hyena_set_launch_override(n, 1) == 0 and L.hyena_set_launch_override(n, -1) == 0
     assert L.hyena_set_launch_override(b"HYENA_MR_NSEG", 1) == -1
     assert L.hyena_set_launch_override(None, 1) == -1

@@ -58,7 +58,7 @@ int hyena_check_launch(const char* what);
 
 // launch-shape overrides set through hyena_set_launch_override (api.hip); -1 = the launcher's own choice
 enum { HYENA_OV_MR_NSEG, HYENA_OV_CL_NSEG, HYENA_OV_SE_NT, HYENA_OV_MR_NT, HYENA_OV_LI_NT, HYENA_OV_CL_NT,
-       HYENA_OV_LI_CPW, HYENA_OV_LI_COOP, HYENA_OV_LI_NSEG, HYENA_OV_COUNT };
+       HYENA_OV_LI_CPW, HYENA_OV_LI_COOP, HYENA_OV_LI_XCD, HYENA_OV_COUNT };
 int64_t hyena_override(int id);
 
 static inline bool rows_aligned8(const hyena_rows* r) {

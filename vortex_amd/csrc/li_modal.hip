@@ -166,6 +166,7 @@ struct LiArgs {
     int dg;
     int d_is_bf16;
     int64_t nquads;           // B * D / 4 wavefront-sized work items
+    uint32_t xchunk;          // blocks an XCD takes in one run (0: plain block order)
 };
 
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0)
@@ -184,11 +185,15 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     __shared__ float2 e_sh[COOP ? 2 * 4 * 64 : 1];             // [step parity][wavefront][lane] piece end states
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // Workgroups are dealt to the 8 XCDs in turn (id mod 8).  XCD x takes the x-th eighth of the rows, so that each XCD
-    // walks one contiguous part of the tensors instead of every eighth row group of all of them: 1.64 -> 1.52 ms at
-    // B = 1, L = 262144, D = 4096 with 256 filter groups, 1.62 -> 1.58 ms with one filter per channel.
+    // Workgroups are dealt to the 8 XCDs in turn (id mod 8).  An XCD takes runs of xchunk consecutive blocks (by
+    // default one run: the x-th eighth of the rows), so that it walks contiguous parts of the tensors instead of every
+    // eighth row group of all of them: 1.64 -> 1.52-1.56 ms at B = 1, L = 262144, D = 4096 with 256 filter groups,
+    // 1.62 -> 1.58 ms with one filter per channel.
     uint32_t xbid = blockIdx.x;
-    if ((gridDim.x & 7u) == 0) xbid = (xbid & 7u) * (gridDim.x >> 3) + (xbid >> 3);
+    if (a.xchunk) {
+        const uint32_t r = xbid >> 3;
+        xbid = (r / a.xchunk) * 8u * a.xchunk + (xbid & 7u) * a.xchunk + r % a.xchunk;
+    }
     const int64_t quad = COOP ? (int64_t)xbid : (int64_t)xbid * 4 + w;   // CPW channels of one batch element
     if (quad >= a.nquads) return;                              // whole wavefront leaves (never with COOP: no barrier is skipped)
     const uint32_t qpb = (uint32_t)(a.D / CPW);
@@ -822,6 +827,14 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
     a.dg = (int)(D / G);
     a.d_is_bf16 = d_is_bf16;
     a.nquads = nquads;
+    {
+        // runs of blocks per XCD: a whole eighth of the grid unless pinned; a run length that does not tile the grid
+        // falls back to the plain order
+        int64_t c = nblk % 8 == 0 ? nblk / 8 : 0;
+        const int64_t x = hyena_override(HYENA_OV_LI_XCD);
+        if (x >= 0) c = (x > 0 && nblk % (8 * x) == 0) ? x : 0;
+        a.xchunk = (uint32_t)c;
+    }
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)nblk);
     bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;

@@ -27,10 +27,15 @@ __device__ __forceinline__ void stnt(bf16_t* p, u32x4 v) { __builtin_nontemporal
 // unit u of this block -> element offset of row r (or -1 when the unit does not exist)
 struct Walk {
     int64_t L, nsets, seg; int nseg; int64_t nunits;
+    int xcd;       // != 0: XCD x (block id mod 8) takes the x-th eighth of the block order instead of every eighth block
+    __device__ __forceinline__ uint32_t block() const {
+        const uint32_t bid = blockIdx.x;
+        return (xcd && (gridDim.x & 7u) == 0) ? (bid & 7u) * (gridDim.x >> 3) + (bid >> 3) : bid;
+    }
     template <int PATTERN>
     __device__ __forceinline__ int64_t at(int64_t u, int w, int lane) const {     // row 0 of the unit; row r is r*L further
         int64_t set, t;                                            // 32-bit index arithmetic (64-bit division is emulated)
-        const uint32_t bid = blockIdx.x, uu = (uint32_t)u;
+        const uint32_t bid = block(), uu = (uint32_t)u;
         if (PATTERN == 0) { set = bid; t = (int64_t)uu * 2048; }
         else { set = bid / (uint32_t)nseg; t = (int64_t)(bid % (uint32_t)nseg) * seg + (int64_t)uu * 2048; }
         return set * R * L + t + 512 * w + lane * 8;
@@ -87,12 +92,14 @@ __global__ __launch_bounds__(256) void stream_probe_kernel(const bf16_t* a, cons
     }
 }
 // pattern 2: block = one row, wavefront w takes samples [2048 w, 2048 w + 2048) of each 8192-sample block step
-__global__ __launch_bounds__(256) void row_probe_kernel(const bf16_t* a, const bf16_t* b, const bf16_t* c, bf16_t* o, int64_t L) {
+__global__ __launch_bounds__(256) void row_probe_kernel(const bf16_t* a, const bf16_t* b, const bf16_t* c, bf16_t* o, int64_t L,
+                                                        int xcd) {
     extern __shared__ char occupancy_limit[];
     constexpr int K = 4;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int64_t step = 4 * K * 512, nsteps = L / step;
-    const int64_t base = (int64_t)blockIdx.x * L + (int64_t)w * K * 512 + lane * 8;
+    const uint32_t bid = (xcd && (gridDim.x & 7u) == 0) ? (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3) : blockIdx.x;
+    const int64_t base = (int64_t)bid * L + (int64_t)w * K * 512 + lane * 8;
     u32x4 x[PF][K], y[PF][K], z[PF][K];
 #pragma unroll
     for (int p = 0; p < PF; ++p)
@@ -131,12 +138,16 @@ __global__ __launch_bounds__(256) void row_probe_kernel(const bf16_t* a, const b
 }  // namespace
 
 // a, b, c, o: D rows of L bf16 samples each (contiguous); D % 4 == 0, L % 2048 == 0.
+// pattern + 8: the same order with XCD x (block id mod 8) taking the x-th eighth of the blocks.
 // pattern 0: seg ignored.  pattern 1: seg a multiple of 2048 dividing L.  pattern 2: seg = blocks per CU (1, 2, 4, 8), L % 8192 == 0.
 // 0 on success, -1 for a rejected argument, a positive hipError_t if the launch failed.
 extern "C" int hyena_stream_probe(const void* a, const void* b, const void* c, void* o, int64_t D, int64_t L, int pattern,
                                   int64_t seg, void* stream) {
+    const int xcd = pattern >= 0 ? (pattern >> 3) & 1 : 0;         // pattern + 8: the XCD-contiguous block order
+    if (pattern >= 0) pattern &= ~8;
     if (!a || !b || !c || !o || D <= 0 || D % R || L <= 0 || L % 2048 || pattern < 0 || pattern > 2) return -1;
     Walk wk = {};
+    wk.xcd = xcd;
     wk.L = L; wk.nsets = D / R;
     int64_t grid;
     if (pattern == 0) { wk.nunits = L / 2048; grid = wk.nsets; }
@@ -148,7 +159,7 @@ extern "C" int hyena_stream_probe(const void* a, const void* b, const void* c, v
         if (L % 8192 || (seg != 1 && seg != 2 && seg != 4 && seg != 8) || D > 0x7fffffffLL) return -1;
         const size_t lds = seg == 1 ? 100000 : seg == 2 ? 70000 : seg == 4 ? 36000 : 0;      // of 160 KiB per CU
         hipLaunchKernelGGL(row_probe_kernel, dim3((unsigned)D), dim3(256), lds, (hipStream_t)stream, (const bf16_t*)a,
-                           (const bf16_t*)b, (const bf16_t*)c, (bf16_t*)o, L);
+                           (const bf16_t*)b, (const bf16_t*)c, (bf16_t*)o, L, xcd);
         return (int)hipGetLastError();
     }
     if (grid > 0x7fffffffLL) return -1;
