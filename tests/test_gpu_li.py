@@ -241,3 +241,25 @@ def test_li_state_with_fast_poles_and_ragged_length(tail, cplx, form, override):
     y = va.iir_step(x1[..., L].contiguous().cuda(), x2[..., L].contiguous().cuda(), v[..., L].contiguous().cuda(),
                     st, torch.exp(lp[..., 0]).cuda(), r.cuda(), Db.cuda())
     assert rel_err(y, full[..., L]) <= 2e-2
+
+
+@pytest.mark.parametrize("form", ["coop4", "cpw1"])
+def test_li_block_order_changes_nothing(form, override):
+    """The order in which blocks take the row groups (runs of consecutive groups per XCD, the li_xcd launch override)
+    is a renumbering: outputs and state are bit-identical for the plain order, short runs and the default, and a run
+    length that does not tile the grid falls back to the plain order."""
+    B, D, L, G = 2, 128, 1024 + 264, 32
+    x2, x1, v = O.make_gates(B, D, L, seed=77)
+    lp, r = O.make_modal_complex(G, 16, seed=5)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(2)).bfloat16()
+    form_kv = dict(li_cpw=4, li_coop=1) if form == "coop4" else dict(li_cpw=1)
+    ref, _, st_ref = O.li_prefill(x2, x1, v, lp, r, Db)
+    res = []
+    for xcd in (0, 2, 4, 3, -1):            # 64 blocks: 3 does not tile them
+        override(li_xcd=xcd, **form_kv)
+        out, _, st = va.hyena_li_fwd(x1.cuda(), x2.cuda(), v.cuda(), lp.cuda(), r.cuda(), Db.cuda(), want_state=True)
+        res.append((out.cpu(), st.cpu()))
+    assert rel_err(res[0][0], ref) <= 2e-2
+    assert rel_err(torch.view_as_real(res[0][1]), torch.view_as_real(st_ref)) <= 1e-4
+    for out, st in res[1:]:
+        assert torch.equal(out, res[0][0]) and torch.equal(st, res[0][1])
