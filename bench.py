@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0     # MI355X published HBM3E bandwidth
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
 # counter reads for the plain copy launch of known size.  These are constants of the committed profile, not
 # measurements of this run: `roofline.traffic_source` names the file they were read from.
-MEASURED_TRAFFIC = {"mr": 2211.99e6, "se": 271.75e6, "li": 8597.09e6}
+MEASURED_TRAFFIC = {"mr": 2148.09e6, "se": 271.75e6, "li": 8592.12e6}
 TRAFFIC_SOURCE = "profiles/bench_default_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; copy-probe calibrated)"
 
 
