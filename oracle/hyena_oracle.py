@@ -36,6 +36,16 @@ How each function is pinned (see tests/test_oracle_*.py):
                                  consistency and the closed-form recurrence,
                                  plus the committed golden vectors in
                                  tests/golden/ when present.
+  prefill_direct_recurrence_ref: the literal loop of engine.py:473-504 (bf16
+                                 state, in-place lanes, lane-0 output): three
+                                 hand-computed three-step cases, and equality
+                                 with the plain recurrence where its quirks
+                                 cannot act (real poles, float32 activations)
+  OracleCascade                : prefill of L+n tokens == prefill of L tokens +
+                                 n one-token calls (outputs and caches) over SE /
+                                 MR / LI x split x interleave x x1-x2 flip, and
+                                 an index known answer (which projection channel
+                                 acts as x2 / x1 / v on either branch)
 """
 
 from __future__ import annotations
@@ -332,10 +342,11 @@ def li_prefill(x2, x1, v, log_poles, residues, D_bias, want_state=True):
 
 
 def prefill_direct_recurrence(x1v, log_poles, residues):
-    """Explicit modal recurrence  s_t = p s_{t-1} + u_t,  y_t = Re sum r s_t.
+    """Explicit modal recurrence  s_t = p s_{t-1} + u_t,  y_t = Re sum r s_t, in double.
 
-    Same arithmetic as engine.py:473-504 (which carries separate re/im lanes),
-    written with complex tensors in double for use as the independent check
+    The mathematics that engine.py:473-504 is meant to evaluate (true complex
+    product, exact state), NOT that loop's own arithmetic, which differs in three
+    ways (see prefill_direct_recurrence_ref below).  Used as the independent check
     of the FFT path.  Returns (y [B, D, L] float64, final state [B, D, S]).
     """
     B, Dch, L = x1v.shape
@@ -352,6 +363,35 @@ def prefill_direct_recurrence(x1v, log_poles, residues):
         acc = (r * s).sum(-1)
         y[:, :, i] = acc.real if cplx else acc
     return y, s
+
+
+def prefill_direct_recurrence_ref(x1v, poles, residues):
+    """Restatement of HyenaInferenceEngine.prefill_via_direct_recurrence as it is written (engine.py:473-504).
+
+    x1v [B, D, L] in the activations' dtype; poles and residues [D, S, 1, 2] with (re, im) lanes (the poles
+    themselves: this branch never exponentiates).  What the loop does, which the mathematics would not:
+      * the state is created as `0 * x1v_[:, :, 0]` (engine.py:487) and so has the activations' dtype: with bf16
+        activations it is rounded to bf16 after every update, and so is the output row (engine.py:488);
+      * the real lane is overwritten first and the imaginary lane then reads the NEW real lane
+        (engine.py:498-499), which is not the complex product unless the poles are real;
+      * the output keeps lane 0 of the lane-wise product residues * state summed over the modes
+        (engine.py:500), i.e. sum_s r_re * s_re without the - r_im * s_im term.
+    Returns (output [B, D, L] in x1v.dtype, state [B, D, S, 2] float32) -- the state is what the reference
+    stores in inference_params.state_dict (engine.py:502).
+    """
+    B, Dch, L = x1v.shape
+    S = poles.shape[1]
+    lanes = x1v[..., None, None].repeat(1, 1, 1, S, 2)         # [B, D, L, S, 2]
+    lanes[..., 1] = 0
+    state = 0 * lanes[:, :, 0]                                 # [B, D, S, 2], activations' dtype
+    out = 0 * lanes[:, :, :, 0, 0]                             # [B, D, L]
+    p = poles[:, :, 0][None]                                   # [1, D, S, 2]
+    r = residues[:, :, 0][None].repeat(B, 1, 1, 1)             # [B, D, S, 2]
+    for i in range(L):
+        state[..., 0] = p[..., 0] * state[..., 0] - p[..., 1] * state[..., 1] + lanes[:, :, i, :, 0]
+        state[..., 1] = p[..., 0] * state[..., 1] + p[..., 1] * state[..., 0] + lanes[:, :, i, :, 1]
+        out[:, :, i] = torch.sum(r * state, dim=-2)[..., 0]
+    return out, state.to(torch.float32)
 
 
 # --------------------------------------------------------------------------
@@ -641,8 +681,11 @@ class OracleCascade:
     """
 
     def __init__(self, engine, params, hidden, n_heads, groups, layer_idx=0, fir_inner_filter_length=None,
-                 column_split_hyena=False, interleave=False, state_size=16, long_fir_threshold=None):
+                 column_split_hyena=False, interleave=False, state_size=16, long_fir_threshold=None,
+                 hyena_flip_x1x2=None):
         self.long_fir_threshold = long_fir_threshold            # model.py:185
+        # model.py:141 and :159 read the same config key into the module and into its engine
+        self.hyena_flip_x1x2 = getattr(engine, "hyena_flip_x1x2", False) if hyena_flip_x1x2 is None else hyena_flip_x1x2
         self.engine, self.p = engine, params
         self.hidden, self.n_heads, self.groups = hidden, n_heads, groups
         self.layer_idx, self.K = layer_idx, fir_inner_filter_length
@@ -703,6 +746,8 @@ class OracleCascade:
         hd = self.hidden // self.n_heads
         x2, x1, v = (column_split(z_pre, self.n_heads, hd) if self.column_split_hyena
                      else z_pre.split([self.hidden] * 3, dim=1))
+        if self.hyena_flip_x1x2:                                                            # model.py:342-343
+            x1, x2 = x2, x1
         if self.K is not None:
             h = p["h"].repeat_interleave(self.hidden // self.groups, 0) if self.groups > 1 else p["h"]
             y, inner = self.engine.step_fir(x1 * v, inference_params.fir_inner_state_dict[self.layer_idx], weight=h,

@@ -241,18 +241,20 @@ def test_operator_module_small_state_sizes(S, bias, L):
             assert rel_err(y_hip, y_ref) <= 2e-2, (fused, i)
 
 
+@pytest.mark.parametrize("flip", [False, True])
 @pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("kind,cs,il", [("se", False, True), ("mr", False, True), ("mr", True, False),
                                          ("li_cplx", False, True), ("li_real", True, False), ("se", False, False),
                                          ("li_real", False, False), ("mr", True, True)])
-def test_operator_module_prefill_then_decode(kind, cs, il, fused):
-    # vortex_amd.cascade.HyenaCascade (fused fast path) against the oracle call sequence
+def test_operator_module_prefill_then_decode(kind, cs, il, fused, flip):
+    # vortex_amd.cascade.HyenaCascade (fused fast path) against the oracle call sequence, with and without
+    # hyena_flip_x1x2 (vortex/model/model.py:342-343, engine.py:157-158, :309-310)
     B, L, D, H, n_dec = 2, 512, 64, 4, 4
     K = {"se": 7, "mr": 128}.get(kind)
     G = 4
     p = make_params(kind, D, G, seed=11)
     cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=cs, interleave=il, short_filter_length=3,
-               short_filter_bias=False, state_size=16)
+               short_filter_bias=False, state_size=16, hyena_flip_x1x2=flip)
     mod = HyenaCascade(cfg, 0, hyena_filter_groups=G, fir_inner_filter_length=K, complex_modal=(kind == "li_cplx"))
     with torch.no_grad():
         mod.short_filter_weight.copy_(p["short_filter_weight"])
@@ -268,10 +270,11 @@ def test_operator_module_prefill_then_decode(kind, cs, il, fused):
     if K is None:     # oracle needs per-channel modal parameters
         pr = dict(p, log_poles=p["log_poles"].repeat_interleave(D // G, 0),
                   residues=p["residues"].repeat_interleave(D // G, 0))
-        ref = O.OracleCascade(O.OracleEngine(), pr, D, H, D, column_split_hyena=cs, interleave=il)
+        ref = O.OracleCascade(O.OracleEngine(hyena_flip_x1x2=flip), pr, D, H, D, column_split_hyena=cs, interleave=il)
     else:
-        ref = O.OracleCascade(O.OracleEngine(), p, D, H, G, fir_inner_filter_length=K, column_split_hyena=cs,
-                              interleave=il)
+        ref = O.OracleCascade(O.OracleEngine(hyena_flip_x1x2=flip), p, D, H, G, fir_inner_filter_length=K,
+                              column_split_hyena=cs, interleave=il)
+    assert ref.hyena_flip_x1x2 == flip
     g = torch.Generator().manual_seed(3)
     u_all = torch.randn(B, L + n_dec, 3 * D, generator=g).bfloat16()
     ip_ref = O.OracleCache()
@@ -523,7 +526,8 @@ def test_operator_module_truncated_fir_config(T, G):
 def test_engine_parallel_iir_recurrence_prefill_seam(cplx, L):
     # prefill_style="recurrence" (vortex/model/engine.py:314-321, :473-504): poles themselves and residues arrive as
     # [D, S, 1, 2] (re, im) lanes, one filter per channel; the state comes back as [B, D, S, 2] float32.  Checked
-    # against the explicit recurrence in float64 (what that branch evaluates, without its bf16 state rounding).
+    # against the explicit recurrence in float64 (what that branch evaluates, without its bf16 state rounding) and,
+    # for real poles, against the literal restatement of the reference's loop.
     B, D, H, S = 2, 16, 2, 16
     g = torch.Generator().manual_seed(L)
     lp, r = (O.make_modal_complex if cplx else O.make_modal_real)(D, S, seed=L, pmax=0.99)
@@ -548,6 +552,14 @@ def test_engine_parallel_iir_recurrence_prefill_seam(cplx, L):
     assert st.shape == (B, D, S, 2) and st.dtype == torch.float32
     s_ref = torch.view_as_real(s64.to(torch.complex128)) if cplx else torch.stack([s64, torch.zeros_like(s64)], -1)
     assert rel_err(st, s_ref) <= 1e-4
+    if not cplx:
+        # distance to the reference's loop as it is written (bf16 state, rounded every step): with real poles its
+        # other two quirks vanish.  The loop itself is 9e-3 (output) and 1.4e-2 (state) away from the exact
+        # recurrence on these inputs; the kernel, which carries the state in float32, stays within 2e-2 / 3e-2 of it.
+        y_lit, s_lit = O.prefill_direct_recurrence_ref(x1v, poles, residues)
+        y_lit = ((y_lit + x1v * Db[:, None]) * x2).permute(0, 2, 1)
+        assert rel_err(y, y_lit) <= 2e-2
+        assert rel_err(st, s_lit) <= 3e-2
     with pytest.raises(ValueError):
         eng.parallel_iir(z_pre.to(DEV), None, Db.to(DEV), L, lp.to(DEV), r.to(DEV), None, dims, 3,
                          inference_params=HyenaCascadeIIRInferenceParams(), prefill_style="recurrence")

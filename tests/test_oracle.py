@@ -453,3 +453,163 @@ def test_inner_hyena_se_ref_vs_bruteforce_and_layouts(K, path):
     y3 = O.inner_hyena_se_ref(x.reshape(B, G, dg, L), k.reshape(B, G, dg, L), q.reshape(B, G, dg, L), h, bias=bias,
                               input_layout="bgdgl", output_layout="bld", kernel_path=path)
     assert torch.equal(y3, y.permute(0, 2, 1))
+
+
+# --------------------------------------------------------------------------
+# OracleCascade: the operator module's call sequence (vortex/model/model.py:214-375)
+# --------------------------------------------------------------------------
+
+def _cascade_params(kind, D, seed, Ks=3, identity_featurizer=False):
+    g = torch.Generator().manual_seed(seed)
+    wf = torch.randn(3 * D, 1, Ks, generator=g) / Ks ** 0.5
+    if identity_featurizer:
+        wf = torch.zeros(3 * D, 1, Ks)
+        wf[..., Ks - 1] = 1.0
+    p = {"short_filter_weight": wf, "short_filter_bias": None}
+    if kind == "se":
+        p["h"], p["D"] = O.make_se_filter(D // 2, 7, seed=seed), None
+    elif kind == "mr":
+        p["h"], p["D"] = O.make_mr_filter(D // 2, 128, seed=seed), torch.randn(D, generator=g).bfloat16()
+    else:
+        p["log_poles"], p["residues"] = O.make_modal_real(D, 4, seed=seed, pmax=0.99)
+        p["D"] = torch.randn(D, generator=g).bfloat16()
+    return p
+
+
+def _make_cascade(kind, p, D, H, cs, il, flip):
+    K = {"se": 7, "mr": 128}.get(kind)
+    G = D // 2 if K else D
+    return O.OracleCascade(O.OracleEngine(hyena_flip_x1x2=flip), p, D, H, G, fir_inner_filter_length=K,
+                           column_split_hyena=cs, interleave=il, state_size=4, hyena_flip_x1x2=flip)
+
+
+@pytest.mark.parametrize("flip", [False, True])
+@pytest.mark.parametrize("il", [False, True])
+@pytest.mark.parametrize("cs", [False, True])
+@pytest.mark.parametrize("kind,L", [("se", 40), ("mr", 150), ("mr", 20), ("li", 64)])
+def test_oracle_cascade_prefill_equals_prefill_plus_steps(kind, L, cs, il, flip):
+    # what the mathematics fixes for the whole call sequence: a causal operator evaluated on L+n tokens at once
+    # equals its evaluation on L tokens followed by n one-token calls, outputs and caches alike.  A wrong split,
+    # a missing flip on either branch, a wrong tap orientation or state hand-off breaks it.
+    B, D, H, n = 2, 8, 2, 5
+    p = _cascade_params(kind, D, seed=70 + L)
+    u = torch.randn(B, L + n, 3 * D, generator=torch.Generator().manual_seed(L)).bfloat16()
+    full = _make_cascade(kind, p, D, H, cs, il, flip)
+    ip_full = O.OracleCache()
+    y_full, _ = full.forward(u, ip_full)
+    inc = _make_cascade(kind, p, D, H, cs, il, flip)
+    ip = O.OracleCache()
+    y0, _ = inc.forward(u[:, :L], ip)
+    scale = y_full.float().abs().max()
+    assert (y0.float() - y_full[:, :L].float()).abs().max() <= 1e-2 * scale
+    for i in range(n):
+        yi, _ = inc.forward(u[:, L + i:L + i + 1], ip)
+        assert yi.shape == (B, 1, D) and yi.dtype == u.dtype
+        assert (yi[:, 0].float() - y_full[:, L + i].float()).abs().max() <= 2e-2 * scale, i
+    # featurizer cache: the last Ks-1 projection rows, exactly
+    assert torch.equal(ip.fir_state_dict[0].float(), ip_full.fir_state_dict[0].float())
+    if kind == "li":
+        a, b = ip.state_dict[0].double(), ip_full.state_dict[0].double()
+        assert (a - b).abs().max() <= 1e-3 * b.abs().max()
+    else:
+        a, b = ip.fir_inner_state_dict[0].float(), ip_full.fir_inner_state_dict[0].float()
+        assert a.shape == b.shape
+        assert (a - b).abs().max() <= 2 ** -7 * b.abs().max()          # x1*v of featurizer outputs: one bf16 ulp
+
+
+def _expected_role(j, D, H, cs, il, flip):
+    """(role, channel) a projection channel j ends up as, written from the definitions: interleave sends channel
+    3c+i to block i (vortex/model/utils.py:26-38); the plain split cuts [x2 | x1 | v] blocks of D; the column split
+    cuts each head's 3*hd channels into [x2 | x1 | v] (utils.py:41-85); the flip swaps the x1 and x2 roles."""
+    hd = D // H
+    if il:
+        j = (j % 3) * D + j // 3
+    if cs:
+        head, within = divmod(j, 3 * hd)
+        role, c = within // hd, head * hd + within % hd
+    else:
+        role, c = divmod(j, D)
+    if flip and role in (0, 1):
+        role = 1 - role
+    return role, c
+
+
+@pytest.mark.parametrize("flip", [False, True])
+@pytest.mark.parametrize("il", [False, True])
+@pytest.mark.parametrize("cs", [False, True])
+def test_oracle_cascade_index_known_answer(cs, il, flip):
+    # identity featurizer, inner filter = one-sample delay: y[c, t] = x2[c, t] * x1[c, t-1] * v[c, t-1].  All inputs 1
+    # except projection channel j, which is 2 at one time step: the 2 shows up in y at that step if j is an x2
+    # channel and one step later if it is an x1 or v channel -- on the prefill branch and on the decode branch.
+    D, H, Ks, L = 8, 2, 3, 6
+    C = 3 * D
+    p = _cascade_params("se", D, seed=1, Ks=Ks, identity_featurizer=True)
+    h = torch.zeros(D // 2, 1, 7)
+    h[..., 5] = 1.0                                     # tap K-2 multiplies the previous sample
+    p["h"] = h
+    t0 = 3
+    u = torch.ones(C, L + 3, C).bfloat16()              # batch element j carries the mark on channel j
+    for j in range(C):
+        u[j, t0, j] = 2.0
+        u[j, L + 1, j] = 2.0                            # and again on the second decode step
+    mod = _make_cascade("se", p, D, H, cs, il, flip)
+    ip = O.OracleCache()
+    y, _ = mod.forward(u[:, :L], ip)
+    steps = [mod.forward(u[:, L + i:L + i + 1], ip)[0][:, 0] for i in range(3)]
+    for j in range(C):
+        role, c = _expected_role(j, D, H, cs, il, flip)
+        want = torch.ones(L, D)
+        want[0] = 0                                     # no history at t = 0
+        want[t0 if role == 0 else t0 + 1, c] = 2.0
+        assert torch.equal(y[j].float(), want), (j, role, c)
+        for i in range(3):
+            w = torch.ones(D)
+            if (role == 0 and i == 1) or (role != 0 and i == 2):
+                w[c] = 2.0
+            assert torch.equal(steps[i][j].float(), w), (j, role, c, i)
+
+
+def test_prefill_direct_recurrence_ref_hand_computed():
+    # three steps by hand.  (1) bf16 state: p = 1 + 2^-8, r = 1, u = 1, 1, 1 in bf16: s = 1; then 2.00390625 which a
+    # bf16 state rounds to 2; then p*2 + 1 = 3.0078125, a tie that rounds to even, 3 (a float32 state would give
+    # 2.0039 and 3.0117, i.e. an output of 3.015625 after the cast).
+    p = torch.tensor([1.0 + 2.0 ** -8, 0.0]).reshape(1, 1, 1, 2)
+    r = torch.tensor([1.0, 0.0]).reshape(1, 1, 1, 2)
+    u = torch.ones(1, 1, 3).bfloat16()
+    y, s = O.prefill_direct_recurrence_ref(u, p, r)
+    assert y.dtype == torch.bfloat16 and s.dtype == torch.float32 and s.shape == (1, 1, 1, 2)
+    assert y.flatten().tolist() == [1.0, 2.0, 3.0]
+    assert s.flatten().tolist() == [3.0, 0.0]
+    # (2) the in-place lane update and the lane-0 output with p = i, r = 1 + 5i, u = 1, 0, 0 in float32: the new real
+    # lane feeds the imaginary one, so (s_re, s_im) = (1, 1), (-1, -1), (1, 1) where the complex product gives
+    # (1, 0), (0, 1), (-1, 0); y = r_re * s_re = 1, -1, 1 where Re(r s) = 1, -5, -1.
+    p = torch.tensor([0.0, 1.0]).reshape(1, 1, 1, 2)
+    r = torch.tensor([1.0, 5.0]).reshape(1, 1, 1, 2)
+    u = torch.tensor([1.0, 0.0, 0.0]).reshape(1, 1, 3)
+    y, s = O.prefill_direct_recurrence_ref(u, p, r)
+    assert y.flatten().tolist() == [1.0, -1.0, 1.0]
+    assert s.flatten().tolist() == [1.0, 1.0]
+    # (3) two modes and two channels, real poles, float32: y = sum_s r_s * s_s by hand
+    p = torch.tensor([[0.5, 0.25], [0.0, 1.0]])[..., None, None].repeat(1, 1, 1, 2)
+    p[..., 1] = 0
+    r = torch.tensor([[2.0, 4.0], [1.0, -1.0]])[..., None, None].repeat(1, 1, 1, 2)
+    u = torch.tensor([[1.0, 1.0, 0.0], [1.0, 2.0, 3.0]])[None]
+    y, s = O.prefill_direct_recurrence_ref(u, p, r)
+    # channel 0: s = (1, 1), (1.5, 1.25), (0.75, 0.3125) -> y = 6, 8, 2.75;  channel 1: s = (1, 1), (2, 3), (3, 6)
+    assert y[0].tolist() == [[6.0, 8.0, 2.75], [0.0, -1.0, -3.0]]
+    assert s[0, :, :, 0].tolist() == [[0.75, 0.3125], [3.0, 6.0]]
+
+
+def test_prefill_direct_recurrence_ref_is_the_recurrence_for_real_poles_in_float32():
+    # with real poles and float32 activations none of the loop's three quirks acts: it is the plain recurrence
+    B, D, S, L = 2, 3, 4, 40
+    g = torch.Generator().manual_seed(81)
+    lp, res = O.make_modal_real(D, S, seed=82, pmax=0.99)
+    u = torch.randn(B, D, L, generator=g)
+    p4 = torch.stack([lp[..., 0].exp(), torch.zeros(D, S)], -1)[:, :, None]
+    r4 = torch.stack([res, torch.zeros(D, S)], -1)[:, :, None]
+    y, s = O.prefill_direct_recurrence_ref(u, p4, r4)
+    y64, s64 = O.prefill_direct_recurrence(u, lp, res)
+    assert (y.double() - y64).abs().max() <= 1e-5 * y64.abs().max()
+    assert (s[..., 0].double() - s64).abs().max() <= 1e-5 * s64.abs().max()
+    assert s[..., 1].abs().max() == 0
