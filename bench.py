@@ -43,13 +43,8 @@ def parse():
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-model", action="store_true", help="skip the end-to-end model prefill legs")
-    ap.add_argument("--copy-probe", action="store_true",
-                    help="also run a plain 1 GiB device copy (calibration of FETCH_SIZE / WRITE_SIZE counters)")
-    ap.add_argument("--li-cached-inputs", action="store_true",
-                    help="also time Hyena-LI at config 3 with its reads served from cache (the kernel's own pace)")
-    ap.add_argument("--pattern-probes", action="store_true",
-                    help="also stream the bytes of the Hyena-LI configuration with no arithmetic in several access "
-                         "orders (whole rows, independent segments) and print what each delivers to stderr")
+    ap.add_argument("--no-copy-probe", action="store_true",
+                    help="skip the plain 1 GiB device copy whose rate is reported as roofline.copy_probe_gbs")
     return ap.parse_args()
 
 
@@ -201,9 +196,31 @@ def build_workload(name, device):
     raise ValueError(name)
 
 
+def _decode_figures(us, algorithmic_bytes, moved_bytes=None):
+    """Figures of one decode kernel or layer set.  A roofline fraction is only formed from bytes the timed launches
+    really move: `frac` where they run the reference's algorithm (whole cache, state on every token), otherwise
+    `frac_of_bytes_moved` from the average bytes per token of the windowed forms."""
+    d = dict(us=us, launch_bound=us < 10.0)
+    if moved_bytes is None:
+        gbs = algorithmic_bytes / (us * 1e-6) / 1e9
+        d.update(bytes=algorithmic_bytes, hbm_gbs=gbs, frac=gbs / HBM_PEAK_GBS)
+    else:
+        gbs = moved_bytes / (us * 1e-6) / 1e9
+        d.update(bytes_moved_per_token=moved_bytes, moved_gbs=gbs, frac_of_bytes_moved=gbs / HBM_PEAK_GBS,
+                 reference_algorithm_bytes=algorithmic_bytes)
+    return d
+
+
 def decode_layer_set(D, device, steps, warmup):
-    """One [SE, MR, LI] layer set of cached decode at batch 64: three fused launches per token."""
+    """One [SE, MR, LI] layer set of cached decode at batch 64: three fused launches per token.
+
+    Timed twice: with the kernels that run the reference's algorithm (the whole FIR cache read and the modal state
+    read and written on every token; SURVEY's algorithmic bytes are exactly what these move, so their rate is a
+    bandwidth and `frac_reference_algorithm` is the roofline figure), and with the steps the steppers bind by default
+    (far sums for the deep cache, the modal state in windows of four tokens), which move fewer bytes per token: for
+    those the headline is `us_per_step`, and the fraction is taken of the bytes they move."""
     import vortex_amd as va
+    from vortex_amd import ops
     O = _Synthetic
     B, S = 64, 16
     g = torch.Generator(device=device).manual_seed(6)
@@ -219,70 +236,76 @@ def decode_layer_set(D, device, steps, warmup):
     state = torch.zeros(B, D, S, dtype=torch.complex64, device=device)
     Dli = rnd(D).to(torch.bfloat16)
     step = va.DecodeLayerSet(ring_se, w_se, ring_mr, w_mr, Dmr, state, poles, res, Dli)
+    # the same set on caches of its own with the reference's algorithm in every kernel
+    ref = va.DecodeLayerSet(va.FirRing(rnd(B, 6, D).to(torch.bfloat16)), w_se, va.FirRing(rnd(B, 127, D).to(torch.bfloat16)),
+                            w_mr, Dmr, torch.zeros_like(state), poles, res, Dli, window_state=False, far_sums=False)
 
-    def fn():
-        step(x[0], x[1], x[2])
-
-    wall, ms = time_steps(fn, steps, warmup)
+    wall, ms = time_steps(lambda: step(x[0], x[1], x[2]), steps, warmup)
+    _, ms_ref = time_steps(lambda: ref(x[0], x[1], x[2]), steps, warmup)
     # algorithmic bytes: caches read once, one ring slot written per FIR, modal state read+written,
     # 3 gate vectors in and 1 output vector out per operator
     gates_io = 4 * B * D * 2
     b_se, b_mr, b_li = B * D * 2 * 6 + B * D * 2 + gates_io, B * D * 2 * 127 + B * D * 2 + gates_io, \
         2 * state.numel() * 8 + gates_io
     byts = b_se + b_mr + b_li
+    # bytes the windowed forms move per token on average
+    m_mr, m_li, n_mr, n_li = b_mr, b_li, None, None
+    if step.mr.far is not None:
+        # far sums: the whole cache every n-th token: per token about (127 / n + (n - 1) / 2) slots, the far buffer
+        # (n - 1 float32 rows written per window, one read on n - 1 of n tokens) and the gates
+        n_mr = step.mr.far.numel() // (B * D)
+        m_mr = B * D * 2 * (127 / n_mr + (n_mr - 1) / 2) + B * D * 4 * 2 * (n_mr - 1) / n_mr + B * D * 2 + gates_io
+    if step.li.win is not None:
+        # windows of n tokens: 1/n of the state traffic per token, a far row (float32) written on n - 1 tokens of n by
+        # the window's first token and read once each, the window's inputs (bf16: one row written per token,
+        # (n + n (n - 1) / 2) / n rows read)
+        n_li = step.li.period
+        m_li = 2 * state.numel() * 8 / n_li + B * D * 4 * 2 * (n_li - 1) / n_li \
+            + B * D * 2 * (1 + (n_li + n_li * (n_li - 1) / 2) / n_li) + gates_io
+    moved = b_se + m_mr + m_li
     # each step alone, launched back to back: kernels shorter than a launch (about 6 us from Python) read as the
     # launch rate, so `launch_bound` marks figures that are an upper bound of the kernel's own duration
     per = {}
-    # the Hyena-MR step as the reference's algorithm has it (the whole cache read every token), on a cache of its own
-    from vortex_amd import ops
-    mr_plain = ops.FirStepper(va.FirRing(rnd(B, 127, D).to(torch.bfloat16)), w_mr, bias=Dmr, gated_bias=True, far_sums=False)
-    # and the Hyena-LI step that reads and writes the modal state on every token, on a state of its own
-    li_plain = ops.IirStepper(torch.zeros_like(state), poles, res, Dli)
-    for nm, st, xx, bb in (("se_step", step.se, x[0], b_se), ("mr_step", step.mr, x[1], b_mr),
-                           ("mr_step_whole_cache", mr_plain, x[1], b_mr), ("iir_step", step.li, x[2], b_li),
-                           ("iir_step_state_every_token", li_plain, x[2], b_li)):
-        o = step.out[0]
+    o = step.out[0]
+    for nm, st, xx, alg, mv in (("se_step", step.se, x[0], b_se, None),
+                                ("mr_step_whole_cache", ref.mr, x[1], b_mr, None),
+                                ("iir_step_state_every_token", ref.li, x[2], b_li, None),
+                                ("mr_step_far_sums", step.mr, x[1], b_mr, m_mr if n_mr else None),
+                                ("iir_step_windowed_state", step.li, x[2], b_li, m_li if n_li else None)):
         _, kms = time_steps(lambda: st(xx[1], xx[0], xx[2], o), max(steps, 100), warmup)
-        per[nm] = dict(us=kms * 1e3, bytes=bb, hbm_gbs=bb / (kms * 1e-3) / 1e9, frac=bb / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                       launch_bound=kms * 1e3 < 10.0)
-    if step.mr.far is not None:
-        # The shipped Hyena-MR step keeps far sums and reads its whole cache only every n-th token: per token about
-        # (127 / n + (n - 1) / 2) slots, the far buffer (n - 1 rows written per window, one read on n - 1 of n tokens)
-        # and the gates.  Its `bytes`, `hbm_gbs` and `frac` above stay those of the reference's algorithm (what a token
-        # costs a kernel that reads the cache whole), so they are a rate of algorithmic bytes, not a bandwidth.
-        n = step.mr.far.numel() // (B * D)
-        moved = B * D * 2 * (127 / n + (n - 1) / 2) + B * D * 4 * 2 * (n - 1) / n + B * D * 2 + gates_io
-        per["mr_step"].update(bytes_moved_per_token=moved, moved_gbs=moved / (per["mr_step"]["us"] * 1e-6) / 1e9,
-                              window_tokens=n, note="bytes / hbm_gbs / frac are algorithmic (whole cache per token); "
-                              "the kernel moves bytes_moved_per_token on average")
-    if step.li.win is not None:
-        # The shipped Hyena-LI step keeps the state in windows of n tokens: per token 1/n of the state traffic, a far
-        # row (float32) written on n - 1 tokens of n by the window's first token and read once each, and the window's
-        # inputs (bf16: one row written per token, (n + n (n - 1) / 2) / n rows read).  `bytes` stays algorithmic.
-        n = step.li.period
-        moved = 2 * state.numel() * 8 / n + B * D * 4 * 2 * (n - 1) / n + B * D * 2 * (1 + (n + n * (n - 1) / 2) / n) + gates_io
-        per["iir_step"].update(bytes_moved_per_token=moved, moved_gbs=moved / (per["iir_step"]["us"] * 1e-6) / 1e9,
-                               window_tokens=n, note="bytes / hbm_gbs / frac are algorithmic (state read and written per "
-                               "token); the kernel moves bytes_moved_per_token on average")
+        per[nm] = _decode_figures(kms * 1e3, alg, mv)
+    if n_mr:
+        per["mr_step_far_sums"]["window_tokens"] = n_mr
+    if n_li:
+        per["iir_step_windowed_state"]["window_tokens"] = n_li
     # The same token step (three launches and the counter update) recorded once as a HIP graph and replayed: the ring
     # positions and the window counter then live in device memory (ops.RingClock).  Every cache is full and more
     # than a window of tokens has been stepped by now, which is what a recording needs.
     clock = ops.RingClock([ring_se, ring_mr] + ([step.li] if step.li.win is not None else []))
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        fn()
+        step(x[0], x[1], x[2])
         clock.advance()
     _, gms = time_steps(graph.replay, steps, warmup)
     clock.release()
-    return dict(us_per_step=ms * 1e3, wall_us_per_step=wall / steps * 1e6, bytes=byts,
-                hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                us_per_step_graph_replay=gms * 1e3, frac_graph_replay=byts / (gms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+    ref_gbs = byts / (ms_ref * 1e-3) / 1e9
+    return dict(us_per_step=ms * 1e3, wall_us_per_step=wall / steps * 1e6, us_per_step_graph_replay=gms * 1e3,
+                what="us_per_step: far-sum Hyena-MR step + modal state in windows (fewer bytes per token than the "
+                     "reference's algorithm; not a bandwidth).  reference_algorithm: whole cache and state on every "
+                     "token; its bytes are the algorithmic ones, so its frac is the roofline figure",
+                bytes_moved_per_token=moved, moved_gbs=moved / (ms * 1e-3) / 1e9,
+                frac_of_bytes_moved=moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                reference_algorithm=dict(us_per_step=ms_ref * 1e3, bytes=byts, hbm_gbs=ref_gbs,
+                                         frac=ref_gbs / HBM_PEAK_GBS),
+                frac_reference_algorithm=ref_gbs / HBM_PEAK_GBS,
                 kernels=per)
 
 
 def decode_layers_from_projection(D, device, steps, warmup):
     """The same layer set stepped from each layer's projection output u [B, 3D] (Evo 2 layout: interleaved
-    gates, K=3 featurizer): featurizer step, split, gates and inner step in one launch per layer."""
+    gates, K=3 featurizer): featurizer step, split, gates and inner step in one launch per layer.  As in
+    decode_layer_set, once with the reference's algorithm in the inner steps (the roofline figure) and once with the
+    far-sum / windowed steps the steppers bind by default (the time per token)."""
     import vortex_amd as va
     from vortex_amd import ops
     O = _Synthetic
@@ -292,22 +315,29 @@ def decode_layers_from_projection(D, device, steps, warmup):
     G = D // 16
     cmap = ops.gate_channel_map(D, interleave=True)
     lp, r = O.make_modal_complex(G, S)
-    state = torch.zeros(B, D, S, dtype=torch.complex64, device=device)
-    inner = [ops.FirStepper(va.FirRing(rnd(B, 6, D).to(torch.bfloat16)), rnd(G, 7) * 7 ** -0.5),
-             ops.FirStepper(va.FirRing(rnd(B, 127, D).to(torch.bfloat16)), rnd(G, 128) * 128 ** -0.5, bias=rnd(D),
-                            gated_bias=True),
-             ops.IirStepper(state, torch.exp(lp[..., 0]).to(device), r.to(device), rnd(D).to(torch.bfloat16),
-                            windowed=True)]
-    frings = [va.FirRing(rnd(B, 2, C).to(torch.bfloat16)) for _ in inner]
-    layers = [ops.LayerStepper(fr, rnd(C, 3) * 3 ** -0.5, None, cmap, n) for fr, n in zip(frings, inner)]
+    w_se, w_mr, b_mr, d_li = rnd(G, 7) * 7 ** -0.5, rnd(G, 128) * 128 ** -0.5, rnd(D), rnd(D).to(torch.bfloat16)
+    wf = [rnd(C, 3) * 3 ** -0.5 for _ in range(3)]
     u = [rnd(B, C).to(torch.bfloat16) for _ in range(3)]
     out = [torch.empty(B, D, dtype=torch.bfloat16, device=device) for _ in range(3)]
 
-    def fn():
-        for l, x, o in zip(layers, u, out):
-            l(x, o)
+    def make(shipped):
+        state = torch.zeros(B, D, S, dtype=torch.complex64, device=device)
+        inner = [ops.FirStepper(va.FirRing(rnd(B, 6, D).to(torch.bfloat16)), w_se),
+                 ops.FirStepper(va.FirRing(rnd(B, 127, D).to(torch.bfloat16)), w_mr, bias=b_mr, gated_bias=True,
+                                far_sums=None if shipped else False),
+                 ops.IirStepper(state, torch.exp(lp[..., 0]).to(device), r.to(device), d_li, windowed=shipped)]
+        frings = [va.FirRing(rnd(B, 2, C).to(torch.bfloat16)) for _ in inner]
+        layers = [ops.LayerStepper(fr, w, None, cmap, n) for fr, w, n in zip(frings, wf, inner)]
 
+        def fn():
+            for l, xx, o in zip(layers, u, out):
+                l(xx, o)
+        return fn, inner, frings, state
+
+    fn, inner, frings, state = make(True)
+    fn_ref, _, _, _ = make(False)
     wall, ms = time_steps(fn, steps, warmup)
+    _, ms_ref = time_steps(fn_ref, steps, warmup)
     # inner caches / state as in decode_layer_set; per layer the projection row, two featurizer slots read and
     # one written (3D channels each) and one output row
     byts = B * D * 2 * (6 + 127) + 2 * B * D * 2 + 2 * state.numel() * 8 + 3 * (4 * B * C * 2 + B * D * 2)
@@ -319,9 +349,10 @@ def decode_layers_from_projection(D, device, steps, warmup):
         clock.advance()
     _, gms = time_steps(graph.replay, steps, warmup)
     clock.release()
-    return dict(us_per_step=ms * 1e3, wall_us_per_step=wall / steps * 1e6, bytes=byts,
-                hbm_gbs=byts / (ms * 1e-3) / 1e9, frac=byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                us_per_step_graph_replay=gms * 1e3, frac_graph_replay=byts / (gms * 1e-3) / 1e9 / HBM_PEAK_GBS)
+    ref_gbs = byts / (ms_ref * 1e-3) / 1e9
+    return dict(us_per_step=ms * 1e3, wall_us_per_step=wall / steps * 1e6, us_per_step_graph_replay=gms * 1e3,
+                reference_algorithm=dict(us_per_step=ms_ref * 1e3, bytes=byts, hbm_gbs=ref_gbs, frac=ref_gbs / HBM_PEAK_GBS),
+                frac_reference_algorithm=ref_gbs / HBM_PEAK_GBS)
 
 
 def model_prefill(device, L, iters=2):
@@ -477,68 +508,19 @@ def main():
         torch.cuda.empty_cache()
         return d
 
-    if args.copy_probe:
+    copy_gbs = None
+    if not args.no_copy_probe:
+        # the practical ceiling beside the nominal 8 TB/s: a plain device copy with the kernels' own access shape
+        # (16 bytes per lane), 1 GiB read + 1 GiB written per launch
+        from vortex_amd import _lib
         a = torch.empty(1 << 29, dtype=torch.bfloat16, device=device).normal_()
         b = torch.empty_like(a)
-        from vortex_amd import _lib
         stream = torch.cuda.current_stream().cuda_stream
         nbytes = a.numel() * 2
         probe = _lib.copy_probe()
-        wall, ms = time_steps(lambda: _lib.check(probe(a.data_ptr(), b.data_ptr(), nbytes, stream), "copy"), 5, 2)
-        print(f"copy probe (copy_probe_kernel, 16 B/lane): 1 GiB read + 1 GiB written per launch, "
-              f"{ms * 1e3:.1f} us, {2 * nbytes / (ms * 1e-3) / 1e9:.0f} GB/s", file=sys.stderr)
+        _, cms = time_steps(lambda: _lib.check(probe(a.data_ptr(), b.data_ptr(), nbytes, stream), "copy"), 10, 3)
+        copy_gbs = 2 * nbytes / (cms * 1e-3) / 1e9
         del a, b
-        torch.cuda.empty_cache()
-
-    if args.pattern_probes:
-        from vortex_amd import _lib
-        D, L = 4096, 262144
-        t = [torch.empty(D, L, dtype=torch.bfloat16, device=device).normal_() for _ in range(3)]
-        o = torch.empty(D, L, dtype=torch.bfloat16, device=device)
-        probe, stream = _lib.stream_probe(), torch.cuda.current_stream().cuda_stream
-        print(f"access-pattern probes: {D} rows of {L} bf16 samples, 3 reads + 1 write, no arithmetic", file=sys.stderr)
-        cases = [("whole rows, one block per 4 rows (a one-pass scan)", 0, 0)]
-        cases += [(f"whole rows, one block per row (4 wavefronts x 4 KiB per step), {256 * n} rows in flight", 2, n) for n in (8, 4, 2, 1)]
-        cases += [(f"independent segments of {s} samples, row sets in order", 1, s) for s in (65536, 16384, 8192, 4096, 2048)]
-        # each order twice: blocks dealt to the 8 XCDs in turn (every XCD touches every eighth block's memory), and XCD x
-        # taking the x-th eighth of the block order (pattern + 8), which is what the row kernels do for streaming shapes
-        for what, pat, seg in cases:
-            res = []
-            for xcd in (0, 8):
-                fn = lambda: _lib.check(probe(t[0].data_ptr(), t[1].data_ptr(), t[2].data_ptr(), o.data_ptr(), D, L,
-                                              pat + xcd, seg, stream), "stream probe")
-                _, ms = time_steps(fn, 5, 2)
-                res.append(f"{ms * 1e3:8.1f} us {8 * D * L / (ms * 1e-3) / 1e9:6.0f} GB/s")
-            print(f"  {what:75s} {res[0]}   XCD-contiguous: {res[1]}", file=sys.stderr)
-        del t, o
-        torch.cuda.empty_cache()
-
-    if args.li_cached_inputs:
-        # Hyena-LI at config 3 with every channel reading the same 16 rows (a row descriptor with row stride L and
-        # batch stride 0 over a 16-row tensor): the reads are served from cache, the 2.1 GB of output is still written.
-        # What is left is the kernel's own pace plus the write stream.
-        import vortex_amd as va
-        from vortex_amd import ops
-        from vortex_amd._lib import Rows
-        B, D, L, G = 1, 4096, 262144, 256
-        small = [torch.randn(16, L, device=device).to(torch.bfloat16) for _ in range(3)]
-        lp, r = _Synthetic.make_modal_complex(G, 16)
-        plan = va.ModalPlan(lp.to(device), r.to(device))
-        Db = torch.randn(D).to(torch.bfloat16).to(device)
-        out = torch.empty(B, D, L, dtype=torch.bfloat16, device=device)
-        rows = [Rows(t.data_ptr(), 0, L, 16, 0) for t in small]            # channel d -> row d % 16
-        full = gates(B, D, L, 4, device)
-        for what, rr in (("inputs from HBM", [ops.rows_of(t) for t in (full[1], full[0], full[2])]), ("inputs cached", rows)):
-            _, ms = time_steps(lambda: ops.li_fwd_rows(rr[0], rr[1], rr[2], plan, Db, B, D, L, device=device, out=out), 10, 3)
-            print(f"hyena_li_fwd config 3, {what}: {ms * 1e3:.1f} us", file=sys.stderr)
-        # the same rows with x1 holding x1*v already (two input streams, what hyena_featurizer_gates_fwd hands over) and
-        # ungated (one input stream)
-        x1v = full[1] * full[2]
-        rx, r2 = ops.rows_of(x1v), ops.rows_of(full[0])
-        for what, a2 in (("x1*v rows and x2 (6 bytes per sample)", r2), ("ungated, one input stream (4 bytes per sample)", None)):
-            _, ms = time_steps(lambda: ops.li_fwd_rows(rx, a2, None, plan, Db, B, D, L, device=device, out=out), 10, 3)
-            print(f"hyena_li_fwd config 3, {what}: {ms * 1e3:.1f} us", file=sys.stderr)
-        del small, full, out, x1v
         torch.cuda.empty_cache()
 
     main_name = args.workload if args.workload != "decode" else "mr"
@@ -550,7 +532,10 @@ def main():
         "vs_baseline": None, "dtype": "bf16 in/out, fp32 accumulate", "data": "synthetic",
         "config": {"workload": m["workload"], "settle_ms": args.settle_ms},
         "roofline": {"bound": "hbm", "achieved": m["hbm_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": m["hbm_gbs"] / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(main_name),
+                     "frac": m["hbm_gbs"] / HBM_PEAK_GBS, "copy_probe_gbs": copy_gbs,
+                     "copy_probe": "hyena_copy_probe: 1 GiB read + 1 GiB written per launch, 16 bytes per lane, timed "
+                                   "in this run; the rate a plain copy reaches beside the nominal peak",
+                     "traffic": MEASURED_TRAFFIC.get(main_name),
                      "traffic_source": TRAFFIC_SOURCE if MEASURED_TRAFFIC.get(main_name) else None,
                      "kernel": m["kernel"],
                      "algorithmic_bytes_per_launch": m["bytes"], "kernel_ms": m["kernel_ms"],

@@ -24,3 +24,20 @@ def test_one_json_line_with_roofline():
     rf = d["roofline"]
     assert rf["bound"] == "hbm" and rf["peak"] == 8000 and abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-9
     assert 0.3 < rf["frac"] < 1.0 and d["value"] > 5e7
+    assert 3000 < rf["copy_probe_gbs"] < rf["peak"]            # the measured plain-copy rate beside the nominal peak
+
+
+def test_decode_figures_never_exceed_the_peak():
+    """Every fraction the decode leg reports is a rate of bytes the timed launches really move: `frac` only for
+    the kernels that run the reference's algorithm, `frac_of_bytes_moved` for the far-sum / windowed steps."""
+    import torch
+    sys.path.insert(0, ROOT)
+    import bench
+    d = bench.decode_layer_set(4096, torch.device("cuda:0"), 20, 3)
+    assert "frac" not in d and d["us_per_step"] > 0 and d["reference_algorithm"]["us_per_step"] >= d["us_per_step"] * 0.9
+    assert 0.2 < d["frac_reference_algorithm"] < 1.0 and 0.05 < d["frac_of_bytes_moved"] < 1.0
+    for name, k in d["kernels"].items():
+        fr = k.get("frac", k.get("frac_of_bytes_moved"))
+        assert fr is not None and 0.0 < fr < 1.0, (name, k)
+        assert ("frac" in k) != ("frac_of_bytes_moved" in k), name
+    assert "frac_of_bytes_moved" in d["kernels"]["mr_step_far_sums"] and "frac" in d["kernels"]["mr_step_whole_cache"]

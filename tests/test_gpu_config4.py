@@ -167,3 +167,83 @@ def test_layer_step_full_shape(D, kind):
         order = ring.reference_order()
         # x1*v of featurizer outputs: the kernel's fp32 sums can land one bf16 ulp from the oracle's, so not bit-exact
         assert tiles_equal(order, D) and rel_err(order[:, :BASE], st_ref) <= 1e-2
+
+
+@pytest.mark.parametrize("D", [4096, 8192])
+def test_decode_layer_set_full_shape(D):
+    """The layer set as it is benchmarked (ops.DecodeLayerSet): the Hyena-SE step, the Hyena-MR step with far sums
+    (its cache read whole every third token) and the Hyena-LI step with the complex modal state in windows of four
+    tokens, 16 channels per filter, for 135 tokens: every output per element against O.step_fir / O.step_iir, the
+    caches bit for bit, the modal state after a flush in the middle of the run and at its end."""
+    g = torch.Generator().manual_seed(D + 4)
+    Gb, S, n_tok = BASE // 16, 16, 135
+    # Hyena-SE (7 taps, plain slicing) and Hyena-MR (128 taps, flipped, gated bias)
+    w_se = torch.randn(Gb, 1, 7, generator=g) / 7 ** 0.5
+    w_mr = O.make_mr_filter(Gb, 128, seed=D)
+    b_mr = torch.randn(BASE, generator=g)
+    st_se = torch.randn(B, BASE, 6, generator=g).bfloat16()
+    st_mr = torch.randn(B, BASE, 127, generator=g).bfloat16()
+    ring_se = va.FirRing.from_reference(tile(st_se, D).to(DEV))
+    ring_mr = va.FirRing.from_reference(tile(st_mr, D).to(DEV))
+    lp, r = O.make_modal_complex(Gb, S, seed=D + 1)
+    Dp = torch.randn(BASE, generator=g).bfloat16()
+    lpD, rD = lp.repeat_interleave(16, 0), r.repeat_interleave(16, 0)
+    st_li = torch.complex(torch.randn(B, BASE, S, generator=g), torch.randn(B, BASE, S, generator=g))
+    state = tile(st_li, D).contiguous().to(DEV)
+    step = ops.DecodeLayerSet(
+        ring_se, tile(w_se.reshape(Gb, 7), D // 16, dim=0).to(DEV),
+        ring_mr, tile(w_mr.reshape(Gb, 128).flip(-1).contiguous(), D // 16, dim=0).to(DEV), tile(b_mr, D, dim=0).to(DEV),
+        state, tile(torch.exp(lp[..., 0]), D // 16, dim=0).to(DEV), tile(r, D // 16, dim=0).to(DEV),
+        tile(Dp, D, dim=0).to(DEV), window_state=True)
+    assert step.mr.far is not None and step.se.far is None and step.li.win is not None
+    far_period = _lib.lib().hyena_fir_far_period(1)
+    wD_se, wD_mr = w_se.repeat_interleave(16, 0), w_mr.repeat_interleave(16, 0)
+    weff_mr = wD_mr[:, 0].flip(-1)
+    worst = 0.0
+
+    def state_ok(tok):
+        step.flush()
+        sv = torch.view_as_real(state)
+        assert tiles_equal(sv, D), tok
+        assert rel_err(sv[:, :BASE], torch.view_as_real(st_li)) <= 1e-4, tok
+
+    for tok in range(n_tok):
+        gates = [tuple(torch.randn(B, BASE, generator=g).bfloat16() for _ in range(3)) for _ in range(3)]    # (x2, x1, v)
+        outs = step(*[tuple(tile(t, D).to(DEV) for t in gt) for gt in gates])
+        # Hyena-SE
+        x2, x1, v = gates[0]
+        z_ref, new_se = O.step_fir(x1 * v, st_se, wD_se)
+        Sabs = (st_se.double().abs() * wD_se[None, :, 0, :6].double().abs()).sum(-1) + (wD_se[None, :, 0, 6] * (x1 * v).float()).abs()
+        assert tiles_equal(outs[0], D), tok
+        worst = max(worst, assert_gated_close(outs[0][:, :BASE], z_ref * x2, z_ref, x2, Sabs, 2.0 ** -16, what=f"se token {tok}"))
+        st_se = new_se
+        # Hyena-MR, far sums: windows staggered over the blocks with period 3
+        x2, x1, v = gates[1]
+        u = x1 * v
+        z_ref, new_mr = O.step_fir(u, st_mr, wD_mr, bias=b_mr, gated_bias=True, flip_filter=True)
+        Sabs = (st_mr.double().abs() * weff_mr[None, :, :127].double().abs()).sum(-1) + (weff_mr[None, :, 127] * u.float()).abs() \
+            + (b_mr[None] * u.float()).abs()
+        assert tiles_equal(outs[1], D, period=far_period), tok
+        for t in range(far_period):
+            worst = max(worst, assert_gated_close(outs[1][:, t * BASE:(t + 1) * BASE], z_ref * x2, z_ref, x2, Sabs,
+                                                  2.0 ** -16, what=f"mr token {tok} tile {t}"))
+        st_mr = new_mr
+        # Hyena-LI, windowed complex state
+        x2, x1, v = gates[2]
+        y_ref, st_li = O.step_iir(x2, x1, v, Dp, rD, lpD, st_li)
+        y_ref = y_ref.real.to(torch.bfloat16)
+        assert tiles_equal(outs[2], D), tok
+        assert rel_err(outs[2][:, :BASE], y_ref) <= 2e-2, tok
+        sabs = (rD[None].abs() * st_li.abs()).sum(-1).double()
+        err = (outs[2][:, :BASE].double().cpu() - y_ref.double()).abs()
+        x1v = (x1 * v).double()
+        bound = x2.double().abs() * (2.0 ** -16 * sabs + 2.0 ** -7 * (sabs + (Dp.double()[None] * x1v).abs())) \
+            + 2.0 ** -7 * y_ref.double().abs() + 1e-30
+        assert (err <= bound).all(), (tok, (err / bound).max())
+        if tok == 66:
+            state_ok(tok)
+    assert worst <= 1.0
+    state_ok(n_tok)
+    for ring, ref in ((ring_se, st_se), (ring_mr, st_mr)):
+        order = ring.reference_order()
+        assert tiles_equal(order, D) and torch.equal(order[:, :BASE].cpu(), ref.float())

@@ -258,3 +258,61 @@ def test_iir_step_windowed_state(cplx, B, D, G, fused, on_clock):
     assert (as_real(states[0]) - as_real(states[1])).abs().max() <= 1e-4 * sr.abs().max()
     if clock is not None:
         clock.release()
+
+
+def test_windowed_stepper_flush_around_a_recorded_step():
+    """A recorded token step (a HIP graph) replays the windowed modal step with "every window open" in its arguments.
+    A flush while that recording can still be replayed is refused; after release() the flush leaves the exact state,
+    eager steps continue the sequence, and a new recording after `period` eager steps replays correctly."""
+    from vortex_amd import _lib, ops
+    cplx, B, D, G, S = True, 64, 1024, 64, 16
+    W = _lib.lib().hyena_iir_window_tokens()
+    g = torch.Generator().manual_seed(77)
+    lp, r = O.make_modal_complex(G, S, seed=78)
+    Dp = torch.randn(D, generator=g).bfloat16()
+    lpD, rD = lp.repeat_interleave(D // G, 0), r.repeat_interleave(D // G, 0)
+    st_ref = (torch.randn(B, D, S, generator=g) * 0.5).to(torch.complex64)
+    state = st_ref.clone().cuda()
+    win = ops.IirStepper(state, torch.exp(lp[..., 0]).cuda(), r.cuda(), Dp.cuda(), windowed=True)
+    assert win.win is not None
+    gx = [torch.empty(B, D, dtype=torch.bfloat16, device="cuda") for _ in range(3)]     # x1, x2, v of the recording
+    y = torch.empty(B, D, dtype=torch.bfloat16, device="cuda")
+
+    def token(run):
+        nonlocal st_ref
+        x1, x2, v = (torch.randn(B, D, generator=g).bfloat16() for _ in range(3))
+        for dst, src in zip(gx, (x1, x2, v)):
+            dst.copy_(src)
+        run()
+        y_ref, st_ref = O.step_iir(x2, x1, v, Dp, rD, lpD, st_ref)
+        assert (y.float().cpu() - y_ref.real.float()).abs().max() <= 2e-2 * y_ref.real.abs().max()
+
+    def record():
+        clock = ops.RingClock([win])
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            win(gx[0], gx[1], gx[2], y)
+            clock.advance()
+        return clock, graph
+
+    eager = lambda: win(gx[0], gx[1], gx[2], y)
+    for _ in range(W + 1):
+        token(eager)
+    clock, graph = record()              # the capture runs no kernel and moves no counter
+    for _ in range(7):
+        token(graph.replay)
+    with pytest.raises(RuntimeError, match="recorded"):
+        win.flush()
+    clock.release()
+    win.flush()
+    sr = torch.view_as_real(st_ref)
+    assert (torch.view_as_real(state).cpu() - sr).abs().max() <= 1e-4 * sr.abs().max()
+    for _ in range(W + 2):
+        token(eager)
+    clock, graph = record()
+    for _ in range(6):
+        token(graph.replay)
+    clock.release()
+    win.flush()
+    sr = torch.view_as_real(st_ref)
+    assert (torch.view_as_real(state).cpu() - sr).abs().max() <= 1e-4 * sr.abs().max()

@@ -310,6 +310,8 @@ def test_operator_module_windowed_modal_state(kind, cs, il, fused):
         mod.D.data = p["D"].clone()
     mod = mod.to(DEV)
     mod.fuse_decode = mod.fuse_prefill = fused
+    assert mod.window_decode_state is False         # the reference keeps the state current: windows are opt-in
+    mod.window_decode_state = True
     pr = dict(p, log_poles=p["log_poles"].repeat_interleave(D // G, 0), residues=p["residues"].repeat_interleave(D // G, 0))
     ref = O.OracleCascade(O.OracleEngine(), pr, D, H, D, column_split_hyena=cs, interleave=il)
     n_dec = 11
@@ -334,6 +336,87 @@ def test_operator_module_windowed_modal_state(kind, cs, il, fused):
     assert rel_err(as_real(ip_hip.state_dict[0]), as_real(ip_ref.state_dict[0])) <= 1e-3
     mod.flush_decode_state()                               # nothing pending: no launch, same state
     assert rel_err(as_real(ip_hip.state_dict[0]), as_real(ip_ref.state_dict[0])) <= 1e-3
+
+
+@pytest.mark.parametrize("windowed", [False, True])
+def test_operator_module_serves_two_cache_objects_in_turn(windowed):
+    # one module, two sequences A and B with their own cache objects, decoded alternately (prefill A, steps on A,
+    # prefill B, steps on B, back to A, ...): every output and both final states against the oracle call sequence.
+    # With the windowed modal state the pending inputs live in the bound stepper, which has to leave a cache object's
+    # state complete whenever the module turns to another one.
+    B, D, H, G = 64, 1024, 8, 64
+    p = make_params("li_cplx", D, G, seed=21)
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=False, interleave=True, short_filter_length=3,
+               short_filter_bias=False, state_size=16)
+    mod = HyenaCascade(cfg, 0, hyena_filter_groups=G, complex_modal=True)
+    with torch.no_grad():
+        mod.short_filter_weight.copy_(p["short_filter_weight"])
+        mod.log_poles.copy_(p["log_poles"])
+        mod.residues.copy_(p["residues"])
+        mod.D.data = p["D"].clone()
+    mod = mod.to(DEV)
+    mod.window_decode_state = windowed
+    pr = dict(p, log_poles=p["log_poles"].repeat_interleave(D // G, 0), residues=p["residues"].repeat_interleave(D // G, 0))
+    ref = O.OracleCascade(O.OracleEngine(), pr, D, H, D, interleave=True)
+    g = torch.Generator().manual_seed(22)
+    seqs = {k: torch.randn(B, 8 + 16, 3 * D, generator=g).bfloat16() for k in "AB"}
+    caches = {k: (O.OracleCache(), HyenaCascadeIIRInferenceParams()) for k in "AB"}
+    used = {k: 0 for k in "AB"}
+
+    def run(k, n):
+        ip_ref, ip_hip = caches[k]
+        for _ in range(n):
+            a = used[k]
+            b = 8 if a == 0 else a + 1
+            u = seqs[k][:, a:b]
+            used[k] = b
+            y_ref, _ = ref.forward(u, ip_ref)
+            y_hip, _ = mod(u.to(DEV), ip_hip)
+            assert rel_err(y_hip, y_ref) <= 2e-2, (k, a)
+
+    for k, n in [("A", 4), ("B", 3), ("A", 3), ("B", 6), ("A", 5), ("B", 1), ("A", 1)]:
+        run(k, n)
+    if windowed:
+        from vortex_amd import ops
+        assert isinstance(mod._decode["inner"], ops.IirStepper) and mod._decode["inner"].win is not None
+    mod.flush_decode_state()
+    for k in "AB":
+        a, b = torch.view_as_real(caches[k][1].state_dict[0]), torch.view_as_real(caches[k][0].state_dict[0])
+        assert rel_err(a, b) <= 1e-3, k
+
+
+def test_operator_module_growing_cache_under_a_far_sum_stepper():
+    # an inner filter of 64 taps with the plain tap slicing (vortex/model/engine.py:424-425) and a prompt shorter than
+    # the filter: the reference grows its cache by one sample per token and shifts the taps with it.  A 63-slot cache
+    # is deep enough for the far-sum stepper, whose sums carry a token's taps into the next two outputs; the steps
+    # that grow the cache therefore have to read it whole.  Decode through the growth and well past it.
+    B, L, D, H, G, K, n_dec = 2, 20, 64, 4, 4, 64, 56
+    g = torch.Generator().manual_seed(41)
+    p = {"short_filter_weight": torch.randn(3 * D, 1, 3, generator=g) / 3 ** 0.5, "short_filter_bias": None,
+         "h": torch.randn(G, 1, K, generator=g) / K ** 0.5, "D": None}
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=False, interleave=True, short_filter_length=3,
+               short_filter_bias=False, state_size=16)
+    ref = O.OracleCascade(O.OracleEngine(), p, D, H, G, fir_inner_filter_length=K, interleave=True)
+    u_all = torch.randn(B, L + n_dec, 3 * D, generator=g).bfloat16()
+    from vortex_amd import ops
+    for fused in (True, False):
+        mod = HyenaCascade(cfg, 0, hyena_filter_groups=G, fir_inner_filter_length=K)
+        with torch.no_grad():
+            mod.short_filter_weight.copy_(p["short_filter_weight"])
+            mod.h.copy_(p["h"])
+        mod = mod.to(DEV)
+        mod.fuse_prefill = mod.fuse_decode = fused
+        ip_ref, ip_hip = O.OracleCache(), HyenaCascadeFIRInferenceParams()
+        y_ref, _ = ref.forward(u_all[:, :L], ip_ref)
+        y_hip, _ = mod(u_all[:, :L].to(DEV), ip_hip)
+        assert rel_err(y_hip, y_ref) <= 2e-2
+        for i in range(n_dec):
+            tok = u_all[:, L + i: L + i + 1]
+            y_ref, _ = ref.forward(tok, ip_ref)
+            y_hip, _ = mod(tok.to(DEV), ip_hip)
+            assert rel_err(y_hip, y_ref) <= 2e-2, (fused, i)
+        assert mod._decode["inner"].far is not None            # the far-sum stepper was the one bound
+        assert rel_err(ip_hip.fir_inner_state_dict[0].reference_order(), ip_ref.fir_inner_state_dict[0]) <= 2e-2
 
 
 @pytest.mark.parametrize("kind", ["se", "mr", "li_real"])

@@ -95,9 +95,7 @@ def test_windowed_modal_state_in_generation():
     want = m(ids).float()[:, L - 1:L + n - 1]
     err = (scores_e.float() - want).abs().max() / want.abs().max()
     assert err <= 3e-2, err
-    for blk in m.blocks:
-        blk.filter.window_decode_state = False
-    _, scores_p = m.generate(ids[:, :L], n, forced=ids[:, L:])
+    _, scores_p = m.generate(ids[:, :L], n, forced=ids[:, L:], window_state=False)
     assert m.blocks[2].filter._decode["inner"].win is None
     err = (scores_e.float() - scores_p.float()).abs().max() / want.abs().max()
     assert err <= 2e-2, err

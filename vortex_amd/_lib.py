@@ -160,17 +160,8 @@ def copy_probe():
         P = ctypes.CDLL(PROBE_PATH)
         P.hyena_copy_probe.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
         P.hyena_copy_probe.restype = c_int
-        P.hyena_stream_probe.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int64, c_void_p]
-        P.hyena_stream_probe.restype = c_int
         _probe = P
     return _probe.hyena_copy_probe
-
-
-def stream_probe():
-    """hyena_stream_probe of libhyena_probe.so: the bytes of a gated long convolution moved with no arithmetic in
-    the access order of a one-pass scan (pattern 0) or of independent segments (1); see csrc/stream_probes.hip."""
-    copy_probe()
-    return _probe.hyena_stream_probe
 
 
 def check(rc, what):

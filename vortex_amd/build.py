@@ -44,7 +44,7 @@ def build(verbose=True, jobs=4):
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(compile_one, srcs))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
-    _run([HIPCC] + FLAGS + ["-shared", os.path.join(CSRC, "copy_probe.hip"), os.path.join(CSRC, "stream_probes.hip"), "-o", PROBE])
+    _run([HIPCC] + FLAGS + ["-shared", os.path.join(CSRC, "copy_probe.hip"), "-o", PROBE])
     _run([HIPCC, "-O2", "-std=c++17", os.path.join(CSRC, "abi_selftest.cpp"), "-o", SELFTEST, "-ldl"])
     if verbose:
         print("built", LIB)

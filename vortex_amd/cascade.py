@@ -128,9 +128,10 @@ class HyenaCascade(nn.Module):
         self._plan = None
         self._decode = None
         self.fuse_decode = True        # one launch per decode step where the fused layer-step kernels apply
-        # decode: the modal state is read and written once per four tokens (ops.IirStepper windowed);
-        # inference_params.state_dict then lags the tokens by up to four inputs until flush_decode_state()
-        self.window_decode_state = True
+        # decode, opt-in: the modal state is read and written once per four tokens (ops.IirStepper windowed);
+        # inference_params.state_dict then lags the tokens by up to four inputs until flush_decode_state().
+        # Off by default: the reference leaves the state current after every token (vortex/model/model.py:362-372)
+        self.window_decode_state = False
         self.fuse_prefill = True       # one launch per SE / MR prefill where the fused layer kernel applies
         self._f32_cache = {}
 
@@ -271,7 +272,7 @@ class HyenaCascade(nn.Module):
                 _, x1, v = self._split(z_pre[..., max(L - (K - 1), pad):])
                 inference_params.fir_inner_state_dict[self.layer_idx] = _ring((x1 * v).permute(0, 2, 1), K - 1,
                                                                               flipped=K >= 128)
-            self._decode = None
+            self._drop_decode()
         if pad:
             y = y[..., pad:]
         return y.permute(0, 2, 1), inference_params
@@ -324,7 +325,7 @@ class HyenaCascade(nn.Module):
         if caching:
             inference_params.state_dict[self.layer_idx] = state
             inference_params.fir_state_dict[self.layer_idx] = _ring(u[:, max(L - (Ks - 1), 0):], Ks - 1)
-            self._decode = None
+            self._drop_decode()
         if pad:
             y = y[..., pad:]
         return y.permute(0, 2, 1)
@@ -346,7 +347,7 @@ class HyenaCascade(nn.Module):
         y, bx = res
         inference_params.fir_state_dict[self.layer_idx] = _ring(u[:, max(L - (Ks - 1), 0):], Ks - 1)
         inference_params.fir_inner_state_dict[self.layer_idx] = _ring(bx, K - 1, flipped=mr)
-        self._decode = None
+        self._drop_decode()
         return y
 
     # ------------------------------------------------------------------
@@ -356,6 +357,7 @@ class HyenaCascade(nn.Module):
         ring = inference_params.fir_state_dict[i]
         if self._decode is not None and self._decode["ring"] is ring:
             return self._decode
+        self._drop_decode()          # bound to another cache object: leave that one's state complete first
         C, Ks, D = 3 * self.hidden_size, self.short_filter_length, self.hidden_size
         dev = ring.buf.device
         d = {"ring": ring}
@@ -393,6 +395,15 @@ class HyenaCascade(nn.Module):
         return ops.LayerStepper(ring, self.short_filter_weight.detach().reshape(3 * self.hidden_size, Ks),
                                 self.short_filter_bias, cmap, inner, flip_x1x2=self.hyena_flip_x1x2)
 
+    def _drop_decode(self):
+        """Unbinds the decode kernels from the caches they were bound to.  A windowed modal stepper holds the last
+        inputs of its open windows itself, so its state tensor is brought up to date first: whoever owns that cache
+        object (another sequence served by this module in turn) finds it complete."""
+        inner = (self._decode or {}).get("inner")
+        if isinstance(inner, ops.IirStepper) and inner.pos_dev is None:
+            inner.flush()
+        self._decode = None
+
     def flush_decode_state(self):
         """Brings inference_params.state_dict[layer_idx] up to the last token (the windowed modal step lets it lag by up
         to four inputs); call it before reading or saving the state during decode.  No-op otherwise."""
@@ -409,9 +420,11 @@ class HyenaCascade(nn.Module):
             ring = stepper.ring
             valid, R = getattr(ring, "valid", stepper.R), stepper.R
             if valid < R:
+                # tap tables that change from token to token: the whole-cache step (far sums carry the taps of the
+                # token that formed them into the next two outputs)
                 full = stepper.w
                 stepper.w = _grown_taps(full, valid)
-                stepper(x1, x2, v, out)
+                stepper(x1, x2, v, out, far=False)
                 stepper.w = full
                 ring.valid = valid + 1
             else:

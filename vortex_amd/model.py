@@ -212,13 +212,18 @@ class StripedHyena2(nn.Module):
         return x @ self.embedding.weight.T
 
     @torch.no_grad()
-    def generate(self, input_ids, num_tokens, forced=None, graph=False):
+    def generate(self, input_ids, num_tokens, forced=None, graph=False, window_state=True):
         """Greedy cached generation in the order of vortex/model/generation.py:164-229: one prefill over the
         prompt, then one token per forward with the caches' seqlen_offset advanced first.  `forced`
         [B, num_tokens] replaces the sampled tokens (teacher forcing).  graph=True replays the token step as a
-        recorded HIP graph from the fifth token on (RecordedDecodeStep).  Returns (tokens, logits of every step)."""
+        recorded HIP graph from the fifth token on (RecordedDecodeStep).  window_state: the Hyena-LI layers keep their
+        modal states in windows of four tokens where that form exists (HyenaCascade.window_decode_state); this loop
+        owns its caches and nobody reads them between tokens.  Returns (tokens, logits of every step)."""
         B, L = input_ids.shape
         ipd = self.initialize_inference_params(max_seqlen=L + num_tokens)
+        for kind, block in zip(self.kinds, self.blocks):
+            if kind != "attn":
+                block.filter.window_decode_state = window_state
         x, toks, scores, rec = input_ids, [], [], None
         for i in range(num_tokens):
             if i > 0:

@@ -522,11 +522,13 @@ class FirStepper:
         self.ring.far_owner = self
         return 1
 
-    def __call__(self, x1, x2, v, out):
+    def __call__(self, x1, x2, v, out, far=True):
+        """far=False: this token reads the whole cache even if the stepper keeps far sums (which the next far step
+        then rebuilds); for callers that change `w` between tokens."""
         B = x1.shape[0]
         ring = self.ring
         dpos = ring.pos_dev is not None
-        if self.far is not None:
+        if self.far is not None and far:
             rc = self._fn_far(
                 x1.data_ptr(), x2.data_ptr() if self.gated else None, v.data_ptr() if self.gated else None,
                 x1.stride(0), ring.buf.data_ptr(), self.R, ring.block, 0 if dpos else ring.pos,
@@ -570,6 +572,7 @@ class IirStepper:
         L = _lib.lib()
         self._fn = L.hyena_iir_step
         self.win = None
+        self.pos_dev, self._recorded, self.warm = None, False, 0
         B = state.shape[0]
         if windowed and L.hyena_iir_window_supported(B, self.D, self.S, int(self.cplx)):
             W = L.hyena_iir_window_tokens()
@@ -584,14 +587,17 @@ class IirStepper:
             self._wref = ctypes.byref(self.win)
             self._fn_win, self._fn_flush = L.hyena_iir_step_win, L.hyena_iir_window_flush
             self.pos, self.period, self.pos_dev, self.warm = 0, W, None, 0
+            self._recorded = False      # a stream capture has taken a step of this stepper (with `warm` baked in)
 
     def _window(self):
         """The window descriptor for this call; advances the host-side counters."""
         w = self.win
         if self.pos_dev is not None:
             # a recorded step replays this call with `warm` frozen: every window has to be open by then
-            if self.warm < self.period and torch.cuda.is_current_stream_capturing():
-                raise RuntimeError(f"step {self.period} tokens eagerly before recording the windowed modal step")
+            if torch.cuda.is_current_stream_capturing():
+                if self.warm < self.period:
+                    raise RuntimeError(f"step {self.period} tokens eagerly before recording the windowed modal step")
+                self._recorded = True
             w.cnt, w.cnt_dev = 0, self.pos_dev.data_ptr()
         else:
             w.cnt, w.cnt_dev = self.pos, None
@@ -621,6 +627,12 @@ class IirStepper:
         stepper).  The next steps start new windows."""
         if self.win is None or self.warm == 0:
             return
+        if self._recorded and self.pos_dev is not None:
+            # the recorded launch has "every window open" in its arguments; after a flush it would fold inputs into
+            # the state that the flush has folded already
+            raise RuntimeError("a recorded token step replays this stepper with its windows open: release the "
+                               "recording (RingClock.release / RecordedDecodeStep.release) before flushing, and "
+                               "record again after at least `period` eager steps")
         w = self.win
         w.cnt, w.cnt_dev = (0, self.pos_dev.data_ptr()) if self.pos_dev is not None else (self.pos, None)
         w.warm = self.warm
@@ -751,17 +763,22 @@ class RingClock:
     def release(self):
         for r, p in zip(self.rings, self.pos.tolist()):
             r.pos, r.pos_dev = p, None
+            if hasattr(r, "_recorded"):
+                r._recorded = False     # recordings made on this clock must not be replayed any more
 
 
 class DecodeLayerSet:
     """Cached decode step of one [Hyena-SE, Hyena-MR, Hyena-LI] layer set: three fused launches.
 
     window_state: the Hyena-LI step keeps its modal state in windows of several tokens where the library has that form
-    (IirStepper windowed=True): state_li then lags the tokens until flush()."""
+    (IirStepper windowed=True): state_li then lags the tokens until flush().  far_sums: as in FirStepper, for the
+    Hyena-MR cache (None: the default for its depth; False: the whole cache on every token).  With both False every
+    kernel runs the reference's own algorithm."""
 
-    def __init__(self, ring_se, w_se, ring_mr, w_mr, D_mr, state_li, poles, residues, D_li, window_state=True):
+    def __init__(self, ring_se, w_se, ring_mr, w_mr, D_mr, state_li, poles, residues, D_li, window_state=True,
+                 far_sums=None):
         self.se = FirStepper(ring_se, w_se)
-        self.mr = FirStepper(ring_mr, w_mr, bias=D_mr, gated_bias=True)
+        self.mr = FirStepper(ring_mr, w_mr, bias=D_mr, gated_bias=True, far_sums=far_sums)
         self.li = IirStepper(state_li, poles, residues, D_li, windowed=window_state)
         B, D = state_li.shape[0], state_li.shape[1]
         self.out = [torch.empty(B, D, dtype=torch.bfloat16, device=state_li.device) for _ in range(3)]
