@@ -74,3 +74,70 @@ def test_small_width_stack_vs_oracle():
 def test_7b_shaped_group_at_L8192_vs_oracle():
     cfg = dict(EVO2_7B, num_layers=4)
     _compare(cfg, 8192, 21)
+
+
+@pytest.mark.timeout(900)
+@pytest.mark.parametrize("kind", ["hcs", "hcm", "hcl"])
+def test_7b_shaped_hyena_layers_at_L131072(kind):
+    """The long leg of the end-to-end configuration (B = 1, L = 131072, hidden 4096): each of the three Hyena operator
+    modules of a [SE, MR, LI, attention] group exactly as the stack runs it (projection u [1, L, 3*4096] in the
+    interleaved layout, fused prefill paths, cache objects filled), against the oracle's call sequence
+    (OracleCascade, vortex/model/model.py:214-375) on sampled filter groups -- the operators are independent per
+    channel, so a slice of the projection is a complete small problem -- plus two properties that need no oracle:
+    the first 8192 outputs equal a prefill of the first 8192 samples alone, and a prefill of L - 8 samples followed
+    by 8 cached one-token steps reproduces the last 8 outputs of the full prefill."""
+    from oracle import hyena_oracle as O
+    from vortex_amd.cascade import HyenaCascadeFIRInferenceParams, HyenaCascadeIIRInferenceParams
+    cfg = dict(EVO2_7B)
+    D, L = cfg["hidden_size"], 131072
+    m = StripedHyena2(dict(cfg, num_layers=4), seed=31, device="cuda").to_inference("cuda")
+    mod = m.blocks[("hcs", "hcm", "hcl").index(kind)].filter
+    K = mod.fir_inner_filter_length
+    g = torch.Generator(device="cuda").manual_seed(32)
+    u = torch.randn(1, L, 3 * D, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    with torch.no_grad():
+        if kind == "hcl":       # slow poles too (|p| up to 0.9999): a memory that spans the whole prompt
+            mod.log_poles.copy_(-(1e-4 + 0.1 * torch.rand(mod.log_poles.shape, generator=g, device="cuda")))
+        if mod.D is not None:   # the skip term is zero-initialised in the stack; give it values
+            mod.D.copy_(torch.randn(D, generator=g, device="cuda"))
+        ip = HyenaCascadeFIRInferenceParams() if K else HyenaCascadeIIRInferenceParams()
+        y, _ = mod(u, ip)
+        torch.cuda.synchronize()
+        assert y.shape == (1, L, D) and bool(torch.isfinite(y.float()).all())
+        # ---- the oracle's call sequence on sampled operator channels d0 .. d0+15 (one filter group of SE / MR)
+        for d0 in (0, 1600, D - 16):
+            sl = slice(3 * d0, 3 * (d0 + 16))
+            p = {"short_filter_weight": mod.short_filter_weight[sl].float().cpu(), "short_filter_bias": None}
+            if K:
+                p["h"] = mod.h[d0 // 16: d0 // 16 + 1].float().cpu().repeat(16, 1, 1)     # the group's filter, per channel
+                p["D"] = mod.D[d0:d0 + 16].cpu() if mod.D is not None else None
+                ref = O.OracleCascade(O.OracleEngine(), p, 16, 1, 16, fir_inner_filter_length=K, interleave=True)
+            else:
+                p["log_poles"], p["residues"] = mod.log_poles[d0:d0 + 16].float().cpu(), mod.residues[d0:d0 + 16].float().cpu()
+                p["D"] = mod.D[d0:d0 + 16].cpu()
+                ref = O.OracleCascade(O.OracleEngine(), p, 16, 1, 16, interleave=True)
+            ip_ref = O.OracleCache()
+            y_ref, _ = ref.forward(u[:, :, sl].cpu(), ip_ref)
+            got = y[:, :, d0:d0 + 16].float().cpu()
+            s = _stat(got, y_ref.float())
+            print(kind, d0, "vs oracle (max, mean):", s, flush=True)
+            assert s[0] <= 2e-2 and s[1] <= 2e-3, (kind, d0, s)
+            if K:
+                a = ip.fir_inner_state_dict[mod.layer_idx].reference_order()[:, d0:d0 + 16].cpu()
+                assert _stat(a, ip_ref.fir_inner_state_dict[0].float())[0] <= 2e-2
+            else:
+                a = ip.state_dict[mod.layer_idx][:, d0:d0 + 16].float().cpu()
+                assert _stat(a, ip_ref.state_dict[0].float())[0] <= 1e-3          # the oracle's state comes from fp32 FFTs
+            fa = ip.fir_state_dict[mod.layer_idx].reference_order()[:, sl].cpu()
+            assert torch.equal(fa, ip_ref.fir_state_dict[0].float())
+        # ---- causality: the first 8192 outputs do not depend on what follows (another launch shape, same values)
+        y_head, _ = mod(u[:, :8192].contiguous())
+        d = (y_head.float() - y[:, :8192].float()).abs().max() / y[:, :8192].float().abs().max()
+        assert d <= 2.0 ** -7, d            # at most the last bf16 digit (another segmentation of the same sums)
+        # ---- prefill of L - 8 samples, then 8 cached steps, against the last 8 outputs of the full prefill
+        ip2 = HyenaCascadeFIRInferenceParams() if K else HyenaCascadeIIRInferenceParams()
+        y0, _ = mod(u[:, :L - 8], ip2)
+        tail = torch.cat([mod(u[:, L - 8 + i: L - 7 + i], ip2)[0] for i in range(8)], dim=1)
+        scale = y.float().abs().max()
+        assert (y0.float() - y[:, :L - 8].float()).abs().max() / scale <= 2.0 ** -7
+        assert (tail.float() - y[:, L - 8:].float()).abs().max() / scale <= 2e-2
