@@ -137,9 +137,45 @@ def _gcg(x, k, q, h, bias, apply_gated_bias):
     return y[..., pad:] if pad else y
 
 
+_WIDE = (torch.float16, torch.float32)      # element types that always run channel-last (hyena_fir_cl_fwd_dtype)
+
+
 def _cl_ok(x, h):
-    """Whether the channel-last MFMA kernel covers (b, l, g, dg) inputs with this filter."""
-    return x.dim() == 4 and x.shape[3] % 16 == 0 and h.shape[-1] <= 128
+    """Whether a channel-last kernel covers (b, l, g, dg) inputs with this filter: the MFMA kernel needs filter
+    groups of a multiple of 16 channels; float16 / float32 tensors also have a direct-form kernel for any group."""
+    return x.dim() == 4 and h.shape[-1] <= 128 and (x.shape[3] % 16 == 0 or x.dtype in _WIDE)
+
+
+def _to_bld(t, layout):
+    """[B, L, D] with contiguous channels from any input layout (a view for blgdg, a transposing copy otherwise)."""
+    if layout == "blgdg":
+        b, l, g, dg = t.shape
+        return t.reshape(b, l, g * dg)
+    return _to_bdl(t, layout).transpose(1, 2).contiguous()
+
+
+def _from_bld(y, layout, num_groups):
+    b, l, d = y.shape
+    if layout == "bld":
+        return y
+    if layout == "blgdg":
+        return y.reshape(b, l, num_groups, d // num_groups)
+    if layout == "bdl":
+        return y.transpose(1, 2)
+    raise NotImplementedError("output_layout must be bld, bdl or blgdg")
+
+
+def _gcg_wide(x, k, q, taps, bias, mode, input_layout, output_layout, num_groups):
+    """q * fir(k * x) for float16 / float32 tensors in any layout, through the channel-last kernels.  taps [G', K]
+    float32 in the F.conv1d orientation; q, k None for the ungated FIR."""
+    if taps.shape[1] > 128:
+        raise NotImplementedError("filters longer than 128 taps have no FIR kernel")
+    xs = _to_bld(x, input_layout)
+    ks = _to_bld(k, input_layout) if k is not None else None
+    qs = _to_bld(q, input_layout) if q is not None else None
+    y = ops.fir_cl_fwd(ks if ks is not None else xs, qs, xs if ks is not None else None, taps, bias=bias,
+                       bias_mode=mode, taps_reversed=True)
+    return _from_bld(y, output_layout, num_groups)
 
 
 def _gcg_cl(x, k, q, h, bias, apply_gated_bias, want_y2=False, want_bx=False):
@@ -162,6 +198,10 @@ def inner_hyena_se(x, k, q, h, bias=None, input_layout="bdl", output_layout="bdl
     with dg a multiple of 16 stay channel-last through the kernel; other cases go through [B, D, L].
     """
     G = h.shape[0]
+    if x.dtype in _WIDE:
+        assert k.shape == q.shape == x.shape, "feature groups must have the same shape"
+        mode = HYENA_BIAS_NONE if bias is None else (HYENA_BIAS_GATED_FP32 if apply_gated_bias else HYENA_BIAS_ADD)
+        return _gcg_wide(x, k, q, ops._f32(h).reshape(G, -1), ops._f32(bias), mode, input_layout, output_layout, G)
     if input_layout == "blgdg" and _cl_ok(x, h):
         assert k.shape == q.shape == x.shape, "feature groups must have the same shape"
         b, l, g, dg = x.shape
@@ -204,7 +244,8 @@ def _bias_rule(weight_dtype, bias, apply_gated_bias, D):
         raise ValueError(f"bias must have {D} elements ([D], or [D, 1] for a gated bias)")
     if not apply_gated_bias:
         return b, HYENA_BIAS_ADD_FP32
-    return b, (HYENA_BIAS_GATED_BF16 if weight_dtype == torch.bfloat16 else HYENA_BIAS_GATED_FP32)
+    # 16-bit weights: the gated bias is tensor arithmetic in that type (three roundings); float32: one float32 sum
+    return b, (HYENA_BIAS_GATED_BF16 if weight_dtype in (torch.bfloat16, torch.float16) else HYENA_BIAS_GATED_FP32)
 
 
 def causal_conv1d_ref(x, weight, bias=None, apply_gated_bias=False, return_final_states=False, final_states_out=None,
@@ -224,7 +265,13 @@ def causal_conv1d_ref(x, weight, bias=None, apply_gated_bias=False, return_final
     if weight.dim() != 2 or weight.shape[0] != D:
         raise ValueError("weight must be [D, K]")
     b, mode = _bias_rule(weight.dtype, bias, apply_gated_bias, D)
-    out = _fir_per_channel(x, ops._f32(weight), None, None, b, mode)
+    if x.dtype in _WIDE:
+        # the arithmetic runs in weight.dtype and the result returns to x.dtype (interface.py:228-243)
+        if weight.dtype not in _WIDE:
+            raise NotImplementedError("float16 / float32 activations need float16 or float32 weights")
+        out = _gcg_wide(x.to(weight.dtype), None, None, ops._f32(weight), b, mode, "bdl", "bdl", D).to(x.dtype)
+    else:
+        out = _fir_per_channel(x, ops._f32(weight), None, None, b, mode)
     return out if not return_final_states else (out, final_states_out)
 
 
@@ -259,6 +306,12 @@ def inner_hyena_se_ref(x, k, q, h, bias=None, input_layout="bdl", output_layout=
         b, mode = _bias_rule(torch.float32, bias, False, D)
     else:
         b, mode = _bias_rule(h.dtype, bias, apply_gated_bias, D)
+    if xb.dtype in _WIDE:
+        # k*x, the convolution (in h.dtype) and the q gate each rounded to the activations' type, as the reference's
+        # tensor arithmetic rounds them; one tap row per channel, so this is the direct-form kernel
+        if h.dtype == torch.bfloat16:
+            raise NotImplementedError("float16 / float32 activations need float16 or float32 weights")
+        return _gcg_wide(xb, kb, qb, taps, b, mode, "bdl", output_layout, G)
     y = _fir_per_channel(xb, taps, qb, kb, b, mode)
     return _from_bdl(y, output_layout, G)
 

@@ -338,6 +338,30 @@ int hyena_fir_cl_fwd(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v,
                      void* out, void* y2_out, void* bx_out, int64_t bx_from,
                      int64_t B, int64_t L, int64_t D, int64_t G, int K, void* stream);
 
+/* Element types of hyena_fir_cl_fwd_dtype. */
+enum hyena_dtype {
+    HYENA_DTYPE_BF16 = 0,
+    HYENA_DTYPE_F16 = 1,
+    HYENA_DTYPE_F32 = 2
+};
+
+/* hyena_fir_cl_fwd for the element types the reference's own parity grid of this operator runs in
+ * (vortex/ops/hyena_se/tests/test_fwd.py:25-54 and tests/test_two_pass_ref.py:17-51: float16 and float32 tensors of
+ * shape (batch, seqlen, groups, group_dim), checked against gcg_fwd_ref_corrected, vortex/ops/hyena_se/ref_fwd.py:80-127).
+ * x1, x2, v, out, y2_out, bx_out hold elements of `dtype`; strides in elements; h and bias stay float32.
+ *   HYENA_DTYPE_BF16: exactly hyena_fir_cl_fwd.
+ *   HYENA_DTYPE_F16:  the same MFMA kernel on float16 operands (v_mfma_f32_32x32x16_f16; taps rounded to float16,
+ *                     bx = f16(x1*v), y2 = f16(conv), out = f16(x2*y2): the roundings of float16 tensor arithmetic)
+ *                     when D/G % 16 == 0, D % 8 == 0 and the operands are 16-byte aligned with strides % 8 == 0;
+ *                     any other shape runs a direct-form kernel with the same roundings and float32 taps.
+ *   HYENA_DTYPE_F32:  direct form, float32 operands and accumulation, nothing rounded below float32; any D/G.
+ * The direct form takes every bias mode (the "bf16" in their names reads as "element type"); the MFMA form those of
+ * hyena_fir_cl_fwd.  1 <= K <= 128. */
+int hyena_fir_cl_fwd_dtype(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v,
+                           const float* h, int taps_reversed, const float* bias, int bias_mode,
+                           void* out, void* y2_out, void* bx_out, int64_t bx_from,
+                           int64_t B, int64_t L, int64_t D, int64_t G, int K, int dtype, void* stream);
+
 /* The featurizer of a Hyena layer at prefill (vortex/model/model.py:233-252: short FIR over the 3D channels
  * of the dense projection, then interleave / split), described so that hyena_fir_layer_fwd can evaluate it on
  * the fly:  z[t][c] = bf16( sum_k w[k][c]*u[t-(Ks-1)+k][c] )  (then + bias[c], rounded again).

@@ -10,11 +10,12 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhyena_mi355x.so")
 
 HYENA_BIAS_NONE, HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_ADD_FP32, HYENA_BIAS_GATED_BF16 = 0, 1, 2, 3, 4
+HYENA_DTYPE_BF16, HYENA_DTYPE_F16, HYENA_DTYPE_F32 = 0, 1, 2
 
 EXPORTS = [
     "hyena_version", "hyena_last_error_string", "hyena_se_fwd", "hyena_mr_fwd",
     "hyena_fir_step", "hyena_iir_step", "hyena_li_plan_bytes", "hyena_li_plan", "hyena_li_fwd", "hyena_li_fwd_static", "hyena_featurizer_fwd", "hyena_set_launch_override",
-    "hyena_fir_layer_step", "hyena_iir_layer_step", "hyena_fir_cl_fwd", "hyena_fir_layer_fwd",
+    "hyena_fir_layer_step", "hyena_iir_layer_step", "hyena_fir_cl_fwd", "hyena_fir_cl_fwd_dtype", "hyena_fir_layer_fwd",
     "hyena_featurizer_gates_fwd",
     "hyena_fir_step_dpos", "hyena_fir_layer_step_dpos", "hyena_ring_advance",
     "hyena_fir_far_period", "hyena_fir_far_bytes", "hyena_fir_step_far", "hyena_fir_layer_step_far",
@@ -116,6 +117,8 @@ def lib():
     C = POINTER(Cl)
     L.hyena_fir_cl_fwd.argtypes = [C, C, C, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64,
                                    c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]
+    L.hyena_fir_cl_fwd_dtype.argtypes = [C, C, C, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64,
+                                         c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_void_p]
     L.hyena_featurizer_gates_fwd.argtypes = [POINTER(ProjFwd), c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]
     L.hyena_fir_layer_fwd.argtypes = [POINTER(ProjFwd), c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int64,
                                       c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]

@@ -12,7 +12,8 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libhyena_mi355x.so")
 PROBE = os.path.join(HERE, "libhyena_probe.so")          # copy kernel for counter calibration; not part of the ABI
 SELFTEST = os.path.join(HERE, "abi_selftest")          # plain C++ program that exercises the C ABI without torch
-SOURCES = ["api.hip", "se_fir.hip", "mr_fir.hip", "li_modal.hip", "decode.hip", "featurizer.hip", "fir_cl.hip"]
+SOURCES = ["api.hip", "se_fir.hip", "mr_fir.hip", "li_modal.hip", "decode.hip", "featurizer.hip", "fir_cl.hip",
+           "fir_cl_direct.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -61,6 +61,11 @@ enum { HYENA_OV_MR_NSEG, HYENA_OV_CL_NSEG, HYENA_OV_SE_NT, HYENA_OV_MR_NT, HYENA
        HYENA_OV_LI_CPW, HYENA_OV_LI_COOP, HYENA_OV_LI_XCD, HYENA_OV_COUNT };
 int64_t hyena_override(int id);
 
+// direct-form channel-last FIR for float16 / float32 tensors (fir_cl_direct.hip); arguments as hyena_fir_cl_fwd_dtype
+int hyena_fir_cl_direct(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, const float* h, int taps_reversed,
+                        const float* bias, int bias_mode, void* out, void* y2_out, void* bx_out, int64_t bx_from,
+                        int64_t B, int64_t L, int64_t D, int64_t G, int K, int dtype, void* stream, const char* who);
+
 static inline bool rows_aligned8(const hyena_rows* r) {
     return r == nullptr || ((((uintptr_t)r->ptr) & 15) == 0 && r->batch_stride % 8 == 0 && r->row_stride % 8 == 0);
 }

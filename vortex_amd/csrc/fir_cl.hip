@@ -49,6 +49,42 @@ __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) {
     return c.b;
 }
 
+// The 16-bit element type of the tensors the gates-given form works on: how a packed pair widens to float, how two
+// floats round (to nearest even) into a pair, and the MFMA that contracts such operands.  bfloat16 is what the
+// model path uses; float16 serves callers of the (batch, seqlen, groups, group_dim) interface, whose reference
+// grid runs in float16 and float32 (vortex/ops/hyena_se/tests/test_fwd.py:25-54).
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
+
+struct ElBf16 {
+    typedef bf16x8 frag;
+    static __device__ __forceinline__ float lo(uint32_t w) { return bf_lo(w); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return bf_hi(w); }
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) { return pack_bf2(a, b); }
+    static __device__ __forceinline__ float round(float f) { return round_bf(f); }
+    static __device__ __forceinline__ frag as_frag(u32x4 x) { return as_bf16x8(x); }
+    static __device__ __forceinline__ f32x16 mfma(frag a, frag b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+
+struct ElF16 {
+    typedef f16x8 frag;
+    static __device__ __forceinline__ float lo(uint32_t w) { union { uint32_t u; f16x2_t h; } c; c.u = w; return (float)c.h[0]; }
+    static __device__ __forceinline__ float hi(uint32_t w) { union { uint32_t u; f16x2_t h; } c; c.u = w; return (float)c.h[1]; }
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+        union { uint32_t u; f16x2_t h; } c;
+        c.h[0] = (_Float16)a;                    // v_cvt_f16_f32, round to nearest even
+        c.h[1] = (_Float16)b;
+        return c.u;
+    }
+    static __device__ __forceinline__ float round(float f) { return (float)(_Float16)f; }
+    static __device__ __forceinline__ frag as_frag(u32x4 x) { union { u32x4 u; frag b; } c; c.u = x; return c.b; }
+    static __device__ __forceinline__ f32x16 mfma(frag a, frag b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
 // 16-bit halves of two dwords: (lo(a), lo(b)) or (hi(a), hi(b)) packed as (first, second)
 __device__ __forceinline__ uint32_t pair_lo(uint32_t first, uint32_t second) {
     return __builtin_amdgcn_perm(second, first, 0x05040100u);
@@ -141,13 +177,15 @@ __device__ __forceinline__ void lane_gates(const u32x4 (&raw)[3][KS + 3], const 
 // blocks 7..9), which leaves three A fragments in registers and five B reads / six MFMAs per step.
 // NT = non-temporal accesses for tensors that stream through the last-level cache: the output rows always, the
 // input rows only without the fused featurizer (its lanes re-read their neighbours' rows, which must stay cached).
-template <bool PRE, bool POST, int BIAS, int FEAT, int KS, bool AUX, int MLO, bool NT>
+// ET = element traits of the 16-bit tensors (ElBf16, or ElF16 without the featurizer).
+template <typename ET, bool PRE, bool POST, int BIAS, int FEAT, int KS, bool AUX, int MLO, bool NT>
 __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMap v, ProjFwd pj,
                                                         const float* __restrict__ h, int K, int reversed,
                                                         const float* __restrict__ bias, bf16_t* __restrict__ out,
                                                         bf16_t* __restrict__ y2_out, bf16_t* __restrict__ bx_out,
                                                         int64_t bx_from, int64_t L, int64_t D, int dg,
                                                         int64_t seg_len, int nseg, int ndb) {
+    static_assert(FEAT == 0 || std::is_same<ET, ElBf16>::value, "the fused featurizer is built for bfloat16");
     constexpr int RF = FEAT ? KS - 1 : 0;          // extra rows a lane reads before its own four
     constexpr int NR = 4 + RF;                     // rows per lane and load piece
     constexpr int NP = (FEAT || (PRE && POST)) ? 3 : (PRE ? 2 : 1);   // load pieces per row
@@ -172,7 +210,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     const bool slab_live = d0 + 16 * w < (uint32_t)D;
     const int g = slab_live ? (int)((d0 + 16 * w) / (uint32_t)dg) : 0;
     const int i_time = 16 * ((n >> 2) & 1) + 4 * (n >> 3) + (n & 3);
-    bf16x8 A[10 - MLO];
+    typename ET::frag A[10 - MLO];
 #pragma unroll
     for (int m = MLO; m < 10; ++m) {
         u32x4 pk;
@@ -186,9 +224,9 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                 if (lag >= 0 && lag < K) val = h[g * K + (reversed ? K - 1 - lag : lag)];
                 t[e] = val;
             }
-            pk[j] = pack_bf2(t[0], t[1]);
+            pk[j] = ET::pack2(t[0], t[1]);
         }
-        A[m - MLO] = as_bf16x8(pk);
+        A[m - MLO] = ET::as_frag(pk);
     }
 
     // ---- this lane's I/O block: rows 4*rb .. 4*rb+3 of the step, channels d0 + 8*cb .. +7
@@ -318,8 +356,8 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                 if (PRE) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        bx[q][j] = pack_bf2(bf_lo(raw[0][q][j]) * bf_lo(raw[1][q][j]),
-                                            bf_hi(raw[0][q][j]) * bf_hi(raw[1][q][j]));
+                        bx[q][j] = ET::pack2(ET::lo(raw[0][q][j]) * ET::lo(raw[1][q][j]),
+                                             ET::hi(raw[0][q][j]) * ET::hi(raw[1][q][j]));
                 } else {
                     bx[q] = raw[0][q];
                 }
@@ -360,9 +398,9 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
             const int c0 = 64 * s + 8 * hh + (cur ^ 1) * TL;     // ring position of the halo chunk's first sample
 #pragma unroll
             for (int mm = MLO; mm < 12; ++mm) {
-                const bf16x8 bf = *(const bf16x8*)(urow + (((c0 + 16 * mm) & (2 * TL - 1)) ^ swz_mm));
-                if (mm <= 9) acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm <= 9 ? mm - MLO : 0], bf, acc0, 0, 0, 0);
-                if (mm - 2 >= MLO) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[mm - 2 >= MLO ? mm - 2 - MLO : 0], bf, acc1, 0, 0, 0);
+                const typename ET::frag bf = ET::as_frag(*(const u32x4*)(urow + (((c0 + 16 * mm) & (2 * TL - 1)) ^ swz_mm)));
+                if (mm <= 9) acc0 = ET::mfma(A[mm <= 9 ? mm - MLO : 0], bf, acc0);
+                if (mm - 2 >= MLO) acc1 = ET::mfma(A[mm - 2 >= MLO ? mm - 2 - MLO : 0], bf, acc1);
                 if ((mm & 3) == 3) __builtin_amdgcn_sched_barrier(0);    // at most four B fragments in registers at a time
             }
         }
@@ -391,14 +429,14 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                     float a0 = acc[2 * j], a1 = acc[2 * j + 1];
                     if (BIAS == HYENA_BIAS_GATED_FP32) {
                         const uint32_t uw = j < 4 ? ua[j] : ub2[j - 4];
-                        a0 = fmaf(bz, bf_lo(uw), a0);
-                        a1 = fmaf(bz, bf_hi(uw), a1);
+                        a0 = fmaf(bz, ET::lo(uw), a0);
+                        a1 = fmaf(bz, ET::hi(uw), a1);
                     }
                     if (BIAS == HYENA_BIAS_ADD) {
-                        a0 = round_bf(a0) + bz;
-                        a1 = round_bf(a1) + bz;
+                        a0 = ET::round(a0) + bz;
+                        a1 = ET::round(a1) + bz;
                     }
-                    const uint32_t p = pack_bf2(a0, a1);
+                    const uint32_t p = ET::pack2(a0, a1);
                     if (j < 4) z0[j] = p; else z1[j - 4] = p;
                 }
                 *(u32x4*)(z_lds + (16 * w + c) * ZRS + (tcol ^ swz_mm)) = z0;
@@ -437,7 +475,7 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
                     if (POST) {
 #pragma unroll
                         for (int j = 0; j < 4; ++j)
-                            o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(g2[q][j]), bf_hi(zz[j]) * bf_hi(g2[q][j]));
+                            o[j] = ET::pack2(ET::lo(zz[j]) * ET::lo(g2[q][j]), ET::hi(zz[j]) * ET::hi(g2[q][j]));
                     }
                     u32x4* const dst = (u32x4*)((char*)out_step + (lane_row_b + q * row_b));
                     if (NT) __builtin_nontemporal_store(o, dst);
@@ -636,11 +674,15 @@ __global__ __launch_bounds__(256, 2) void proj_gates_kernel(ProjFwd pj, bf16_t* 
     for (; c0 < c_end; c0 += GT) tile_step(c0, std::false_type{});
 }
 
+// the float16 traits where that form exists (no featurizer), bfloat16 otherwise (the launcher refuses float16 there)
+template <int FEAT> using F16For = typename std::conditional<FEAT == 0, ElF16, ElBf16>::type;
+
 struct LaunchArgs {
     ClMap x1, x2, v;
     ProjFwd pj;
     int feat, ks;
     bool pre, post;
+    bool f16;                  // float16 tensors (gates given, no featurizer); bfloat16 otherwise
 };
 
 static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed, const float* bias, int bias_mode,
@@ -658,6 +700,7 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     if (bias_mode > HYENA_BIAS_GATED_FP32)
         return hyena_fail(HYENA_ENOSUP, "%s: bias_mode %d is built for the sequence-major kernels only", who, bias_mode);
     if (bx_out && (bx_from < 0 || bx_from > L)) return hyena_fail(HYENA_EINVAL, "%s: bx_from outside 0..L", who);
+    if (a.f16 && a.feat) return hyena_fail(HYENA_ENOSUP, "%s: the fused featurizer takes bfloat16 only", who);
     if (bx_out && a.feat && L - bx_from > K - 1)
         return hyena_fail(HYENA_ENOSUP, "%s: with the featurizer fused, bx is the cache tail (at most K-1 = %d samples)",
                           who, K - 1);
@@ -699,10 +742,16 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
     { const int64_t x = hyena_override(HYENA_OV_CL_NT); if (x >= 0) nt = x != 0; }
     bool ok = false;
-#define CL_GO(P, Q, M, F, KSV, AX, ML, N)                                                                         \
-    hipLaunchKernelGGL((fir_cl_kernel<P, Q, M, F, KSV, AX, ML, N>), grid, dim3(256), 0, s, a.x1, a.x2, a.v, a.pj, h, \
+#define CL_GO_T(T, P, Q, M, F, KSV, AX, ML, N)                                                                       \
+    hipLaunchKernelGGL((fir_cl_kernel<T, P, Q, M, F, KSV, AX, ML, N>), grid, dim3(256), 0, s, a.x1, a.x2, a.v, a.pj, h, \
                        K, taps_reversed, bias, (bf16_t*)out, (bf16_t*)y2_out, (bf16_t*)bx_out, bx_from, L, D, dg,   \
                        seg_len, (int)nseg, (int)ndb)
+// float16 only exists for the form with the gates given as tensors (F == 0)
+#define CL_GO(P, Q, M, F, KSV, AX, ML, N)                                                                         \
+    do {                                                                                                          \
+        if (a.f16) CL_GO_T(F16For<F>, P, Q, M, F, KSV, AX, ML, N);                                                \
+        else CL_GO_T(ElBf16, P, Q, M, F, KSV, AX, ML, N);                                                         \
+    } while (0)
 #define CL_CASE(P, Q, M, F, KSV)                                                                                  \
     if (!ok && a.pre == P && a.post == Q && bias_mode == M && a.feat == F && (F == 0 || a.ks == KSV)) {           \
         if (aux && shortk) CL_GO(P, Q, M, F, KSV, true, (P && M == HYENA_BIAS_NONE) ? 7 : 0, false);              \
@@ -729,6 +778,7 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     CL_CASE(true, true, HYENA_BIAS_GATED_FP32, 3, 4)
 #undef CL_CASE
 #undef CL_GO
+#undef CL_GO_T
     if (!ok) return hyena_fail(HYENA_ENOSUP, "%s: this gate / bias / featurizer-length combination has no kernel", who);
     return hyena_check_launch(who);
 }
@@ -788,6 +838,48 @@ extern "C" int hyena_fir_cl_fwd(const hyena_cl* x1, const hyena_cl* x2, const hy
     }
     a.feat = 0; a.ks = 3; a.pre = pre; a.post = post;
     return fir_cl_launch(a, h, taps_reversed, bias, bias_mode, out, y2_out, bx_out, bx_from, B, L, D, G, K, stream, who);
+}
+
+extern "C" int hyena_fir_cl_fwd_dtype(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, const float* h,
+                                      int taps_reversed, const float* bias, int bias_mode, void* out, void* y2_out,
+                                      void* bx_out, int64_t bx_from, int64_t B, int64_t L, int64_t D, int64_t G, int K,
+                                      int dtype, void* stream) {
+    const char* who = "hyena_fir_cl_fwd_dtype";
+    if (dtype == HYENA_DTYPE_BF16)
+        return hyena_fir_cl_fwd(x1, x2, v, h, taps_reversed, bias, bias_mode, out, y2_out, bx_out, bx_from, B, L, D, G, K,
+                                stream);
+    if (dtype != HYENA_DTYPE_F16 && dtype != HYENA_DTYPE_F32) return hyena_fail(HYENA_EINVAL, "%s: unknown dtype %d", who, dtype);
+    if (!x1 || !x1->ptr || !h || !out) return hyena_fail(HYENA_EINVAL, "%s: x1, h and out are required", who);
+    const bool pre = v && v->ptr, post = x2 && x2->ptr;
+    if (pre != post) return hyena_fail(HYENA_ENOSUP, "%s: pass both gates v and x2, or neither", who);
+    if (B < 0 || D <= 0 || L < 0 || G <= 0 || D % G != 0 || D >= (1LL << 24))
+        return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld L=%lld G=%lld", who, (long long)B, (long long)D,
+                          (long long)L, (long long)G);
+    if (K < 1 || K > 128) return hyena_fail(HYENA_ENOSUP, "%s: K=%d outside 1..128", who, K);
+    if (bias_mode < 0 || bias_mode > 4 || (bias_mode != HYENA_BIAS_NONE && !bias))
+        return hyena_fail(HYENA_EINVAL, "%s: bias_mode %d needs a bias pointer", who, bias_mode);
+    if (bx_out && (bx_from < 0 || bx_from > L)) return hyena_fail(HYENA_EINVAL, "%s: bx_from outside 0..L", who);
+    const uintptr_t esz = dtype == HYENA_DTYPE_F32 ? 4 : 2;
+    auto el_ok = [&](const hyena_cl* c) { return ((uintptr_t)c->ptr & (esz - 1)) == 0 && c->time_stride >= 0; };
+    if (!el_ok(x1) || (pre && (!el_ok(v) || !el_ok(x2))) ||
+        (((uintptr_t)out | (uintptr_t)y2_out | (uintptr_t)bx_out) & (esz - 1)))
+        return hyena_fail(HYENA_EALIGN, "%s: pointers must be aligned to the element size, time strides non-negative", who);
+    if (B == 0 || L == 0) return 0;
+    // float16: the MFMA form where its shape and alignment rules hold
+    if (dtype == HYENA_DTYPE_F16 && (D / G) % 16 == 0 && D % 8 == 0 && bias_mode <= HYENA_BIAS_GATED_FP32 && cl_ok(x1) &&
+        cl_stride_ok(x1) && (!pre || (cl_ok(v) && cl_ok(x2) && cl_stride_ok(v) && cl_stride_ok(x2))) &&
+        !(((uintptr_t)out | (uintptr_t)y2_out | (uintptr_t)bx_out) & 15)) {
+        LaunchArgs a = {};
+        a.x1 = {(const bf16_t*)x1->ptr, x1->batch_stride, x1->time_stride};
+        if (pre) {
+            a.v = {(const bf16_t*)v->ptr, v->batch_stride, v->time_stride};
+            a.x2 = {(const bf16_t*)x2->ptr, x2->batch_stride, x2->time_stride};
+        }
+        a.feat = 0; a.ks = 3; a.pre = pre; a.post = post; a.f16 = true;
+        return fir_cl_launch(a, h, taps_reversed, bias, bias_mode, out, y2_out, bx_out, bx_from, B, L, D, G, K, stream, who);
+    }
+    return hyena_fir_cl_direct(x1, x2, v, h, taps_reversed, bias, bias_mode, out, y2_out, bx_out, bx_from, B, L, D, G, K,
+                               dtype, stream, who);
 }
 
 extern "C" int hyena_fir_layer_fwd(const hyena_proj_fwd* proj, const float* h, int taps_reversed, const float* bias,

@@ -1,0 +1,151 @@
+// Channel-last gated FIR in direct form for float32 and float16 tensors: the (batch, seqlen, groups, group_dim)
+// operator of vortex/ops/hyena_se/fwd.py:17-43 for the element types its reference grid runs in
+// (vortex/ops/hyena_se/tests/test_fwd.py:25-54: float16 and float32, filters of 4, 32 and 128 taps drawn from N(0, 1)).
+//
+// float32 inputs cannot go through one bf16 or fp16 MFMA term at that grid's tolerance (1e-2 absolute on outputs whose
+// accumulation runs over magnitudes of sqrt(K) ~ 11), so this kernel accumulates in float32 on the vector ALUs with
+// float32 operands: out = x2 * (sum_k h[g][k] * (x1*v)[t-k]), nothing rounded below float32.  float16 tensors take
+// the same kernel for shapes the MFMA form does not cover (filter groups that are not multiples of 16 channels,
+// unaligned strides), with the roundings of float16 tensor arithmetic: bx = f16(x1*v), z = f16(conv), out = f16(x2*z).
+//
+// Block = 64 channels x 128 output samples.  bx of the tile and its K-1 samples of history sit in LDS as float32
+// [row][channel] (a lane reads its own channel: consecutive banks), the taps as [lag][channel].  A thread owns one
+// channel and 32 consecutive outputs; it walks the lags 32 at a time with a 63-sample window of bx in registers, so
+// every product has compile-time register operands: 63 + 32 LDS reads per 1024 FMAs.
+#include <type_traits>
+
+#include "common.h"
+
+namespace {
+
+constexpr int DT = 128;        // output samples per block
+constexpr int DC = 64;         // channels per block
+constexpr int DK = 128;        // lags the tap table is padded to
+
+template <typename T> struct ElT;
+template <> struct ElT<float> {
+    static __device__ __forceinline__ float rnd(float f) { return f; }
+};
+template <> struct ElT<_Float16> {
+    static __device__ __forceinline__ float rnd(float f) { return (float)(_Float16)f; }     // round to nearest even
+};
+
+template <typename T>
+struct ClMapT {                // channel-last operand: (b, t, d) at ptr + b*bs + t*ts + d
+    const T* ptr;
+    int64_t bs, ts;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void fir_cl_direct_kernel(ClMapT<T> x1, ClMapT<T> x2, ClMapT<T> v,
+                                                            const float* __restrict__ h, int K, int reversed,
+                                                            const float* __restrict__ bias, int bias_mode,
+                                                            T* __restrict__ out, T* __restrict__ y2_out,
+                                                            T* __restrict__ bx_out, int64_t bx_from, int64_t L,
+                                                            int64_t D, int dg, int ndb, int ntt) {
+    __shared__ float bx_lds[(DT + DK - 1) * DC];
+    __shared__ float h_lds[DK * DC];
+    const int tid = threadIdx.x, c = tid & (DC - 1), tq = tid >> 6;
+    const uint32_t bid = blockIdx.x;
+    const uint32_t db = bid % (uint32_t)ndb;
+    const uint32_t tt = (bid / (uint32_t)ndb) % (uint32_t)ntt;
+    const int64_t b = bid / ((uint32_t)ndb * (uint32_t)ntt);
+    const int64_t d = (int64_t)db * DC + c;
+    const bool ch_ok = d < D;
+    const int64_t t0 = (int64_t)tt * DT;
+    const bool pre = v.ptr != nullptr, post = x2.ptr != nullptr;
+
+    // taps of this thread's channel by lag (0 = the current sample), zero from K on
+    {
+        const int g = ch_ok ? (int)((uint32_t)d / (uint32_t)dg) : 0;
+        for (int k = tq; k < DK; k += 4) {
+            float val = 0.f;
+            if (ch_ok && k < K) val = h[(int64_t)g * K + (reversed ? K - 1 - k : k)];
+            h_lds[k * DC + c] = val;
+        }
+    }
+    // bx rows t0 - (K-1) .. t0 + DT - 1 -> LDS rows (DK-1) - (K-1) + r; rows below stay unread (their taps are zero, and
+    // the window clamps its row index at 0, which is then a row of finite values)
+    const int r0 = DK - K;     // LDS row of sample t0 - (K-1)
+    for (int r = tq; r < DT + K - 1; r += 4) {
+        const int64_t t = t0 - (K - 1) + r;
+        float val = 0.f;
+        if (ch_ok && t >= 0 && t < L) {
+            val = (float)x1.ptr[b * x1.bs + t * x1.ts + d];
+            if (pre) val = ElT<T>::rnd(val * (float)v.ptr[b * v.bs + t * v.ts + d]);
+            if (bx_out && r >= K - 1 && t >= bx_from) bx_out[(b * (L - bx_from) + (t - bx_from)) * D + d] = (T)val;
+        }
+        bx_lds[(r0 + r) * DC + c] = val;
+    }
+    if (r0 > 0) {              // rows 0 .. r0-1 are read (times zero taps) when the clamp does not apply: keep them finite
+        for (int r = tq; r < r0; r += 4) bx_lds[r * DC + c] = 0.f;
+    }
+    __syncthreads();
+
+    // outputs j = 0..31 at t0 + 32*tq + j; LDS row of output j at lag k: base + j - k
+    const int base = (DK - 1) + 32 * tq;
+    float acc[32];
+#pragma unroll
+    for (int j = 0; j < 32; ++j) acc[j] = 0.f;
+    for (int kb = 0; kb < K; kb += 32) {
+        float win[63];
+#pragma unroll
+        for (int i = 0; i < 63; ++i) win[i] = bx_lds[(base - kb - 31 + i) * DC + c];      // row >= DK-1-96-31 = 0
+#pragma unroll
+        for (int kk = 0; kk < 32; ++kk) {
+            const float hk = h_lds[(kb + kk) * DC + c];
+#pragma unroll
+            for (int j = 0; j < 32; ++j) acc[j] = fmaf(hk, win[j - kk + 31], acc[j]);
+        }
+    }
+
+    const float bz = (bias_mode != HYENA_BIAS_NONE && ch_ok) ? bias[d] : 0.f;
+#pragma unroll 4
+    for (int j = 0; j < 32; ++j) {
+        const int64_t t = t0 + 32 * tq + j;
+        if (!ch_ok || t >= L) continue;
+        const float u = bx_lds[(base + j) * DC + c];
+        float z;
+        switch (bias_mode) {
+            case HYENA_BIAS_ADD:        z = ElT<T>::rnd(ElT<T>::rnd(acc[j]) + bz); break;
+            case HYENA_BIAS_ADD_FP32:   z = ElT<T>::rnd(acc[j] + bz); break;
+            case HYENA_BIAS_GATED_FP32: z = ElT<T>::rnd(fmaf(bz, u, acc[j])); break;
+            case HYENA_BIAS_GATED_BF16: z = ElT<T>::rnd(ElT<T>::rnd(acc[j]) + ElT<T>::rnd(bz * u)); break;   // element-type tensor arithmetic
+            default:                    z = ElT<T>::rnd(acc[j]);
+        }
+        const int64_t o = (b * L + t) * D + d;
+        if (y2_out) y2_out[o] = (T)z;
+        if (post) z = ElT<T>::rnd(z * (float)x2.ptr[b * x2.bs + t * x2.ts + d]);
+        out[o] = (T)z;
+    }
+}
+
+template <typename T>
+int direct_launch(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, const float* h, int taps_reversed,
+                  const float* bias, int bias_mode, void* out, void* y2_out, void* bx_out, int64_t bx_from, int64_t B,
+                  int64_t L, int64_t D, int64_t G, int K, void* stream, const char* who) {
+    const int64_t ndb = (D + DC - 1) / DC, ntt = (L + DT - 1) / DT;
+    if (B * ndb * ntt > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: problem too large for one launch", who);
+    ClMapT<T> m1 = {(const T*)x1->ptr, x1->batch_stride, x1->time_stride};
+    ClMapT<T> m2 = {nullptr, 0, 0}, mv = {nullptr, 0, 0};
+    if (x2 && x2->ptr) m2 = {(const T*)x2->ptr, x2->batch_stride, x2->time_stride};
+    if (v && v->ptr) mv = {(const T*)v->ptr, v->batch_stride, v->time_stride};
+    hipLaunchKernelGGL((fir_cl_direct_kernel<T>), dim3((unsigned)(B * ndb * ntt)), dim3(256), 0, (hipStream_t)stream, m1,
+                       m2, mv, h, K, taps_reversed, bias, bias_mode, (T*)out, (T*)y2_out, (T*)bx_out, bx_from, L, D,
+                       (int)(D / G), (int)ndb, (int)ntt);
+    return hyena_check_launch(who);
+}
+
+}  // namespace
+
+// Direct-form launch for float16 (dtype 1) or float32 (dtype 2) channel-last tensors; arguments as hyena_fir_cl_fwd,
+// already validated by the caller except for what is specific to this form.
+int hyena_fir_cl_direct(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, const float* h, int taps_reversed,
+                        const float* bias, int bias_mode, void* out, void* y2_out, void* bx_out, int64_t bx_from,
+                        int64_t B, int64_t L, int64_t D, int64_t G, int K, int dtype, void* stream, const char* who) {
+    if (dtype == HYENA_DTYPE_F32)
+        return direct_launch<float>(x1, x2, v, h, taps_reversed, bias, bias_mode, out, y2_out, bx_out, bx_from, B, L, D,
+                                    G, K, stream, who);
+    return direct_launch<_Float16>(x1, x2, v, h, taps_reversed, bias, bias_mode, out, y2_out, bx_out, bx_from, B, L, D, G,
+                                   K, stream, who);
+}

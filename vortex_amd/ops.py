@@ -10,6 +10,8 @@ import torch
 from . import _lib
 from ._lib import HYENA_BIAS_ADD, HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE, Cl, ProjFwd, ProjStep, Rows
 
+_CL_DTYPES = {torch.bfloat16: _lib.HYENA_DTYPE_BF16, torch.float16: _lib.HYENA_DTYPE_F16, torch.float32: _lib.HYENA_DTYPE_F32}
+
 
 def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -134,35 +136,48 @@ def fir_fwd_rows(x1r, x2r, vr, taps, B, D, L, K, *, device, bias=None, bias_mode
     return out
 
 
-def _cl_of(t):
-    """hyena_cl of a [B, L, D] bf16 tensor with contiguous channels (any batch / time stride)."""
+def _cl_of(t, dtype=torch.bfloat16):
+    """hyena_cl of a [B, L, D] tensor of `dtype` with contiguous channels (any batch / time stride)."""
     if t is None:
         return None
-    if t.dtype != torch.bfloat16 or t.dim() != 3 or (t.shape[2] > 1 and t.stride(2) != 1):
-        raise ValueError("expected a [B, L, D] bfloat16 tensor with contiguous channels")
+    if t.dtype != dtype or t.dim() != 3 or (t.shape[2] > 1 and t.stride(2) != 1):
+        raise ValueError(f"expected a [B, L, D] {dtype} tensor with contiguous channels")
     bs, ts, _ = _strides(t)
     return Cl(t.data_ptr(), bs, ts)
 
 
 def fir_cl_fwd(x1, x2, v, taps, *, bias=None, bias_mode=HYENA_BIAS_NONE, taps_reversed=False, want_y2=False,
                want_bx=False, bx_from=0, out=None):
-    """Gated FIR on channel-last [B, L, D] tensors: out = x2 * conv(taps, x1*v), MFMA kernel, 1 <= K <= 128.
+    """Gated FIR on channel-last [B, L, D] tensors: out = x2 * conv(taps, x1*v), 1 <= K <= 128.
 
+    bfloat16 tensors (the model path) and float16 tensors run the MFMA kernel (filter groups of a multiple of 16
+    channels); float32 tensors, and float16 shapes the MFMA kernel does not cover, run a direct-form kernel
+    (hyena_fir_cl_fwd_dtype).  All tensors share x1's dtype, which is also the dtype of the results.
     taps [G, K] float32, convolution orientation unless taps_reversed.  Returns out, or (out, y2, bx) when an
-    intermediate is requested (y2: the convolution before the x2 gate; bx: rows bx_from.. of bf16(x1*v)).
+    intermediate is requested (y2: the convolution before the x2 gate; bx: rows bx_from.. of x1*v in that dtype).
     """
     _need_cuda(x1, x2, v, taps)
+    dt = x1.dtype
+    if dt not in _CL_DTYPES:
+        raise TypeError(f"channel-last FIR takes bfloat16, float16 or float32 tensors, got {dt}")
     taps = _f32(taps)
     G, K = taps.shape
     B, L, D = x1.shape
     if out is None:
-        out = torch.empty((B, L, D), dtype=torch.bfloat16, device=x1.device)
+        out = torch.empty((B, L, D), dtype=dt, device=x1.device)
+    elif out.dtype != dt or not out.is_contiguous():
+        raise ValueError("out must be contiguous and of the inputs' dtype")
     y2 = torch.empty_like(out) if want_y2 else None
-    bx = torch.empty((B, L - bx_from, D), dtype=torch.bfloat16, device=x1.device) if want_bx else None
+    bx = torch.empty((B, L - bx_from, D), dtype=dt, device=x1.device) if want_bx else None
     if out.numel():
-        c1, c2, cv = _cl_of(x1), _cl_of(x2), _cl_of(v)
-        rc = _lib.lib().hyena_fir_cl_fwd(_ref(c1), _ref(c2), _ref(cv), _ptr(taps), int(taps_reversed), _ptr(_f32(bias)),
-                                         bias_mode, _ptr(out), _ptr(y2), _ptr(bx), bx_from, B, L, D, G, K, _stream())
+        c1, c2, cv = _cl_of(x1, dt), _cl_of(x2, dt), _cl_of(v, dt)
+        if dt == torch.bfloat16:
+            rc = _lib.lib().hyena_fir_cl_fwd(_ref(c1), _ref(c2), _ref(cv), _ptr(taps), int(taps_reversed), _ptr(_f32(bias)),
+                                             bias_mode, _ptr(out), _ptr(y2), _ptr(bx), bx_from, B, L, D, G, K, _stream())
+        else:
+            rc = _lib.lib().hyena_fir_cl_fwd_dtype(_ref(c1), _ref(c2), _ref(cv), _ptr(taps), int(taps_reversed),
+                                                   _ptr(_f32(bias)), bias_mode, _ptr(out), _ptr(y2), _ptr(bx), bx_from,
+                                                   B, L, D, G, K, _CL_DTYPES[dt], _stream())
         _lib.check(rc, "hyena_fir_cl_fwd")
     return (out, y2, bx) if (want_y2 or want_bx) else out
 
