@@ -349,14 +349,17 @@ enum hyena_dtype {
  * (vortex/ops/hyena_se/tests/test_fwd.py:25-54 and tests/test_two_pass_ref.py:17-51: float16 and float32 tensors of
  * shape (batch, seqlen, groups, group_dim), checked against gcg_fwd_ref_corrected, vortex/ops/hyena_se/ref_fwd.py:80-127).
  * x1, x2, v, out, y2_out, bx_out hold elements of `dtype`; strides in elements; h and bias stay float32.
- *   HYENA_DTYPE_BF16: exactly hyena_fir_cl_fwd.
+ *   HYENA_DTYPE_BF16: exactly hyena_fir_cl_fwd for K <= 128; longer filters (vortex/model/engine.py:174-187 takes any
+ *                     length through its FFT, :339-349 any long_fir_threshold) run the direct form below with the
+ *                     roundings of bfloat16 tensor arithmetic.
  *   HYENA_DTYPE_F16:  the same MFMA kernel on float16 operands (v_mfma_f32_32x32x16_f16; taps rounded to float16,
  *                     bx = f16(x1*v), y2 = f16(conv), out = f16(x2*y2): the roundings of float16 tensor arithmetic)
  *                     when D/G % 16 == 0, D % 8 == 0 and the operands are 16-byte aligned with strides % 8 == 0;
  *                     any other shape runs a direct-form kernel with the same roundings and float32 taps.
  *   HYENA_DTYPE_F32:  direct form, float32 operands and accumulation, nothing rounded below float32; any D/G.
- * The direct form takes every bias mode (the "bf16" in their names reads as "element type"); the MFMA form those of
- * hyena_fir_cl_fwd.  1 <= K <= 128. */
+ * The direct form takes every bias mode (the "bf16" in their names reads as "element type") and any K >= 1 (filters
+ * beyond 128 taps in blocks of 128 lags, in every element type); the MFMA form takes the bias modes of hyena_fir_cl_fwd
+ * and 1 <= K <= 128. */
 int hyena_fir_cl_fwd_dtype(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v,
                            const float* h, int taps_reversed, const float* bias, int bias_mode,
                            void* out, void* y2_out, void* bx_out, int64_t bx_from,

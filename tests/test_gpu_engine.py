@@ -575,9 +575,66 @@ def test_engine_parallel_iir_truncated_fir_branch(T, L, cs):
     with pytest.raises(NotImplementedError):                        # the reference cannot prefill a cache on this branch
         eng.parallel_iir(z_pre.to(DEV), h.to(DEV), Db.to(DEV), L, lp.to(DEV), r.to(DEV), None, dims, 0,
                          inference_params=HyenaCascadeIIRInferenceParams(), long_fir_threshold=T)
-    with pytest.raises(NotImplementedError):
-        eng.parallel_iir(z_pre.to(DEV), h.to(DEV), Db.to(DEV), L, lp.to(DEV), r.to(DEV), None, dims, 0,
-                         long_fir_threshold=200)
+
+
+@pytest.mark.parametrize("T,L,cs", [(200, 1024, False), (129, 515, True), (700, 1500, False)])
+def test_engine_parallel_iir_truncated_fir_longer_than_128(T, L, cs):
+    # a long_fir_threshold beyond the MFMA kernel's 128 taps (vortex/model/engine.py:339-349 takes any): the
+    # direct-form kernel in blocks of 128 lags, same arithmetic, against the oracle's restatement
+    B, D, H = 2, 48, 4
+    g = torch.Generator().manual_seed(T)
+    lp, r = O.make_modal_real(D, 16, seed=T, pmax=0.99)
+    h = O.modal_filter(lp, r, L)
+    z_pre = torch.randn(B, 3 * D, L, generator=g).bfloat16()
+    Db = torch.randn(D, generator=g).bfloat16()
+    dims = (D, H, D // H, 16, D)
+    y_ref, _ = O.parallel_iir(z_pre, h, Db, L, lp, r, dims, column_split_hyena=cs, long_fir_threshold=T)
+    y = HyenaInferenceEngine().parallel_iir(z_pre.to(DEV), h.to(DEV), Db.to(DEV), L, lp.to(DEV), r.to(DEV), None, dims, 0,
+                                            column_split_hyena=cs, long_fir_threshold=T)
+    assert y.shape == (B, L, D) and rel_err(y, y_ref) <= 2e-2
+
+
+@pytest.mark.parametrize("K,L", [(200, 700), (384, 1030), (129, 130)])
+def test_inner_fir_longer_than_128(K, L):
+    # FIR layers longer than 128 taps (vortex/model/engine.py:174-187 takes any length through its FFT): the operator
+    # module and the engine seam against the oracle call sequence, prefill, cache hand-off and decode steps
+    B, D, H, G, n_dec = 2, 64, 4, 4, 3
+    g = torch.Generator().manual_seed(K)
+    p = {"short_filter_weight": torch.randn(3 * D, 1, 3, generator=g) / 3 ** 0.5, "short_filter_bias": None,
+         "h": O.make_mr_filter(G, K, seed=K), "D": torch.randn(D, generator=g).bfloat16()}
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=False, interleave=True, short_filter_length=3,
+               short_filter_bias=False, state_size=16)
+    u_all = torch.randn(B, L + n_dec, 3 * D, generator=g).bfloat16()
+    ref = O.OracleCascade(O.OracleEngine(), p, D, H, G, fir_inner_filter_length=K, interleave=True)
+    ip_ref = O.OracleCache()
+    y_ref, _ = ref.forward(u_all[:, :L], ip_ref)
+    # the engine seam under the reference's own call sequence
+    hip = O.OracleCascade(HyenaInferenceEngine(), to_dev(p), D, H, G, fir_inner_filter_length=K, interleave=True)
+    ip_e = HyenaCascadeFIRInferenceParams()
+    y_e, _ = hip.forward(u_all[:, :L].to(DEV), ip_e)
+    assert rel_err(y_e, y_ref) <= 2e-2
+    # the operator module
+    mod = HyenaCascade(cfg, 0, hyena_filter_groups=G, fir_inner_filter_length=K)
+    with torch.no_grad():
+        mod.short_filter_weight.copy_(p["short_filter_weight"])
+        mod.h.copy_(p["h"])
+        mod.D.data = p["D"].clone()
+    mod = mod.to(DEV)
+    ip_m = HyenaCascadeFIRInferenceParams()
+    y_m, _ = mod(u_all[:, :L].to(DEV), ip_m)
+    assert rel_err(y_m, y_ref) <= 2e-2
+    for i in range(n_dec):
+        tok = u_all[:, L + i: L + i + 1]
+        y_ref, _ = ref.forward(tok, ip_ref)
+        y_e, _ = hip.forward(tok.to(DEV), ip_e)
+        y_m, _ = mod(tok.to(DEV), ip_m)
+        assert rel_err(y_e, y_ref) <= 2e-2 and rel_err(y_m, y_ref) <= 2e-2, i
+    # and the functional entry point on explicit gates
+    import vortex_amd as va
+    x2, x1, v = O.make_gates(B, D, L, seed=K)
+    Df = torch.randn(D, generator=g)
+    got = va.hyena_mr_fwd(x1.to(DEV), x2.to(DEV), v.to(DEV), p["h"].to(DEV), Df.to(DEV))
+    assert rel_err(got, O.mr_fir(x2, x1, v, p["h"], Df)[0]) <= 2e-2
 
 
 @pytest.mark.parametrize("T,G", [(128, 4), (16, 64)])

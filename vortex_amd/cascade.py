@@ -237,7 +237,10 @@ class HyenaCascade(nn.Module):
         K = self.fir_inner_filter_length
         if K:
             taps = self._f32_param("h", (self.h.shape[0], K))
-            if K >= 128:
+            if K > 128:     # no MFMA kernel for such filters: the direct-form kernel on the gates as tensors
+                x2t, x1t, vt = self._split(z_pre)
+                y = ops.fir_fwd_long(x1t, x2t, vt, taps[:, :L], bias=self._f32_param("D"), bias_mode=HYENA_BIAS_GATED_FP32)
+            elif K >= 128:
                 y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, K, device=u.device, bias=self._f32_param("D"),
                                      bias_mode=HYENA_BIAS_GATED_FP32, taps_reversed=False, force_mfma=True)
             else:
@@ -251,15 +254,17 @@ class HyenaCascade(nn.Module):
                 raise NotImplementedError("long_fir_threshold with a cache: the reference has no state prefill on "
                                           "this branch (vortex/model/engine.py:380-392 reads an unassigned X_s)")
             T = min(int(self.long_fir_threshold), L_true)
-            if T > 128:
-                raise NotImplementedError("long_fir_threshold above 128 taps has no kernel")
             with torch.no_grad():
                 h = self.compute_filter(T, u.device)[0][0]
             taps = h.to(torch.bfloat16).to(torch.float32).contiguous()                     # [G, T]
             # (bf16(y) + x1v*D) in the tensors' own dtype (engine.py:351-353): bf16 arithmetic with a bf16 D
             mode = HYENA_BIAS_GATED_BF16 if self.D.dtype == torch.bfloat16 else HYENA_BIAS_GATED_FP32
-            y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, T, device=u.device, bias=self._f32_param("D"),
-                                 bias_mode=mode, taps_reversed=True, force_mfma=True)
+            if T > 128:     # beyond the MFMA kernel's filter length: the direct-form kernel on the gates as tensors
+                x2t, x1t, vt = self._split(z_pre)
+                y = ops.fir_fwd_long(x1t, x2t, vt, taps, bias=self._f32_param("D"), bias_mode=mode, taps_reversed=True)
+            else:
+                y = ops.fir_fwd_rows(r1, r2, rv, taps, B, D, L, T, device=u.device, bias=self._f32_param("D"),
+                                     bias_mode=mode, taps_reversed=True, force_mfma=True)
         else:
             y, _, state = ops.li_fwd_rows(r1, r2, rv, self.modal_plan(), self.D, B, D, L, device=u.device,
                                           want_state=caching)

@@ -845,17 +845,18 @@ extern "C" int hyena_fir_cl_fwd_dtype(const hyena_cl* x1, const hyena_cl* x2, co
                                       void* bx_out, int64_t bx_from, int64_t B, int64_t L, int64_t D, int64_t G, int K,
                                       int dtype, void* stream) {
     const char* who = "hyena_fir_cl_fwd_dtype";
-    if (dtype == HYENA_DTYPE_BF16)
+    if (dtype == HYENA_DTYPE_BF16 && K <= 128)
         return hyena_fir_cl_fwd(x1, x2, v, h, taps_reversed, bias, bias_mode, out, y2_out, bx_out, bx_from, B, L, D, G, K,
                                 stream);
-    if (dtype != HYENA_DTYPE_F16 && dtype != HYENA_DTYPE_F32) return hyena_fail(HYENA_EINVAL, "%s: unknown dtype %d", who, dtype);
+    if (dtype != HYENA_DTYPE_BF16 && dtype != HYENA_DTYPE_F16 && dtype != HYENA_DTYPE_F32)
+        return hyena_fail(HYENA_EINVAL, "%s: unknown dtype %d", who, dtype);
     if (!x1 || !x1->ptr || !h || !out) return hyena_fail(HYENA_EINVAL, "%s: x1, h and out are required", who);
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
     if (pre != post) return hyena_fail(HYENA_ENOSUP, "%s: pass both gates v and x2, or neither", who);
     if (B < 0 || D <= 0 || L < 0 || G <= 0 || D % G != 0 || D >= (1LL << 24))
         return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld L=%lld G=%lld", who, (long long)B, (long long)D,
                           (long long)L, (long long)G);
-    if (K < 1 || K > 128) return hyena_fail(HYENA_ENOSUP, "%s: K=%d outside 1..128", who, K);
+    if (K < 1 || K > (1 << 20)) return hyena_fail(HYENA_ENOSUP, "%s: K=%d outside 1..2^20", who, K);
     if (bias_mode < 0 || bias_mode > 4 || (bias_mode != HYENA_BIAS_NONE && !bias))
         return hyena_fail(HYENA_EINVAL, "%s: bias_mode %d needs a bias pointer", who, bias_mode);
     if (bx_out && (bx_from < 0 || bx_from > L)) return hyena_fail(HYENA_EINVAL, "%s: bx_from outside 0..L", who);
@@ -866,7 +867,7 @@ extern "C" int hyena_fir_cl_fwd_dtype(const hyena_cl* x1, const hyena_cl* x2, co
         return hyena_fail(HYENA_EALIGN, "%s: pointers must be aligned to the element size, time strides non-negative", who);
     if (B == 0 || L == 0) return 0;
     // float16: the MFMA form where its shape and alignment rules hold
-    if (dtype == HYENA_DTYPE_F16 && (D / G) % 16 == 0 && D % 8 == 0 && bias_mode <= HYENA_BIAS_GATED_FP32 && cl_ok(x1) &&
+    if (dtype == HYENA_DTYPE_F16 && K <= 128 && (D / G) % 16 == 0 && D % 8 == 0 && bias_mode <= HYENA_BIAS_GATED_FP32 && cl_ok(x1) &&
         cl_stride_ok(x1) && (!pre || (cl_ok(v) && cl_ok(x2) && cl_stride_ok(v) && cl_stride_ok(x2))) &&
         !(((uintptr_t)out | (uintptr_t)y2_out | (uintptr_t)bx_out) & 15)) {
         LaunchArgs a = {};

@@ -8,10 +8,13 @@
 // the same kernel for shapes the MFMA form does not cover (filter groups that are not multiples of 16 channels,
 // unaligned strides), with the roundings of float16 tensor arithmetic: bx = f16(x1*v), z = f16(conv), out = f16(x2*z).
 //
-// Block = 64 channels x 128 output samples.  bx of the tile and its K-1 samples of history sit in LDS as float32
+// Block = 64 channels x 128 output samples.  bx of the tile and 127 samples of history sit in LDS as float32
 // [row][channel] (a lane reads its own channel: consecutive banks), the taps as [lag][channel].  A thread owns one
 // channel and 32 consecutive outputs; it walks the lags 32 at a time with a 63-sample window of bx in registers, so
-// every product has compile-time register operands: 63 + 32 LDS reads per 1024 FMAs.
+// every product has compile-time register operands: 63 + 32 LDS reads per 1024 FMAs.  Filters longer than 128 taps
+// run as blocks of 128 lags: the same LDS tile is refilled with the rows 128 samples further back and the next 128
+// taps, and the sums carry on in the same registers.  That covers the filter lengths no MFMA kernel is built for
+// (vortex/model/engine.py:174-187 takes any length through its FFT, :339-349 any long_fir_threshold), in bfloat16 too.
 #include <type_traits>
 
 #include "common.h"
@@ -28,6 +31,9 @@ template <> struct ElT<float> {
 };
 template <> struct ElT<_Float16> {
     static __device__ __forceinline__ float rnd(float f) { return (float)(_Float16)f; }     // round to nearest even
+};
+template <> struct ElT<__bf16> {
+    static __device__ __forceinline__ float rnd(float f) { return round_bf(f); }
 };
 
 template <typename T>
@@ -55,56 +61,58 @@ __global__ __launch_bounds__(256) void fir_cl_direct_kernel(ClMapT<T> x1, ClMapT
     const int64_t t0 = (int64_t)tt * DT;
     const bool pre = v.ptr != nullptr, post = x2.ptr != nullptr;
 
-    // taps of this thread's channel by lag (0 = the current sample), zero from K on
-    {
-        const int g = ch_ok ? (int)((uint32_t)d / (uint32_t)dg) : 0;
-        for (int k = tq; k < DK; k += 4) {
+    const int g = ch_ok ? (int)((uint32_t)d / (uint32_t)dg) : 0;
+    // outputs j = 0..31 at t0 + 32*tq + j; LDS row of output j at lag k of the current lag block: base + j - k
+    const int base = (DK - 1) + 32 * tq;
+    float acc[32], ucur[32];
+#pragma unroll
+    for (int j = 0; j < 32; ++j) { acc[j] = 0.f; ucur[j] = 0.f; }
+    // lag blocks of DK = 128: block lb holds lags 128*lb .. 128*lb + 127.  LDS row r holds sample
+    // t0 - 128*lb - (DK-1) + r, so that row base + j - k is sample (t0 + 32*tq + j) - (128*lb + k).
+    for (int lb = 0; lb * DK < K; ++lb) {
+        if (lb) __syncthreads();                       // the tile of the block before has been consumed
+        const int kofs = lb * DK;
+        for (int k = tq; k < DK; k += 4) {             // taps by lag (0 = the current sample), zero from K on
             float val = 0.f;
-            if (ch_ok && k < K) val = h[(int64_t)g * K + (reversed ? K - 1 - k : k)];
+            if (ch_ok && kofs + k < K) val = h[(int64_t)g * K + (reversed ? K - 1 - (kofs + k) : kofs + k)];
             h_lds[k * DC + c] = val;
         }
-    }
-    // bx rows t0 - (K-1) .. t0 + DT - 1 -> LDS rows (DK-1) - (K-1) + r; rows below stay unread (their taps are zero, and
-    // the window clamps its row index at 0, which is then a row of finite values)
-    const int r0 = DK - K;     // LDS row of sample t0 - (K-1)
-    for (int r = tq; r < DT + K - 1; r += 4) {
-        const int64_t t = t0 - (K - 1) + r;
-        float val = 0.f;
-        if (ch_ok && t >= 0 && t < L) {
-            val = (float)x1.ptr[b * x1.bs + t * x1.ts + d];
-            if (pre) val = ElT<T>::rnd(val * (float)v.ptr[b * v.bs + t * v.ts + d]);
-            if (bx_out && r >= K - 1 && t >= bx_from) bx_out[(b * (L - bx_from) + (t - bx_from)) * D + d] = (T)val;
+        for (int r = tq; r < DT + DK - 1; r += 4) {
+            const int64_t t = t0 - kofs - (DK - 1) + r;
+            float val = 0.f;
+            if (ch_ok && t >= 0 && t < L) {
+                val = (float)x1.ptr[b * x1.bs + t * x1.ts + d];
+                if (pre) val = ElT<T>::rnd(val * (float)v.ptr[b * v.bs + t * v.ts + d]);
+                if (lb == 0 && bx_out && r >= DK - 1 && t >= bx_from)
+                    bx_out[(b * (L - bx_from) + (t - bx_from)) * D + d] = (T)val;
+            }
+            bx_lds[r * DC + c] = val;
         }
-        bx_lds[(r0 + r) * DC + c] = val;
-    }
-    if (r0 > 0) {              // rows 0 .. r0-1 are read (times zero taps) when the clamp does not apply: keep them finite
-        for (int r = tq; r < r0; r += 4) bx_lds[r * DC + c] = 0.f;
-    }
-    __syncthreads();
-
-    // outputs j = 0..31 at t0 + 32*tq + j; LDS row of output j at lag k: base + j - k
-    const int base = (DK - 1) + 32 * tq;
-    float acc[32];
+        __syncthreads();
+        if (lb == 0) {
 #pragma unroll
-    for (int j = 0; j < 32; ++j) acc[j] = 0.f;
-    for (int kb = 0; kb < K; kb += 32) {
-        float win[63];
+            for (int j = 0; j < 32; ++j) ucur[j] = bx_lds[(base + j) * DC + c];      // u at the outputs (gated bias)
+        }
+        const int kend = (K - kofs < DK) ? K - kofs : DK;
+        for (int kb = 0; kb < kend; kb += 32) {
+            float win[63];
 #pragma unroll
-        for (int i = 0; i < 63; ++i) win[i] = bx_lds[(base - kb - 31 + i) * DC + c];      // row >= DK-1-96-31 = 0
+            for (int i = 0; i < 63; ++i) win[i] = bx_lds[(base - kb - 31 + i) * DC + c];      // row >= DK-1-96-31 = 0
 #pragma unroll
-        for (int kk = 0; kk < 32; ++kk) {
-            const float hk = h_lds[(kb + kk) * DC + c];
+            for (int kk = 0; kk < 32; ++kk) {
+                const float hk = h_lds[(kb + kk) * DC + c];
 #pragma unroll
-            for (int j = 0; j < 32; ++j) acc[j] = fmaf(hk, win[j - kk + 31], acc[j]);
+                for (int j = 0; j < 32; ++j) acc[j] = fmaf(hk, win[j - kk + 31], acc[j]);
+            }
         }
     }
 
     const float bz = (bias_mode != HYENA_BIAS_NONE && ch_ok) ? bias[d] : 0.f;
-#pragma unroll 4
+#pragma unroll
     for (int j = 0; j < 32; ++j) {
         const int64_t t = t0 + 32 * tq + j;
         if (!ch_ok || t >= L) continue;
-        const float u = bx_lds[(base + j) * DC + c];
+        const float u = ucur[j];
         float z;
         switch (bias_mode) {
             case HYENA_BIAS_ADD:        z = ElT<T>::rnd(ElT<T>::rnd(acc[j]) + bz); break;
@@ -138,14 +146,17 @@ int direct_launch(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, con
 
 }  // namespace
 
-// Direct-form launch for float16 (dtype 1) or float32 (dtype 2) channel-last tensors; arguments as hyena_fir_cl_fwd,
-// already validated by the caller except for what is specific to this form.
+// Direct-form launch for channel-last tensors of any of the three element types, any K >= 1; arguments as
+// hyena_fir_cl_fwd_dtype, already validated by the caller.
 int hyena_fir_cl_direct(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, const float* h, int taps_reversed,
                         const float* bias, int bias_mode, void* out, void* y2_out, void* bx_out, int64_t bx_from,
                         int64_t B, int64_t L, int64_t D, int64_t G, int K, int dtype, void* stream, const char* who) {
     if (dtype == HYENA_DTYPE_F32)
         return direct_launch<float>(x1, x2, v, h, taps_reversed, bias, bias_mode, out, y2_out, bx_out, bx_from, B, L, D,
                                     G, K, stream, who);
+    if (dtype == HYENA_DTYPE_BF16)
+        return direct_launch<__bf16>(x1, x2, v, h, taps_reversed, bias, bias_mode, out, y2_out, bx_out, bx_from, B, L, D,
+                                     G, K, stream, who);
     return direct_launch<_Float16>(x1, x2, v, h, taps_reversed, bias, bias_mode, out, y2_out, bx_out, bx_from, B, L, D, G,
                                    K, stream, who);
 }

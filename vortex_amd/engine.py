@@ -89,6 +89,21 @@ class HyenaInferenceEngine:
                 r1, r2 = r2, r1
             D = hidden
             taps = _group_taps(weight, D, groups)
+            if taps.shape[1] > 128:
+                # longer than any MFMA kernel is built for: the direct-form kernel on the gates as tensors, with the
+                # arithmetic of the K >= 128 branch (engine.py:174-187: true convolution, fp32 `+ D*u`) or of the
+                # short branch (cross-correlation, bias after the cast) by K, as below
+                z2, x1t, vt = self._gate_views(u, hidden, hd)
+                if K >= 128:
+                    mode = HYENA_BIAS_NONE if bias is None else HYENA_BIAS_GATED_FP32
+                    z = ops.fir_fwd_long(x1t, z2, vt, taps[:, :L], bias=ops._f32(bias), bias_mode=mode)
+                else:
+                    mode = HYENA_BIAS_NONE if bias is None else (HYENA_BIAS_GATED_BF16 if gated_bias else HYENA_BIAS_ADD)
+                    z = ops.fir_fwd_long(x1t, z2, vt, taps, bias=ops._f32(bias), bias_mode=mode, taps_reversed=True)
+                state = (x1t[..., -(K - 1):] * vt[..., -(K - 1):]) if inference_params is not None else None
+                if isinstance(padding_mask, torch.Tensor):
+                    z = z * padding_mask[:, None].to(z.dtype)
+                return z, state
             if K >= 128:
                 # true convolution with the fp32 `+ D*u` term (engine.py:174-187, :78)
                 mode = HYENA_BIAS_NONE if bias is None else HYENA_BIAS_GATED_FP32
@@ -134,6 +149,17 @@ class HyenaInferenceEngine:
         if isinstance(padding_mask, torch.Tensor):
             z = z * padding_mask[:, None].to(z.dtype)      # 0/1 masks commute exactly with the gate
         return z, state
+
+    def _gate_views(self, u, hidden, head_dim):
+        """(x2, x1, v) views of the [B, 3D, L] projection (vortex/model/engine.py:150-158), flip applied."""
+        if head_dim is None:
+            x2, x1, v = u.split([hidden, hidden, hidden], dim=1)
+        else:
+            ur = u.reshape(u.shape[0], -1, 3, head_dim, u.shape[-1])
+            x2, x1, v = (ur[:, :, i].reshape(u.shape[0], hidden, u.shape[-1]) for i in range(3))
+        if self.hyena_flip_x1x2:
+            x1, x2 = x2, x1
+        return x2, x1, v
 
     def _gate_tails(self, u, hidden, head_dim, n):
         t = u[..., -n:]
@@ -181,12 +207,14 @@ class HyenaInferenceEngine:
                 raise NotImplementedError("long_fir_threshold with a cache: the reference has no state prefill on "
                                           "this branch (vortex/model/engine.py:380-392 reads an unassigned X_s)")
             T = min(int(long_fir_threshold), h.shape[-1])
-            if T > 128:
-                raise NotImplementedError("long_fir_threshold above 128 taps has no kernel")
             assert h.shape[0] == 1, "batch size must be 1 for long_fir_threshold"
             taps = h[0][:, :T].to(torch.bfloat16).to(torch.float32).contiguous()       # [D, T], bf16-rounded
             # (bf16(y) + x1v*D) in the tensors' own dtype (engine.py:351-353): bf16 arithmetic with a bf16 D
             mode = HYENA_BIAS_GATED_BF16 if D.dtype == torch.bfloat16 else HYENA_BIAS_GATED_FP32
+            if T > 128:     # beyond the MFMA kernel's filter length: direct form on the gates as tensors
+                x2t, x1t, vt = self._gate_views(z_pre, hidden, hd)
+                out = ops.fir_fwd_long(x1t, x2t, vt, taps, bias=ops._f32(D), bias_mode=mode, taps_reversed=True)
+                return out.permute(0, 2, 1)
             out = ops.fir_fwd_rows(r1, r2, rv, taps, B, hidden, L + pad, T, device=z_pre.device, bias=ops._f32(D),
                                    bias_mode=mode, taps_reversed=True, force_mfma=True)
             if pad:

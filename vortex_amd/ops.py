@@ -171,7 +171,7 @@ def fir_cl_fwd(x1, x2, v, taps, *, bias=None, bias_mode=HYENA_BIAS_NONE, taps_re
     bx = torch.empty((B, L - bx_from, D), dtype=dt, device=x1.device) if want_bx else None
     if out.numel():
         c1, c2, cv = _cl_of(x1, dt), _cl_of(x2, dt), _cl_of(v, dt)
-        if dt == torch.bfloat16:
+        if dt == torch.bfloat16 and K <= 128:
             rc = _lib.lib().hyena_fir_cl_fwd(_ref(c1), _ref(c2), _ref(cv), _ptr(taps), int(taps_reversed), _ptr(_f32(bias)),
                                              bias_mode, _ptr(out), _ptr(y2), _ptr(bx), bx_from, B, L, D, G, K, _stream())
         else:
@@ -180,6 +180,16 @@ def fir_cl_fwd(x1, x2, v, taps, *, bias=None, bias_mode=HYENA_BIAS_NONE, taps_re
                                                    B, L, D, G, K, _CL_DTYPES[dt], _stream())
         _lib.check(rc, "hyena_fir_cl_fwd")
     return (out, y2, bx) if (want_y2 or want_bx) else out
+
+
+def fir_fwd_long(x1, x2, v, taps, *, bias=None, bias_mode=HYENA_BIAS_NONE, taps_reversed=False):
+    """Gated FIR with more than 128 taps on [B, D, L] bf16 gates (views welcome): out [B, D, L].
+
+    No MFMA kernel is built for such filters (none of the reference's configurations has one); they run the
+    direct-form channel-last kernel (hyena_fir_cl_fwd_dtype) between two layout changes through torch."""
+    cl = lambda t: None if t is None else t.transpose(1, 2).contiguous()
+    y = fir_cl_fwd(cl(x1), cl(x2), cl(v), taps, bias=bias, bias_mode=bias_mode, taps_reversed=taps_reversed)
+    return y.transpose(1, 2).contiguous()
 
 
 def fir_layer_fwd(u, feat_w, feat_bias, channel_map, taps, *, bias=None, bias_mode=HYENA_BIAS_NONE,
@@ -270,6 +280,8 @@ def hyena_mr_fwd(x1, x2, v, h, D_bias=None):
     taps = _f32(h).reshape(h.shape[0], -1)
     K = taps.shape[1]
     b = _f32(D_bias)
+    if K > 128:
+        return fir_fwd_long(x1, x2, v, taps, bias=b, bias_mode=_bias_mode(b, True, True))
     (x1, pad), (x2, _), (v, _) = front_pad8(x1), front_pad8(x2), front_pad8(v)
     out = fir_fwd_rows(rows_of(x1), rows_of(x2), rows_of(v), taps, B, D, L + pad, K, device=x1.device, bias=b,
                        bias_mode=_bias_mode(b, True, True), taps_reversed=False, force_mfma=True)
