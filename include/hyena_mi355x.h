@@ -64,6 +64,8 @@ const char* hyena_last_error_string(void);
  *   "se_nt", "mr_nt", "li_nt", "cl_nt"         0 = cached, 1 = non-temporal global accesses
  *   "li_cpw"                                    1 / 4 = channels per wavefront in hyena_li_fwd (4 needs D/G % 4 == 0)
  *   "li_coop"                                   0 / 1 = lone / cooperating wavefronts in hyena_li_fwd
+ *   "cl_ns"                                     1 = one 64-channel strip per block in hyena_fir_cl_fwd / layer_fwd, 2 or
+ *                                               more = the form with several strips per block wherever it exists
  * Returns 0, or HYENA_EINVAL for an unknown name. */
 int hyena_set_launch_override(const char* name, int64_t value);
 

@@ -141,12 +141,71 @@ def test_layer_fwd_vs_oracle(B, L, D, H, G, K, Ks, cs, il, flip, sbias, segments
     assert rel_err(bx.permute(0, 2, 1), tail) <= 1e-2
 
 
+@pytest.mark.parametrize("nseg", [1, 3])
+@pytest.mark.parametrize("B,D,G,L,K", [(2, 384, 24, 640, 128), (1, 448, 28, 1333, 128), (1, 400, 25, 700, 7),
+                                       (2, 1024, 64, 300, 17), (1, 384, 6, 2100, 100)])
+def test_cl_several_strips_per_block(B, D, G, L, K, nseg, override):
+    # blocks of three 64-channel strips that share their barriers (what large tensors run): against the oracle and
+    # bit for bit against the one-strip form, with widths that leave the last block one or two empty strips
+    # (448 = 7 strips, 400 = 6.25) and segments along L
+    from vortex_amd._lib import HYENA_BIAS_NONE as NONE
+    x2, x1, v = O.make_gates(B, D, L, seed=L + K)
+    mr = K >= 100
+    h = O.make_mr_filter(G, K, seed=K) if mr else O.make_se_filter(G, K, seed=K)
+    Db = torch.randn(D, generator=torch.Generator().manual_seed(5)) if mr else None
+    ref = (O.mr_fir(x2, x1, v, h, Db) if mr else O.se_fir(x2, x1, v, h))[0]
+    res = []
+    for ns in (3, 1):
+        override(cl_ns=ns, cl_nseg=nseg)
+        res.append(ops.fir_cl_fwd(cl(x1), cl(x2), cl(v), h.reshape(G, K).to(DEV), bias=None if Db is None else Db.to(DEV),
+                                  bias_mode=HYENA_BIAS_GATED_FP32 if mr else NONE, taps_reversed=not mr))
+    assert rel_err(res[0].permute(0, 2, 1), ref) <= 2e-2
+    assert torch.equal(res[0], res[1])
+
+
+@pytest.mark.parametrize("nseg", [1, 2])
+@pytest.mark.parametrize("B,L,D,H,G,K,Ks,cs,il,flip,sbias", [
+    (2, 512, 256, 4, 16, 7, 3, False, True, False, False),
+    (1, 700, 320, 4, 20, 128, 3, False, True, False, True),      # five strips: the last block has an empty one
+    (1, 384, 256, 4, 16, 128, 4, True, False, True, False),      # head-blocked split (head_dim 64), 4-tap featurizer
+])
+def test_layer_fwd_several_strips_per_block(B, L, D, H, G, K, Ks, cs, il, flip, sbias, nseg, override):
+    g = torch.Generator().manual_seed(L + K + Ks)
+    C = 3 * D
+    u = torch.randn(B, L, C, generator=g).bfloat16()
+    wf = torch.randn(C, 1, Ks, generator=g) / Ks ** 0.5
+    bf = torch.randn(C, generator=g).bfloat16() if sbias else None
+    mr = K >= 128
+    h = O.make_mr_filter(G, K, seed=3) if mr else O.make_se_filter(G, K, seed=3)
+    Dcoef = torch.randn(D, generator=g) if mr else None
+    ref, _ = oracle_layer(u, wf, bf, h, Dcoef, D, H, cs, il, flip)
+    cmap = ops.gate_channel_map(D, interleave=il, head_dim=D // H if cs else None)
+    res = []
+    for ns in (2, 1):
+        override(cl_ns=ns, cl_nseg=nseg)
+        res.append(ops.fir_layer_fwd(u.to(DEV), wf.reshape(C, Ks).t().contiguous().to(DEV), None if bf is None else bf.to(DEV),
+                                     cmap, h.reshape(G, K).to(DEV), bias=None if Dcoef is None else Dcoef.to(DEV),
+                                     bias_mode=HYENA_BIAS_GATED_FP32 if mr else HYENA_BIAS_NONE, taps_reversed=not mr,
+                                     flip_x1x2=flip))
+    assert rel_err(res[0].permute(0, 2, 1), ref) <= 2e-2
+    assert torch.equal(res[0], res[1])
+
+
 def test_cl_rejects_unsupported():
     x = torch.zeros(1, 16, 24, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(NotImplementedError):       # 24 channels in 3 groups: group size 8 is not a multiple of 16
         ops.fir_cl_fwd(x, x, x, torch.zeros(3, 4, device=DEV))
-    with pytest.raises(NotImplementedError):
-        ops.fir_cl_fwd(torch.zeros(1, 16, 32, dtype=torch.bfloat16, device=DEV), None, None, torch.zeros(2, 200, device=DEV))
+
+
+def test_cl_filter_longer_than_128_taps_runs_the_direct_form():
+    # no MFMA kernel beyond 128 taps: the direct-form kernel in blocks of 128 lags, ungated, against a float32 conv1d
+    B, D, L, G, K = 2, 32, 700, 2, 200
+    g = torch.Generator().manual_seed(K)
+    x = torch.randn(B, D, L, generator=g).bfloat16()
+    w = torch.randn(G, K, generator=g) / K ** 0.5                      # w[:, 0] on the current sample
+    ref = O.short_fir_fp32(x, w.flip(-1).repeat_interleave(D // G, 0)[:, None], K).bfloat16()
+    y = ops.fir_cl_fwd(cl(x), None, None, w.to(DEV))
+    assert rel_err(y.permute(0, 2, 1), ref) <= 2e-2
 
 
 def test_cl_impulse_response_across_steps_and_segments():

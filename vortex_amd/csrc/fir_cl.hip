@@ -178,8 +178,12 @@ __device__ __forceinline__ void lane_gates(const u32x4 (&raw)[3][KS + 3], const 
 // NT = non-temporal accesses for tensors that stream through the last-level cache: the output rows always, the
 // input rows only without the fused featurizer (its lanes re-read their neighbours' rows, which must stay cached).
 // ET = element traits of the 16-bit tensors (ElBf16, or ElF16 without the featurizer).
-template <typename ET, bool PRE, bool POST, int BIAS, int FEAT, int KS, bool AUX, int MLO, bool NT>
-__global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMap v, ProjFwd pj,
+// NS = strips of 64 channels per block.  With NS > 1 a block is NS groups of four wavefronts, each working on its own
+// strip with its own LDS tiles exactly as a block of the NS = 1 form does; all they share is the two barriers of a
+// step, which keeps neighbouring strips of the same time rows in step, so that their requests for adjacent 128-byte
+// (384-byte with the featurizer) pieces of a row reach the memory system together.
+template <typename ET, bool PRE, bool POST, int BIAS, int FEAT, int KS, bool AUX, int MLO, bool NT, int NS = 1>
+__global__ __launch_bounds__(256 * NS, NS == 1 ? 2 : 1) void fir_cl_kernel(ClMap x1, ClMap x2, ClMap v, ProjFwd pj,
                                                         const float* __restrict__ h, int K, int reversed,
                                                         const float* __restrict__ bias, bf16_t* __restrict__ out,
                                                         bf16_t* __restrict__ y2_out, bf16_t* __restrict__ bx_out,
@@ -189,18 +193,23 @@ __global__ __launch_bounds__(256, 2) void fir_cl_kernel(ClMap x1, ClMap x2, ClMa
     constexpr int RF = FEAT ? KS - 1 : 0;          // extra rows a lane reads before its own four
     constexpr int NR = 4 + RF;                     // rows per lane and load piece
     constexpr int NP = (FEAT || (PRE && POST)) ? 3 : (PRE ? 2 : 1);   // load pieces per row
-    __shared__ __attribute__((aligned(16))) bf16_t u_lds[CB * URS];
-    __shared__ __attribute__((aligned(16))) bf16_t z_lds[CB * ZRS];
-    __shared__ __attribute__((aligned(16))) float w_lds[FEAT ? (KS + 1) * 3 * CB : 4];
+    __shared__ __attribute__((aligned(16))) bf16_t u_lds_all[NS * CB * URS];
+    __shared__ __attribute__((aligned(16))) bf16_t z_lds_all[NS * CB * ZRS];
+    __shared__ __attribute__((aligned(16))) float w_lds_all[FEAT ? NS * (KS + 1) * 3 * CB : 4];
 
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int sub = NS == 1 ? 0 : __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));     // this thread's strip
+    bf16_t* const u_lds = u_lds_all + sub * CB * URS;
+    bf16_t* const z_lds = z_lds_all + sub * CB * ZRS;
+    float* const w_lds = w_lds_all + (FEAT ? sub * (KS + 1) * 3 * CB : 0);
+    const int tid = threadIdx.x & 255, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t bid = blockIdx.x;
     // channel blocks fastest: the blocks resident at one time read neighbouring 128-byte pieces of the same rows.
     // Workgroups are dealt to the 8 XCDs in turn (id mod 8), so every XCD takes every eighth channel block of all
     // row tiles; giving an XCD neighbouring channel blocks (0.457 -> 0.509 ms with the gates given as tensors), whole
     // row tiles (0.488 ms) or an eighth of the block order (0.487 ms) all measured slower.
-    const uint32_t db = bid % (uint32_t)ndb;
+    // (ndb counts blocks: groups of NS strips; a strip past the last channel runs empty but meets every barrier)
+    const uint32_t db = (bid % (uint32_t)ndb) * NS + sub;
     const int seg = (int)((bid / (uint32_t)ndb) % (uint32_t)nseg);
     const int64_t b = bid / ((uint32_t)nseg * (uint32_t)ndb);
     const uint32_t d0 = db * CB;
@@ -714,7 +723,17 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     const bool aux = y2_out || bx_out;
     const bool shortk = K <= 17 && a.pre && bias_mode == HYENA_BIAS_NONE;
     const double halo_cost = shortk ? 40.0 : (double)TL;
-    const int64_t ndb = (D + CB - 1) / CB;
+    // Strips of 64 channels per block (see the kernel): three with the gates given, two with the featurizer fused in
+    // (its registers allow two wavefronts per SIMD), for bfloat16 launches without intermediates on tensors that stream
+    // through the last-level cache.  Measured against one strip per block on tensors of 0.5 to 8.6 GB (D = 1024 .. 8192,
+    // rows of 8192 .. 262144 samples, 7 and 128 taps): 3-14 % less time with the gates given, 1-11 % for the fused layers;
+    // tensors that stay in the cache lose 2-11 %, as do rows shorter than 4096 samples in the fused form.
+    const bool streams = 8.0 * (double)B * (double)D * (double)L > 384e6;
+    const int ns_form = a.feat ? 2 : 3;
+    const bool ns_able = !(y2_out || bx_out) && !a.f16 && (D + CB - 1) / CB >= 2 * ns_form;
+    int ns = (ns_able && streams && L >= 4096) ? ns_form : 1;
+    { const int64_t x = hyena_override(HYENA_OV_CL_NS); if (x >= 1) ns = (x > 1 && ns_able) ? ns_form : 1; }
+    const int64_t ndb = ((D + CB - 1) / CB + ns - 1) / ns;       // blocks along the channels
     const int64_t rows = B * ndb;
     int64_t nseg = 1;
     {
@@ -723,7 +742,8 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
         for (int64_t c = 1; c <= (max_seg < 1 ? 1 : max_seg); ++c) {
             const int64_t sl = ((L + c - 1) / c + TL - 1) / TL * TL;
             const int64_t nb = rows * ((L + sl - 1) / sl);
-            const double fill = (double)nb / (double)((nb + 511) / 512 * 512);
+            const int64_t resident = ns == 1 ? 512 : 256;
+            const double fill = (double)nb / (double)((nb + resident - 1) / resident * resident);
             const double score = fill * (double)sl / ((double)sl + halo_cost);
             if (score > best + 1e-9) { best = score; nseg = c; }
         }
@@ -739,13 +759,21 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     dim3 grid((unsigned)nblk);
     const int dg = (int)(D / G);
     // tensors larger than the last-level cache stream through it: non-temporal accesses then
-    bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
+    bool nt = streams;
     { const int64_t x = hyena_override(HYENA_OV_CL_NT); if (x >= 0) nt = x != 0; }
     bool ok = false;
+#define CL_GO_NS(T, P, Q, M, F, KSV, AX, ML, N, NSV)                                                                 \
+    hipLaunchKernelGGL((fir_cl_kernel<T, P, Q, M, F, KSV, AX, ML, N, NSV>), grid, dim3(256 * NSV), 0, s, a.x1, a.x2, a.v, \
+                       a.pj, h, K, taps_reversed, bias, (bf16_t*)out, (bf16_t*)y2_out, (bf16_t*)bx_out, bx_from, L, D, \
+                       dg, seg_len, (int)nseg, (int)ndb)
+// several strips per block: bfloat16 without intermediates only (three strips with the gates given, two with the featurizer)
 #define CL_GO_T(T, P, Q, M, F, KSV, AX, ML, N)                                                                       \
-    hipLaunchKernelGGL((fir_cl_kernel<T, P, Q, M, F, KSV, AX, ML, N>), grid, dim3(256), 0, s, a.x1, a.x2, a.v, a.pj, h, \
-                       K, taps_reversed, bias, (bf16_t*)out, (bf16_t*)y2_out, (bf16_t*)bx_out, bx_from, L, D, dg,   \
-                       seg_len, (int)nseg, (int)ndb)
+    do {                                                                                                             \
+        if constexpr (!(AX) && std::is_same<T, ElBf16>::value) {                                                     \
+            if (ns > 1) { CL_GO_NS(T, P, Q, M, F, KSV, false, ML, N, ((F) == 0 ? 3 : 2)); break; }                   \
+        }                                                                                                            \
+        CL_GO_NS(T, P, Q, M, F, KSV, AX, ML, N, 1);                                                                  \
+    } while (0)
 // float16 only exists for the form with the gates given as tensors (F == 0)
 #define CL_GO(P, Q, M, F, KSV, AX, ML, N)                                                                         \
     do {                                                                                                          \
@@ -779,6 +807,7 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
 #undef CL_CASE
 #undef CL_GO
 #undef CL_GO_T
+#undef CL_GO_NS
     if (!ok) return hyena_fail(HYENA_ENOSUP, "%s: this gate / bias / featurizer-length combination has no kernel", who);
     return hyena_check_launch(who);
 }
