@@ -195,8 +195,9 @@ def test_argument_errors():
     r = ops.rows_of(x)
     with pytest.raises(ValueError):
         ops.fir_fwd_rows(r, r, r, torch.zeros(2, 7, device="cuda"), 1, 32, 60, 7, device=x.device)
-    with pytest.raises(NotImplementedError):              # K > 128
-        va.hyena_mr_fwd(x, x, x, torch.zeros(2, 1, 200, device="cuda"))
+    with pytest.raises(NotImplementedError):              # K > 128 has no MFMA kernel (the C entry point says so;
+        ops.fir_fwd_rows(r, r, r, torch.zeros(2, 200, device="cuda"), 1, 32, 64, 200, device=x.device, force_mfma=True)
+    assert va.hyena_mr_fwd(x, x, x, torch.zeros(2, 1, 200, device="cuda")).shape == x.shape     # hyena_mr_fwd takes the direct form)
     with pytest.raises(TypeError):
         va.hyena_se_fwd(x.float(), x, x, torch.zeros(2, 1, 7, device="cuda"))
     out = va.hyena_se_fwd(x[:0], x[:0], x[:0], torch.zeros(2, 1, 7, device="cuda"))     # empty batch
