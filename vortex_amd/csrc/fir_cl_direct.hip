@@ -8,8 +8,11 @@
 // the same kernel for shapes the MFMA form does not cover (filter groups that are not multiples of 16 channels,
 // unaligned strides), with the roundings of float16 tensor arithmetic: bx = f16(x1*v), z = f16(conv), out = f16(x2*z).
 //
-// Block = 64 channels x 128 output samples.  bx of the tile and 127 samples of history sit in LDS as float32
-// [row][channel] (a lane reads its own channel: consecutive banks), the taps as [lag][channel].  A thread owns one
+// Block = 64 channels x 128 output samples.  bx of the tile and up to 127 samples of history sit in LDS as float32
+// [row][channel] (a lane reads its own channel: consecutive banks), the taps as [lag][channel], or as one row where
+// the block's channels share a filter; the LDS is sized by the filter length, so short filters fit several blocks per CU.
+// Global requests go out in batches with clamped addresses and no branch around them (rows of bx sixteen per thread at
+// a time, the output gate's thirty-two at the start), so that a batch costs one memory round trip, not one per row.  A thread owns one
 // channel and 32 consecutive outputs; it walks the lags 32 at a time with a 63-sample window of bx in registers, so
 // every product has compile-time register operands: 63 + 32 LDS reads per 1024 FMAs.  Filters longer than 128 taps
 // run as blocks of 128 lags: the same LDS tile is refilled with the rows 128 samples further back and the next 128
@@ -42,15 +45,20 @@ struct ClMapT {                // channel-last operand: (b, t, d) at ptr + b*bs 
     int64_t bs, ts;
 };
 
+// NGB = filter groups a block of 64 channels can touch: its tap table is [lag][NGB], read as a broadcast by the lanes
+// of one group (one column when groups are multiples of 64 channels, 64 columns with one filter per channel).
 template <typename T>
 __global__ __launch_bounds__(256) void fir_cl_direct_kernel(ClMapT<T> x1, ClMapT<T> x2, ClMapT<T> v,
                                                             const float* __restrict__ h, int K, int reversed,
                                                             const float* __restrict__ bias, int bias_mode,
                                                             T* __restrict__ out, T* __restrict__ y2_out,
                                                             T* __restrict__ bx_out, int64_t bx_from, int64_t L,
-                                                            int64_t D, int dg, int ndb, int ntt) {
-    __shared__ float bx_lds[(DT + DK - 1) * DC];
-    __shared__ float h_lds[DK * DC];
+                                                            int64_t D, int dg, int ndb, int ntt, int KP, int NGB,
+                                                            int G) {
+    // KP = lags per lag block held in LDS: min(K, 128) rounded up to 32.  bx rows: DT + KP - 1; tap rows: KP.
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float* const bx_lds = smem;
+    float* const h_lds = smem + (DT + KP - 1) * DC;
     const int tid = threadIdx.x, c = tid & (DC - 1), tq = tid >> 6;
     const uint32_t bid = blockIdx.x;
     const uint32_t db = bid % (uint32_t)ndb;
@@ -58,60 +66,90 @@ __global__ __launch_bounds__(256) void fir_cl_direct_kernel(ClMapT<T> x1, ClMapT
     const int64_t b = bid / ((uint32_t)ndb * (uint32_t)ntt);
     const int64_t d = (int64_t)db * DC + c;
     const bool ch_ok = d < D;
+    const int64_t dcl = ch_ok ? d : D - 1;             // a channel that exists, for requests whose result is dropped
     const int64_t t0 = (int64_t)tt * DT;
     const bool pre = v.ptr != nullptr, post = x2.ptr != nullptr;
+    const int nrows = DT + KP - 1;
 
-    const int g = ch_ok ? (int)((uint32_t)d / (uint32_t)dg) : 0;
+    const int g0 = (int)(((uint32_t)db * DC) / (uint32_t)dg);              // first filter group of the block
+    const int gl = (int)((uint32_t)dcl / (uint32_t)dg) - g0;             // this thread's column of the tap table
     // outputs j = 0..31 at t0 + 32*tq + j; LDS row of output j at lag k of the current lag block: base + j - k
-    const int base = (DK - 1) + 32 * tq;
+    const int base = (KP - 1) + 32 * tq;
     float acc[32], ucur[32];
 #pragma unroll
     for (int j = 0; j < 32; ++j) { acc[j] = 0.f; ucur[j] = 0.f; }
-    // lag blocks of DK = 128: block lb holds lags 128*lb .. 128*lb + 127.  LDS row r holds sample
-    // t0 - 128*lb - (DK-1) + r, so that row base + j - k is sample (t0 + 32*tq + j) - (128*lb + k).
-    for (int lb = 0; lb * DK < K; ++lb) {
-        if (lb) __syncthreads();                       // the tile of the block before has been consumed
-        const int kofs = lb * DK;
-        for (int k = tq; k < DK; k += 4) {             // taps by lag (0 = the current sample), zero from K on
-            float val = 0.f;
-            if (ch_ok && kofs + k < K) val = h[(int64_t)g * K + (reversed ? K - 1 - (kofs + k) : kofs + k)];
-            h_lds[k * DC + c] = val;
+    // the output gate of this thread's 32 samples: requested now, used at the end (clamped addresses, no branch around
+    // a request: the thirty-two travel together instead of one round trip each)
+    T gate[32];
+    if (post) {
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            int64_t t = t0 + 32 * tq + j;
+            t = t < L ? t : L - 1;
+            gate[j] = x2.ptr[b * x2.bs + t * x2.ts + dcl];
         }
-        for (int r = tq; r < DT + DK - 1; r += 4) {
-            const int64_t t = t0 - kofs - (DK - 1) + r;
-            float val = 0.f;
-            if (ch_ok && t >= 0 && t < L) {
-                val = (float)x1.ptr[b * x1.bs + t * x1.ts + d];
-                if (pre) val = ElT<T>::rnd(val * (float)v.ptr[b * v.bs + t * v.ts + d]);
-                if (lb == 0 && bx_out && r >= DK - 1 && t >= bx_from)
-                    bx_out[(b * (L - bx_from) + (t - bx_from)) * D + d] = (T)val;
+    }
+    // lag blocks of KP <= 128: block lb holds lags KP*lb .. KP*lb + KP - 1.  LDS row r holds sample
+    // t0 - KP*lb - (KP-1) + r, so that row base + j - k is sample (t0 + 32*tq + j) - (KP*lb + k).
+    for (int lb = 0; lb * KP < K; ++lb) {
+        if (lb) __syncthreads();                       // the tile of the block before has been consumed
+        const int kofs = lb * KP;
+        // taps by lag (0 = the current sample), zero from K on
+        for (int e = tid; e < KP * NGB; e += 256) {
+            const int kk = e / NGB, gc = e - kk * NGB;
+            const int k = kofs + kk, gg = g0 + gc;
+            const int kc = k < K ? k : K - 1, gcl = gg < G ? gg : G - 1;
+            const float val = h[(int64_t)gcl * K + (reversed ? K - 1 - kc : kc)];
+            h_lds[e] = (k < K && gg < G) ? val : 0.f;
+        }
+        // rows of bx, sixteen per thread at a time: every request of a pass goes out before the first is used
+        const int64_t tfirst = t0 - kofs - (KP - 1);
+        for (int r0 = 0; r0 < nrows; r0 += 64) {
+            T xa[16], va[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                int64_t t = tfirst + r0 + tq + 4 * i;
+                t = t < 0 ? 0 : (t < L ? t : L - 1);
+                xa[i] = x1.ptr[b * x1.bs + t * x1.ts + dcl];
+                if (pre) va[i] = v.ptr[b * v.bs + t * v.ts + dcl];
             }
-            bx_lds[r * DC + c] = val;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int r = r0 + tq + 4 * i;
+                const int64_t t = tfirst + r;
+                float val = (float)xa[i];
+                if (pre) val = ElT<T>::rnd(val * (float)va[i]);
+                if (!(ch_ok && t >= 0 && t < L)) val = 0.f;
+                if (r < nrows) {
+                    bx_lds[r * DC + c] = val;
+                    if (lb == 0 && bx_out && ch_ok && r >= KP - 1 && t < L && t >= bx_from)
+                        bx_out[(b * (L - bx_from) + (t - bx_from)) * D + d] = (T)val;
+                }
+            }
         }
         __syncthreads();
         if (lb == 0) {
 #pragma unroll
             for (int j = 0; j < 32; ++j) ucur[j] = bx_lds[(base + j) * DC + c];      // u at the outputs (gated bias)
         }
-        const int kend = (K - kofs < DK) ? K - kofs : DK;
+        const int kend = (K - kofs < KP) ? K - kofs : KP;
         for (int kb = 0; kb < kend; kb += 32) {
             float win[63];
 #pragma unroll
-            for (int i = 0; i < 63; ++i) win[i] = bx_lds[(base - kb - 31 + i) * DC + c];      // row >= DK-1-96-31 = 0
+            for (int i = 0; i < 63; ++i) win[i] = bx_lds[(base - kb - 31 + i) * DC + c];      // row >= (KP-1) - (KP-32) - 31 = 0
 #pragma unroll
             for (int kk = 0; kk < 32; ++kk) {
-                const float hk = h_lds[(kb + kk) * DC + c];
+                const float hk = h_lds[(kb + kk) * NGB + gl];
 #pragma unroll
                 for (int j = 0; j < 32; ++j) acc[j] = fmaf(hk, win[j - kk + 31], acc[j]);
             }
         }
     }
 
-    const float bz = (bias_mode != HYENA_BIAS_NONE && ch_ok) ? bias[d] : 0.f;
+    const float bz = bias_mode != HYENA_BIAS_NONE ? bias[dcl] : 0.f;
 #pragma unroll
     for (int j = 0; j < 32; ++j) {
         const int64_t t = t0 + 32 * tq + j;
-        if (!ch_ok || t >= L) continue;
         const float u = ucur[j];
         float z;
         switch (bias_mode) {
@@ -121,10 +159,12 @@ __global__ __launch_bounds__(256) void fir_cl_direct_kernel(ClMapT<T> x1, ClMapT
             case HYENA_BIAS_GATED_BF16: z = ElT<T>::rnd(ElT<T>::rnd(acc[j]) + ElT<T>::rnd(bz * u)); break;   // element-type tensor arithmetic
             default:                    z = ElT<T>::rnd(acc[j]);
         }
-        const int64_t o = (b * L + t) * D + d;
-        if (y2_out) y2_out[o] = (T)z;
-        if (post) z = ElT<T>::rnd(z * (float)x2.ptr[b * x2.bs + t * x2.ts + d]);
-        out[o] = (T)z;
+        if (ch_ok && t < L) {
+            const int64_t o = (b * L + t) * D + d;
+            if (y2_out) y2_out[o] = (T)z;
+            if (post) z = ElT<T>::rnd(z * (float)gate[j]);
+            out[o] = (T)z;
+        }
     }
 }
 
@@ -138,9 +178,20 @@ int direct_launch(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, con
     ClMapT<T> m2 = {nullptr, 0, 0}, mv = {nullptr, 0, 0};
     if (x2 && x2->ptr) m2 = {(const T*)x2->ptr, x2->batch_stride, x2->time_stride};
     if (v && v->ptr) mv = {(const T*)v->ptr, v->batch_stride, v->time_stride};
-    hipLaunchKernelGGL((fir_cl_direct_kernel<T>), dim3((unsigned)(B * ndb * ntt)), dim3(256), 0, (hipStream_t)stream, m1,
-                       m2, mv, h, K, taps_reversed, bias, bias_mode, (T*)out, (T*)y2_out, (T*)bx_out, bx_from, L, D,
-                       (int)(D / G), (int)ndb, (int)ntt);
+    const int KP = ((K < DK ? K : DK) + 31) / 32 * 32;
+    const int64_t dg = D / G;
+    // filter groups a block of 64 consecutive channels (starting at a multiple of 64) can touch
+    const int NGB = dg % DC == 0 ? 1 : (DC % dg == 0 ? (int)(DC / dg) : (int)((DC - 1) / dg + 2));
+    const size_t lds = ((size_t)(DT + KP - 1) * DC + (size_t)KP * NGB) * sizeof(float);
+    const dim3 grid((unsigned)(B * ndb * ntt));
+    static bool big = false;                            // allow more than the default dynamic LDS, once per instantiation
+    if (!big) {
+        (void)hipFuncSetAttribute((const void*)fir_cl_direct_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);
+        big = true;
+    }
+    hipLaunchKernelGGL((fir_cl_direct_kernel<T>), grid, dim3(256), lds, (hipStream_t)stream, m1, m2, mv, h, K,
+                       taps_reversed, bias, bias_mode, (T*)out, (T*)y2_out, (T*)bx_out, bx_from, L, D, (int)dg, (int)ndb,
+                       (int)ntt, KP, NGB, (int)G);
     return hyena_check_launch(who);
 }
 
