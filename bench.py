@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="mr", choices=["mr", "se", "se_b8", "li", "li_g4096", "decode", "mr_cl", "mr_layer", "li_layer",
-                                                         "se_layer"])
+                                                         "se_layer", "mr_cl_f16", "cl_f32"])
     ap.add_argument("--settle-ms", type=float, default=150.0,
                     help="untimed run of each workload before its warm-up steps, until clocks have settled")
     ap.add_argument("--no-extras", action="store_true")
@@ -172,6 +172,22 @@ def build_workload(name, device):
             what, keep = ("hyena_mr" if mr else "hyena_se") + "_layer featurizer+operator from the projection", (u, wf, h, Db, out)
         return fn, dict(workload=f"{what} B={B} L={L} D={D} groups={G} K={K}", tokens=B * L, bytes=8 * B * D * L,
                         kernel="fir_cl_kernel", keep=keep)
+    if name in ("mr_cl_f16", "cl_f32"):
+        # the element types of the reference's own grid for this operator (vortex/ops/hyena_se/tests/test_fwd.py:25-54):
+        # float16 on the MFMA kernel at the config-2 shape, float32 on the direct-form kernel at the grid's largest
+        # case (batch 2, seqlen 8192, d 4096, one filter group, 128 taps from N(0, 1))
+        f16 = name == "mr_cl_f16"
+        B, D, L, G, K = (2, 4096, 32768, 256, 128) if f16 else (2, 4096, 8192, 1, 128)
+        dt = torch.float16 if f16 else torch.float32
+        g = torch.Generator(device=device).manual_seed(11)
+        x = [torch.randn(B, L, D, generator=g, device=device, dtype=torch.float32).to(dt) for _ in range(3)]
+        h = (O.make_mr_filter(G, K) if f16 else torch.randn(G, 1, K, generator=torch.Generator().manual_seed(12))).reshape(G, K).to(device)
+        out = torch.empty(B, L, D, dtype=dt, device=device)
+        fn = lambda: ops.fir_cl_fwd(x[1], x[0], x[2], h, taps_reversed=True, out=out)
+        es = 2 if f16 else 4
+        return fn, dict(workload=f"gated FIR on (b, l, g, dg) tensors, {'float16 (MFMA)' if f16 else 'float32 (direct form)'} "
+                                 f"B={B} L={L} D={D} groups={G} K={K}", tokens=B * L, bytes=4 * es * B * D * L,
+                        kernel="fir_cl_kernel" if f16 else "fir_cl_direct_kernel", flops=2.0 * K * B * D * L, keep=(x, h, out))
     if name == "li_layer":
         # a whole Hyena-LI layer from the projection at the config-3 shape: featurizer + split + x1*v in one launch
         # (rows xv, x2), then the modal scan on them; 8 bytes per output element would be a one-pass layer, the two
@@ -555,8 +571,12 @@ def main():
                 continue
             steps = max(3, min(args.steps, 20 if name.startswith("li") else args.steps))
             extra[name] = entry(run(name, steps, extra_warmup))
-        for name in ("mr_cl", "mr_layer", "se_layer", "li_layer"):
-            extra[name] = entry(run(name, max(3, min(args.steps, 10 if name == "li_layer" else 20)), extra_warmup))
+        for name in ("mr_cl", "mr_layer", "se_layer", "li_layer", "mr_cl_f16", "cl_f32"):
+            e = run(name, max(3, min(args.steps, 10 if name == "li_layer" else 20)), extra_warmup)
+            extra[name] = entry(e)
+            if "flops" in e:    # the float32 form runs on the vector ALUs; the published float32 peak is the matrix cores'
+                tf = e["flops"] / (e["kernel_ms"] * 1e-3) / 1e12
+                extra[name].update(tflops=tf, frac_of_fp32_mfma_peak=tf / 157.3)
         for D in (4096, 8192):
             extra[f"decode_D{D}"] = decode_layer_set(D, device, max(args.steps, 50), max(args.warmup, 5))
         extra["decode_from_projection_D4096"] = decode_layers_from_projection(4096, device, max(args.steps, 50),
