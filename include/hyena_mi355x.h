@@ -152,7 +152,7 @@ int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v
 /* hyena_li_plan + hyena_li_fwd in a form that allocates nothing and takes no workspace.  No counterpart in the
  * reference: it is for callers that cannot allocate device memory or keep a workspace alive -- code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  The coefficient tables go into a static device
- * array inside the library (6 KB per filter group; at most 4096 groups = 24 MiB, which each GPU the library runs
+ * array inside the library (6 KB per filter group; at most 8192 groups = 48 MiB, which each GPU the library runs
  * on holds until the process ends); more groups are refused with HYENA_ENOSUP.  The tables are rebuilt from
  * log_poles / residues ([G][S][2] float32) on every call, on `stream`, ahead of the main launch.  Same arguments,
  * arithmetic and results as hyena_li_fwd otherwise.  Every call on a GPU shares that GPU's array: calls that

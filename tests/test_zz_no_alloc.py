@@ -59,9 +59,9 @@ def test_static_form_matches_workspace_form_twice_in_a_row():
 def test_static_form_rejects_more_groups_than_its_table_holds():
     L_ = _lib.lib()
     P = 4096
-    r = _lib.Rows(P, 8192 * 64, 64, 8192, 8192)
+    r = _lib.Rows(P, 16384 * 64, 64, 16384, 16384)
     rc = L_.hyena_li_fwd_static(ctypes.byref(r), ctypes.byref(r), ctypes.byref(r), P, P, None, 1, P, None, None,
-                                1, 8192, 64, 8192, 16, None)
-    assert rc == -3 and b"4096" in L_.hyena_last_error_string()
+                                1, 16384, 64, 16384, 16, None)
+    assert rc == -3 and b"8192" in L_.hyena_last_error_string()
     with pytest.raises(NotImplementedError):
         _lib.check(rc, "hyena_li_fwd_static")

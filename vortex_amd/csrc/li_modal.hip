@@ -720,7 +720,9 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
 // must not use the array's name as an address: each device holds its own copy, whose address is looked up
 // once per device (hipGetSymbolAddress with that device current) and kept.
 namespace {
-constexpr int64_t LI_STATIC_MAX_GROUPS = 4096;                 // 24 MiB per device, held until the process ends
+constexpr int64_t LI_STATIC_MAX_GROUPS = 8192;                 // 48 MiB per device, held until the process ends: the
+                                                               // largest filter bank of the reference's configurations
+                                                               // (hcl_filter_groups: 8192, configs/evo2-40b-8k.yml)
 constexpr int LI_STATIC_MAX_DEVICES = 64;
 static __device__ __align__(256) float scratch[LI_STATIC_MAX_GROUPS * WS_GROUP];
 std::mutex g_scratch_mu;
