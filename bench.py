@@ -45,6 +45,9 @@ def parse():
     ap.add_argument("--no-model", action="store_true", help="skip the end-to-end model prefill legs")
     ap.add_argument("--no-copy-probe", action="store_true",
                     help="skip the plain 1 GiB device copy whose rate is reported as roofline.copy_probe_gbs")
+    ap.add_argument("--launch-override", action="append", default=[], metavar="NAME=VALUE",
+                    help="pin one launch-shape choice of the library for the whole run (hyena_set_launch_override), "
+                         "e.g. cl_ns=1 for one channel strip per block; recorded in config.launch_overrides")
     return ap.parse_args()
 
 
@@ -511,6 +514,12 @@ def main():
     torch.cuda.set_device(device)
     global SETTLE_S
     SETTLE_S = max(args.settle_ms, 0.0) / 1e3
+    from vortex_amd import _lib
+    overrides = {}
+    for item in args.launch_override:
+        k, _, v = item.partition("=")
+        overrides[k] = int(v)
+        _lib.check(_lib.lib().hyena_set_launch_override(k.encode(), int(v)), "hyena_set_launch_override")
 
     def run(name, steps, warmup):
         fn, d = build_workload(name, device)
@@ -529,7 +538,6 @@ def main():
     if not args.no_copy_probe:
         # the practical ceiling beside the nominal 8 TB/s: a plain device copy with the kernels' own access shape
         # (16 bytes per lane), 1 GiB read + 1 GiB written per launch
-        from vortex_amd import _lib
         a = torch.empty(1 << 29, dtype=torch.bfloat16, device=device).normal_()
         b = torch.empty_like(a)
         stream = torch.cuda.current_stream().cuda_stream
@@ -547,7 +555,8 @@ def main():
         "value": m["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": m["wall_s"] / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16 in/out, fp32 accumulate", "data": "synthetic",
-        "config": {"workload": m["workload"], "settle_ms": args.settle_ms},
+        "config": {"workload": m["workload"], "settle_ms": args.settle_ms,
+                   **({"launch_overrides": overrides} if overrides else {})},
         "roofline": {"bound": "hbm", "achieved": m["hbm_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": m["hbm_gbs"] / HBM_PEAK_GBS, "copy_probe_gbs": copy_gbs,
                      "copy_probe": "hyena_copy_probe: 1 GiB read + 1 GiB written per launch, 16 bytes per lane, timed "
