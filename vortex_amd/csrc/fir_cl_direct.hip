@@ -184,10 +184,16 @@ int direct_launch(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, con
     const int NGB = dg % DC == 0 ? 1 : (DC % dg == 0 ? (int)(DC / dg) : (int)((DC - 1) / dg + 2));
     const size_t lds = ((size_t)(DT + KP - 1) * DC + (size_t)KP * NGB) * sizeof(float);
     const dim3 grid((unsigned)(B * ndb * ntt));
-    static bool big = false;                            // allow more than the default dynamic LDS, once per instantiation
-    if (!big) {
-        (void)hipFuncSetAttribute((const void*)fir_cl_direct_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);
-        big = true;
+    // more than the default dynamic LDS: asked for once per device and instantiation (the attribute belongs to the
+    // function as loaded on one device)
+    static bool big[64] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+    if (dev < 0 || !big[dev]) {
+        const hipError_t e = hipFuncSetAttribute((const void*)fir_cl_direct_kernel<T>,
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);
+        if (e != hipSuccess) return hyena_fail((int)e, "%s: hipFuncSetAttribute: %s", who, hipGetErrorString(e));
+        if (dev >= 0) big[dev] = true;
     }
     hipLaunchKernelGGL((fir_cl_direct_kernel<T>), grid, dim3(256), lds, (hipStream_t)stream, m1, m2, mv, h, K,
                        taps_reversed, bias, bias_mode, (T*)out, (T*)y2_out, (T*)bx_out, bx_from, L, D, (int)dg, (int)ndb,
