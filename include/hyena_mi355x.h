@@ -149,6 +149,27 @@ int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v
                  void* out, float* y_conv_fp32, float* state_out,
                  int64_t B, int64_t D, int64_t L, int64_t G, int64_t S, void* stream);
 
+/* A whole Hyena-LI layer in one pass over a projection that is stored sequence-major: the featurizer FIR
+ * (HyenaCascade.parallel_forward's first parallel_fir call, vortex/model/model.py:233-246, i.e.
+ * vortex/model/engine.py:188-223 with gate = False), the split into x2 | x1 | v with or without `interleave` /
+ * column_split (vortex/model/model.py:250-252, vortex/model/utils.py:26-85) and parallel_iir with its state prefill
+ * (vortex/model/engine.py:283-353, :525-559), 6 bytes read and 2 written per (batch, channel, sample):
+ *   f_i[t] = bf16(w_i[d][0]*p_i[t-2] + w_i[d][1]*p_i[t-1] + w_i[d][2]*p_i[t])     i = x1, x2, v; p_i = the rows given
+ *   out    = hyena_li_fwd on (x1, x2, v) = (f_x1, f_x2, f_v)
+ * x1, x2, v describe rows of the RAW projection p [B][3D][L] (L contiguous) -- what the producing GEMM writes when it
+ * is asked for the transposed product; the reference permutes its [B][L][3D] projection to this shape itself before
+ * the convolution (engine.py:189-190), so the values and their order along L are the same.  Channel maps: plain split
+ * rows i*D + d (ch_inner = ch_outer = D), head-blocked split (ch_inner = head_dim, ch_outer = 3*head_dim), interleaved
+ * rows 3*d + i (ch_inner = 1, ch_outer = 3, ptr advanced by i rows).  feat_taps: [3][D][feat_len] float32, the
+ * featurizer weight rows of the x1, x2 and v row of every operator channel, oldest sample first (F.conv1d's weight
+ * order); feat_len must be 3; no featurizer bias.  Gates are bit-identical to hyena_featurizer_fwd /
+ * hyena_featurizer_gates_fwd, outputs and state to hyena_li_fwd on those gates in the same work decomposition.
+ * The featurizer cache of a following decode is the last feat_len-1 samples of the projection itself. */
+int hyena_li_layer_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v,
+                       const float* feat_taps, int feat_len, const void* workspace, const float* Dcoef,
+                       int d_is_bf16, void* out, float* state_out,
+                       int64_t B, int64_t D, int64_t L, int64_t G, int64_t S, void* stream);
+
 /* hyena_li_plan + hyena_li_fwd in a form that allocates nothing and takes no workspace.  No counterpart in the
  * reference: it is for callers that cannot allocate device memory or keep a workspace alive -- code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  The coefficient tables go into a static device

@@ -748,3 +748,48 @@ def test_engine_short_fir_gated_bias_in_bf16():
                                                groups=G, gated_bias=True, dim_last=False, fir_length=K, gate=True)
     assert rel_err(z, ref) <= 2e-2
     assert (z.cpu() == ref).float().mean() > 0.97
+
+
+@pytest.mark.parametrize("flip", [False, True])
+@pytest.mark.parametrize("kind,cs,il", [("li_cplx", False, True), ("li_real", True, False), ("li_real", False, False)])
+def test_operator_module_sequence_major_projection(kind, cs, il, flip):
+    """A Hyena-LI layer handed its projection as the [B, L, 3D] view of a [B, 3D, L] tensor (what the projection GEMM
+    writes when asked for the transposed product) runs featurizer, gates and scan in one launch
+    (hyena_li_layer_fwd).  Against the oracle's call sequence (vortex/model/model.py:214-375): prefill outputs, the
+    modal state and the featurizer cache it leaves, and the decode steps that follow from them."""
+    B, L, D, H, G, n_dec = 2, 512, 64, 4, 4, 4
+    p = make_params(kind, D, G, seed=23)
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=cs, interleave=il, short_filter_length=3,
+               short_filter_bias=False, state_size=16, hyena_flip_x1x2=flip)
+    mod = HyenaCascade(cfg, 0, hyena_filter_groups=G, complex_modal=(kind == "li_cplx"))
+    with torch.no_grad():
+        mod.short_filter_weight.copy_(p["short_filter_weight"])
+        mod.log_poles.copy_(p["log_poles"])
+        mod.residues.copy_(p["residues"])
+        mod.D.data = p["D"].clone()
+    mod = mod.to(DEV)
+    pr = dict(p, log_poles=p["log_poles"].repeat_interleave(D // G, 0), residues=p["residues"].repeat_interleave(D // G, 0))
+    ref = O.OracleCascade(O.OracleEngine(hyena_flip_x1x2=flip), pr, D, H, D, column_split_hyena=cs, interleave=il)
+    u_all = torch.randn(B, L + n_dec, 3 * D, generator=torch.Generator().manual_seed(5)).bfloat16()
+    ip_ref, ip_hip = O.OracleCache(), HyenaCascadeIIRInferenceParams()
+    y_ref, _ = ref.forward(u_all[:, :L], ip_ref)
+    u_seq = u_all[:, :L].to(DEV).transpose(1, 2).contiguous().transpose(1, 2)       # same values, samples contiguous
+    assert u_seq.stride(1) == 1 and mod._can_scan_projection_rows(u_seq)
+    y_hip, _ = mod(u_seq, ip_hip)
+    assert "wf_rows" in mod._f32_cache                       # the one-launch path ran
+    assert y_hip.shape == (B, L, D) and rel_err(y_hip, y_ref) <= 2e-2
+    s_ref = ip_ref.state_dict[0]
+    s_hip = ip_hip.state_dict[0].cpu()
+    if not s_hip.is_complex() and s_ref.is_complex():
+        s_ref = s_ref.real
+    assert rel_err(torch.view_as_real(s_hip) if s_hip.is_complex() else s_hip,
+                   torch.view_as_real(s_ref) if s_ref.is_complex() else s_ref) <= 1e-4
+    assert torch.equal(ip_hip.fir_state_dict[0].reference_order().cpu().float(), ip_ref.fir_state_dict[0].float())
+    # the same module on the same values stored channel-last (two launches): one bf16 digit at most
+    y_cl, _ = mod(u_all[:, :L].to(DEV), HyenaCascadeIIRInferenceParams())
+    assert rel_err(y_hip, y_cl) <= 2.0 ** -7
+    for i in range(n_dec):
+        tok = u_all[:, L + i: L + i + 1]
+        y_ref, _ = ref.forward(tok, ip_ref)
+        y_hip, _ = mod(tok.to(DEV), ip_hip)
+        assert rel_err(y_hip, y_ref) <= 2e-2, i

@@ -222,6 +222,8 @@ class HyenaCascade(nn.Module):
         caching = inference_params is not None
         if not masked and self.fuse_prefill and self._can_fuse_prefill(u, L, caching):
             return self._fused_prefill(u, inference_params), inference_params
+        if not masked and self.fuse_prefill and self._can_scan_projection_rows(u):
+            return self._modal_prefill_from_rows(u, inference_params), inference_params
         if not masked and self.fuse_prefill and self._can_fuse_gates(u):
             return self._modal_prefill_from_projection(u, inference_params), inference_params
         w = self._f32_param("short_filter_weight", (C, Ks))
@@ -307,6 +309,52 @@ class HyenaCascade(nn.Module):
         if D % 8 or (self.column_split_hyena and hd % 8):
             return False
         return u.stride(2) == 1 and u.stride(1) % 8 == 0 and u.stride(0) % 8 == 0 and u.data_ptr() % 16 == 0
+
+    def _can_scan_projection_rows(self, u):
+        """Whether hyena_li_layer_fwd covers this call: a Hyena-LI layer with a three-tap featurizer without bias and a
+        closed channel map, whose projection u [B, L, 3D] is stored sequence-major (the [B, 3D, L] product the
+        projection GEMM writes when asked for it transposed, handed over as `p.transpose(1, 2)`), a whole number of
+        8-sample pieces long."""
+        if not self._can_fuse_gates_layer() or self.short_filter_length != 3 or self.short_filter_bias is not None:
+            return False
+        B, L, C = u.shape
+        return (L % 8 == 0 and L > 1 and C > 1 and u.stride(1) == 1 and u.stride(2) % 8 == 0 and u.stride(0) % 8 == 0
+                and u.data_ptr() % 16 == 0)
+
+    def _can_fuse_gates_layer(self):
+        if self.fir_inner_filter_length or self.long_fir_threshold is not None:
+            return False
+        return self._channel_map() is not None
+
+    def _modal_prefill_from_rows(self, u, inference_params):
+        """Hyena-LI prefill in one launch from a sequence-major projection: featurizer, split, gates and the modal
+        scan (vortex/model/model.py:233-252, :295-312), 6 bytes read and 2 written per (batch, channel, sample)."""
+        B, L, C = u.shape
+        D, Ks = self.hidden_size, self.short_filter_length
+        caching = inference_params is not None
+        p = u.transpose(1, 2)                                                       # [B, 3D, L], samples contiguous
+        (q2, q1, qv), chan = ops.projection_rows(
+            p, D, interleave=self.interleave,
+            head_dim=self.hidden_size_per_attention_head if self.column_split_hyena else None)
+        key = ("feat_rows", id(self.short_filter_weight), self.short_filter_weight.data_ptr(),
+               self.short_filter_weight._version, self.hyena_flip_x1x2)
+        hit = self._f32_cache.get("wf_rows")
+        if hit is None or hit[0] != key:
+            w = self._f32_param("short_filter_weight", (C, Ks))
+            t2, t1, tv = w[chan[0]], w[chan[1]], w[chan[2]]
+            if self.hyena_flip_x1x2:
+                t1, t2 = t2, t1
+            hit = (key, torch.stack([t1, t2, tv]).contiguous())
+            self._f32_cache["wf_rows"] = hit
+        if self.hyena_flip_x1x2:
+            q1, q2 = q2, q1
+        y, state = ops.li_layer_fwd_rows(q1, q2, qv, hit[1], self.modal_plan(), self.D, B, D, L, device=u.device,
+                                         want_state=caching)
+        if caching:
+            inference_params.state_dict[self.layer_idx] = state
+            inference_params.fir_state_dict[self.layer_idx] = _ring(u[:, max(L - (Ks - 1), 0):], Ks - 1)
+            self._drop_decode()
+        return y.permute(0, 2, 1)
 
     def _featurizer_taps_t(self, C, Ks):
         key = ("short_filter_weight_t", id(self.short_filter_weight), self.short_filter_weight.data_ptr(),

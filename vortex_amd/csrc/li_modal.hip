@@ -167,6 +167,7 @@ struct LiArgs {
     int d_is_bf16;
     int64_t nquads;           // B * D / 4 wavefront-sized work items
     uint32_t xchunk;          // blocks an XCD takes in one run (0: plain block order)
+    const float* ftaps;       // FEAT: featurizer taps [3: x1, x2, v][D][FEAT], oldest sample first
 };
 
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0)
@@ -175,10 +176,19 @@ struct LiArgs {
 // four times as long, so that a block reads 4 KiB (CPW = 4) or 16 KiB (CPW = 1) of each row in one go and a quarter
 // as many rows are in flight on the chip: long rows stream faster that way.  The modal state crosses the
 // wavefronts through LDS once per step (one block barrier); everything else stays private to a wavefront.
-template <bool PRE, bool POST, bool NT, int PF, int DMODE, bool Y32, int CPW, bool COOP>
+//
+// FEAT = 3: the rows are the raw projection of the layer, sequence-major, and the three-tap featurizer FIR of
+// vortex/model/model.py:233-246 (engine.py:188-223 with gate = False) runs on every 16-byte piece at the moment the
+// step consumes it: a lane needs the two samples ahead of its eight, which are the last dword of the lane to its
+// left (a wavefront shift) or, for lane 0, of lane 63 of the piece before it in time, carried in a scalar register.
+// The products and their order are those of the other featurizer kernels (fp32 FMAs, oldest sample first, one
+// rounding to bf16), so the gates are bit-identical to theirs.  Lone wavefronts only: a cooperating wavefront's
+// predecessor piece belongs to another wavefront.
+template <bool PRE, bool POST, bool NT, int PF, int DMODE, bool Y32, int CPW, bool COOP, int FEAT = 0>
 __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     static_assert(CPW == 4 || CPW == 1, "4 channels x 512 samples or 1 channel x 2048 samples per step");
     static_assert(!COOP || CPW == 4, "the cooperative form is built for four channels per work item");
+    static_assert(FEAT == 0 || (FEAT == 3 && PRE && POST && !COOP && !Y32), "featurizer: three taps, all three gates, lone wavefronts");
     constexpr int TLW = TL * (4 / CPW);                        // samples of one channel per step and wavefront
     constexpr int STEP = COOP ? 4 * TLW : TLW;                 // distance between two steps of one wavefront
     __shared__ __attribute__((aligned(16))) unsigned char lds_all[4 * WAVE_LDS_BYTES];
@@ -401,6 +411,65 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
         for (int k = 1; k < 16 / CPW; ++k) { const float t = ppr * pcr - ppi * pci; ppi = ppr * pci + ppi * pcr; ppr = t; }
     }
 
+    // ---- FEAT: taps of this wavefront's channels (wave-uniform, kept in scalar registers) and the carried dwords
+    constexpr int NCH = CPW == 4 ? 4 : 1;                      // distinct channels, and carry chains, per stream
+    float fw[FEAT ? 3 : 1][NCH][3];
+    uint32_t car1[NCH], carv[NCH], car2[NCH];                  // last two raw samples of the piece consumed before
+#pragma unroll
+    for (int r = 0; r < NCH; ++r) {
+        car1[r] = carv[r] = car2[r] = 0u;                      // the row starts behind zeros
+        if constexpr (FEAT != 0) {
+#pragma unroll
+            for (int i = 0; i < 3; ++i)
+#pragma unroll
+                for (int k = 0; k < 3; ++k)
+                    fw[i][r][k] = __uint_as_float((uint32_t)__builtin_amdgcn_readfirstlane(
+                        (int)__float_as_uint(a.ftaps[((int64_t)i * a.D + d0 + r) * 3 + k])));
+        }
+    }
+    auto feat = [&](const u32x4 cc, uint32_t& carry, const float (&wt)[3]) __attribute__((always_inline)) -> u32x4 {
+        // samples -2, -1: lane l takes the last dword of lane l-1, lane 0 keeps `carry`
+        const uint32_t hw = (uint32_t)__builtin_amdgcn_update_dpp((int)carry, (int)cc[3], 0x138 /* wave_shr:1 */, 0xf, 0xf, false);
+        carry = (uint32_t)__builtin_amdgcn_readlane((int)cc[3], 63);
+        float rr[10];
+        rr[0] = bf_lo(hw);
+        rr[1] = bf_hi(hw);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { rr[2 + 2 * j] = bf_lo(cc[j]); rr[3 + 2 * j] = bf_hi(cc[j]); }
+        u32x4 o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float f0 = fmaf(wt[2], rr[2 * j + 2], fmaf(wt[1], rr[2 * j + 1], fmaf(wt[0], rr[2 * j], 0.f)));
+            const float f1 = fmaf(wt[2], rr[2 * j + 3], fmaf(wt[1], rr[2 * j + 2], fmaf(wt[0], rr[2 * j + 1], 0.f)));
+            o[j] = pack_bf2(f0, f1);
+        }
+        return o;
+    };
+    auto chain = [](int r) { return CPW == 4 ? r : 0; };       // CPW = 1: the four pieces of a step follow each other in time
+
+    // FEAT with four channels per wavefront: u = bf16(f(x1) * f(v)) of the step held by register stage p (row time
+    // ts) is formed one step ahead, behind the Toeplitz MFMAs of the step before, so that the featurizer's vector
+    // instructions run in their shadow; it waits in registers until its step writes it to LDS, and the stage is
+    // refilled with step ts + PF*STEP at once (1.87 -> 1.80 ms at B = 1, L = 262144, D = 4096 with 256 filters).  With
+    // one channel per wavefront the same order needs a register stage less and measured 11 % slower (2.04 against
+    // 1.83 ms): that form runs its featurizer at the top of the step.
+    constexpr bool EARLY = FEAT != 0 && CPW == 4;
+    u32x4 un[EARLY ? 4 : 1];
+    auto prepare_u = [&](const int p, const int64_t ts) __attribute__((always_inline)) {
+        if constexpr (EARLY) {
+            const int64_t tn = ts + (int64_t)PF * STEP;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const u32x4 f1 = feat(c1[p][r], car1[chain(r)], fw[0][chain(r)]);
+                const u32x4 fv = feat(cv[p][r], carv[chain(r)], fw[2][chain(r)]);
+                un[r] = gate_mul<true>(f1, fv);
+                const bool okn = tn + roff(r) + lane * 8 < Lw;
+                c1[p][r] = okn ? ld16<NT>(lane_at(p1[r] + tn)) : zero4;
+                cv[p][r] = okn ? ld16<NT>(lane_at(pv[r] + tn)) : zero4;
+            }
+        }
+    };
+
     // One step.  GUARD = true tests every access against the row's bounds (a wave-uniform test for whole pieces, per-lane
     // predicates otherwise); GUARD = false is for steps whose loads, stores and refills are all whole pieces inside the
     // row: no branch surrounds a memory instruction there, which is what lets the compiler count exactly how many
@@ -412,28 +481,39 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
         const int64_t tn = ts + (int64_t)PF * STEP;            // step that reuses this register stage
 
         // u = bf16(x1*v) of this step -> LDS; refill the stage with step ts + PF*TLW
+        if constexpr (EARLY) {
+            // formed one step ahead (prepare_u, in the shadow of the step before): only the LDS write is left here
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            if constexpr (PRE) *(u32x4*)(u_w + r * URS + lofs) = gate_mul<true>(c1[p][r], cv[p][r]);
-            else *(u32x4*)(u_w + r * URS + lofs) = c1[p][r];
-        }
-        // whole pieces inside the row (a wave-uniform test) are requested without per-lane predicates
-        if (!GUARD || tn + TLW <= Lw) {
-            // (without branches around them the scheduler would move these requests, and what waits on the registers
-            // they overwrite, far from here and run out of registers: pin the group where the branches used to hold it)
-            if (!GUARD) __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                c1[p][r] = ld16<NT>(lane_at(p1[r] + tn));
-                if constexpr (PRE) cv[p][r] = ld16<NT>(lane_at(pv[r] + tn));
-            }
-            if (!GUARD) __builtin_amdgcn_sched_barrier(0);
+            for (int r = 0; r < 4; ++r) *(u32x4*)(u_w + r * URS + lofs) = un[r];
         } else {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const bool okn = tn + roff(r) + lane * 8 < Lw;
-                c1[p][r] = okn ? ld16<NT>(lane_at(p1[r] + tn)) : zero4;
-                if constexpr (PRE) cv[p][r] = okn ? ld16<NT>(lane_at(pv[r] + tn)) : zero4;
+                if constexpr (FEAT != 0) {
+                    const u32x4 f1 = feat(c1[p][r], car1[chain(r)], fw[0][chain(r)]);
+                    const u32x4 fv = feat(cv[p][r], carv[chain(r)], fw[2][chain(r)]);
+                    *(u32x4*)(u_w + r * URS + lofs) = gate_mul<true>(f1, fv);
+                    __builtin_amdgcn_sched_barrier(0);         // one row at a time: its temporaries are dead before the next starts
+                } else if constexpr (PRE) *(u32x4*)(u_w + r * URS + lofs) = gate_mul<true>(c1[p][r], cv[p][r]);
+                else *(u32x4*)(u_w + r * URS + lofs) = c1[p][r];
+            }
+            // whole pieces inside the row (a wave-uniform test) are requested without per-lane predicates
+            if (!GUARD || tn + TLW <= Lw) {
+                // (without branches around them the scheduler would move these requests, and what waits on the registers
+                // they overwrite, far from here and run out of registers: pin the group where the branches used to hold it)
+                if (!GUARD) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    c1[p][r] = ld16<NT>(lane_at(p1[r] + tn));
+                    if constexpr (PRE) cv[p][r] = ld16<NT>(lane_at(pv[r] + tn));
+                }
+                if (!GUARD) __builtin_amdgcn_sched_barrier(0);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const bool okn = tn + roff(r) + lane * 8 < Lw;
+                    c1[p][r] = okn ? ld16<NT>(lane_at(p1[r] + tn)) : zero4;
+                    if constexpr (PRE) cv[p][r] = okn ? ld16<NT>(lane_at(pv[r] + tn)) : zero4;
+                }
             }
         }
         wave_sync();
@@ -477,6 +557,8 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                 acc[Sg][ib] = t;
             }
 
+        if constexpr (EARLY) prepare_u((p + 1) % PF, ts + STEP);
+
         // ---- deferred output of the previous step: gate with x2, store, refill its x2 stage
         {
             const int64_t ts_out = ts - STEP, t_refill = ts - STEP + (int64_t)PF * STEP;
@@ -485,9 +567,16 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
             for (int r = 0; r < 4; ++r) {
                 o[r] = zz[r];
                 if constexpr (POST) {
+                    u32x4 g2 = c2[pp][r];
+                    if constexpr (FEAT != 0) {
+                        // the first step has no output behind it: its stage holds a later piece, which is consumed,
+                        // and carried on, when its own turn comes
+                        if (!GUARD || ts_out >= 0) g2 = feat(c2[pp][r], car2[chain(r)], fw[1][chain(r)]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        o[r][j] = pack_bf2(bf_lo(zz[r][j]) * bf_lo(c2[pp][r][j]), bf_hi(zz[r][j]) * bf_hi(c2[pp][r][j]));
+                        o[r][j] = pack_bf2(bf_lo(zz[r][j]) * bf_lo(g2[j]), bf_hi(zz[r][j]) * bf_hi(g2[j]));
                 }
             }
             if (!GUARD || (ts_out >= 0 && (ts_out > 0 || lo <= 0) && t_refill + TLW <= Lw)) {   // wave-uniform: store and refill whole pieces
@@ -634,10 +723,11 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     // The one-channel form with all three gate streams keeps guarded steps throughout: it runs at the ceiling of its
     // access order either way, and three register stages under guarded steps measured 2 % faster there (1.628 against
     // 1.659 ms at L = 262144) than the two stages that fit whole-piece steps.
-    constexpr bool WHOLE_ROTATIONS = !(CPW == 1 && PRE && POST);
+    constexpr bool WHOLE_ROTATIONS = !(CPW == 1 && PRE && POST) && FEAT == 0;
     constexpr int VMCNT0 = 0x0F70;                             // s_waitcnt vmcnt(0), other counters unconstrained
     const int64_t whole_until = Lv - (COOP ? 3 * TLW : 0) - TLW - (int64_t)(2 * PF - 1) * STEP;
     if (WHOLE_ROTATIONS) __builtin_amdgcn_s_waitcnt(VMCNT0);
+    if constexpr (EARLY) prepare_u(0, 0);
     for (int64_t ts = 0; ts < Lv; ts += (int64_t)PF * STEP) {
         if (WHOLE_ROTATIONS && ts > 0 && ts <= whole_until) {
             if constexpr (WHOLE_ROTATIONS) {
@@ -666,6 +756,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
 #pragma unroll
                 for (int p = 1; p < PF; ++p)
                     if (p == pl) x2v = c2[p][r];
+                if constexpr (FEAT != 0) x2v = feat(x2v, car2[chain(r)], fw[1][chain(r)]);
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                     o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(x2v[j]), bf_hi(zz[j]) * bf_hi(x2v[j]));
@@ -705,7 +796,8 @@ extern "C" int hyena_li_plan(const float* log_poles, const float* residues, int6
 namespace {
 int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const void* workspace,
                 const float* Dcoef, int d_is_bf16, void* out, float* y_conv_fp32, float* state_out,
-                int64_t B, int64_t D, int64_t L, int64_t G, int64_t S_, void* stream, bool check_only);
+                int64_t B, int64_t D, int64_t L, int64_t G, int64_t S_, void* stream, bool check_only,
+                const float* ftaps = nullptr);
 }
 
 extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const void* workspace,
@@ -713,6 +805,18 @@ extern "C" int hyena_li_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
                             int64_t B, int64_t D, int64_t L, int64_t G, int64_t S_, void* stream) {
     return li_fwd_impl("hyena_li_fwd", x1, x2, v, workspace, Dcoef, d_is_bf16, out, y_conv_fp32, state_out, B, D, L, G,
                        S_, stream, false);
+}
+
+extern "C" int hyena_li_layer_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const float* feat_taps,
+                                  int feat_len, const void* workspace, const float* Dcoef, int d_is_bf16, void* out,
+                                  float* state_out, int64_t B, int64_t D, int64_t L, int64_t G, int64_t S_, void* stream) {
+    const char* who = "hyena_li_layer_fwd";
+    if (!feat_taps) return hyena_fail(HYENA_EINVAL, "%s: feat_taps is required", who);
+    if (feat_len != 3) return hyena_fail(HYENA_ENOSUP, "%s: featurizer of %d taps (3)", who, feat_len);
+    if (!x1 || !x1->ptr || !x2 || !x2->ptr || !v || !v->ptr)
+        return hyena_fail(HYENA_EINVAL, "%s: the three row sets of the projection are required", who);
+    return li_fwd_impl(who, x1, x2, v, workspace, Dcoef, d_is_bf16, out, nullptr, state_out, B, D, L, G, S_, stream,
+                       false, feat_taps);
 }
 
 // ------------------------------------------------------------------ the form that allocates nothing
@@ -778,7 +882,8 @@ extern "C" int hyena_li_fwd_static(const hyena_rows* x1, const hyena_rows* x2, c
 namespace {
 int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const void* workspace,
                 const float* Dcoef, int d_is_bf16, void* out, float* y_conv_fp32, float* state_out,
-                int64_t B, int64_t D, int64_t L, int64_t G, int64_t S_, void* stream, bool check_only) {
+                int64_t B, int64_t D, int64_t L, int64_t G, int64_t S_, void* stream, bool check_only,
+                const float* ftaps) {
     if (!x1 || !x1->ptr || !workspace || !out)
         return hyena_fail(HYENA_EINVAL, "%s: x1, workspace and out are required", who);
     if (B < 0 || D <= 0 || L < 0 || G <= 0 || D % G != 0)
@@ -794,6 +899,8 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
         return hyena_fail(HYENA_EINVAL, "%s: B*D and the channel map must fit 31 bits", who);
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
     if (pre && !post) return hyena_fail(HYENA_ENOSUP, "%s: v without x2 (pass both, x2 alone with x1 holding x1*v, or neither)", who);
+    if (ftaps && (!pre || !post || y_conv_fp32))
+        return hyena_fail(HYENA_EINVAL, "%s: the featurizer form takes all three projection row sets and no float32 output", who);
     if (B == 0 || L == 0) return 0;
     // Work decomposition (measured on B*D = 1024 .. 8192 rows, L = 8192 .. 524288):
     //  * rows of 65536 samples or more: one channel per wavefront, 2048 samples per step.  A wavefront then reads
@@ -805,12 +912,14 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
     //    consecutive pieces of the same four rows; 1-4 % faster than one channel per wavefront from 65536 samples
     //    on, e.g. 1.61 against 1.64-1.65 ms with three gate streams and 1.25 against 1.29 ms on x1*v rows at L = 262144).
     const bool can4 = (D / G) % 4 == 0;
-    const bool long_coop = can4 && L >= 65536 && post;
+    const bool long_coop = can4 && L >= 65536 && post && !ftaps;      // the featurizer form runs lone wavefronts only
     int cpw = (can4 && (L < 65536 || long_coop)) ? 4 : 1;    // channels per wavefront (they share one filter)
+    if (ftaps && can4) cpw = 4;     // featurizer form: 1.80 against 1.83 ms at L = 262144, and faster below
     { const int64_t x = hyena_override(HYENA_OV_LI_CPW); if (x == 1) cpw = 1; else if (x == 4 && can4) cpw = 4; }
     const int64_t nquads = B * (D / cpw);
     bool coop = cpw == 4 && (nquads <= 512 || long_coop);
     { const int64_t x = hyena_override(HYENA_OV_LI_COOP); if (x >= 0) coop = cpw == 4 && x != 0; }
+    if (ftaps) coop = false;
     const int64_t nblk = coop ? nquads : (nquads + 3) / 4;
     if (nquads > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: problem too large for one launch", who);
     if (check_only) return 0;
@@ -829,6 +938,7 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
     a.dg = (int)(D / G);
     a.d_is_bf16 = d_is_bf16;
     a.nquads = nquads;
+    a.ftaps = ftaps;
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)nblk);
     bool nt = 8.0 * (double)B * (double)D * (double)L > 384e6;
@@ -859,9 +969,18 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
     } while (0)
 #define LI_M(P, Q, N, Y) do { if (dmode == 1) LI_LAUNCH(P, Q, N, 1, Y); else if (dmode == 2) LI_LAUNCH(P, Q, N, 2, Y); else LI_LAUNCH(P, Q, N, 0, Y); } while (0)
 #define LI_N(P, Q) do { if (y32) LI_M(P, Q, false, true); else if (nt) LI_M(P, Q, true, false); else LI_M(P, Q, false, false); } while (0)
-    if (pre && post) LI_N(true, true);
+#define LI_F(N, M)                                                                                          \
+    do {                                                                                                   \
+        if (cpw == 4) hipLaunchKernelGGL((li_kernel<true, true, N, 2, M, false, 4, false, 3>), grid, dim3(256), 0, s, a);   \
+        else hipLaunchKernelGGL((li_kernel<true, true, N, 3, M, false, 1, false, 3>), grid, dim3(256), 0, s, a);             \
+    } while (0)
+#define LI_FM(N) do { if (dmode == 1) LI_F(N, 1); else if (dmode == 2) LI_F(N, 2); else LI_F(N, 0); } while (0)
+    if (ftaps) { if (nt) LI_FM(true); else LI_FM(false); }
+    else if (pre && post) LI_N(true, true);
     else if (post) LI_N(false, true);          // x1 already holds bf16(x1*v) (hyena_featurizer_gates_fwd)
     else LI_N(false, false);
+#undef LI_FM
+#undef LI_F
 #undef LI_N
 #undef LI_M
 #undef LI_LAUNCH

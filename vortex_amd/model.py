@@ -142,11 +142,19 @@ class HyenaBlock(nn.Module):
         groups = cfg[f"{kind}_filter_groups"]
         K = {"hcs": cfg["hcs_filter_length"], "hcm": cfg["hcm_filter_length"], "hcl": None}[kind]
         self.filter = HyenaCascade(cfg, layer_idx, hyena_filter_groups=groups, fir_inner_filter_length=K)
+        self.kind = kind
         self.out_filter_dense = nn.Linear(D, D, bias=True)
         self.mlp = GatedMLP(D, cfg["inner_mlp_size"], cfg["evo2_style_activations"] and layer_idx > 0)
 
     def forward(self, u, inference_params=None):
-        z = self.projections(self.pre_norm(u))
+        xn = self.pre_norm(u)
+        if self.kind == "hcl" and xn.shape[1] > 1 and xn.shape[1] % 8 == 0:
+            # a prefill of a Hyena-LI layer: the projection GEMM writes its product transposed, [B, 3D, L] with the
+            # samples contiguous, which the layer then reads once (featurizer, gates and scan in one launch); the
+            # values are those of self.projections(xn), handed over as the [B, L, 3D] view of that memory
+            z = torch.matmul(self.projections.weight, xn.transpose(1, 2)).transpose(1, 2)
+        else:
+            z = self.projections(xn)
         z, _ = self.filter(z, inference_params=inference_params)
         z_in = self.out_filter_dense(z) + u
         return self.mlp(self.post_norm(z_in)) + z_in, None

@@ -355,6 +355,51 @@ def li_fwd_rows(x1r, x2r, vr, plan, Dcoef, B, D, L, *, device, want_state=False,
     return out, y32, state
 
 
+def projection_rows(p, hidden, *, interleave=False, head_dim=None):
+    """Row descriptors (x2, x1, v) of a raw sequence-major projection p [B, 3*hidden, L] under the channel maps of
+    vortex/model/utils.py:26-85, and the projection channel of every (gate, operator channel) as an int64 tensor
+    [3, hidden] in the same (x2, x1, v) order.  interleave: projection channel 3*d + i; head_dim: the head-blocked
+    column split; neither: the plain split i*hidden + d.  interleave with head_dim has no closed map (ValueError)."""
+    if interleave and head_dim is not None:
+        raise ValueError("interleave combined with column_split has no closed channel map")
+    if p.dtype != torch.bfloat16 or p.dim() != 3 or p.stride(2) != 1:
+        raise ValueError("expected a [B, 3D, L] bfloat16 tensor with contiguous samples")
+    d = torch.arange(hidden, device=p.device)
+    if interleave:
+        es = p.element_size()
+        rows = tuple(Rows(p.data_ptr() + i * p.stride(1) * es, p.stride(0), p.stride(1), 1, 3) for i in range(3))
+        chan = torch.stack([3 * d + i for i in range(3)])
+    elif head_dim is not None:
+        rows = tuple(rows_of_projection(p, hidden, i, head_dim) for i in range(3))
+        chan = torch.stack([(d // head_dim) * 3 * head_dim + d % head_dim + i * head_dim for i in range(3)])
+    else:
+        rows = tuple(rows_of_projection(p, hidden, i) for i in range(3))
+        chan = torch.stack([d + i * hidden for i in range(3)])
+    return rows, chan
+
+
+def li_layer_fwd_rows(x1r, x2r, vr, feat_taps, plan, Dcoef, B, D, L, *, device, want_state=False, out=None,
+                      single_rounding=False):
+    """hyena_li_layer_fwd: featurizer FIR, gates and the modal scan in one pass over the rows of a raw sequence-major
+    projection.  feat_taps [3, D, 3] float32: the featurizer weight rows of the x1, x2 and v row of every operator
+    channel.  Returns (out [B, D, L] bf16, state or None) as li_fwd_rows does."""
+    if out is None:
+        out = torch.empty((B, D, L), dtype=torch.bfloat16, device=device)
+    state = torch.zeros((B, D, plan.S, 2), dtype=torch.float32, device=device) if want_state else None
+    if out.numel():
+        if feat_taps.dtype != torch.float32 or not feat_taps.is_contiguous() or tuple(feat_taps.shape) != (3, D, 3):
+            raise ValueError("feat_taps must be a contiguous float32 [3, D, 3] tensor")
+        dco = _f32(Dcoef)
+        d_is_bf16 = 2 if single_rounding else int(Dcoef is None or Dcoef.dtype == torch.bfloat16)
+        rc = _lib.lib().hyena_li_layer_fwd(_ref(x1r), _ref(x2r), _ref(vr), _ptr(feat_taps), 3, _ptr(plan.workspace),
+                                           _ptr(dco), d_is_bf16, _ptr(out), _ptr(state), B, D, L, plan.G, plan.S,
+                                           _stream())
+        _lib.check(rc, "hyena_li_layer_fwd")
+    if state is not None:
+        state = torch.view_as_complex(state) if plan.is_complex else state[..., 0].contiguous()
+    return out, state
+
+
 def hyena_li_fwd(x1, x2, v, log_poles, residues, D_bias=None, *, plan=None, want_state=False, want_fp32=False,
                  single_rounding=False):
     """Hyena-LI prefill on [B, D, L] bf16 gates with grouped modal parameters.
