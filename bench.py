@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="mr", choices=["mr", "se", "se_b8", "li", "li_g4096", "decode", "mr_cl", "mr_layer", "li_layer",
-                                                         "se_layer", "mr_cl_f16", "cl_f32", "li_layer_seq", "li_layer_seq_g4096"])
+                                                         "se_layer", "mr_cl_f16", "cl_f32", "li_layer_seq", "li_layer_seq_g4096", "mr_layer_seq"])
     ap.add_argument("--settle-ms", type=float, default=150.0,
                     help="untimed run of each workload before its warm-up steps, until clocks have settled")
     ap.add_argument("--no-extras", action="store_true")
@@ -213,6 +213,23 @@ def build_workload(name, device):
         return fn, dict(workload=f"hyena_li_layer featurizer+gates then modal scan, from the projection B={B} L={L} D={D} "
                                  f"groups={G} poles={S} complex", tokens=B * L, bytes=8 * B * D * L,
                         kernel="proj_gates_kernel + li_kernel", keep=(u, wf, plan, Db, out))
+    if name == "mr_layer_seq":
+        # the Hyena-MR layer of config 2 from a projection stored sequence-major: featurizer, split, gates and the
+        # inner FIR in one launch of the sequence-major MFMA kernel; 6 bytes read + 2 written per (channel, sample)
+        B, D, L, G, K = 2, 4096, 32768, 256, 128
+        g = torch.Generator(device=device).manual_seed(9)
+        p = torch.randn(B, 3 * D, L, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+        w = torch.randn(3 * D, 3, generator=g, device=device, dtype=torch.float32) * 3 ** -0.5
+        (q2, q1, qv), chan = ops.projection_rows(p, D, interleave=True)
+        taps = torch.stack([w[chan[1]], w[chan[0]], w[chan[2]]]).contiguous()
+        h = O.make_mr_filter(G, K).reshape(G, K).to(device)
+        Db = torch.randn(D, generator=g, device=device, dtype=torch.float32)
+        out = torch.empty(B, D, L, dtype=torch.bfloat16, device=device)
+        fn = lambda: ops.fir_layer_fwd_rows(q1, q2, qv, taps, h, B, D, L, K, device=device, bias=Db,
+                                            bias_mode=ops.HYENA_BIAS_GATED_FP32, out=out)
+        return fn, dict(workload=f"hyena_mr_layer in one launch from a sequence-major projection B={B} L={L} D={D} "
+                                 f"groups={G} K={K}", tokens=B * L, bytes=8 * B * D * L, kernel="mr_fir_kernel",
+                        keep=(p, taps, h, Db, out))
     if name in ("li_layer_seq", "li_layer_seq_g4096"):
         # the same layer from the same projection values stored sequence-major ([B, 3D, L], what the projection GEMM
         # writes when asked for the transposed product): featurizer, split, gates and the modal scan in ONE launch,
@@ -600,7 +617,8 @@ def main():
                 continue
             steps = max(3, min(args.steps, 20 if name.startswith("li") else args.steps))
             extra[name] = entry(run(name, steps, extra_warmup))
-        for name in ("mr_cl", "mr_layer", "se_layer", "li_layer", "li_layer_seq", "li_layer_seq_g4096", "mr_cl_f16", "cl_f32"):
+        for name in ("mr_cl", "mr_layer", "mr_layer_seq", "se_layer", "li_layer", "li_layer_seq", "li_layer_seq_g4096", "mr_cl_f16",
+                     "cl_f32"):
             e = run(name, max(3, min(args.steps, 10 if name.startswith("li_layer") else 20)), extra_warmup)
             extra[name] = entry(e)
             if "flops" in e:    # the float32 direct form is arithmetic-bound on the vector ALUs (the float16 form,

@@ -170,6 +170,21 @@ int hyena_li_layer_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_r
                        int d_is_bf16, void* out, float* state_out,
                        int64_t B, int64_t D, int64_t L, int64_t G, int64_t S, void* stream);
 
+/* A whole Hyena-SE / MR layer in one pass over a projection that is stored sequence-major: the featurizer FIR
+ * (vortex/model/model.py:233-246, vortex/model/engine.py:188-223 with gate = False), the split under any channel map
+ * (vortex/model/model.py:250-252, vortex/model/utils.py:26-85) and the gated inner FIR of hyena_mr_fwd
+ * (vortex/model/model.py:268-291, vortex/model/engine.py:131-260), 6 bytes read and 2 written per sample:
+ *   f_i[t] = bf16(w_i[d][0]*p_i[t-2] + w_i[d][1]*p_i[t-1] + w_i[d][2]*p_i[t])     i = x1, x2, v; p_i = the rows given
+ *   out    = hyena_mr_fwd on (x1, x2, v) = (f_x1, f_x2, f_v)        any 1 <= K <= 128, on the matrix cores
+ * Rows, channel maps and feat_taps as in hyena_li_layer_fwd.  bias_mode: HYENA_BIAS_NONE or HYENA_BIAS_GATED_FP32.
+ * Bit-identical to hyena_featurizer_fwd followed by hyena_mr_fwd.  out: [B][D][L] bf16.  The inner FIR cache of a
+ * following decode (the last K-1 values of bf16(f_x1 * f_v)) is not written; callers form it from the tail of the
+ * projection (hyena_featurizer_fwd on the last K+1 samples). */
+int hyena_fir_layer_fwd_rows(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v,
+                             const float* feat_taps, int feat_len, const float* h, int taps_reversed,
+                             const float* bias, int bias_mode, void* out,
+                             int64_t B, int64_t D, int64_t L, int64_t G, int K, void* stream);
+
 /* hyena_li_plan + hyena_li_fwd in a form that allocates nothing and takes no workspace.  No counterpart in the
  * reference: it is for callers that cannot allocate device memory or keep a workspace alive -- code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  The coefficient tables go into a static device

@@ -793,3 +793,43 @@ def test_operator_module_sequence_major_projection(kind, cs, il, flip):
         y_ref, _ = ref.forward(tok, ip_ref)
         y_hip, _ = mod(tok.to(DEV), ip_hip)
         assert rel_err(y_hip, y_ref) <= 2e-2, i
+
+
+@pytest.mark.parametrize("flip", [False, True])
+@pytest.mark.parametrize("kind,cs,il", [("mr", False, True), ("se", False, True), ("mr", True, False), ("se", False, False)])
+def test_operator_module_sequence_major_projection_fir(kind, cs, il, flip):
+    """A Hyena-SE / MR layer handed its projection as the [B, L, 3D] view of a [B, 3D, L] tensor runs featurizer, gates
+    and the inner FIR in one launch (hyena_fir_layer_fwd_rows).  Against the oracle's call sequence
+    (vortex/model/model.py:214-375): prefill outputs, both FIR caches it leaves, and the decode steps after them."""
+    B, L, D, H, G, n_dec = 2, 512, 64, 4, 4, 4
+    K = {"se": 7, "mr": 128}[kind]
+    p = make_params(kind, D, G, seed=29)
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=cs, interleave=il, short_filter_length=3,
+               short_filter_bias=False, state_size=16, hyena_flip_x1x2=flip)
+    mod = HyenaCascade(cfg, 0, hyena_filter_groups=G, fir_inner_filter_length=K)
+    with torch.no_grad():
+        mod.short_filter_weight.copy_(p["short_filter_weight"])
+        mod.h.copy_(p["h"])
+        if mod.D is not None:
+            mod.D.data = p["D"].clone()
+    mod = mod.to(DEV)
+    ref = O.OracleCascade(O.OracleEngine(hyena_flip_x1x2=flip), p, D, H, G, fir_inner_filter_length=K,
+                          column_split_hyena=cs, interleave=il)
+    u_all = torch.randn(B, L + n_dec, 3 * D, generator=torch.Generator().manual_seed(6)).bfloat16()
+    ip_ref, ip_hip = O.OracleCache(), HyenaCascadeFIRInferenceParams()
+    y_ref, _ = ref.forward(u_all[:, :L], ip_ref)
+    u_seq = u_all[:, :L].to(DEV).transpose(1, 2).contiguous().transpose(1, 2)
+    assert mod._can_filter_projection_rows(u_seq)
+    y_hip, _ = mod(u_seq, ip_hip)
+    assert "wf_rows" in mod._f32_cache                       # the one-launch path ran
+    assert y_hip.shape == (B, L, D) and rel_err(y_hip, y_ref) <= 2e-2
+    assert torch.equal(ip_hip.fir_state_dict[0].reference_order().cpu().float(), ip_ref.fir_state_dict[0].float())
+    inner = ip_hip.fir_inner_state_dict[0].reference_order().cpu().float()
+    assert rel_err(inner, ip_ref.fir_inner_state_dict[0].float()) <= 2.0 ** -7
+    y_cl, _ = mod(u_all[:, :L].to(DEV), HyenaCascadeFIRInferenceParams())          # channel-last: the fused kernel
+    assert rel_err(y_hip, y_cl) <= 2.0 ** -7
+    for i in range(n_dec):
+        tok = u_all[:, L + i: L + i + 1]
+        y_ref, _ = ref.forward(tok, ip_ref)
+        y_hip, _ = mod(tok.to(DEV), ip_hip)
+        assert rel_err(y_hip, y_ref) <= 2e-2, i

@@ -14,7 +14,7 @@ HYENA_DTYPE_BF16, HYENA_DTYPE_F16, HYENA_DTYPE_F32 = 0, 1, 2
 
 EXPORTS = [
     "hyena_version", "hyena_last_error_string", "hyena_se_fwd", "hyena_mr_fwd",
-    "hyena_fir_step", "hyena_iir_step", "hyena_li_plan_bytes", "hyena_li_plan", "hyena_li_fwd", "hyena_li_layer_fwd", "hyena_li_fwd_static", "hyena_featurizer_fwd", "hyena_set_launch_override",
+    "hyena_fir_step", "hyena_iir_step", "hyena_li_plan_bytes", "hyena_li_plan", "hyena_li_fwd", "hyena_li_layer_fwd", "hyena_fir_layer_fwd_rows", "hyena_li_fwd_static", "hyena_featurizer_fwd", "hyena_set_launch_override",
     "hyena_fir_layer_step", "hyena_iir_layer_step", "hyena_fir_cl_fwd", "hyena_fir_cl_fwd_dtype", "hyena_fir_layer_fwd",
     "hyena_featurizer_gates_fwd",
     "hyena_fir_step_dpos", "hyena_fir_layer_step_dpos", "hyena_ring_advance",
@@ -82,6 +82,8 @@ def lib():
     L.hyena_li_plan.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]
     L.hyena_li_fwd.argtypes = [R, R, R, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
                                c_int64, c_int64, c_int64, c_void_p]
+    L.hyena_fir_layer_fwd_rows.argtypes = [R, R, R, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64,
+                                           c_int64, c_int64, c_int64, c_int, c_void_p]
     L.hyena_li_layer_fwd.argtypes = [R, R, R, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int64,
                                      c_int64, c_int64, c_int64, c_int64, c_void_p]
     L.hyena_li_fwd_static.argtypes = [R, R, R, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64,

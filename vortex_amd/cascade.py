@@ -224,6 +224,8 @@ class HyenaCascade(nn.Module):
             return self._fused_prefill(u, inference_params), inference_params
         if not masked and self.fuse_prefill and self._can_scan_projection_rows(u):
             return self._modal_prefill_from_rows(u, inference_params), inference_params
+        if not masked and self.fuse_prefill and self._can_filter_projection_rows(u):
+            return self._fir_prefill_from_rows(u, inference_params), inference_params
         if not masked and self.fuse_prefill and self._can_fuse_gates(u):
             return self._modal_prefill_from_projection(u, inference_params), inference_params
         w = self._f32_param("short_filter_weight", (C, Ks))
@@ -315,11 +317,63 @@ class HyenaCascade(nn.Module):
         closed channel map, whose projection u [B, L, 3D] is stored sequence-major (the [B, 3D, L] product the
         projection GEMM writes when asked for it transposed, handed over as `p.transpose(1, 2)`), a whole number of
         8-sample pieces long."""
-        if not self._can_fuse_gates_layer() or self.short_filter_length != 3 or self.short_filter_bias is not None:
-            return False
+        return self._can_fuse_gates_layer() and self._rows_layout_ok(u)
+
+    def _rows_layout_ok(self, u):
         B, L, C = u.shape
-        return (L % 8 == 0 and L > 1 and C > 1 and u.stride(1) == 1 and u.stride(2) % 8 == 0 and u.stride(0) % 8 == 0
-                and u.data_ptr() % 16 == 0)
+        return (self.short_filter_length == 3 and self.short_filter_bias is None and self._channel_map() is not None
+                and L % 8 == 0 and L > 1 and C > 1 and u.stride(1) == 1 and u.stride(2) % 8 == 0
+                and u.stride(0) % 8 == 0 and u.data_ptr() % 16 == 0)
+
+    def _can_filter_projection_rows(self, u):
+        """Whether hyena_fir_layer_fwd_rows covers this call: a Hyena-SE / MR layer (inner filter of at most 128 taps)
+        whose projection is stored sequence-major, under the conditions of _can_scan_projection_rows, and a prompt
+        long enough to fill the inner cache from its own tail."""
+        K = self.fir_inner_filter_length
+        return bool(K) and K <= 128 and self._rows_layout_ok(u) and u.shape[1] >= K + 1
+
+    def _feat_rows_taps(self, chan, C, Ks):
+        """Featurizer weight rows [3, D, Ks] of the (x1, x2, v) row of every operator channel (flip applied)."""
+        key = ("feat_rows", id(self.short_filter_weight), self.short_filter_weight.data_ptr(),
+               self.short_filter_weight._version, self.hyena_flip_x1x2)
+        hit = self._f32_cache.get("wf_rows")
+        if hit is None or hit[0] != key:
+            w = self._f32_param("short_filter_weight", (C, Ks))
+            t2, t1, tv = w[chan[0]], w[chan[1]], w[chan[2]]
+            if self.hyena_flip_x1x2:
+                t1, t2 = t2, t1
+            hit = (key, torch.stack([t1, t2, tv]).contiguous())
+            self._f32_cache["wf_rows"] = hit
+        return hit[1]
+
+    def _fir_prefill_from_rows(self, u, inference_params):
+        """Hyena-SE / MR prefill in one launch from a sequence-major projection: featurizer, split, gates and the
+        inner FIR on the matrix cores (vortex/model/model.py:233-291)."""
+        B, L, C = u.shape
+        D, Ks, K = self.hidden_size, self.short_filter_length, self.fir_inner_filter_length
+        caching = inference_params is not None
+        mr = K >= 128
+        p = u.transpose(1, 2)                                                       # [B, 3D, L], samples contiguous
+        (q2, q1, qv), chan = ops.projection_rows(
+            p, D, interleave=self.interleave,
+            head_dim=self.hidden_size_per_attention_head if self.column_split_hyena else None)
+        ft = self._feat_rows_taps(chan, C, Ks)
+        if self.hyena_flip_x1x2:
+            q1, q2 = q2, q1
+        y = ops.fir_layer_fwd_rows(q1, q2, qv, ft, self._f32_param("h", (self.h.shape[0], K)), B, D, L, K,
+                                   device=u.device, bias=self._f32_param("D") if mr else None,
+                                   bias_mode=HYENA_BIAS_GATED_FP32 if mr else HYENA_BIAS_NONE, taps_reversed=not mr)
+        if caching:
+            inference_params.fir_state_dict[self.layer_idx] = _ring(u[:, L - (Ks - 1):], Ks - 1)
+            # the inner cache is the last K-1 values of bf16(x1*v): the featurizer kernel on the prompt's tail (its
+            # first Ks-1 outputs lack their history and are dropped)
+            n = K - 1 + Ks - 1
+            z = ops.featurizer_fwd(u[:, L - n:].contiguous(), self._f32_param("short_filter_weight", (C, Ks)), None,
+                                   interleave=self.interleave, front_pad=(-n) % 8)
+            _, x1, v = self._split(z[..., z.shape[-1] - (K - 1):])
+            inference_params.fir_inner_state_dict[self.layer_idx] = _ring((x1 * v).permute(0, 2, 1), K - 1, flipped=mr)
+            self._drop_decode()
+        return y.permute(0, 2, 1)
 
     def _can_fuse_gates_layer(self):
         if self.fir_inner_filter_length or self.long_fir_threshold is not None:
@@ -336,19 +390,10 @@ class HyenaCascade(nn.Module):
         (q2, q1, qv), chan = ops.projection_rows(
             p, D, interleave=self.interleave,
             head_dim=self.hidden_size_per_attention_head if self.column_split_hyena else None)
-        key = ("feat_rows", id(self.short_filter_weight), self.short_filter_weight.data_ptr(),
-               self.short_filter_weight._version, self.hyena_flip_x1x2)
-        hit = self._f32_cache.get("wf_rows")
-        if hit is None or hit[0] != key:
-            w = self._f32_param("short_filter_weight", (C, Ks))
-            t2, t1, tv = w[chan[0]], w[chan[1]], w[chan[2]]
-            if self.hyena_flip_x1x2:
-                t1, t2 = t2, t1
-            hit = (key, torch.stack([t1, t2, tv]).contiguous())
-            self._f32_cache["wf_rows"] = hit
+        ft = self._feat_rows_taps(chan, C, Ks)
         if self.hyena_flip_x1x2:
             q1, q2 = q2, q1
-        y, state = ops.li_layer_fwd_rows(q1, q2, qv, hit[1], self.modal_plan(), self.D, B, D, L, device=u.device,
+        y, state = ops.li_layer_fwd_rows(q1, q2, qv, ft, self.modal_plan(), self.D, B, D, L, device=u.device,
                                          want_state=caching)
         if caching:
             inference_params.state_dict[self.layer_idx] = state

@@ -53,11 +53,35 @@ __device__ __forceinline__ u32x4 gate_mul(u32x4 a, u32x4 b) {
     return r;
 }
 
-template <bool PRE, bool POST, int BIAS, bool NT, bool FULL>
+// Three-tap featurizer FIR on one 16-byte piece (8 samples of a raw projection row): hw holds the two samples ahead
+// of it.  fp32 FMAs, oldest sample first, one rounding to bf16: the arithmetic of the other featurizer kernels.
+__device__ __forceinline__ u32x4 feat3(const u32x4 cc, const uint32_t hw, const float w0, const float w1, const float w2) {
+    float rr[10];
+    rr[0] = bf_lo(hw);
+    rr[1] = bf_hi(hw);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { rr[2 + 2 * j] = bf_lo(cc[j]); rr[3 + 2 * j] = bf_hi(cc[j]); }
+    u32x4 o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float f0 = fmaf(w2, rr[2 * j + 2], fmaf(w1, rr[2 * j + 1], fmaf(w0, rr[2 * j], 0.f)));
+        const float f1 = fmaf(w2, rr[2 * j + 3], fmaf(w1, rr[2 * j + 2], fmaf(w0, rr[2 * j + 1], 0.f)));
+        o[j] = pack_bf2(f0, f1);
+    }
+    return o;
+}
+
+// FEAT = 3: the rows are the raw projection of the layer, stored sequence-major, and the three-tap featurizer FIR of
+// vortex/model/model.py:233-246 (vortex/model/engine.py:188-223 with gate = False) runs on every 16-byte piece as the
+// step consumes it.  A wavefront instruction covers 512 consecutive samples of one row, so a lane's two samples of
+// history are the last dword of the lane to its left (a wavefront shift); lane 0 takes them from the piece the
+// wavefront consumed one step earlier, carried in a scalar register, and at the start of a segment from memory.
+template <bool PRE, bool POST, int BIAS, bool NT, bool FULL, int FEAT = 0>
 __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, RowMap v, const float* __restrict__ h,
                                                         int K, int reversed, const float* __restrict__ bias,
                                                         bf16_t* __restrict__ out, int64_t D, int64_t L, int dg,
-                                                        int64_t seg_len, int nseg) {
+                                                        int64_t seg_len, int nseg, const float* __restrict__ ftaps) {
+    static_assert(FEAT == 0 || (FEAT == 3 && PRE && POST), "featurizer: three taps, all three gates");
     __shared__ __attribute__((aligned(16))) bf16_t u_lds[16 * URS];
     __shared__ __attribute__((aligned(16))) bf16_t z_lds[16 * ZRS];
 
@@ -130,14 +154,52 @@ __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
     const int64_t t_end = (t_begin + seg_len < L) ? t_begin + seg_len : L;
     if (t_begin >= t_end) return;
 
+    // ---- FEAT: taps of this wavefront's four rows (wave-uniform) and the dwords carried from piece to piece
+    float fw[FEAT ? 3 : 1][4][3];
+    uint32_t car1[4], carv[4], car2[4];
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+        car1[r4] = carv[r4] = car2[r4] = 0u;
+        if constexpr (FEAT != 0) {
+            const int64_t d = rlive[r4] ? d0 + 4 * r4 + w : d0;
+#pragma unroll
+            for (int i = 0; i < 3; ++i)
+#pragma unroll
+                for (int k = 0; k < 3; ++k)
+                    fw[i][r4][k] = __uint_as_float((uint32_t)__builtin_amdgcn_readfirstlane(
+                        (int)__float_as_uint(ftaps[((int64_t)i * D + d) * 3 + k])));
+            if (t_begin > 0) {          // the two samples ahead of the segment (t_begin is a multiple of 8: aligned dwords)
+                car1[r4] = (uint32_t)__builtin_amdgcn_readfirstlane((int)*(const uint32_t*)(p1[r4] + t_begin - 2));
+                carv[r4] = (uint32_t)__builtin_amdgcn_readfirstlane((int)*(const uint32_t*)(pv[r4] + t_begin - 2));
+                car2[r4] = (uint32_t)__builtin_amdgcn_readfirstlane((int)*(const uint32_t*)(p2[r4] + t_begin - 2));
+            }
+        }
+    }
+    auto feat = [&](const u32x4 cc, uint32_t& carry, const float (&wt)[3]) __attribute__((always_inline)) -> u32x4 {
+        const uint32_t hw = (uint32_t)__builtin_amdgcn_update_dpp((int)carry, (int)cc[3], 0x138 /* wave_shr:1 */, 0xf, 0xf, false);
+        carry = (uint32_t)__builtin_amdgcn_readlane((int)cc[3], 63);
+        return feat3(cc, hw, wt[0], wt[1], wt[2]);
+    };
+
     // ---- halo of the segment: the 128 samples before t_begin (zeros at the sequence start)
     {
         const int ch = tid >> 4, tt = (tid & 15) * 8;
         u32x4 hu = {0, 0, 0, 0};
         if (t_begin > 0 && ch < c_live) {
-            const u32x4 a = *(const u32x4*)(x1.row(b, d0 + ch) + t_begin - HALO + tt);
+            const bf16_t* r1 = x1.row(b, d0 + ch) + t_begin - HALO + tt;
+            u32x4 a = *(const u32x4*)r1;
             u32x4 c = {0, 0, 0, 0};
             if (PRE) c = *(const u32x4*)(v.row(b, d0 + ch) + t_begin - HALO + tt);
+            if constexpr (FEAT != 0) {
+                // every thread fetches its own two samples of history here (once per segment)
+                const bf16_t* rv = v.row(b, d0 + ch) + t_begin - HALO + tt;
+                const bool hist = t_begin - HALO + tt >= 2;
+                const uint32_t h1 = hist ? *(const uint32_t*)(r1 - 2) : 0u, hv = hist ? *(const uint32_t*)(rv - 2) : 0u;
+                const float* t1 = ftaps + (d0 + ch) * 3;
+                const float* tv = ftaps + (2 * D + d0 + ch) * 3;
+                a = feat3(a, h1, t1[0], t1[1], t1[2]);
+                c = feat3(c, hv, tv[0], tv[1], tv[2]);
+            }
             hu = gate_mul<PRE>(a, c);
         }
         *(u32x4*)(u_lds + ch * URS + tt) = hu;
@@ -162,8 +224,16 @@ __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
         constexpr bool WHOLE = decltype(whole_tag)::value;
         // u of this step -> LDS
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4)
-            *(u32x4*)(u_lds + (4 * r4 + w) * URS + HALO + lane * 8) = gate_mul<PRE>(c1[r4], cv[r4]);
+        for (int r4 = 0; r4 < 4; ++r4) {
+            if constexpr (FEAT != 0) {
+                const u32x4 f1 = feat(c1[r4], car1[r4], fw[0][r4]);
+                const u32x4 fv = feat(cv[r4], carv[r4], fw[2][r4]);
+                *(u32x4*)(u_lds + (4 * r4 + w) * URS + HALO + lane * 8) = gate_mul<true>(f1, fv);
+                __builtin_amdgcn_sched_barrier(0);         // one row at a time: its temporaries are dead before the next starts
+            } else {
+                *(u32x4*)(u_lds + (4 * r4 + w) * URS + HALO + lane * 8) = gate_mul<PRE>(c1[r4], cv[r4]);
+            }
+        }
         __syncthreads();
 
         // prefetch the next step's x1, v, x2 (x2 of this step moves to c2)
@@ -245,6 +315,15 @@ __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
         __syncthreads();
 
         *(u32x4*)(u_lds + (tid >> 4) * URS + (tid & 15) * 8) = tail;
+        if constexpr (FEAT != 0) {
+            // the output gate of this step, outside any test: every wavefront carries every piece on.  (Behind the
+            // MFMAs instead, with both accumulators live, it spills 13 registers and measured 1 % slower.)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                c2[r4] = feat(c2[r4], car2[r4], fw[1][r4]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
         // ---- gate with x2 and store, coalesced
         if (WHOLE || ts + lane * 8 < t_end) {
             uint32_t lo = lane_b;
@@ -278,21 +357,48 @@ __global__ __launch_bounds__(256, 3) void mr_fir_kernel(RowMap x1, RowMap x2, Ro
 
 }  // namespace
 
+namespace {
+int mr_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const float* h,
+                int taps_reversed, const float* bias, int bias_mode, void* out, int64_t B, int64_t D, int64_t L,
+                int64_t G, int K, void* stream, const float* ftaps);
+}
+
 extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const float* h,
                             int taps_reversed, const float* bias, int bias_mode, void* out, int64_t B, int64_t D,
                             int64_t L, int64_t G, int K, void* stream) {
-    if (!x1 || !x1->ptr || !h || !out) return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: x1, h and out are required");
+    return mr_fwd_impl("hyena_mr_fwd", x1, x2, v, h, taps_reversed, bias, bias_mode, out, B, D, L, G, K, stream, nullptr);
+}
+
+extern "C" int hyena_fir_layer_fwd_rows(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v,
+                                        const float* feat_taps, int feat_len, const float* h, int taps_reversed,
+                                        const float* bias, int bias_mode, void* out, int64_t B, int64_t D, int64_t L,
+                                        int64_t G, int K, void* stream) {
+    const char* who = "hyena_fir_layer_fwd_rows";
+    if (!feat_taps) return hyena_fail(HYENA_EINVAL, "%s: feat_taps is required", who);
+    if (feat_len != 3) return hyena_fail(HYENA_ENOSUP, "%s: featurizer of %d taps (3)", who, feat_len);
+    if (!x1 || !x1->ptr || !x2 || !x2->ptr || !v || !v->ptr)
+        return hyena_fail(HYENA_EINVAL, "%s: the three row sets of the projection are required", who);
+    if (bias_mode != HYENA_BIAS_NONE && bias_mode != HYENA_BIAS_GATED_FP32)
+        return hyena_fail(HYENA_ENOSUP, "%s: bias_mode %d (none or gated float32)", who, bias_mode);
+    return mr_fwd_impl(who, x1, x2, v, h, taps_reversed, bias, bias_mode, out, B, D, L, G, K, stream, feat_taps);
+}
+
+namespace {
+int mr_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const float* h,
+                int taps_reversed, const float* bias, int bias_mode, void* out, int64_t B, int64_t D, int64_t L,
+                int64_t G, int K, void* stream, const float* ftaps) {
+    if (!x1 || !x1->ptr || !h || !out) return hyena_fail(HYENA_EINVAL, "%s: x1, h and out are required", who);
     if (B < 0 || D <= 0 || L < 0 || G <= 0 || D % G != 0)
-        return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: bad sizes B=%lld D=%lld L=%lld G=%lld", (long long)B,
+        return hyena_fail(HYENA_EINVAL, "%s: bad sizes B=%lld D=%lld L=%lld G=%lld", who, (long long)B,
                           (long long)D, (long long)L, (long long)G);
-    if (K < 1 || K > 128) return hyena_fail(HYENA_ENOSUP, "hyena_mr_fwd: K=%d outside 1..128", K);
+    if (K < 1 || K > 128) return hyena_fail(HYENA_ENOSUP, "%s: K=%d outside 1..128", who, K);
     if (bias_mode < 0 || bias_mode > 4 || (bias_mode != HYENA_BIAS_NONE && !bias))
-        return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: bias_mode %d needs a bias pointer", bias_mode);
+        return hyena_fail(HYENA_EINVAL, "%s: bias_mode %d needs a bias pointer", who, bias_mode);
     if (L % 8 != 0 || !rows_aligned8(x1) || !rows_aligned8(x2) || !rows_aligned8(v) || (((uintptr_t)out) & 15))
-        return hyena_fail(HYENA_EALIGN, "hyena_mr_fwd: L and strides must be multiples of 8, pointers 16-byte aligned");
+        return hyena_fail(HYENA_EALIGN, "%s: L and strides must be multiples of 8, pointers 16-byte aligned", who);
     // the kernels do the channel arithmetic in 32 bits: reject maps and sizes that would wrap or divide by zero
     if (!rows_valid(x1) || !rows_valid(x2) || !rows_valid(v) || B * D >= (1LL << 31) || L / 8 >= (1LL << 31))
-        return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: B*D, L/8 and the channel map must fit 31 bits");
+        return hyena_fail(HYENA_EINVAL, "%s: B*D, L/8 and the channel map must fit 31 bits", who);
     if (B == 0 || L == 0) return 0;
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
 
@@ -319,7 +425,7 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     seg_len = (seg_len + TL - 1) / TL * TL;
     nseg = (L + seg_len - 1) / seg_len;
     const int64_t nblk = rows * nseg;
-    if (nblk > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "hyena_mr_fwd: problem too large for one launch");
+    if (nblk > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: problem too large for one launch", who);
 
     RowMap m1 = make_rowmap(x1), m2 = make_rowmap(post ? x2 : nullptr), mv = make_rowmap(pre ? v : nullptr);
     hipStream_t s = (hipStream_t)stream;
@@ -332,7 +438,7 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     const bool full = K > 98;
 #define MR_LAUNCH(P, Q, M, N, F)                                                                              \
     hipLaunchKernelGGL((mr_fir_kernel<P, Q, M, N, F>), grid, dim3(256), 0, s, m1, m2, mv, h, K, taps_reversed, \
-                       bias, (bf16_t*)out, D, L, dg, seg_len, (int)nseg)
+                       bias, (bf16_t*)out, D, L, dg, seg_len, (int)nseg, ftaps)
 #define MR_CASE(P, Q, M)                                                                                      \
     if (pre == P && post == Q && bias_mode == M) {                                                            \
         if (nt && full) MR_LAUNCH(P, Q, M, true, true);                                                       \
@@ -341,6 +447,21 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
         else MR_LAUNCH(P, Q, M, false, false);                                                                \
         ok = true;                                                                                            \
     }
+#define MR_FEAT(M)                                                                                            \
+    if (ftaps && bias_mode == M) {                                                                            \
+        if (nt && full) hipLaunchKernelGGL((mr_fir_kernel<true, true, M, true, true, 3>), grid, dim3(256), 0, s, m1, m2, mv, h, K, taps_reversed, bias, (bf16_t*)out, D, L, dg, seg_len, (int)nseg, ftaps);   \
+        else if (nt) hipLaunchKernelGGL((mr_fir_kernel<true, true, M, true, false, 3>), grid, dim3(256), 0, s, m1, m2, mv, h, K, taps_reversed, bias, (bf16_t*)out, D, L, dg, seg_len, (int)nseg, ftaps);    \
+        else if (full) hipLaunchKernelGGL((mr_fir_kernel<true, true, M, false, true, 3>), grid, dim3(256), 0, s, m1, m2, mv, h, K, taps_reversed, bias, (bf16_t*)out, D, L, dg, seg_len, (int)nseg, ftaps); \
+        else hipLaunchKernelGGL((mr_fir_kernel<true, true, M, false, false, 3>), grid, dim3(256), 0, s, m1, m2, mv, h, K, taps_reversed, bias, (bf16_t*)out, D, L, dg, seg_len, (int)nseg, ftaps);         \
+        ok = true;                                                                                            \
+    }
+    if (ftaps) {
+        MR_FEAT(HYENA_BIAS_GATED_FP32)
+        MR_FEAT(HYENA_BIAS_NONE)
+        if (!ok) return hyena_fail(HYENA_ENOSUP, "%s: this bias mode has no featurizer kernel", who);
+        return hyena_check_launch(who);
+    }
+#undef MR_FEAT
     MR_CASE(true, true, HYENA_BIAS_GATED_FP32)
     MR_CASE(true, true, HYENA_BIAS_NONE)
     MR_CASE(true, true, HYENA_BIAS_ADD)
@@ -353,6 +474,7 @@ extern "C" int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hy
     MR_CASE(false, false, HYENA_BIAS_GATED_BF16)
 #undef MR_CASE
 #undef MR_LAUNCH
-    if (!ok) return hyena_fail(HYENA_ENOSUP, "hyena_mr_fwd: this gate/bias combination has no kernel");
-    return hyena_check_launch("hyena_mr_fwd");
+    if (!ok) return hyena_fail(HYENA_ENOSUP, "%s: this gate/bias combination has no kernel", who);
+    return hyena_check_launch(who);
 }
+}  // namespace

@@ -136,6 +136,27 @@ def fir_fwd_rows(x1r, x2r, vr, taps, B, D, L, K, *, device, bias=None, bias_mode
     return out
 
 
+def fir_layer_fwd_rows(x1r, x2r, vr, feat_taps, taps, B, D, L, K, *, device, bias=None, bias_mode=HYENA_BIAS_NONE,
+                       taps_reversed=False, out=None):
+    """hyena_fir_layer_fwd_rows: a whole Hyena-SE / MR layer in one pass over the rows of a raw sequence-major
+    projection -- the three-tap featurizer FIR on every piece as it is read, then the gated FIR of fir_fwd_rows on the
+    matrix cores (any K <= 128).  feat_taps [3, D, 3] float32: the featurizer weight rows of the x1, x2 and v row of
+    every operator channel, oldest sample first.  Returns out [B, D, L] bf16."""
+    taps = _f32(taps)
+    G = taps.shape[0]
+    if out is None:
+        out = torch.empty((B, D, L), dtype=torch.bfloat16, device=device)
+    if out.numel() == 0:
+        return out
+    if feat_taps.dtype != torch.float32 or not feat_taps.is_contiguous() or tuple(feat_taps.shape) != (3, D, 3):
+        raise ValueError("feat_taps must be a contiguous float32 [3, D, 3] tensor")
+    rc = _lib.lib().hyena_fir_layer_fwd_rows(_ref(x1r), _ref(x2r), _ref(vr), _ptr(feat_taps), 3, _ptr(taps),
+                                             int(taps_reversed), _ptr(bias), bias_mode, _ptr(out), B, D, L, G, K,
+                                             _stream())
+    _lib.check(rc, "hyena_fir_layer_fwd_rows")
+    return out
+
+
 def _cl_of(t, dtype=torch.bfloat16):
     """hyena_cl of a [B, L, D] tensor of `dtype` with contiguous channels (any batch / time stride)."""
     if t is None:
