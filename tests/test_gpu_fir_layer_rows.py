@@ -2,7 +2,7 @@
 featurizer FIR of vortex/model/model.py:233-246 (vortex/model/engine.py:188-223), the split under every channel map of
 vortex/model/utils.py:26-85 and the gated inner FIR of engine.py:131-260 on the matrix cores.
 
-(1) bit for bit the featurizer kernel followed by hyena_mr_fwd on its gates, across channel maps, filter lengths,
+(1) bit for bit the featurizer kernel followed by hyena_mr_fwd (hyena_se_fwd for filters of at most 8 taps) on its gates, across channel maps, filter lengths,
 segmentations along L, group sizes that do not fill an MFMA tile and ragged lengths; (2) against the oracle's
 featurizer + gated convolution within the bf16 tolerance 2e-2 and the per-element forward-error bound."""
 import pytest
@@ -25,7 +25,7 @@ def _case(B, L, D, G, K, seed):
     return u, w, h, Dc
 
 
-def _both(u, w, h, Dc, D, K, il, hd, **ov):
+def _both(u, w, h, Dc, D, K, il, hd, mfma=None, **ov):
     B, L, _ = u.shape
     mr = K >= 128
     bm = HYENA_BIAS_GATED_FP32 if mr else HYENA_BIAS_NONE
@@ -33,7 +33,7 @@ def _both(u, w, h, Dc, D, K, il, hd, **ov):
         z = ops.featurizer_fwd(u, w, None, interleave=il)
         r2, r1, rv = (ops.rows_of_projection(z, D, i, hd) for i in range(3))
         y0 = ops.fir_fwd_rows(r1, r2, rv, h, B, D, L, K, device=DEV, bias=Dc, bias_mode=bm, taps_reversed=not mr,
-                              force_mfma=True)
+                              force_mfma=K > 8 if mfma is None else mfma)      # short filters: the direct-form kernel on both sides
         p = u.transpose(1, 2).contiguous()
         (q2, q1, qv), chan = ops.projection_rows(p, D, interleave=il, head_dim=hd)
         taps = torch.stack([w[chan[1]], w[chan[0]], w[chan[2]]]).contiguous()
@@ -48,6 +48,12 @@ def _both(u, w, h, Dc, D, K, il, hd, **ov):
                                           (1, 8192, 256, 16, 128, {"mr_nseg": 4}),         # segments along L: carried history at each start
                                           (1, 4096, 256, 16, 20, {"mr_nseg": 3, "mr_nt": 1}),
                                           (2, 72, 128, 8, 128, {}),                        # shorter than a step
+                                          (2, 72, 128, 8, 7, {}),                          # short filter: blocks straddle rows
+                                          (3, 8, 128, 8, 4, {}),                           # one octet per row
+                                          (1, 2072, 120, 8, 7, {}),
+                                          (2, 16, 64, 64, 2, {}),
+                                          (1, 16384, 64, 4, 7, {"se_nt": 1}),              # whole blocks per row, streaming accesses
+                                          (1, 16384, 64, 4, 7, {"mr_nseg": 2}),
                                           (1, 2048, 120, 8, 128, {}),                      # groups of 15 channels: a part-filled slab
                                           (3, 1536, 64, 64, 128, {"mr_nseg": 3})])         # one filter per channel
 def test_fir_layer_rows_equals_featurizer_then_fir(mode, B, L, D, G, K, ov):
@@ -99,6 +105,19 @@ def test_fir_layer_rows_argument_errors():
     assert call(*args(K=200)) == ENOSUP
     assert call(*args(L=60)) == EALIGN
     torch.cuda.synchronize()
+
+
+@pytest.mark.timeout(600)
+def test_fir_layer_rows_short_filter_on_streaming_tensors():
+    """Hyena-SE rows at batch 8 (2.1 GB: beyond the last-level cache), where the entry point runs short filters on the
+    matrix-core kernel: bit for bit the featurizer kernel followed by hyena_mr_fwd with the same filter."""
+    B, L, D, G, K = 8, 8192, 4096, 256, 7
+    g = torch.Generator(device=DEV).manual_seed(2)
+    u = torch.randn(B, L, 3 * D, generator=g, device=DEV, dtype=torch.float32).to(torch.bfloat16)
+    w = (torch.randn(3 * D, 3, generator=g, device=DEV) / 3 ** 0.5).to(torch.bfloat16).float()
+    h = O.make_se_filter(G, K).reshape(G, K).to(DEV)
+    y0, y1 = _both(u, w, h, None, D, K, True, None, mfma=True)
+    assert torch.equal(y0, y1)
 
 
 @pytest.mark.timeout(600)

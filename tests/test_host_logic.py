@@ -278,3 +278,24 @@ def test_hyena_ops_reshape_helpers_follow_the_index_definitions():
     f, w = DefaultTwoPassChunkedGateConvGateFwdConfig(), DefaultTwoPassChunkedGateConvGateBwdConfig()
     assert (f.autotune, f.CHUNK_SIZE, f.BLOCK_D, f.RETURN_Y2) == (True, 128, 32, True)
     assert (w.LOAD_TOEPLITZ, w.LOAD_BX_LAG, w.name) == (False, False, "bwd")
+
+
+def test_projection_row_descriptors_reject_maps_outside_the_tensor():
+    # the row descriptors address rows up to 3*hidden - 1 of the projection; a head size that does not divide the
+    # width, or a tensor of another height, would make a kernel read outside it
+    import pytest
+    import torch
+    from vortex_amd import ops
+    p = torch.zeros(1, 3 * 64, 16, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.rows_of_projection(p, 64, 2, head_dim=128)
+    with pytest.raises(ValueError):
+        ops.projection_rows(p, 64, head_dim=48)
+    with pytest.raises(ValueError):
+        ops.projection_rows(p, 32)
+    with pytest.raises(ValueError):
+        ops.projection_rows(p, 64, interleave=True, head_dim=16)
+    rows, chan = ops.projection_rows(p, 64, head_dim=16)
+    assert chan.shape == (3, 64) and int(chan.max()) == 3 * 64 - 1 and len(set(chan.flatten().tolist())) == 3 * 64
+    rows, chan = ops.projection_rows(p, 64, interleave=True)
+    assert chan[:, 5].tolist() == [15, 16, 17]

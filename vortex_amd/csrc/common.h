@@ -66,6 +66,11 @@ int hyena_fir_cl_direct(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* 
                         const float* bias, int bias_mode, void* out, void* y2_out, void* bx_out, int64_t bx_from,
                         int64_t B, int64_t L, int64_t D, int64_t G, int K, int dtype, void* stream, const char* who);
 
+// short-filter form of hyena_fir_layer_fwd_rows (se_fir.hip): 2 <= K <= 8, no inner bias, taps[g][K-1] on the current sample
+int hyena_se_layer_rows(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v, const float* feat_taps,
+                        const float* taps, void* out, int64_t B, int64_t D, int64_t L, int64_t G, int K, void* stream,
+                        const char* who);
+
 static inline bool rows_aligned8(const hyena_rows* r) {
     return r == nullptr || ((((uintptr_t)r->ptr) & 15) == 0 && r->batch_stride % 8 == 0 && r->row_stride % 8 == 0);
 }

@@ -149,12 +149,12 @@ class HyenaBlock(nn.Module):
     def forward(self, u, inference_params=None):
         xn = self.pre_norm(u)
         B, L = xn.shape[0], xn.shape[1]
-        # Prefills of Hyena-LI layers, and of Hyena-MR layers on prompts that stream through the cache (where the
-        # sequence-major form measured 7-10 % faster than the channel-last one; it is slower on cache-resident ones):
+        # Prefills of Hyena-LI layers, and of Hyena-SE / MR layers on prompts that stream through the cache (where the
+        # sequence-major form measured 7-10 % faster than the channel-last one; it is no faster on cache-resident ones):
         # the projection GEMM writes its product transposed, [B, 3D, L] with the samples contiguous, which the layer
         # then reads once (featurizer, gates and operator in one launch).  The values are those of
         # self.projections(xn), handed over as the [B, L, 3D] view of that memory.
-        if L > 1 and L % 8 == 0 and (self.kind == "hcl" or (self.kind == "hcm" and B * L >= 65536)):
+        if L > 1 and L % 8 == 0 and (self.kind == "hcl" or B * L >= 65536):
             z = torch.matmul(self.projections.weight, xn.transpose(1, 2)).transpose(1, 2)
         else:
             z = self.projections(xn)

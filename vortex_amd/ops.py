@@ -59,6 +59,10 @@ def rows_of_projection(u, hidden, which, head_dim=None):
     """
     if u.dtype != torch.bfloat16 or u.dim() != 3 or u.stride(2) != 1:
         raise ValueError("expected a [B, 3D, L] bfloat16 tensor with contiguous samples")
+    if u.shape[1] != 3 * hidden or (head_dim is not None and (head_dim <= 0 or hidden % head_dim)):
+        # the descriptors address rows up to 3*hidden - 1: anything else would read outside the tensor
+        raise ValueError(f"a [B, {3 * hidden}, L] projection and a head_dim that divides {hidden} are required "
+                         f"(got {tuple(u.shape)}, head_dim={head_dim})")
     es = u.element_size()
     if head_dim is None:
         return Rows(u.data_ptr() + which * hidden * u.stride(1) * es, u.stride(0), u.stride(1), hidden, hidden)
@@ -385,6 +389,9 @@ def projection_rows(p, hidden, *, interleave=False, head_dim=None):
         raise ValueError("interleave combined with column_split has no closed channel map")
     if p.dtype != torch.bfloat16 or p.dim() != 3 or p.stride(2) != 1:
         raise ValueError("expected a [B, 3D, L] bfloat16 tensor with contiguous samples")
+    if p.shape[1] != 3 * hidden or (head_dim is not None and (head_dim <= 0 or hidden % head_dim)):
+        raise ValueError(f"a [B, {3 * hidden}, L] projection and a head_dim that divides {hidden} are required "
+                         f"(got {tuple(p.shape)}, head_dim={head_dim})")
     d = torch.arange(hidden, device=p.device)
     if interleave:
         es = p.element_size()
