@@ -28,6 +28,9 @@ EVO2_7B = dict(
 )
 
 
+SEQ_MAJOR = "auto"      # "never": every Hyena block hands its operator a channel-last projection
+
+
 class RMSNorm(nn.Module):
     def __init__(self, hidden, eps):
         super().__init__()
@@ -149,17 +152,27 @@ class HyenaBlock(nn.Module):
     def forward(self, u, inference_params=None):
         xn = self.pre_norm(u)
         B, L = xn.shape[0], xn.shape[1]
-        # Prefills of Hyena-LI layers, and of Hyena-SE / MR layers on prompts that stream through the cache (where the
-        # sequence-major form measured 7-10 % faster than the channel-last one; it is no faster on cache-resident ones):
-        # the projection GEMM writes its product transposed, [B, 3D, L] with the samples contiguous, which the layer
-        # then reads once (featurizer, gates and operator in one launch).  The values are those of
-        # self.projections(xn), handed over as the [B, L, 3D] view of that memory.
-        if L > 1 and L % 8 == 0 and (self.kind == "hcl" or B * L >= 65536):
-            z = torch.matmul(self.projections.weight, xn.transpose(1, 2)).transpose(1, 2)
+        # Prefill of a Hyena-LI layer: the projection GEMM writes its product transposed, [B, 3D, L] with the samples
+        # contiguous, which the layer then reads once (featurizer, gates and scan in one launch).  The values are
+        # those of self.projections(xn), handed over as the [B, L, 3D] view of that memory.  One plain 2-D product per
+        # batch element: torch.matmul on the broadcast pair takes twice as long (16.6 against 8.9 ms at L = 131072).
+        # Hyena-SE / MR layers keep the channel-last projection: their sequence-major kernels are 7-10 % faster on long
+        # prompts, which the slower transposed GEMMs around them (+0.4 ms each at L = 131072) take back.
+        if SEQ_MAJOR != "never" and self.kind == "hcl" and L > 1 and L % 8 == 0:
+            W = self.projections.weight
+            p = torch.empty(B, W.shape[0], L, dtype=xn.dtype, device=xn.device)
+            for b in range(B):
+                torch.mm(W, xn[b].t(), out=p[b])
+            z = p.transpose(1, 2)
         else:
             z = self.projections(xn)
         z, _ = self.filter(z, inference_params=inference_params)
-        z_in = self.out_filter_dense(z) + u
+        if B == 1 and L > 1 and z.stride(1) == 1 and z.stride(2) == L:
+            # the operator's output is the [B, L, D] view of [B, D, L] memory: the transposed operand goes to the GEMM as it is
+            o = torch.addmm(self.out_filter_dense.bias, z[0], self.out_filter_dense.weight.t()).unsqueeze(0)
+        else:
+            o = self.out_filter_dense(z)
+        z_in = o + u
         return self.mlp(self.post_norm(z_in)) + z_in, None
 
 
