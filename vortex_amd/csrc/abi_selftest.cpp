@@ -1,6 +1,8 @@
 // Stand-alone check of the C ABI from plain C++: no torch, no Python.  Loads the shared library given
 // on the command line, allocates with hipMalloc, and verifies known answers bit for bit:
 //   hyena_mr_fwd / hyena_fir_cl_fwd   impulse response with bf16-exact taps equals the filter
+//   hyena_fir_layer_fwd_rows          the same impulse response behind a featurizer that delays by two samples
+//   hyena_li_layer_fwd                with identity featurizer taps equals hyena_li_fwd, outputs and state
 //   hyena_fir_step                    dot product over a ring cache, slot rotation
 //   hyena_fir_step_far                the same step on a deep cache read whole only every third token, 3 ring periods
 //   hyena_iir_step                    one modal update against the closed form
@@ -46,6 +48,8 @@ int main(int argc, char** argv) {
     SYM(hyena_iir_step) SYM(hyena_se_fwd) SYM(hyena_fir_step_dpos) SYM(hyena_ring_advance)
     SYM(hyena_fir_step_far) SYM(hyena_fir_far_period) SYM(hyena_fir_far_bytes)
     SYM(hyena_iir_step_win) SYM(hyena_iir_window_flush) SYM(hyena_iir_window_tokens) SYM(hyena_iir_window_supported)
+    SYM(hyena_fir_layer_fwd_rows) SYM(hyena_li_layer_fwd) SYM(hyena_li_fwd) SYM(hyena_li_plan) SYM(hyena_li_plan_bytes)
+    SYM(hyena_set_launch_override)
     printf("%s\n", p_hyena_version());
     hipStream_t stream; HIP_OK(hipStreamCreate(&stream));
 
@@ -87,6 +91,71 @@ int main(int argc, char** argv) {
                   from_bf16(o[t * D + d]), e);
         }
         printf("hyena_fir_cl_fwd impulse response: ok\n");
+    }
+
+    // ---- a layer from a sequence-major projection p [B][3D][L] (plain split: rows x2 | x1 | v).  Featurizer taps:
+    // x1 (1, 0, 0) = a delay of two samples, x2 (0.5, 0.25, 0.25) = 1 from t = 2 on for a row of ones, v (0, 0, 1) = the
+    // identity.  The x1 rows hold the impulses, so the output is the filter's impulse response two samples late.
+    {
+        std::vector<uint16_t> proj(B * 3 * D * L, to_bf16(1.f));
+        for (int d = 0; d < D; ++d) for (int t = 0; t < L; ++t) proj[(D + d) * L + t] = imp[d * L + t];
+        std::vector<float> ft(3 * D * 3, 0.f);
+        for (int d = 0; d < D; ++d) {
+            ft[(0 * D + d) * 3 + 0] = 1.f;
+            ft[(1 * D + d) * 3 + 0] = 0.5f; ft[(1 * D + d) * 3 + 1] = 0.25f; ft[(1 * D + d) * 3 + 2] = 0.25f;
+            ft[(2 * D + d) * 3 + 2] = 1.f;
+        }
+        uint16_t* d_p = dev(proj); float* d_ft = dev(ft);
+        hyena_rows q2 = {d_p, 3 * D * L, L, D, D}, q1 = {d_p + D * L, 3 * D * L, L, D, D}, qv = {d_p + 2 * D * L, 3 * D * L, L, D, D};
+        int rc = p_hyena_fir_layer_fwd_rows(&q1, &q2, &qv, d_ft, 3, dh, 0, nullptr, HYENA_BIAS_NONE, d_out, B, D, L, G, K, stream);
+        CHECK(rc == 0, "hyena_fir_layer_fwd_rows rc=%d: %s", rc, p_hyena_last_error_string());
+        HIP_OK(hipStreamSynchronize(stream));
+        auto o = host(d_out, (size_t)(B * D * L));
+        for (int d = 0; d < D; ++d) for (int t = 0; t < L; ++t) {
+            float e = 0.f;
+            for (int pp : pos) if (t - 2 >= pp && t - 2 - pp < K) e += h[(d / 16) * K + t - 2 - pp];
+            CHECK(from_bf16(o[d * L + t]) == from_bf16(to_bf16(e)), "hyena_fir_layer_fwd_rows d=%d t=%d got %g want %g", d, t,
+                  from_bf16(o[d * L + t]), e);
+        }
+        printf("hyena_fir_layer_fwd_rows impulse response behind a two-sample featurizer delay: ok\n");
+
+        // the same projection through hyena_li_layer_fwd with identity featurizer taps on every row must be
+        // hyena_li_fwd on the rows themselves, bit for bit (lone wavefronts on both sides)
+        const int64_t S = 16;
+        std::vector<float> lp(G * S * 2, 0.f), rs(G * S * 2, 0.f);
+        for (int g = 0; g < G; ++g) for (int m = 0; m < S; ++m) {
+            lp[(g * S + m) * 2] = -0.02f * (float)(m + 1 + g);  lp[(g * S + m) * 2 + 1] = 0.1f * (float)m;
+            rs[(g * S + m) * 2] = 0.25f - 0.03f * (float)m;     rs[(g * S + m) * 2 + 1] = 0.01f * (float)(m + g);
+        }
+        std::vector<float> idt(3 * D * 3, 0.f);
+        for (int i = 0; i < 3 * D; ++i) idt[i * 3 + 2] = 1.f;
+        for (int d = 0; d < D; ++d) for (int t = 0; t < L; ++t) {               // less trivial gates than ones
+            proj[d * L + t] = to_bf16((float)((t * 7 + d) % 13 - 6) / 8.f);
+            proj[(2 * D + d) * L + t] = to_bf16((float)((t * 3 + d * 5) % 11 - 5) / 4.f);
+            proj[(D + d) * L + t] = to_bf16((float)((t + d * 2) % 9 - 4) / 4.f);
+        }
+        HIP_OK(hipMemcpy(d_p, proj.data(), proj.size() * 2, hipMemcpyHostToDevice));
+        float *d_lp = dev(lp), *d_rs = dev(rs), *d_id = dev(idt), *d_st0, *d_st1; void* d_ws; uint16_t* d_out2;
+        HIP_OK(hipMalloc(&d_ws, (size_t)p_hyena_li_plan_bytes(G, S)));
+        HIP_OK(hipMalloc(&d_out2, B * D * L * 2));
+        HIP_OK(hipMalloc(&d_st0, B * D * S * 2 * 4)); HIP_OK(hipMalloc(&d_st1, B * D * S * 2 * 4));
+        rc = p_hyena_li_plan(d_lp, d_rs, G, S, d_ws, stream);
+        CHECK(rc == 0, "hyena_li_plan rc=%d: %s", rc, p_hyena_last_error_string());
+        CHECK(p_hyena_set_launch_override("li_coop", 0) == 0, "li_coop override");
+        rc = p_hyena_li_fwd(&q1, &q2, &qv, d_ws, nullptr, 1, d_out, nullptr, d_st0, B, D, L, G, S, stream);
+        CHECK(rc == 0, "hyena_li_fwd rc=%d: %s", rc, p_hyena_last_error_string());
+        CHECK(p_hyena_set_launch_override("li_coop", -1) == 0, "li_coop override reset");
+        rc = p_hyena_li_layer_fwd(&q1, &q2, &qv, d_id, 3, d_ws, nullptr, 1, d_out2, d_st1, B, D, L, G, S, stream);
+        CHECK(rc == 0, "hyena_li_layer_fwd rc=%d: %s", rc, p_hyena_last_error_string());
+        HIP_OK(hipStreamSynchronize(stream));
+        auto oa = host(d_out, (size_t)(B * D * L)); auto ob = host(d_out2, (size_t)(B * D * L));
+        CHECK(oa == ob, "hyena_li_layer_fwd with identity featurizer taps differs from hyena_li_fwd");
+        auto sa = host(d_st0, (size_t)(B * D * S * 2)); auto sb = host(d_st1, (size_t)(B * D * S * 2));
+        CHECK(memcmp(sa.data(), sb.data(), sa.size() * 4) == 0, "hyena_li_layer_fwd state differs from hyena_li_fwd");
+        bool nonzero = false;
+        for (auto x : ob) nonzero |= (x & 0x7fff) != 0;
+        CHECK(nonzero, "hyena_li_layer_fwd wrote only zeros");
+        printf("hyena_li_layer_fwd with identity featurizer taps equals hyena_li_fwd (outputs and state): ok\n");
     }
 
     // ---- decode FIR step: ring [B=2][R=6][D=16], per-channel taps, two steps (slot rotation)
