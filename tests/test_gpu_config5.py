@@ -80,7 +80,7 @@ def test_7b_shaped_stack_at_full_depth_vs_oracle():
 
 
 @pytest.mark.timeout(900)
-@pytest.mark.parametrize("kind", ["hcs", "hcm", "hcl"])
+@pytest.mark.parametrize("kind", ["hcs", "hcm", "hcl", "hcl_rows", "hcm_rows"])
 def test_7b_shaped_hyena_layers_at_L131072(kind):
     """The long leg of the end-to-end configuration (B = 1, L = 131072, hidden 4096): each of the three Hyena operator
     modules of a [SE, MR, LI, attention] group exactly as the stack runs it (projection u [1, L, 3*4096] in the
@@ -93,11 +93,17 @@ def test_7b_shaped_hyena_layers_at_L131072(kind):
     from vortex_amd.cascade import HyenaCascadeFIRInferenceParams, HyenaCascadeIIRInferenceParams
     cfg = dict(EVO2_7B)
     D, L = cfg["hidden_size"], 131072
+    # "_rows": the same projection values stored sequence-major ([1, 3D, L], as the stack's Hyena-LI blocks ask their
+    # projection GEMM to write them), which the module runs in one launch with the featurizer inside the operator kernel
+    rows, kind = kind.endswith("_rows"), kind.split("_")[0]
     m = StripedHyena2(dict(cfg, num_layers=4), seed=31, device="cuda").to_inference("cuda")
     mod = m.blocks[("hcs", "hcm", "hcl").index(kind)].filter
     K = mod.fir_inner_filter_length
     g = torch.Generator(device="cuda").manual_seed(32)
     u = torch.randn(1, L, 3 * D, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    if rows:
+        u = u.transpose(1, 2).contiguous().transpose(1, 2)
+        assert mod._can_scan_projection_rows(u) or mod._can_filter_projection_rows(u)
     with torch.no_grad():
         if kind == "hcl":       # slow poles too (|p| up to 0.9999): a memory that spans the whole prompt
             mod.log_poles.copy_(-(1e-4 + 0.1 * torch.rand(mod.log_poles.shape, generator=g, device="cuda")))
@@ -134,7 +140,7 @@ def test_7b_shaped_hyena_layers_at_L131072(kind):
             fa = ip.fir_state_dict[mod.layer_idx].reference_order()[:, sl].cpu()
             assert torch.equal(fa, ip_ref.fir_state_dict[0].float())
         # ---- causality: the first 8192 outputs do not depend on what follows (another launch shape, same values)
-        y_head, _ = mod(u[:, :8192].contiguous())
+        y_head, _ = mod(u[:, :8192].contiguous())          # (a channel-last copy: the other path of the module)
         d = (y_head.float() - y[:, :8192].float()).abs().max() / y[:, :8192].float().abs().max()
         assert d <= 2.0 ** -7, d            # at most the last bf16 digit (another segmentation of the same sums)
         # ---- prefill of L - 8 samples, then 8 cached steps, against the last 8 outputs of the full prefill

@@ -544,6 +544,8 @@ class HyenaCascade(nn.Module):
         """Decode: u [B, 3D] or [B, 1, 3D] bf16 -> y [B, 1, D] (vortex/model/model.py:318-375)."""
         if u.dim() > 2:
             u = u[:, -1]
+        if u.shape[1] > 1 and u.stride(1) != 1:      # a token cut from a sequence-major projection: the step kernels
+            u = u.contiguous()                        # take contiguous channels (a copy of 6*D bytes per batch element)
         d = self._decode_plan(inference_params)
         B = u.shape[0]
         rings = [d["ring"]] + ([d["inner"].ring] if self.fir_inner_filter_length else [])
