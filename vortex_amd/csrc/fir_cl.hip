@@ -730,7 +730,7 @@ static int fir_cl_launch(const LaunchArgs& a, const float* h, int taps_reversed,
     // tensors that stay in the cache lose 2-11 %, as do rows shorter than 4096 samples in the fused form.
     const bool streams = 8.0 * (double)B * (double)D * (double)L > 384e6;
     const int ns_form = a.feat ? 2 : 3;
-    const bool ns_able = !(y2_out || bx_out) && !a.f16 && (D + CB - 1) / CB >= 2 * ns_form;
+    const bool ns_able = !(y2_out || bx_out) && !a.f16 && (D + CB - 1) / CB >= 2 * ns_form;   // (the float16 kernels are built for one strip per block only)
     int ns = (ns_able && streams && L >= 4096) ? ns_form : 1;
     { const int64_t x = hyena_override(HYENA_OV_CL_NS); if (x >= 1) ns = (x > 1 && ns_able) ? ns_form : 1; }
     const int64_t ndb = ((D + CB - 1) / CB + ns - 1) / ns;       // blocks along the channels
