@@ -833,3 +833,34 @@ def test_operator_module_sequence_major_projection_fir(kind, cs, il, flip):
         y_ref, _ = ref.forward(tok, ip_ref)
         y_hip, _ = mod(tok.to(DEV), ip_hip)
         assert rel_err(y_hip, y_ref) <= 2e-2, i
+
+
+def test_sequence_major_projection_wrapper_feeds_the_one_launch_layer():
+    """use_hip_filters(model, sequence_major_projections=True): the wrapped projection of a Hyena-LI block hands the
+    cascade the projection's values stored sequence-major, the cascade runs one launch, and the result agrees with
+    the same block on the plain linear layer (channel-last projection, two launches) to the last bf16 digit."""
+    import types
+    from vortex_amd.cascade import SequenceMajorProjection, use_hip_filters
+    B, L, D, H, G = 2, 256, 64, 4, 4
+    p = make_params("li_real", D, G, seed=31)
+    cfg = dict(hidden_size=D, num_attention_heads=H, column_split_hyena=False, interleave=True, short_filter_length=3,
+               short_filter_bias=False, state_size=16)
+    mod = HyenaCascade(cfg, 0, hyena_filter_groups=G)
+    with torch.no_grad():
+        mod.short_filter_weight.copy_(p["short_filter_weight"])
+        mod.log_poles.copy_(p["log_poles"])
+        mod.residues.copy_(p["residues"])
+        mod.D.data = p["D"].clone()
+    lin = torch.nn.Linear(D, 3 * D, bias=False)
+    block = types.SimpleNamespace(filter=mod.to(DEV), projections=lin.to(DEV).to(torch.bfloat16))
+    use_hip_filters(types.SimpleNamespace(blocks=[block]), sequence_major_projections=True)
+    assert isinstance(block.projections, SequenceMajorProjection)
+    x = torch.randn(B, L, D, generator=torch.Generator().manual_seed(7)).bfloat16().to(DEV)
+    z_seq, z_cl = block.projections(x), block.projections.linear(x)
+    assert z_seq.shape == z_cl.shape and z_seq.stride(1) == 1
+    assert rel_err(z_seq, z_cl) <= 2.0 ** -7                     # two GEMM kernels, one bf16 digit
+    assert block.projections(x[:, :1]).is_contiguous()           # a decode token goes through the layer itself
+    y_seq, _ = block.filter(z_seq)
+    assert "wf_rows" in block.filter._f32_cache
+    y_cl, _ = block.filter(z_seq.contiguous())                   # the same values channel-last: two launches
+    assert rel_err(y_seq, y_cl) <= 2.0 ** -7

@@ -157,6 +157,20 @@ def test_from_vortex_shares_parameters_and_config():
     model = types.SimpleNamespace(blocks=blocks)
     assert use_hip_filters(model) == 2 and use_hip_filters(model) == 0
     assert isinstance(blocks[2].filter, HyenaCascade) and blocks[2].filter.log_poles is modal.log_poles
+    # sequence_major_projections wraps the projection of the Hyena-LI block only, keeps the layer's parameters, and
+    # falls back to the layer itself wherever the one-launch path does not apply (here: tensors on the CPU)
+    from vortex_amd.cascade import SequenceMajorProjection, project_sequence_major
+    lin_fir, lin_modal = torch.nn.Linear(64, 192, bias=False), torch.nn.Linear(64, 192, bias=False)
+    blocks[0].projections, blocks[2].projections = lin_fir, lin_modal
+    assert use_hip_filters(model, sequence_major_projections=True) == 0
+    assert blocks[0].projections is lin_fir
+    wrapped = blocks[2].projections
+    assert isinstance(wrapped, SequenceMajorProjection) and wrapped.linear is lin_modal and wrapped.weight is lin_modal.weight
+    x = torch.randn(2, 16, 64)
+    assert torch.equal(wrapped(x), lin_modal(x)) and wrapped(x).is_contiguous()
+    z = project_sequence_major(lin_modal.weight.detach(), x)
+    assert z.shape == (2, 16, 192) and z.stride(1) == 1 and z.stride(2) == 16
+    assert torch.allclose(z, lin_modal(x), atol=1e-5)
 
 
 def test_hyena_ops_utils_toeplitz_factors():

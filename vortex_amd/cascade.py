@@ -74,16 +74,62 @@ def _cfg(config, key, default=None):
     return default if v is None else v
 
 
-def use_hip_filters(model):
+def project_sequence_major(weight, x):
+    """The dense projection x [B, L, H] -> [B, L, C] with weight [C, H] (no bias), computed as W x^T so that the GEMM
+    writes [B, C, L] with the samples contiguous; returned as the [B, L, C] view of that memory.  Same values as
+    F.linear(x, weight) up to the GEMM's own summation order.  One plain 2-D product per batch element (torch.matmul
+    on the broadcast pair measured twice as slow)."""
+    B, L, _ = x.shape
+    weight, x = weight.detach(), x.detach()         # forward only: the products are written in place
+    p = torch.empty(B, weight.shape[0], L, dtype=x.dtype, device=x.device)
+    for b in range(B):
+        torch.mm(weight, x[b].t(), out=p[b])
+    return p.transpose(1, 2)
+
+
+class SequenceMajorProjection(nn.Module):
+    """Stands in for the `projections` linear layer of a Hyena block (vortex/model/model.py:490-492 calls it on the
+    normalised input): the same projection, stored sequence-major for prefills, so that a Hyena-LI cascade behind it
+    runs featurizer, gates and scan in one launch.  Decode tokens, prompts that are not a whole number of 8-sample
+    pieces, biased layers and anything that is not a plain linear layer on the GPU go through the wrapped layer
+    unchanged.  The wrapped layer keeps its parameters (and their names under `.linear`)."""
+
+    def __init__(self, linear):
+        super().__init__()
+        self.linear = linear
+
+    @property
+    def weight(self):
+        return self.linear.weight
+
+    @property
+    def bias(self):
+        return getattr(self.linear, "bias", None)
+
+    def forward(self, x):
+        lin = self.linear
+        if (isinstance(lin, nn.Linear) and lin.bias is None and x.dim() == 3 and x.is_cuda and x.shape[1] > 1
+                and x.shape[1] % 8 == 0 and x.dtype == lin.weight.dtype):
+            return project_sequence_major(lin.weight, x)
+        return lin(x)
+
+
+def use_hip_filters(model, sequence_major_projections=False):
     """Replaces the `filter` of every Hyena block of a vortex model (an object with `.blocks`, each Hyena block
     holding its HyenaCascade as `.filter`, vortex/model/model.py:523-575) by its counterpart on the HIP kernels.
-    Returns the number of blocks switched."""
+    sequence_major_projections=True also wraps the `projections` layer of the Hyena-LI blocks in a
+    SequenceMajorProjection, so that their prefill runs in one launch.  Returns the number of blocks switched."""
     n = 0
     for block in model.blocks:
         f = getattr(block, "filter", None)
         if f is not None and hasattr(f, "short_filter_weight") and not isinstance(f, HyenaCascade):
             block.filter = HyenaCascade.from_vortex(f)
             n += 1
+        f = getattr(block, "filter", None)
+        proj = getattr(block, "projections", None)
+        if (sequence_major_projections and isinstance(f, HyenaCascade) and f._can_fuse_gates_layer()
+                and isinstance(proj, nn.Linear) and proj.bias is None):
+            block.projections = SequenceMajorProjection(proj)
     return n
 
 

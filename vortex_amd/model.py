@@ -17,7 +17,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import ops
-from .cascade import HyenaCascade, HyenaCascadeFIRInferenceParams, HyenaCascadeIIRInferenceParams
+from .cascade import (HyenaCascade, HyenaCascadeFIRInferenceParams, HyenaCascadeIIRInferenceParams,
+                      project_sequence_major)
 
 EVO2_7B = dict(
     vocab_size=512, hidden_size=4096, num_layers=32, num_attention_heads=32, inner_mlp_size=11008,
@@ -159,11 +160,7 @@ class HyenaBlock(nn.Module):
         # Hyena-SE / MR layers keep the channel-last projection: their sequence-major kernels are 7-10 % faster on long
         # prompts, which the slower transposed GEMMs around them (+0.4 ms each at L = 131072) take back.
         if SEQ_MAJOR != "never" and self.kind == "hcl" and L > 1 and L % 8 == 0:
-            W = self.projections.weight
-            p = torch.empty(B, W.shape[0], L, dtype=xn.dtype, device=xn.device)
-            for b in range(B):
-                torch.mm(W, xn[b].t(), out=p[b])
-            z = p.transpose(1, 2)
+            z = project_sequence_major(self.projections.weight, xn)
         else:
             z = self.projections(xn)
         z, _ = self.filter(z, inference_params=inference_params)
