@@ -325,3 +325,57 @@ def test_offsets_beyond_32_bits():
         ref = O.mr_fir(a2, a1, av, h128[g:g + 1], Db[rows])[0]
         err = (out[1:2, :, rows].transpose(1, 2).float().cpu() - ref.float()).abs().max() / ref.float().abs().max()
         assert err <= 2e-2, (g, err.item())
+
+
+@pytest.mark.parametrize("B,L,seed", cases(7, 14))
+def test_rows_layers_random(B, L, seed, override):
+    """The one-launch layers from a sequence-major projection (hyena_fir_layer_fwd_rows, hyena_li_layer_fwd) on ragged
+    shapes, random channel maps, group sizes and segmentations: bit for bit the featurizer kernel followed by the
+    operator kernel on its gates, and against the oracle's layer (OracleCascade) within the bf16 tolerance."""
+    from vortex_amd._lib import HYENA_BIAS_GATED_FP32, HYENA_BIAS_NONE
+    rng = random.Random(seed)
+    kind = rng.choice(["se", "mr", "mr_short", "li", "li"])
+    H = rng.choice([1, 2, 4])
+    dg = rng.choice([4, 8, 16, 24, 1]) if kind == "li" else rng.choice([8, 16, 15, 32])
+    G = H * rng.randint(1, 2)
+    D = G * dg
+    if D % 8 or D % H:
+        D, G = D * 8, G * 8
+    mode = rng.choice(["plain", "interleave", "head"])
+    il, hd = mode == "interleave", (D // H if mode == "head" else None)
+    override(mr_nseg=rng.randint(1, 3), mr_nt=rng.randint(0, 1), se_nt=rng.randint(0, 1), li_nt=rng.randint(0, 1))
+    g = torch.Generator().manual_seed(seed)
+    u = torch.randn(B, L, 3 * D, generator=g).to(torch.bfloat16)
+    w = (torch.randn(3 * D, 3, generator=g) / 3 ** 0.5).to(torch.bfloat16).float()
+    ud, wd = u.cuda(), w.cuda()
+    z = ops.featurizer_fwd(ud, wd, None, interleave=il)
+    r2, r1, rv = (ops.rows_of_projection(z, D, i, hd) for i in range(3))
+    p = ud.transpose(1, 2).contiguous()
+    (q2, q1, qv), chan = ops.projection_rows(p, D, interleave=il, head_dim=hd)
+    ft = torch.stack([wd[chan[1]], wd[chan[0]], wd[chan[2]]]).contiguous()
+    params = {"short_filter_weight": w.reshape(3 * D, 1, 3), "short_filter_bias": None}
+    if kind == "li":
+        lp, rs = O.make_modal_real(G, 16, seed=seed + 1, pmax=0.999)
+        Dc = torch.randn(D, generator=g).to(torch.bfloat16)
+        plan = ops.ModalPlan(lp.cuda(), rs.cuda())
+        override(li_coop=0)
+        y0, _, s0 = ops.li_fwd_rows(r1, r2, rv, plan, Dc.cuda(), B, D, L, device="cuda", want_state=True)
+        y1, s1 = ops.li_layer_fwd_rows(q1, q2, qv, ft, plan, Dc.cuda(), B, D, L, device="cuda", want_state=True)
+        assert torch.equal(s0, s1), (B, L, D, G, mode)
+        params.update(D=Dc, log_poles=lp.repeat_interleave(dg, 0), residues=rs.repeat_interleave(dg, 0))
+        ref = O.OracleCascade(O.OracleEngine(), params, D, H, D, column_split_hyena=hd is not None, interleave=il)
+    else:
+        K = {"se": rng.randint(2, 8), "mr": 128, "mr_short": rng.choice([9, 33, 100])}[kind]
+        mr = K >= 128
+        h = (torch.randn(G, K, generator=g) / K ** 0.5).to(torch.bfloat16).float()
+        Dc = torch.randn(D, generator=g).to(torch.bfloat16) if mr else None
+        kw = dict(device="cuda", bias=Dc.float().cuda() if mr else None,
+                  bias_mode=HYENA_BIAS_GATED_FP32 if mr else HYENA_BIAS_NONE, taps_reversed=not mr)
+        y0 = ops.fir_fwd_rows(r1, r2, rv, h.cuda(), B, D, L, K, force_mfma=K > 8, **kw)
+        y1 = ops.fir_layer_fwd_rows(q1, q2, qv, ft, h.cuda(), B, D, L, K, **kw)
+        params.update(D=Dc, h=h.reshape(G, 1, K))
+        ref = O.OracleCascade(O.OracleEngine(), params, D, H, G, fir_inner_filter_length=K,
+                              column_split_hyena=hd is not None, interleave=il)
+    assert torch.equal(y0, y1), (kind, B, L, D, G, mode)
+    y_ref, _ = ref.forward(u)
+    assert rel_err(y1.permute(0, 2, 1), y_ref) <= 2e-2, (kind, B, L, D, G, mode)
