@@ -188,9 +188,9 @@ def build_workload(name, device):
         out = torch.empty(B, L, D, dtype=dt, device=device)
         fn = lambda: ops.fir_cl_fwd(x[1], x[0], x[2], h, taps_reversed=True, out=out)
         es = 2 if f16 else 4
-        return fn, dict(workload=f"gated FIR on (b, l, g, dg) tensors, {'float16 (MFMA)' if f16 else 'float32 (direct form)'} "
+        return fn, dict(workload=f"gated FIR on (b, l, g, dg) tensors, {'float16 (MFMA)' if f16 else 'float32 (float32 MFMA)'} "
                                  f"B={B} L={L} D={D} groups={G} K={K}", tokens=B * L, bytes=4 * es * B * D * L,
-                        kernel="fir_cl_kernel" if f16 else "fir_cl_direct_kernel", keep=(x, h, out),
+                        kernel="fir_cl_kernel" if f16 else "fir_cl_f32_mfma_kernel", keep=(x, h, out),
                         **({} if f16 else {"flops": 2.0 * K * B * D * L}))
     if name == "li_layer":
         # a whole Hyena-LI layer from the projection at the config-3 shape: featurizer + split + x1*v in one launch
@@ -621,9 +621,8 @@ def main():
                      "cl_f32"):
             e = run(name, max(3, min(args.steps, 10 if name.startswith("li_layer") else 20)), extra_warmup)
             extra[name] = entry(e)
-            if "flops" in e:    # the float32 direct form is arithmetic-bound on the vector ALUs (the float16 form,
-                                # on the matrix cores, is bound by memory like the bfloat16 one); the published
-                                # float32 peak is the matrix cores'
+            if "flops" in e:    # the float32 form (v_mfma_f32_16x16x4_f32) against the published float32 matrix peak;
+                                # the float16 form is bound by memory like the bfloat16 one
                 tf = e["flops"] / (e["kernel_ms"] * 1e-3) / 1e12
                 extra[name].update(tflops=tf, frac_of_fp32_mfma_peak=tf / 157.3)
         for D in (4096, 8192):

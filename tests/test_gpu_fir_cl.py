@@ -208,6 +208,58 @@ def test_cl_filter_longer_than_128_taps_runs_the_direct_form():
     assert rel_err(y.permute(0, 2, 1), ref) <= 2e-2
 
 
+@pytest.mark.parametrize("gated", [True, False])
+@pytest.mark.parametrize("B,L,D,G,K,rev", [(2, 1024, 64, 4, 128, True), (1, 333, 48, 3, 7, True), (3, 130, 128, 1, 32, False),
+                                           (1, 2000, 80, 5, 100, True), (2, 520, 96, 2, 60, False), (1, 256, 32, 2, 40, True),
+                                           (1, 8, 16, 1, 20, True), (2, 129, 144, 3, 1, True), (1, 700, 4096, 4, 128, True)])
+def test_cl_float32_matrix_core_form(B, L, D, G, K, rev, gated, override):
+    """float32 tensors with 16-channel filter groups run on v_mfma_f32_16x16x4_f32 (hyena_fir_cl_fwd_dtype): against
+    a float64 convolution to float32 rounding (1e-5 of the largest output), against the direct form on the vector
+    ALUs (the same sums in another order), with the y2 / Bx outputs, for every set of skipped row groups
+    (K = 128, 100 | 60 | 40 | 32, 20, 7, 1), ragged lengths and channel counts that leave wavefronts idle."""
+    g = torch.Generator().manual_seed(L + K)
+    x2, x1, v = (torch.randn(B, L, D, generator=g) for _ in range(3))
+    h = torch.randn(G, K, generator=g)
+    kw = dict(taps_reversed=rev, want_y2=True, want_bx=True, bx_from=max(L - 9, 0))
+    a1, a2, av = (x1.to(DEV), x2.to(DEV), v.to(DEV)) if gated else (x1.to(DEV), None, None)
+    res = {}
+    for form in (1, 0):
+        override(cl_f32_mfma=form)
+        res[form] = ops.fir_cl_fwd(a1, a2, av, h.to(DEV), **kw)
+    u = (x1 * v if gated else x1).double().permute(0, 2, 1)
+    taps = (h if rev else h.flip(-1)).double().repeat_interleave(D // G, 0)[:, None]       # [D, 1, K], last tap on the current sample
+    z = torch.nn.functional.conv1d(torch.nn.functional.pad(u, (K - 1, 0)), taps, groups=D).permute(0, 2, 1)
+    y = z * x2.double() if gated else z
+    for form in (1, 0):
+        out, y2, bx = (t.cpu().double() for t in res[form])
+        scale = y.abs().max()
+        assert ((out - y).abs().max() / scale).item() <= 1e-5, form
+        assert ((y2 - z).abs().max() / z.abs().max()).item() <= 1e-5, form
+        assert torch.equal(bx.float(), u.permute(0, 2, 1)[:, max(L - 9, 0):].float()), form
+    assert torch.equal(res[0][2], res[1][2])
+    assert ((res[0][0] - res[1][0]).abs().max() / y.abs().max().to(DEV)).item() <= 2e-6
+
+
+def test_cl_float32_falls_back_to_the_direct_form():
+    # groups of 12 channels, an inner bias, or more than 128 taps: no matrix-core form, same entry point, same answers
+    from vortex_amd._lib import HYENA_BIAS_GATED_FP32
+    g = torch.Generator().manual_seed(2)
+    for (D, G, K, bias) in ((48, 4, 16, False), (64, 4, 16, True), (64, 4, 150, False)):
+        B, L = 2, 300
+        x2, x1, v = (torch.randn(B, L, D, generator=g) for _ in range(3))
+        h = torch.randn(G, K, generator=g)
+        Db = torch.randn(D, generator=g) if bias else None
+        out = ops.fir_cl_fwd(x1.to(DEV), x2.to(DEV), v.to(DEV), h.to(DEV), taps_reversed=True,
+                             bias=Db.to(DEV) if bias else None, bias_mode=HYENA_BIAS_GATED_FP32 if bias else 0)
+        u = (x1 * v).double().permute(0, 2, 1)
+        z = torch.nn.functional.conv1d(torch.nn.functional.pad(u, (K - 1, 0)),
+                                       h.double().repeat_interleave(D // G, 0)[:, None], groups=D)
+        if bias:
+            z = z + Db.double()[None, :, None] * u
+        y = z.permute(0, 2, 1) * x2.double()
+        assert ((out.cpu().double() - y).abs().max() / y.abs().max()).item() <= 1e-5
+
+
 def test_cl_impulse_response_across_steps_and_segments():
     # bf16-exact taps, unit gates: the output is the filter itself wherever an impulse sits, bit for bit
     B, D, L, G, K = 1, 64, 4096, 4, 128

@@ -29,8 +29,8 @@ extern "C" const char* hyena_last_error_string(void) { return g_err; }
 // Launch-shape overrides: process-wide, set explicitly through the C ABI (nothing is read from the environment).
 namespace {
 const char* const kOverrideNames[HYENA_OV_COUNT] = {"mr_nseg", "cl_nseg", "se_nt", "mr_nt", "li_nt", "cl_nt",
-                                                    "li_cpw", "li_coop", "li_xcd", "cl_ns"};
-std::atomic<int64_t> g_override[HYENA_OV_COUNT] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
+                                                    "li_cpw", "li_coop", "li_xcd", "cl_ns", "cl_f32_mfma"};
+std::atomic<int64_t> g_override[HYENA_OV_COUNT] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
 }  // namespace
 
 int64_t hyena_override(int id) { return g_override[id].load(std::memory_order_relaxed); }

@@ -58,7 +58,7 @@ int hyena_check_launch(const char* what);
 
 // launch-shape overrides set through hyena_set_launch_override (api.hip); -1 = the launcher's own choice
 enum { HYENA_OV_MR_NSEG, HYENA_OV_CL_NSEG, HYENA_OV_SE_NT, HYENA_OV_MR_NT, HYENA_OV_LI_NT, HYENA_OV_CL_NT,
-       HYENA_OV_LI_CPW, HYENA_OV_LI_COOP, HYENA_OV_LI_XCD, HYENA_OV_CL_NS, HYENA_OV_COUNT };
+       HYENA_OV_LI_CPW, HYENA_OV_LI_COOP, HYENA_OV_LI_XCD, HYENA_OV_CL_NS, HYENA_OV_CL_F32_MFMA, HYENA_OV_COUNT };
 int64_t hyena_override(int id);
 
 // direct-form channel-last FIR for float16 / float32 tensors (fir_cl_direct.hip); arguments as hyena_fir_cl_fwd_dtype

@@ -3,8 +3,9 @@
 // (vortex/ops/hyena_se/tests/test_fwd.py:25-54: float16 and float32, filters of 4, 32 and 128 taps drawn from N(0, 1)).
 //
 // float32 inputs cannot go through one bf16 or fp16 MFMA term at that grid's tolerance (1e-2 absolute on outputs whose
-// accumulation runs over magnitudes of sqrt(K) ~ 11), so this kernel accumulates in float32 on the vector ALUs with
-// float32 operands: out = x2 * (sum_k h[g][k] * (x1*v)[t-k]), nothing rounded below float32.  float16 tensors take
+// accumulation runs over magnitudes of sqrt(K) ~ 11).  Two float32 forms: the float32 matrix-core kernel at the end of
+// this file (16-channel filter groups, K <= 128, no inner bias), and this direct-form kernel for everything else, which
+// accumulates in float32 on the vector ALUs with float32 operands: out = x2 * (sum_k h[g][k] * (x1*v)[t-k]), nothing rounded below float32.  float16 tensors take
 // the same kernel for shapes the MFMA form does not cover (filter groups that are not multiples of 16 channels,
 // unaligned strides), with the roundings of float16 tensor arithmetic: bx = f16(x1*v), z = f16(conv), out = f16(x2*z).
 //
@@ -201,6 +202,185 @@ int direct_launch(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, con
     return hyena_check_launch(who);
 }
 
+
+// ------------------------------------------------------------------ float32 on the matrix cores
+// The same operator for float32 tensors whose filter groups are multiples of 16 channels (the reference grid's are
+// 1024 .. 4096 wide), K <= 128, no inner bias: v_mfma_f32_16x16x4_f32 with full float32 operands.  A block takes 64
+// channels x 128 outputs; bx = x1*v of the tile and its 128 samples of history sits in LDS as [channel][256 rows]
+// (row r = sample t0 - 128 + r; row stride 260 floats, so the sixteen channels x four row quads of a B operand fall
+// into 64 different banks).  Wavefront w owns channels 16w .. 16w+15 and all eight 16-sample output blocks.  Output
+// block b at lags 0 .. 127 reads rows 16b .. 16b+143, nine groups of 16 rows; group G meets the 16 x 16 Toeplitz
+// block A_G[i][j] = h[128 + i - 16G - j], which does not depend on b, so the 36 A operands (nine groups x four
+// slices of four rows) stay in registers and every 16-row group of the tile is read from LDS once (one 16-byte read
+// per lane: the K index of slice q is rows 4k + q, k = lane / 16) and used by up to eight output blocks: 288 MFMAs
+// and 16 LDS reads per wavefront and tile.  Results leave through LDS again (the wavefront's own history rows, dead
+// by then) so that the gate and the stores run channel-last with 16 bytes per lane.
+constexpr int MRS = 260;       // LDS row stride of one channel (floats)
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float ff4;
+
+// GMIN: row groups below it only meet lags >= K (short filters) and are neither staged nor multiplied
+template <int GMIN>
+__global__ __launch_bounds__(256, 2) void fir_cl_f32_mfma_kernel(ClMapT<float> x1, ClMapT<float> x2, ClMapT<float> v,
+                                                                 const float* __restrict__ h, int K, int reversed,
+                                                                 float* __restrict__ out, float* __restrict__ y2_out,
+                                                                 float* __restrict__ bx_out, int64_t bx_from, int64_t L,
+                                                                 int64_t D, int dg, int ndb, int ntt) {
+    extern __shared__ __attribute__((aligned(16))) float smem[];       // [64][MRS]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t bid = blockIdx.x;
+    const uint32_t db = bid % (uint32_t)ndb;
+    const uint32_t tt = (bid / (uint32_t)ndb) % (uint32_t)ntt;
+    const int64_t b = bid / ((uint32_t)ndb * (uint32_t)ntt);
+    const int64_t d0 = (int64_t)db * DC, t0 = (int64_t)tt * DT;
+    const bool pre = v.ptr != nullptr, post = x2.ptr != nullptr;
+
+    // ---- staging: thread = 4 channels x one row of each pass of 16 rows; four passes of requests in flight
+    const int c4 = tid & 15, rr = tid >> 4;
+    const int64_t dq = d0 + 4 * c4;
+    const bool q_ok = dq < D;                                  // D is a multiple of 4: a quad exists whole or not at all
+    const int64_t dql = q_ok ? dq : 0;
+    const ff4 zero = {0.f, 0.f, 0.f, 0.f};
+    constexpr int NB = 16;                                     // passes of 16 rows requested together: the whole tile in one round trip
+#pragma unroll
+    for (int p0 = GMIN; p0 < 16; p0 += NB) {
+        ff4 xa[NB], va[NB];
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            if (p0 + i >= 16) continue;
+            int64_t t = t0 - 128 + 16 * (p0 + i) + rr;
+            t = t < 0 ? 0 : (t < L ? t : L - 1);
+            xa[i] = *(const ff4*)(x1.ptr + b * x1.bs + t * x1.ts + dql);
+            if (pre) va[i] = *(const ff4*)(v.ptr + b * v.bs + t * v.ts + dql);
+        }
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            if (p0 + i >= 16) continue;
+            const int r = 16 * (p0 + i) + rr;
+            const int64_t t = t0 - 128 + r;
+            ff4 val = xa[i];
+            if (pre) val = val * va[i];
+            if (!(q_ok && t >= 0 && t < L)) val = zero;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) smem[(4 * c4 + e) * MRS + r] = val[e];
+            if (bx_out && q_ok && r >= 128 && t < L && t >= bx_from)
+                *(ff4*)(bx_out + (b * (L - bx_from) + (t - bx_from)) * D + dq) = val;
+        }
+    }
+    // the output gate of this thread's eight (row, quad) pieces: requested now, used at the end
+    ff4 gate[8];
+    if (post) {
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            int64_t t = t0 + 16 * p + rr;
+            t = t < L ? t : L - 1;
+            gate[p] = *(const ff4*)(x2.ptr + b * x2.bs + t * x2.ts + dql);
+        }
+    }
+
+    // ---- Toeplitz operands of this wavefront's filter group
+    const int n = lane & 15, k = lane >> 4;
+    const int64_t dw = d0 + 16 * w;
+    const bool w_ok = dw < D;                                  // wave-uniform
+    const int g = (int)((uint32_t)(w_ok ? dw : 0) / (uint32_t)dg);
+    float A[9][4];
+#pragma unroll
+    for (int G = 0; G < 9; ++G)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int lag = 128 + n - 16 * G - 4 * k - q;       // output row i = n of the block, input row 16G + 4k + q
+            const int lc = lag < 0 ? 0 : (lag < K ? lag : K - 1);
+            const float hv = h[(int64_t)g * K + (reversed ? K - 1 - lc : lc)];
+            A[G][q] = (lag >= 0 && lag < K) ? hv : 0.f;
+        }
+    __syncthreads();
+
+    ff4 acc[8];
+#pragma unroll
+    for (int bb = 0; bb < 8; ++bb) acc[bb] = zero;
+    float* const mine = smem + (16 * w + n) * MRS;
+    if (w_ok) {
+#pragma unroll
+        for (int J = GMIN; J < 16; ++J) {
+            const ff4 Bq = *(const ff4*)(mine + 16 * J + 4 * k);
+#pragma unroll
+            for (int bb = 0; bb < 8; ++bb) {
+                const int G = J - bb;
+                if (G < GMIN || G > 8) continue;
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    acc[bb] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[G][q], Bq[q], acc[bb], 0, 0, 0);
+            }
+        }
+        // lane (n, k) holds outputs 16bb + 4k .. + 3 of channel 16w + n: into this channel's history rows, which no
+        // other wavefront reads (an LDS read and write of one wavefront complete in order)
+#pragma unroll
+        for (int bb = 0; bb < 8; ++bb) *(ff4*)(mine + 16 * bb + 4 * k) = acc[bb];
+    }
+    __syncthreads();
+
+    // ---- channel-last output: the staging layout again (4 channels x one row of each pass)
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+        const int tl = 16 * p + rr;
+        const int64_t t = t0 + tl;
+        ff4 z;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) z[e] = smem[(4 * c4 + e) * MRS + tl];
+        if (q_ok && t < L) {
+            const int64_t o = (b * L + t) * D + dq;
+            if (y2_out) *(ff4*)(y2_out + o) = z;
+            if (post) z = z * gate[p];
+            *(ff4*)(out + o) = z;
+        }
+    }
+}
+
+int f32_mfma_launch(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, const float* h, int taps_reversed,
+                    void* out, void* y2_out, void* bx_out, int64_t bx_from, int64_t B, int64_t L, int64_t D, int64_t G,
+                    int K, void* stream, const char* who) {
+    const int64_t ndb = (D + DC - 1) / DC, ntt = (L + DT - 1) / DT;
+    if (B * ndb * ntt > 0x7fffffffLL) return hyena_fail(HYENA_EINVAL, "%s: problem too large for one launch", who);
+    ClMapT<float> m1 = {(const float*)x1->ptr, x1->batch_stride, x1->time_stride};
+    ClMapT<float> m2 = {nullptr, 0, 0}, mv = {nullptr, 0, 0};
+    if (x2 && x2->ptr) m2 = {(const float*)x2->ptr, x2->batch_stride, x2->time_stride};
+    if (v && v->ptr) mv = {(const float*)v->ptr, v->batch_stride, v->time_stride};
+    const size_t lds = (size_t)DC * MRS * sizeof(float);
+    static bool big[64] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+    if (dev < 0 || !big[dev]) {
+        const void* fns[4] = {(const void*)fir_cl_f32_mfma_kernel<0>, (const void*)fir_cl_f32_mfma_kernel<3>,
+                              (const void*)fir_cl_f32_mfma_kernel<5>, (const void*)fir_cl_f32_mfma_kernel<6>};
+        for (const void* f : fns) {
+            const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return hyena_fail((int)e, "%s: hipFuncSetAttribute: %s", who, hipGetErrorString(e));
+        }
+        if (dev >= 0) big[dev] = true;
+    }
+    // row group G meets lags 113 - 16G .. 143 - 16G: groups with 113 - 16G >= K hold no tap
+    const int gz = K <= 113 ? (113 - K) / 16 + 1 : 0;           // all-zero groups ahead of the first live one
+    const dim3 grid((unsigned)(B * ndb * ntt));
+#define F32_GO(GM)                                                                                                  \
+    hipLaunchKernelGGL(fir_cl_f32_mfma_kernel<GM>, grid, dim3(256), lds, (hipStream_t)stream, m1, m2, mv, h, K,       \
+                       taps_reversed, (float*)out, (float*)y2_out, (float*)bx_out, bx_from, L, D, (int)(D / G), (int)ndb, \
+                       (int)ntt)
+    if (gz >= 6) F32_GO(6); else if (gz >= 5) F32_GO(5); else if (gz >= 3) F32_GO(3); else F32_GO(0);
+#undef F32_GO
+    return hyena_check_launch(who);
+}
+
+// whether the matrix-core form takes a float32 launch: 16-channel filter groups, at most 128 taps, no inner bias, and
+// 16-byte pieces of four channels everywhere
+bool f32_mfma_ok(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, int bias_mode, const void* out,
+                 const void* y2_out, const void* bx_out, int64_t D, int64_t G, int K) {
+    auto cl4 = [](const hyena_cl* c) {
+        return !c || !c->ptr || ((((uintptr_t)c->ptr) & 15) == 0 && c->batch_stride % 4 == 0 && c->time_stride % 4 == 0);
+    };
+    return K >= 1 && K <= 128 && (D / G) % 16 == 0 && bias_mode == HYENA_BIAS_NONE && cl4(x1) && cl4(x2) && cl4(v) &&
+           !((((uintptr_t)out) | ((uintptr_t)y2_out) | ((uintptr_t)bx_out)) & 15);
+}
+
 }  // namespace
 
 // Direct-form launch for channel-last tensors of any of the three element types, any K >= 1; arguments as
@@ -208,6 +388,9 @@ int direct_launch(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, con
 int hyena_fir_cl_direct(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, const float* h, int taps_reversed,
                         const float* bias, int bias_mode, void* out, void* y2_out, void* bx_out, int64_t bx_from,
                         int64_t B, int64_t L, int64_t D, int64_t G, int K, int dtype, void* stream, const char* who) {
+    if (dtype == HYENA_DTYPE_F32 && hyena_override(HYENA_OV_CL_F32_MFMA) != 0 &&
+        f32_mfma_ok(x1, x2, v, bias_mode, out, y2_out, bx_out, D, G, K))
+        return f32_mfma_launch(x1, x2, v, h, taps_reversed, out, y2_out, bx_out, bx_from, B, L, D, G, K, stream, who);
     if (dtype == HYENA_DTYPE_F32)
         return direct_launch<float>(x1, x2, v, h, taps_reversed, bias, bias_mode, out, y2_out, bx_out, bx_from, B, L, D,
                                     G, K, stream, who);
