@@ -190,7 +190,7 @@ def build_workload(name, device):
         es = 2 if f16 else 4
         return fn, dict(workload=f"gated FIR on (b, l, g, dg) tensors, {'float16 (MFMA)' if f16 else 'float32 (float32 MFMA)'} "
                                  f"B={B} L={L} D={D} groups={G} K={K}", tokens=B * L, bytes=4 * es * B * D * L,
-                        kernel="fir_cl_kernel" if f16 else "fir_cl_f32_mfma_kernel", keep=(x, h, out),
+                        kernel="fir_cl_kernel" if f16 else "fir_cl_f32_ring_kernel", keep=(x, h, out),
                         **({} if f16 else {"flops": 2.0 * K * B * D * L}))
     if name == "li_layer":
         # a whole Hyena-LI layer from the projection at the config-3 shape: featurizer + split + x1*v in one launch

@@ -66,7 +66,9 @@ const char* hyena_last_error_string(void);
  *   "li_coop"                                   0 / 1 = lone / cooperating wavefronts in hyena_li_fwd
  *   "cl_ns"                                     1 = one 64-channel strip per block in hyena_fir_cl_fwd / layer_fwd, 2 or
  *                                               more = the form with several strips per block wherever it exists
- *   "cl_f32_mfma"                               0 = float32 tensors always take the direct form in hyena_fir_cl_fwd_dtype
+ *   "cl_f32_mfma"                               float32 tensors in hyena_fir_cl_fwd_dtype: 0 = always the direct form,
+ *                                               1 / 2 = the matrix-core form with one tile per block / blocks that walk
+ *                                               a ring of tiles, wherever the matrix-core form applies
  * Returns 0, or HYENA_EINVAL for an unknown name. */
 int hyena_set_launch_override(const char* name, int64_t value);
 

@@ -211,7 +211,8 @@ def test_cl_filter_longer_than_128_taps_runs_the_direct_form():
 @pytest.mark.parametrize("gated", [True, False])
 @pytest.mark.parametrize("B,L,D,G,K,rev", [(2, 1024, 64, 4, 128, True), (1, 333, 48, 3, 7, True), (3, 130, 128, 1, 32, False),
                                            (1, 2000, 80, 5, 100, True), (2, 520, 96, 2, 60, False), (1, 256, 32, 2, 40, True),
-                                           (1, 8, 16, 1, 20, True), (2, 129, 144, 3, 1, True), (1, 700, 4096, 4, 128, True)])
+                                           (1, 8, 16, 1, 20, True), (2, 129, 144, 3, 1, True), (1, 700, 4096, 4, 128, True),
+                                           (2, 2048 + 40, 64, 2, 128, False)])
 def test_cl_float32_matrix_core_form(B, L, D, G, K, rev, gated, override):
     """float32 tensors with 16-channel filter groups run on v_mfma_f32_16x16x4_f32 (hyena_fir_cl_fwd_dtype): against
     a float64 convolution to float32 rounding (1e-5 of the largest output), against the direct form on the vector
@@ -223,13 +224,15 @@ def test_cl_float32_matrix_core_form(B, L, D, G, K, rev, gated, override):
     kw = dict(taps_reversed=rev, want_y2=True, want_bx=True, bx_from=max(L - 9, 0))
     a1, a2, av = (x1.to(DEV), x2.to(DEV), v.to(DEV)) if gated else (x1.to(DEV), None, None)
     res = {}
-    for form in (1, 0):
+    for form in (2, 1, 0):          # blocks that walk a ring of tiles, one tile per block, the direct form
         override(cl_f32_mfma=form)
         res[form] = ops.fir_cl_fwd(a1, a2, av, h.to(DEV), **kw)
     u = (x1 * v if gated else x1).double().permute(0, 2, 1)
     taps = (h if rev else h.flip(-1)).double().repeat_interleave(D // G, 0)[:, None]       # [D, 1, K], last tap on the current sample
     z = torch.nn.functional.conv1d(torch.nn.functional.pad(u, (K - 1, 0)), taps, groups=D).permute(0, 2, 1)
     y = z * x2.double() if gated else z
+    for i in range(3):
+        assert torch.equal(res[2][i], res[1][i])          # the two matrix-core forms: the same sums in the same order
     for form in (1, 0):
         out, y2, bx = (t.cpu().double() for t in res[form])
         scale = y.abs().max()

@@ -336,6 +336,161 @@ __global__ __launch_bounds__(256, 2) void fir_cl_f32_mfma_kernel(ClMapT<float> x
     }
 }
 
+
+// The same arithmetic as fir_cl_f32_mfma_kernel for launches with many tiles along L: a block walks `seg_tiles`
+// consecutive 128-output tiles of its 64 channels.  The two 128-row halves of the LDS tile form a ring -- the half
+// staged for one tile is the next tile's history, and the half that held the history takes the results on their way
+// out and then the next tile's rows -- so every sample is staged once (plus 128 samples at the start of a segment),
+// and the next tile's rows are requested ahead of the MFMAs of this one and travel during them.
+template <int GMIN>
+__global__ __launch_bounds__(256, 2) void fir_cl_f32_ring_kernel(ClMapT<float> x1, ClMapT<float> x2, ClMapT<float> v,
+                                                                 const float* __restrict__ h, int K, int reversed,
+                                                                 float* __restrict__ out, float* __restrict__ y2_out,
+                                                                 float* __restrict__ bx_out, int64_t bx_from, int64_t L,
+                                                                 int64_t D, int dg, int ndb, int ntt, int nseg,
+                                                                 int seg_tiles) {
+    extern __shared__ __attribute__((aligned(16))) float smem[];       // [64][MRS]: rows 0..127 and 128..255 are the ring's halves
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t bid = blockIdx.x;
+    const uint32_t db = bid % (uint32_t)ndb;
+    const uint32_t seg = (bid / (uint32_t)ndb) % (uint32_t)nseg;
+    const int64_t b = bid / ((uint32_t)ndb * (uint32_t)nseg);
+    const int i0 = (int)seg * seg_tiles;
+    const int i1 = i0 + seg_tiles < ntt ? i0 + seg_tiles : ntt;
+    if (i0 >= i1) return;                                      // the whole block leaves: no barrier is skipped
+    const int64_t d0 = (int64_t)db * DC;
+    const bool pre = v.ptr != nullptr, post = x2.ptr != nullptr;
+    const int c4 = tid & 15, rr = tid >> 4;
+    const int64_t dq = d0 + 4 * c4;
+    const bool q_ok = dq < D;
+    const int64_t dql = q_ok ? dq : 0;
+    const ff4 zero = {0.f, 0.f, 0.f, 0.f};
+    const float* const px1 = x1.ptr + b * x1.bs + dql;
+    const float* const pxv = pre ? v.ptr + b * v.bs + dql : nullptr;
+    const float* const px2 = post ? x2.ptr + b * x2.bs + dql : nullptr;
+
+    const int n = lane & 15, k = lane >> 4;
+    const int64_t dw = d0 + 16 * w;
+    const bool w_ok = dw < D;
+    const int g = (int)((uint32_t)(w_ok ? dw : 0) / (uint32_t)dg);
+    float A[9][4];
+#pragma unroll
+    for (int G = 0; G < 9; ++G)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int lag = 128 + n - 16 * G - 4 * k - q;
+            const int lc = lag < 0 ? 0 : (lag < K ? lag : K - 1);
+            const float hv = h[(int64_t)g * K + (reversed ? K - 1 - lc : lc)];
+            A[G][q] = (lag >= 0 && lag < K) ? hv : 0.f;
+        }
+
+    // eight passes of 16 rows: the 128 samples that start at ts
+    ff4 xa[8], va[8];
+    auto request = [&](const int64_t ts) __attribute__((always_inline)) {
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            int64_t t = ts + 16 * p + rr;
+            t = t < 0 ? 0 : (t < L ? t : L - 1);
+            xa[p] = *(const ff4*)(px1 + t * x1.ts);
+            if (pre) va[p] = *(const ff4*)(pxv + t * v.ts);
+        }
+    };
+    auto stage = [&](const int64_t ts, const int half, const bool store_bx, const int p_first) __attribute__((always_inline)) {
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            if (p < p_first) continue;
+            const int r = 128 * half + 16 * p + rr;
+            const int64_t t = ts + 16 * p + rr;
+            ff4 val = xa[p];
+            if (pre) val = val * va[p];
+            if (!(q_ok && t >= 0 && t < L)) val = zero;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) smem[(4 * c4 + e) * MRS + r] = val[e];
+            if (store_bx && bx_out && q_ok && t < L && t >= bx_from)
+                *(ff4*)(bx_out + (b * (L - bx_from) + (t - bx_from)) * D + dq) = val;
+        }
+    };
+    // history of the segment's first tile -> the half that tile does not stage (row groups below GMIN meet no tap)
+    request((int64_t)i0 * DT - 128);
+    stage((int64_t)i0 * DT - 128, 1, false, GMIN);
+    request((int64_t)i0 * DT);
+
+    float* const mine = smem + (16 * w + n) * MRS;
+    for (int i = i0; i < i1; ++i) {
+        const int64_t t0 = (int64_t)i * DT;
+        const int c = (i - i0) & 1;                            // the half this tile's rows go to; its history is in the other
+        stage(t0, c, true, 0);
+        __syncthreads();
+        ff4 gate[8];
+        if (post) {
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+                int64_t t = t0 + 16 * p + rr;
+                t = t < L ? t : L - 1;
+                gate[p] = *(const ff4*)(px2 + t * x2.ts);
+            }
+        }
+        if (i + 1 < i1) request(t0 + DT);                      // travels during the MFMAs below
+
+        ff4 acc[8];
+#pragma unroll
+        for (int bb = 0; bb < 8; ++bb) acc[bb] = zero;
+        float* const hist = mine + 128 * (c ^ 1);
+        float* const cur = mine + 128 * c;
+        if (w_ok) {
+#pragma unroll
+            for (int J = GMIN; J < 16; ++J) {
+                const ff4 Bq = *(const ff4*)((J < 8 ? hist : cur) + 16 * (J & 7) + 4 * k);
+#pragma unroll
+                for (int bb = 0; bb < 8; ++bb) {
+                    const int G = J - bb;
+                    if (G < GMIN || G > 8) continue;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        acc[bb] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[G][q], Bq[q], acc[bb], 0, 0, 0);
+                }
+            }
+            // results into the history half, which is dead now (only this wavefront reads its channels' rows)
+#pragma unroll
+            for (int bb = 0; bb < 8; ++bb) *(ff4*)(hist + 16 * bb + 4 * k) = acc[bb];
+        }
+        __syncthreads();
+        const int zb = 128 * (c ^ 1);
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            const int tl = 16 * p + rr;
+            const int64_t t = t0 + tl;
+            ff4 z;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) z[e] = smem[(4 * c4 + e) * MRS + zb + tl];
+            if (q_ok && t < L) {
+                const int64_t o = (b * L + t) * D + dq;
+                if (y2_out) *(ff4*)(y2_out + o) = z;
+                if (post) z = z * gate[p];
+                *(ff4*)(out + o) = z;
+            }
+        }
+        __syncthreads();                                       // the next tile stages its rows over these results
+    }
+}
+
+// dynamic LDS beyond the default for the ring kernels, once per device
+int big_ring_ready(const char* who) {
+    static bool big[64] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+    if (dev >= 0 && big[dev]) return 0;
+    const void* fns[4] = {(const void*)fir_cl_f32_ring_kernel<0>, (const void*)fir_cl_f32_ring_kernel<3>,
+                          (const void*)fir_cl_f32_ring_kernel<5>, (const void*)fir_cl_f32_ring_kernel<6>};
+    for (const void* f : fns) {
+        const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(DC * MRS * sizeof(float)));
+        if (e != hipSuccess) return hyena_fail((int)e, "%s: hipFuncSetAttribute: %s", who, hipGetErrorString(e));
+    }
+    if (dev >= 0) big[dev] = true;
+    return 0;
+}
+
 int f32_mfma_launch(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, const float* h, int taps_reversed,
                     void* out, void* y2_out, void* bx_out, int64_t bx_from, int64_t B, int64_t L, int64_t D, int64_t G,
                     int K, void* stream, const char* who) {
@@ -360,6 +515,29 @@ int f32_mfma_launch(const hyena_cl* x1, const hyena_cl* x2, const hyena_cl* v, c
     }
     // row group G meets lags 113 - 16G .. 143 - 16G: groups with 113 - 16G >= K hold no tap
     const int gz = K <= 113 ? (113 - K) / 16 + 1 : 0;           // all-zero groups ahead of the first live one
+    // many tiles along L: blocks that walk a segment of them (about two blocks per CU, at least four tiles each)
+    {
+        const int64_t rows = B * ndb;
+        int64_t nseg = (512 + rows - 1) / rows;
+        nseg = nseg < 1 ? 1 : (nseg > ntt ? ntt : nseg);
+        int64_t seg_tiles = (ntt + nseg - 1) / nseg;
+        if (seg_tiles < 4) seg_tiles = ntt < 4 ? ntt : 4;
+        nseg = (ntt + seg_tiles - 1) / seg_tiles;
+        const int64_t x = hyena_override(HYENA_OV_CL_F32_MFMA);
+        // (short filters skip most of the history in the one-tile form, which then measured 5 % faster: 219 against 231 us
+        // at B = 2, L = 8192, D = 4096, K = 4; at K = 128 the ring takes 267 against 315 us)
+        if ((x == 2 || (x < 0 && seg_tiles >= 4 && gz < 5)) && x != 1) {
+            if (int rc = big_ring_ready(who)) return rc;
+            const dim3 rgrid((unsigned)(rows * nseg));
+#define F32_RING(GM)                                                                                                \
+    hipLaunchKernelGGL(fir_cl_f32_ring_kernel<GM>, rgrid, dim3(256), lds, (hipStream_t)stream, m1, m2, mv, h, K,     \
+                       taps_reversed, (float*)out, (float*)y2_out, (float*)bx_out, bx_from, L, D, (int)(D / G), (int)ndb, \
+                       (int)ntt, (int)nseg, (int)seg_tiles)
+            if (gz >= 6) F32_RING(6); else if (gz >= 5) F32_RING(5); else if (gz >= 3) F32_RING(3); else F32_RING(0);
+#undef F32_RING
+            return hyena_check_launch(who);
+        }
+    }
     const dim3 grid((unsigned)(B * ndb * ntt));
 #define F32_GO(GM)                                                                                                  \
     hipLaunchKernelGGL(fir_cl_f32_mfma_kernel<GM>, grid, dim3(256), lds, (hipStream_t)stream, m1, m2, mv, h, K,       \
