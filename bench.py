@@ -271,7 +271,7 @@ def decode_layer_set(D, device, steps, warmup):
     """One [SE, MR, LI] layer set of cached decode at batch 64: three fused launches per token.
 
     Timed twice: with the kernels that run the reference's algorithm (the whole FIR cache read and the modal state
-    read and written on every token; SURVEY's algorithmic bytes are exactly what these move, so their rate is a
+    read and written on every token; the algorithmic bytes of that algorithm are exactly what these move, so their rate is a
     bandwidth and `frac_reference_algorithm` is the roofline figure), and with the steps the steppers bind by default
     (far sums for the deep cache, the modal state in windows of four tokens), which move fewer bytes per token: for
     those the headline is `us_per_step`, and the fraction is taken of the bytes they move."""
