@@ -350,9 +350,7 @@ class HyenaCascade(nn.Module):
         """Whether hyena_featurizer_gates_fwd covers this layer: a Hyena-LI layer (modal filter, no truncated-FIR
         branch) with a 3- or 4-tap featurizer, a closed channel map and an aligned projection."""
         D, hd = self.hidden_size, self.hidden_size_per_attention_head
-        if self.fir_inner_filter_length or self.long_fir_threshold is not None:
-            return False
-        if self.short_filter_length not in (3, 4) or self._channel_map() is None:
+        if not self._can_fuse_gates_layer() or self.short_filter_length not in (3, 4):
             return False
         if D % 8 or (self.column_split_hyena and hd % 8):
             return False
@@ -422,6 +420,7 @@ class HyenaCascade(nn.Module):
         return y.permute(0, 2, 1)
 
     def _can_fuse_gates_layer(self):
+        """A Hyena-LI layer (modal filter, no truncated-FIR branch) with a closed channel map."""
         if self.fir_inner_filter_length or self.long_fir_threshold is not None:
             return False
         return self._channel_map() is not None
