@@ -88,7 +88,7 @@ def project_sequence_major(weight, x):
 
 
 class SequenceMajorProjection(nn.Module):
-    """Stands in for the `projections` linear layer of a Hyena block (vortex/model/model.py:490-492 calls it on the
+    """Stands in for the `projections` linear layer of a Hyena block (vortex/model/model.py:487-490 calls it on the
     normalised input): the same projection, stored sequence-major for prefills, so that a Hyena-LI cascade behind it
     runs featurizer, gates and scan in one launch.  Decode tokens, prompts that are not a whole number of 8-sample
     pieces, biased layers and anything that is not a plain linear layer on the GPU go through the wrapped layer
