@@ -362,7 +362,7 @@ __global__ __launch_bounds__(256 * NS, NS == 1 ? 2 : 1) void fir_cl_kernel(ClMap
         } else {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                if (PRE) {
+                if constexpr (PRE) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
                         bx[q][j] = ET::pack2(ET::lo(raw[0][q][j]) * ET::lo(raw[1][q][j]),
@@ -370,7 +370,7 @@ __global__ __launch_bounds__(256 * NS, NS == 1 ? 2 : 1) void fir_cl_kernel(ClMap
                 } else {
                     bx[q] = raw[0][q];
                 }
-                if (POST) g2[q] = raw[NP - 1][q];
+                if constexpr (POST) g2[q] = raw[NP - 1][q];
             }
         }
         // ---- (b) next step's rows (NEARLY pieces of them) are requested now and arrive during the MFMA phase
