@@ -3,8 +3,9 @@ of vortex/model/model.py:233-246 (vortex/model/engine.py:188-223), the split of 
 vortex/model/utils.py:26-85, and parallel_iir with its state (engine.py:283-353, :525-559).
 
 Two statements: (1) bit for bit the result of the featurizer kernel followed by hyena_li_fwd on its gates (the same
-products in the same order, in the lone-wavefront work decomposition this entry point runs), on small and ragged
-shapes and at the full long-convolution shape; (2) against the oracle's featurizer + gates + FFT convolution
+products in the same order when both run the same work decomposition: lone wavefronts of one or of four channels;
+across the two decompositions the scan adds in a different order and the results agree to rounding), on small and
+ragged shapes and at the full long-convolution shape; (2) against the oracle's featurizer + gates + FFT convolution
 (oracle.hyena_oracle, float32) within the tolerances of hyena_li_fwd: bf16 outputs 2e-2, state 1e-4."""
 import pytest
 import torch
@@ -54,11 +55,17 @@ def test_li_layer_equals_featurizer_then_scan(mode, B, L, D, G):
     u, w, lp, rs, Dc = _case(B, L, D, G, seed=L + D + G)
     u, w, Dc = u.to(DEV), w.to(DEV), Dc.to(DEV)
     plan = ops.ModalPlan(lp.to(DEV), rs.to(DEV))
-    y0, s0 = _two_launches(u, w, plan, Dc, D, il, hd)
-    y1, s1 = _one_pass(u, w, plan, Dc, D, il, hd)
-    assert torch.equal(y0, y1)
-    assert torch.equal(s0, s1)
-    assert bool(torch.isfinite(y1.float()).all())
+    for cpw in ((1, 4) if (D // G) % 4 == 0 else (1,)):
+        with _lib.launch_override(li_cpw=cpw):
+            y0, s0 = _two_launches(u, w, plan, Dc, D, il, hd)
+            y1, s1 = _one_pass(u, w, plan, Dc, D, il, hd)
+        assert torch.equal(y0, y1), cpw
+        assert torch.equal(s0, s1), cpw
+        assert bool(torch.isfinite(y1.float()).all())
+    # whatever decomposition the library picks by itself for this shape: the same result up to the order of the scan
+    y2, s2 = _one_pass(u, w, plan, Dc, D, il, hd)
+    assert ((y2.float() - y1.float()).abs().max() / y1.float().abs().max()).item() <= 1e-2
+    assert ((s2 - s1).abs().max() / s1.abs().max().clamp_min(1e-30)).item() <= 1e-5
 
 
 @pytest.mark.parametrize("cpw", [1, 4])
@@ -69,10 +76,16 @@ def test_li_layer_forms(cpw, nt):
     u, w, lp, rs, Dc = _case(B, L, D, G, seed=5, cplx=True)
     u, w, Dc = u.to(DEV), w.to(DEV), Dc.to(DEV)
     plan = ops.ModalPlan(lp.to(DEV), rs.to(DEV))
-    y0, s0 = _two_launches(u, w, plan, Dc, D, True, None)
+    with _lib.launch_override(li_cpw=cpw):
+        y0, s0 = _two_launches(u, w, plan, Dc, D, True, None)
     with _lib.launch_override(li_cpw=cpw, li_nt=nt):
         y1, s1 = _one_pass(u, w, plan, Dc, D, True, None)
     assert torch.equal(y0, y1) and torch.equal(torch.view_as_real(s0), torch.view_as_real(s1))
+    # the other decomposition adds the scan's terms in another order: the same result to rounding
+    with _lib.launch_override(li_cpw=5 - cpw):
+        y2, s2 = _one_pass(u, w, plan, Dc, D, True, None)
+    assert ((y2.float() - y1.float()).abs().max() / y1.float().abs().max()).item() <= 1e-2
+    assert ((s2 - s1).abs().max() / s1.abs().max()).item() <= 1e-5
 
 
 @pytest.mark.parametrize("cplx", [False, True])
@@ -140,7 +153,8 @@ def test_li_layer_full_size(G):
     lp, rs = O.make_modal_complex(G, 16, seed=G, pmax=0.9999)
     Dc = torch.randn(D, generator=g, device=DEV).to(torch.bfloat16)
     plan = ops.ModalPlan(lp.to(DEV), rs.to(DEV))
-    y0, s0 = _two_launches(u, w, plan, Dc, D, True, None)
+    with _lib.launch_override(li_cpw=1):       # what the one-pass form picks for rows this long; pinned for the scan alone
+        y0, s0 = _two_launches(u, w, plan, Dc, D, True, None)
     y1, s1 = _one_pass(u, w, plan, Dc, D, True, None)
     assert torch.equal(y0, y1)
     assert torch.equal(torch.view_as_real(s0), torch.view_as_real(s1))

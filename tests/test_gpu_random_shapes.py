@@ -358,7 +358,8 @@ def test_rows_layers_random(B, L, seed, override):
         lp, rs = O.make_modal_real(G, 16, seed=seed + 1, pmax=0.999)
         Dc = torch.randn(D, generator=g).to(torch.bfloat16)
         plan = ops.ModalPlan(lp.cuda(), rs.cuda())
-        override(li_coop=0)
+        # lone wavefronts and the same channels per wavefront on both sides: the scan's additions then come in the same order
+        override(li_coop=0, li_cpw=rng.choice([1, 4]) if dg % 4 == 0 else 1)
         y0, _, s0 = ops.li_fwd_rows(r1, r2, rv, plan, Dc.cuda(), B, D, L, device="cuda", want_state=True)
         y1, s1 = ops.li_layer_fwd_rows(q1, q2, qv, ft, plan, Dc.cuda(), B, D, L, device="cuda", want_state=True)
         assert torch.equal(s0, s1), (B, L, D, G, mode)

@@ -141,12 +141,15 @@ int main(int argc, char** argv) {
         HIP_OK(hipMalloc(&d_st0, B * D * S * 2 * 4)); HIP_OK(hipMalloc(&d_st1, B * D * S * 2 * 4));
         rc = p_hyena_li_plan(d_lp, d_rs, G, S, d_ws, stream);
         CHECK(rc == 0, "hyena_li_plan rc=%d: %s", rc, p_hyena_last_error_string());
+        // (the same work decomposition on both sides: the order of the scan's additions depends on it)
         CHECK(p_hyena_set_launch_override("li_coop", 0) == 0, "li_coop override");
+        CHECK(p_hyena_set_launch_override("li_cpw", 4) == 0, "li_cpw override");
         rc = p_hyena_li_fwd(&q1, &q2, &qv, d_ws, nullptr, 1, d_out, nullptr, d_st0, B, D, L, G, S, stream);
         CHECK(rc == 0, "hyena_li_fwd rc=%d: %s", rc, p_hyena_last_error_string());
-        CHECK(p_hyena_set_launch_override("li_coop", -1) == 0, "li_coop override reset");
         rc = p_hyena_li_layer_fwd(&q1, &q2, &qv, d_id, 3, d_ws, nullptr, 1, d_out2, d_st1, B, D, L, G, S, stream);
         CHECK(rc == 0, "hyena_li_layer_fwd rc=%d: %s", rc, p_hyena_last_error_string());
+        CHECK(p_hyena_set_launch_override("li_coop", -1) == 0, "li_coop override reset");
+        CHECK(p_hyena_set_launch_override("li_cpw", -1) == 0, "li_cpw override reset");
         HIP_OK(hipStreamSynchronize(stream));
         auto oa = host(d_out, (size_t)(B * D * L)); auto ob = host(d_out2, (size_t)(B * D * L));
         CHECK(oa == ob, "hyena_li_layer_fwd with identity featurizer taps differs from hyena_li_fwd");

@@ -18,11 +18,14 @@
 // sequence alone.  With CPW = 4 a step is 512 samples (4 chunks) and the 16 MFMA columns are
 // 4 channels x 4 chunks; the 64 lanes hold the 4 x 16 complex states of the scan, one each.
 // With CPW = 1 (filter groups narrower than 4 channels, e.g. one filter per channel) a step is
-// 2048 samples of one channel and the 16 columns are its 16 chunks.  Either way one B fragment
+// 2048 samples of one channel and the 16 columns are its 16 chunks; each of the four lane rows
+// scans one 512-sample piece from a zero state and the pieces are joined with two lane-row swaps
+// (v_permlane16_swap, v_permlane32_swap).  Either way one B fragment
 // serves every column of the step.  Nothing is shared between wavefronts: there is no
 // block barrier anywhere, only the in-order LDS pipe of the wavefront itself, and the four
 // wavefronts of a CU drift apart and cover each other's memory latency.  Global traffic is
-// coalesced 16 B per lane (1 KiB per row and instruction), prefetched PF steps ahead in registers.
+// coalesced 16 B per lane (1 KiB per row and instruction), prefetched PF steps ahead in registers,
+// and goes through buffer descriptors whose range check stands in for every bounds test.
 #include <mutex>
 #include <type_traits>
 
@@ -191,6 +194,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     static_assert(FEAT == 0 || (FEAT == 3 && PRE && POST && !COOP && !Y32), "featurizer: three taps, all three gates, lone wavefronts");
     constexpr int TLW = TL * (4 / CPW);                        // samples of one channel per step and wavefront
     constexpr int STEP = COOP ? 4 * TLW : TLW;                 // distance between two steps of one wavefront
+    constexpr int NROW = CPW == 4 ? 4 : 1;                     // distinct rows per stream
     __shared__ __attribute__((aligned(16))) unsigned char lds_all[4 * WAVE_LDS_BYTES];
     __shared__ float2 e_sh[COOP ? 2 * 4 * 64 : 1];             // [step parity][wavefront][lane] piece end states
     const int tid = threadIdx.x, lane = tid & 63;
@@ -240,25 +244,43 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
 
     // ---- coalesced layout: lane moves samples 8*lane..8*lane+7 of each of the 4 rows
     const int lofs = lane * 8 + 32 * (lane >> 4);              // position inside a padded LDS row
-    const bf16_t *p1[4], *pv[4], *p2[4];
-    bf16_t* po[4];
-    // uniform 64-bit row addresses plus one 32-bit lane offset keep the sixteen row pointers out of the vector registers
-    const uint32_t lane_b = (uint32_t)lane * 16u;
-    auto lane_at = [&](const bf16_t* p) -> const bf16_t* { return (const bf16_t*)((const char*)p + lane_b); };
-    auto lane_to = [&](bf16_t* p) -> bf16_t* { return (bf16_t*)((char*)p + lane_b); };
+    // Rows are addressed through buffer descriptors (base = sample 0 of the row, range = its L samples): a request
+    // outside the row reads zeros and a store outside it is dropped by the address unit, so no access of the main
+    // loop sits under a branch or a predicate, neither the padding ahead of sample 0 nor the tail behind sample
+    // L-1 nor the pieces of a step that do not exist, and the compiler can count exactly how many younger requests
+    // may still be in flight when a register stage is consumed.  An access is out of range when its per-lane offset
+    // is >= range - scalar offset (unsigned): the per-lane offset carries everything that can be negative (lane,
+    // piece, padding), the scalar offset the time, which is kept >= 0 by moving one step into the lane offset.
+    __amdgpu_buffer_rsrc_t r1[NROW], rv[PRE ? NROW : 1], r2[POST ? NROW : 1], ro[NROW];
+    const int range = (int)(L * 2);                            // bytes (the launcher keeps rows below 2 GiB)
+#pragma unroll
+    for (int r = 0; r < NROW; ++r) {
+        const int64_t d = d0 + r;
+        r1[r] = __builtin_amdgcn_make_buffer_rsrc((void*)a.x1.row(b, d), 0, range, 0x00020000);
+        if constexpr (PRE) rv[r] = __builtin_amdgcn_make_buffer_rsrc((void*)a.v.row(b, d), 0, range, 0x00020000);
+        if constexpr (POST) r2[r] = __builtin_amdgcn_make_buffer_rsrc((void*)a.x2.row(b, d), 0, range, 0x00020000);
+        ro[r] = __builtin_amdgcn_make_buffer_rsrc((void*)(a.out + (b * a.D + d) * L), 0, range, 0x00020000);
+    }
     // LDS row r is channel d0 + r (CPW = 4) or the r-th 512-sample piece of channel d0 (CPW = 1)
     auto roff = [](int r) -> int64_t { return CPW == 4 ? 0 : (int64_t)TL * r; };
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int64_t d = d0 + (CPW == 4 ? r : 0);
-        const int64_t o = woff + roff(r) - pad;                // virtual positions, never used below lo; wave-uniform: the
-                                                               // lane's 16 bytes are added at each access (lane_at)
-        p1[r] = a.x1.row(b, d) + o;
-        pv[r] = PRE ? a.v.row(b, d) + o : nullptr;
-        p2[r] = POST ? a.x2.row(b, d) + o : nullptr;
-        po[r] = a.out + (b * a.D + d) * L + o;
-    }
-    const u32x4 zero4 = {0, 0, 0, 0};
+    auto rrow = [](int r) { return CPW == 4 ? r : 0; };
+    constexpr uint32_t STEP2 = (uint32_t)STEP * 2u;
+    // byte offset of this lane's piece of row r at row time t = STEP (virtual position -> real sample: minus lo)
+    const uint32_t vo0 = (uint32_t)(((int)lane * 8 - (int)lo + STEP) * 2);
+    auto vo = [&](int r) -> uint32_t { return vo0 + (uint32_t)(roff(r) * 2); };
+    // row time t -> (what to take off the lane offset, scalar offset): t >= STEP in the main loop
+    auto ld_at = [&](const __amdgpu_buffer_rsrc_t& rs, int r, int64_t t) -> u32x4 {     // t >= STEP
+        return __builtin_amdgcn_raw_buffer_load_b128(rs, vo(r), (uint32_t)(t - STEP) * 2u, NT ? 2 : 0);
+    };
+    auto ld_any = [&](const __amdgpu_buffer_rsrc_t& rs, int r, int64_t t) -> u32x4 {    // t >= 0
+        const uint32_t back = t >= STEP ? 0u : STEP2, so = t >= STEP ? (uint32_t)(t - STEP) * 2u : 0u;
+        return __builtin_amdgcn_raw_buffer_load_b128(rs, vo(r) - back, so, NT ? 2 : 0);
+    };
+    auto st_any = [&](const __amdgpu_buffer_rsrc_t& rs, int r, int64_t t, u32x4 val) {  // any t; t < 0: dropped
+        const uint32_t back = t >= STEP ? 0u : STEP2;
+        const uint32_t so = t >= STEP ? (uint32_t)(t - STEP) * 2u : (t >= 0 ? 0u : 0xFFFFFFFFu);
+        __builtin_amdgcn_raw_buffer_store_b128(val, rs, vo(r) - back, so, NT ? 2 : 0);
+    };
     u32x4 c1[PF][4], cv[PRE ? PF : 1][4], c2[POST ? PF : 1][4];      // register stages (absent gates take none)
     auto request_rows = [&]() {
 #pragma unroll
@@ -266,11 +288,9 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int64_t t = (int64_t)p * STEP;
-                const int64_t pos = t + roff(r) + lane * 8;
-                const bool ok = pos < Lw && pos >= lo;
-                c1[p][r] = ok ? ld16<NT>(lane_at(p1[r] + t)) : zero4;
-                if constexpr (PRE) cv[p][r] = ok ? ld16<NT>(lane_at(pv[r] + t)) : zero4;
-                if constexpr (POST) c2[p][r] = ok ? ld16<NT>(lane_at(p2[r] + t)) : zero4;
+                c1[p][r] = ld_any(r1[rrow(r)], r, t);
+                if constexpr (PRE) cv[p][r] = ld_any(rv[rrow(r)], r, t);
+                if constexpr (POST) c2[p][r] = ld_any(r2[rrow(r)], r, t);
             }
     };
     // With four channels per wavefront the rows are requested before the fragment build and travel during it
@@ -398,17 +418,31 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
     const int n = lane & 15, q = lane >> 4;
     const int c = n & 3, s = n >> 2;
     // scan-side lane geometry: one complex state per lane
-    const int sc = CPW == 4 ? (lane >> 4) : 0, sp = lane & 15;
+    // (sq: the lane row, which is the channel with CPW = 4 and the 512-sample piece of the step with CPW = 1)
+    const int sq = lane >> 4, sc = CPW == 4 ? sq : 0, sp = lane & 15;
     float Xr = 0.f, Xi = 0.f;
     float Xfr = 0.f, Xfi = 0.f;                                // state after the chunk that holds sample L-1
-    bool have_final = !COOP;                                   // COOP: only the wavefront whose piece holds sample L-1
+    bool have_final = !COOP && CPW == 4;                       // otherwise only the wavefront / lane row whose piece holds sample L-1
     float dco = 0.f;
     if (a.Dcoef) dco = a.Dcoef[d0 + (CPW == 4 ? c : 0)];
-    float X0r = 0.f, X0i = 0.f;                                // COOP: state at the start of the block's step
+    float X0r = 0.f, X0i = 0.f;                                // COOP, CPW = 1: state at the start of the step
     float ppr = pcr, ppi = pci;                                // COOP: p^TLW, one wavefront's piece
     if (COOP) {
 #pragma unroll
         for (int k = 1; k < 16 / CPW; ++k) { const float t = ppr * pcr - ppi * pci; ppi = ppr * pci + ppi * pcr; ppr = t; }
+    }
+    // CPW = 1: powers of the pole that carry a state over one, two and four 512-sample pieces, and over the pieces
+    // ahead of this lane row's own (p^0, p^512, p^1024, p^1536)
+    float p4r = 1.f, p4i = 0.f, p8r = 1.f, p8i = 0.f, p16r = 1.f, p16i = 0.f, mqr = 1.f, mqi = 0.f;
+    if constexpr (CPW == 1) {
+        auto sqr = [](float& r, float& i) { const float t = r * r - i * i; i = 2.f * r * i; r = t; };
+        p4r = pcr; p4i = pci;
+        sqr(p4r, p4i); sqr(p4r, p4i);                          // p^512
+        p8r = p4r; p8i = p4i; sqr(p8r, p8i);                   // p^1024
+        p16r = p8r; p16i = p8i; sqr(p16r, p16i);               // p^2048
+        const float p12r = p8r * p4r - p8i * p4i, p12i = p8r * p4i + p8i * p4r;
+        mqr = sq == 0 ? 1.f : sq == 1 ? p4r : sq == 2 ? p8r : p12r;
+        mqi = sq == 0 ? 0.f : sq == 1 ? p4i : sq == 2 ? p8i : p12i;
     }
 
     // ---- FEAT: taps of this wavefront's channels (wave-uniform, kept in scalar registers) and the carried dwords
@@ -463,24 +497,18 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                 const u32x4 f1 = feat(c1[p][r], car1[chain(r)], fw[0][chain(r)]);
                 const u32x4 fv = feat(cv[p][r], carv[chain(r)], fw[2][chain(r)]);
                 un[r] = gate_mul<true>(f1, fv);
-                const bool okn = tn + roff(r) + lane * 8 < Lw;
-                c1[p][r] = okn ? ld16<NT>(lane_at(p1[r] + tn)) : zero4;
-                cv[p][r] = okn ? ld16<NT>(lane_at(pv[r] + tn)) : zero4;
+                c1[p][r] = ld_at(r1[rrow(r)], r, tn);
+                cv[p][r] = ld_at(rv[rrow(r)], r, tn);
             }
         }
     };
 
-    // One step.  GUARD = true tests every access against the row's bounds (a wave-uniform test for whole pieces, per-lane
-    // predicates otherwise); GUARD = false is for steps whose loads, stores and refills are all whole pieces inside the
-    // row: no branch surrounds a memory instruction there, which is what lets the compiler count exactly how many
-    // younger requests may still be in flight when a register stage is consumed (with branches around them it has to
-    // wait for everything outstanding, the prefetched stages included).
-    auto step = [&](auto guard_tag, const int p, const int64_t ts) __attribute__((always_inline)) {
-        constexpr bool GUARD = decltype(guard_tag)::value;
+    // One step.  No memory access is conditional: what lies outside the row is handled by the buffer descriptors.
+    auto step = [&](const int p, const int64_t ts) __attribute__((always_inline)) {
         const int pp = (p + PF - 1) % PF;                      // register stage of the previous step
         const int64_t tn = ts + (int64_t)PF * STEP;            // step that reuses this register stage
 
-        // u = bf16(x1*v) of this step -> LDS; refill the stage with step ts + PF*TLW
+        // u = bf16(x1*v) of this step -> LDS; refill the stage with step ts + PF*STEP
         if constexpr (EARLY) {
             // formed one step ahead (prepare_u, in the shadow of the step before): only the LDS write is left here
 #pragma unroll
@@ -496,25 +524,15 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                 } else if constexpr (PRE) *(u32x4*)(u_w + r * URS + lofs) = gate_mul<true>(c1[p][r], cv[p][r]);
                 else *(u32x4*)(u_w + r * URS + lofs) = c1[p][r];
             }
-            // whole pieces inside the row (a wave-uniform test) are requested without per-lane predicates
-            if (!GUARD || tn + TLW <= Lw) {
-                // (without branches around them the scheduler would move these requests, and what waits on the registers
-                // they overwrite, far from here and run out of registers: pin the group where the branches used to hold it)
-                if (!GUARD) __builtin_amdgcn_sched_barrier(0);
+            // (the scheduler would move these requests, and what waits on the registers they overwrite, far from
+            // here and run out of registers: pin the group)
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    c1[p][r] = ld16<NT>(lane_at(p1[r] + tn));
-                    if constexpr (PRE) cv[p][r] = ld16<NT>(lane_at(pv[r] + tn));
-                }
-                if (!GUARD) __builtin_amdgcn_sched_barrier(0);
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const bool okn = tn + roff(r) + lane * 8 < Lw;
-                    c1[p][r] = okn ? ld16<NT>(lane_at(p1[r] + tn)) : zero4;
-                    if constexpr (PRE) cv[p][r] = okn ? ld16<NT>(lane_at(pv[r] + tn)) : zero4;
-                }
+            for (int r = 0; r < 4; ++r) {
+                c1[p][r] = ld_at(r1[rrow(r)], r, tn);
+                if constexpr (PRE) cv[p][r] = ld_at(rv[rrow(r)], r, tn);
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
         wave_sync();
 
@@ -571,7 +589,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                     if constexpr (FEAT != 0) {
                         // the first step has no output behind it: its stage holds a later piece, which is consumed,
                         // and carried on, when its own turn comes
-                        if (!GUARD || ts_out >= 0) g2 = feat(c2[pp][r], car2[chain(r)], fw[1][chain(r)]);
+                        if (ts_out >= 0) g2 = feat(c2[pp][r], car2[chain(r)], fw[1][chain(r)]);
                         __builtin_amdgcn_sched_barrier(0);
                     }
 #pragma unroll
@@ -579,39 +597,70 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                         o[r][j] = pack_bf2(bf_lo(zz[r][j]) * bf_lo(g2[j]), bf_hi(zz[r][j]) * bf_hi(g2[j]));
                 }
             }
-            if (!GUARD || (ts_out >= 0 && (ts_out > 0 || lo <= 0) && t_refill + TLW <= Lw)) {   // wave-uniform: store and refill whole pieces
-                if (!GUARD) __builtin_amdgcn_sched_barrier(0);
+            // (in the first step of a row ts_out < 0: the store is dropped, and with FEAT the refill asks again
+            // for the piece the stage already holds)
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    st16<NT>(lane_to(po[r] + ts_out), o[r]);
-                    if constexpr (POST) c2[pp][r] = ld16<NT>(lane_at(p2[r] + t_refill));
-                }
-                if (!GUARD) __builtin_amdgcn_sched_barrier(0);
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int64_t pos = ts_out + roff(r) + lane * 8;
-                    const bool okc = ts_out >= 0 && pos < Lw && pos >= lo;
-                    const bool okr = ts_out >= 0 && t_refill + roff(r) + lane * 8 < Lw;
-                    if (okc) st16<NT>(lane_to(po[r] + ts_out), o[r]);
-                    if constexpr (POST) { if (ts_out >= 0) c2[pp][r] = okr ? ld16<NT>(lane_at(p2[r] + t_refill)) : zero4; }
-                }
+            for (int r = 0; r < 4; ++r) {
+                st_any(ro[rrow(r)], r, ts_out, o[r]);
+                if constexpr (POST) c2[pp][r] = ld_at(r2[rrow(r)], r, t_refill);
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
         wave_sync();
 
-        // ---- scan over the chunks of the step in time order: lane = (channel sc, pole sp).
-        // Column n = c + 4s sits in row n of l_w / x*_w; in time order chunk k is (c, s) = (sc, k) for
-        // CPW = 4 and (k / 4, k % 4) for CPW = 1, where all 64 lanes repeat the work of lanes 0..15.
+        // ---- scan over the chunks of the step in time order: lane = (lane row sq, pole sp).
+        // Column n = c + 4s sits in row n of l_w / x*_w, and a lane row walks the four chunks s = 0..3 of its c = sq:
+        // the four chunks of the step of its channel (CPW = 4), or the sq-th 512-sample piece of the one channel's
+        // step (CPW = 1), whose entering state comes from the lane rows before it.
         {
-            constexpr int NK = 16 / CPW;
+            constexpr int NK = 4;
             float lr[NK], li[NK];
 #pragma unroll
             for (int k = 0; k < NK; ++k) {
-                const int row = CPW == 4 ? (k * 4 + sc) : ((k & 3) * 4 + (k >> 2));
+                const int row = k * 4 + sq;
                 const float2 t = *(const float2*)(l_w + row * LRS + 2 * sp);
                 lr[k] = t.x;
                 li[k] = t.y;
+            }
+            float nX0r = 0.f, nX0i = 0.f;
+            if constexpr (CPW == 1) {
+                // What a piece adds to the state (its end state from a zero start), gathered over the four lane rows
+                // with two lane-row swaps: a wavefront-wide exchange in the vector ALU, no trip through LDS.
+                float er = 0.f, ei = 0.f;
+#pragma unroll
+                for (int k = 0; k < NK; ++k) {
+                    const float nr = fmaf(pcr, er, fmaf(-pci, ei, lr[k]));
+                    ei = fmaf(pcr, ei, fmaf(pci, er, li[k]));
+                    er = nr;
+                }
+                // v_permlane16_swap of a register with itself: [0] holds rows (0, 0, 2, 2), [1] rows (1, 1, 3, 3)
+                const auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(er), __float_as_uint(er), false, false);
+                const auto i16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(ei), __float_as_uint(ei), false, false);
+                const float ar = __uint_as_float(r16[0]), ai = __uint_as_float(i16[0]);
+                const float br = __uint_as_float(r16[1]), bi = __uint_as_float(i16[1]);
+                // pieces (0, 1) and (2, 3) joined: rows (c01, c01, c23, c23)
+                const float cr = fmaf(p4r, ar, fmaf(-p4i, ai, br)), ci = fmaf(p4r, ai, fmaf(p4i, ar, bi));
+                // v_permlane32_swap: [0] holds rows (0, 1, 0, 1), [1] rows (2, 3, 2, 3)
+                const auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(cr), __float_as_uint(cr), false, false);
+                const auto i32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(ci), __float_as_uint(ci), false, false);
+                const float c01r = __uint_as_float(r32[0]), c01i = __uint_as_float(i32[0]);
+                const float c23r = __uint_as_float(r32[1]), c23i = __uint_as_float(i32[1]);
+                // state entering piece sq: X0 pushed through the pieces before it plus what those pieces added
+                //   sq 0: X0    1: p^512 X0 + e0    2: p^1024 X0 + c01    3: p^1536 X0 + p^512 c01 + e2
+                // (selected, not multiplied by 0 / 1: what later pieces hold never reaches an earlier one)
+                float xr = mqr * X0r - mqi * X0i, xi = mqr * X0i + mqi * X0r;
+                const float tr = (sq & 1) ? p4r * c01r - p4i * c01i : c01r;
+                const float ti = (sq & 1) ? p4r * c01i + p4i * c01r : c01i;
+                xr += (sq & 2) ? tr : 0.f;
+                xi += (sq & 2) ? ti : 0.f;
+                xr += (sq & 1) ? ar : 0.f;
+                xi += (sq & 1) ? ai : 0.f;
+                Xr = xr;
+                Xi = xi;
+                // state after the step, the same in every lane row
+                nX0r = fmaf(p16r, X0r, fmaf(-p16i, X0i, fmaf(p8r, c01r, fmaf(-p8i, c01i, c23r))));
+                nX0i = fmaf(p16r, X0i, fmaf(p16i, X0r, fmaf(p8r, c01i, fmaf(p8i, c01r, c23i))));
             }
             if (COOP) {
                 // what this piece adds to the state (its end state from a zero start) goes to the other wavefronts;
@@ -640,7 +689,7 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
             }
 #pragma unroll
             for (int k = 0; k < NK; ++k) {
-                const int row = CPW == 4 ? (k * 4 + sc) : ((k & 3) * 4 + (k >> 2));
+                const int row = k * 4 + sq;
                 const uint32_t xh = pack_bf2(Xr, Xi);
                 const int o = row * XRS + 2 * sp;
                 *(uint32_t*)(xh_w + o) = xh;
@@ -649,11 +698,12 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                 const float ni = fmaf(pcr, Xi, fmaf(pci, Xr, li[k]));
                 Xr = nr;
                 Xi = ni;
-                if (GUARD) {                                   // chunk k of the step covers ts + 128k .. + 127
-                    const int64_t te = ts + (int64_t)C * (k + 1);
+                {                                              // this chunk covers te - 128 .. te - 1
+                    const int64_t te = ts + (int64_t)C * ((CPW == 4 ? k : 4 * sq + k) + 1);
                     if (te >= Lw && te - C < Lw) { Xfr = Xr; Xfi = Xi; have_final = true; }
                 }
             }
+            if constexpr (CPW == 1) { X0r = nX0r; X0i = nX0i; }
         }
         wave_sync();
 
@@ -712,43 +762,24 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
         // the wave_sync after the next step's u write orders these z writes before their coalesced reads
     };
 
-    const std::integral_constant<bool, true> guarded;
-    const std::integral_constant<bool, false> whole;
-    // Rotations of PF steps.  A rotation is `whole` when every access of its steps is a whole piece inside the row: not
-    // the first one (its stores start at sample 0, behind the padding), and the refill of its last step, PF steps ahead,
-    // still ends inside the row of every wavefront of the block (the last one starts 3 pieces further on with COOP).
-    // Every guarded rotation, and the prologue, ends with a wait for all outstanding requests, so that the whole
-    // rotations start from a known state; they are the first and the last two of a row.
-    // The bounds are the block's (Lv, not Lw): with COOP every wavefront runs every step and meets every barrier.
-    // The one-channel form with all three gate streams keeps guarded steps throughout: it runs at the ceiling of its
-    // access order either way, and three register stages under guarded steps measured 2 % faster there (1.628 against
-    // 1.659 ms at L = 262144) than the two stages that fit whole-piece steps.
-    constexpr bool WHOLE_ROTATIONS = !(CPW == 1 && PRE && POST) && FEAT == 0;
-    constexpr int VMCNT0 = 0x0F70;                             // s_waitcnt vmcnt(0), other counters unconstrained
-    const int64_t whole_until = Lv - (COOP ? 3 * TLW : 0) - TLW - (int64_t)(2 * PF - 1) * STEP;
-    if (WHOLE_ROTATIONS) __builtin_amdgcn_s_waitcnt(VMCNT0);
+    // Rotations of PF steps while a whole rotation lies inside the block's row (Lv, not Lw: with COOP every wavefront
+    // runs every step and meets every barrier), then the steps that are left.  Steps may ask for pieces behind the
+    // end of the row (they read zeros) and the first one stores nothing.
     if constexpr (EARLY) prepare_u(0, 0);
-    for (int64_t ts = 0; ts < Lv; ts += (int64_t)PF * STEP) {
-        if (WHOLE_ROTATIONS && ts > 0 && ts <= whole_until) {
-            if constexpr (WHOLE_ROTATIONS) {
+    int64_t ts = 0;
+    for (; ts + (int64_t)(PF - 1) * STEP < Lv; ts += (int64_t)PF * STEP) {
 #pragma unroll
-                for (int p = 0; p < PF; ++p) step(whole, p, ts + (int64_t)p * STEP);
-            }
-        } else {
-#pragma unroll
-            for (int p = 0; p < PF; ++p)
-                if (ts + (int64_t)p * STEP < Lv) step(guarded, p, ts + (int64_t)p * STEP);
-            if (WHOLE_ROTATIONS) __builtin_amdgcn_s_waitcnt(VMCNT0);
-        }
+        for (int p = 0; p < PF; ++p) step(p, ts + (int64_t)p * STEP);
     }
+#pragma unroll
+    for (int p = 0; p < PF - 1; ++p)
+        if (ts + (int64_t)p * STEP < Lv) step(p, ts + (int64_t)p * STEP);
     {   // output of the last step
         const int64_t ts_last = ((Lv + STEP - 1) / STEP - 1) * STEP;
         wave_sync();
         const int pl = (int)((ts_last / STEP) % PF);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int64_t pos = ts_last + roff(r) + lane * 8;
-            const bool okc = pos < Lw && pos >= lo;
             const u32x4 zz = *(const u32x4*)(z_w + r * URS + lofs);
             u32x4 o = zz;
             if constexpr (POST) {
@@ -761,13 +792,13 @@ __global__ __launch_bounds__(256, 1) void li_kernel(LiArgs a) {
                 for (int j = 0; j < 4; ++j)
                     o[j] = pack_bf2(bf_lo(zz[j]) * bf_lo(x2v[j]), bf_hi(zz[j]) * bf_hi(x2v[j]));
             }
-            if (okc) st16<NT>(lane_to(po[r] + ts_last), o);
+            st_any(ro[rrow(r)], r, ts_last, o);
         }
     }
 
     if (a.state_out && have_final) {
         // the last chunk of the virtual row ends on sample L-1: the scan's state after it is the decode state
-        if ((CPW == 4 || lane < 16) && sp < a.sr) {
+        if (sp < a.sr) {                                       // CPW = 1: the lane row whose piece ended the row
             float* sp_ = a.state_out + ((b * a.D + d0 + sc) * a.sr + sp) * 2;
             sp_[0] = Xfr;
             sp_[1] = Xfi;
@@ -895,8 +926,11 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
         return hyena_fail(HYENA_EALIGN, "%s: L and strides must be multiples of 8, pointers 16-byte aligned", who);
     if (d_is_bf16 < 0 || d_is_bf16 > 2) return hyena_fail(HYENA_EINVAL, "%s: d_is_bf16 must be 0, 1 or 2", who);
     // the kernel does the channel arithmetic in 32 bits: reject maps and sizes that would wrap or divide by zero
-    if (!rows_valid(x1) || !rows_valid(x2) || !rows_valid(v) || B * D >= (1LL << 31) || L >= (1LL << 40))
+    if (!rows_valid(x1) || !rows_valid(x2) || !rows_valid(v) || B * D >= (1LL << 31))
         return hyena_fail(HYENA_EINVAL, "%s: B*D and the channel map must fit 31 bits", who);
+    // rows are addressed through 32-bit byte offsets inside a buffer descriptor
+    if (L > (1LL << 30) - (1LL << 16))
+        return hyena_fail(HYENA_ENOSUP, "%s: rows of L=%lld samples (up to 2^30 - 2^16)", who, (long long)L);
     const bool pre = v && v->ptr, post = x2 && x2->ptr;
     if (pre && !post) return hyena_fail(HYENA_ENOSUP, "%s: v without x2 (pass both, x2 alone with x1 holding x1*v, or neither)", who);
     if (ftaps && (!pre || !post || y_conv_fp32))
@@ -914,7 +948,10 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
     const bool can4 = (D / G) % 4 == 0;
     const bool long_coop = can4 && L >= 65536 && post && !ftaps;      // the featurizer form runs lone wavefronts only
     int cpw = (can4 && (L < 65536 || long_coop)) ? 4 : 1;    // channels per wavefront (they share one filter)
-    if (ftaps && can4) cpw = 4;     // featurizer form: 1.80 against 1.83 ms at L = 262144, and faster below
+    // featurizer form (lone wavefronts only): four channels per wavefront on rows below 65536 samples when that
+    // still gives every SIMD a wavefront (B = 1, D = 4096: 61 against 88 us at L = 8192, 430 against 413 us at
+    // L = 65536, 1.67 against 1.59 ms at L = 262144; D = 1024, L = 16384: 102 against 36 us)
+    if (ftaps) cpw = (can4 && L < 65536 && B * (D / 4) >= 1024) ? 4 : 1;
     { const int64_t x = hyena_override(HYENA_OV_LI_CPW); if (x == 1) cpw = 1; else if (x == 4 && can4) cpw = 4; }
     const int64_t nquads = B * (D / cpw);
     bool coop = cpw == 4 && (nquads <= 512 || long_coop);
@@ -957,10 +994,10 @@ int li_fwd_impl(const char* who, const hyena_rows* x1, const hyena_rows* x2, con
         if (x >= 0) c = (x > 0 && nblk % (8 * x) == 0) ? x : 0;
         a.xchunk = (uint32_t)c;
     }
-// prefetch depth in steps: two with four channels per wavefront (measured 1-3 % faster than three, which in turn
-// beats four, whose registers spill).  One channel per wavefront: three, except on x1*v rows (three stages of two
-// input streams leave the whole-piece steps short of registers: 110 spilled dwords and 1.63 against 1.52 ms at
-// L = 262144); the three-gate form runs its three stages under guarded steps (see the step loop)
+// prefetch depth in steps: two with four channels per wavefront (three measured the same: 1.528 ms either way in
+// the cooperative form, 1.615 against 1.618 ms for lone wavefronts, 1.708 against 1.702 ms with the featurizer
+// inside, at B = 1, L = 262144, D = 4096).  One channel per wavefront: three (two measured 1.569 against 1.576 ms),
+// two on x1*v rows.
 #define LI_LAUNCH(P, Q, N, M, Y)                                                                           \
     do {                                                                                                   \
         if (cpw == 4 && coop) hipLaunchKernelGGL((li_kernel<P, Q, N, 2, M, Y, 4, true>), grid, dim3(256), 0, s, a);   \
