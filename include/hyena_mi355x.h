@@ -136,7 +136,9 @@ int hyena_mr_fwd(const hyena_rows* x1, const hyena_rows* x2, const hyena_rows* v
  * owns the workspace: hyena_li_plan_bytes(G, S) bytes of device memory, reusable until the parameters change.
  * S is 1..16 (fewer than 16 modes are filled up with poles of residue zero inside the table).
  *
- * hyena_li_fwd: L and strides must be multiples of 8; any D/G (groups of a multiple of 4 channels are fastest).
+ * hyena_li_fwd: L and strides must be multiples of 8, L at most 2^30 - 2^16 (rows are addressed with 32-bit byte
+ * offsets; HYENA_ENOSUP beyond); any D/G (groups of a multiple of 4 channels are fastest).  Nothing outside the
+ * B*D rows of L samples is read or written.
  * y_conv_fp32 (optional, [B][D][L]) receives the fp32 convolution before any rounding;
  * state_out (optional, [B][D][S][2] float32) the modal state after the last sample.
  * d_is_bf16 selects the rounding of z = y + Dcoef*x1v: 1 = bf16(bf16(y) + bf16(Dcoef*x1v)), what

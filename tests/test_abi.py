@@ -175,6 +175,21 @@ def test_bad_row_descriptors_are_rejected_by_every_prefill_entry_point():
     assert L.hyena_li_fwd(g, g, g, P, None, 1, P, None, None, 1 << 20, 1 << 12, 64, 1, 16, None) == -1
 
 
+def test_li_row_length_limit_is_checked_before_launch():
+    # the long-convolution kernel addresses a row with 32-bit byte offsets: rows beyond 2^30 - 2^16 samples are refused
+    from vortex_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built in this tree")
+    L = _lib.lib()
+    P = 4096
+    big = (1 << 30) - (1 << 16) + 8
+    g = ctypes.byref(_lib.Rows(P, 16 * big, big, 16, 16))
+    assert L.hyena_li_fwd(g, g, g, P, None, 1, P, None, None, 1, 16, big, 1, 16, None) == -3
+    assert b"2^30" in L.hyena_last_error_string()
+    taps = P
+    assert L.hyena_li_layer_fwd(g, g, g, taps, 3, P, None, 1, P, None, 1, 16, big, 1, 16, None) == -3
+
+
 def test_launch_override_names():
     from vortex_amd import _lib
     if not os.path.exists(_lib.LIB_PATH):

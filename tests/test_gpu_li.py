@@ -6,6 +6,7 @@ import pytest
 import torch
 
 import vortex_amd as va
+from vortex_amd import ops
 from oracle import hyena_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -263,3 +264,45 @@ def test_li_block_order_changes_nothing(form, override):
     assert rel_err(torch.view_as_real(res[0][1]), torch.view_as_real(st_ref)) <= 1e-4
     for out, st in res[1:]:
         assert torch.equal(out, res[0][0]) and torch.equal(st, res[0][1])
+
+
+@pytest.mark.parametrize("form", ["lone4", "coop4", "cpw1", "feat4", "feat1"])
+@pytest.mark.parametrize("L", [8, 1544, 2048 * 3, 4096 + 2048 + 120])
+def test_li_touches_nothing_outside_its_rows(form, L, override):
+    """Steps past the end of a row ask for pieces that do not exist and the first step has no output behind it: such
+    requests read zeros and such stores are dropped.  The output lies inside a larger buffer whose neighbouring rows
+    must keep their sentinel, the inputs are rows of padded buffers whose padding holds NaN (a read past a row's end
+    would poison the row's state and its last outputs), and the result equals the one from plain tensors."""
+    B, D, G = 2, 16, 4
+    override(**{"lone4": dict(li_cpw=4, li_coop=0), "coop4": dict(li_cpw=4, li_coop=1), "cpw1": dict(li_cpw=1),
+                "feat4": dict(li_cpw=4), "feat1": dict(li_cpw=1)}[form])
+    g = torch.Generator().manual_seed(L)
+    lp, r = O.make_modal_complex(G, 16, seed=L + 1)
+    Db = torch.randn(D, generator=g).bfloat16().cuda()
+    plan = ops.ModalPlan(lp.cuda(), r.cuda())
+    nrow = 3 * D if form.startswith("feat") else D
+    pad = 64
+    bufs = [torch.full((B, nrow, pad + L + pad), float("nan"), dtype=torch.bfloat16, device="cuda") for _ in range(3)]
+    plain = [torch.randn(B, nrow, L, generator=g).bfloat16().cuda() for _ in range(3)]
+    for bf, pl in zip(bufs, plain):
+        bf[:, :, pad:pad + L] = pl
+    views = [bf[:, :, pad:pad + L] for bf in bufs]
+    big = torch.full((B * D + 2, L), 7.0, dtype=torch.bfloat16, device="cuda")
+    out = big[1:1 + B * D].view(B, D, L)
+
+    def run(ts, o):
+        if form.startswith("feat"):
+            (q2, q1, qv), chan = ops.projection_rows(ts[0], D)
+            w = (torch.randn(3 * D, 3, generator=torch.Generator().manual_seed(3)) / 3 ** 0.5).cuda()
+            taps = torch.stack([w[chan[1]], w[chan[0]], w[chan[2]]]).contiguous()
+            return ops.li_layer_fwd_rows(q1, q2, qv, taps, plan, Db, B, D, L, device="cuda", want_state=True, out=o)
+        y, _, st = ops.li_fwd_rows(ops.rows_of(ts[0]), ops.rows_of(ts[1]), ops.rows_of(ts[2]), plan, Db, B, D, L,
+                                   device="cuda", want_state=True, out=o)
+        return y, st
+
+    y, st = run(views, out)
+    y_ref, st_ref = run(plain, None)
+    torch.cuda.synchronize()
+    assert bool((big[0] == 7.0).all()) and bool((big[-1] == 7.0).all())
+    assert bool(torch.isfinite(y.float()).all()) and bool(torch.isfinite(torch.view_as_real(st)).all())
+    assert torch.equal(y, y_ref) and torch.equal(torch.view_as_real(st), torch.view_as_real(st_ref))
